@@ -1,0 +1,284 @@
+/*
+ * zllm_attn — C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * GQA / MLA decode and chunked-prefill attention over a Q8g64 paged KV cache,
+ * plus the quantizing page appends that feed it.  Every entry point stands in
+ * for one launcher (`try_*`) of zllm-lab/zllm's ROCm kernel layer; the comment
+ * above each names the reference interface it replaces (paths relative to the
+ * zLLM tree).
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; device pointers are marked [dev].
+ *   - the caller owns every allocation, including the workspace whose size the
+ *     matching *_workspace_bytes function returns.  Nothing here allocates,
+ *     frees or synchronises; launches are asynchronous on `stream`.
+ *   - re-entrant: no mutable global state; the error text is thread-local.
+ *   - return value: 0 = ok, negative = invalid argument (see
+ *     zllm_attn_last_error), positive = a hipError_t from the launch.
+ *   - shape errors are reported before anything is launched, as the reference
+ *     launchers do (src/kernel/rocm/hip/tensor/attention.rs:1022-1030,
+ *     src/kernel/rocm/hip/attention/paged_mla.rs:2940-2977).
+ *
+ * KV layout (kept from src/kv_cache/mod.rs:179-331 and
+ * src/kernel/rocm/hip/attention/paged_mla/source.hip:46-54,191-201):
+ *   planar per tensor; row = one token; physical row of logical token t is
+ *   table[t / block_tokens] * block_tokens + t % block_tokens (a NULL table is
+ *   the identity); codes plane int8 [rows][cols]; scales plane one 16-bit (or
+ *   f32) value per 64 contiguous columns [rows][cols / 64].
+ */
+#ifndef ZLLM_ATTN_H
+#define ZLLM_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t, passed opaquely so that bindings need no HIP headers. */
+typedef void* zllm_stream_t;
+
+/* Exported from libzllm_attn.so (everything else in the library is hidden). */
+#define ZLLM_API __attribute__((visibility("default")))
+
+/* Scale storage of a Q8g64 plane; numbering of `zllm_scale`
+ * (src/kernel/rocm/hip/hiprtc.rs:104-116). */
+enum { ZLLM_SCALE_BF16 = 0, ZLLM_SCALE_F16 = 1, ZLLM_SCALE_F32 = 2 };
+
+/* Element type of activations handed in / out. */
+enum { ZLLM_DTYPE_F32 = 0, ZLLM_DTYPE_BF16 = 1, ZLLM_DTYPE_F16 = 2 };
+
+/* KV storage format (src/config.rs:1108-1114 KvCacheFormat {F16, Q8g64}). */
+enum { ZLLM_KV_Q8G64 = 0, ZLLM_KV_F16 = 1 };
+
+/* Which reference quantizer the codes follow:
+ *   ROCM_MLA : scale = absmax * (1/127) (1.0 if 0), stored bf16, codes =
+ *              nearbyint(x / f32(stored))   (paged_mla/source.hip:183-201)
+ *   METAL_GQA: scale = absmax / 127 (1.0 if 0), stored f16, codes =
+ *              rint(x * (1 / scale))        (kernel/metal/attention/mod.rs:114-127)
+ *   CUDA_GQA : as METAL_GQA, stored f32     (kernel/cuda/attention.rs:331-341) */
+enum { ZLLM_QUANT_ROCM_MLA = 0, ZLLM_QUANT_METAL_GQA = 1, ZLLM_QUANT_CUDA_GQA = 2 };
+
+/* RoPE pair layout (src/attention/rope.rs:106-110). */
+enum { ZLLM_ROTARY_INTERLEAVED = 0, ZLLM_ROTARY_SPLIT_HALF = 1 };
+
+#define ZLLM_GROUP_SIZE 64 /* src/kv_cache/mod.rs:29 DEFAULT_GROUP_SIZE */
+
+/* Library / device bring-up.  Optional: every entry point works without it.
+ * Returns 0 and fills `cu_count` (may be NULL) when a gfx950 device is current. */
+ZLLM_API int zllm_attn_init(int device, int* cu_count);
+
+/* Text of the last failure on the calling thread ("" if none). */
+ZLLM_API const char* zllm_attn_last_error(void);
+
+/* ------------------------------------------------------------------------- *
+ * Host-side layout arithmetic (no GPU).                                      *
+ * ------------------------------------------------------------------------- */
+
+/* CausalWindow::key_range (src/attention/gqa.rs:54-62); window 0 = Full. */
+ZLLM_API void zllm_attn_key_range(uint64_t window, uint64_t query_position, uint64_t key_end,
+                         uint64_t* start, uint64_t* end);
+
+/* KvCacheSpec::bytes_per_token (src/kv_cache/mod.rs:570-585).  kind 0 = MLA
+ * (a = kv_lora_rank, b = qk_rope_head_dim), 1 = GQA (a = kv heads, b = head
+ * dim).  0 on invalid input. */
+ZLLM_API uint64_t zllm_kv_bytes_per_token(int kind, uint64_t a, uint64_t b, uint64_t group);
+
+/* KvCacheLayout planar offsets (src/kv_cache/mod.rs:246-330), Int8 format.
+ * MLA: offsets = {base, codes, scales, rope}; GQA: {base, K codes, K scales,
+ * V codes, V scales}.  Returns total bytes, 0 on invalid input. */
+ZLLM_API uint64_t zllm_kv_layout_offsets(int kind, uint64_t a, uint64_t b, uint64_t group, uint64_t layer_count,
+                                uint64_t capacity, uint64_t layer, uint64_t offsets[5]);
+
+/* HybridGqaCacheLayout::write_plan (src/kv_cache/mod.rs:440-455): ring append
+ * plan for a sliding-window layer.  plan = {end, source_start, token_count,
+ * first_slot, first_count, second_count}.  0 ok, -1 invalid. */
+ZLLM_API int zllm_kv_ring_write_plan(uint64_t capacity, uint64_t max_sequence_len, uint64_t position, uint64_t count,
+                            uint64_t plan[6]);
+
+/* ------------------------------------------------------------------------- *
+ * Page appends.                                                              *
+ * ------------------------------------------------------------------------- */
+
+/* Quantize `rows` rows of `cols` values to Q8g64 and scatter them through the
+ * block table at logical tokens [position, position + rows).
+ * Replaces try_paged_cache_append_f32_q8
+ * (src/kernel/rocm/hip/attention/paged_mla.rs:347; kernel
+ * paged_mla/source.hip:164-202) and, with rule METAL_GQA / CUDA_GQA, the GQA
+ * quantizers (kernel/metal/attention/mod.rs:89-128,
+ * kernel/cuda/attention.rs:314-343).  Codes and scale bits are bit-exact with
+ * the rule named. */
+typedef struct zllm_q8_append_args {
+    const void* src;           /* [dev] [rows, cols], src_dtype */
+    int8_t* codes;             /* [dev] codes plane */
+    void* scales;              /* [dev] scales plane (16-bit or f32 per rule) */
+    const uint32_t* table;     /* [dev] block table or NULL (identity) */
+    const uint32_t* positions; /* [dev] optional: positions[0] overrides `position`
+                                  (graph replay; source.hip:787-807) */
+    uint32_t position;         /* first logical token written */
+    uint32_t rows;
+    uint32_t cols;             /* multiple of 64 */
+    uint32_t block_tokens;     /* tokens per page (any value >= 1) */
+    uint32_t ring_capacity;    /* 0, or token -> token % ring_capacity first
+                                  (kernel/cuda/attention.rs:82-88) */
+    int src_dtype;             /* ZLLM_DTYPE_* */
+    int rule;                  /* ZLLM_QUANT_* */
+} zllm_q8_append_args;
+ZLLM_API int zllm_attn_q8g64_append(const zllm_q8_append_args* args, zllm_stream_t stream);
+
+/* f32/bf16/f16 -> bf16 or f16 scatter through the table (unquantized KV).
+ * Replaces try_paged_cache_append_f32_bf16 (paged_mla/source.hip:146-162) and
+ * append_rows_f16 (kernel/cuda/attention.rs:82-88). */
+typedef struct zllm_half_append_args {
+    const void* src;       /* [dev] [rows, cols] */
+    void* cache;           /* [dev] 16-bit plane */
+    const uint32_t* table; /* [dev] or NULL */
+    uint32_t position, rows, cols, block_tokens, ring_capacity;
+    int src_dtype;         /* ZLLM_DTYPE_* */
+    int dst_dtype;         /* ZLLM_DTYPE_BF16 or ZLLM_DTYPE_F16 */
+} zllm_half_append_args;
+ZLLM_API int zllm_attn_half_append(const zllm_half_append_args* args, zllm_stream_t stream);
+
+/* MLA append: quantize the latent (rule ROCM_MLA), optionally rotate the last
+ * `rotary_dim` rope columns, store rope as bf16; one launch.
+ * Replaces try_paged_cache_append_mla_{,rope_}f32_q8_bf16
+ * (src/kernel/rocm/hip/attention/paged_mla.rs:1038-1160; kernel
+ * paged_mla/source.hip:672-785, `_indirect` :787-807). */
+typedef struct zllm_mla_append_args {
+    const float* latent;       /* [dev] [rows, latent_cols] */
+    const float* k_rope;       /* [dev] [rows, rope_cols] */
+    const float* cosine;       /* [dev] [*, rotary_dim / 2] or NULL when rotary_dim == 0 */
+    const float* sine;         /* [dev] */
+    int8_t* latent_codes;      /* [dev] */
+    uint16_t* latent_scales;   /* [dev] bf16 bits */
+    uint16_t* rope_cache;      /* [dev] bf16 bits */
+    const uint32_t* table;     /* [dev] or NULL */
+    const uint32_t* positions; /* [dev] optional {position, rope_position} */
+    uint32_t position;
+    uint32_t rope_position;    /* row of the cos/sin tables for the first token */
+    uint32_t rows, latent_cols, rope_cols, rotary_dim;
+    int rotary_layout;         /* ZLLM_ROTARY_* */
+    uint32_t block_tokens;
+} zllm_mla_append_args;
+ZLLM_API int zllm_attn_mla_append(const zllm_mla_append_args* args, zllm_stream_t stream);
+
+/* Bit-exact gather of plane rows: out[r] = plane[paged_row(first + r)].
+ * Serves KV snapshot download (src/backend/rocm/kv_cache.rs:3344) and is the
+ * page/index gathering check. */
+typedef struct zllm_gather_args {
+    const void* plane;     /* [dev] */
+    void* out;             /* [dev] [count, row_bytes] dense */
+    const uint32_t* table; /* [dev] or NULL */
+    uint32_t first, count, row_bytes, block_tokens, ring_capacity;
+} zllm_gather_args;
+ZLLM_API int zllm_attn_gather_rows(const zllm_gather_args* args, zllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * GQA decode: one query row per sequence, split-KV flash decoding.           *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces try_gqa_decode_cached_f32
+ * (src/kernel/rocm/hip/tensor/attention.rs:1021-1074; kernels
+ * tensor/attention/source.hip:1272-1362), extended to a batch of sequences
+ * over a paged Q8g64 (or f16) cache.  Sequence b attends logical tokens
+ * [first_visible[b], kv_lens[b]) (CausalWindow::key_range of its last row,
+ * src/attention/gqa.rs:54-62).  An empty range yields zeros, never NaN
+ * (gqa.rs:201-204, source.hip:1361). */
+typedef struct zllm_gqa_decode_args {
+    const void* q;                 /* [dev] [batch, num_heads * head_dim], q_dtype */
+    const void* k_plane;           /* [dev] K codes (Q8) or f16 K rows */
+    const void* k_scales;          /* [dev] K scales (Q8 only) */
+    const void* v_plane;           /* [dev] */
+    const void* v_scales;          /* [dev] */
+    const uint32_t* tables;        /* [dev] [batch, table_stride] block tables */
+    const uint32_t* kv_lens;       /* [dev] [batch] */
+    const uint32_t* first_visible; /* [dev] [batch] or NULL (= 0) */
+    float* out;                    /* [dev] [batch, num_heads * head_dim] f32 */
+    void* workspace;               /* [dev] zllm_attn_gqa_decode_workspace_bytes */
+    uint64_t workspace_bytes;
+    uint32_t batch;
+    uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 256} */
+    uint32_t table_stride;         /* entries per sequence in `tables` */
+    uint32_t max_kv_len;           /* host upper bound of kv_lens (sizes the grid) */
+    uint32_t block_tokens;
+    uint32_t ring_capacity;        /* 0 or sliding-window ring rows (token % capacity) */
+    float score_scale;             /* > 0 */
+    float softcap;                 /* 0 = off; else s <- softcap * tanh(s / softcap) */
+    int kv_format;                 /* ZLLM_KV_* */
+    int scale_dtype;               /* ZLLM_SCALE_* (Q8 only) */
+    int q_dtype;                   /* ZLLM_DTYPE_* */
+} zllm_gqa_decode_args;
+ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* args);
+ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * GQA chunked prefill: T query rows appended at `position`.                  *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces try_block_attention_resident_f32 driven with causal ranges
+ * (src/kernel/rocm/hip/tensor/attention.rs:727-798,
+ * src/backend/rocm/attention.rs:2232-2242).  Row r attends logical tokens
+ * key_range(position + r, position + rows) of one sequence whose K/V
+ * (including the chunk's own rows) are already in the paged cache. */
+typedef struct zllm_gqa_prefill_args {
+    const void* q;         /* [dev] [rows, num_heads * head_dim], q_dtype */
+    const void* k_plane;   /* [dev] */
+    const void* k_scales;  /* [dev] */
+    const void* v_plane;   /* [dev] */
+    const void* v_scales;  /* [dev] */
+    const uint32_t* table; /* [dev] block table of the sequence */
+    void* out;             /* [dev] [rows, num_heads * head_dim], out_dtype */
+    void* workspace;       /* [dev] */
+    uint64_t workspace_bytes;
+    uint32_t rows;         /* chunk length T */
+    uint32_t position;     /* tokens already cached before the chunk */
+    uint32_t window;       /* 0 = full causal, else sliding window size */
+    uint32_t num_heads, num_kv_heads, head_dim;
+    uint32_t block_tokens;
+    float score_scale;
+    float softcap;
+    int kv_format, scale_dtype, q_dtype, out_dtype;
+} zllm_gqa_prefill_args;
+ZLLM_API uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* args);
+ZLLM_API int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* args, zllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * MLA absorbed decode over the Q8g64 latent cache.                           *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces try_paged_mla_attention_ct_into for query_rows == 1 per sequence
+ * (src/kernel/rocm/hip/attention/paged_mla.rs:2870-2914, inner :2917-3634):
+ * absorb (q_nope . W_kv_b[h, 0:nope, :] -> bf16) -> split-KV partial -> LSE
+ * merge -> project value (weighted . W_kv_b[h, nope:, :]^T).  Output rows have
+ * stride q_head_dim with only the first value_dim entries of each head slot
+ * written (src/attention/mla.rs:134) when out_compact == 0, or are compact
+ * [batch, heads * value_dim] (src/kernel/cpu/mla.rs:1064-1075) otherwise. */
+typedef struct zllm_mla_decode_args {
+    const void* q;                /* [dev] [batch, heads * q_head_dim], q_dtype */
+    const uint16_t* kv_b;         /* [dev] bf16 bits [heads * kv_head_dim, latent_dim] */
+    const int8_t* latent_codes;   /* [dev] [rows, latent_dim] */
+    const uint16_t* latent_scales;/* [dev] bf16 bits [rows, latent_dim / 64] */
+    const uint16_t* rope_cache;   /* [dev] bf16 bits [rows, rope_dim] */
+    const uint32_t* tables;       /* [dev] [batch, table_stride] */
+    const uint32_t* ctx_lens;     /* [dev] [batch] tokens visible to the query row */
+    void* out;                    /* [dev] out_dtype */
+    void* workspace;              /* [dev] */
+    uint64_t workspace_bytes;
+    uint32_t batch, heads;
+    uint32_t q_head_dim;          /* nope + rope */
+    uint32_t kv_head_dim;         /* nope + value */
+    uint32_t latent_dim;          /* 512 */
+    uint32_t rope_dim;            /* 64 */
+    uint32_t table_stride, max_ctx_len, block_tokens;
+    int q_dtype;                  /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
+    int out_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
+    int out_compact;
+} zllm_mla_decode_args;
+ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
+ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZLLM_ATTN_H */

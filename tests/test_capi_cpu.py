@@ -1,0 +1,103 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every declared symbol, and its host-side
+layout arithmetic reproduces the reference's known answers (no GPU call is made here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from zllm_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(capi.LIB_PATH):
+        from zllm_amd.build import build_library
+
+        build_library()
+    return capi.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "zllm_attn.h")).read()
+    declared = set(re.findall(r"\b(zllm_(?:attn|kv)_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(capi.SYMBOLS), declared ^ set(capi.SYMBOLS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_struct_sizes_follow_the_header():
+    # pointers first, then 32-bit fields: natural alignment, no surprises for an FFI binding
+    assert C.sizeof(capi.Q8AppendArgs) == 5 * 8 + 7 * 4 + 4
+    assert C.sizeof(capi.GqaDecodeArgs) == 10 * 8 + 8 + 8 * 4 + 2 * 4 + 3 * 4 + 4
+    assert C.sizeof(capi.MlaDecodeArgs) == 9 * 8 + 8 + 9 * 4 + 3 * 4
+
+
+def test_key_range_known_answers(lib):
+    # src/attention/gqa.rs:334-339
+    def kr(w, q, e):
+        s, t = C.c_uint64(), C.c_uint64()
+        lib.zllm_attn_key_range(w, q, e, C.byref(s), C.byref(t))
+        return s.value, t.value
+
+    assert kr(3, 4, 5) == (2, 5) and kr(3, 1, 2) == (0, 2) and kr(0, 4, 5) == (0, 5)
+    assert kr(1024, 8191, 8192) == (7168, 8192)
+
+
+def test_layout_known_answers(lib, oracle):
+    # src/kv_cache/mod.rs:615-625, 667-675; src/backend/rocm/kv_cache.rs:3617-3624
+    assert lib.zllm_kv_bytes_per_token(0, 8, 4, 4) == 20
+    assert lib.zllm_kv_bytes_per_token(1, 2, 4, 4) == 24
+    assert lib.zllm_kv_bytes_per_token(0, 512, 64, 64) == 656
+    assert lib.zllm_kv_bytes_per_token(1, 8, 128, 64) == 2112
+    assert lib.zllm_kv_bytes_per_token(0, 8, 4, 3) == 0
+    off = (C.c_uint64 * 5)()
+    assert lib.zllm_kv_layout_offsets(0, 8, 4, 4, 2, 3, 1, off) == 120
+    assert (off[1], off[2], off[3]) == (60, 84, 96)
+    # agrees with the oracle's restatement on a sweep
+    for kind, a, b, g, layers, cap, layer in [(1, 8, 128, 64, 3, 1000, 2), (0, 512, 64, 64, 4, 77, 1), (1, 4, 128, 64, 1, 4096, 0)]:
+        total = lib.zllm_kv_layout_offsets(kind, a, b, g, layers, cap, layer, off)
+        t2, o2 = oracle.layout_offsets(kind, a, b, g, layers, cap, layer)
+        n = 4 if kind == 0 else 5
+        assert total == t2 and list(off)[:n] == [int(v) for v in o2[:n]]
+
+
+def test_ring_plan_known_answers(lib, oracle):
+    plan = (C.c_uint64 * 6)()
+    assert lib.zllm_kv_ring_write_plan(3, 10, 0, 5, plan) == 0
+    assert (plan[1], plan[3], plan[4], plan[5]) == (2, 2, 1, 2)  # src/kv_cache/mod.rs:705-709
+    assert lib.zllm_kv_ring_write_plan(3, 10, 0, 0, plan) == -1
+    assert lib.zllm_kv_ring_write_plan(3, 10, 8, 5, plan) == -1
+    assert b"ring write plan" in lib.zllm_attn_last_error()
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        cap, pos, cnt = int(rng.integers(1, 40)), int(rng.integers(0, 100)), int(rng.integers(1, 60))
+        rc = lib.zllm_kv_ring_write_plan(cap, 200, pos, cnt, plan)
+        ref = oracle.ring_write_plan(cap, 200, pos, cnt)
+        assert (rc == 0) == (ref is not None)
+        if ref:
+            assert list(plan) == [ref[k] for k in ("end", "source_start", "token_count", "first_slot", "first_count", "second_count")]
+
+
+def test_invalid_shapes_are_reported_without_a_gpu(lib):
+    args = capi.GqaDecodeArgs()
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) == 0
+    assert lib.zllm_attn_gqa_decode(C.byref(args), None) == -1
+    assert b"invalid shape" in lib.zllm_attn_last_error()
+    args.batch, args.num_heads, args.num_kv_heads, args.head_dim = 1, 16, 3, 128  # heads % kv_heads != 0
+    assert lib.zllm_attn_gqa_decode(C.byref(args), None) == -1
+    args.num_kv_heads, args.head_dim = 4, 96
+    assert lib.zllm_attn_gqa_decode(C.byref(args), None) == -1
+    args.head_dim, args.block_tokens, args.max_kv_len, args.score_scale = 128, 16, 4096, 0.0
+    assert lib.zllm_attn_gqa_decode(C.byref(args), None) == -1
+    assert b"score_scale" in lib.zllm_attn_last_error()
+    args.score_scale = 0.088
+    args.kv_format, args.scale_dtype, args.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_F32
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) > 0
+    assert lib.zllm_attn_gqa_decode(C.byref(args), None) == -1  # null pointers
+    assert b"null pointer" in lib.zllm_attn_last_error()
+    q8 = capi.Q8AppendArgs()
+    assert lib.zllm_attn_q8g64_append(C.byref(q8), None) == -1

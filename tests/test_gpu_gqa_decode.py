@@ -1,0 +1,223 @@
+"""Parity of the split-KV GQA decode kernels with the CPU oracle, through the C ABI.
+
+Tolerance (stated by the north star): max-abs <= 2e-3 and relative <= 1e-2, fp32 accumulation.
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tests.cases import assert_attention_close, draw_tables, make_gqa_q8_case, oracle_gqa_decode, to_torch_bf16, upload
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_capacity=0):
+    from zllm_amd import capi, ops
+
+    pl = case["planes"]
+    lens = case["lens"]
+    q = to_torch_bf16(case["q_bits"], "cuda") if case["q_bits"] is not None else upload(case["q"])
+    first = None
+    if window:
+        first = upload(np.array([O.key_range(window, int(l) - 1, int(l))[0] if l else 0 for l in lens], dtype=np.uint32))
+    out = ops.gqa_decode(q, upload(pl["k_codes"]), upload(pl["k_scales"]), upload(pl["v_codes"]), upload(pl["v_scales"]),
+                         upload(case["tables"]), upload(lens), case["hq"], case["hkv"], case["d"], case["block_tokens"],
+                         score_scale, max_kv_len or max(int(lens.max()), 1), first_visible=first, softcap=softcap,
+                         ring_capacity=ring_capacity, kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"])
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def test_config1_cpu_oracle_case():
+    """BASELINE config 1: B=1, 16q/4kv, d=128, L=4096, f32 q, f16 scales, 16-token pages, random table."""
+    case = make_gqa_q8_case(1, [4096], 16, 4, 128)
+    scale = 1.0 / np.sqrt(128.0)
+    got = run_decode(case, scale)
+    want = oracle_gqa_decode(case, scale)
+    print("config1", assert_attention_close(got, want, "config 1"))
+
+
+def test_config2_shape_ragged_batch_bf16_queries_outliers():
+    """BASELINE config 2 at oracle-sized lengths: B=8, 64q/8kv, ragged, bf16 q, 1 % outlier channels x8."""
+    rng = np.random.default_rng(2)
+    lens = rng.integers(100, 3000, size=8)
+    case = make_gqa_q8_case(2, lens, 64, 8, 128, outliers=True, q_bf16=True)
+    scale = 1.0 / np.sqrt(128.0)
+    got = run_decode(case, scale)
+    want = oracle_gqa_decode(case, scale)
+    print("config2-small", assert_attention_close(got, want, "config 2 (small)"))
+
+
+@pytest.mark.parametrize("block_tokens,layout", [(1, "random"), (4, "random"), (64, "reversed"), (128, "identity"), (1024, "random"), (48, "random")])
+def test_page_sizes_and_tables(block_tokens, layout):
+    """block_size is a run-time argument in the reference (tests use 1, 4, 64, 128, 1024); 48 is not a power of two."""
+    case = make_gqa_q8_case(block_tokens, [777, 1500], 8, 2, 128, block_tokens=block_tokens, layout=layout)
+    got = run_decode(case, 0.09)
+    want = oracle_gqa_decode(case, 0.09)
+    assert_attention_close(got, want, f"block_tokens={block_tokens}")
+
+
+@pytest.mark.parametrize("lens", [[1], [15, 16, 17], [31, 32, 33, 0], [255, 256, 257, 1023], [0]])
+def test_edge_lengths(lens):
+    case = make_gqa_q8_case(sum(lens) + 3, lens, 16, 4, 128)
+    got = run_decode(case, 0.1, max_kv_len=max(max(lens), 1))
+    want = oracle_gqa_decode(case, 0.1)
+    assert_attention_close(got, want, f"lens={lens}")
+    for b, l in enumerate(lens):
+        if l == 0:
+            assert (got[b] == 0).all()  # nothing visible -> zeros, never NaN
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 8, 128), (32, 1, 128), (40, 2, 128), (12, 3, 128), (8, 2, 64), (8, 2, 256), (64, 16, 128)])
+def test_head_geometries(hq, hkv, d):
+    case = make_gqa_q8_case(hq * 7 + d, [600, 90], hq, hkv, d)
+    got = run_decode(case, 1.0 / np.sqrt(d))
+    want = oracle_gqa_decode(case, 1.0 / np.sqrt(d))
+    assert_attention_close(got, want, f"{hq}/{hkv} d={d}")
+
+
+@pytest.mark.parametrize("rule", [O.RULE_ROCM_MLA, O.RULE_METAL_GQA])
+def test_scale_storage_conventions(rule):
+    case = make_gqa_q8_case(33 + rule, [900], 16, 4, 128, rule=rule)
+    got = run_decode(case, 0.088)
+    want = oracle_gqa_decode(case, 0.088)
+    assert_attention_close(got, want, f"rule={rule}")
+
+
+@pytest.mark.parametrize("window", [1, 100, 1024])
+def test_sliding_window(window):
+    case = make_gqa_q8_case(70 + window, [2100, 50, 1024], 16, 4, 128)
+    got = run_decode(case, 0.088, window=window)
+    want = oracle_gqa_decode(case, 0.088, window=window)
+    assert_attention_close(got, want, f"window={window}")
+
+
+def test_softcap():
+    case = make_gqa_q8_case(81, [1200, 333], 16, 8, 128, q_std=4.0)
+    got = run_decode(case, 0.5, softcap=50.0)
+    want = oracle_gqa_decode(case, 0.5, softcap=50.0)
+    assert_attention_close(got, want, "softcap 50")
+    plain = run_decode(case, 0.5)
+    assert np.abs(plain - got).max() > 1e-4  # the cap changes these logits
+    huge = run_decode(case, 0.5, softcap=1e9)
+    assert_attention_close(huge, oracle_gqa_decode(case, 0.5), "softcap -> inf recovers the uncapped result")
+
+
+def test_zero_query_gives_mean_of_values_and_split_invariance():
+    case = make_gqa_q8_case(90, [5000], 8, 2, 128)
+    case["q"][:] = 0.0
+    got = run_decode(case, 0.1)
+    v = O.gather_dequant_rows(O.FMT_Q8, case["planes"]["v_codes"], case["planes"]["v_scales"], case["scale_dtype"],
+                              case["tables"][0], 16, 0, 5000, 256)
+    mean = v.reshape(5000, 2, 128).mean(0)
+    assert np.abs(got.reshape(8, 128) - np.repeat(mean, 4, axis=0)).max() < 1e-4
+    # any number of KV splits gives the same answer: max_kv_len only changes the split plan
+    case2 = make_gqa_q8_case(91, [5000], 8, 2, 128)
+    a = run_decode(case2, 0.1, max_kv_len=5000)
+    b = run_decode(case2, 0.1, max_kv_len=400000)
+    assert np.abs(a - b).max() < 2e-5
+
+
+def test_dominant_key_returns_its_value_row():
+    case = make_gqa_q8_case(92, [3000], 8, 2, 128)
+    k = O.gather_dequant_rows(O.FMT_Q8, case["planes"]["k_codes"], case["planes"]["k_scales"], case["scale_dtype"],
+                              case["tables"][0], 16, 1234, 1, 256).reshape(2, 128)
+    case["q"][0] = np.repeat(k, 4, axis=0).reshape(-1) * 3.0  # |k|^2 * 3 ~ 380 >> any other logit
+    got = run_decode(case, 1.0)
+    want = oracle_gqa_decode(case, 1.0)
+    assert_attention_close(got, want, "dominant key")
+    v = O.gather_dequant_rows(O.FMT_Q8, case["planes"]["v_codes"], case["planes"]["v_scales"], case["scale_dtype"],
+                              case["tables"][0], 16, 1234, 1, 256).reshape(2, 128)
+    assert np.abs(got.reshape(8, 128) - np.repeat(v, 4, axis=0)).max() < 1e-4
+
+
+def test_large_pool_exercises_64_bit_offsets():
+    """Physical block ids beyond 2^32 bytes of plane offset (the reference casts to u64 for the same reason)."""
+    from zllm_amd import capi, ops
+
+    hq, hkv, d, bt = 16, 8, 128, 16
+    cols = hkv * d
+    pool_rows = (5 << 30) // cols  # 5 GiB codes plane per tensor
+    pool_blocks = pool_rows // bt
+    rng = np.random.default_rng(5)
+    lens = [700]
+    nblk = (lens[0] + bt - 1) // bt
+    table = np.sort(rng.choice(np.arange(pool_blocks - 4096, pool_blocks), size=nblk, replace=False)).astype(np.uint32)[::-1].copy()
+    k = rng.standard_normal((lens[0], cols)).astype(np.float32)
+    v = rng.standard_normal((lens[0], cols)).astype(np.float32)
+    q = rng.standard_normal((1, hq * d)).astype(np.float32)
+    kc = torch.zeros((pool_rows, cols), dtype=torch.int8, device="cuda")
+    vc = torch.zeros((pool_rows, cols), dtype=torch.int8, device="cuda")
+    ks = torch.zeros((pool_rows, cols // 64), dtype=torch.int16, device="cuda")
+    vs = torch.zeros((pool_rows, cols // 64), dtype=torch.int16, device="cuda")
+    tbl = upload(table)
+    ops.q8g64_append(upload(k), kc, ks, tbl, 0, bt, capi.QUANT_METAL_GQA)
+    ops.q8g64_append(upload(v), vc, vs, tbl, 0, bt, capi.QUANT_METAL_GQA)
+    out = ops.gqa_decode(upload(q), kc, ks, vc, vs, tbl.view(1, -1), upload(np.array(lens, dtype=np.uint32)), hq, hkv, d, bt,
+                         0.088, lens[0]).cpu().numpy()
+    # oracle on a compact identity pool built from the same rows
+    codes = np.zeros((nblk * bt, cols), dtype=np.int8)
+    kscale = np.zeros((nblk * bt, cols // 64), dtype=np.uint16)
+    vcodes, vscale = codes.copy(), kscale.copy()
+    O.q8g64_append_paged(O.RULE_METAL_GQA, k, codes, kscale, None, 0, bt)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, vcodes, vscale, None, 0, bt)
+    # the appended device bytes are the oracle's bytes (gathered back through the far table)
+    got_rows = ops.gather_rows(kc, tbl, 0, lens[0], cols, bt).cpu().numpy()
+    assert np.array_equal(got_rows.view(np.int8), codes[: lens[0]])
+    kd = O.gather_dequant_rows(O.FMT_Q8, codes, kscale, O.SCALE_F16, None, bt, 0, lens[0], cols)
+    vd = O.gather_dequant_rows(O.FMT_Q8, vcodes, vscale, O.SCALE_F16, None, bt, 0, lens[0], cols)
+    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, lens[0], lens[0] - 1, hq, hkv, d, score_scale=0.088)
+    assert rc == 0
+    assert_attention_close(out, want, "far pool")
+
+
+# ---------------------------------------------------------------------------- f16 KV (config 3)
+def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0):
+    rng = np.random.default_rng(seed)
+    cols = hkv * d
+    cap_lens = [min(l, ring_capacity) if ring_capacity else l for l in lens]
+    tables, pool_blocks = draw_tables(rng, cap_lens, block_tokens)
+    rows = pool_blocks * block_tokens
+    planes = {"k": np.zeros((rows, cols), dtype=np.uint16), "v": np.zeros((rows, cols), dtype=np.uint16)}
+    for b, l in enumerate(lens):
+        k = rng.standard_normal((l, cols)).astype(np.float32)
+        v = rng.standard_normal((l, cols)).astype(np.float32)
+        O.half_append_paged(1, k, planes["k"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
+        O.half_append_paged(1, v, planes["v"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
+    q = rng.standard_normal((len(lens), hq * d)).astype(np.float32)
+    return dict(q=q, q_bits=None, lens=np.array(lens, dtype=np.uint32), tables=tables, planes=planes, hq=hq, hkv=hkv, d=d,
+                block_tokens=block_tokens, scale_dtype=0)
+
+
+def run_f16(case, score_scale, window=0, softcap=0.0, ring_capacity=0):
+    from zllm_amd import capi, ops
+
+    lens = case["lens"]
+    first = None
+    if window:
+        first = upload(np.array([O.key_range(window, int(l) - 1, int(l))[0] for l in lens], dtype=np.uint32))
+    out = ops.gqa_decode(upload(case["q"]), upload(case["planes"]["k"]), None, upload(case["planes"]["v"]), None,
+                         upload(case["tables"]), upload(lens), case["hq"], case["hkv"], case["d"], case["block_tokens"],
+                         score_scale, int(lens.max()), first_visible=first, softcap=softcap, ring_capacity=ring_capacity,
+                         kv_format=capi.KV_F16)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("window,ring", [(0, 0), (1024, 0), (1024, 1024)])
+def test_config3_f16_kv_sliding_window_softcap(window, ring):
+    """BASELINE config 3: B=4, 16q/8kv, d=256, ctx 8192, window 1024 on sliding layers (optionally stored as a
+    1024-row ring), soft-cap 50."""
+    case = make_f16_case(3, [8192, 8192, 5000, 8192], 16, 8, 256, ring_capacity=ring)
+    scale = 1.0 / 16.0
+    got = run_f16(case, scale, window=window, softcap=50.0, ring_capacity=ring)
+    want = oracle_gqa_decode(case, scale, window=window, softcap=50.0, fmt=O.FMT_F16, ring_capacity=ring)
+    print("config3", window, ring, assert_attention_close(got, want, f"config 3 window={window} ring={ring}"))
+
+
+def test_f16_kv_head_dim_128():
+    case = make_f16_case(4, [333, 1000], 8, 2, 128, block_tokens=64)
+    got = run_f16(case, 0.088)
+    want = oracle_gqa_decode(case, 0.088, fmt=O.FMT_F16)
+    assert_attention_close(got, want, "f16 d=128")

@@ -1,0 +1,50 @@
+"""Builds libzllm_attn.so (the C-ABI library) for gfx950 with hipcc, in-tree."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libzllm_attn.so")
+SOURCES = ["api.hip", "append.hip", "gqa_decode.hip", "mla_decode.hip", "gqa_prefill.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fvisibility=hidden",
+    # packed-FP32 VALU forms are kept out of all device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-Wno-unknown-warning-option",
+]
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    result = subprocess.run(cmd, capture_output=True, text=True)
+    if result.returncode != 0:
+        sys.stderr.write(result.stdout + result.stderr)
+        raise RuntimeError(f"hipcc failed on {src}")
+    noise = "'-packed-fp32-ops' is not a recognized feature"
+    for line in result.stderr.splitlines():
+        if line.strip() and noise not in line and "warning generated" not in line and "warnings generated" not in line:
+            sys.stderr.write(line + "\n")
+    return obj
+
+
+def build_library(jobs: int = 4) -> str:
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objects = list(pool.map(_compile, SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objects]
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library())

@@ -1,0 +1,347 @@
+// C ABI of the attention hot path: argument validation, workspace carving, launches.
+// Nothing here allocates, frees or synchronises.
+#include "../../include/zllm_attn.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "kernels.hpp"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* format, ...)
+{
+    va_list args;
+    va_start(args, format);
+    vsnprintf(g_error, sizeof(g_error), format, args);
+    va_end(args);
+    return code;
+}
+
+int hip_status(hipError_t err, const char* what)
+{
+    if (err == hipSuccess) {
+        return 0;
+    }
+    snprintf(g_error, sizeof(g_error), "%s: %s", what, hipGetErrorString(err));
+    return (int)err;
+}
+
+constexpr unsigned int kComputeUnits = 256; // MI355X
+
+unsigned int shift_of(unsigned int block_tokens)
+{
+    unsigned int shift = 0;
+    while ((1u << shift) < block_tokens) {
+        ++shift;
+    }
+    return shift;
+}
+
+uint64_t align_up(uint64_t value, uint64_t to)
+{
+    return (value + to - 1) / to * to;
+}
+
+bool valid_head_dim(uint32_t d)
+{
+    return d == 64 || d == 128 || d == 256;
+}
+
+// Tokens per KV split: enough workgroups to occupy every CU about twice, but
+// splits long enough that the partial write / merge stay a few percent of the
+// KV bytes a split reads.
+void plan_splits(uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    const uint64_t target = 2ull * kComputeUnits;
+    uint64_t chunk = ((uint64_t)max_len * columns + target - 1) / target;
+    chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
+    *chunk_tokens = (uint32_t)chunk;
+    const uint64_t chunks = ((uint64_t)max_len + chunk - 1) / chunk;
+    *max_chunks = (uint32_t)(chunks == 0 ? 1 : chunks);
+}
+
+int validate_gqa_decode(const zllm_gqa_decode_args* a)
+{
+    if (a == nullptr) {
+        return fail(-1, "GQA decode: null args");
+    }
+    // shape rules of try_gqa_decode_cached_f32 (tensor/attention.rs:1022-1024)
+    if (a->batch == 0 || a->num_heads == 0 || a->num_kv_heads == 0 || a->num_heads % a->num_kv_heads != 0 ||
+        !valid_head_dim(a->head_dim)) {
+        return fail(-1, "GQA decode: invalid shape batch=%u heads=%u/%u dim=%u", a->batch, a->num_heads, a->num_kv_heads, a->head_dim);
+    }
+    if (a->block_tokens == 0 || a->max_kv_len == 0) {
+        return fail(-1, "GQA decode: block_tokens=%u max_kv_len=%u must be non-zero", a->block_tokens, a->max_kv_len);
+    }
+    if (!isfinite(a->score_scale) || a->score_scale <= 0.0f || !(a->softcap >= 0.0f) || !isfinite(a->softcap)) {
+        return fail(-1, "GQA decode: invalid score_scale=%g softcap=%g", (double)a->score_scale, (double)a->softcap);
+    }
+    if (a->kv_format != ZLLM_KV_Q8G64 && a->kv_format != ZLLM_KV_F16) {
+        return fail(-1, "GQA decode: unknown kv_format %d", a->kv_format);
+    }
+    if (a->kv_format == ZLLM_KV_Q8G64 && a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
+        return fail(-1, "GQA decode: Q8g64 scales must be bf16 or f16 (got %d)", a->scale_dtype);
+    }
+    if (a->kv_format == ZLLM_KV_F16 && a->head_dim == 64) {
+        return fail(-1, "GQA decode: f16 KV supports head_dim 128 and 256");
+    }
+    if (a->q_dtype < ZLLM_DTYPE_F32 || a->q_dtype > ZLLM_DTYPE_F16) {
+        return fail(-1, "GQA decode: unknown q_dtype %d", a->q_dtype);
+    }
+    return 0;
+}
+
+void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    const uint32_t max_waves = a->head_dim > 128 ? 4u : 8u;
+    const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
+    const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
+    const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
+    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, chunk_tokens, max_chunks);
+}
+
+} // namespace
+
+extern "C" {
+
+int zllm_attn_init(int device, int* cu_count)
+{
+    hipDeviceProp_t prop;
+    hipError_t err = hipGetDeviceProperties(&prop, device);
+    if (err != hipSuccess) {
+        return hip_status(err, "hipGetDeviceProperties");
+    }
+    if (cu_count != nullptr) {
+        *cu_count = prop.multiProcessorCount;
+    }
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        return fail(-2, "zllm_attn is built for gfx950 only; device %d is %s", device, prop.gcnArchName);
+    }
+    return 0;
+}
+
+const char* zllm_attn_last_error(void)
+{
+    return g_error;
+}
+
+/* ---- host layout arithmetic ------------------------------------------------------------- */
+
+void zllm_attn_key_range(uint64_t window, uint64_t query_position, uint64_t key_end, uint64_t* start, uint64_t* end)
+{
+    uint64_t causal_end = query_position + 1 < key_end ? query_position + 1 : key_end;
+    uint64_t s = 0;
+    if (window != 0) {
+        s = query_position + 1 > window ? query_position + 1 - window : 0;
+    }
+    *start = s < causal_end ? s : causal_end;
+    *end = causal_end;
+}
+
+uint64_t zllm_kv_bytes_per_token(int kind, uint64_t a, uint64_t b, uint64_t group)
+{
+    if (group == 0) {
+        return 0;
+    }
+    if (kind == 0) {
+        if (a == 0 || b == 0 || a % group != 0) {
+            return 0;
+        }
+        return a + (a / group) * 2 + b * 2;
+    }
+    if (a == 0 || b == 0 || b % group != 0) {
+        return 0;
+    }
+    return 2 * (a * b) + 4 * (a * (b / group));
+}
+
+uint64_t zllm_kv_layout_offsets(int kind, uint64_t a, uint64_t b, uint64_t group, uint64_t layer_count, uint64_t capacity,
+                                uint64_t layer, uint64_t offsets[5])
+{
+    const uint64_t per_token = zllm_kv_bytes_per_token(kind, a, b, group);
+    if (per_token == 0 || capacity == 0 || layer_count == 0 || layer >= layer_count) {
+        return 0;
+    }
+    const uint64_t stride = capacity * per_token;
+    const uint64_t base = layer * stride;
+    offsets[0] = base;
+    if (kind == 0) {
+        const uint64_t codes = capacity * a;
+        const uint64_t scales = capacity * (a / group) * 2;
+        offsets[1] = base;
+        offsets[2] = base + codes;
+        offsets[3] = base + codes + scales;
+        offsets[4] = 0;
+    } else {
+        const uint64_t codes = capacity * a * b;
+        const uint64_t scales = capacity * a * (b / group) * 2;
+        offsets[1] = base;
+        offsets[2] = base + codes;
+        offsets[3] = base + codes + scales;
+        offsets[4] = base + 2 * codes + scales;
+    }
+    return layer_count * stride;
+}
+
+int zllm_kv_ring_write_plan(uint64_t capacity, uint64_t max_sequence_len, uint64_t position, uint64_t count, uint64_t plan[6])
+{
+    if (count == 0 || capacity == 0 || position + count > max_sequence_len) {
+        return fail(-1, "ring write plan: capacity=%llu position=%llu count=%llu max=%llu", (unsigned long long)capacity,
+                    (unsigned long long)position, (unsigned long long)count, (unsigned long long)max_sequence_len);
+    }
+    const uint64_t end = position + count;
+    const uint64_t oldest_kept = end > capacity ? end - capacity : 0;
+    const uint64_t write_start = position > oldest_kept ? position : oldest_kept;
+    const uint64_t tokens = end - write_start;
+    const uint64_t first_slot = write_start % capacity;
+    const uint64_t first_count = tokens < capacity - first_slot ? tokens : capacity - first_slot;
+    plan[0] = end;
+    plan[1] = write_start - position;
+    plan[2] = tokens;
+    plan[3] = first_slot;
+    plan[4] = first_count;
+    plan[5] = tokens - first_count;
+    return 0;
+}
+
+/* ---- appends ---------------------------------------------------------------------------- */
+
+int zllm_attn_q8g64_append(const zllm_q8_append_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->src == nullptr || a->codes == nullptr || a->scales == nullptr) {
+        return fail(-1, "Q8g64 append: null pointer");
+    }
+    if (a->cols == 0 || a->cols % ZLLM_GROUP_SIZE != 0 || a->block_tokens == 0) {
+        return fail(-1, "Q8g64 append: cols=%u must be a non-zero multiple of 64, block_tokens=%u non-zero", a->cols, a->block_tokens);
+    }
+    if (a->rule < ZLLM_QUANT_ROCM_MLA || a->rule > ZLLM_QUANT_CUDA_GQA || a->src_dtype < ZLLM_DTYPE_F32 || a->src_dtype > ZLLM_DTYPE_F16) {
+        return fail(-1, "Q8g64 append: unknown rule %d or src_dtype %d", a->rule, a->src_dtype);
+    }
+    if ((uint64_t)a->position + a->rows > 0xffffffffull) {
+        return fail(-1, "Q8g64 append: position + rows overflows u32");
+    }
+    zllm::Q8AppendParams p{a->src, (signed char*)a->codes, a->scales, a->table, a->positions, a->position, a->rows, a->cols,
+                           a->block_tokens, a->ring_capacity, a->src_dtype, a->rule};
+    return hip_status(zllm::launch_q8g64_append(p, (hipStream_t)stream), "Q8g64 append launch");
+}
+
+int zllm_attn_half_append(const zllm_half_append_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->src == nullptr || a->cache == nullptr) {
+        return fail(-1, "half append: null pointer");
+    }
+    if (a->cols == 0 || a->block_tokens == 0) {
+        return fail(-1, "half append: cols and block_tokens must be non-zero");
+    }
+    if (a->dst_dtype != ZLLM_DTYPE_BF16 && a->dst_dtype != ZLLM_DTYPE_F16) {
+        return fail(-1, "half append: dst_dtype must be bf16 or f16");
+    }
+    if (a->src_dtype < ZLLM_DTYPE_F32 || a->src_dtype > ZLLM_DTYPE_F16) {
+        return fail(-1, "half append: unknown src_dtype %d", a->src_dtype);
+    }
+    zllm::HalfAppendParams p{a->src, (unsigned short*)a->cache, a->table, a->position, a->rows, a->cols, a->block_tokens,
+                             a->ring_capacity, a->src_dtype, a->dst_dtype};
+    return hip_status(zllm::launch_half_append(p, (hipStream_t)stream), "half append launch");
+}
+
+int zllm_attn_mla_append(const zllm_mla_append_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->latent == nullptr || a->k_rope == nullptr || a->latent_codes == nullptr || a->latent_scales == nullptr ||
+        a->rope_cache == nullptr) {
+        return fail(-1, "MLA append: null pointer");
+    }
+    if (a->latent_cols == 0 || a->latent_cols % ZLLM_GROUP_SIZE != 0 || a->rope_cols == 0 || a->block_tokens == 0) {
+        return fail(-1, "MLA append: latent_cols=%u (multiple of 64) rope_cols=%u block_tokens=%u", a->latent_cols, a->rope_cols,
+                    a->block_tokens);
+    }
+    if (a->rotary_dim > a->rope_cols || a->rotary_dim % 2 != 0 || (a->rotary_dim != 0 && (a->cosine == nullptr || a->sine == nullptr))) {
+        return fail(-1, "MLA append: rotary_dim=%u invalid for rope_cols=%u (or missing cos/sin)", a->rotary_dim, a->rope_cols);
+    }
+    if (a->rotary_layout != ZLLM_ROTARY_INTERLEAVED && a->rotary_layout != ZLLM_ROTARY_SPLIT_HALF) {
+        return fail(-1, "MLA append: unknown rotary layout %d", a->rotary_layout);
+    }
+    zllm::MlaAppendParams p{a->latent, a->k_rope, a->cosine, a->sine, (signed char*)a->latent_codes, a->latent_scales, a->rope_cache,
+                            a->table, a->positions, a->position, a->rope_position, a->rows, a->latent_cols, a->rope_cols,
+                            a->rotary_dim, a->rotary_layout == ZLLM_ROTARY_SPLIT_HALF ? 1u : 0u, a->block_tokens};
+    return hip_status(zllm::launch_mla_append(p, (hipStream_t)stream), "MLA append launch");
+}
+
+int zllm_attn_gather_rows(const zllm_gather_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->plane == nullptr || a->out == nullptr) {
+        return fail(-1, "gather rows: null pointer");
+    }
+    if (a->block_tokens == 0) {
+        return fail(-1, "gather rows: block_tokens must be non-zero");
+    }
+    zllm::GatherParams p{a->plane, a->out, a->table, a->first, a->count, a->row_bytes, a->block_tokens, a->ring_capacity};
+    return hip_status(zllm::launch_gather_rows(p, (hipStream_t)stream), "gather rows launch");
+}
+
+/* ---- GQA decode ------------------------------------------------------------------------- */
+
+uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* a)
+{
+    if (validate_gqa_decode(a) != 0) {
+        return 0;
+    }
+    uint32_t chunk_tokens, max_chunks;
+    plan_gqa_decode(a, &chunk_tokens, &max_chunks);
+    const uint64_t rows = (uint64_t)a->batch * max_chunks * a->num_heads;
+    return align_up(rows * a->head_dim * 4, 256) + align_up(rows * 8, 256);
+}
+
+int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
+{
+    const int rc = validate_gqa_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    if (a->q == nullptr || a->k_plane == nullptr || a->v_plane == nullptr || a->kv_lens == nullptr || a->out == nullptr ||
+        a->workspace == nullptr || (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
+        return fail(-1, "GQA decode: null pointer");
+    }
+    const uint64_t need = zllm_attn_gqa_decode_workspace_bytes(a);
+    if (a->workspace_bytes < need) {
+        return fail(-1, "GQA decode: workspace %llu bytes, need %llu", (unsigned long long)a->workspace_bytes, (unsigned long long)need);
+    }
+    if (a->tables != nullptr && (uint64_t)a->table_stride * a->block_tokens < a->max_kv_len && a->ring_capacity == 0) {
+        return fail(-1, "GQA decode: table_stride=%u pages of %u tokens cannot cover max_kv_len=%u", a->table_stride, a->block_tokens,
+                    a->max_kv_len);
+    }
+    zllm::GqaDecodeParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q;
+    p.k_plane = (const unsigned char*)a->k_plane;
+    p.k_scales = (const unsigned char*)a->k_scales;
+    p.v_plane = (const unsigned char*)a->v_plane;
+    p.v_scales = (const unsigned char*)a->v_scales;
+    p.tables = a->tables;
+    p.kv_lens = a->kv_lens;
+    p.first_visible = a->first_visible;
+    p.out = a->out;
+    plan_gqa_decode(a, &p.chunk_tokens, &p.max_chunks);
+    const uint64_t rows = (uint64_t)a->batch * p.max_chunks * a->num_heads;
+    p.partial = (float*)a->workspace;
+    p.stats = (float*)((char*)a->workspace + align_up(rows * a->head_dim * 4, 256));
+    p.batch = a->batch;
+    p.num_heads = a->num_heads;
+    p.num_kv_heads = a->num_kv_heads;
+    p.head_dim = a->head_dim;
+    p.group = a->num_heads / a->num_kv_heads;
+    p.table_stride = a->table_stride;
+    p.block_tokens = a->block_tokens;
+    p.block_shift = shift_of(a->block_tokens);
+    p.ring_capacity = a->ring_capacity;
+    p.score_scale = a->score_scale;
+    p.softcap = a->softcap;
+    p.q_dtype = a->q_dtype;
+    return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA decode launch");
+}
+
+} // extern "C"

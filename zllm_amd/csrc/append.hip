@@ -1,0 +1,200 @@
+// Page appends: Q8g64 quantize + scatter, 16-bit scatter, fused MLA append, row gather.
+//
+// One wave64 owns one 64-element quantization group, so the group absmax is a
+// wave reduction (max is order-independent, hence bit-exact with the reference's
+// tree reduction, src/kernel/rocm/hip/attention/paged_mla/source.hip:175-181).
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace zllm {
+
+__device__ __forceinline__ float wave_max_all(float v)
+{
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, offset));
+    }
+    return v;
+}
+
+// Quantize one value of a 64-group held one-per-lane; returns the code and
+// writes the scale slot from lane 0.
+//   rule 0 (paged_mla/source.hip:183-201): scale = absmax * (1/127), stored
+//          bf16, code = nearbyint(x / f32(stored)).
+//   rule 1 (kernel/metal/attention/mod.rs:114-127): scale = absmax / 127,
+//          stored f16, code = rint(x * (1 / scale)).
+//   rule 2 (kernel/cuda/attention.rs:331-341): as rule 1, stored f32.
+__device__ __forceinline__ signed char quantize_lane(float value, int rule, void* scales, unsigned long long scale_index,
+                                                     unsigned int lane)
+{
+    const float maximum = wave_max_all(fabsf(value));
+    float quantized;
+    if (rule == 0) {
+        const float scale = maximum == 0.0f ? 1.0f : __fmul_rn(maximum, 1.0f / 127.0f);
+        const unsigned short encoded = f32_to_bf16_bits(scale);
+        if (lane == 0) {
+            ((unsigned short*)scales)[scale_index] = encoded;
+        }
+        quantized = nearbyintf(__fdiv_rn(value, bf16_bits_to_f32(encoded)));
+    } else {
+        const float scale = maximum > 0.0f ? __fdiv_rn(maximum, 127.0f) : 1.0f;
+        if (lane == 0) {
+            if (rule == 1) {
+                ((unsigned short*)scales)[scale_index] = f32_to_f16_bits(scale);
+            } else {
+                ((float*)scales)[scale_index] = scale;
+            }
+        }
+        const float inverse = __fdiv_rn(1.0f, scale);
+        quantized = rintf(__fmul_rn(value, inverse));
+    }
+    return (signed char)fmaxf(-127.0f, fminf(127.0f, quantized));
+}
+
+__global__ __launch_bounds__(256) void q8g64_append_kernel(Q8AppendParams p)
+{
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int groups_per_row = p.cols / 64u;
+    const unsigned long long group_index = (unsigned long long)blockIdx.x * 4u + (threadIdx.x >> 6);
+    const unsigned long long total_groups = (unsigned long long)p.rows * groups_per_row;
+    if (group_index >= total_groups) {
+        return;
+    }
+    const unsigned int row = (unsigned int)(group_index / groups_per_row);
+    const unsigned int group = (unsigned int)(group_index - (unsigned long long)row * groups_per_row);
+    const unsigned int column = group * 64u + lane;
+    const unsigned int position = p.positions != nullptr ? p.positions[0] : p.position;
+    const float value = load_as_f32(p.src, (size_t)row * p.cols + column, p.src_dtype);
+    const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, p.ring_capacity);
+    const signed char code = quantize_lane(value, p.rule, p.scales, physical * groups_per_row + group, lane);
+    p.codes[physical * p.cols + column] = code;
+}
+
+__global__ __launch_bounds__(256) void half_append_kernel(HalfAppendParams p)
+{
+    const unsigned long long index = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned long long elements = (unsigned long long)p.rows * p.cols;
+    if (index >= elements) {
+        return;
+    }
+    const unsigned int row = (unsigned int)(index / p.cols);
+    const unsigned int column = (unsigned int)(index - (unsigned long long)row * p.cols);
+    const unsigned long long physical = paged_row(p.table, p.position + row, p.block_tokens, p.ring_capacity);
+    const float value = load_as_f32(p.src, index, p.src_dtype);
+    p.cache[physical * p.cols + column] = p.dst_dtype == 1 ? f32_to_bf16_bits(value) : f32_to_f16_bits(value);
+}
+
+// Fused MLA append (semantics of paged_cache_append_mla_body,
+// paged_mla/source.hip:672-758): blocks [0, rows * groups) quantize the latent,
+// the remaining blocks rotate and store k_rope as bf16.  The rotation uses
+// separately rounded products (no fused multiply-add) so results do not depend
+// on the compiler's contraction choices.
+__global__ __launch_bounds__(64) void mla_append_kernel(MlaAppendParams p)
+{
+    const unsigned int lane = threadIdx.x;
+    const unsigned int groups_per_row = p.latent_cols / 64u;
+    const unsigned int latent_groups = p.rows * groups_per_row;
+    const unsigned int position = p.positions != nullptr ? p.positions[0] : p.position;
+    const unsigned int rope_position = p.positions != nullptr ? p.positions[1] : p.rope_position;
+    if (blockIdx.x >= latent_groups) {
+        const unsigned long long rope_index = (unsigned long long)(blockIdx.x - latent_groups) * 64u + lane;
+        const unsigned long long rope_elements = (unsigned long long)p.rows * p.rope_cols;
+        if (rope_index >= rope_elements) {
+            return;
+        }
+        const unsigned int row = (unsigned int)(rope_index / p.rope_cols);
+        const unsigned int column = (unsigned int)(rope_index - (unsigned long long)row * p.rope_cols);
+        const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, 0);
+        float value = p.k_rope[rope_index];
+        if (p.rotary_dim != 0 && column >= p.rope_cols - p.rotary_dim) {
+            const unsigned int start = p.rope_cols - p.rotary_dim;
+            const unsigned int rotary = column - start;
+            const unsigned int half = p.rotary_dim / 2;
+            const unsigned int pair = p.split_half ? rotary % half : rotary / 2;
+            const unsigned int real_column = p.split_half ? start + pair : start + pair * 2;
+            const unsigned int imag_column = p.split_half ? start + half + pair : real_column + 1;
+            const float real = p.k_rope[(unsigned long long)row * p.rope_cols + real_column];
+            const float imaginary = p.k_rope[(unsigned long long)row * p.rope_cols + imag_column];
+            const float c = p.cosine[(unsigned long long)(rope_position + row) * half + pair];
+            const float s = p.sine[(unsigned long long)(rope_position + row) * half + pair];
+            value = column == real_column ? __fsub_rn(__fmul_rn(real, c), __fmul_rn(imaginary, s))
+                                          : __fadd_rn(__fmul_rn(imaginary, c), __fmul_rn(real, s));
+        }
+        p.rope_cache[physical * p.rope_cols + column] = f32_to_bf16_bits(value);
+        return;
+    }
+    const unsigned int row = blockIdx.x / groups_per_row;
+    const unsigned int group = blockIdx.x - row * groups_per_row;
+    const unsigned int column = group * 64u + lane;
+    const float value = p.latent[(unsigned long long)row * p.latent_cols + column];
+    const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, 0);
+    const signed char code = quantize_lane(value, 0, p.latent_scales, physical * groups_per_row + group, lane);
+    p.latent_codes[physical * p.latent_cols + column] = code;
+}
+
+template <typename T> __global__ __launch_bounds__(256) void gather_rows_kernel(GatherParams p, unsigned int units_per_row)
+{
+    const unsigned long long index = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned long long total = (unsigned long long)p.count * units_per_row;
+    if (index >= total) {
+        return;
+    }
+    const unsigned int row = (unsigned int)(index / units_per_row);
+    const unsigned int unit = (unsigned int)(index - (unsigned long long)row * units_per_row);
+    const unsigned long long physical = paged_row(p.table, p.first + row, p.block_tokens, p.ring_capacity);
+    ((T*)p.out)[index] = ((const T*)p.plane)[physical * units_per_row + unit];
+}
+
+hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream)
+{
+    const unsigned long long groups = (unsigned long long)p.rows * (p.cols / 64u);
+    if (groups == 0) {
+        return hipSuccess;
+    }
+    q8g64_append_kernel<<<dim3((unsigned int)((groups + 3) / 4)), dim3(256), 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream)
+{
+    const unsigned long long elements = (unsigned long long)p.rows * p.cols;
+    if (elements == 0) {
+        return hipSuccess;
+    }
+    half_append_kernel<<<dim3((unsigned int)((elements + 255) / 256)), dim3(256), 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream)
+{
+    const unsigned long long latent_groups = (unsigned long long)p.rows * (p.latent_cols / 64u);
+    const unsigned long long rope_blocks = ((unsigned long long)p.rows * p.rope_cols + 63) / 64;
+    if (latent_groups + rope_blocks == 0) {
+        return hipSuccess;
+    }
+    mla_append_kernel<<<dim3((unsigned int)(latent_groups + rope_blocks)), dim3(64), 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream)
+{
+    if (p.count == 0 || p.row_bytes == 0) {
+        return hipSuccess;
+    }
+    const bool aligned16 = p.row_bytes % 16 == 0 && ((uintptr_t)p.plane % 16 == 0) && ((uintptr_t)p.out % 16 == 0);
+    const bool aligned4 = p.row_bytes % 4 == 0 && ((uintptr_t)p.plane % 4 == 0) && ((uintptr_t)p.out % 4 == 0);
+    const unsigned int unit = aligned16 ? 16 : (aligned4 ? 4 : 1);
+    const unsigned int units_per_row = p.row_bytes / unit;
+    const unsigned long long total = (unsigned long long)p.count * units_per_row;
+    const dim3 grid((unsigned int)((total + 255) / 256));
+    if (unit == 16) {
+        gather_rows_kernel<uint4><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    } else if (unit == 4) {
+        gather_rows_kernel<unsigned int><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    } else {
+        gather_rows_kernel<unsigned char><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    }
+    return hipGetLastError();
+}
+
+} // namespace zllm

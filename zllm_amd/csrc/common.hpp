@@ -1,0 +1,117 @@
+// Shared device helpers for the gfx950 attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace zllm {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr float kNegInf = -__builtin_inff();
+
+// bf16 <-> f32, bit-compatible with zllm_bf16_to_f32 / zllm_f32_to_bf16
+// (src/kernel/rocm/hip/hiprtc.rs:62-75): round-to-nearest-even by adding
+// 0x7fff + lsb, NaN not special-cased.
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned short v)
+{
+    return __uint_as_float(((unsigned int)v) << 16);
+}
+
+__device__ __forceinline__ unsigned short f32_to_bf16_bits(float value)
+{
+    const unsigned int bits = __float_as_uint(value);
+    const unsigned int rounding = 0x7fffu + ((bits >> 16) & 1u);
+    return (unsigned short)((bits + rounding) >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(unsigned short v)
+{
+    union {
+        unsigned short u;
+        _Float16 h;
+    } c;
+    c.u = v;
+    return (float)c.h;
+}
+
+__device__ __forceinline__ unsigned short f32_to_f16_bits(float value)
+{
+    union {
+        unsigned short u;
+        _Float16 h;
+    } c;
+    c.h = (_Float16)value; // v_cvt_f16_f32: IEEE round-to-nearest-even
+    return c.u;
+}
+
+// Stored scale -> f32; numbering of zllm_scale (hiprtc.rs:104-116).
+template <int SCALE_DTYPE> __device__ __forceinline__ float scale_bits_to_f32(unsigned short v)
+{
+    if constexpr (SCALE_DTYPE == 0) {
+        return bf16_bits_to_f32(v);
+    } else {
+        return f16_bits_to_f32(v);
+    }
+}
+
+__device__ __forceinline__ float load_as_f32(const void* base, size_t index, int dtype)
+{
+    if (dtype == 0) {
+        return ((const float*)base)[index];
+    }
+    if (dtype == 1) {
+        return bf16_bits_to_f32(((const unsigned short*)base)[index]);
+    }
+    return f16_bits_to_f32(((const unsigned short*)base)[index]);
+}
+
+// Logical token -> physical cache row
+// (src/kernel/rocm/hip/attention/paged_mla/source.hip:46-54), with the optional
+// sliding-window ring applied first (src/kernel/cuda/attention.rs:82-88).
+__device__ __forceinline__ unsigned long long paged_row(const unsigned int* table, unsigned int token,
+                                                        unsigned int block_tokens, unsigned int ring_capacity)
+{
+    if (ring_capacity != 0) {
+        token %= ring_capacity;
+    }
+    if (table == nullptr) {
+        return token;
+    }
+    return (unsigned long long)table[token / block_tokens] * block_tokens + token % block_tokens;
+}
+
+// Two f32 -> packed bf16x2 (low half = a).  Truncation is exact for the small
+// integers (|x| <= 255) it is used on.
+__device__ __forceinline__ unsigned int pack_bf16_trunc(float lo, float hi)
+{
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+// Two f32 -> packed bf16x2 with round-to-nearest-even.
+__device__ __forceinline__ unsigned int pack_bf16_rne(float lo, float hi)
+{
+    return (unsigned int)f32_to_bf16_bits(lo) | ((unsigned int)f32_to_bf16_bits(hi) << 16);
+}
+
+__device__ __forceinline__ float wave_max_16x4(float v)
+{
+    // reduce across the four 16-lane groups of a wave (lanes l, l^16, l^32, l^48)
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum_16x4(float v)
+{
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+} // namespace zllm

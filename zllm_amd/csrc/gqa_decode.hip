@@ -1,0 +1,710 @@
+// GQA split-KV flash decoding over a paged Q8g64 (or f16) KV cache — gfx950.
+//
+// Work decomposition
+//   grid = (split, kv-head block x head block, sequence); one wave64 per KV head.
+//   The waves of a workgroup cover neighbouring KV heads of the SAME tokens, so
+//   together they read whole cache rows (all KV heads of a token are contiguous:
+//   row = num_kv_heads * head_dim bytes) and share the row's scale line.
+//   Waves never synchronise with each other.
+//
+// Per wave, per 32-token step (two 16-token tiles):
+//   S^T[token, head] = K[token, :] . Q[head, :]      MFMA 16x16x32 bf16, A = K codes
+//                                                    (exact in bf16), B = Q (bf16 hi [+ lo])
+//     one accumulator per 64-column scale group, so the group scale is applied to
+//     the finished partial dot: s = sum_g scale_g * dot_g  (no per-element multiply)
+//   online softmax: row max / row sum over the four 16-lane groups by wave shuffles
+//   O^T[dim, head] += V^T[dim, token] . P'[token, head]   MFMA, A = V codes (bf16),
+//     B = P' = p * v_scale_g split into bf16 hi + lo (16 significant bits)
+//   The C layout of S^T (lane = head column, 4 token rows) is exactly the B layout
+//   needed for P', so probabilities never leave their registers.
+//
+// Why MFMA for a bandwidth-bound op: with 8 query heads per KV head the path needs
+// 7.8 FMA per KV byte; at 70 % of 8 TB/s that is 43 T FMA/s, above the 39 T FMA/s
+// the chip's (non-packed) FP32 vector units can issue.  On the matrix cores the
+// same work is < 15 % of peak and the vector units only convert int8 -> bf16.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace zllm {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+union Frag {
+    u32x4 u;
+    bf16x8 b;
+    f16x8 h;
+};
+
+// 4 int8 codes in a dword -> two packed bf16 pairs (exact).
+__device__ __forceinline__ u32x2 codes4_to_bf16(unsigned int w)
+{
+    const float c0 = (float)(int)(signed char)(w & 0xffu);
+    const float c1 = (float)(int)(signed char)((w >> 8) & 0xffu);
+    const float c2 = (float)(int)(signed char)((w >> 16) & 0xffu);
+    const float c3 = (float)(int)(signed char)(w >> 24);
+    return u32x2{pack_bf16_trunc(c0, c1), pack_bf16_trunc(c2, c3)};
+}
+
+__device__ __forceinline__ float byte_to_f32(unsigned int w, int e)
+{
+    return (float)(int)(signed char)((w >> (8 * e)) & 0xffu);
+}
+
+__device__ __forceinline__ float fast_tanh(float x)
+{
+    // tanh(x) = 1 - 2 / (exp(2x) + 1); saturates cleanly for large |x|
+    const float e = __builtin_amdgcn_exp2f(fminf(x * (2.0f * kLog2e), 80.0f));
+    return 1.0f - __fdividef(2.0f, e + 1.0f);
+}
+
+template <int G> struct ScaleRow; // G 16-bit scales of one token / KV head
+template <> struct ScaleRow<1> {
+    unsigned short v;
+    __device__ __forceinline__ unsigned short get(int a) const { return v; }
+};
+template <> struct ScaleRow<2> {
+    unsigned int v;
+    __device__ __forceinline__ unsigned short get(int a) const { return (unsigned short)(a == 0 ? (v & 0xffffu) : (v >> 16)); }
+};
+template <> struct ScaleRow<4> {
+    u32x2 v;
+    __device__ __forceinline__ unsigned short get(int a) const
+    {
+        const unsigned int w = a < 2 ? v.x : v.y;
+        return (unsigned short)((a & 1) == 0 ? (w & 0xffffu) : (w >> 16));
+    }
+};
+
+// Everything one wave loads for a 32-token step of a Q8g64 cache.
+template <int G> struct Q8Step {
+    u32x4 k[2][G];      // K codes: tile i, group a -> 16 codes of the lane's token
+    unsigned int v[8][G]; // V codes: token slot s = i*4 + r, group a -> 4 codes (dims a*64 + 4m .. +4)
+    ScaleRow<G> ks[8];  // K scales of token slot s
+    ScaleRow<G> vs[8];  // V scales of token slot s
+};
+
+template <int D, int SDT, bool QSPLIT, bool FAST>
+__global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(GqaDecodeParams p)
+{
+    constexpr int G = D / 64;           // scale groups per head row
+    constexpr int MT = D / 16;          // output M tiles
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int m = lane & 15u;  // MFMA row / column index of this lane
+    const unsigned int j = lane >> 4;   // k-slice index of this lane
+    const unsigned int waves = blockDim.x >> 6;
+    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
+    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
+    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const unsigned int b = blockIdx.z;
+    const unsigned int chunk = blockIdx.x;
+    if (kvh >= p.num_kv_heads) {
+        return;
+    }
+    const unsigned int len = p.kv_lens[b];
+    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+    first = min(first, len);
+    const unsigned int first_al = first & ~31u;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned int head_in_group = head_block * 16u + m;
+    const bool head_valid = head_in_group < p.group;
+    const unsigned int head = kvh * p.group + head_in_group;
+
+    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    if (c_start64 >= len) {
+        if (head_valid && j == 0) {
+            p.stats[stat_index] = kNegInf;
+            p.stats[stat_index + 1] = 0.0f;
+        }
+        return;
+    }
+    const unsigned int c_start = (unsigned int)c_start64;
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int steps = (c_end - c_start + 31u) / 32u;
+
+    // ---- Q fragments: B operand, lane = (head column m, k-slice j) ------------------------
+    Frag qhi[G][2], qlo[G][2];
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[e] = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + a * 64 + j * 16 + hf * 8 + e, p.q_dtype) : 0.0f;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const unsigned short h0 = f32_to_bf16_bits(x[2 * e]);
+                const unsigned short h1 = f32_to_bf16_bits(x[2 * e + 1]);
+                qhi[a][hf].u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
+                if constexpr (QSPLIT) {
+                    qlo[a][hf].u[e] = pack_bf16_rne(x[2 * e] - bf16_bits_to_f32(h0), x[2 * e + 1] - bf16_bits_to_f32(h1));
+                }
+            }
+        }
+    }
+
+    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int k_row = p.num_kv_heads * D;           // bytes per cache row (codes)
+    const unsigned int s_row = p.num_kv_heads * G * 2u;      // bytes per scale row
+    const unsigned char* k_base = p.k_plane + (size_t)kvh * D;
+    const unsigned char* v_base = p.v_plane + (size_t)kvh * D;
+    const unsigned char* ks_base = p.k_scales + (size_t)kvh * G * 2u;
+    const unsigned char* vs_base = p.v_scales + (size_t)kvh * G * 2u;
+    const unsigned int block_mask = p.block_tokens - 1u;
+    const unsigned int lo_tile = first & ~15u;
+    const unsigned int hi_tile = (len - 1u) & ~15u;
+
+    // physical row of the first token of the (clamped) 16-token tile starting at T
+    auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
+        unsigned int t = min(max(T, lo_tile), hi_tile);
+        if (p.ring_capacity != 0) {
+            t %= p.ring_capacity;
+        }
+        const unsigned int entry = p.tables != nullptr ? __builtin_amdgcn_readfirstlane(table[t >> p.block_shift]) : (t >> p.block_shift);
+        return ((unsigned long long)entry << p.block_shift) + (t & block_mask);
+    };
+    // physical row of one token (generic path: any page size / ring)
+    auto token_row = [&](unsigned int t) __attribute__((always_inline)) -> unsigned long long {
+        t = min(max(t, first), len - 1u);
+        return paged_row(p.tables != nullptr ? table : nullptr, t, p.block_tokens, p.ring_capacity);
+    };
+
+    auto load_step = [&](Q8Step<G>& s, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            if constexpr (FAST) {
+                const unsigned long long R = tile_row(t0 + 16u * i);
+                const unsigned char* kr = k_base + (R + m) * k_row + j * 16u;
+#pragma unroll
+                for (int a = 0; a < G; ++a) {
+                    s.k[i][a] = *(const u32x4*)(kr + a * 64);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const unsigned long long row = R + 4u * j + r;
+                    const unsigned char* vr = v_base + row * k_row + 4u * m;
+#pragma unroll
+                    for (int a = 0; a < G; ++a) {
+                        s.v[i * 4 + r][a] = *(const unsigned int*)(vr + a * 64);
+                    }
+                    s.ks[i * 4 + r] = *(const ScaleRow<G>*)(ks_base + row * s_row);
+                    s.vs[i * 4 + r] = *(const ScaleRow<G>*)(vs_base + row * s_row);
+                }
+            } else {
+                const unsigned long long rk = token_row(t0 + 16u * i + m);
+                const unsigned char* kr = k_base + rk * k_row + j * 16u;
+#pragma unroll
+                for (int a = 0; a < G; ++a) {
+                    s.k[i][a] = *(const u32x4*)(kr + a * 64);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const unsigned long long row = token_row(t0 + 16u * i + 4u * j + r);
+                    const unsigned char* vr = v_base + row * k_row + 4u * m;
+#pragma unroll
+                    for (int a = 0; a < G; ++a) {
+                        s.v[i * 4 + r][a] = *(const unsigned int*)(vr + a * 64);
+                    }
+                    s.ks[i * 4 + r] = *(const ScaleRow<G>*)(ks_base + row * s_row);
+                    s.vs[i * 4 + r] = *(const ScaleRow<G>*)(vs_base + row * s_row);
+                }
+            }
+        }
+    };
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float run_max = kNegInf; // log2 units
+    float run_sum = 0.0f;    // lane-partial (this lane's 8 token slots per step)
+    const float scale_log2 = p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e;
+
+    auto compute_step = [&](const Q8Step<G>& s, unsigned int t0) __attribute__((always_inline)) {
+        // ---- S^T = K . Q^T, one accumulator per scale group -----------------------------
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float tile_s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int a = 0; a < G; ++a) {
+                Frag k0, k1;
+                const u32x2 c0 = codes4_to_bf16(s.k[i][a].x), c1 = codes4_to_bf16(s.k[i][a].y);
+                const u32x2 c2 = codes4_to_bf16(s.k[i][a].z), c3 = codes4_to_bf16(s.k[i][a].w);
+                k0.u = u32x4{c0.x, c0.y, c1.x, c1.y};
+                k1.u = u32x4{c2.x, c2.y, c3.x, c3.y};
+                f32x4 d = {0.f, 0.f, 0.f, 0.f};
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qhi[a][0].b, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qhi[a][1].b, d, 0, 0, 0);
+                if constexpr (QSPLIT) {
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qlo[a][0].b, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qlo[a][1].b, d, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(s.ks[i * 4 + r].get(a)), tile_s[r]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float x = tile_s[r] * scale_log2;
+                if (p.softcap > 0.0f) {
+                    x = p.softcap * fast_tanh(x / p.softcap) * kLog2e;
+                }
+                const unsigned int token = t0 + 16u * i + 4u * j + r;
+                sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
+            }
+        }
+        // ---- online softmax (base 2) -----------------------------------------------------
+        float step_max = sc[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) {
+            step_max = fmaxf(step_max, sc[e]);
+        }
+        step_max = wave_max_16x4(step_max);
+        const float new_max = fmaxf(run_max, step_max);
+        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+        const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
+        float pr[8];
+        float step_sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+            step_sum += pr[e];
+        }
+        run_sum = run_sum * alpha + step_sum;
+        run_max = new_max;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[t] *= alpha;
+            }
+        }
+        // ---- O^T += V^T . P', P' = p * v_scale split into bf16 hi + lo --------------------
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+            Frag phi, plo;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(s.vs[2 * e].get(a));
+                const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(s.vs[2 * e + 1].get(a));
+                const unsigned short h0 = f32_to_bf16_bits(x0);
+                const unsigned short h1 = f32_to_bf16_bits(x1);
+                phi.u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
+                plo.u[e] = pack_bf16_rne(x0 - bf16_bits_to_f32(h0), x1 - bf16_bits_to_f32(h1));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Frag vf;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    vf.u[c] = pack_bf16_trunc(byte_to_f32(s.v[2 * c][a], e), byte_to_f32(s.v[2 * c + 1][a], e));
+                }
+                f32x4 d = acc[a * 4 + e];
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi.b, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo.b, d, 0, 0, 0);
+                acc[a * 4 + e] = d;
+            }
+        }
+    };
+
+    // ---- software pipeline: loads of step n+1 in flight while step n computes ---------
+    Q8Step<G> buf0, buf1;
+    load_step(buf0, c_start);
+    unsigned int step = 0;
+    while (true) {
+        const unsigned int t0 = c_start + step * 32u;
+        if (step + 1 < steps) {
+            load_step(buf1, t0 + 32u);
+        }
+        compute_step(buf0, t0);
+        if (++step >= steps) {
+            break;
+        }
+        if (step + 1 < steps) {
+            load_step(buf0, t0 + 64u);
+        }
+        compute_step(buf1, t0 + 32u);
+        if (++step >= steps) {
+            break;
+        }
+    }
+
+    // ---- write the un-normalised partial and (max, sum) -------------------------------------
+    const float total = wave_sum_16x4(run_sum);
+    if (head_valid) {
+        if (j == 0) {
+            p.stats[stat_index] = run_max;
+            p.stats[stat_index + 1] = total;
+        }
+        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
+        // tile (a, e), register r holds dim a*64 + 16*j + 4*r + e
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const f32x4 v = {acc[a * 4 + 0][r], acc[a * 4 + 1][r], acc[a * 4 + 2][r], acc[a * 4 + 3][r]};
+                *(f32x4*)(out + a * 64 + 16 * j + 4 * r) = v;
+            }
+        }
+    }
+}
+
+// ---- f16 KV (no scales): f16 MFMA, Q and P split into f16 hi + lo -------------------------
+template <int D> struct F16Step {
+    u32x4 k[2][D / 32];     // K: tile i, k-step ks -> 8 f16 (dims ks*32 + j*8 .. +8)
+    u32x4 v[8][D / 128];    // V: token slot s -> D/16 f16 (dims m*(D/16) ..), 16 B units
+};
+
+template <int D, bool FAST>
+__global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(GqaDecodeParams p)
+{
+    static_assert(D % 128 == 0, "f16 KV path supports head_dim 128 and 256");
+    constexpr int KS = D / 32;  // QK k-steps
+    constexpr int MT = D / 16;  // output M tiles
+    constexpr int VU = D / 128; // 16-byte units of V per lane per token
+    constexpr float kPScale = 16384.0f; // keeps f16(p) out of the subnormal range
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    const unsigned int waves = blockDim.x >> 6;
+    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
+    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
+    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const unsigned int b = blockIdx.z;
+    const unsigned int chunk = blockIdx.x;
+    if (kvh >= p.num_kv_heads) {
+        return;
+    }
+    const unsigned int len = p.kv_lens[b];
+    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+    first = min(first, len);
+    const unsigned int first_al = first & ~31u;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned int head_in_group = head_block * 16u + m;
+    const bool head_valid = head_in_group < p.group;
+    const unsigned int head = kvh * p.group + head_in_group;
+    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    if (c_start64 >= len) {
+        if (head_valid && j == 0) {
+            p.stats[stat_index] = kNegInf;
+            p.stats[stat_index + 1] = 0.0f;
+        }
+        return;
+    }
+    const unsigned int c_start = (unsigned int)c_start64;
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int steps = (c_end - c_start + 31u) / 32u;
+
+    // Q: per-head power-of-two normalisation keeps q inside the f16 range; hi + lo split.
+    float q_norm = 1.0f;
+    {
+        float amax = 0.0f;
+        for (int e = 0; e < D / 4; ++e) {
+            const float x = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + j * (D / 4) + e, p.q_dtype) : 0.0f;
+            amax = fmaxf(amax, fabsf(x));
+        }
+        amax = wave_max_16x4(amax);
+        if (amax > 0.0f && amax < __builtin_inff()) {
+            int ex;
+            frexpf(amax, &ex);        // amax = f * 2^ex, f in [0.5, 1)
+            q_norm = ldexpf(1.0f, -ex); // |q| * q_norm < 1
+        }
+    }
+    Frag qhi[KS], qlo[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + ks * 32 + j * 8 + e, p.q_dtype) * q_norm : 0.0f;
+            const _Float16 h = (_Float16)x;
+            qhi[ks].h[e] = h;
+            qlo[ks].h[e] = (_Float16)(x - (float)h);
+        }
+    }
+
+    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int k_row = p.num_kv_heads * D * 2u; // bytes per cache row
+    const unsigned char* k_base = p.k_plane + (size_t)kvh * D * 2u;
+    const unsigned char* v_base = p.v_plane + (size_t)kvh * D * 2u;
+    const unsigned int block_mask = p.block_tokens - 1u;
+    const unsigned int lo_tile = first & ~15u;
+    const unsigned int hi_tile = (len - 1u) & ~15u;
+    auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
+        unsigned int t = min(max(T, lo_tile), hi_tile);
+        if (p.ring_capacity != 0) {
+            t %= p.ring_capacity;
+        }
+        const unsigned int entry = p.tables != nullptr ? __builtin_amdgcn_readfirstlane(table[t >> p.block_shift]) : (t >> p.block_shift);
+        return ((unsigned long long)entry << p.block_shift) + (t & block_mask);
+    };
+    auto token_row = [&](unsigned int t) __attribute__((always_inline)) -> unsigned long long {
+        t = min(max(t, first), len - 1u);
+        return paged_row(p.tables != nullptr ? table : nullptr, t, p.block_tokens, p.ring_capacity);
+    };
+    auto load_step = [&](F16Step<D>& s, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            unsigned long long R = 0;
+            if constexpr (FAST) {
+                R = tile_row(t0 + 16u * i);
+            }
+            const unsigned long long rk = FAST ? R + m : token_row(t0 + 16u * i + m);
+            const unsigned char* kr = k_base + rk * k_row + j * 16u;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                s.k[i][ks] = *(const u32x4*)(kr + ks * 64);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const unsigned long long row = FAST ? R + 4u * j + r : token_row(t0 + 16u * i + 4u * j + r);
+                const unsigned char* vr = v_base + row * k_row + m * (D / 8);
+#pragma unroll
+                for (int u = 0; u < VU; ++u) {
+                    s.v[i * 4 + r][u] = *(const u32x4*)(vr + u * 16);
+                }
+            }
+        }
+    };
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float run_max = kNegInf;
+    float run_sum = 0.0f;
+    const float scale_eff = (p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e) / q_norm;
+
+    auto compute_step = [&](const F16Step<D>& s, unsigned int t0) __attribute__((always_inline)) {
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                Frag kf;
+                kf.u = s.k[i][ks];
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf.h, qhi[ks].h, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf.h, qlo[ks].h, d, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float x = d[r] * scale_eff;
+                if (p.softcap > 0.0f) {
+                    x = p.softcap * fast_tanh(x / p.softcap) * kLog2e;
+                }
+                const unsigned int token = t0 + 16u * i + 4u * j + r;
+                sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
+            }
+        }
+        float step_max = sc[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) {
+            step_max = fmaxf(step_max, sc[e]);
+        }
+        step_max = wave_max_16x4(step_max);
+        const float new_max = fmaxf(run_max, step_max);
+        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+        const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
+        float pr[8];
+        float step_sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+            step_sum += pr[e];
+        }
+        run_sum = run_sum * alpha + step_sum;
+        run_max = new_max;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[t] *= alpha;
+            }
+        }
+        Frag phi, plo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = pr[e] * kPScale;
+            const _Float16 h = (_Float16)x;
+            phi.h[e] = h;
+            plo.h[e] = (_Float16)(x - (float)h);
+        }
+        // V^T fragments: element t of the lane's D/16 dims, across the 8 token slots
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int u = t / 8;         // which 16-byte unit
+            const int w = (t % 8) / 2;   // dword inside the unit
+            const bool upper = (t & 1) != 0;
+            Frag vf;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const unsigned int a0 = s.v[2 * c][u][w];
+                const unsigned int a1 = s.v[2 * c + 1][u][w];
+                vf.u[c] = upper ? __builtin_amdgcn_perm(a1, a0, 0x07060302u) : __builtin_amdgcn_perm(a1, a0, 0x05040100u);
+            }
+            f32x4 d = acc[t];
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf.h, phi.h, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf.h, plo.h, d, 0, 0, 0);
+            acc[t] = d;
+        }
+    };
+
+    F16Step<D> buf0, buf1;
+    load_step(buf0, c_start);
+    unsigned int step = 0;
+    while (true) {
+        const unsigned int t0 = c_start + step * 32u;
+        if (step + 1 < steps) {
+            load_step(buf1, t0 + 32u);
+        }
+        compute_step(buf0, t0);
+        if (++step >= steps) {
+            break;
+        }
+        if (step + 1 < steps) {
+            load_step(buf0, t0 + 64u);
+        }
+        compute_step(buf1, t0 + 32u);
+        if (++step >= steps) {
+            break;
+        }
+    }
+
+    const float total = wave_sum_16x4(run_sum);
+    if (head_valid) {
+        if (j == 0) {
+            p.stats[stat_index] = run_max;
+            p.stats[stat_index + 1] = total;
+        }
+        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
+        // tile t, register r holds dim (4*j + r) * (D/16) + t ; undo the P scaling
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                out[(4 * j + r) * (D / 16) + t] = acc[t][r] * (1.0f / kPScale);
+            }
+        }
+    }
+}
+
+// ---- split combine by log-sum-exp ---------------------------------------------------------
+// out[b, head, :] = sum_c partial_c * 2^(m_c - m) / sum_c l_c * 2^(m_c - m); zero when nothing
+// was visible.  Same algebra as gqa_decode_merge_f32
+// (src/kernel/rocm/hip/tensor/attention/source.hip:1339-1362), in base 2.
+__global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
+{
+    const unsigned int quads = p.head_dim / 4u;
+    const unsigned int heads_per_block = 256u / quads;
+    const unsigned int head = blockIdx.x * heads_per_block + threadIdx.x / quads;
+    const unsigned int quad = threadIdx.x % quads;
+    const unsigned int b = blockIdx.y;
+    if (head >= p.num_heads) {
+        return;
+    }
+    const unsigned int len = p.kv_lens[b];
+    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+    first = min(first, len);
+    const unsigned int first_al = first & ~31u;
+    const unsigned int chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    const size_t stat_stride = (size_t)p.num_heads * 2;
+    float m = kNegInf;
+    for (unsigned int c = 0; c < chunks; ++c) {
+        m = fmaxf(m, stats[c * stat_stride]);
+    }
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.0f;
+    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;
+    const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
+    for (unsigned int c = 0; c < chunks; ++c) {
+        const float cm = stats[c * stat_stride];
+        const float cl = stats[c * stat_stride + 1];
+        if (cl <= 0.0f) {
+            continue;
+        }
+        const float w = __builtin_amdgcn_exp2f(cm - m);
+        l += cl * w;
+        acc += *(const f32x4*)(partial + c * partial_stride) * w;
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    f32x4 result = acc * inv;
+    if (!(l > 0.0f)) {
+        result = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    *(f32x4*)(p.out + ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u) = result;
+}
+
+template <int D, int SDT, bool QSPLIT>
+hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block, hipStream_t stream)
+{
+    if (fast) {
+        gqa_decode_q8_partial<D, SDT, QSPLIT, true><<<grid, block, 0, stream>>>(p);
+    } else {
+        gqa_decode_q8_partial<D, SDT, QSPLIT, false><<<grid, block, 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
+template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtype, bool fast, dim3 grid, dim3 block, hipStream_t stream)
+{
+    const bool split = p.q_dtype != 1; // bf16 queries are exact in one bf16 term
+    if (scale_dtype == 0) {
+        return split ? launch_q8<D, 0, true>(p, fast, grid, block, stream) : launch_q8<D, 0, false>(p, fast, grid, block, stream);
+    }
+    return split ? launch_q8<D, 1, true>(p, fast, grid, block, stream) : launch_q8<D, 1, false>(p, fast, grid, block, stream);
+}
+
+} // namespace
+
+hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, hipStream_t stream)
+{
+    const unsigned int max_waves = p.head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
+    const unsigned int waves = p.num_kv_heads < max_waves ? p.num_kv_heads : max_waves;
+    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
+    const unsigned int head_blocks = (p.group + 15u) / 16u;
+    const dim3 grid(p.max_chunks, kvh_blocks * head_blocks, p.batch);
+    const dim3 block(waves * 64u);
+    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
+    const bool fast = pow2 && p.block_tokens >= 16u && p.ring_capacity % 16u == 0;
+    hipError_t err = hipSuccess;
+    if (kv_format == 0) {
+        switch (p.head_dim) {
+        case 64: err = launch_q8_d<64>(p, scale_dtype, fast, grid, block, stream); break;
+        case 128: err = launch_q8_d<128>(p, scale_dtype, fast, grid, block, stream); break;
+        case 256: err = launch_q8_d<256>(p, scale_dtype, fast, grid, block, stream); break;
+        default: return hipErrorInvalidValue;
+        }
+    } else {
+        if (p.head_dim == 128) {
+            if (fast) {
+                gqa_decode_f16_partial<128, true><<<grid, block, 0, stream>>>(p);
+            } else {
+                gqa_decode_f16_partial<128, false><<<grid, block, 0, stream>>>(p);
+            }
+        } else if (p.head_dim == 256) {
+            if (fast) {
+                gqa_decode_f16_partial<256, true><<<grid, block, 0, stream>>>(p);
+            } else {
+                gqa_decode_f16_partial<256, false><<<grid, block, 0, stream>>>(p);
+            }
+        } else {
+            return hipErrorInvalidValue;
+        }
+        err = hipGetLastError();
+    }
+    if (err != hipSuccess) {
+        return err;
+    }
+    const unsigned int quads = p.head_dim / 4u;
+    const unsigned int heads_per_block = 256u / quads;
+    gqa_decode_merge<<<dim3((p.num_heads + heads_per_block - 1) / heads_per_block, p.batch), dim3(256), 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+} // namespace zllm

@@ -1,0 +1,117 @@
+// Kernel parameter blocks and launch functions (internal; the public surface is include/zllm_attn.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace zllm {
+
+struct Q8AppendParams {
+    const void* src;
+    signed char* codes;
+    void* scales;
+    const unsigned int* table;
+    const unsigned int* positions;
+    unsigned int position, rows, cols, block_tokens, ring_capacity;
+    int src_dtype, rule;
+};
+
+struct HalfAppendParams {
+    const void* src;
+    unsigned short* cache;
+    const unsigned int* table;
+    unsigned int position, rows, cols, block_tokens, ring_capacity;
+    int src_dtype, dst_dtype;
+};
+
+struct MlaAppendParams {
+    const float* latent;
+    const float* k_rope;
+    const float* cosine;
+    const float* sine;
+    signed char* latent_codes;
+    unsigned short* latent_scales;
+    unsigned short* rope_cache;
+    const unsigned int* table;
+    const unsigned int* positions;
+    unsigned int position, rope_position, rows, latent_cols, rope_cols, rotary_dim, split_half, block_tokens;
+};
+
+struct GatherParams {
+    const void* plane;
+    void* out;
+    const unsigned int* table;
+    unsigned int first, count, row_bytes, block_tokens, ring_capacity;
+};
+
+// Split-KV geometry shared by the partial and merge kernels.
+struct SplitPlan {
+    unsigned int chunk_tokens; // tokens per split (multiple of 32)
+    unsigned int max_chunks;   // grid extent over splits
+};
+
+struct GqaDecodeParams {
+    const void* q;
+    const unsigned char* k_plane;
+    const unsigned char* k_scales;
+    const unsigned char* v_plane;
+    const unsigned char* v_scales;
+    const unsigned int* tables;
+    const unsigned int* kv_lens;
+    const unsigned int* first_visible;
+    float* out;
+    float* partial; // [batch][max_chunks][num_heads][head_dim]
+    float* stats;   // [batch][max_chunks][num_heads][2] = (max, sum)
+    unsigned int batch, num_heads, num_kv_heads, head_dim, group;
+    unsigned int table_stride, block_tokens, block_shift, ring_capacity;
+    unsigned int chunk_tokens, max_chunks;
+    float score_scale, softcap;
+    int q_dtype;
+};
+
+struct GqaPrefillParams {
+    const void* q;
+    const unsigned char* k_plane;
+    const unsigned char* k_scales;
+    const unsigned char* v_plane;
+    const unsigned char* v_scales;
+    const unsigned int* table;
+    void* out;
+    unsigned int rows, position, window;
+    unsigned int num_heads, num_kv_heads, head_dim, group;
+    unsigned int block_tokens, block_shift;
+    float score_scale, softcap;
+    int q_dtype, out_dtype;
+};
+
+struct MlaDecodeParams {
+    const void* q;
+    const unsigned short* kv_b;
+    const signed char* latent_codes;
+    const unsigned short* latent_scales;
+    const unsigned short* rope_cache;
+    const unsigned int* tables;
+    const unsigned int* ctx_lens;
+    void* out;
+    unsigned short* absorbed; // bf16 [batch][heads][latent_dim + rope_dim] (absorbed nope | q_rope)
+    float* partial;           // [batch][max_chunks][heads][latent_dim]
+    float* stats;             // [batch][max_chunks][heads][2]
+    float* weighted;          // [batch][heads][latent_dim]
+    unsigned int batch, heads, q_head_dim, kv_head_dim, latent_dim, rope_dim, nope_dim, value_dim;
+    unsigned int table_stride, block_tokens, block_shift;
+    unsigned int chunk_tokens, max_chunks;
+    float score_scale;
+    int q_dtype, out_dtype, out_compact;
+};
+
+hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream);
+hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream);
+hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream);
+hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);
+
+// kv_format: 0 = Q8g64, 1 = f16; scale_dtype: 0 = bf16, 1 = f16 (Q8 only).
+hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, hipStream_t stream);
+hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream);
+hipError_t launch_mla_decode(const MlaDecodeParams& p, hipStream_t stream);
+
+} // namespace zllm
