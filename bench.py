@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+Default workload = BASELINE.json configs[1]: Qwen3-style Q8g64 GQA decode, batch 8, 64 query heads /
+8 KV heads, head_dim 128, every sequence at 32,768 tokens (the "32K ctx" case the metric is quoted
+on), 16-token pages scattered over a large pool, bf16 queries, K/V ~ N(0,1) with 1 % outlier
+channels x8.  One "step" = one decode attention call (split-KV partial + LSE merge) over the batch.
+
+Prints ONE JSON line.  `value` = effective KV GB/s of the whole call (KV codes + scales inside the
+visible window, each counted once; inputs resident in HBM).  `roofline` prices the dominant kernel
+(the split-KV partial kernel) alone, timed with HIP events on the launch stream.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+METRIC = "decode attn effective KV GB/s (% of HBM peak) + tokens/s at 32K ctx, 1 GPU"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="gqa_decode_32k",
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk"])
+    ap.add_argument("--pool-gib", type=float, default=160.0, help="address span of the paged pool (all four planes)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=2)
+    return ap.parse_args()
+
+
+def event_time_ms(fn, steps):
+    """Average duration per call of `fn` over `steps` back-to-back launches, by HIP events on the stream."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def wall_time_ms(fn, steps):
+    import torch
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+# ------------------------------------------------------------------------------------------- GQA decode
+def build_gqa_pool(args, lens, hq, hkv, d, block_tokens):
+    """Fill a paged Q8g64 pool on the device: K/V ~ N(0,1), 1 % outlier channels x8, quantized by the library's
+    own append kernel (bit-exact with the oracle's quantizer), pages drawn without replacement from the pool."""
+    import torch
+
+    from zllm_amd import capi, ops
+
+    dev = "cuda"
+    cols = hkv * d
+    groups = cols // 64
+    bytes_per_row = 2 * (cols + groups * 2)
+    free, _ = torch.cuda.mem_get_info()
+    span = min(int(args.pool_gib * (1 << 30)), int(free * 0.80))
+    need_blocks = sum((l + block_tokens - 1) // block_tokens for l in lens)
+    pool_blocks = max(span // (bytes_per_row * block_tokens), need_blocks + 1)
+    pool_rows = pool_blocks * block_tokens
+    planes = dict(
+        k_codes=torch.empty((pool_rows, cols), dtype=torch.int8, device=dev),
+        k_scales=torch.empty((pool_rows, groups), dtype=torch.int16, device=dev),
+        v_codes=torch.empty((pool_rows, cols), dtype=torch.int8, device=dev),
+        v_scales=torch.empty((pool_rows, groups), dtype=torch.int16, device=dev),
+    )
+    rng = np.random.default_rng(args.seed)
+    ids = rng.choice(pool_blocks, size=need_blocks, replace=False).astype(np.uint32)
+    stride = max((l + block_tokens - 1) // block_tokens for l in lens)
+    tables = np.zeros((len(lens), stride), dtype=np.uint32)
+    at = 0
+    for b, l in enumerate(lens):
+        n = (l + block_tokens - 1) // block_tokens
+        tables[b, :n] = ids[at:at + n]
+        at += n
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed)
+    gain = torch.ones(cols, device=dev)
+    gain[torch.from_numpy(rng.choice(cols, size=max(1, cols // 100), replace=False)).to(dev)] = 8.0
+    tables_dev = torch.from_numpy(tables.view(np.int32)).to(dev)
+    step = 4096
+    for b, l in enumerate(lens):
+        for pos in range(0, l, step):
+            n = min(step, l - pos)
+            k = torch.randn((n, cols), generator=gen, device=dev) * gain
+            v = torch.randn((n, cols), generator=gen, device=dev) * gain
+            ops.q8g64_append(k, planes["k_codes"], planes["k_scales"], tables_dev[b], pos, block_tokens, capi.QUANT_METAL_GQA)
+            ops.q8g64_append(v, planes["v_codes"], planes["v_scales"], tables_dev[b], pos, block_tokens, capi.QUANT_METAL_GQA)
+    q = torch.randn((len(lens), hq * d), generator=gen, device=dev).to(torch.bfloat16)
+    torch.cuda.synchronize()
+    span_bytes = int(ids.max()) * block_tokens * cols
+    return planes, tables, tables_dev, q, dict(pool_rows=pool_rows, pool_blocks=pool_blocks,
+                                               pool_bytes=pool_rows * bytes_per_row, max_code_offset=span_bytes)
+
+
+def gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, block_tokens, scale, budget_s=12.0):
+    """The CPU oracle (port of the reference's f32 path: dequantize the Q8g64 rows, then causal_head_range per
+    (token, head) task) over the whole batch, repeated until about `budget_s` seconds of CPU work are spent."""
+    import oracle as O
+    from zllm_amd import ops
+
+    cols = hkv * d
+    threads = O.set_threads(min(len(os.sched_getaffinity(0)), 16))
+    host = []
+    for b, l in enumerate(lens):
+        rows = {}
+        for name, width in (("k_codes", cols), ("k_scales", cols // 64 * 2), ("v_codes", cols), ("v_scales", cols // 64 * 2)):
+            rows[name] = ops.gather_rows(planes[name], tables_dev[b], 0, l, width, block_tokens).cpu().numpy()
+        host.append(rows)
+    q_host = q.float().cpu().numpy()
+    total_bytes = sum(lens) * 2 * (cols + cols // 64 * 2)
+    outs = np.zeros((len(lens), hq * d), dtype=np.float32)
+    passes, t_deq, t_att = [], 0.0, 0.0
+    started = time.perf_counter()
+    while time.perf_counter() - started < budget_s or not passes:
+        p_deq = p_att = 0.0
+        for b, l in enumerate(lens):
+            t0 = time.perf_counter()
+            k = O.gather_dequant_rows(O.FMT_Q8, host[b]["k_codes"].view(np.int8), host[b]["k_scales"].view(np.uint16), O.SCALE_F16,
+                                      None, block_tokens, 0, l, cols)
+            v = O.gather_dequant_rows(O.FMT_Q8, host[b]["v_codes"].view(np.int8), host[b]["v_scales"].view(np.uint16), O.SCALE_F16,
+                                      None, block_tokens, 0, l, cols)
+            t1 = time.perf_counter()
+            rc, out = O.gqa_prefill_at_visible(q_host[b:b + 1], k, v, 0, l, l - 1, hq, hkv, d, score_scale=scale)
+            t2 = time.perf_counter()
+            assert rc == 0
+            outs[b] = out[0]
+            p_deq += t1 - t0
+            p_att += t2 - t1
+        passes.append(p_deq + p_att)
+        t_deq += p_deq
+        t_att += p_att
+    median = float(np.median(passes))
+    n = len(passes)
+    return dict(value=round(total_bytes / median / 1e9, 3), unit="GB/s", cores=threads, kind="port",
+                sample=f"whole batch ({len(lens)} sequences, all heads), {n} passes in {sum(passes):.1f}s, median pass {median:.3f}s; "
+                       f"per pass: dequantize {t_deq / n:.3f}s + f32 attention {t_att / n:.3f}s"), outs
+
+
+def run_gqa_decode(args, ragged):
+    import torch
+
+    from zllm_amd import capi, ops
+
+    hq, hkv, d, bt, batch = 64, 8, 128, 16, 8
+    rng = np.random.default_rng(args.seed)
+    lens = [int(x) for x in rng.integers(1024, 32769, size=batch)] if ragged else [32768] * batch
+    scale = 1.0 / float(np.sqrt(d))
+    ops.init(0)
+    planes, tables, tables_dev, q, pool = build_gqa_pool(args, lens, hq, hkv, d, bt)
+    lens_dev = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    call_args, out, workspace = ops.gqa_decode_args(q, planes["k_codes"], planes["k_scales"], planes["v_codes"], planes["v_scales"],
+                                                    tables_dev, lens_dev, hq, hkv, d, bt, scale, max(lens),
+                                                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16)
+    lib = capi.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def full():
+        call_args.stages = capi.STAGE_ALL
+        capi.check(lib.zllm_attn_gqa_decode(C.byref(call_args), stream))
+
+    def partial_only():
+        call_args.stages = capi.STAGE_PARTIAL
+        capi.check(lib.zllm_attn_gqa_decode(C.byref(call_args), stream))
+
+    for _ in range(args.warmup):
+        full()
+    ms_step = wall_time_ms(full, args.steps)
+    ms_events = event_time_ms(full, args.steps)
+    ms_partial = event_time_ms(partial_only, args.steps)
+    full()
+    torch.cuda.synchronize()
+
+    bytes_per_token = 2 * (hkv * d + 2 * hkv * d // 64)  # 2,112 B: K+V codes + 16-bit scales
+    kv_bytes = sum(lens) * bytes_per_token
+    gbps = kv_bytes / (ms_step * 1e-3) / 1e9
+    achieved = kv_bytes / (ms_partial * 1e-3) / 1e9
+    record = {
+        "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": ("C2 Q8g64 GQA decode, B=8, 64q/8kv, d=128, " + ("ragged L~U[1024,32768]" if ragged else "all L=32768")
+                                + ", 16-token pages"),
+                   "kv_lens": lens, "kv_bytes_per_call": kv_bytes, "bytes_per_token": bytes_per_token, "seed": args.seed,
+                   "pool_bytes": pool["pool_bytes"], "pool_blocks": pool["pool_blocks"], "max_code_plane_offset": pool["max_code_offset"],
+                   "q_dtype": "bf16", "scale_dtype": "f16", "kv_arithmetic": "int8 codes -> bf16 MFMA operands, f32 accumulate"},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
+        "ms_per_step_events": round(ms_events, 5),
+        "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_partial", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel_ms": round(ms_partial, 5)},
+    }
+    if not args.no_cpu_baseline:
+        cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)
+        record["cpu_baseline"] = cpu
+        record["parity_vs_oracle_max_abs"] = float(np.abs(out.cpu().numpy() - cpu_out).max())
+    print(json.dumps(record))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build targets one MI355X; --gpus must be 1 (multi-GPU sharding is design-only)", file=sys.stderr)
+        sys.exit(2)
+    if args.workload == "gqa_decode_32k":
+        run_gqa_decode(args, ragged=False)
+    elif args.workload == "gqa_decode_ragged":
+        run_gqa_decode(args, ragged=True)
+    else:
+        from zllm_amd import bench_extra
+
+        bench_extra.run(args)
+
+
+if __name__ == "__main__":
+    main()

@@ -63,6 +63,9 @@ enum { ZLLM_QUANT_ROCM_MLA = 0, ZLLM_QUANT_METAL_GQA = 1, ZLLM_QUANT_CUDA_GQA = 
 /* RoPE pair layout (src/attention/rope.rs:106-110). */
 enum { ZLLM_ROTARY_INTERLEAVED = 0, ZLLM_ROTARY_SPLIT_HALF = 1 };
 
+/* Stage selection for the split-KV entry points. */
+enum { ZLLM_STAGE_ALL = 0, ZLLM_STAGE_PARTIAL = 1, ZLLM_STAGE_MERGE = 2 };
+
 #define ZLLM_GROUP_SIZE 64 /* src/kv_cache/mod.rs:29 DEFAULT_GROUP_SIZE */
 
 /* Library / device bring-up.  Optional: every entry point works without it.
@@ -208,6 +211,12 @@ typedef struct zllm_gqa_decode_args {
     int kv_format;                 /* ZLLM_KV_* */
     int scale_dtype;               /* ZLLM_SCALE_* (Q8 only) */
     int q_dtype;                   /* ZLLM_DTYPE_* */
+    uint32_t stages;               /* 0 = partial + merge; ZLLM_STAGE_PARTIAL leaves the
+                                      un-merged (partial, max, sum) records in the workspace
+                                      for a caller that combines shards itself
+                                      (cf. try_paged_mla_attention_ct_shard,
+                                      paged_mla.rs:3642); ZLLM_STAGE_MERGE combines records
+                                      already in the workspace */
 } zllm_gqa_decode_args;
 ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* args);
 ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);

@@ -17,6 +17,7 @@ DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 KV_Q8G64, KV_F16 = 0, 1
 QUANT_ROCM_MLA, QUANT_METAL_GQA, QUANT_CUDA_GQA = 0, 1, 2
 ROTARY_INTERLEAVED, ROTARY_SPLIT_HALF = 0, 1
+STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
 
 _u32, _u64, _f32, _int, _ptr = C.c_uint32, C.c_uint64, C.c_float, C.c_int, C.c_void_p
 
@@ -50,7 +51,7 @@ class GqaDecodeArgs(C.Structure):
                 ("workspace_bytes", _u64), ("batch", _u32), ("num_heads", _u32), ("num_kv_heads", _u32),
                 ("head_dim", _u32), ("table_stride", _u32), ("max_kv_len", _u32), ("block_tokens", _u32),
                 ("ring_capacity", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
-                ("scale_dtype", _int), ("q_dtype", _int)]
+                ("scale_dtype", _int), ("q_dtype", _int), ("stages", _u32)]
 
 
 class GqaPrefillArgs(C.Structure):

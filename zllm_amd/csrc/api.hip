@@ -55,9 +55,9 @@ bool valid_head_dim(uint32_t d)
 // Tokens per KV split: enough workgroups to occupy every CU about twice, but
 // splits long enough that the partial write / merge stay a few percent of the
 // KV bytes a split reads.
-void plan_splits(uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t* chunk_tokens, uint32_t* max_chunks)
+void plan_splits(uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t rounds, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
-    const uint64_t target = 2ull * kComputeUnits;
+    const uint64_t target = (uint64_t)rounds * kComputeUnits;
     uint64_t chunk = ((uint64_t)max_len * columns + target - 1) / target;
     chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
     *chunk_tokens = (uint32_t)chunk;
@@ -93,6 +93,9 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
     if (a->q_dtype < ZLLM_DTYPE_F32 || a->q_dtype > ZLLM_DTYPE_F16) {
         return fail(-1, "GQA decode: unknown q_dtype %d", a->q_dtype);
     }
+    if (a->stages > ZLLM_STAGE_MERGE) {
+        return fail(-1, "GQA decode: unknown stages %u", a->stages);
+    }
     return 0;
 }
 
@@ -102,7 +105,54 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
-    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, chunk_tokens, max_chunks);
+    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, 2, chunk_tokens, max_chunks);
+}
+
+int validate_mla_decode(const zllm_mla_decode_args* a)
+{
+    if (a == nullptr) {
+        return fail(-1, "MLA decode: null args");
+    }
+    // shape rules of try_paged_mla_attention_ct_inner (paged_mla.rs:2940-2949)
+    if (a->batch == 0 || a->heads == 0 || a->q_head_dim == 0 || a->kv_head_dim == 0 || a->rope_dim > a->q_head_dim ||
+        a->q_head_dim - a->rope_dim > a->kv_head_dim || a->q_head_dim > 1024) {
+        return fail(-1, "MLA decode: invalid shape batch=%u heads=%u q_head=%u kv_head=%u rope=%u", a->batch, a->heads, a->q_head_dim,
+                    a->kv_head_dim, a->rope_dim);
+    }
+    if (a->latent_dim != 512 || a->rope_dim != 64) {
+        return fail(-1, "MLA decode: this build handles latent_dim 512 + rope_dim 64 (got %u + %u)", a->latent_dim, a->rope_dim);
+    }
+    if (a->block_tokens == 0 || a->max_ctx_len == 0) {
+        return fail(-1, "MLA decode: block_tokens=%u max_ctx_len=%u must be non-zero", a->block_tokens, a->max_ctx_len);
+    }
+    if ((a->q_dtype != ZLLM_DTYPE_F32 && a->q_dtype != ZLLM_DTYPE_BF16) || (a->out_dtype != ZLLM_DTYPE_F32 && a->out_dtype != ZLLM_DTYPE_BF16)) {
+        return fail(-1, "MLA decode: q_dtype / out_dtype must be f32 or bf16");
+    }
+    return 0;
+}
+
+void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
+    // (above 64 heads two workgroups share a split, each owning half of the output columns)
+    const uint32_t head_blocks = a->heads > 64 ? 2 * ((a->heads + 127) / 128) : 1;
+    plan_splits(a->max_ctx_len, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
+}
+
+struct MlaWorkspace {
+    uint64_t absorbed, partial, stats, weighted, total;
+};
+
+MlaWorkspace mla_workspace(const zllm_mla_decode_args* a, uint32_t max_chunks)
+{
+    MlaWorkspace w;
+    const uint64_t rows = (uint64_t)a->batch * a->heads;
+    w.absorbed = 0;
+    w.partial = align_up(rows * (a->latent_dim + a->rope_dim) * 2, 256);
+    w.stats = w.partial + align_up(rows * max_chunks * a->latent_dim * 4, 256);
+    w.weighted = w.stats + align_up(rows * max_chunks * 8, 256);
+    w.total = w.weighted + align_up(rows * a->latent_dim * 4, 256);
+    return w;
 }
 
 } // namespace
@@ -341,7 +391,72 @@ int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
     p.score_scale = a->score_scale;
     p.softcap = a->softcap;
     p.q_dtype = a->q_dtype;
-    return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA decode launch");
+    return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, a->stages, (hipStream_t)stream), "GQA decode launch");
+}
+
+/* ---- MLA decode ------------------------------------------------------------------------- */
+
+uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* a)
+{
+    if (validate_mla_decode(a) != 0) {
+        return 0;
+    }
+    uint32_t chunk_tokens, max_chunks;
+    plan_mla_decode(a, &chunk_tokens, &max_chunks);
+    return mla_workspace(a, max_chunks).total;
+}
+
+int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
+{
+    const int rc = validate_mla_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    if (a->q == nullptr || a->kv_b == nullptr || a->latent_codes == nullptr || a->latent_scales == nullptr || a->rope_cache == nullptr ||
+        a->ctx_lens == nullptr || a->out == nullptr || a->workspace == nullptr) {
+        return fail(-1, "MLA decode: null pointer");
+    }
+    zllm::MlaDecodeParams p;
+    memset(&p, 0, sizeof(p));
+    plan_mla_decode(a, &p.chunk_tokens, &p.max_chunks);
+    const MlaWorkspace w = mla_workspace(a, p.max_chunks);
+    if (a->workspace_bytes < w.total) {
+        return fail(-1, "MLA decode: workspace %llu bytes, need %llu", (unsigned long long)a->workspace_bytes, (unsigned long long)w.total);
+    }
+    if (a->tables != nullptr && (uint64_t)a->table_stride * a->block_tokens < a->max_ctx_len) {
+        return fail(-1, "MLA decode: table_stride=%u pages of %u tokens cannot cover max_ctx_len=%u", a->table_stride, a->block_tokens,
+                    a->max_ctx_len);
+    }
+    char* ws = (char*)a->workspace;
+    p.q = a->q;
+    p.kv_b = a->kv_b;
+    p.latent_codes = (const signed char*)a->latent_codes;
+    p.latent_scales = a->latent_scales;
+    p.rope_cache = a->rope_cache;
+    p.tables = a->tables;
+    p.ctx_lens = a->ctx_lens;
+    p.out = a->out;
+    p.absorbed = (unsigned short*)(ws + w.absorbed);
+    p.partial = (float*)(ws + w.partial);
+    p.stats = (float*)(ws + w.stats);
+    p.weighted = (float*)(ws + w.weighted);
+    p.batch = a->batch;
+    p.heads = a->heads;
+    p.q_head_dim = a->q_head_dim;
+    p.kv_head_dim = a->kv_head_dim;
+    p.latent_dim = a->latent_dim;
+    p.rope_dim = a->rope_dim;
+    p.nope_dim = a->q_head_dim - a->rope_dim;
+    p.value_dim = a->kv_head_dim - p.nope_dim;
+    p.table_stride = a->table_stride;
+    p.block_tokens = a->block_tokens;
+    p.block_shift = shift_of(a->block_tokens);
+    // 1 / sqrt(q_head_dim): the reference's scale (src/attention/mla.rs:109, kernel/cpu/mla.rs:790)
+    p.score_scale = 1.0f / sqrtf((float)a->q_head_dim);
+    p.q_dtype = a->q_dtype;
+    p.out_dtype = a->out_dtype;
+    p.out_compact = a->out_compact;
+    return hip_status(zllm::launch_mla_decode(p, (hipStream_t)stream), "MLA decode launch");
 }
 
 } // extern "C"

@@ -54,9 +54,13 @@ __device__ __forceinline__ float byte_to_f32(unsigned int w, int e)
 
 __device__ __forceinline__ float fast_tanh(float x)
 {
-    // tanh(x) = 1 - 2 / (exp(2x) + 1); saturates cleanly for large |x|
-    const float e = __builtin_amdgcn_exp2f(fminf(x * (2.0f * kLog2e), 80.0f));
-    return 1.0f - __fdividef(2.0f, e + 1.0f);
+    // small |x|: odd Taylor polynomial (the exponential form cancels to zero there);
+    // otherwise tanh(x) = 1 - 2 / (exp(2x) + 1), which saturates cleanly.
+    const float x2 = x * x;
+    const float poly = x * (1.0f + x2 * (-1.0f / 3.0f + x2 * (2.0f / 15.0f + x2 * (-17.0f / 315.0f))));
+    const float e = __builtin_amdgcn_exp2f(fminf(fabsf(x) * (2.0f * kLog2e), 80.0f));
+    const float big = copysignf(1.0f - __fdividef(2.0f, e + 1.0f), x);
+    return fabsf(x) < 0.1f ? poly : big;
 }
 
 template <int G> struct ScaleRow; // G 16-bit scales of one token / KV head
@@ -599,14 +603,14 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
 // (src/kernel/rocm/hip/tensor/attention/source.hip:1339-1362), in base 2.
 __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
 {
+    // one workgroup per (head, sequence): threads = (dim quad) x (split lane); every split lane folds
+    // its share of the splits with independent loads, then the lanes are combined through LDS.
     const unsigned int quads = p.head_dim / 4u;
-    const unsigned int heads_per_block = 256u / quads;
-    const unsigned int head = blockIdx.x * heads_per_block + threadIdx.x / quads;
+    const unsigned int lanes = 256u / quads;
     const unsigned int quad = threadIdx.x % quads;
+    const unsigned int sl = threadIdx.x / quads;
+    const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
-    if (head >= p.num_heads) {
-        return;
-    }
     const unsigned int len = p.kv_lens[b];
     unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
     first = min(first, len);
@@ -614,30 +618,66 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     const unsigned int chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
     const size_t stat_stride = (size_t)p.num_heads * 2;
-    float m = kNegInf;
-    for (unsigned int c = 0; c < chunks; ++c) {
-        m = fmaxf(m, stats[c * stat_stride]);
-    }
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    float l = 0.0f;
     const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;
     const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
-    for (unsigned int c = 0; c < chunks; ++c) {
-        const float cm = stats[c * stat_stride];
-        const float cl = stats[c * stat_stride + 1];
-        if (cl <= 0.0f) {
-            continue;
+
+    // single pass, four splits per trip with all eight loads issued before any is used
+    float m = kNegInf;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.0f;
+    for (unsigned int c0 = sl; c0 < chunks; c0 += 4u * lanes) {
+        float cm[4], cl[4];
+        f32x4 part[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned int c = min(c0 + u * lanes, chunks - 1u);
+            const bool live = c0 + u * lanes < chunks;
+            const float2 st = *(const float2*)(stats + c * stat_stride);
+            cm[u] = live ? st.x : kNegInf;
+            cl[u] = live ? st.y : 0.0f;
+            part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
-        const float w = __builtin_amdgcn_exp2f(cm - m);
-        l += cl * w;
-        acc += *(const f32x4*)(partial + c * partial_stride) * w;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (cl[u] > 0.0f) {
+                const float nm = fmaxf(m, cm[u]);
+                const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+                const float w = __builtin_amdgcn_exp2f(cm[u] - nm);
+                acc = acc * a + part[u] * w;
+                l = l * a + cl[u] * w;
+                m = nm;
+            }
+        }
     }
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    f32x4 result = acc * inv;
-    if (!(l > 0.0f)) {
-        result = f32x4{0.f, 0.f, 0.f, 0.f};
+    __shared__ float sm[256];
+    __shared__ float sl_sum[256];
+    __shared__ f32x4 sacc[256];
+    sm[threadIdx.x] = m;
+    sl_sum[threadIdx.x] = l;
+    sacc[threadIdx.x] = acc;
+    __syncthreads();
+    if (sl == 0) {
+        float gm = kNegInf;
+        for (unsigned int i = 0; i < lanes; ++i) {
+            gm = fmaxf(gm, sm[i * quads + quad]);
+        }
+        const float safe_g = gm == kNegInf ? 0.0f : gm;
+        f32x4 total = {0.f, 0.f, 0.f, 0.f};
+        float denom = 0.0f;
+        for (unsigned int i = 0; i < lanes; ++i) {
+            const float li = sl_sum[i * quads + quad];
+            if (li > 0.0f) {
+                const float w = __builtin_amdgcn_exp2f(sm[i * quads + quad] - safe_g);
+                denom += li * w;
+                total += sacc[i * quads + quad] * w;
+            }
+        }
+        f32x4 result = {0.f, 0.f, 0.f, 0.f};
+        if (denom > 0.0f && denom < __builtin_inff()) {
+            result = total * (1.0f / denom);
+        }
+        *(f32x4*)(p.out + ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u) = result;
     }
-    *(f32x4*)(p.out + ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u) = result;
 }
 
 template <int D, int SDT, bool QSPLIT>
@@ -662,7 +702,7 @@ template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtyp
 
 } // namespace
 
-hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, hipStream_t stream)
+hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream)
 {
     const unsigned int max_waves = p.head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
     const unsigned int waves = p.num_kv_heads < max_waves ? p.num_kv_heads : max_waves;
@@ -673,7 +713,9 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const bool fast = pow2 && p.block_tokens >= 16u && p.ring_capacity % 16u == 0;
     hipError_t err = hipSuccess;
-    if (kv_format == 0) {
+    if (stages == 2u) {
+        // merge only
+    } else if (kv_format == 0) {
         switch (p.head_dim) {
         case 64: err = launch_q8_d<64>(p, scale_dtype, fast, grid, block, stream); break;
         case 128: err = launch_q8_d<128>(p, scale_dtype, fast, grid, block, stream); break;
@@ -698,12 +740,15 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_
         }
         err = hipGetLastError();
     }
-    if (err != hipSuccess) {
+    if (err != hipSuccess || stages == 1u) {
         return err;
     }
-    const unsigned int quads = p.head_dim / 4u;
-    const unsigned int heads_per_block = 256u / quads;
-    gqa_decode_merge<<<dim3((p.num_heads + heads_per_block - 1) / heads_per_block, p.batch), dim3(256), 0, stream>>>(p);
+    return launch_split_merge(p, stream);
+}
+
+hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)
+{
+    gqa_decode_merge<<<dim3(p.num_heads, p.batch), dim3(256), 0, stream>>>(p);
     return hipGetLastError();
 }
 
