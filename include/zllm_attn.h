@@ -66,6 +66,8 @@ enum { ZLLM_ROTARY_INTERLEAVED = 0, ZLLM_ROTARY_SPLIT_HALF = 1 };
 /* Stage selection for the split-KV entry points. */
 enum { ZLLM_STAGE_ALL = 0, ZLLM_STAGE_PARTIAL = 1, ZLLM_STAGE_MERGE = 2 };
 
+enum { ZLLM_MLA_ABSORB = 1, ZLLM_MLA_PARTIAL = 2, ZLLM_MLA_MERGE = 4, ZLLM_MLA_PROJECT = 8 };
+
 #define ZLLM_GROUP_SIZE 64 /* src/kv_cache/mod.rs:29 DEFAULT_GROUP_SIZE */
 
 /* Library / device bring-up.  Optional: every entry point works without it.
@@ -283,6 +285,10 @@ typedef struct zllm_mla_decode_args {
     int q_dtype;                  /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
     int out_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
     int out_compact;
+    uint32_t stage_mask;          /* 0 = whole chain; else OR of ZLLM_MLA_ABSORB / _PARTIAL / _MERGE /
+                                     _PROJECT: run only those stages on the records already in the
+                                     workspace (shard exchange, per-stage timing;
+                                     cf. paged_mla.rs:3068-3081 per-stage profile) */
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
 ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);

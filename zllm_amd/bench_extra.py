@@ -1,0 +1,146 @@
+"""Secondary bench workloads (`bench.py --workload ...`): MLA decode at 64K context and chunked GQA prefill.
+Same one-JSON-line contract as the default workload."""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import os
+import time
+
+import numpy as np
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+HBM_PEAK_GBPS = 8000.0
+
+
+def _event_ms(fn, steps):
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def _wall_ms(fn, steps):
+    import torch
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def run_mla_decode(args):
+    """BASELINE.json configs[3]: B=4, 128 heads, latent 512 (Q8g64, bf16 scales) + rope 64 (bf16), ctx 65,536,
+    bf16 queries, softmax scale 1/sqrt(192); W_kv_b ~ N(0, 1/512) in bf16; 64-token pages in a random permutation."""
+    import torch
+
+    import oracle as O
+    from zllm_amd import capi, ops
+
+    dev = "cuda"
+    batch, heads, nope, rope, value, latent, bt, ctx = 4, 128, 128, 64, 128, 512, 64, 65536
+    lens = [ctx] * batch
+    ops.init(0)
+    rng = np.random.default_rng(args.seed)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed)
+    need_blocks = batch * ctx // bt
+    pool_blocks = max(need_blocks * 8, need_blocks + 1)
+    rows = pool_blocks * bt
+    codes = torch.empty((rows, latent), dtype=torch.int8, device=dev)
+    scales = torch.empty((rows, latent // 64), dtype=torch.int16, device=dev)
+    rope_cache = torch.empty((rows, rope), dtype=torch.int16, device=dev)
+    ids = rng.choice(pool_blocks, size=need_blocks, replace=False).astype(np.uint32).reshape(batch, -1)
+    tables = torch.from_numpy(ids.view(np.int32)).to(dev)
+    for b in range(batch):
+        for pos in range(0, ctx, 8192):
+            lat = torch.randn((8192, latent), generator=gen, device=dev)
+            kr = torch.randn((8192, rope), generator=gen, device=dev)
+            ops.mla_append(lat, kr, codes, scales, rope_cache, tables[b], pos, bt)
+    q = torch.randn((batch, heads * (nope + rope)), generator=gen, device=dev).to(torch.bfloat16)
+    kv_b = (torch.randn((heads * (nope + value), latent), generator=gen, device=dev) / np.sqrt(latent)).to(torch.bfloat16)
+    lens_dev = torch.tensor(lens, dtype=torch.int32, device=dev)
+    call, out, workspace = ops.mla_decode_args(q, kv_b, codes, scales, rope_cache, tables, lens_dev, heads, nope + rope, nope + value,
+                                               latent, rope, bt, ctx, out_dtype=torch.float32, out_compact=True)
+    lib = capi.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(mask):
+        def fn():
+            call.stage_mask = mask
+            capi.check(lib.zllm_attn_mla_decode(C.byref(call), stream))
+        return fn
+
+    for _ in range(args.warmup):
+        run(0)()
+    ms_step = _wall_ms(run(0), args.steps)
+    ms_events = _event_ms(run(0), args.steps)
+    stage_ms = {name: _event_ms(run(mask), args.steps) for name, mask in
+                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge", capi.MLA_MERGE), ("project", capi.MLA_PROJECT))}
+    run(0)()
+    torch.cuda.synchronize()
+    flops = sum(lens) * heads * (2 * (latent + rope) + 2 * latent)  # QK^T over 576 + PV over 512, multiply-add = 2
+    kv_bytes = sum(lens) * (latent + latent // 64 * 2 + rope * 2)   # 656 B/token
+    tflops_call = flops / (ms_step * 1e-3) / 1e12
+    achieved = flops / (stage_ms["partial"] * 1e-3) / 1e12
+    record = {
+        "metric": "MLA decode attn TFLOP/s (% of bf16 MFMA peak) + tokens/s at 64K ctx, 1 GPU",
+        "value": round(tflops_call, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C4 absorbed MLA decode, B=4, 128 heads, latent 512 Q8g64 + rope 64 bf16, ctx 65536, 64-token pages",
+                   "algorithmic_flops_per_call": flops, "kv_bytes_per_call": kv_bytes, "seed": args.seed,
+                   "q_head_dim": nope + rope, "kv_head_dim": nope + value},
+        "pct_of_mfma_peak": round(100.0 * tflops_call / MFMA_BF16_PEAK_TFLOPS, 2),
+        "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
+        "effective_kv_gbps": round(kv_bytes / (ms_step * 1e-3) / 1e9, 1),
+        "ms_per_step_events": round(ms_events, 5),
+        "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
+        "roofline": {"bound": "mfma", "kernel": "mla_partial", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel_ms": round(stage_ms["partial"], 5)},
+    }
+    if not args.no_cpu_baseline:
+        # CPU oracle (port of mla_attention_absorbed_q8_history) on a bounded sample: sequence 0, the first 8 heads,
+        # the first 16,384 tokens of context.
+        sample_heads, sample_ctx = 8, 16384
+        threads = O.set_threads(min(len(os.sched_getaffinity(0)), 16))
+        h_codes = ops.gather_rows(codes, tables[0], 0, sample_ctx, latent, bt).cpu().numpy()
+        h_scales = ops.gather_rows(scales, tables[0], 0, sample_ctx, latent // 64 * 2, bt).cpu().numpy().view(np.uint16)
+        h_rope = ops.gather_rows(rope_cache, tables[0], 0, sample_ctx, rope * 2, bt).cpu().numpy().view(np.uint16)
+        spec = O.MlaSpec(latent, rope, sample_heads * (nope + rope), sample_heads * (nope + value), sample_heads)
+        q_bits = q[0].view(torch.int16).cpu().numpy().view(np.uint16)[: sample_heads * (nope + rope)].reshape(1, -1)
+        w = kv_b.float().cpu().numpy()[: sample_heads * (nope + value)]
+        t0 = time.perf_counter()
+        rc, _, out_f, _ = O.mla_absorbed_q8_history(spec, q_bits, 1, sample_ctx - 1, h_codes, h_scales, 64, h_rope, sample_ctx, w)
+        seconds = time.perf_counter() - t0
+        assert rc == 0
+        cpu_flops = sample_ctx * sample_heads * (2 * (latent + rope) + 2 * latent)
+        record["cpu_baseline"] = {"value": round(cpu_flops / seconds / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                                  "sample": f"sequence 0, heads 0..{sample_heads - 1}, first {sample_ctx} tokens; {seconds:.2f}s "
+                                            f"(one task per head, so {min(threads, sample_heads)} cores busy)"}
+        # parity of the same slice on the device (separate small call)
+        small = ops.mla_decode(q[0:1, : sample_heads * (nope + rope)].contiguous(), kv_b[: sample_heads * (nope + value)].contiguous(),
+                               codes, scales, rope_cache, tables[0:1].contiguous(), torch.tensor([sample_ctx], dtype=torch.int32, device=dev),
+                               sample_heads, nope + rope, nope + value, latent, rope, bt, sample_ctx)
+        record["parity_vs_oracle_max_abs"] = float(np.abs(small.cpu().numpy().ravel() - out_f).max())
+    print(json.dumps(record))
+
+
+def run(args):
+    if args.workload == "mla_decode_64k":
+        run_mla_decode(args)
+    elif args.workload == "gqa_prefill_chunk":
+        from zllm_amd import bench_prefill
+
+        bench_prefill.run(args)
+    else:
+        raise SystemExit(f"unknown workload {args.workload}")

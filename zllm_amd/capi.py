@@ -18,6 +18,7 @@ KV_Q8G64, KV_F16 = 0, 1
 QUANT_ROCM_MLA, QUANT_METAL_GQA, QUANT_CUDA_GQA = 0, 1, 2
 ROTARY_INTERLEAVED, ROTARY_SPLIT_HALF = 0, 1
 STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
+MLA_ABSORB, MLA_PARTIAL, MLA_MERGE, MLA_PROJECT = 1, 2, 4, 8
 
 _u32, _u64, _f32, _int, _ptr = C.c_uint32, C.c_uint64, C.c_float, C.c_int, C.c_void_p
 
@@ -67,7 +68,7 @@ class MlaDecodeArgs(C.Structure):
                 ("tables", _ptr), ("ctx_lens", _ptr), ("out", _ptr), ("workspace", _ptr), ("workspace_bytes", _u64),
                 ("batch", _u32), ("heads", _u32), ("q_head_dim", _u32), ("kv_head_dim", _u32), ("latent_dim", _u32),
                 ("rope_dim", _u32), ("table_stride", _u32), ("max_ctx_len", _u32), ("block_tokens", _u32),
-                ("q_dtype", _int), ("out_dtype", _int), ("out_compact", _int)]
+                ("q_dtype", _int), ("out_dtype", _int), ("out_compact", _int), ("stage_mask", _u32)]
 
 
 # every symbol include/zllm_attn.h declares: name -> (restype, argtypes)

@@ -128,6 +128,9 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
     if ((a->q_dtype != ZLLM_DTYPE_F32 && a->q_dtype != ZLLM_DTYPE_BF16) || (a->out_dtype != ZLLM_DTYPE_F32 && a->out_dtype != ZLLM_DTYPE_BF16)) {
         return fail(-1, "MLA decode: q_dtype / out_dtype must be f32 or bf16");
     }
+    if (a->stage_mask > 15u) {
+        return fail(-1, "MLA decode: unknown stage_mask %u", a->stage_mask);
+    }
     return 0;
 }
 
@@ -456,7 +459,7 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     p.q_dtype = a->q_dtype;
     p.out_dtype = a->out_dtype;
     p.out_compact = a->out_compact;
-    return hip_status(zllm::launch_mla_decode(p, (hipStream_t)stream), "MLA decode launch");
+    return hip_status(zllm::launch_mla_decode(p, a->stage_mask, (hipStream_t)stream), "MLA decode launch");
 }
 
 } // extern "C"

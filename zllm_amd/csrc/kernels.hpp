@@ -112,7 +112,7 @@ hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);
 // kv_format: 0 = Q8g64, 1 = f16; scale_dtype: 0 = bf16, 1 = f16 (Q8 only).
 hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream);
 hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream);
-hipError_t launch_mla_decode(const MlaDecodeParams& p, hipStream_t stream);
+hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream);
 // LSE combine of split records: uses kv_lens, first_visible, partial, stats, out, batch, num_heads,
 // head_dim, chunk_tokens, max_chunks of the parameter block.
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream);

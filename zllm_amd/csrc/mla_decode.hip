@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
 {
     constexpr int MT = 32 / DSPLIT; // output M tiles (16 latent columns each) of this workgroup
     __shared__ __align__(16) unsigned char lds[2 * kTileBytes];
-    __shared__ __align__(16) float lds_scale[2][kStepTokens][8];
+    __shared__ __align__(16) float lds_scale[2][8][kStepTokens]; // [buffer][group][token]
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
         const unsigned long long row = row_of(t0 + rope_t);
         r.rope = *(const u32x4*)(p.rope_cache + row * kRope + rope_c * 8u);
     };
-    auto store_step = [&](const StepRegs& r, unsigned char* tile, float (*scale_tile)[8]) __attribute__((always_inline)) {
+    auto store_step = [&](const StepRegs& r, unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const unsigned int row = t_lo + 8u * i;
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
             *(u32x4*)(tile + tile_offset(row, cc * 2u)) = out[0];
             *(u32x4*)(tile + tile_offset(row, cc * 2u + 1u)) = out[1];
             if ((cc & 3u) == 0) {
-                scale_tile[row][cc >> 2] = bf16_bits_to_f32(r.scale[i]);
+                scale_tile[cc >> 2][row] = bf16_bits_to_f32(r.scale[i]);
             }
         }
         *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = r.rope;
@@ -232,24 +232,16 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
     }
 
     constexpr int GROUPS = 8 / DSPLIT; // scale groups among this workgroup's output columns
-    auto compute_step = [&](const unsigned char* tile, const float (*scale_tile)[8], unsigned int t0) __attribute__((always_inline)) {
+    auto compute_step = [&](const unsigned char* tile, const float (*scale_tile)[kStepTokens], unsigned int t0) __attribute__((always_inline)) {
         // ---- S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope -----------------------------
         f32x4 s[2][TPW];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            // group scales of this lane's four token rows (same address for all lanes of a 16-lane group)
-            f32x4 sc_lo[4], sc_hi[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float* row = scale_tile[i * 16 + 4 * j + r];
-                sc_lo[r] = *(const f32x4*)(row);
-                sc_hi[r] = *(const f32x4*)(row + 4);
-            }
-            // rope columns (k-steps 16, 17): unscaled
 #pragma unroll
             for (int h = 0; h < TPW; ++h) {
                 s[i][h] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
+            // rope columns (k-steps 16, 17): unscaled
 #pragma unroll
             for (int ks = 16; ks < 18; ++ks) {
                 Frag kf;
@@ -259,11 +251,14 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
                     s[i][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[h][ks].b, s[i][h], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 Frag k0, k1;
                 k0.u = *(const u32x4*)(tile + qk_base[0] + (i * 16 * kRowBytes + g * 128));
                 k1.u = *(const u32x4*)(tile + qk_base[1] + (i * 16 * kRowBytes + g * 128));
+                // group scales of this lane's four token rows (one address per 16-lane group)
+                const f32x4 gs = *(const f32x4*)(&scale_tile[g][i * 16 + 4 * j]);
 #pragma unroll
                 for (int h = 0; h < TPW; ++h) {
                     f32x4 d = {0.f, 0.f, 0.f, 0.f};
@@ -271,17 +266,14 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
                     d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[h][2 * g + 1].b, d, 0, 0, 0);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const float scale = g < 4 ? sc_lo[r][g & 3] : sc_hi[r][g & 3];
-                        s[i][h][r] = fmaf(d[r], scale, s[i][h][r]);
+                        s[i][h][r] = fmaf(d[r], gs[r], s[i][h][r]);
                     }
                 }
-                if ((g & 1) == 1) {
-                    __builtin_amdgcn_sched_barrier(0); // bound the number of LDS fragments kept live
-                }
+                __builtin_amdgcn_sched_barrier(0); // bound the number of LDS fragments kept live
             }
         }
-        // ---- online softmax per head column; P'_g = bf16(p * scale_g) -------------------------------
-        Frag pf[TPW][GROUPS];
+        // ---- online softmax per head column ---------------------------------------------------------
+        float pr[TPW][8];
         bool rescale = false;
         float alpha[TPW];
 #pragma unroll
@@ -304,24 +296,13 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
             alpha[h] = __builtin_amdgcn_exp2f(run_max[h] - safe_max);
             rescale = rescale || (alpha[h] != 1.0f && run_sum[h] != 0.0f);
             float step_sum = 0.0f;
-            float pr[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
-                step_sum += pr[e];
+                pr[h][e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+                step_sum += pr[h][e];
             }
             run_sum[h] = run_sum[h] * alpha[h] + step_sum;
             run_max[h] = new_max;
-#pragma unroll
-            for (int g = 0; g < GROUPS; ++g) {
-                const unsigned int gg = dsplit * GROUPS + g;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float s0 = scale_tile[16 * ((2 * e) >> 2) + 4 * j + ((2 * e) & 3)][gg];
-                    const float s1 = scale_tile[16 * ((2 * e + 1) >> 2) + 4 * j + ((2 * e + 1) & 3)][gg];
-                    pf[h][g].u[e] = pack_bf16_rne(pr[2 * e] * s0, pr[2 * e + 1] * s1);
-                }
-            }
         }
         if (__any(rescale)) {
 #pragma unroll
@@ -332,26 +313,40 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
                 }
             }
         }
-        // ---- O^T += codes^T . P' -------------------------------------------------------------------
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g) --------------------------------------
         const unsigned char* pv_tile = tile + dsplit * (MT / 4) * 128;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const unsigned char* at = pv_tile + pv_base[t & 3] + (t >> 2) * 128;
-            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
-            union {
-                s16x4 s[2];
-                bf16x8 b;
-            } vf;
-            vf.s[0] = lo;
-            vf.s[1] = hi;
+        for (int g = 0; g < GROUPS; ++g) {
+            const float* gs_row = scale_tile[dsplit * GROUPS + g];
+            const f32x4 gs0 = *(const f32x4*)(gs_row + 4 * j);
+            const f32x4 gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
+            Frag pf[TPW];
 #pragma unroll
             for (int h = 0; h < TPW; ++h) {
-                acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pf[h][t >> 2].b, acc[h][t], 0, 0, 0);
+                pf[h].u[0] = pack_bf16_rne(pr[h][0] * gs0[0], pr[h][1] * gs0[1]);
+                pf[h].u[1] = pack_bf16_rne(pr[h][2] * gs0[2], pr[h][3] * gs0[3]);
+                pf[h].u[2] = pack_bf16_rne(pr[h][4] * gs1[0], pr[h][5] * gs1[1]);
+                pf[h].u[3] = pack_bf16_rne(pr[h][6] * gs1[2], pr[h][7] * gs1[3]);
             }
-            if ((t & 3) == 3) {
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                const int t = g * 4 + tt;
+                const unsigned char* at = pv_tile + pv_base[tt] + g * 128;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+                union {
+                    s16x4 s[2];
+                    bf16x8 b;
+                } vf;
+                vf.s[0] = lo;
+                vf.s[1] = hi;
+#pragma unroll
+                for (int h = 0; h < TPW; ++h) {
+                    acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pf[h].b, acc[h][t], 0, 0, 0);
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -430,40 +425,51 @@ __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
 
 } // namespace
 
-hipError_t launch_mla_decode(const MlaDecodeParams& p, hipStream_t stream)
+hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
 {
-    mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) {
-        return err;
+    const unsigned int stages = stage_mask == 0 ? 15u : stage_mask;
+    hipError_t err = hipSuccess;
+    if (stages & 1u) {
+        mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        err = hipGetLastError();
+        if (err != hipSuccess) {
+            return err;
+        }
     }
-    if (p.heads > 64) {
-        mla_partial<2, 2><<<dim3(p.max_chunks, 2 * ((p.heads + 127) / 128), p.batch), dim3(256), 0, stream>>>(p);
-    } else {
-        mla_partial<1, 1><<<dim3(p.max_chunks, 1, p.batch), dim3(256), 0, stream>>>(p);
+    if (stages & 2u) {
+        if (p.heads > 64) {
+            mla_partial<2, 2><<<dim3(p.max_chunks, 2 * ((p.heads + 127) / 128), p.batch), dim3(256), 0, stream>>>(p);
+        } else {
+            mla_partial<1, 1><<<dim3(p.max_chunks, 1, p.batch), dim3(256), 0, stream>>>(p);
+        }
+        err = hipGetLastError();
+        if (err != hipSuccess) {
+            return err;
+        }
     }
-    err = hipGetLastError();
-    if (err != hipSuccess) {
-        return err;
+    if (stages & 4u) {
+        // LSE combine into weighted[b, h, 0:512] (f32)
+        GqaDecodeParams mp = {};
+        mp.kv_lens = p.ctx_lens;
+        mp.first_visible = nullptr;
+        mp.out = p.weighted;
+        mp.partial = p.partial;
+        mp.stats = p.stats;
+        mp.batch = p.batch;
+        mp.num_heads = p.heads;
+        mp.head_dim = p.latent_dim;
+        mp.chunk_tokens = p.chunk_tokens;
+        mp.max_chunks = p.max_chunks;
+        err = launch_split_merge(mp, stream);
+        if (err != hipSuccess) {
+            return err;
+        }
     }
-    // LSE combine into weighted[b, h, 0:512] (f32)
-    GqaDecodeParams mp = {};
-    mp.kv_lens = p.ctx_lens;
-    mp.first_visible = nullptr;
-    mp.out = p.weighted;
-    mp.partial = p.partial;
-    mp.stats = p.stats;
-    mp.batch = p.batch;
-    mp.num_heads = p.heads;
-    mp.head_dim = p.latent_dim;
-    mp.chunk_tokens = p.chunk_tokens;
-    mp.max_chunks = p.max_chunks;
-    err = launch_split_merge(mp, stream);
-    if (err != hipSuccess) {
-        return err;
+    if (stages & 8u) {
+        mla_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        err = hipGetLastError();
     }
-    mla_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
-    return hipGetLastError();
+    return err;
 }
 
 } // namespace zllm
