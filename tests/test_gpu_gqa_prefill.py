@@ -1,0 +1,103 @@
+"""Parity of chunked-prefill GQA attention (new chunk quantized into fresh pages, then attended causally against the
+Q8g64 prefix) with the CPU oracle `prefill_attention_at_visible_with_dot_f32` (src/attention/gqa.rs:243-282)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from tests.cases import assert_attention_close, draw_tables, to_torch_bf16, upload
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
+             out_dtype=None, scale=None):
+    from zllm_amd import capi, ops
+
+    d = 128
+    out_dtype = out_dtype or torch.float32
+    rng = np.random.default_rng(seed)
+    cols = hkv * d
+    total = prefix + chunk
+    tables, pool_blocks = draw_tables(rng, [total], block_tokens)
+    rows = pool_blocks * block_tokens
+    sdt = O.SCALE_F16 if rule == O.RULE_METAL_GQA else O.SCALE_BF16
+    k = rng.standard_normal((total, cols)).astype(np.float32)
+    v = rng.standard_normal((total, cols)).astype(np.float32)
+    # the chunk's K/V arrive as bf16 activations
+    k[prefix:] = O.bf16_to_f32(O.f32_to_bf16(k[prefix:]))
+    v[prefix:] = O.bf16_to_f32(O.f32_to_bf16(v[prefix:]))
+    planes = {n: np.zeros((rows, cols if "codes" in n else cols // 64), dtype=np.int8 if "codes" in n else np.uint16)
+              for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    # prefix already cached (oracle quantizer); host copy of the full cache for the oracle
+    O.q8g64_append_paged(rule, k, planes["k_codes"], planes["k_scales"], tables[0], 0, block_tokens)
+    O.q8g64_append_paged(rule, v, planes["v_codes"], planes["v_scales"], tables[0], 0, block_tokens)
+    dev = {n: upload(a) for n, a in planes.items()}
+    table = upload(tables[0])
+    # wipe the chunk's pages on the device, then let the library quantize the new rows into them
+    first_new_block = prefix // block_tokens
+    for n in dev:
+        for blk in tables[0][first_new_block + (1 if prefix % block_tokens else 0):]:
+            dev[n][int(blk) * block_tokens:(int(blk) + 1) * block_tokens] = 0
+    kc = to_torch_bf16(O.f32_to_bf16(k[prefix:]), "cuda")
+    vc = to_torch_bf16(O.f32_to_bf16(v[prefix:]), "cuda")
+    ops.q8g64_append(kc, dev["k_codes"], dev["k_scales"], table, prefix, block_tokens, rule)
+    ops.q8g64_append(vc, dev["v_codes"], dev["v_scales"], table, prefix, block_tokens, rule)
+    torch.cuda.synchronize()
+    for n in dev:  # appended bytes == oracle bytes on every row the sequence owns
+        got = ops.gather_rows(dev[n], table, 0, total, planes[n].shape[1] * planes[n].itemsize, block_tokens).cpu().numpy()
+        want = O.gather_rows_bytes(planes[n], tables[0], block_tokens, 0, total, planes[n].shape[1] * planes[n].itemsize)
+        assert np.array_equal(got, want), n
+    q = rng.standard_normal((chunk, hq * d)).astype(np.float32)
+    q_bits = O.f32_to_bf16(q)
+    q = O.bf16_to_f32(q_bits) if q_bf16 else q
+    scale = scale or 1.0 / np.sqrt(d)
+    out = ops.gqa_prefill_chunk(to_torch_bf16(q_bits, "cuda") if q_bf16 else upload(q), dev["k_codes"], dev["k_scales"], dev["v_codes"],
+                                dev["v_scales"], table, prefix, hq, hkv, d, block_tokens, scale, window=window, softcap=softcap,
+                                scale_dtype=sdt, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, tables[0], block_tokens, 0, total, cols)
+    vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, tables[0], block_tokens, 0, total, cols)
+    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
+    assert rc == 0
+    return out, want
+
+
+@pytest.mark.parametrize("prefix,chunk,hq,hkv", [(1000, 200, 64, 8), (0, 77, 8, 2), (333, 1, 16, 4), (50, 300, 8, 8), (700, 65, 12, 3),
+                                                  (129, 40, 32, 1)])
+def test_prefill_chunk_matches_oracle(prefix, chunk, hq, hkv):
+    out, want = run_case(prefix + chunk, prefix, chunk, hq, hkv)
+    print("prefill", prefix, chunk, hq, hkv, assert_attention_close(out.cpu().numpy(), want, f"prefix={prefix} chunk={chunk} {hq}/{hkv}"))
+
+
+def test_prefill_config5_shape_at_oracle_size():
+    """BASELINE config 5 geometry (64q/8kv, d=128, bf16 activations, 16-token pages, chunk into fresh pages) with a
+    3,000-token prefix and a 256-row chunk, which the CPU oracle finishes in seconds."""
+    out, want = run_case(5, 3000, 256, 64, 8)
+    print("config5-small", assert_attention_close(out.cpu().numpy(), want, "config 5 (small)"))
+
+
+@pytest.mark.parametrize("window", [1, 64, 500])
+def test_prefill_sliding_window(window):
+    out, want = run_case(60 + window, 900, 150, 16, 4, window=window)
+    assert_attention_close(out.cpu().numpy(), want, f"window={window}")
+
+
+def test_prefill_softcap_pages_and_outputs():
+    out, want = run_case(71, 400, 100, 16, 8, softcap=30.0, block_tokens=64, rule=O.RULE_ROCM_MLA, scale=0.3)
+    assert_attention_close(out.cpu().numpy(), want, "softcap + bf16 scales + 64-token pages")
+    out, want = run_case(72, 200, 50, 8, 2, block_tokens=1, q_bf16=False)
+    assert_attention_close(out.cpu().numpy(), want, "1-token pages, f32 queries (rounded to bf16 operands)", atol=4e-3)
+    out, want = run_case(73, 200, 50, 8, 2, out_dtype=torch.bfloat16)
+    got = out.float().cpu().numpy()
+    assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 2e-3
+
+
+def test_prefill_rejects_unsupported_shapes():
+    from zllm_amd import capi, ops
+
+    z = torch.zeros((16, 64), dtype=torch.int8, device="cuda")
+    s = torch.zeros((16, 1), dtype=torch.int16, device="cuda")
+    q = torch.zeros((1, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(capi.ZllmAttnError, match="head_dim 128"):
+        ops.gqa_prefill_chunk(q, z, s, z, s, None, 0, 1, 1, 64, 16, 1.0)

@@ -462,4 +462,78 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     return hip_status(zllm::launch_mla_decode(p, a->stage_mask, (hipStream_t)stream), "MLA decode launch");
 }
 
+/* ---- GQA chunked prefill ---------------------------------------------------------------- */
+
+static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
+{
+    if (a == nullptr) {
+        return fail(-1, "GQA prefill: null args");
+    }
+    // shape rules of try_block_attention_resident_f32 (tensor/attention.rs:727-745)
+    if (a->rows == 0 || a->num_heads == 0 || a->num_kv_heads == 0 || a->num_heads % a->num_kv_heads != 0) {
+        return fail(-1, "GQA prefill: invalid shape rows=%u heads=%u/%u", a->rows, a->num_heads, a->num_kv_heads);
+    }
+    if (a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64) {
+        return fail(-1, "GQA prefill: this build handles head_dim 128 over a Q8g64 cache (got dim=%u format=%d)", a->head_dim, a->kv_format);
+    }
+    if (a->num_heads / a->num_kv_heads > 256) {
+        return fail(-1, "GQA prefill: at most 256 query heads per KV head");
+    }
+    if (a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
+        return fail(-1, "GQA prefill: Q8g64 scales must be bf16 or f16 (got %d)", a->scale_dtype);
+    }
+    if (a->block_tokens == 0 || (uint64_t)a->position + a->rows > 0xffffffffull) {
+        return fail(-1, "GQA prefill: block_tokens must be non-zero and position + rows fit u32");
+    }
+    if (!isfinite(a->score_scale) || a->score_scale <= 0.0f || !(a->softcap >= 0.0f) || !isfinite(a->softcap)) {
+        return fail(-1, "GQA prefill: invalid score_scale=%g softcap=%g", (double)a->score_scale, (double)a->softcap);
+    }
+    if (a->q_dtype < ZLLM_DTYPE_F32 || a->q_dtype > ZLLM_DTYPE_F16 || a->out_dtype < ZLLM_DTYPE_F32 || a->out_dtype > ZLLM_DTYPE_F16) {
+        return fail(-1, "GQA prefill: unknown q_dtype %d / out_dtype %d", a->q_dtype, a->out_dtype);
+    }
+    return 0;
+}
+
+uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* a)
+{
+    /* the prefill kernel keeps all of its state on chip */
+    (void)validate_gqa_prefill(a);
+    return 0;
+}
+
+int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t stream)
+{
+    const int rc = validate_gqa_prefill(a);
+    if (rc != 0) {
+        return rc;
+    }
+    if (a->q == nullptr || a->k_plane == nullptr || a->k_scales == nullptr || a->v_plane == nullptr || a->v_scales == nullptr ||
+        a->out == nullptr) {
+        return fail(-1, "GQA prefill: null pointer");
+    }
+    zllm::GqaPrefillParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q;
+    p.k_plane = (const unsigned char*)a->k_plane;
+    p.k_scales = (const unsigned char*)a->k_scales;
+    p.v_plane = (const unsigned char*)a->v_plane;
+    p.v_scales = (const unsigned char*)a->v_scales;
+    p.table = a->table;
+    p.out = a->out;
+    p.rows = a->rows;
+    p.position = a->position;
+    p.window = a->window;
+    p.num_heads = a->num_heads;
+    p.num_kv_heads = a->num_kv_heads;
+    p.head_dim = a->head_dim;
+    p.group = a->num_heads / a->num_kv_heads;
+    p.block_tokens = a->block_tokens;
+    p.block_shift = shift_of(a->block_tokens);
+    p.score_scale = a->score_scale;
+    p.softcap = a->softcap;
+    p.q_dtype = a->q_dtype;
+    p.out_dtype = a->out_dtype;
+    return hip_status(zllm::launch_gqa_prefill(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA prefill launch");
+}
+
 } // extern "C"

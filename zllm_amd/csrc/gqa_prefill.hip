@@ -1,6 +1,368 @@
-#include "../../include/zllm_attn.h"
+// Chunked-prefill GQA attention over a paged Q8g64 KV cache — gfx950, bf16 MFMA.
+//
+// T query rows appended at `position` attend the cached prefix plus the chunk itself (causal,
+// optional sliding window).  Replaces the per-(row, head) block attention the reference runs for this
+// case (src/backend/rocm/attention.rs:2232-2242 -> tensor/attention/source.hip:618-686).
+//
+// A workgroup (4 waves) owns one KV head and a tile of query rows; its 256 MFMA columns enumerate
+// (row, head-in-group) pairs, 64 per wave, so one K/V tile serves every query head of the group.
+// Per 32-token step the workgroup converts the K and V codes ONCE into LDS as bf16 integers (exact)
+// with their f32 group scales beside them; each wave then runs
+//   S^T[token, col]  = sum_g k_scale[token, g] * (Kcodes_g[token, :] . Q_g[col, :])   (MFMA, exact products)
+//   online softmax per column (wave shuffles)
+//   O^T[dim, col]   += Vcodes^T[dim, token] . P'_g[token, col],  P'_g = p * v_scale_g as bf16 hi + lo
+// K is read from LDS with ds_read_b128, V transposed with ds_read_b64_tr_b16; a 16-byte XOR swizzle
+// keeps both conflict-free.
+#include "common.hpp"
 #include "kernels.hpp"
-extern "C" {
-uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args*) { return 0; }
-int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args*, zllm_stream_t) { return -3; }
+
+namespace zllm {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kStep = 32;                 // tokens per step
+constexpr int kD = 128;                   // head_dim handled by this kernel
+constexpr int kRowBytes = kD * 2;         // one token of one KV head as bf16
+constexpr int kTileBytes = kStep * kRowBytes; // 8 KiB
+constexpr int kColTiles = 4;              // 16-column MFMA tiles per wave
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+union Frag {
+    u32x4 u;
+    bf16x8 b;
+};
+
+__device__ __forceinline__ unsigned int swz(unsigned int row)
+{
+    const unsigned int x = row & 7u;
+    return ((x & 3u) << 1) | (x >> 2);
 }
+
+__device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned int chunk)
+{
+    return row * kRowBytes + ((chunk ^ swz(row)) << 4);
+}
+
+__device__ __forceinline__ float soft_tanh(float x)
+{
+    const float x2 = x * x;
+    const float poly = x * (1.0f + x2 * (-1.0f / 3.0f + x2 * (2.0f / 15.0f + x2 * (-17.0f / 315.0f))));
+    const float e = __builtin_amdgcn_exp2f(fminf(fabsf(x) * (2.0f * kLog2e), 80.0f));
+    const float big = copysignf(1.0f - __fdividef(2.0f, e + 1.0f), x);
+    return fabsf(x) < 0.1f ? poly : big;
+}
+
+struct StepRegs {
+    u32x4 k, v;            // 16 codes each
+    unsigned int ks, vs;   // two 16-bit scales each (groups 0, 1)
+};
+
+template <int SDT>
+__global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
+{
+    __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
+    __shared__ __align__(16) unsigned char lds_v[2][kTileBytes];
+    __shared__ __align__(16) float lds_ks[2][2][kStep]; // [buffer][group][token]
+    __shared__ __align__(16) float lds_vs[2][2][kStep];
+
+    const unsigned int tid = threadIdx.x;
+    const unsigned int lane = tid & 63u;
+    const unsigned int wave = tid >> 6;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    const unsigned int kvh = blockIdx.y;
+    const unsigned int rows_per_wg = max(1u, 256u / p.group);
+    const unsigned int row0 = blockIdx.x * rows_per_wg;
+    const unsigned int cols_used = rows_per_wg * p.group;
+
+    // visible token range of the workgroup: union over its rows of key_range(position + row, kv_end)
+    const unsigned int last_row = min(row0 + rows_per_wg, p.rows) - 1u;
+    const unsigned int t_end = p.position + last_row + 1u;
+    unsigned int t_begin = 0;
+    if (p.window != 0) {
+        const unsigned int first_pos = p.position + row0 + 1u;
+        t_begin = first_pos > p.window ? first_pos - p.window : 0u;
+    }
+    t_begin &= ~31u;
+    const unsigned int steps = (t_end - t_begin + kStep - 1) / kStep;
+
+    // ---- this wave's columns and Q fragments -------------------------------------------------
+    unsigned int col_row[kColTiles], col_head[kColTiles];
+    bool col_valid[kColTiles];
+    Frag qf[kColTiles][4];
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ++ct) {
+        const unsigned int col = wave * 64u + ct * 16u + m;
+        const unsigned int r = row0 + col / p.group;
+        col_row[ct] = r;
+        col_head[ct] = kvh * p.group + col % p.group;
+        col_valid[ct] = col < cols_used && r < p.rows;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[e] = col_valid[ct] ? load_as_f32(p.q, ((size_t)r * p.num_heads + col_head[ct]) * kD + ks * 32 + j * 8 + e, p.q_dtype) : 0.0f;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                qf[ct][ks].u[e] = pack_bf16_rne(x[2 * e], x[2 * e + 1]);
+            }
+        }
+    }
+
+    const unsigned int k_row = p.num_kv_heads * kD;
+    const unsigned int s_row = p.num_kv_heads * 4u; // two 16-bit scales per KV head
+    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
+    const unsigned int last_token = t_end - 1u;
+    auto row_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned long long {
+        token = min(token, last_token);
+        if (p.table == nullptr) {
+            return token;
+        }
+        if (pow2) {
+            return ((unsigned long long)p.table[token >> p.block_shift] << p.block_shift) + (token & (p.block_tokens - 1u));
+        }
+        return (unsigned long long)p.table[token / p.block_tokens] * p.block_tokens + token % p.block_tokens;
+    };
+    const unsigned int st_token = tid >> 3; // staging: token of the step, 16-code chunk cc
+    const unsigned int cc = tid & 7u;
+    auto load_step = [&](StepRegs& r, unsigned int t0) __attribute__((always_inline)) {
+        const unsigned long long row = row_of(t0 + st_token);
+        r.k = *(const u32x4*)(p.k_plane + row * k_row + kvh * kD + cc * 16u);
+        r.v = *(const u32x4*)(p.v_plane + row * k_row + kvh * kD + cc * 16u);
+        r.ks = *(const unsigned int*)(p.k_scales + row * s_row + kvh * 4u);
+        r.vs = *(const unsigned int*)(p.v_scales + row * s_row + kvh * 4u);
+    };
+    auto convert16 = [&](const u32x4& codes, u32x4& lo, u32x4& hi) __attribute__((always_inline)) {
+        unsigned int out[8];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const unsigned int word = codes[w];
+            const float c0 = (float)(int)(signed char)(word & 0xffu);
+            const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
+            const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
+            const float c3 = (float)(int)(signed char)(word >> 24);
+            out[2 * w] = pack_bf16_trunc(c0, c1);
+            out[2 * w + 1] = pack_bf16_trunc(c2, c3);
+        }
+        lo = u32x4{out[0], out[1], out[2], out[3]};
+        hi = u32x4{out[4], out[5], out[6], out[7]};
+    };
+    auto store_step = [&](const StepRegs& r, int buf) __attribute__((always_inline)) {
+        u32x4 lo, hi;
+        convert16(r.k, lo, hi);
+        *(u32x4*)(lds_k[buf] + tile_offset(st_token, cc * 2u)) = lo;
+        *(u32x4*)(lds_k[buf] + tile_offset(st_token, cc * 2u + 1u)) = hi;
+        convert16(r.v, lo, hi);
+        *(u32x4*)(lds_v[buf] + tile_offset(st_token, cc * 2u)) = lo;
+        *(u32x4*)(lds_v[buf] + tile_offset(st_token, cc * 2u + 1u)) = hi;
+        if (cc == 0) {
+            lds_ks[buf][0][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.ks & 0xffffu));
+            lds_ks[buf][1][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.ks >> 16));
+            lds_vs[buf][0][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.vs & 0xffffu));
+            lds_vs[buf][1][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.vs >> 16));
+        }
+    };
+
+    f32x4 acc[kColTiles][8];
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ++ct) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            acc[ct][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    float run_max[kColTiles], run_sum[kColTiles];
+    unsigned int vis_lo[kColTiles], vis_hi[kColTiles]; // visible tokens [lo, hi) of each column's row
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ++ct) {
+        run_max[ct] = kNegInf;
+        run_sum[ct] = 0.0f;
+        const unsigned int pos = p.position + col_row[ct];
+        vis_hi[ct] = col_valid[ct] ? pos + 1u : 0u;
+        vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+    }
+    const float scale_log2 = p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e;
+
+    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ swz(m)) << 4), m * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
+    const unsigned int tr_row = 4u * j + (m >> 2);
+    unsigned int pv_base[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+    }
+
+    auto compute_step = [&](int buf, unsigned int t0) __attribute__((always_inline)) {
+        const unsigned char* kt = lds_k[buf];
+        const unsigned char* vt = lds_v[buf];
+        // ---- S^T = sum_g k_scale_g * (Kcodes_g . Q_g) -------------------------------------------
+        f32x4 s[2][kColTiles];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int ct = 0; ct < kColTiles; ++ct) {
+                s[i][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                Frag k0, k1;
+                k0.u = *(const u32x4*)(kt + qk_base[0] + (i * 16 * kRowBytes + g * 128));
+                k1.u = *(const u32x4*)(kt + qk_base[1] + (i * 16 * kRowBytes + g * 128));
+                const f32x4 gs = *(const f32x4*)(&lds_ks[buf][g][i * 16 + 4 * j]);
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ++ct) {
+                    f32x4 d = {0.f, 0.f, 0.f, 0.f};
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[ct][2 * g].b, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[ct][2 * g + 1].b, d, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        s[i][ct][r] = fmaf(d[r], gs[r], s[i][ct][r]);
+                    }
+                }
+            }
+        }
+        // ---- online softmax per column --------------------------------------------------------------
+        float pr[kColTiles][8];
+        float alpha[kColTiles];
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ++ct) {
+            float sc[8];
+            float step_max = kNegInf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+                float x = s[e >> 2][ct][e & 3] * scale_log2;
+                if (p.softcap > 0.0f) {
+                    x = p.softcap * soft_tanh(x / p.softcap) * kLog2e;
+                }
+                sc[e] = (token >= vis_lo[ct] && token < vis_hi[ct]) ? x : kNegInf;
+                step_max = fmaxf(step_max, sc[e]);
+            }
+            step_max = wave_max_16x4(step_max);
+            const float new_max = fmaxf(run_max[ct], step_max);
+            const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+            alpha[ct] = __builtin_amdgcn_exp2f(run_max[ct] - safe_max);
+            float step_sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                pr[ct][e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+                step_sum += pr[ct][e];
+            }
+            run_sum[ct] = run_sum[ct] * alpha[ct] + step_sum;
+            run_max[ct] = new_max;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                acc[ct][t] *= alpha[ct];
+            }
+        }
+        // ---- O^T += Vcodes^T . P'_g ----------------------------------------------------------------------
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const f32x4 gs0 = *(const f32x4*)(&lds_vs[buf][g][4 * j]);
+            const f32x4 gs1 = *(const f32x4*)(&lds_vs[buf][g][16 + 4 * j]);
+            Frag phi[kColTiles], plo[kColTiles];
+#pragma unroll
+            for (int ct = 0; ct < kColTiles; ++ct) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
+                    const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
+                    const unsigned short h0 = f32_to_bf16_bits(x0);
+                    const unsigned short h1 = f32_to_bf16_bits(x1);
+                    phi[ct].u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
+                    plo[ct].u[e] = pack_bf16_rne(x0 - bf16_bits_to_f32(h0), x1 - bf16_bits_to_f32(h1));
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                const int t = g * 4 + tt;
+                const unsigned char* at = vt + pv_base[tt] + g * 128;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+                union {
+                    s16x4 s[2];
+                    bf16x8 b;
+                } vf;
+                vf.s[0] = lo;
+                vf.s[1] = hi;
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ++ct) {
+                    f32x4 d = acc[ct][t];
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi[ct].b, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo[ct].b, d, 0, 0, 0);
+                    acc[ct][t] = d;
+                }
+            }
+        }
+    };
+
+    StepRegs regs;
+    load_step(regs, t_begin);
+    store_step(regs, 0);
+    __syncthreads();
+    for (unsigned int step = 0; step < steps; ++step) {
+        const bool more = step + 1 < steps;
+        if (more) {
+            load_step(regs, t_begin + (step + 1u) * kStep);
+        }
+        compute_step((int)(step & 1u), t_begin + step * kStep);
+        if (more) {
+            store_step(regs, (int)((step + 1u) & 1u));
+        }
+        __syncthreads();
+    }
+
+    // ---- normalise and store ------------------------------------------------------------------------
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ++ct) {
+        const float total = wave_sum_16x4(run_sum[ct]);
+        if (!col_valid[ct]) {
+            continue;
+        }
+        const float inv = (total > 0.0f && total < __builtin_inff()) ? 1.0f / total : 0.0f;
+        const size_t base = ((size_t)col_row[ct] * p.num_heads + col_head[ct]) * kD;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            f32x4 v = acc[ct][t] * inv;
+            if (inv == 0.0f) {
+                v = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            const size_t at = base + t * 16 + 4 * j;
+            if (p.out_dtype == 0) {
+                *(f32x4*)((float*)p.out + at) = v;
+            } else {
+                unsigned short* o = (unsigned short*)p.out + at;
+                u32x2 packed;
+                if (p.out_dtype == 1) {
+                    packed = u32x2{pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3])};
+                } else {
+                    packed = u32x2{(unsigned int)f32_to_f16_bits(v[0]) | ((unsigned int)f32_to_f16_bits(v[1]) << 16),
+                                   (unsigned int)f32_to_f16_bits(v[2]) | ((unsigned int)f32_to_f16_bits(v[3]) << 16)};
+                }
+                *(u32x2*)o = packed;
+            }
+        }
+    }
+}
+
+} // namespace
+
+hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream)
+{
+    if (kv_format != 0 || p.head_dim != (unsigned int)kD) {
+        return hipErrorInvalidValue;
+    }
+    const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
+    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
+    if (scale_dtype == 0) {
+        gqa_prefill_q8<0><<<grid, dim3(256), 0, stream>>>(p);
+    } else {
+        gqa_prefill_q8<1><<<grid, dim3(256), 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
+} // namespace zllm
