@@ -5,6 +5,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "kernels.hpp"
@@ -101,11 +102,13 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
 
 void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
-    const uint32_t max_waves = a->head_dim > 128 ? 4u : 8u;
+    const uint32_t max_waves = zllm::gqa_decode_max_waves(a->head_dim);
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
-    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, 2, chunk_tokens, max_chunks);
+    const char* rounds_env = getenv("ZLLM_TUNE_ROUNDS");
+    const uint32_t rounds = rounds_env ? (uint32_t)atoi(rounds_env) : 2u;
+    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, rounds, chunk_tokens, max_chunks);
 }
 
 int validate_mla_decode(const zllm_mla_decode_args* a)
@@ -137,8 +140,7 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
 void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
     // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
-    // (above 64 heads two workgroups share a split, each owning half of the output columns)
-    const uint32_t head_blocks = a->heads > 64 ? 2 * ((a->heads + 127) / 128) : 1;
+    const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     plan_splits(a->max_ctx_len, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
 }
 

@@ -99,6 +99,25 @@ __device__ __forceinline__ unsigned int pack_bf16_rne(float lo, float hi)
     return (unsigned int)f32_to_bf16_bits(lo) | ((unsigned int)f32_to_bf16_bits(hi) << 16);
 }
 
+// Same rounding for finite values, one v_cvt_pk_bf16_f32 (used where NaN payloads do not matter:
+// attention probabilities and query fragments, never cache contents).
+__device__ __forceinline__ unsigned int pack_bf16_hw(float lo, float hi)
+{
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2_t));
+}
+
+// hi + lo bf16 split of two values: hi = bf16(x), lo = bf16(x - hi); 16 significant bits together.
+__device__ __forceinline__ void split_bf16_pair(float x0, float x1, unsigned int& hi, unsigned int& lo)
+{
+    hi = pack_bf16_hw(x0, x1);
+    const float h0 = __uint_as_float(hi << 16);
+    const float h1 = __uint_as_float(hi & 0xffff0000u);
+    lo = pack_bf16_hw(x0 - h0, x1 - h1);
+}
+
 __device__ __forceinline__ float wave_max_16x4(float v)
 {
     // reduce across the four 16-lane groups of a wave (lanes l, l^16, l^32, l^48)

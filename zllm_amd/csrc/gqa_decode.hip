@@ -22,6 +22,8 @@
 // 7.8 FMA per KV byte; at 70 % of 8 TB/s that is 43 T FMA/s, above the 39 T FMA/s
 // the chip's (non-packed) FP32 vector units can issue.  On the matrix cores the
 // same work is < 15 % of peak and the vector units only convert int8 -> bf16.
+#include <stdlib.h>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -140,11 +142,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const unsigned short h0 = f32_to_bf16_bits(x[2 * e]);
-                const unsigned short h1 = f32_to_bf16_bits(x[2 * e + 1]);
-                qhi[a][hf].u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
+                unsigned int hi, lo;
+                split_bf16_pair(x[2 * e], x[2 * e + 1], hi, lo);
+                qhi[a][hf].u[e] = hi;
                 if constexpr (QSPLIT) {
-                    qlo[a][hf].u[e] = pack_bf16_rne(x[2 * e] - bf16_bits_to_f32(h0), x[2 * e + 1] - bf16_bits_to_f32(h1));
+                    qlo[a][hf].u[e] = lo;
                 }
             }
         }
@@ -296,10 +298,10 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             for (int e = 0; e < 4; ++e) {
                 const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(s.vs[2 * e].get(a));
                 const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(s.vs[2 * e + 1].get(a));
-                const unsigned short h0 = f32_to_bf16_bits(x0);
-                const unsigned short h1 = f32_to_bf16_bits(x1);
-                phi.u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
-                plo.u[e] = pack_bf16_rne(x0 - bf16_bits_to_f32(h0), x1 - bf16_bits_to_f32(h1));
+                unsigned int hi, lo;
+                split_bf16_pair(x0, x1, hi, lo);
+                phi.u[e] = hi;
+                plo.u[e] = lo;
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -702,9 +704,18 @@ template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtyp
 
 } // namespace
 
+unsigned int gqa_decode_max_waves(unsigned int head_dim)
+{
+    const char* env = getenv("ZLLM_TUNE_WAVES");
+    if (env != nullptr) {
+        return (unsigned int)atoi(env);
+    }
+    return head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
+}
+
 hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream)
 {
-    const unsigned int max_waves = p.head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
+    const unsigned int max_waves = gqa_decode_max_waves(p.head_dim);
     const unsigned int waves = p.num_kv_heads < max_waves ? p.num_kv_heads : max_waves;
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int head_blocks = (p.group + 15u) / 16u;

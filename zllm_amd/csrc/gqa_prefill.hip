@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                qf[ct][ks].u[e] = pack_bf16_rne(x[2 * e], x[2 * e + 1]);
+                qf[ct][ks].u[e] = pack_bf16_hw(x[2 * e], x[2 * e + 1]);
             }
         }
     }
@@ -270,10 +270,10 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
                 for (int e = 0; e < 4; ++e) {
                     const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
                     const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
-                    const unsigned short h0 = f32_to_bf16_bits(x0);
-                    const unsigned short h1 = f32_to_bf16_bits(x1);
-                    phi[ct].u[e] = (unsigned int)h0 | ((unsigned int)h1 << 16);
-                    plo[ct].u[e] = pack_bf16_rne(x0 - bf16_bits_to_f32(h0), x1 - bf16_bits_to_f32(h1));
+                    unsigned int hi, lo;
+                    split_bf16_pair(x0, x1, hi, lo);
+                    phi[ct].u[e] = hi;
+                    plo[ct].u[e] = lo;
                 }
             }
 #pragma unroll

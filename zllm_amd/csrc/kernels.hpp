@@ -104,6 +104,9 @@ struct MlaDecodeParams {
     int q_dtype, out_dtype, out_compact;
 };
 
+// KV heads (= waves) per GQA decode workgroup for a head dimension.
+unsigned int gqa_decode_max_waves(unsigned int head_dim);
+
 hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream);
 hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream);
 hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream);

@@ -27,6 +27,10 @@ namespace zllm {
 
 namespace {
 
+// Fences for the instruction scheduler between phases of a step: without them LDS fragment loads of
+// later phases are hoisted to the top and the kernel spills.
+#define MLA_PHASE_FENCE() __builtin_amdgcn_sched_barrier(0)
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLatent = 512;
 constexpr int kRope = 64;
@@ -91,43 +95,44 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 // ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
+// Workgroup = (split, block of 64 heads, sequence), 8 waves = 4 head tiles x 2 halves.  Wave (hw, dh) owns
+// heads [16 hw, 16 hw + 16) and output columns [256 dh, 256 dh + 256): 64 accumulator registers + 72 query
+// fragment registers per lane, so two waves share a SIMD and hide each other's LDS latency.  The two waves
+// of a head tile split the score work by token tile (wave dh scores tokens [16 dh, 16 dh + 16) of the step)
+// and exchange the 16 x 16 score tiles through LDS.
 struct StepRegs {
-    u32x4 codes[4];          // 4 items x 16 int8 codes
-    unsigned short scale[4]; // bf16 scale of each item's group
-    u32x4 rope;              // 8 bf16 rope values
+    u32x4 codes[2];          // 2 items x 16 int8 codes
+    unsigned short scale[2]; // bf16 scale of each item's group
+    u32x4 rope;              // 8 bf16 rope values (threads 0..255)
 };
 
-// TPW = head tiles (16 heads) per wave, 4 waves per workgroup.  DSPLIT = number of workgroups that
-// share one (split, sequence, head block): each accumulates 512 / DSPLIT output columns (and repeats the
-// score computation), which keeps accumulators + query fragments inside the register file.
-template <int TPW, int DSPLIT>
-__global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
+struct StepRows {
+    unsigned long long row[3];
+};
+
+__global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
 {
-    constexpr int MT = 32 / DSPLIT; // output M tiles (16 latent columns each) of this workgroup
     __shared__ __align__(16) unsigned char lds[2 * kTileBytes];
     __shared__ __align__(16) float lds_scale[2][8][kStepTokens]; // [buffer][group][token]
+    __shared__ __align__(16) float lds_s[4][2][16][16];          // [head tile][token tile][token][head]
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
+    const unsigned int hw = wave >> 1;
+    const unsigned int dh = wave & 1u;
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     const unsigned int chunk = blockIdx.x;
-    const unsigned int dsplit = blockIdx.y % DSPLIT;
-    const unsigned int head_base = (blockIdx.y / DSPLIT) * (64u * TPW) + wave * (16u * TPW);
+    const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
     const unsigned int b = blockIdx.z;
     const unsigned int len = p.ctx_lens[b];
     const unsigned long long c_start64 = (unsigned long long)chunk * p.chunk_tokens;
+    const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
 
-    // (max, sum) records for an empty split
-    if (c_start64 >= len) {
-#pragma unroll
-        for (int h = 0; h < TPW; ++h) {
-            const unsigned int head = head_base + 16u * h + m;
-            if (head < p.heads && j == 0 && dsplit == 0) {
-                const size_t si = (((size_t)b * p.max_chunks + chunk) * p.heads + head) * 2;
-                p.stats[si] = kNegInf;
-                p.stats[si + 1] = 0.0f;
-            }
+    if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
+        if (head < p.heads && j == 0 && dh == 0) {
+            p.stats[rec * 2] = kNegInf;
+            p.stats[rec * 2 + 1] = 0.0f;
         }
         return;
     }
@@ -137,10 +142,8 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
 
     // ---- Q fragments (B operand): lane = (head column m, k-slice j); k-step ks covers dims
     //      ks*32 + j*8 .. +8 of the 576-wide absorbed query ------------------------------------
-    Frag qf[TPW][18];
-#pragma unroll
-    for (int h = 0; h < TPW; ++h) {
-        const unsigned int head = head_base + 16u * h + m;
+    Frag qf[18];
+    {
         const unsigned short* qa = p.absorbed + ((size_t)b * p.heads + min(head, p.heads - 1u)) * kRowElems;
 #pragma unroll
         for (int ks = 0; ks < 18; ++ks) {
@@ -148,42 +151,68 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
             if (head >= p.heads) {
                 v = u32x4{0u, 0u, 0u, 0u};
             }
-            qf[h][ks].u = v;
+            qf[ks].u = v;
         }
     }
 
     const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
-    auto row_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned long long {
-        token = min(token, len - 1u);
-        if (table == nullptr) {
-            return token;
-        }
-        if (pow2) {
-            return ((unsigned long long)table[token >> p.block_shift] << p.block_shift) + (token & (p.block_tokens - 1u));
-        }
-        return (unsigned long long)table[token / p.block_tokens] * p.block_tokens + token % p.block_tokens;
-    };
 
-    // cooperative staging: item i of a thread = token (tid >> 5) + 8 i, 16-code chunk cc = tid & 31
+    // cooperative staging: item i of a thread = token (tid >> 5) + 16 i, 16-code chunk cc = tid & 31;
+    // threads 0..255 also move one rope item: token tid >> 3, 8-value chunk tid & 7
     const unsigned int cc = tid & 31u;
     const unsigned int t_lo = tid >> 5;
-    const unsigned int rope_t = tid >> 3;
+    const unsigned int rope_t = (tid >> 3) & 31u;
     const unsigned int rope_c = tid & 7u;
-    auto load_step = [&](StepRegs& r, unsigned int t0) __attribute__((always_inline)) {
+    const bool has_rope = tid < 256u;
+    // physical rows of the thread's tokens of a step: the table loads are issued together, one step ahead
+    // of the data loads that use them
+    auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
+        unsigned int token[3];
+        token[0] = min(t0 + t_lo, len - 1u);
+        token[1] = min(t0 + t_lo + 16u, len - 1u);
+        token[2] = min(t0 + rope_t, len - 1u);
+        if (table == nullptr) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned long long row = row_of(t0 + t_lo + 8u * i);
-            r.codes[i] = *(const u32x4*)(p.latent_codes + row * kLatent + cc * 16u);
-            r.scale[i] = p.latent_scales[row * (kLatent / 64) + (cc >> 2)];
+            for (int i = 0; i < 3; ++i) {
+                r.row[i] = token[i];
+            }
+        } else if (pow2) {
+            unsigned int entry[3];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                entry[i] = table[token[i] >> p.block_shift];
+            }
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                r.row[i] = ((unsigned long long)entry[i] << p.block_shift) + (token[i] & (p.block_tokens - 1u));
+            }
+        } else {
+            unsigned int entry[3];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                entry[i] = table[token[i] / p.block_tokens];
+            }
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                r.row[i] = (unsigned long long)entry[i] * p.block_tokens + token[i] % p.block_tokens;
+            }
         }
-        const unsigned long long row = row_of(t0 + rope_t);
-        r.rope = *(const u32x4*)(p.rope_cache + row * kRope + rope_c * 8u);
+    };
+    auto load_step = [&](StepRegs& r, const StepRows& rows) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            r.codes[i] = *(const u32x4*)(p.latent_codes + rows.row[i] * kLatent + cc * 16u);
+            r.scale[i] = p.latent_scales[rows.row[i] * (kLatent / 64) + (cc >> 2)];
+        }
+        if (has_rope) {
+            r.rope = *(const u32x4*)(p.rope_cache + rows.row[2] * kRope + rope_c * 8u);
+        }
     };
     auto store_step = [&](const StepRegs& r, unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned int row = t_lo + 8u * i;
+        for (int i = 0; i < 2; ++i) {
+            const unsigned int row = t_lo + 16u * i;
             u32x4 out[2];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
@@ -201,138 +230,108 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
                 scale_tile[cc >> 2][row] = bf16_bits_to_f32(r.scale[i]);
             }
         }
-        *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = r.rope;
+        if (has_rope) {
+            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = r.rope;
+        }
     };
 
-    f32x4 acc[TPW][MT];
+    constexpr int MT = 16; // output M tiles (16 latent columns each) of this wave
+    f32x4 acc[MT];
 #pragma unroll
-    for (int h = 0; h < TPW; ++h) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            acc[h][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    float run_max[TPW], run_sum[TPW];
-#pragma unroll
-    for (int h = 0; h < TPW; ++h) {
-        run_max[h] = kNegInf;
-        run_sum[h] = 0.0f;
-    }
+    float run_max = kNegInf, run_sum = 0.0f;
     const float scale_log2 = p.score_scale * kLog2e;
-    constexpr float kRescaleSlack = 8.0f; // log2 units: keep a stale maximum while p stays below 2^8
 
     // LDS byte offsets of this lane's fragments, split into a lane part and a compile-time part so
     // that every read is `base + immediate`:  chunk = (hi << 3) | lo, and only `lo` meets the swizzle.
-    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ swz(m)) << 4), m * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
+    const unsigned int qk_row = dh * 16u + m; // this wave scores token tile dh
+    const unsigned int qk_base[2] = {qk_row * kRowBytes + ((j ^ swz(m)) << 4), qk_row * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
     const unsigned int tr_row = 4u * j + (m >> 2);
     unsigned int pv_base[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u + dh * 4u * 128u;
     }
 
-    constexpr int GROUPS = 8 / DSPLIT; // scale groups among this workgroup's output columns
     auto compute_step = [&](const unsigned char* tile, const float (*scale_tile)[kStepTokens], unsigned int t0) __attribute__((always_inline)) {
-        // ---- S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope -----------------------------
-        f32x4 s[2][TPW];
+        // ---- scores of token tile dh: S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope -------------
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
+            Frag kf;
+            kf.u = *(const u32x4*)(tile + qk_base[ks & 1] + (ks >> 1) * 128);
+            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
+        }
 #pragma unroll
-            for (int h = 0; h < TPW; ++h) {
-                s[i][h] = f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-            // rope columns (k-steps 16, 17): unscaled
+        for (int g = 0; g < 8; ++g) {
+            Frag k0, k1;
+            k0.u = *(const u32x4*)(tile + qk_base[0] + g * 128);
+            k1.u = *(const u32x4*)(tile + qk_base[1] + g * 128);
+            const f32x4 gs = *(const f32x4*)(&scale_tile[g][dh * 16 + 4 * j]); // one address per 16-lane group
+            f32x4 d = {0.f, 0.f, 0.f, 0.f};
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d, 0, 0, 0);
 #pragma unroll
-            for (int ks = 16; ks < 18; ++ks) {
-                Frag kf;
-                kf.u = *(const u32x4*)(tile + qk_base[ks & 1] + (i * 16 * kRowBytes + (ks >> 1) * 128));
-#pragma unroll
-                for (int h = 0; h < TPW; ++h) {
-                    s[i][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[h][ks].b, s[i][h], 0, 0, 0);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                Frag k0, k1;
-                k0.u = *(const u32x4*)(tile + qk_base[0] + (i * 16 * kRowBytes + g * 128));
-                k1.u = *(const u32x4*)(tile + qk_base[1] + (i * 16 * kRowBytes + g * 128));
-                // group scales of this lane's four token rows (one address per 16-lane group)
-                const f32x4 gs = *(const f32x4*)(&scale_tile[g][i * 16 + 4 * j]);
-#pragma unroll
-                for (int h = 0; h < TPW; ++h) {
-                    f32x4 d = {0.f, 0.f, 0.f, 0.f};
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[h][2 * g].b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[h][2 * g + 1].b, d, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        s[i][h][r] = fmaf(d[r], gs[r], s[i][h][r]);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0); // bound the number of LDS fragments kept live
+            for (int r = 0; r < 4; ++r) {
+                s[r] = fmaf(d[r], gs[r], s[r]);
             }
         }
-        // ---- online softmax per head column ---------------------------------------------------------
-        float pr[TPW][8];
-        bool rescale = false;
-        float alpha[TPW];
+        float mine[4];
 #pragma unroll
-        for (int h = 0; h < TPW; ++h) {
-            float sc[8];
-            float step_max = kNegInf;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
-                sc[e] = token < len ? s[e >> 2][h][e & 3] * scale_log2 : kNegInf;
-                step_max = fmaxf(step_max, sc[e]);
-            }
-            step_max = wave_max_16x4(step_max);
-            // lazy rescaling: the stored maximum only moves when a score exceeds it by the slack
-            float new_max = run_max[h];
-            if (step_max > run_max[h] + kRescaleSlack || run_max[h] == kNegInf) {
-                new_max = fmaxf(run_max[h], step_max);
-            }
-            const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-            alpha[h] = __builtin_amdgcn_exp2f(run_max[h] - safe_max);
-            rescale = rescale || (alpha[h] != 1.0f && run_sum[h] != 0.0f);
-            float step_sum = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                pr[h][e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
-                step_sum += pr[h][e];
-            }
-            run_sum[h] = run_sum[h] * alpha[h] + step_sum;
-            run_max[h] = new_max;
+        for (int r = 0; r < 4; ++r) {
+            const unsigned int token = t0 + 16u * dh + 4u * j + r;
+            mine[r] = token < len ? s[r] * scale_log2 : kNegInf;
+            lds_s[hw][dh][4 * j + r][m] = mine[r];
         }
-        if (__any(rescale)) {
+        __syncthreads();
+        float sc[8];
 #pragma unroll
-            for (int h = 0; h < TPW; ++h) {
+        for (int r = 0; r < 4; ++r) {
+            const float other = lds_s[hw][dh ^ 1u][4 * j + r][m];
+            sc[dh * 4 + r] = mine[r];
+            sc[(dh ^ 1u) * 4 + r] = other;
+        }
+        // ---- online softmax for this head column (both waves of the pair compute the same values) --------
+        float step_max = sc[0];
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    acc[h][t] *= alpha[h];
-                }
+        for (int e = 1; e < 8; ++e) {
+            step_max = fmaxf(step_max, sc[e]);
+        }
+        step_max = wave_max_16x4(step_max);
+        const float new_max = fmaxf(run_max, step_max);
+        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+        const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
+        float pr[8];
+        float step_sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+            step_sum += pr[e];
+        }
+        run_sum = run_sum * alpha + step_sum;
+        run_max = new_max;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[t] *= alpha;
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g) --------------------------------------
-        const unsigned char* pv_tile = tile + dsplit * (MT / 4) * 128;
+        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g), for this wave's four scale groups ------------
 #pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-            const float* gs_row = scale_tile[dsplit * GROUPS + g];
+        for (int g = 0; g < 4; ++g) {
+            const float* gs_row = scale_tile[dh * 4 + g];
             const f32x4 gs0 = *(const f32x4*)(gs_row + 4 * j);
             const f32x4 gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
-            Frag pf[TPW];
-#pragma unroll
-            for (int h = 0; h < TPW; ++h) {
-                pf[h].u[0] = pack_bf16_rne(pr[h][0] * gs0[0], pr[h][1] * gs0[1]);
-                pf[h].u[1] = pack_bf16_rne(pr[h][2] * gs0[2], pr[h][3] * gs0[3]);
-                pf[h].u[2] = pack_bf16_rne(pr[h][4] * gs1[0], pr[h][5] * gs1[1]);
-                pf[h].u[3] = pack_bf16_rne(pr[h][6] * gs1[2], pr[h][7] * gs1[3]);
-            }
+            Frag pf;
+            pf.u[0] = pack_bf16_hw(pr[0] * gs0[0], pr[1] * gs0[1]);
+            pf.u[1] = pack_bf16_hw(pr[2] * gs0[2], pr[3] * gs0[3]);
+            pf.u[2] = pack_bf16_hw(pr[4] * gs1[0], pr[5] * gs1[1]);
+            pf.u[3] = pack_bf16_hw(pr[6] * gs1[2], pr[7] * gs1[3]);
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt) {
-                const int t = g * 4 + tt;
-                const unsigned char* at = pv_tile + pv_base[tt] + g * 128;
+                const unsigned char* at = tile + pv_base[tt] + g * 128;
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
                 const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
                 union {
@@ -341,18 +340,20 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
                 } vf;
                 vf.s[0] = lo;
                 vf.s[1] = hi;
-#pragma unroll
-                for (int h = 0; h < TPW; ++h) {
-                    acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pf[h].b, acc[h][t], 0, 0, 0);
-                }
+                acc[g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pf.b, acc[g * 4 + tt], 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // ---- pipeline: global loads of step n+1 overlap the MFMA work of step n; LDS double-buffered
+    // ---- pipeline: table lookups run two steps ahead, global loads one step ahead of the MFMA work;
+    //      LDS tile double-buffered; two barriers per step (score exchange, tile hand-over) -----------
     StepRegs regs;
-    load_step(regs, c_start);
+    StepRows rows;
+    lookup_step(rows, c_start);
+    load_step(regs, rows);
+    if (steps > 1) {
+        lookup_step(rows, c_start + kStepTokens);
+    }
     store_step(regs, lds, lds_scale[0]);
     __syncthreads();
     for (unsigned int step = 0; step < steps; ++step) {
@@ -360,7 +361,10 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
         unsigned char* nxt = lds + ((step + 1u) & 1u) * kTileBytes;
         const bool more = step + 1 < steps;
         if (more) {
-            load_step(regs, c_start + (step + 1u) * kStepTokens);
+            load_step(regs, rows);
+            if (step + 2 < steps) {
+                lookup_step(rows, c_start + (step + 2u) * kStepTokens);
+            }
         }
         compute_step(cur, lds_scale[step & 1u], c_start + step * kStepTokens);
         if (more) {
@@ -370,21 +374,16 @@ __global__ __launch_bounds__(256) void mla_partial(MlaDecodeParams p)
     }
 
     // ---- write un-normalised partials and (max, sum) -------------------------------------------
+    const float total = wave_sum_16x4(run_sum);
+    if (head < p.heads) {
+        if (j == 0 && dh == 0) {
+            p.stats[rec * 2] = run_max;
+            p.stats[rec * 2 + 1] = total;
+        }
+        float* out = p.partial + rec * kLatent + dh * 256u;
 #pragma unroll
-    for (int h = 0; h < TPW; ++h) {
-        const unsigned int head = head_base + 16u * h + m;
-        const float total = wave_sum_16x4(run_sum[h]);
-        if (head < p.heads) {
-            const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
-            if (j == 0 && dsplit == 0) {
-                p.stats[rec * 2] = run_max[h];
-                p.stats[rec * 2 + 1] = total;
-            }
-            float* out = p.partial + rec * kLatent + dsplit * (MT * 16);
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                *(f32x4*)(out + t * 16 + 4 * j) = acc[h][t];
-            }
+        for (int t = 0; t < MT; ++t) {
+            *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
         }
     }
 }
@@ -437,11 +436,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if (stages & 2u) {
-        if (p.heads > 64) {
-            mla_partial<2, 2><<<dim3(p.max_chunks, 2 * ((p.heads + 127) / 128), p.batch), dim3(256), 0, stream>>>(p);
-        } else {
-            mla_partial<1, 1><<<dim3(p.max_chunks, 1, p.batch), dim3(256), 0, stream>>>(p);
-        }
+        mla_partial<<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
         err = hipGetLastError();
         if (err != hipSuccess) {
             return err;
