@@ -95,31 +95,39 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 // ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
-// Workgroup = (split, block of 64 heads, sequence), 8 waves = 4 head tiles x 2 halves.  Wave (hw, dh) owns
-// heads [16 hw, 16 hw + 16) and output columns [256 dh, 256 dh + 256): 64 accumulator registers + 72 query
-// fragment registers per lane, so two waves share a SIMD and hide each other's LDS latency.  The two waves
-// of a head tile split the score work by token tile (wave dh scores tokens [16 dh, 16 dh + 16) of the step)
-// and exchange the 16 x 16 score tiles through LDS.
+// Workgroup = (split, block of 64 heads, sequence) with 4 * NDH waves; wave (hw, dh) owns heads
+// [16 hw, 16 hw + 16) and output columns [512 dh / NDH, 512 (dh + 1) / NDH).
+//   NDH = 1: four waves, one per SIMD with the whole 512-register file: 128 accumulator + 72 query
+//            registers leave room to keep many LDS fragment loads in flight; one barrier per step.
+//   NDH = 2: eight waves; the two waves of a head tile split the score work by token tile and exchange
+//            16 x 16 score tiles through LDS (two barriers per step).
+constexpr int kItemsMax = 4;
 struct StepRegs {
-    u32x4 codes[2];          // 2 items x 16 int8 codes
-    unsigned short scale[2]; // bf16 scale of each item's group
-    u32x4 rope;              // 8 bf16 rope values (threads 0..255)
+    u32x4 codes[kItemsMax];          // items x 16 int8 codes
+    unsigned short scale[kItemsMax]; // bf16 scale of each item's group
+    u32x4 rope;                      // 8 bf16 rope values (threads 0..255)
 };
 
 struct StepRows {
-    unsigned long long row[3];
+    unsigned long long row[kItemsMax + 1];
 };
 
-__global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
+template <int NDH>
+__global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
 {
+    constexpr int ITEMS = 4 / NDH;      // staging items per thread
+    constexpr int TROWS = 8 * NDH;      // token rows covered by one pass of the threads
+    constexpr int MT = 32 / NDH;        // output M tiles (16 latent columns each) of this wave
+    constexpr int GROUPS = 8 / NDH;     // scale groups among them
+    constexpr int TILES = 2 / NDH;      // token tiles this wave scores itself
     __shared__ __align__(16) unsigned char lds[2 * kTileBytes];
     __shared__ __align__(16) float lds_scale[2][8][kStepTokens]; // [buffer][group][token]
-    __shared__ __align__(16) float lds_s[4][2][16][16];          // [head tile][token tile][token][head]
+    __shared__ __align__(16) float lds_s[NDH == 2 ? 4 : 1][2][16][16]; // [head tile][token tile][token][head]
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
-    const unsigned int hw = wave >> 1;
-    const unsigned int dh = wave & 1u;
+    const unsigned int hw = wave / NDH;
+    const unsigned int dh = wave % NDH;
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     const unsigned int chunk = blockIdx.x;
@@ -158,7 +166,7 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
     const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
-    // cooperative staging: item i of a thread = token (tid >> 5) + 16 i, 16-code chunk cc = tid & 31;
+    // cooperative staging: item i of a thread = token (tid >> 5) + TROWS * i, 16-code chunk cc = tid & 31;
     // threads 0..255 also move one rope item: token tid >> 3, 8-value chunk tid & 7
     const unsigned int cc = tid & 31u;
     const unsigned int t_lo = tid >> 5;
@@ -168,51 +176,53 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
     // physical rows of the thread's tokens of a step: the table loads are issued together, one step ahead
     // of the data loads that use them
     auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
-        unsigned int token[3];
-        token[0] = min(t0 + t_lo, len - 1u);
-        token[1] = min(t0 + t_lo + 16u, len - 1u);
-        token[2] = min(t0 + rope_t, len - 1u);
+        unsigned int token[ITEMS + 1];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            token[i] = min(t0 + t_lo + TROWS * i, len - 1u);
+        }
+        token[ITEMS] = min(t0 + rope_t, len - 1u);
         if (table == nullptr) {
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i <= ITEMS; ++i) {
                 r.row[i] = token[i];
             }
         } else if (pow2) {
-            unsigned int entry[3];
+            unsigned int entry[ITEMS + 1];
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i <= ITEMS; ++i) {
                 entry[i] = table[token[i] >> p.block_shift];
             }
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i <= ITEMS; ++i) {
                 r.row[i] = ((unsigned long long)entry[i] << p.block_shift) + (token[i] & (p.block_tokens - 1u));
             }
         } else {
-            unsigned int entry[3];
+            unsigned int entry[ITEMS + 1];
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i <= ITEMS; ++i) {
                 entry[i] = table[token[i] / p.block_tokens];
             }
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i <= ITEMS; ++i) {
                 r.row[i] = (unsigned long long)entry[i] * p.block_tokens + token[i] % p.block_tokens;
             }
         }
     };
     auto load_step = [&](StepRegs& r, const StepRows& rows) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < ITEMS; ++i) {
             r.codes[i] = *(const u32x4*)(p.latent_codes + rows.row[i] * kLatent + cc * 16u);
             r.scale[i] = p.latent_scales[rows.row[i] * (kLatent / 64) + (cc >> 2)];
         }
         if (has_rope) {
-            r.rope = *(const u32x4*)(p.rope_cache + rows.row[2] * kRope + rope_c * 8u);
+            r.rope = *(const u32x4*)(p.rope_cache + rows.row[ITEMS] * kRope + rope_c * 8u);
         }
     };
     auto store_step = [&](const StepRegs& r, unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const unsigned int row = t_lo + 16u * i;
+        for (int i = 0; i < ITEMS; ++i) {
+            const unsigned int row = t_lo + TROWS * i;
             u32x4 out[2];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
@@ -235,7 +245,6 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
         }
     };
 
-    constexpr int MT = 16; // output M tiles (16 latent columns each) of this wave
     f32x4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -246,61 +255,95 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
 
     // LDS byte offsets of this lane's fragments, split into a lane part and a compile-time part so
     // that every read is `base + immediate`:  chunk = (hi << 3) | lo, and only `lo` meets the swizzle.
-    const unsigned int qk_row = dh * 16u + m; // this wave scores token tile dh
+    const unsigned int qk_row = (NDH == 2 ? dh * 16u : 0u) + m;
     const unsigned int qk_base[2] = {qk_row * kRowBytes + ((j ^ swz(m)) << 4), qk_row * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
     const unsigned int tr_row = 4u * j + (m >> 2);
     unsigned int pv_base[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u + dh * 4u * 128u;
+        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u +
+                     dh * GROUPS * 128u;
     }
 
     auto compute_step = [&](const unsigned char* tile, const float (*scale_tile)[kStepTokens], unsigned int t0) __attribute__((always_inline)) {
-        // ---- scores of token tile dh: S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope -------------
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
-            Frag kf;
-            kf.u = *(const u32x4*)(tile + qk_base[ks & 1] + (ks >> 1) * 128);
-            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
-        }
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            Frag k0, k1;
-            k0.u = *(const u32x4*)(tile + qk_base[0] + g * 128);
-            k1.u = *(const u32x4*)(tile + qk_base[1] + g * 128);
-            const f32x4 gs = *(const f32x4*)(&scale_tile[g][dh * 16 + 4 * j]); // one address per 16-lane group
-            f32x4 d = {0.f, 0.f, 0.f, 0.f};
-            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, d, 0, 0, 0);
-            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                s[r] = fmaf(d[r], gs[r], s[r]);
-            }
-        }
-        float mine[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const unsigned int token = t0 + 16u * dh + 4u * j + r;
-            mine[r] = token < len ? s[r] * scale_log2 : kNegInf;
-            lds_s[hw][dh][4 * j + r][m] = mine[r];
-        }
-        __syncthreads();
+        // ---- scores: S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope ------------------------------
         float sc[8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float other = lds_s[hw][dh ^ 1u][4 * j + r][m];
-            sc[dh * 4 + r] = mine[r];
-            sc[(dh ^ 1u) * 4 + r] = other;
+        for (int i = 0; i < TILES; ++i) {
+            const unsigned int tile_i = NDH == 2 ? dh : (unsigned int)i;          // token tile scored here
+            const unsigned char* kt = tile + (NDH == 2 ? 0 : i * 16 * kRowBytes); // qk_base already holds dh
+            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
+                Frag kf;
+                kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
+                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
+            }
+#pragma unroll
+            for (int half = 0; half < 2; ++half) { // four independent accumulators at a time: no MFMA -> MFMA stalls
+                f32x4 d[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int g = half * 4 + u;
+                    Frag k0;
+                    k0.u = *(const u32x4*)(kt + qk_base[0] + g * 128);
+                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int g = half * 4 + u;
+                    Frag k1;
+                    k1.u = *(const u32x4*)(kt + qk_base[1] + g * 128);
+                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int g = half * 4 + u;
+                    const f32x4 gs = *(const f32x4*)(&scale_tile[g][tile_i * 16 + 4 * j]); // one address per 16-lane group
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        s[r] = fmaf(d[u][r], gs[r], s[r]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const unsigned int token = t0 + 16u * tile_i + 4u * j + r;
+                const float x = token < len ? s[r] * scale_log2 : kNegInf;
+                if constexpr (NDH == 2) {
+                    sc[r] = x; // staged below
+                } else {
+                    sc[i * 4 + r] = x;
+                }
+            }
         }
-        // ---- online softmax for this head column (both waves of the pair compute the same values) --------
+        if constexpr (NDH == 2) {
+            float mine[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                mine[r] = sc[r];
+                lds_s[hw][dh][4 * j + r][m] = mine[r];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float other = lds_s[hw][dh ^ 1u][4 * j + r][m];
+                sc[dh * 4 + r] = mine[r];
+                sc[(dh ^ 1u) * 4 + r] = other;
+            }
+        }
+        // ---- online softmax for this head column ---------------------------------------------------------
         float step_max = sc[0];
 #pragma unroll
         for (int e = 1; e < 8; ++e) {
             step_max = fmaxf(step_max, sc[e]);
         }
         step_max = wave_max_16x4(step_max);
-        const float new_max = fmaxf(run_max, step_max);
+        // lazy rescaling: the stored maximum only moves when a score exceeds it by 2^8 (p stays <= 256)
+        float new_max = run_max;
+        if (step_max > run_max + 8.0f || run_max == kNegInf) {
+            new_max = fmaxf(run_max, step_max);
+        }
         const float safe_max = new_max == kNegInf ? 0.0f : new_max;
         const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
         float pr[8];
@@ -310,18 +353,21 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
             pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
             step_sum += pr[e];
         }
+        const bool had_mass = run_sum != 0.0f; // nothing accumulated yet -> nothing to rescale
         run_sum = run_sum * alpha + step_sum;
         run_max = new_max;
-        if (__any(alpha != 1.0f)) {
+        __builtin_amdgcn_sched_barrier(0); // keep the (rare) rescale at a point of low register pressure
+        if (__any(alpha != 1.0f && had_mass)) {
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 acc[t] *= alpha;
             }
         }
-        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g), for this wave's four scale groups ------------
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g), for this wave's scale groups ----------------
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const float* gs_row = scale_tile[dh * 4 + g];
+        for (int g = 0; g < GROUPS; ++g) {
+            const float* gs_row = scale_tile[dh * GROUPS + g];
             const f32x4 gs0 = *(const f32x4*)(gs_row + 4 * j);
             const f32x4 gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
             Frag pf;
@@ -346,7 +392,7 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
     };
 
     // ---- pipeline: table lookups run two steps ahead, global loads one step ahead of the MFMA work;
-    //      LDS tile double-buffered; two barriers per step (score exchange, tile hand-over) -----------
+    //      LDS tile double-buffered ---------------------------------------------------------------------
     StepRegs regs;
     StepRows rows;
     lookup_step(rows, c_start);
@@ -380,7 +426,7 @@ __global__ __launch_bounds__(512) void mla_partial(MlaDecodeParams p)
             p.stats[rec * 2] = run_max;
             p.stats[rec * 2 + 1] = total;
         }
-        float* out = p.partial + rec * kLatent + dh * 256u;
+        float* out = p.partial + rec * kLatent + dh * (MT * 16u);
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
@@ -436,7 +482,8 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if (stages & 2u) {
-        mla_partial<<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
+        // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
+        mla_partial<2><<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
         err = hipGetLastError();
         if (err != hipSuccess) {
             return err;
