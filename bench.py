@@ -176,24 +176,39 @@ def run_gqa_decode(args, ragged):
     lens_dev = torch.tensor(lens, dtype=torch.int32, device="cuda")
     call_args, out, workspace = ops.gqa_decode_args(q, planes["k_codes"], planes["k_scales"], planes["v_codes"], planes["v_scales"],
                                                     tables_dev, lens_dev, hq, hkv, d, bt, scale, max(lens),
-                                                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16)
+                                                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, total_kv_tokens=sum(lens))
     lib = capi.load()
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def launch(stages):
+        call_args.stages = stages
+        capi.check(lib.zllm_attn_gqa_decode(C.byref(call_args), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
 
     def full():
-        call_args.stages = capi.STAGE_ALL
-        capi.check(lib.zllm_attn_gqa_decode(C.byref(call_args), stream))
+        launch(capi.STAGE_ALL)
 
     def partial_only():
-        call_args.stages = capi.STAGE_PARTIAL
-        capi.check(lib.zllm_attn_gqa_decode(C.byref(call_args), stream))
+        launch(capi.STAGE_PARTIAL)
 
     for _ in range(args.warmup):
         full()
-    ms_step = wall_time_ms(full, args.steps)
-    ms_events = event_time_ms(full, args.steps)
+    ms_eager = wall_time_ms(full, args.steps)
+    # The decode step is replayed from a HIP graph, as the reference replays its decode launches
+    # (src/kernel/rocm/hip/graph.rs): same kernels, same arguments, without per-launch host overhead.
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        full()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        full()
+    for _ in range(args.warmup):
+        graph.replay()
+    ms_step = wall_time_ms(graph.replay, args.steps)
+    ms_events = event_time_ms(graph.replay, args.steps)
     ms_partial = event_time_ms(partial_only, args.steps)
-    full()
+    out.zero_()
+    graph.replay()
     torch.cuda.synchronize()
 
     bytes_per_token = 2 * (hkv * d + 2 * hkv * d // 64)  # 2,112 B: K+V codes + 16-bit scales
@@ -212,6 +227,8 @@ def run_gqa_decode(args, ragged):
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "ms_per_step_events": round(ms_events, 5),
+        "ms_per_step_eager_launch": round(ms_eager, 5),
+        "launch": "hipGraph replay of one decode step (partial + merge)",
         "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_partial", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel_ms": round(ms_partial, 5)},

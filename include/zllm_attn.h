@@ -206,6 +206,8 @@ typedef struct zllm_gqa_decode_args {
     uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 256} */
     uint32_t table_stride;         /* entries per sequence in `tables` */
     uint32_t max_kv_len;           /* host upper bound of kv_lens (sizes the grid) */
+    uint32_t total_kv_tokens;      /* optional host hint: sum of the visible lengths (0 = unknown,
+                                      batch * max_kv_len is assumed); only tunes the split size */
     uint32_t block_tokens;
     uint32_t ring_capacity;        /* 0 or sliding-window ring rows (token % capacity) */
     float score_scale;             /* > 0 */

@@ -50,8 +50,8 @@ class GqaDecodeArgs(C.Structure):
     _fields_ = [("q", _ptr), ("k_plane", _ptr), ("k_scales", _ptr), ("v_plane", _ptr), ("v_scales", _ptr),
                 ("tables", _ptr), ("kv_lens", _ptr), ("first_visible", _ptr), ("out", _ptr), ("workspace", _ptr),
                 ("workspace_bytes", _u64), ("batch", _u32), ("num_heads", _u32), ("num_kv_heads", _u32),
-                ("head_dim", _u32), ("table_stride", _u32), ("max_kv_len", _u32), ("block_tokens", _u32),
-                ("ring_capacity", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
+                ("head_dim", _u32), ("table_stride", _u32), ("max_kv_len", _u32), ("total_kv_tokens", _u32),
+                ("block_tokens", _u32), ("ring_capacity", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
                 ("scale_dtype", _int), ("q_dtype", _int), ("stages", _u32)]
 
 

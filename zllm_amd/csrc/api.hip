@@ -53,13 +53,15 @@ bool valid_head_dim(uint32_t d)
     return d == 64 || d == 128 || d == 256;
 }
 
-// Tokens per KV split: enough workgroups to occupy every CU about twice, but
-// splits long enough that the partial write / merge stay a few percent of the
-// KV bytes a split reads.
-void plan_splits(uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t rounds, uint32_t* chunk_tokens, uint32_t* max_chunks)
+// Tokens per KV split: one workgroup per CU over the call (a second round would repeat every
+// workgroup's prologue), but splits long enough that the partial write / merge stay a few percent of
+// the KV bytes a split reads.
+void plan_splits(uint64_t total_tokens, uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t rounds, uint32_t* chunk_tokens,
+                 uint32_t* max_chunks)
 {
+    // `columns` workgroups run per split; aim at `rounds` workgroups per CU over the whole call
     const uint64_t target = (uint64_t)rounds * kComputeUnits;
-    uint64_t chunk = ((uint64_t)max_len * columns + target - 1) / target;
+    uint64_t chunk = (total_tokens * columns + target - 1) / target;
     chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
     *chunk_tokens = (uint32_t)chunk;
     const uint64_t chunks = ((uint64_t)max_len + chunk - 1) / chunk;
@@ -107,8 +109,20 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
     const char* rounds_env = getenv("ZLLM_TUNE_ROUNDS");
-    const uint32_t rounds = rounds_env ? (uint32_t)atoi(rounds_env) : 2u;
-    plan_splits(a->max_kv_len, a->batch * kvh_blocks * head_blocks, 256, rounds, chunk_tokens, max_chunks);
+    const uint32_t rounds = rounds_env ? (uint32_t)atoi(rounds_env) : 1u;
+    const uint32_t columns = a->batch * kvh_blocks * head_blocks;
+    const uint64_t uniform_total = (uint64_t)a->batch * a->max_kv_len;
+    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && rounds * kComputeUnits > 2 * columns) {
+        // ragged batch: sum_b ceil(len_b / chunk) <= total / chunk + batch, so size the splits for the
+        // workgroups that will really run and keep them within one round of the CUs
+        const uint64_t slots = (uint64_t)rounds * kComputeUnits / (kvh_blocks * head_blocks) - a->batch;
+        uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
+        chunk = align_up(chunk < 256 ? 256 : chunk, 32);
+        *chunk_tokens = (uint32_t)chunk;
+        *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
+        return;
+    }
+    plan_splits(a->max_kv_len, a->max_kv_len, columns, 256, rounds, chunk_tokens, max_chunks);
 }
 
 int validate_mla_decode(const zllm_mla_decode_args* a)
@@ -141,7 +155,7 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
 {
     // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
-    plan_splits(a->max_ctx_len, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
+    plan_splits(a->max_ctx_len, a->max_ctx_len, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {

@@ -84,14 +84,40 @@ template <> struct ScaleRow<4> {
 };
 
 // Everything one wave loads for a 32-token step of a Q8g64 cache.
-template <int G> struct Q8Step {
-    u32x4 k[2][G];      // K codes: tile i, group a -> 16 codes of the lane's token
+//   FAST (pages of >= 16 tokens): the 16 scale rows a 16-lane row needs in a step (2 tiles x 4 token slots x
+//   {K, V}) are loaded one per lane and handed out with DPP row broadcasts — one load instead of sixteen.
+//   Generic: every lane loads the scale rows of its eight token slots itself.
+template <int G, bool FAST> struct Q8Step {
+    u32x4 k[2][G];        // K codes: tile i, group a -> 16 codes of the lane's token
     unsigned int v[8][G]; // V codes: token slot s = i*4 + r, group a -> 4 codes (dims a*64 + 4m .. +4)
-    ScaleRow<G> ks[8];  // K scales of token slot s
-    ScaleRow<G> vs[8];  // V scales of token slot s
+    ScaleRow<G> ks[FAST ? 1 : 8]; // FAST: lane x of a row holds scale row (kv = x>>3, tile (x>>2)&1, slot x&3)
+    ScaleRow<G> vs[FAST ? 1 : 8];
 };
 
-template <int D, int SDT, bool QSPLIT, bool FAST>
+// lane `n` of each 16-lane row, broadcast to the row (v_mov_b32 row_newbcast)
+template <int N> __device__ __forceinline__ unsigned int row_bcast(unsigned int v)
+{
+    return __builtin_amdgcn_update_dpp(0u, v, 0x150 + N, 0xf, 0xf, false);
+}
+
+template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(const ScaleRow<G>& r)
+{
+    ScaleRow<G> out;
+    if constexpr (G == 1) {
+        out.v = (unsigned short)row_bcast<N>((unsigned int)r.v);
+    } else if constexpr (G == 2) {
+        out.v = row_bcast<N>(r.v);
+    } else {
+        out.v.x = row_bcast<N>(r.v.x);
+        out.v.y = row_bcast<N>(r.v.y);
+    }
+    return out;
+}
+
+// NBUF = steps of KV kept in registers: loads run NBUF - 1 steps (32 tokens each) ahead of the MFMA work.
+// With pages scattered over a large pool every page costs an address translation as well as an HBM access,
+// and one step of prefetch leaves the wave waiting ~3.5 us per step.
+template <int D, int SDT, bool QSPLIT, bool FAST, bool SOFTCAP, int NBUF>
 __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(GqaDecodeParams p)
 {
     constexpr int G = D / 64;           // scale groups per head row
@@ -163,13 +189,31 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int lo_tile = first & ~15u;
     const unsigned int hi_tile = (len - 1u) & ~15u;
 
-    // physical row of the first token of the (clamped) 16-token tile starting at T
+    // physical row of the first token of the (clamped) 16-token tile starting at T.  When the split spans
+    // at most 128 pages (and no ring), the wave loads its block-table entries once into two registers
+    // (lane i = entry first_page + i / + 64 + i) and reads them with v_readlane: no table load inside the loop.
+    const unsigned int first_page = min(max(c_start, lo_tile), hi_tile) >> p.block_shift;
+    const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
+    const bool cached_table = FAST && p.ring_capacity == 0 && ((min(max(c_end - 1u, lo_tile), hi_tile) >> p.block_shift) - first_page) < 128u;
+    unsigned int entries0 = 0, entries1 = 0;
+    if (cached_table) {
+        entries0 = p.tables != nullptr ? table[min(first_page + lane, last_page)] : first_page + lane;
+        entries1 = p.tables != nullptr ? table[min(first_page + 64u + lane, last_page)] : first_page + 64u + lane;
+    }
     auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
         unsigned int t = min(max(T, lo_tile), hi_tile);
         if (p.ring_capacity != 0) {
             t %= p.ring_capacity;
         }
-        const unsigned int entry = p.tables != nullptr ? __builtin_amdgcn_readfirstlane(table[t >> p.block_shift]) : (t >> p.block_shift);
+        unsigned int entry;
+        if (cached_table) {
+            const unsigned int idx = __builtin_amdgcn_readfirstlane((t >> p.block_shift) - first_page);
+            const unsigned int e0 = __builtin_amdgcn_readlane(entries0, idx & 63u);
+            const unsigned int e1 = __builtin_amdgcn_readlane(entries1, idx & 63u);
+            entry = idx < 64u ? e0 : e1;
+        } else {
+            entry = p.tables != nullptr ? __builtin_amdgcn_readfirstlane(table[t >> p.block_shift]) : (t >> p.block_shift);
+        }
         return ((unsigned long long)entry << p.block_shift) + (t & block_mask);
     };
     // physical row of one token (generic path: any page size / ring)
@@ -178,28 +222,45 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         return paged_row(p.tables != nullptr ? table : nullptr, t, p.block_tokens, p.ring_capacity);
     };
 
-    auto load_step = [&](Q8Step<G>& s, unsigned int t0) __attribute__((always_inline)) {
+    // lane-constant byte offsets (FAST path): every load is `uniform tile base + lane offset [+ immediate]`
+    const unsigned int k_off = m * k_row + j * 16u;
+    unsigned int v_off[4], s_off = 0;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            if constexpr (FAST) {
-                const unsigned long long R = tile_row(t0 + 16u * i);
-                const unsigned char* kr = k_base + (R + m) * k_row + j * 16u;
+    for (int r = 0; r < 4; ++r) {
+        v_off[r] = (4u * j + r) * k_row + 4u * m;
+    }
+    const unsigned int sx = lane & 15u;                   // this lane's role in the scale load
+    const bool sx_value = (sx >> 3) != 0;                 // V scales (else K)
+    const bool sx_tile1 = ((sx >> 2) & 1u) != 0;          // second tile of the step
+    s_off = (4u * j + (sx & 3u)) * s_row;
+    const unsigned char* s_plane = sx_value ? vs_base : ks_base;
+
+    auto load_step = [&](Q8Step<G, FAST>& s, unsigned int t0) __attribute__((always_inline)) {
+        if constexpr (FAST) {
+            const unsigned long long R0 = tile_row(t0);
+            const unsigned long long R1 = tile_row(t0 + 16u);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const unsigned long long R = i == 0 ? R0 : R1;
+                const unsigned char* kt = k_base + R * k_row; // uniform
+                const unsigned char* vt = v_base + R * k_row;
 #pragma unroll
                 for (int a = 0; a < G; ++a) {
-                    s.k[i][a] = *(const u32x4*)(kr + a * 64);
+                    s.k[i][a] = *(const u32x4*)(kt + k_off + a * 64);
                 }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const unsigned long long row = R + 4u * j + r;
-                    const unsigned char* vr = v_base + row * k_row + 4u * m;
 #pragma unroll
                     for (int a = 0; a < G; ++a) {
-                        s.v[i * 4 + r][a] = *(const unsigned int*)(vr + a * 64);
+                        s.v[i * 4 + r][a] = *(const unsigned int*)(vt + v_off[r] + a * 64);
                     }
-                    s.ks[i * 4 + r] = *(const ScaleRow<G>*)(ks_base + row * s_row);
-                    s.vs[i * 4 + r] = *(const ScaleRow<G>*)(vs_base + row * s_row);
                 }
-            } else {
+            }
+            const unsigned long long Rs = sx_tile1 ? R1 : R0;
+            s.ks[0] = *(const ScaleRow<G>*)(s_plane + Rs * s_row + s_off);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
                 const unsigned long long rk = token_row(t0 + 16u * i + m);
                 const unsigned char* kr = k_base + rk * k_row + j * 16u;
 #pragma unroll
@@ -228,9 +289,37 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     }
     float run_max = kNegInf; // log2 units
     float run_sum = 0.0f;    // lane-partial (this lane's 8 token slots per step)
-    const float scale_log2 = p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e;
+    const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
+    const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
+    const float cap_log2 = p.softcap * kLog2e;
 
-    auto compute_step = [&](const Q8Step<G>& s, unsigned int t0) __attribute__((always_inline)) {
+    auto compute_step = [&](const Q8Step<G, FAST>& s, unsigned int t0) __attribute__((always_inline)) {
+        // scale rows of this lane's eight token slots (K then V)
+        ScaleRow<G> ksr[8], vsr[8];
+        if constexpr (FAST) {
+            ksr[0] = row_bcast_scales<G, 0>(s.ks[0]);
+            ksr[1] = row_bcast_scales<G, 1>(s.ks[0]);
+            ksr[2] = row_bcast_scales<G, 2>(s.ks[0]);
+            ksr[3] = row_bcast_scales<G, 3>(s.ks[0]);
+            ksr[4] = row_bcast_scales<G, 4>(s.ks[0]);
+            ksr[5] = row_bcast_scales<G, 5>(s.ks[0]);
+            ksr[6] = row_bcast_scales<G, 6>(s.ks[0]);
+            ksr[7] = row_bcast_scales<G, 7>(s.ks[0]);
+            vsr[0] = row_bcast_scales<G, 8>(s.ks[0]);
+            vsr[1] = row_bcast_scales<G, 9>(s.ks[0]);
+            vsr[2] = row_bcast_scales<G, 10>(s.ks[0]);
+            vsr[3] = row_bcast_scales<G, 11>(s.ks[0]);
+            vsr[4] = row_bcast_scales<G, 12>(s.ks[0]);
+            vsr[5] = row_bcast_scales<G, 13>(s.ks[0]);
+            vsr[6] = row_bcast_scales<G, 14>(s.ks[0]);
+            vsr[7] = row_bcast_scales<G, 15>(s.ks[0]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ksr[e] = s.ks[e];
+                vsr[e] = s.vs[e];
+            }
+        }
         // ---- S^T = K . Q^T, one accumulator per scale group -----------------------------
         float sc[8];
 #pragma unroll
@@ -252,14 +341,14 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
                 }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(s.ks[i * 4 + r].get(a)), tile_s[r]);
+                    tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(ksr[i * 4 + r].get(a)), tile_s[r]);
                 }
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 float x = tile_s[r] * scale_log2;
-                if (p.softcap > 0.0f) {
-                    x = p.softcap * fast_tanh(x / p.softcap) * kLog2e;
+                if constexpr (SOFTCAP) {
+                    x = cap_log2 * fast_tanh(x * inv_cap);
                 }
                 const unsigned int token = t0 + 16u * i + 4u * j + r;
                 sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
@@ -296,8 +385,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             Frag phi, plo;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(s.vs[2 * e].get(a));
-                const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(s.vs[2 * e + 1].get(a));
+                const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(vsr[2 * e].get(a));
+                const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(vsr[2 * e + 1].get(a));
                 unsigned int hi, lo;
                 split_bf16_pair(x0, x1, hi, lo);
                 phi.u[e] = hi;
@@ -318,25 +407,25 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         }
     };
 
-    // ---- software pipeline: loads of step n+1 in flight while step n computes ---------
-    Q8Step<G> buf0, buf1;
-    load_step(buf0, c_start);
-    unsigned int step = 0;
-    while (true) {
-        const unsigned int t0 = c_start + step * 32u;
-        if (step + 1 < steps) {
-            load_step(buf1, t0 + 32u);
+    // ---- software pipeline: loads of steps n+1 .. n+NBUF-1 in flight while step n computes ----------
+    Q8Step<G, FAST> buf[NBUF];
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u) {
+        if ((unsigned int)u < steps) {
+            load_step(buf[u], c_start + u * 32u);
         }
-        compute_step(buf0, t0);
-        if (++step >= steps) {
-            break;
-        }
-        if (step + 1 < steps) {
-            load_step(buf0, t0 + 64u);
-        }
-        compute_step(buf1, t0 + 32u);
-        if (++step >= steps) {
-            break;
+    }
+    for (unsigned int base = 0; base < steps; base += NBUF) {
+#pragma unroll
+        for (int u = 0; u < NBUF; ++u) {
+            const unsigned int step = base + u;
+            if (step < steps) {
+                const unsigned int ahead = step + NBUF - 1;
+                if (ahead < steps) {
+                    load_step(buf[(u + NBUF - 1) % NBUF], c_start + ahead * 32u);
+                }
+                compute_step(buf[u], c_start + step * 32u);
+            }
         }
     }
 
@@ -685,10 +774,26 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
 template <int D, int SDT, bool QSPLIT>
 hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
+    const bool cap = p.softcap > 0.0f;
+    constexpr int kDeep = (D <= 128 && !QSPLIT) ? 4 : (D <= 128 ? 3 : 2); // register budget: 256 per lane
+    const char* env = getenv("ZLLM_TUNE_NBUF");
+    const int nbuf = env != nullptr ? atoi(env) : 2;
     if (fast) {
-        gqa_decode_q8_partial<D, SDT, QSPLIT, true><<<grid, block, 0, stream>>>(p);
+        if (cap) {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, true, true, 2><<<grid, block, 0, stream>>>(p);
+        } else if (nbuf >= 4 && kDeep >= 4) {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, kDeep><<<grid, block, 0, stream>>>(p);
+        } else if (nbuf == 3 && kDeep >= 3) {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, (kDeep >= 3 ? 3 : 2)><<<grid, block, 0, stream>>>(p);
+        } else {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, 2><<<grid, block, 0, stream>>>(p);
+        }
     } else {
-        gqa_decode_q8_partial<D, SDT, QSPLIT, false><<<grid, block, 0, stream>>>(p);
+        if (cap) {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, false, true, 2><<<grid, block, 0, stream>>>(p);
+        } else {
+            gqa_decode_q8_partial<D, SDT, QSPLIT, false, false, 2><<<grid, block, 0, stream>>>(p);
+        }
     }
     return hipGetLastError();
 }

@@ -71,7 +71,7 @@ def gather_rows(plane, table, first, count, row_bytes, block_tokens, ring_capaci
 
 def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, num_heads, num_kv_heads, head_dim,
                     block_tokens, score_scale, max_kv_len, first_visible=None, softcap=0.0, ring_capacity=0,
-                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None):
+                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None, total_kv_tokens=0):
     batch = q.shape[0]
     if out is None:
         out = torch.empty((batch, num_heads * head_dim), dtype=torch.float32, device=q.device)
@@ -83,6 +83,7 @@ def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, nu
     args.batch, args.num_heads, args.num_kv_heads, args.head_dim = batch, num_heads, num_kv_heads, head_dim
     args.table_stride = 0 if tables is None else tables.shape[1]
     args.max_kv_len, args.block_tokens, args.ring_capacity = max_kv_len, block_tokens, ring_capacity
+    args.total_kv_tokens = total_kv_tokens
     args.score_scale, args.softcap = score_scale, softcap
     args.kv_format, args.scale_dtype, args.q_dtype = kv_format, scale_dtype, _DTYPE[q.dtype]
     need = capi.load().zllm_attn_gqa_decode_workspace_bytes(C.byref(args))
