@@ -24,6 +24,8 @@
 // same work is < 15 % of peak and the vector units only convert int8 -> bf16.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -114,6 +116,151 @@ template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(
     return out;
 }
 
+// Q fragments: B operand of the int8 MFMA, lane = (head column m, k-slice j).
+// The head's query row is quantized to 15-bit fixed point (step = max|q| / 16256) and split into two
+// signed-byte digits q = 128 * hi + lo, hi in [-127, 127], lo in [-64, 63]: K codes then feed the matrix
+// cores as raw bytes and the integer dot products are exact.
+template <int D>
+__device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsigned int b, unsigned int head, bool head_valid,
+                                                  unsigned int j, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64], float& q_step)
+{
+    constexpr int G = D / 64;
+    float x[G][16];
+    float q_absmax = 0.0f;
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            x[a][e] = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + a * 64 + j * 16 + e, p.q_dtype) : 0.0f;
+            q_absmax = fmaxf(q_absmax, fabsf(x[a][e]));
+        }
+    }
+    q_absmax = wave_max_16x4(q_absmax);
+    const bool q_ok = q_absmax > 0.0f && q_absmax < __builtin_inff();
+    q_step = q_ok ? q_absmax * (1.0f / 16256.0f) : 0.0f;
+    const float inv_step = q_ok ? 16256.0f / q_absmax : 0.0f;
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            unsigned int hi_word = 0, lo_word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                int qi = (int)rintf(x[a][4 * w + e] * inv_step);
+                qi = max(-16256, min(16256, qi));
+                const int hi = (qi + 64) >> 7;
+                const int lo = qi - hi * 128;
+                hi_word |= ((unsigned int)hi & 0xffu) << (8 * e);
+                lo_word |= ((unsigned int)lo & 0xffu) << (8 * e);
+            }
+            qhi[a][w] = (int)hi_word;
+            qlo[a][w] = (int)lo_word;
+        }
+    }
+}
+
+// One 32-token step, first half: scores, masking and the online-softmax update.
+//   k[i][a]   16 K codes of the lane's token of tile i, scale group a (raw bytes = int8 MFMA A operand)
+//   ksr[i*4+r] scale row of token slot (tile i, row 4j + r) -- the C layout of the score tile
+// Leaves the step's probabilities in pr[] (same slots) and rescales acc when the running max moved.
+template <int G, int SDT, bool SOFTCAP>
+__device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const ScaleRow<G> (&ksr)[8], const i32x4 (&qhi)[G],
+                                            const i32x4 (&qlo)[G], float scale_log2, float inv_cap, float cap_log2,
+                                            unsigned int t0, unsigned int j, unsigned int first, unsigned int len,
+                                            float& run_max, float& run_sum, f32x4 (&acc)[G * 4], float (&pr)[8])
+{
+    constexpr int MT = G * 4;
+    // ---- S^T = K . Q^T, one accumulator per scale group -----------------------------
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        float tile_s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+            const i32x4 kc = __builtin_bit_cast(i32x4, k[i][a]);
+            const i32x4 zero = {0, 0, 0, 0};
+            const i32x4 dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qhi[a], zero, 0, 0, 0);
+            const i32x4 dl = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qlo[a], zero, 0, 0, 0);
+            f32x4 d;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                d[r] = (float)(dh[r] * 128 + dl[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(ksr[i * 4 + r].get(a)), tile_s[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float x = tile_s[r] * scale_log2;
+            if constexpr (SOFTCAP) {
+                x = cap_log2 * fast_tanh(x * inv_cap);
+            }
+            const unsigned int token = t0 + 16u * i + 4u * j + r;
+            sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
+        }
+    }
+    // ---- online softmax (base 2) -----------------------------------------------------
+    float step_max = sc[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) {
+        step_max = fmaxf(step_max, sc[e]);
+    }
+    step_max = wave_max_16x4(step_max);
+    const float new_max = fmaxf(run_max, step_max);
+    const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+    const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
+    float step_sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+        step_sum += pr[e];
+    }
+    run_sum = run_sum * alpha + step_sum;
+    run_max = new_max;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            acc[t] *= alpha;
+        }
+    }
+}
+
+// Second half: O^T += V^T . P' with P' = p * v_scale split into bf16 hi + lo.
+//   v[i*4+r][a]  4 V codes (dims a*64 + 4m .. +4) of token slot (tile i, row 4j + r)
+template <int G, int SDT>
+__device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const ScaleRow<G> (&vsr)[8], const float (&pr)[8],
+                                    f32x4 (&acc)[G * 4])
+{
+    // ---- O^T += V^T . P', P' = p * v_scale split into bf16 hi + lo --------------------
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+        Frag phi, plo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(vsr[2 * e].get(a));
+            const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(vsr[2 * e + 1].get(a));
+            unsigned int hi, lo;
+            split_bf16_pair(x0, x1, hi, lo);
+            phi.u[e] = hi;
+            plo.u[e] = lo;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            Frag vf;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                vf.u[c] = pack_bf16_trunc(byte_to_f32(v[2 * c][a], e), byte_to_f32(v[2 * c + 1][a], e));
+            }
+            f32x4 d = acc[a * 4 + e];
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi.b, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo.b, d, 0, 0, 0);
+            acc[a * 4 + e] = d;
+        }
+    }
+}
+
 // NBUF = steps of KV kept in registers: loads run NBUF - 1 steps (32 tokens each) ahead of the MFMA work.
 // With pages scattered over a large pool every page costs an address translation as well as an HBM access,
 // and one step of prefetch leaves the wave waiting ~3.5 us per step.
@@ -155,28 +302,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
-    // ---- Q fragments: B operand, lane = (head column m, k-slice j) ------------------------
-    Frag qhi[G][2], qlo[G][2];
-#pragma unroll
-    for (int a = 0; a < G; ++a) {
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            float x[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[e] = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + a * 64 + j * 16 + hf * 8 + e, p.q_dtype) : 0.0f;
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                unsigned int hi, lo;
-                split_bf16_pair(x[2 * e], x[2 * e + 1], hi, lo);
-                qhi[a][hf].u[e] = hi;
-                if constexpr (QSPLIT) {
-                    qlo[a][hf].u[e] = lo;
-                }
-            }
-        }
-    }
+    i32x4 qhi[G], qlo[G];
+    float q_step; // value of one fixed-point unit of this lane's head
+    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
 
     const unsigned int* table = p.tables + (size_t)b * p.table_stride;
     const unsigned int k_row = p.num_kv_heads * D;           // bytes per cache row (codes)
@@ -200,6 +328,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         entries0 = p.tables != nullptr ? table[min(first_page + lane, last_page)] : first_page + lane;
         entries1 = p.tables != nullptr ? table[min(first_page + 64u + lane, last_page)] : first_page + 64u + lane;
     }
+    // Pin the two registers here: the wait for their loads is placed at this point, once, instead of in
+    // front of every v_readlane inside the loop (where a full vmcnt(0) would also drain the KV prefetch).
+    asm volatile("" : "+v"(entries0), "+v"(entries1));
     auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
         unsigned int t = min(max(T, lo_tile), hi_tile);
         if (p.ring_capacity != 0) {
@@ -289,7 +420,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     }
     float run_max = kNegInf; // log2 units
     float run_sum = 0.0f;    // lane-partial (this lane's 8 token slots per step)
-    const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
+    const float scale_log2 = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_step;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
     const float cap_log2 = p.softcap * kLog2e;
 
@@ -320,91 +451,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
                 vsr[e] = s.vs[e];
             }
         }
-        // ---- S^T = K . Q^T, one accumulator per scale group -----------------------------
-        float sc[8];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            float tile_s[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int a = 0; a < G; ++a) {
-                Frag k0, k1;
-                const u32x2 c0 = codes4_to_bf16(s.k[i][a].x), c1 = codes4_to_bf16(s.k[i][a].y);
-                const u32x2 c2 = codes4_to_bf16(s.k[i][a].z), c3 = codes4_to_bf16(s.k[i][a].w);
-                k0.u = u32x4{c0.x, c0.y, c1.x, c1.y};
-                k1.u = u32x4{c2.x, c2.y, c3.x, c3.y};
-                f32x4 d = {0.f, 0.f, 0.f, 0.f};
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qhi[a][0].b, d, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qhi[a][1].b, d, 0, 0, 0);
-                if constexpr (QSPLIT) {
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qlo[a][0].b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qlo[a][1].b, d, 0, 0, 0);
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(ksr[i * 4 + r].get(a)), tile_s[r]);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float x = tile_s[r] * scale_log2;
-                if constexpr (SOFTCAP) {
-                    x = cap_log2 * fast_tanh(x * inv_cap);
-                }
-                const unsigned int token = t0 + 16u * i + 4u * j + r;
-                sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
-            }
-        }
-        // ---- online softmax (base 2) -----------------------------------------------------
-        float step_max = sc[0];
-#pragma unroll
-        for (int e = 1; e < 8; ++e) {
-            step_max = fmaxf(step_max, sc[e]);
-        }
-        step_max = wave_max_16x4(step_max);
-        const float new_max = fmaxf(run_max, step_max);
-        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-        const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
         float pr[8];
-        float step_sum = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
-            step_sum += pr[e];
-        }
-        run_sum = run_sum * alpha + step_sum;
-        run_max = new_max;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[t] *= alpha;
-            }
-        }
-        // ---- O^T += V^T . P', P' = p * v_scale split into bf16 hi + lo --------------------
-#pragma unroll
-        for (int a = 0; a < G; ++a) {
-            Frag phi, plo;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(vsr[2 * e].get(a));
-                const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(vsr[2 * e + 1].get(a));
-                unsigned int hi, lo;
-                split_bf16_pair(x0, x1, hi, lo);
-                phi.u[e] = hi;
-                plo.u[e] = lo;
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                Frag vf;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    vf.u[c] = pack_bf16_trunc(byte_to_f32(s.v[2 * c][a], e), byte_to_f32(s.v[2 * c + 1][a], e));
-                }
-                f32x4 d = acc[a * 4 + e];
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi.b, d, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo.b, d, 0, 0, 0);
-                acc[a * 4 + e] = d;
-            }
-        }
+        qk_softmax_step<G, SDT, SOFTCAP>(s.k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
+        pv_step<G, SDT>(s.v, vsr, pr, acc);
     };
 
     // ---- software pipeline: loads of steps n+1 .. n+NBUF-1 in flight while step n computes ----------
@@ -415,17 +464,22 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             load_step(buf[u], c_start + u * 32u);
         }
     }
-    for (unsigned int base = 0; base < steps; base += NBUF) {
+    // The main loop issues its loads unconditionally (past the end it re-reads the last step, an L2 hit):
+    // a conditional load would make the compiler merge "loads in flight" with "none in flight" and wait for
+    // everything before each compute step, which serialises the prefetch.
+    unsigned int base = 0;
+    for (; base + NBUF <= steps; base += NBUF) {
 #pragma unroll
         for (int u = 0; u < NBUF; ++u) {
             const unsigned int step = base + u;
-            if (step < steps) {
-                const unsigned int ahead = step + NBUF - 1;
-                if (ahead < steps) {
-                    load_step(buf[(u + NBUF - 1) % NBUF], c_start + ahead * 32u);
-                }
-                compute_step(buf[u], c_start + step * 32u);
-            }
+            load_step(buf[(u + NBUF - 1) % NBUF], c_start + min(step + NBUF - 1, steps - 1u) * 32u);
+            compute_step(buf[u], c_start + step * 32u);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u) {
+        if (base + u < steps) {
+            compute_step(buf[u], c_start + (base + u) * 32u);
         }
     }
 
@@ -438,6 +492,235 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         }
         float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
         // tile (a, e), register r holds dim a*64 + 16*j + 4*r + e
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const f32x4 v = {acc[a * 4 + 0][r], acc[a * 4 + 1][r], acc[a * 4 + 2][r], acc[a * 4 + 3][r]};
+                *(f32x4*)(out + a * 64 + 16 * j + 4 * r) = v;
+            }
+        }
+    }
+}
+
+// ---- head_dim 128: K, V and scale rows travel global -> LDS without touching registers ---------
+// Each wave owns a private LDS region (no barriers): rings of two 32-token steps for the K codes, the V
+// codes and the scale rows of its KV head.  global_load_lds moves 64 x 16 B per instruction; eight
+// neighbouring lanes fetch one whole 128-byte row slice, so every request is a full cache line and the
+// loads can be marked non-temporal (lines are used exactly once).  The 16-byte chunk a lane fetches is
+// XOR-swizzled with its row, which makes the later ds_read_b128 of MFMA operands bank-conflict free.
+// The compiler does not order LDS reads against these loads, so the waits are explicit: loads are issued
+// in a fixed order, unconditionally, and s_waitcnt vmcnt(N) counts the instructions issued since.
+constexpr int kDmaPlaneStep = 2 * 16 * 128;                              // one plane, one step, one KV head
+constexpr int kDmaScaleStep = 2 * 32 * 4;                                // K and V scale rows of one step
+constexpr int kDmaWaveBytes = 4 * kDmaPlaneStep + 2 * kDmaScaleStep;     // 16896
+constexpr int kDmaWaves = 8;
+
+template <int N> __device__ __forceinline__ void wait_vmcnt()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void wait_lds_reads()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+template <int SDT, bool SOFTCAP>
+__global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
+{
+    constexpr int D = 128, G = 2, MT = 8;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_all[kDmaWaves * kDmaWaveBytes];
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned int waves = blockDim.x >> 6;
+    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
+    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
+    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const unsigned int b = blockIdx.z;
+    const unsigned int chunk = blockIdx.x;
+    if (kvh >= p.num_kv_heads) {
+        return;
+    }
+    const unsigned int len = p.kv_lens[b];
+    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+    first = min(first, len);
+    const unsigned int first_al = first & ~31u;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned int head_in_group = head_block * 16u + m;
+    const bool head_valid = head_in_group < p.group;
+    const unsigned int head = kvh * p.group + head_in_group;
+    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    if (c_start64 >= len) {
+        if (head_valid && j == 0) {
+            p.stats[stat_index] = kNegInf;
+            p.stats[stat_index + 1] = 0.0f;
+        }
+        return;
+    }
+    const unsigned int c_start = (unsigned int)c_start64;
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int steps = (c_end - c_start + 31u) / 32u;
+
+    i32x4 qhi[G], qlo[G];
+    float q_step;
+    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
+
+    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int k_row = p.num_kv_heads * D;
+    const unsigned int s_row = p.num_kv_heads * G * 2u;
+    const unsigned char* k_base = p.k_plane + (size_t)kvh * D;
+    const unsigned char* v_base = p.v_plane + (size_t)kvh * D;
+    const unsigned int block_mask = p.block_tokens - 1u;
+    const unsigned int lo_tile = first & ~15u;
+    const unsigned int hi_tile = (len - 1u) & ~15u;
+
+    // block-table entries of this split: lane i holds entry first_page + i (+ 64); the launcher keeps a
+    // split within 128 pages
+    const unsigned int first_page = min(max(c_start, lo_tile), hi_tile) >> p.block_shift;
+    const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
+    unsigned int entries0 = p.tables != nullptr ? table[min(first_page + lane, last_page)] : first_page + lane;
+    unsigned int entries1 = p.tables != nullptr ? table[min(first_page + 64u + lane, last_page)] : first_page + 64u + lane;
+    asm volatile("" : "+v"(entries0), "+v"(entries1)); // their wait happens here, not inside the loop
+    auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
+        const unsigned int t = min(max(T, lo_tile), hi_tile);
+        const unsigned int idx = __builtin_amdgcn_readfirstlane((t >> p.block_shift) - first_page) & 127u;
+        const unsigned int e0 = __builtin_amdgcn_readlane(entries0, idx & 63u);
+        const unsigned int e1 = __builtin_amdgcn_readlane(entries1, idx & 63u);
+        const unsigned int entry = idx < 64u ? e0 : e1;
+        return ((unsigned long long)entry << p.block_shift) + (t & block_mask);
+    };
+
+    // ---- LDS map of this wave -----------------------------------------------------------------
+    unsigned char* const wave_lds = lds_all + wave * kDmaWaveBytes;
+    unsigned char* const lds_k = wave_lds;                      // [slot 2][tile 2][row 16][128]
+    unsigned char* const lds_v = wave_lds + 2 * kDmaPlaneStep;  // same
+    unsigned char* const lds_s = wave_lds + 4 * kDmaPlaneStep;  // [slot 2][plane K,V][token 32][4]
+
+    // global side of a code-tile load: lane -> (row lane / 8 [+ 8], swizzled 16-byte chunk)
+    const unsigned int code_goff = (lane >> 3) * k_row + (((lane & 7u) ^ (lane >> 3)) << 4);
+    // global side of the scale load: lane -> (plane lane / 32, token lane % 32)
+    const bool s_tile1 = ((lane >> 4) & 1u) != 0;
+    const unsigned char* s_lane_base = (lane >= 32u ? p.v_scales : p.k_scales) + (size_t)kvh * G * 2u + (size_t)(lane & 15u) * s_row;
+    // LDS side: MFMA operand addresses (chunk c of row r sits at r * 128 + ((c ^ (r & 7)) << 4))
+    unsigned int k_lds[G], v_lds[4];
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+        k_lds[a] = m * 128u + (((4u * a + j) ^ (m & 7u)) << 4);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const unsigned int row = 4u * j + r;
+        v_lds[r] = row * 128u + (((m >> 2) ^ (row & 7u)) << 4) + (m & 3u) * 4u; // group 0; group 1 = ^ 64
+    }
+    const unsigned int s_lds = 16u * j;
+
+    auto issue_codes = [&](const unsigned char* plane_base, unsigned char* ring, int slot, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const unsigned long long R = tile_row(t0 + 16u * i);
+            const unsigned char* src = plane_base + R * k_row; // uniform
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)h * 8u * k_row + code_goff),
+                                                 (lds_ptr_t)(ring + slot * kDmaPlaneStep + i * 2048 + h * 1024), 16, 0, 2);
+            }
+        }
+    };
+    auto issue_scales = [&](int slot, unsigned int t0) __attribute__((always_inline)) {
+        const unsigned long long R0 = tile_row(t0);
+        const unsigned long long R1 = tile_row(t0 + 16u);
+        const unsigned long long R = s_tile1 ? R1 : R0;
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(s_lane_base + R * s_row), (lds_ptr_t)(lds_s + slot * kDmaScaleStep), 4, 0, 0);
+    };
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float run_max = kNegInf;
+    float run_sum = 0.0f;
+    const float scale_log2 = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_step;
+    const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
+    const float cap_log2 = p.softcap * kLog2e;
+
+    // Issue order per step n (9 instructions): K(n+2) x4, scales(n+2) x1, [QK, softmax], V(n+2) x4.
+    //   K(n), scales(n) complete  <=> at most 13 newer loads outstanding (V(n), K/S/V(n+1))
+    //   V(n) complete             <=> at most 14 newer loads outstanding (K/S/V(n+1), K/S(n+2))
+    auto step = [&](auto slot_c, unsigned int n) __attribute__((always_inline)) {
+        constexpr int slot = decltype(slot_c)::value;
+        const unsigned int t0 = c_start + n * 32u;
+        const unsigned int t_next = c_start + min(n + 2u, steps - 1u) * 32u; // past the end: re-read the last step
+        wait_vmcnt<13>();
+        u32x4 k[2][G];
+        ScaleRow<G> ksr[8], vsr[8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int a = 0; a < G; ++a) {
+                k[i][a] = *(const u32x4*)(lds_k + slot * kDmaPlaneStep + i * 2048 + k_lds[a]);
+            }
+            const u32x4 ks4 = *(const u32x4*)(lds_s + slot * kDmaScaleStep + i * 64 + s_lds);
+            const u32x4 vs4 = *(const u32x4*)(lds_s + slot * kDmaScaleStep + 128 + i * 64 + s_lds);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                ksr[i * 4 + r].v = ks4[r];
+                vsr[i * 4 + r].v = vs4[r];
+            }
+        }
+        wait_lds_reads();
+        issue_codes(k_base, lds_k, slot, t_next);
+        issue_scales(slot, t_next);
+        float pr[8];
+        qk_softmax_step<G, SDT, SOFTCAP>(k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
+        wait_vmcnt<14>();
+        unsigned int v[8][G];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                v[i * 4 + r][0] = *(const unsigned int*)(lds_v + slot * kDmaPlaneStep + i * 2048 + v_lds[r]);
+                v[i * 4 + r][1] = *(const unsigned int*)(lds_v + slot * kDmaPlaneStep + i * 2048 + (v_lds[r] ^ 64u));
+            }
+        }
+        wait_lds_reads();
+        issue_codes(v_base, lds_v, slot, t_next);
+        pv_step<G, SDT>(v, vsr, pr, acc);
+    };
+
+    // prologue: steps 0 and 1 in the same order the loop issues them
+    {
+        const unsigned int t1 = c_start + min(1u, steps - 1u) * 32u;
+        issue_codes(k_base, lds_k, 0, c_start);
+        issue_scales(0, c_start);
+        issue_codes(v_base, lds_v, 0, c_start);
+        issue_codes(k_base, lds_k, 1, t1);
+        issue_scales(1, t1);
+        issue_codes(v_base, lds_v, 1, t1);
+    }
+    unsigned int n = 0;
+    for (; n + 2u <= steps; n += 2u) {
+        step(std::integral_constant<int, 0>{}, n);
+        step(std::integral_constant<int, 1>{}, n + 1u);
+    }
+    if (n < steps) {
+        step(std::integral_constant<int, 0>{}, n);
+    }
+    wait_vmcnt<0>(); // no load may still be writing this workgroup's LDS when the wave ends
+
+    const float total = wave_sum_16x4(run_sum);
+    if (head_valid) {
+        if (j == 0) {
+            p.stats[stat_index] = run_max;
+            p.stats[stat_index + 1] = total;
+        }
+        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
 #pragma unroll
         for (int a = 0; a < G; ++a) {
 #pragma unroll
@@ -775,6 +1058,18 @@ template <int D, int SDT, bool QSPLIT>
 hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
     const bool cap = p.softcap > 0.0f;
+    if constexpr (D == 128) {
+        // direct-to-LDS pipeline: needs the whole split's block-table entries in two registers (128 pages)
+        if (fast && p.ring_capacity == 0 && p.chunk_tokens <= 127u * p.block_tokens && block.x <= 64u * kDmaWaves &&
+            getenv("ZLLM_TUNE_NODMA") == nullptr) {
+            if (cap) {
+                gqa_decode_q8_dma128<SDT, true><<<grid, block, 0, stream>>>(p);
+            } else {
+                gqa_decode_q8_dma128<SDT, false><<<grid, block, 0, stream>>>(p);
+            }
+            return hipGetLastError();
+        }
+    }
     constexpr int kDeep = (D <= 128 && !QSPLIT) ? 4 : (D <= 128 ? 3 : 2); // register budget: 256 per lane
     const char* env = getenv("ZLLM_TUNE_NBUF");
     const int nbuf = env != nullptr ? atoi(env) : 2;
@@ -800,11 +1095,10 @@ hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block,
 
 template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtype, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
-    const bool split = p.q_dtype != 1; // bf16 queries are exact in one bf16 term
     if (scale_dtype == 0) {
-        return split ? launch_q8<D, 0, true>(p, fast, grid, block, stream) : launch_q8<D, 0, false>(p, fast, grid, block, stream);
+        return launch_q8<D, 0, false>(p, fast, grid, block, stream);
     }
-    return split ? launch_q8<D, 1, true>(p, fast, grid, block, stream) : launch_q8<D, 1, false>(p, fast, grid, block, stream);
+    return launch_q8<D, 1, false>(p, fast, grid, block, stream);
 }
 
 } // namespace
