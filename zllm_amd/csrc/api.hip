@@ -375,6 +375,10 @@ int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
         a->workspace == nullptr || (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
         return fail(-1, "GQA decode: null pointer");
     }
+    if ((((uintptr_t)a->q | (uintptr_t)a->k_plane | (uintptr_t)a->v_plane | (uintptr_t)a->workspace | (uintptr_t)a->out) & 15u) != 0 ||
+        (((uintptr_t)a->k_scales | (uintptr_t)a->v_scales) & 3u) != 0) {
+        return fail(-1, "GQA decode: q, cache planes, out and workspace must be 16-byte aligned (scale planes 4-byte)");
+    }
     const uint64_t need = zllm_attn_gqa_decode_workspace_bytes(a);
     if (a->workspace_bytes < need) {
         return fail(-1, "GQA decode: workspace %llu bytes, need %llu", (unsigned long long)a->workspace_bytes, (unsigned long long)need);

@@ -116,6 +116,45 @@ template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(
     return out;
 }
 
+// Split-KV work items are numbered densely over the batch: item = (sequence b, split c) with
+// c < splits(b), sequences in order.  Workgroups are handed to the XCDs round-robin by their linear id, so
+// a dense numbering spreads the live workgroups of a ragged batch evenly (a [split][sequence] grid leaves
+// gaps where short sequences end, and one XCD can end up with more live workgroups than CUs).  Every wave
+// finds its item by a prefix sum over the sequences' split counts; ids past the last item exit.
+__device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned int item, unsigned int lane, unsigned int& b_out,
+                                             unsigned int& chunk_out)
+{
+    unsigned int base = 0;
+    for (unsigned int b0 = 0; b0 < p.batch; b0 += 64u) {
+        const unsigned int i = b0 + lane;
+        unsigned int n = 0;
+        if (i < p.batch) {
+            const unsigned int len = p.kv_lens[i];
+            unsigned int first = p.first_visible != nullptr ? p.first_visible[i] : 0u;
+            first = min(first, len);
+            const unsigned int first_al = first & ~31u;
+            n = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+        }
+        unsigned int incl = n; // inclusive prefix sum over the wave
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned int up = __shfl_up(incl, d);
+            incl += lane >= (unsigned int)d ? up : 0u;
+        }
+        const unsigned int total = __builtin_amdgcn_readlane(incl, 63);
+        if (item < base + total) {
+            const unsigned int local = item - base;
+            const unsigned long long hit = __ballot(local >= incl - n && local < incl);
+            const unsigned int src = (unsigned int)__builtin_ctzll(hit);
+            b_out = b0 + src;
+            chunk_out = local - (__builtin_amdgcn_readlane(incl, src) - __builtin_amdgcn_readlane(n, src));
+            return true;
+        }
+        base += total;
+    }
+    return false;
+}
+
 // Q fragments: B operand of the int8 MFMA, lane = (head column m, k-slice j).
 // The head's query row is quantized to 15-bit fixed point (step = max|q| / 16256) and split into two
 // signed-byte digits q = 128 * hi + lo, hi in [-127, 127], lo in [-64, 63]: K codes then feed the matrix
@@ -126,12 +165,56 @@ __device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsi
 {
     constexpr int G = D / 64;
     float x[G][16];
+    // 16 consecutive elements per scale group, fetched as whole 16-byte vectors (one round trip, not 32)
+    const size_t q_index = ((size_t)b * p.num_heads + head) * D + j * 16;
+    if (!head_valid) {
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                x[a][e] = 0.0f;
+            }
+        }
+    } else if (p.q_dtype == 0) {
+        f32x4 raw[G][4];
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                raw[a][w] = *(const f32x4*)((const float*)p.q + q_index + a * 64 + 4 * w);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                x[a][e] = raw[a][e / 4][e % 4];
+            }
+        }
+    } else {
+        u32x4 raw[G][2];
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                raw[a][w] = *(const u32x4*)((const unsigned short*)p.q + q_index + a * 64 + 8 * w);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < G; ++a) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const unsigned int word = raw[a][e / 8][(e % 8) / 2];
+                const unsigned short bits = (unsigned short)((e & 1) ? (word >> 16) : (word & 0xffffu));
+                x[a][e] = p.q_dtype == 1 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+            }
+        }
+    }
     float q_absmax = 0.0f;
 #pragma unroll
     for (int a = 0; a < G; ++a) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            x[a][e] = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + a * 64 + j * 16 + e, p.q_dtype) : 0.0f;
             q_absmax = fmaxf(q_absmax, fabsf(x[a][e]));
         }
     }
@@ -276,9 +359,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    const unsigned int b = blockIdx.z;
-    const unsigned int chunk = blockIdx.x;
-    if (kvh >= p.num_kv_heads) {
+    unsigned int b, chunk;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
         return;
     }
     const unsigned int len = p.kv_lens[b];
@@ -515,6 +597,9 @@ constexpr int kDmaPlaneStep = 2 * 16 * 128;                              // one 
 constexpr int kDmaScaleStep = 2 * 32 * 4;                                // K and V scale rows of one step
 constexpr int kDmaWaveBytes = 4 * kDmaPlaneStep + 2 * kDmaScaleStep;     // 16896
 constexpr int kDmaWaves = 8;
+#ifndef ZLLM_CODE_AUX
+#define ZLLM_CODE_AUX 2 /* nt */
+#endif
 
 template <int N> __device__ __forceinline__ void wait_vmcnt()
 {
@@ -542,9 +627,8 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    const unsigned int b = blockIdx.z;
-    const unsigned int chunk = blockIdx.x;
-    if (kvh >= p.num_kv_heads) {
+    unsigned int b, chunk;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
         return;
     }
     const unsigned int len = p.kv_lens[b];
@@ -566,10 +650,6 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int c_start = (unsigned int)c_start64;
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
-
-    i32x4 qhi[G], qlo[G];
-    float q_step;
-    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
 
     const unsigned int* table = p.tables + (size_t)b * p.table_stride;
     const unsigned int k_row = p.num_kv_heads * D;
@@ -628,7 +708,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)h * 8u * k_row + code_goff),
-                                                 (lds_ptr_t)(ring + slot * kDmaPlaneStep + i * 2048 + h * 1024), 16, 0, 2);
+                                                 (lds_ptr_t)(ring + slot * kDmaPlaneStep + i * 2048 + h * 1024), 16, 0, ZLLM_CODE_AUX);
             }
         }
     };
@@ -646,6 +726,22 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     }
     float run_max = kNegInf;
     float run_sum = 0.0f;
+
+    // prologue: steps 0 and 1 in the same order the loop issues them; the query is fetched and quantized
+    // while these loads are in flight
+    {
+        const unsigned int t1 = c_start + min(1u, steps - 1u) * 32u;
+        issue_codes(k_base, lds_k, 0, c_start);
+        issue_scales(0, c_start);
+        issue_codes(v_base, lds_v, 0, c_start);
+        issue_codes(k_base, lds_k, 1, t1);
+        issue_scales(1, t1);
+        issue_codes(v_base, lds_v, 1, t1);
+    }
+    i32x4 qhi[G], qlo[G];
+    float q_step;
+    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
+
     const float scale_log2 = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_step;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
     const float cap_log2 = p.softcap * kLog2e;
@@ -658,6 +754,13 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         const unsigned int t0 = c_start + n * 32u;
         const unsigned int t_next = c_start + min(n + 2u, steps - 1u) * 32u; // past the end: re-read the last step
         wait_vmcnt<13>();
+#ifdef ZLLM_PROBE_LOADS_ONLY
+        issue_codes(k_base, lds_k, slot, t_next);
+        issue_scales(slot, t_next);
+        wait_vmcnt<14>();
+        issue_codes(v_base, lds_v, slot, t_next);
+        return;
+#endif
         u32x4 k[2][G];
         ScaleRow<G> ksr[8], vsr[8];
 #pragma unroll
@@ -694,16 +797,6 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         pv_step<G, SDT>(v, vsr, pr, acc);
     };
 
-    // prologue: steps 0 and 1 in the same order the loop issues them
-    {
-        const unsigned int t1 = c_start + min(1u, steps - 1u) * 32u;
-        issue_codes(k_base, lds_k, 0, c_start);
-        issue_scales(0, c_start);
-        issue_codes(v_base, lds_v, 0, c_start);
-        issue_codes(k_base, lds_k, 1, t1);
-        issue_scales(1, t1);
-        issue_codes(v_base, lds_v, 1, t1);
-    }
     unsigned int n = 0;
     for (; n + 2u <= steps; n += 2u) {
         step(std::integral_constant<int, 0>{}, n);
@@ -753,9 +846,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    const unsigned int b = blockIdx.z;
-    const unsigned int chunk = blockIdx.x;
-    if (kvh >= p.num_kv_heads) {
+    unsigned int b, chunk;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
         return;
     }
     const unsigned int len = p.kv_lens[b];
@@ -1118,7 +1210,7 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_
     const unsigned int waves = p.num_kv_heads < max_waves ? p.num_kv_heads : max_waves;
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int head_blocks = (p.group + 15u) / 16u;
-    const dim3 grid(p.max_chunks, kvh_blocks * head_blocks, p.batch);
+    const dim3 grid(p.max_chunks * p.batch, kvh_blocks * head_blocks, 1);
     const dim3 block(waves * 64u);
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const bool fast = pow2 && p.block_tokens >= 16u && p.ring_capacity % 16u == 0;
