@@ -25,6 +25,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+# HBM bytes one launch of the partial kernel moves on the default workload: rocprofv3 FETCH_SIZE and WRITE_SIZE
+# per dispatch, each scaled by what the same counter reads for a 1 GiB device copy (FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0); the runs and their numbers are in profiles/gqa_decode_q8_dma128__gqa_decode_32k.md.
+GQA_32K_TRAFFIC_BYTES = 585164609
 METRIC = "decode attn effective KV GB/s (% of HBM peak) + tokens/s at 32K ctx, 1 GPU"
 
 
@@ -34,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk", "copy_calibration"])
     ap.add_argument("--pool-gib", type=float, default=160.0, help="address span of the paged pool (all four planes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -223,14 +227,15 @@ def run_gqa_decode(args, ragged):
                                 + ", 16-token pages"),
                    "kv_lens": lens, "kv_bytes_per_call": kv_bytes, "bytes_per_token": bytes_per_token, "seed": args.seed,
                    "pool_bytes": pool["pool_bytes"], "pool_blocks": pool["pool_blocks"], "max_code_plane_offset": pool["max_code_offset"],
-                   "q_dtype": "bf16", "scale_dtype": "f16", "kv_arithmetic": "int8 codes -> bf16 MFMA operands, f32 accumulate"},
+                   "q_dtype": "bf16", "scale_dtype": "f16", "kv_arithmetic": "K.Q on int8 MFMA (K codes raw, Q as two 8-bit digits); P.V on bf16 MFMA (V codes exact in bf16); f32 accumulate"},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "ms_per_step_events": round(ms_events, 5),
         "ms_per_step_eager_launch": round(ms_eager, 5),
         "launch": "hipGraph replay of one decode step (partial + merge)",
-        "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_partial", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_dma128", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None if ragged or args.seed != 2 else GQA_32K_TRAFFIC_BYTES,
                      "kernel_ms": round(ms_partial, 5)},
     }
     if not args.no_cpu_baseline:
@@ -238,6 +243,22 @@ def run_gqa_decode(args, ragged):
         record["cpu_baseline"] = cpu
         record["parity_vs_oracle_max_abs"] = float(np.abs(out.cpu().numpy() - cpu_out).max())
     print(json.dumps(record))
+
+
+def run_copy_calibration(args):
+    """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters of the
+    attention kernels are scaled by (the counters do not report bytes one-to-one on this GPU)."""
+    import torch
+
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        dst.copy_(src)
+    ms = event_time_ms(lambda: dst.copy_(src), args.steps)
+    print(json.dumps({"metric": "device copy (counter calibration)", "value": round(2 * n / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+                      "config": {"workload": "torch uint8 copy_", "bytes_read": n, "bytes_written": n}}))
 
 
 def main():
@@ -249,6 +270,8 @@ def main():
         run_gqa_decode(args, ragged=False)
     elif args.workload == "gqa_decode_ragged":
         run_gqa_decode(args, ragged=True)
+    elif args.workload == "copy_calibration":
+        run_copy_calibration(args)
     else:
         from zllm_amd import bench_extra
 
