@@ -108,8 +108,7 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
-    const char* rounds_env = getenv("ZLLM_TUNE_ROUNDS");
-    const uint32_t rounds = rounds_env ? (uint32_t)atoi(rounds_env) : 1u;
+    const uint32_t rounds = 1u; // workgroups per CU over the call
     const uint32_t columns = a->batch * kvh_blocks * head_blocks;
     const uint64_t uniform_total = (uint64_t)a->batch * a->max_kv_len;
     if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && rounds * kComputeUnits > 2 * columns) {

@@ -1,29 +1,32 @@
 // GQA split-KV flash decoding over a paged Q8g64 (or f16) KV cache — gfx950.
 //
 // Work decomposition
-//   grid = (split, kv-head block x head block, sequence); one wave64 per KV head.
+//   grid = (work item, kv-head block x head block); work item = (sequence, split), numbered
+//   densely over the batch; one wave64 per KV head.
 //   The waves of a workgroup cover neighbouring KV heads of the SAME tokens, so
 //   together they read whole cache rows (all KV heads of a token are contiguous:
 //   row = num_kv_heads * head_dim bytes) and share the row's scale line.
 //   Waves never synchronise with each other.
 //
 // Per wave, per 32-token step (two 16-token tiles):
-//   S^T[token, head] = K[token, :] . Q[head, :]      MFMA 16x16x32 bf16, A = K codes
-//                                                    (exact in bf16), B = Q (bf16 hi [+ lo])
-//     one accumulator per 64-column scale group, so the group scale is applied to
-//     the finished partial dot: s = sum_g scale_g * dot_g  (no per-element multiply)
+//   S^T[token, head] = K[token, :] . Q[head, :]      int8 MFMA 16x16x64, A = K codes as stored,
+//                                                    B = Q in 15-bit fixed point, two 8-bit digits
+//     one MFMA pair per 64-column scale group, so the group scale is applied to the finished
+//     integer dot: s = sum_g scale_g * dot_g  (no per-element multiply, no K conversion)
 //   online softmax: row max / row sum over the four 16-lane groups by wave shuffles
-//   O^T[dim, head] += V^T[dim, token] . P'[token, head]   MFMA, A = V codes (bf16),
-//     B = P' = p * v_scale_g split into bf16 hi + lo (16 significant bits)
+//   O^T[dim, head] += V^T[dim, token] . P'[token, head]   bf16 MFMA 16x16x32, A = V codes
+//     (exact in bf16), B = P' = p * v_scale_g split into bf16 hi + lo (16 significant bits)
 //   The C layout of S^T (lane = head column, 4 token rows) is exactly the B layout
 //   needed for P', so probabilities never leave their registers.
+//
+// Two kernels share that step: gqa_decode_q8_dma128 (head_dim 128, pages of >= 16 tokens, no ring)
+// streams K, V and scales global -> LDS with non-temporal full-line loads; gqa_decode_q8_partial
+// covers every other geometry with a two-deep register pipeline.
 //
 // Why MFMA for a bandwidth-bound op: with 8 query heads per KV head the path needs
 // 7.8 FMA per KV byte; at 70 % of 8 TB/s that is 43 T FMA/s, above the 39 T FMA/s
 // the chip's (non-packed) FP32 vector units can issue.  On the matrix cores the
-// same work is < 15 % of peak and the vector units only convert int8 -> bf16.
-#include <stdlib.h>
-
+// same work is < 15 % of peak and the vector units only convert V codes and probabilities.
 #include <type_traits>
 
 #include "common.hpp"
@@ -347,7 +350,7 @@ __device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const Sca
 // NBUF = steps of KV kept in registers: loads run NBUF - 1 steps (32 tokens each) ahead of the MFMA work.
 // With pages scattered over a large pool every page costs an address translation as well as an HBM access,
 // and one step of prefetch leaves the wave waiting ~3.5 us per step.
-template <int D, int SDT, bool QSPLIT, bool FAST, bool SOFTCAP, int NBUF>
+template <int D, int SDT, bool FAST, bool SOFTCAP, int NBUF>
 __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(GqaDecodeParams p)
 {
     constexpr int G = D / 64;           // scale groups per head row
@@ -597,9 +600,7 @@ constexpr int kDmaPlaneStep = 2 * 16 * 128;                              // one 
 constexpr int kDmaScaleStep = 2 * 32 * 4;                                // K and V scale rows of one step
 constexpr int kDmaWaveBytes = 4 * kDmaPlaneStep + 2 * kDmaScaleStep;     // 16896
 constexpr int kDmaWaves = 8;
-#ifndef ZLLM_CODE_AUX
-#define ZLLM_CODE_AUX 2 /* nt */
-#endif
+constexpr int kAuxNonTemporal = 2; // cache-policy bits of the load builtin: nt
 
 template <int N> __device__ __forceinline__ void wait_vmcnt()
 {
@@ -708,7 +709,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)h * 8u * k_row + code_goff),
-                                                 (lds_ptr_t)(ring + slot * kDmaPlaneStep + i * 2048 + h * 1024), 16, 0, ZLLM_CODE_AUX);
+                                                 (lds_ptr_t)(ring + slot * kDmaPlaneStep + i * 2048 + h * 1024), 16, 0, kAuxNonTemporal);
             }
         }
     };
@@ -754,13 +755,6 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         const unsigned int t0 = c_start + n * 32u;
         const unsigned int t_next = c_start + min(n + 2u, steps - 1u) * 32u; // past the end: re-read the last step
         wait_vmcnt<13>();
-#ifdef ZLLM_PROBE_LOADS_ONLY
-        issue_codes(k_base, lds_k, slot, t_next);
-        issue_scales(slot, t_next);
-        wait_vmcnt<14>();
-        issue_codes(v_base, lds_v, slot, t_next);
-        return;
-#endif
         u32x4 k[2][G];
         ScaleRow<G> ksr[8], vsr[8];
 #pragma unroll
@@ -1146,14 +1140,13 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     }
 }
 
-template <int D, int SDT, bool QSPLIT>
+template <int D, int SDT>
 hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
     const bool cap = p.softcap > 0.0f;
     if constexpr (D == 128) {
         // direct-to-LDS pipeline: needs the whole split's block-table entries in two registers (128 pages)
-        if (fast && p.ring_capacity == 0 && p.chunk_tokens <= 127u * p.block_tokens && block.x <= 64u * kDmaWaves &&
-            getenv("ZLLM_TUNE_NODMA") == nullptr) {
+        if (fast && p.ring_capacity == 0 && p.chunk_tokens <= 127u * p.block_tokens && block.x <= 64u * kDmaWaves) {
             if (cap) {
                 gqa_decode_q8_dma128<SDT, true><<<grid, block, 0, stream>>>(p);
             } else {
@@ -1162,24 +1155,17 @@ hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block,
             return hipGetLastError();
         }
     }
-    constexpr int kDeep = (D <= 128 && !QSPLIT) ? 4 : (D <= 128 ? 3 : 2); // register budget: 256 per lane
-    const char* env = getenv("ZLLM_TUNE_NBUF");
-    const int nbuf = env != nullptr ? atoi(env) : 2;
     if (fast) {
         if (cap) {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, true, true, 2><<<grid, block, 0, stream>>>(p);
-        } else if (nbuf >= 4 && kDeep >= 4) {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, kDeep><<<grid, block, 0, stream>>>(p);
-        } else if (nbuf == 3 && kDeep >= 3) {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, (kDeep >= 3 ? 3 : 2)><<<grid, block, 0, stream>>>(p);
+            gqa_decode_q8_partial<D, SDT, true, true, 2><<<grid, block, 0, stream>>>(p);
         } else {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, true, false, 2><<<grid, block, 0, stream>>>(p);
+            gqa_decode_q8_partial<D, SDT, true, false, 2><<<grid, block, 0, stream>>>(p);
         }
     } else {
         if (cap) {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, false, true, 2><<<grid, block, 0, stream>>>(p);
+            gqa_decode_q8_partial<D, SDT, false, true, 2><<<grid, block, 0, stream>>>(p);
         } else {
-            gqa_decode_q8_partial<D, SDT, QSPLIT, false, false, 2><<<grid, block, 0, stream>>>(p);
+            gqa_decode_q8_partial<D, SDT, false, false, 2><<<grid, block, 0, stream>>>(p);
         }
     }
     return hipGetLastError();
@@ -1188,19 +1174,15 @@ hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block,
 template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtype, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
     if (scale_dtype == 0) {
-        return launch_q8<D, 0, false>(p, fast, grid, block, stream);
+        return launch_q8<D, 0>(p, fast, grid, block, stream);
     }
-    return launch_q8<D, 1, false>(p, fast, grid, block, stream);
+    return launch_q8<D, 1>(p, fast, grid, block, stream);
 }
 
 } // namespace
 
 unsigned int gqa_decode_max_waves(unsigned int head_dim)
 {
-    const char* env = getenv("ZLLM_TUNE_WAVES");
-    if (env != nullptr) {
-        return (unsigned int)atoi(env);
-    }
     return head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
 }
 
