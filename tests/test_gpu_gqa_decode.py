@@ -222,3 +222,45 @@ def test_f16_kv_head_dim_128():
     got = run_f16(case, 0.088)
     want = oracle_gqa_decode(case, 0.088, fmt=O.FMT_F16)
     assert_attention_close(got, want, "f16 d=128")
+
+
+def test_batch_larger_than_a_wave_with_empty_sequences():
+    """Work items are numbered over the batch by a 64-lane prefix sum: 70 sequences need two passes of it, and
+    empty sequences in the middle must take no work item and still produce zero rows."""
+    rng = np.random.default_rng(70)
+    lens = rng.integers(1, 600, size=70)
+    lens[[3, 17, 64, 69]] = 0
+    case = make_gqa_q8_case(70, lens, 8, 2, 128)
+    got = run_decode(case, 0.1)
+    want = oracle_gqa_decode(case, 0.1)
+    assert_attention_close(got, want, "batch 70")
+    assert not got[[3, 17, 64, 69]].any()
+
+
+@pytest.mark.parametrize("q_kind", ["f32", "bf16", "f16"])
+def test_query_dtypes_through_fixed_point_digits(q_kind):
+    """The kernel quantizes each query row to 15-bit fixed point for the int8 matrix cores; every input
+    dtype must stay within the attention tolerance, including rows whose elements span a wide range."""
+    from zllm_amd import capi, ops
+
+    case = make_gqa_q8_case(11, [900, 333], 16, 4, 128)
+    q = case["q"].copy().reshape(2, 16, 128)
+    q[0, 0, :] *= 1e-3           # a tiny head
+    q[0, 1, 5] = 40.0            # one dominant element: the other 127 fall to few fixed-point levels
+    q[1, 2, :] = 0.0             # an all-zero head: uniform attention
+    q = q.reshape(2, -1)
+    if q_kind == "bf16":
+        qt = torch.from_numpy(q).to(torch.bfloat16)
+    elif q_kind == "f16":
+        qt = torch.from_numpy(q).to(torch.float16)
+    else:
+        qt = torch.from_numpy(q)
+    case["q"] = qt.float().numpy()
+    case["q_bits"] = None
+    pl, lens = case["planes"], case["lens"]
+    out = ops.gqa_decode(qt.cuda(), upload(pl["k_codes"]), upload(pl["k_scales"]), upload(pl["v_codes"]), upload(pl["v_scales"]),
+                         upload(case["tables"]), upload(lens), 16, 4, 128, case["block_tokens"], 0.09, int(lens.max()),
+                         kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"])
+    torch.cuda.synchronize()
+    want = oracle_gqa_decode(case, 0.09)
+    assert_attention_close(out.cpu().numpy(), want, f"q dtype {q_kind}")
