@@ -4,8 +4,9 @@
 // optional sliding window).  Replaces the per-(row, head) block attention the reference runs for this
 // case (src/backend/rocm/attention.rs:2232-2242 -> tensor/attention/source.hip:618-686).
 //
-// A workgroup (4 waves) owns one KV head and a tile of query rows; its 256 MFMA columns enumerate
-// (row, head-in-group) pairs, 64 per wave, so one K/V tile serves every query head of the group.
+// A workgroup (8 waves) owns one KV head and a tile of query rows; its 256 MFMA columns enumerate
+// (row, head-in-group) pairs, 32 per wave, so one K/V tile serves every query head of the group.
+// Two waves share a SIMD, so the LDS and MFMA latencies of one are covered by the other.
 // Per 32-token step the workgroup converts the K and V codes ONCE into LDS as bf16 integers (exact)
 // with their f32 group scales beside them; each wave then runs
 //   S^T[token, col]  = sum_g k_scale[token, g] * (Kcodes_g[token, :] . Q_g[col, :])   (MFMA, exact products)
@@ -25,7 +26,9 @@ constexpr int kStep = 32;                 // tokens per step
 constexpr int kD = 128;                   // head_dim handled by this kernel
 constexpr int kRowBytes = kD * 2;         // one token of one KV head as bf16
 constexpr int kTileBytes = kStep * kRowBytes; // 8 KiB
-constexpr int kColTiles = 4;              // 16-column MFMA tiles per wave
+constexpr int kColTiles = 2;              // 16-column MFMA tiles per wave
+constexpr int kWaves = 256 / (16 * kColTiles);
+constexpr int kThreads = 64 * kWaves;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -55,12 +58,12 @@ __device__ __forceinline__ float soft_tanh(float x)
 }
 
 struct StepRegs {
-    u32x4 k, v;            // 16 codes each
-    unsigned int ks, vs;   // two 16-bit scales each (groups 0, 1)
+    u32x4 codes;           // 16 codes of the thread's plane (K for threads 0..255, V for 256..511)
+    unsigned int scales;   // two 16-bit scales (groups 0, 1) of the token
 };
 
 template <int SDT>
-__global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
+__global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
     __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
     __shared__ __align__(16) unsigned char lds_v[2][kTileBytes];
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
     Frag qf[kColTiles][4];
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ++ct) {
-        const unsigned int col = wave * 64u + ct * 16u + m;
+        const unsigned int col = wave * (16u * kColTiles) + ct * 16u + m;
         const unsigned int r = row0 + col / p.group;
         col_row[ct] = r;
         col_head[ct] = kvh * p.group + col % p.group;
@@ -117,24 +120,29 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
     const unsigned int s_row = p.num_kv_heads * 4u; // two 16-bit scales per KV head
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const unsigned int last_token = t_end - 1u;
-    auto row_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned long long {
+    // The block-table entry of a staging thread's token is fetched one step before the data that needs
+    // it, so no step waits on a table -> data load chain.
+    auto entry_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned int {
         token = min(token, last_token);
-        if (p.table == nullptr) {
-            return token;
-        }
-        if (pow2) {
-            return ((unsigned long long)p.table[token >> p.block_shift] << p.block_shift) + (token & (p.block_tokens - 1u));
-        }
-        return (unsigned long long)p.table[token / p.block_tokens] * p.block_tokens + token % p.block_tokens;
+        const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+        return p.table != nullptr ? p.table[page] : page;
     };
-    const unsigned int st_token = tid >> 3; // staging: token of the step, 16-code chunk cc
+    auto row_from = [&](unsigned int token, unsigned int entry) __attribute__((always_inline)) -> unsigned long long {
+        token = min(token, last_token);
+        if (pow2) {
+            return ((unsigned long long)entry << p.block_shift) + (token & (p.block_tokens - 1u));
+        }
+        return (unsigned long long)entry * p.block_tokens + token % p.block_tokens;
+    };
+    const bool stage_v = tid >= 256u;          // threads 0..255 stage K, 256..511 stage V
+    const unsigned int st_token = (tid & 255u) >> 3; // staging: token of the step, 16-code chunk cc
     const unsigned int cc = tid & 7u;
-    auto load_step = [&](StepRegs& r, unsigned int t0) __attribute__((always_inline)) {
-        const unsigned long long row = row_of(t0 + st_token);
-        r.k = *(const u32x4*)(p.k_plane + row * k_row + kvh * kD + cc * 16u);
-        r.v = *(const u32x4*)(p.v_plane + row * k_row + kvh * kD + cc * 16u);
-        r.ks = *(const unsigned int*)(p.k_scales + row * s_row + kvh * 4u);
-        r.vs = *(const unsigned int*)(p.v_scales + row * s_row + kvh * 4u);
+    const unsigned char* st_codes = (stage_v ? p.v_plane : p.k_plane) + kvh * kD + cc * 16u;
+    const unsigned char* st_scales = (stage_v ? p.v_scales : p.k_scales) + kvh * 4u;
+    auto load_step = [&](StepRegs& r, unsigned int t0, unsigned int entry) __attribute__((always_inline)) {
+        const unsigned long long row = row_from(t0 + st_token, entry);
+        r.codes = *(const u32x4*)(st_codes + row * k_row);
+        r.scales = *(const unsigned int*)(st_scales + row * s_row);
     };
     auto convert16 = [&](const u32x4& codes, u32x4& lo, u32x4& hi) __attribute__((always_inline)) {
         unsigned int out[8];
@@ -153,17 +161,14 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
     };
     auto store_step = [&](const StepRegs& r, int buf) __attribute__((always_inline)) {
         u32x4 lo, hi;
-        convert16(r.k, lo, hi);
-        *(u32x4*)(lds_k[buf] + tile_offset(st_token, cc * 2u)) = lo;
-        *(u32x4*)(lds_k[buf] + tile_offset(st_token, cc * 2u + 1u)) = hi;
-        convert16(r.v, lo, hi);
-        *(u32x4*)(lds_v[buf] + tile_offset(st_token, cc * 2u)) = lo;
-        *(u32x4*)(lds_v[buf] + tile_offset(st_token, cc * 2u + 1u)) = hi;
+        convert16(r.codes, lo, hi);
+        unsigned char* tile = stage_v ? lds_v[buf] : lds_k[buf];
+        *(u32x4*)(tile + tile_offset(st_token, cc * 2u)) = lo;
+        *(u32x4*)(tile + tile_offset(st_token, cc * 2u + 1u)) = hi;
         if (cc == 0) {
-            lds_ks[buf][0][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.ks & 0xffffu));
-            lds_ks[buf][1][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.ks >> 16));
-            lds_vs[buf][0][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.vs & 0xffffu));
-            lds_vs[buf][1][st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.vs >> 16));
+            float* dst = stage_v ? &lds_vs[buf][0][0] : &lds_ks[buf][0][0];
+            dst[st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales & 0xffffu));
+            dst[kStep + st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales >> 16));
         }
     };
 
@@ -253,9 +258,11 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
             }
             run_sum[ct] = run_sum[ct] * alpha[ct] + step_sum;
             run_max[ct] = new_max;
+            if (__any(alpha[ct] != 1.0f)) { // the running max settles early in a long prefix
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                acc[ct][t] *= alpha[ct];
+                for (int t = 0; t < 8; ++t) {
+                    acc[ct][t] *= alpha[ct];
+                }
             }
         }
         // ---- O^T += Vcodes^T . P'_g ----------------------------------------------------------------------
@@ -300,13 +307,16 @@ __global__ __launch_bounds__(256) void gqa_prefill_q8(GqaPrefillParams p)
     };
 
     StepRegs regs;
-    load_step(regs, t_begin);
+    load_step(regs, t_begin, entry_of(t_begin + st_token));
+    unsigned int entry_next = entry_of(t_begin + kStep + st_token);
     store_step(regs, 0);
     __syncthreads();
     for (unsigned int step = 0; step < steps; ++step) {
         const bool more = step + 1 < steps;
         if (more) {
-            load_step(regs, t_begin + (step + 1u) * kStep);
+            const unsigned int t_next = t_begin + (step + 1u) * kStep;
+            load_step(regs, t_next, entry_next);
+            entry_next = entry_of(t_next + kStep + st_token);
         }
         compute_step((int)(step & 1u), t_begin + step * kStep);
         if (more) {
@@ -358,9 +368,9 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
     if (scale_dtype == 0) {
-        gqa_prefill_q8<0><<<grid, dim3(256), 0, stream>>>(p);
+        gqa_prefill_q8<0><<<grid, dim3(kThreads), 0, stream>>>(p);
     } else {
-        gqa_prefill_q8<1><<<grid, dim3(256), 0, stream>>>(p);
+        gqa_prefill_q8<1><<<grid, dim3(kThreads), 0, stream>>>(p);
     }
     return hipGetLastError();
 }
