@@ -62,7 +62,7 @@ struct StepRegs {
     unsigned int scales;   // two 16-bit scales (groups 0, 1) of the token
 };
 
-template <int SDT>
+template <int SDT, bool SOFTCAP>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
     __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
@@ -116,6 +116,9 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         }
     }
 
+    const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
+    const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
+    const float cap_log2 = p.softcap * kLog2e;
     const unsigned int k_row = p.num_kv_heads * kD;
     const unsigned int s_row = p.num_kv_heads * 4u; // two 16-bit scales per KV head
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
@@ -166,9 +169,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         *(u32x4*)(tile + tile_offset(st_token, cc * 2u)) = lo;
         *(u32x4*)(tile + tile_offset(st_token, cc * 2u + 1u)) = hi;
         if (cc == 0) {
+            // K scales carry the score scale (and log2 e) so that the hot loop does not multiply again
             float* dst = stage_v ? &lds_vs[buf][0][0] : &lds_ks[buf][0][0];
-            dst[st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales & 0xffffu));
-            dst[kStep + st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales >> 16));
+            const float fold = stage_v ? 1.0f : scale_log2;
+            dst[st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales & 0xffffu)) * fold;
+            dst[kStep + st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales >> 16)) * fold;
         }
     };
 
@@ -190,7 +195,6 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         vis_hi[ct] = col_valid[ct] ? pos + 1u : 0u;
         vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
     }
-    const float scale_log2 = p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e;
 
     const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ swz(m)) << 4), m * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
     const unsigned int tr_row = 4u * j + (m >> 2);
@@ -236,14 +240,25 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         for (int ct = 0; ct < kColTiles; ++ct) {
             float sc[8];
             float step_max = kNegInf;
+            // only steps that touch a causal or window edge of some column need the per-token masks
+            const bool edge = __any(t0 + kStep > vis_hi[ct] || t0 < vis_lo[ct]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
-                float x = s[e >> 2][ct][e & 3] * scale_log2;
-                if (p.softcap > 0.0f) {
-                    x = p.softcap * soft_tanh(x / p.softcap) * kLog2e;
+                float x = s[e >> 2][ct][e & 3];
+                if constexpr (SOFTCAP) {
+                    x = cap_log2 * soft_tanh(x * inv_cap);
                 }
-                sc[e] = (token >= vis_lo[ct] && token < vis_hi[ct]) ? x : kNegInf;
+                sc[e] = x;
+            }
+            if (edge) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+                    sc[e] = (token >= vis_lo[ct] && token < vis_hi[ct]) ? sc[e] : kNegInf;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
                 step_max = fmaxf(step_max, sc[e]);
             }
             step_max = wave_max_16x4(step_max);
@@ -367,10 +382,19 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
     }
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
+    const bool cap = p.softcap > 0.0f;
     if (scale_dtype == 0) {
-        gqa_prefill_q8<0><<<grid, dim3(kThreads), 0, stream>>>(p);
+        if (cap) {
+            gqa_prefill_q8<0, true><<<grid, dim3(kThreads), 0, stream>>>(p);
+        } else {
+            gqa_prefill_q8<0, false><<<grid, dim3(kThreads), 0, stream>>>(p);
+        }
     } else {
-        gqa_prefill_q8<1><<<grid, dim3(kThreads), 0, stream>>>(p);
+        if (cap) {
+            gqa_prefill_q8<1, true><<<grid, dim3(kThreads), 0, stream>>>(p);
+        } else {
+            gqa_prefill_q8<1, false><<<grid, dim3(kThreads), 0, stream>>>(p);
+        }
     }
     return hipGetLastError();
 }
