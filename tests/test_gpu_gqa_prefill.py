@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
-             out_dtype=None, scale=None):
+             out_dtype=None, scale=None, outliers=False):
     from zllm_amd import capi, ops
 
     d = 128
@@ -22,8 +22,11 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     tables, pool_blocks = draw_tables(rng, [total], block_tokens)
     rows = pool_blocks * block_tokens
     sdt = O.SCALE_F16 if rule == O.RULE_METAL_GQA else O.SCALE_BF16
-    k = rng.standard_normal((total, cols)).astype(np.float32)
-    v = rng.standard_normal((total, cols)).astype(np.float32)
+    gain = np.ones(cols, dtype=np.float32)
+    if outliers:  # 1 % of the channels carry values eight times larger
+        gain[rng.choice(cols, size=max(1, cols // 100), replace=False)] = 8.0
+    k = rng.standard_normal((total, cols)).astype(np.float32) * gain
+    v = rng.standard_normal((total, cols)).astype(np.float32) * gain
     # the chunk's K/V arrive as bf16 activations
     k[prefix:] = O.bf16_to_f32(O.f32_to_bf16(k[prefix:]))
     v[prefix:] = O.bf16_to_f32(O.f32_to_bf16(v[prefix:]))
@@ -75,6 +78,15 @@ def test_prefill_config5_shape_at_oracle_size():
     3,000-token prefix and a 256-row chunk, which the CPU oracle finishes in seconds."""
     out, want = run_case(5, 3000, 256, 64, 8)
     print("config5-small", assert_attention_close(out.cpu().numpy(), want, "config 5 (small)"))
+
+
+@pytest.mark.parametrize("scale", [None, 1.0])
+def test_prefill_long_prefix_with_outlier_channels(scale):
+    """Far into a long prefix no single probability weighs much against the running sum and the kernel drops
+    the low-order half of P'; with score_scale 1.0 attention is peaked and it must keep it.  Outlier channels
+    make |v| large, which is where a lost low-order term would show against the absolute tolerance."""
+    out, want = run_case(90, 8000, 64, 16, 2, outliers=True, scale=scale)
+    print("long prefix", scale, assert_attention_close(out.cpu().numpy(), want, f"long prefix, scale={scale}"))
 
 
 @pytest.mark.parametrize("window", [1, 64, 500])

@@ -26,6 +26,7 @@ constexpr int kStep = 32;                 // tokens per step
 constexpr int kD = 128;                   // head_dim handled by this kernel
 constexpr int kRowBytes = kD * 2;         // one token of one KV head as bf16
 constexpr int kTileBytes = kStep * kRowBytes; // 8 KiB
+constexpr float kLoThreshold = 64.0f;       // see the P.V stage
 constexpr int kColTiles = 2;              // 16-column MFMA tiles per wave
 constexpr int kWaves = 256 / (16 * kColTiles);
 constexpr int kThreads = 64 * kWaves;
@@ -236,6 +237,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         // ---- online softmax per column --------------------------------------------------------------
         float pr[kColTiles][8];
         float alpha[kColTiles];
+        bool heavy = false; // some probability of this step is not small against the sum so far
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ++ct) {
             float sc[8];
@@ -273,6 +275,9 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             }
             run_sum[ct] = run_sum[ct] * alpha[ct] + step_sum;
             run_max[ct] = new_max;
+            const float p_top = fmaxf(fmaxf(fmaxf(pr[ct][0], pr[ct][1]), fmaxf(pr[ct][2], pr[ct][3])),
+                                      fmaxf(fmaxf(pr[ct][4], pr[ct][5]), fmaxf(pr[ct][6], pr[ct][7])));
+            heavy = heavy || p_top * kLoThreshold > run_sum[ct];
             if (__any(alpha[ct] != 1.0f)) { // the running max settles early in a long prefix
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
@@ -281,6 +286,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             }
         }
         // ---- O^T += Vcodes^T . P'_g ----------------------------------------------------------------------
+        // P' is carried as bf16 hi + lo (16 significant bits) while any probability of the step weighs more
+        // than 1/64 of its lane's running sum (a lane sums a quarter of the tokens, so < 1/256 of the row's);
+        // below that the hi term's rounding (2^-9 relative, random
+        // sign) moves the normalised output by < 2^-9 / 16 of |v|, so the lo product is skipped.
+        const bool lo_pass = __any(heavy);
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             const f32x4 gs0 = *(const f32x4*)(&lds_vs[buf][g][4 * j]);
@@ -292,10 +302,20 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                 for (int e = 0; e < 4; ++e) {
                     const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
                     const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
-                    unsigned int hi, lo;
-                    split_bf16_pair(x0, x1, hi, lo);
-                    phi[ct].u[e] = hi;
-                    plo[ct].u[e] = lo;
+                    phi[ct].u[e] = pack_bf16_hw(x0, x1);
+                }
+            }
+            if (lo_pass) {
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ++ct) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
+                        const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
+                        unsigned int hi, lo;
+                        split_bf16_pair(x0, x1, hi, lo);
+                        plo[ct].u[e] = lo;
+                    }
                 }
             }
 #pragma unroll
@@ -312,10 +332,13 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                 vf.s[1] = hi;
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
-                    f32x4 d = acc[ct][t];
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi[ct].b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo[ct].b, d, 0, 0, 0);
-                    acc[ct][t] = d;
+                    acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi[ct].b, acc[ct][t], 0, 0, 0);
+                }
+                if (lo_pass) {
+#pragma unroll
+                    for (int ct = 0; ct < kColTiles; ++ct) {
+                        acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo[ct].b, acc[ct][t], 0, 0, 0);
+                    }
                 }
             }
         }
