@@ -102,15 +102,19 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 //   NDH = 2: eight waves; the two waves of a head tile split the score work by token tile and exchange
 //            16 x 16 score tiles through LDS (two barriers per step).
 constexpr int kItemsMax = 4;
-struct StepRegs {
-    u32x4 codes[kItemsMax];          // items x 16 int8 codes
-    unsigned short scale[kItemsMax]; // bf16 scale of each item's group
-    u32x4 rope;                      // 8 bf16 rope values (threads 0..255)
+constexpr int kRawCodes = kStepTokens * kLatent;        // 16 KiB  [token][512] int8
+constexpr int kRawRope = kStepTokens * kRope * 2;       //  4 KiB  [token][64] bf16
+constexpr int kRawScales = kStepTokens * (kLatent / 64) * 2; // 512 B [token][8] bf16
+
+// Block-table entries of a thread's staging items: fetched one step before the loads that use them, so
+// nothing waits on a table -> data chain.  Slot ITEMS belongs to the rope role (threads 0..255) or the
+// scale role (threads 256..287).
+struct StepRows {
+    unsigned int entry[kItemsMax + 1];
 };
 
-struct StepRows {
-    unsigned long long row[kItemsMax + 1];
-};
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
 template <int NDH>
 __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
@@ -119,15 +123,21 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
     constexpr int TROWS = 8 * NDH;      // token rows covered by one pass of the threads
     constexpr int MT = 32 / NDH;        // output M tiles (16 latent columns each) of this wave
     constexpr int GROUPS = 8 / NDH;     // scale groups among them
-    constexpr int TILES = 2 / NDH;      // token tiles this wave scores itself
+    constexpr int TILES = NDH == 1 ? 2 : 1; // token tiles this wave scores itself
+    constexpr int KSPLIT = NDH == 4 ? 2 : 1; // waves that share one token tile's dot products (by column half)
+    constexpr int QF = 18 / KSPLIT;          // query k-steps held by this wave
     __shared__ __align__(16) unsigned char lds[2 * kTileBytes];
     __shared__ __align__(16) float lds_scale[2][8][kStepTokens]; // [buffer][group][token]
-    __shared__ __align__(16) float lds_s[NDH == 2 ? 4 : 1][2][16][16]; // [head tile][token tile][token][head]
+    // raw bytes of the next step, written by global -> LDS loads (no registers held across the MFMA work)
+    __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
+    __shared__ __align__(16) float lds_s[NDH >= 2 ? 4 : 1][2][KSPLIT][16][16]; // [head tile][token tile][column half][token][head]
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
     const unsigned int hw = wave / NDH;
     const unsigned int dh = wave % NDH;
+    const unsigned int ti = NDH == 4 ? dh >> 1 : dh; // token tile this wave scores (NDH >= 2)
+    const unsigned int kh = NDH == 4 ? dh & 1u : 0u; // column half of the dot products it computes
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     const unsigned int chunk = blockIdx.x;
@@ -150,83 +160,84 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
 
     // ---- Q fragments (B operand): lane = (head column m, k-slice j); k-step ks covers dims
     //      ks*32 + j*8 .. +8 of the 576-wide absorbed query ------------------------------------
-    Frag qf[18];
+    // With KSPLIT = 2 a wave keeps the k-steps of its column half only: latent groups 4 kh .. 4 kh + 3
+    // (k-steps 8 kh .. 8 kh + 7) in qf[0..7] and rope k-step 16 + kh in qf[8].
+    Frag qf[QF];
     {
         const unsigned short* qa = p.absorbed + ((size_t)b * p.heads + min(head, p.heads - 1u)) * kRowElems;
 #pragma unroll
-        for (int ks = 0; ks < 18; ++ks) {
+        for (int q = 0; q < QF; ++q) {
+            const unsigned int ks = KSPLIT == 1 ? (unsigned int)q : (q < 8 ? 8u * kh + q : 16u + kh);
             u32x4 v = *(const u32x4*)(qa + ks * 32 + j * 8);
             if (head >= p.heads) {
                 v = u32x4{0u, 0u, 0u, 0u};
             }
-            qf[ks].u = v;
+            qf[q].u = v;
         }
     }
 
     const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
-    // cooperative staging: item i of a thread = token (tid >> 5) + TROWS * i, 16-code chunk cc = tid & 31;
-    // threads 0..255 also move one rope item: token tid >> 3, 8-value chunk tid & 7
+    // Cooperative staging, in two halves.
+    //   issue_step:   every thread starts global -> LDS loads of its raw items of the NEXT step: item i = 16 codes
+    //                 of token (tid >> 5) + TROWS * i, chunk cc = tid & 31; threads 0..255 also one 16-byte rope
+    //                 chunk (token tid >> 3); threads 256..287 the eight scales of token tid - 256.
+    //   convert_step: after the MFMA work each thread waits for ITS OWN loads (issued a whole step earlier),
+    //                 reads its raw items back and writes them into the bf16 tile / f32 scale table.
+    // A thread only ever reads raw bytes it loaded itself, so no barrier sits between the two halves.
+    const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const unsigned int cc = tid & 31u;
     const unsigned int t_lo = tid >> 5;
     const unsigned int rope_t = (tid >> 3) & 31u;
     const unsigned int rope_c = tid & 7u;
     const bool has_rope = tid < 256u;
-    // physical rows of the thread's tokens of a step: the table loads are issued together, one step ahead
-    // of the data loads that use them
+    const bool has_scales = tid >= 256u && tid < 256u + kStepTokens;
+    const unsigned int extra_t = has_rope ? rope_t : (tid - 256u) & 31u; // token of the rope / scale item
+    unsigned char* const raw_codes = lds_raw;
+    unsigned char* const raw_rope = lds_raw + kRawCodes;
+    unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
     auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
-        unsigned int token[ITEMS + 1];
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            token[i] = min(t0 + t_lo + TROWS * i, len - 1u);
-        }
-        token[ITEMS] = min(t0 + rope_t, len - 1u);
-        if (table == nullptr) {
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                r.row[i] = token[i];
-            }
-        } else if (pow2) {
-            unsigned int entry[ITEMS + 1];
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                entry[i] = table[token[i] >> p.block_shift];
-            }
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                r.row[i] = ((unsigned long long)entry[i] << p.block_shift) + (token[i] & (p.block_tokens - 1u));
-            }
-        } else {
-            unsigned int entry[ITEMS + 1];
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                entry[i] = table[token[i] / p.block_tokens];
-            }
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                r.row[i] = (unsigned long long)entry[i] * p.block_tokens + token[i] % p.block_tokens;
-            }
+        for (int i = 0; i <= ITEMS; ++i) {
+            const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+            const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+            r.entry[i] = table != nullptr ? table[page] : page;
         }
     };
-    auto load_step = [&](StepRegs& r, const StepRows& rows) __attribute__((always_inline)) {
+    auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
+        const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+        if (pow2) {
+            return ((unsigned long long)r.entry[i] << p.block_shift) + (token & (p.block_tokens - 1u));
+        }
+        return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
+    };
+    auto issue_step = [&](const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-            r.codes[i] = *(const u32x4*)(p.latent_codes + rows.row[i] * kLatent + cc * 16u);
-            r.scale[i] = p.latent_scales[rows.row[i] * (kLatent / 64) + (cc >> 2)];
+            // the wave's 64 lanes cover token rows 2 * wave and 2 * wave + 1 (+ TROWS * i): 1 KiB, contiguous in LDS
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
+                                             (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
         }
-        if (has_rope) {
-            r.rope = *(const u32x4*)(p.rope_cache + rows.row[ITEMS] * kRope + rope_c * 8u);
+        if (has_rope) { // waves 0..3: token rows 8 * wave .. + 8 of the rope plane, 128 B each
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
+                                             (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+        }
+        if (has_scales) { // wave 4, lanes 0..31: the 16 bytes of scales of one token each
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
+                                             (lds_ptr_t)(raw_scales), 16, 0, 0);
         }
     };
-    auto store_step = [&](const StepRegs& r, unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
+    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's raw items have landed
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
             const unsigned int row = t_lo + TROWS * i;
+            const u32x4 codes = *(const u32x4*)(raw_codes + row * kLatent + cc * 16u);
             u32x4 out[2];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const unsigned int word = r.codes[i][w];
+                const unsigned int word = codes[w];
                 const float c0 = (float)(int)(signed char)(word & 0xffu);
                 const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
                 const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
@@ -236,13 +247,19 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
             }
             *(u32x4*)(tile + tile_offset(row, cc * 2u)) = out[0];
             *(u32x4*)(tile + tile_offset(row, cc * 2u + 1u)) = out[1];
-            if ((cc & 3u) == 0) {
-                scale_tile[cc >> 2][row] = bf16_bits_to_f32(r.scale[i]);
-            }
         }
         if (has_rope) {
-            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = r.rope;
+            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = *(const u32x4*)(raw_rope + tid * 16u);
         }
+        if (has_scales) {
+            const u32x4 sc8 = *(const u32x4*)(raw_scales + (tid - 256u) * 16u);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const unsigned int word = sc8[g >> 1];
+                scale_tile[g][tid - 256u] = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // raw bytes are in registers before the next loads overwrite them
     };
 
     f32x4 acc[MT];
@@ -255,7 +272,7 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
 
     // LDS byte offsets of this lane's fragments, split into a lane part and a compile-time part so
     // that every read is `base + immediate`:  chunk = (hi << 3) | lo, and only `lo` meets the swizzle.
-    const unsigned int qk_row = (NDH == 2 ? dh * 16u : 0u) + m;
+    const unsigned int qk_row = (NDH >= 2 ? ti * 16u : 0u) + m;
     const unsigned int qk_base[2] = {qk_row * kRowBytes + ((j ^ swz(m)) << 4), qk_row * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
     const unsigned int tr_row = 4u * j + (m >> 2);
     unsigned int pv_base[4];
@@ -270,36 +287,41 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
         float sc[8];
 #pragma unroll
         for (int i = 0; i < TILES; ++i) {
-            const unsigned int tile_i = NDH == 2 ? dh : (unsigned int)i;          // token tile scored here
-            const unsigned char* kt = tile + (NDH == 2 ? 0 : i * 16 * kRowBytes); // qk_base already holds dh
+            const unsigned int tile_i = NDH >= 2 ? ti : (unsigned int)i;          // token tile scored here
+            const unsigned char* kt = tile + (NDH >= 2 ? 0 : i * 16 * kRowBytes); // qk_base already holds ti
             f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (KSPLIT == 1) {
 #pragma unroll
-            for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
-                Frag kf;
-                kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
-                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
+                for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
+                    Frag kf;
+                    kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
+                }
+            } else {
+                Frag kf; // rope k-step 16 + kh
+                kf.u = *(const u32x4*)(kt + (kh == 0 ? qk_base[0] : qk_base[1]) + 8 * 128);
+                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[8].b, s, 0, 0, 0);
             }
 #pragma unroll
-            for (int half = 0; half < 2; ++half) { // four independent accumulators at a time: no MFMA -> MFMA stalls
+            for (int half = 0; half < 2 / KSPLIT; ++half) { // four independent accumulators at a time: no MFMA -> MFMA stalls
                 f32x4 d[4];
+                const unsigned int g0 = KSPLIT == 1 ? half * 4u : kh * 4u; // first scale group of this batch
+                const int q0 = KSPLIT == 1 ? half * 8 : 0;                 // its first query k-step
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int g = half * 4 + u;
                     Frag k0;
-                    k0.u = *(const u32x4*)(kt + qk_base[0] + g * 128);
-                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    k0.u = *(const u32x4*)(kt + qk_base[0] + (g0 + u) * 128);
+                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[q0 + 2 * u].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int g = half * 4 + u;
                     Frag k1;
-                    k1.u = *(const u32x4*)(kt + qk_base[1] + g * 128);
-                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                    k1.u = *(const u32x4*)(kt + qk_base[1] + (g0 + u) * 128);
+                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[q0 + 2 * u + 1].b, d[u], 0, 0, 0);
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int g = half * 4 + u;
-                    const f32x4 gs = *(const f32x4*)(&scale_tile[g][tile_i * 16 + 4 * j]); // one address per 16-lane group
+                    const f32x4 gs = *(const f32x4*)(&scale_tile[g0 + u][tile_i * 16 + 4 * j]); // one address per 16-lane group
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         s[r] = fmaf(d[u][r], gs[r], s[r]);
@@ -308,28 +330,32 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const unsigned int token = t0 + 16u * tile_i + 4u * j + r;
-                const float x = token < len ? s[r] * scale_log2 : kNegInf;
-                if constexpr (NDH == 2) {
-                    sc[r] = x; // staged below
+                if constexpr (NDH >= 2) {
+                    sc[r] = s[r]; // partial or whole dot of (token 16 ti + 4 j + r, head m): exchanged below
                 } else {
-                    sc[i * 4 + r] = x;
+                    const unsigned int token = t0 + 16u * tile_i + 4u * j + r;
+                    sc[i * 4 + r] = token < len ? s[r] * scale_log2 : kNegInf;
                 }
             }
         }
-        if constexpr (NDH == 2) {
-            float mine[4];
+        if constexpr (NDH >= 2) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                mine[r] = sc[r];
-                lds_s[hw][dh][4 * j + r][m] = mine[r];
+                lds_s[hw][ti][kh][4 * j + r][m] = sc[r];
             }
             __syncthreads();
+            // every wave of the head tile rebuilds the same 32 scores in the same order
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float other = lds_s[hw][dh ^ 1u][4 * j + r][m];
-                sc[dh * 4 + r] = mine[r];
-                sc[(dh ^ 1u) * 4 + r] = other;
+            for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float x = lds_s[hw][t2][0][4 * j + r][m];
+                    if constexpr (KSPLIT == 2) {
+                        x += lds_s[hw][t2][1][4 * j + r][m];
+                    }
+                    const unsigned int token = t0 + 16u * t2 + 4u * j + r;
+                    sc[t2 * 4 + r] = token < len ? x * scale_log2 : kNegInf;
+                }
             }
         }
         // ---- online softmax for this head column ---------------------------------------------------------
@@ -393,31 +419,31 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
 
     // ---- pipeline: table lookups run two steps ahead, global loads one step ahead of the MFMA work;
     //      LDS tile double-buffered ---------------------------------------------------------------------
-    StepRegs regs;
     StepRows rows;
     lookup_step(rows, c_start);
-    load_step(regs, rows);
+    issue_step(rows, c_start);
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    store_step(regs, lds, lds_scale[0]);
+    convert_step(lds, lds_scale[0]);
     __syncthreads();
     for (unsigned int step = 0; step < steps; ++step) {
         unsigned char* cur = lds + (step & 1u) * kTileBytes;
         unsigned char* nxt = lds + ((step + 1u) & 1u) * kTileBytes;
         const bool more = step + 1 < steps;
         if (more) {
-            load_step(regs, rows);
+            issue_step(rows, c_start + (step + 1u) * kStepTokens);
             if (step + 2 < steps) {
                 lookup_step(rows, c_start + (step + 2u) * kStepTokens);
             }
         }
         compute_step(cur, lds_scale[step & 1u], c_start + step * kStepTokens);
         if (more) {
-            store_step(regs, nxt, lds_scale[(step + 1u) & 1u]);
+            convert_step(nxt, lds_scale[(step + 1u) & 1u]);
         }
         __syncthreads();
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no load may still target this workgroup's LDS at exit
 
     // ---- write un-normalised partials and (max, sum) -------------------------------------------
     const float total = wave_sum_16x4(run_sum);
