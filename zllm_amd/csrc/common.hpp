@@ -119,19 +119,31 @@ __device__ __forceinline__ void split_bf16_pair(float x0, float x1, unsigned int
     lo = pack_bf16_hw(x0 - h0, x1 - h1);
 }
 
+// Reductions across the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48): every lane ends up with
+// the result.  v_permlane16_swap / v_permlane32_swap exchange rows inside the vector ALU, so the reduction
+// does not take the round trip through the LDS crossbar that a generic lane shuffle does.
+typedef unsigned int u32x2_swap __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float wave_max_16x4(float v)
 {
-    // reduce across the four 16-lane groups of a wave (lanes l, l^16, l^32, l^48)
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+    const unsigned int bits = __float_as_uint(v);
+    // swap odd rows of the first copy with even rows of the second: {r0, r0, r2, r2} and {r1, r1, r3, r3}
+    const u32x2_swap a = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const float m = fmaxf(__uint_as_float(a.x), __uint_as_float(a.y));
+    const unsigned int mbits = __float_as_uint(m);
+    // swap the upper half of the first copy with the lower half of the second
+    const u32x2_swap b = __builtin_amdgcn_permlane32_swap(mbits, mbits, false, false);
+    return fmaxf(__uint_as_float(b.x), __uint_as_float(b.y));
 }
 
 __device__ __forceinline__ float wave_sum_16x4(float v)
 {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    const unsigned int bits = __float_as_uint(v);
+    const u32x2_swap a = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const float s = __uint_as_float(a.x) + __uint_as_float(a.y);
+    const unsigned int sbits = __float_as_uint(s);
+    const u32x2_swap b = __builtin_amdgcn_permlane32_swap(sbits, sbits, false, false);
+    return __uint_as_float(b.x) + __uint_as_float(b.y);
 }
 
 } // namespace zllm

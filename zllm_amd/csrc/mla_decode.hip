@@ -101,6 +101,14 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 //            registers leave room to keep many LDS fragment loads in flight; one barrier per step.
 //   NDH = 2: eight waves; the two waves of a head tile split the score work by token tile and exchange
 //            16 x 16 score tiles through LDS (two barriers per step).
+// Workgroup barrier for LDS traffic only.  __syncthreads() also fences the global -> LDS loads in flight
+// (s_waitcnt vmcnt(0)), which would drain the prefetch of the next step at every barrier; the data those
+// loads bring is consumed by the issuing thread alone, after its own explicit wait.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 constexpr int kItemsMax = 4;
 constexpr int kRawCodes = kStepTokens * kLatent;        // 16 KiB  [token][512] int8
 constexpr int kRawRope = kStepTokens * kRope * 2;       //  4 KiB  [token][64] bf16
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
             for (int r = 0; r < 4; ++r) {
                 lds_s[hw][ti][kh][4 * j + r][m] = sc[r];
             }
-            __syncthreads();
+            lds_barrier();
             // every wave of the head tile rebuilds the same 32 scores in the same order
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
@@ -426,7 +434,7 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
         lookup_step(rows, c_start + kStepTokens);
     }
     convert_step(lds, lds_scale[0]);
-    __syncthreads();
+    lds_barrier();
     for (unsigned int step = 0; step < steps; ++step) {
         unsigned char* cur = lds + (step & 1u) * kTileBytes;
         unsigned char* nxt = lds + ((step + 1u) & 1u) * kTileBytes;
@@ -441,7 +449,7 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
         if (more) {
             convert_step(nxt, lds_scale[(step + 1u) & 1u]);
         }
-        __syncthreads();
+        lds_barrier();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no load may still target this workgroup's LDS at exit
 
