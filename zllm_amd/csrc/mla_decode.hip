@@ -471,28 +471,53 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
 // ---------------------------------------------------------------------------------------------
 // 4. project value
 // ---------------------------------------------------------------------------------------------
-// grid = (heads, batch), 256 threads = 4 waves; each wave produces value columns v = wave, wave+4, ...
-// with a 64-lane dot over the 512 latent columns.
+// grid = (heads, batch), 256 threads = 4 waves.  A wave works on eight value columns at a time: lane =
+// (column v0 + lane / 8, slice lane % 8 of 64 latent columns); the lane keeps its 64 weighted values in
+// registers, reads its 64 weights as eight 16-byte vectors, and the eight slices are summed with DPP row
+// shifts.  The weight rows of a head are read exactly once, as whole 128-byte lines.
 __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int wave = threadIdx.x >> 6;
-    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * p.latent_dim;
-    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * p.latent_dim;
+    const unsigned int slice = lane & 7u;
+    const unsigned int sub = lane >> 3;
+    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * kLatent + slice * 64u;
+    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 64u;
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     const size_t out_base = ((size_t)b * p.heads + head) * out_stride;
-    for (unsigned int v = wave; v < p.value_dim; v += 4) {
-        float sum = 0.0f;
-        for (unsigned int c = lane; c < p.latent_dim; c += 64) {
-            sum = fmaf(weighted[c], bf16_bits_to_f32(w[(size_t)v * p.latent_dim + c]), sum);
-        }
+    float x[64];
 #pragma unroll
-        for (int offset = 32; offset > 0; offset >>= 1) {
-            sum += __shfl_xor(sum, offset);
+    for (int i = 0; i < 16; ++i) {
+        const f32x4 t = *(const f32x4*)(weighted + 4 * i);
+        x[4 * i] = t[0];
+        x[4 * i + 1] = t[1];
+        x[4 * i + 2] = t[2];
+        x[4 * i + 3] = t[3];
+    }
+    for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
+        const unsigned int v = v0 + sub;
+        const unsigned int vr = min(v, p.value_dim - 1u);
+        u32x4 raw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 8 * i);
         }
-        if (lane == 0) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                sum = fmaf(x[8 * i + 2 * e], __uint_as_float(raw[i][e] << 16), sum);
+                sum = fmaf(x[8 * i + 2 * e + 1], __uint_as_float(raw[i][e] & 0xffff0000u), sum);
+            }
+        }
+        // sum the eight slices of a column: lanes 8 sub .. 8 sub + 7 sit in one 16-lane row
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x114, 0xf, 0xf, true)); // row_shr:4
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x112, 0xf, 0xf, true)); // row_shr:2
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x111, 0xf, 0xf, true)); // row_shr:1
+        if (slice == 7u && v < p.value_dim) {
             if (p.out_dtype == 0) {
                 ((float*)p.out)[out_base + v] = sum;
             } else {
