@@ -1,0 +1,277 @@
+// Parity of the C++ host layer (zllm_amd/host/rocm_backend.hpp) with the CPU oracle, written the way the
+// reference tests its backends: build inputs, call the trait method, compare with the CPU reference
+// (src/backend/mod.rs tests around gqa_prefill_attention_cached; tolerance of the attention path:
+// max-abs 2e-3, relative 1e-2).  Run by tests/test_gpu_host_backend.py on a GPU box.
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../zllm_amd/host/rocm_backend.hpp"
+
+extern "C" {
+// oracle/zllm_oracle.c (test infrastructure)
+uint16_t zo_f32_to_bf16(float value);
+float zo_bf16_to_f32(uint16_t value);
+int zo_q8g64_append_paged(int rule, const float* input, int8_t* codes, void* scales, const uint32_t* block_table, uint64_t position,
+                          uint64_t rows, uint64_t cols, uint64_t group, uint32_t block_size, uint64_t ring_capacity);
+int zo_half_append_paged(int dtype, const float* input, uint16_t* cache, const uint32_t* block_table, uint64_t position, uint64_t rows,
+                         uint64_t cols, uint32_t block_size, uint64_t ring_capacity);
+int zo_gather_dequant_rows(int format, const void* plane, const void* scales, int scale_dtype, const uint32_t* block_table,
+                           uint32_t block_size, uint64_t ring_capacity, uint64_t first, uint64_t count, uint64_t cols, uint64_t group,
+                           float* out);
+int zo_gather_rows_bytes(const uint8_t* plane, const uint32_t* block_table, uint32_t block_size, uint64_t ring_capacity, uint64_t first,
+                         uint64_t count, uint64_t row_bytes, uint8_t* out);
+int zo_gqa_prefill_at_visible_f32(const float* query, const float* key, const float* value, uint64_t query_tokens, uint64_t kv_start,
+                                  uint64_t kv_end, uint64_t position, uint64_t num_heads, uint64_t num_kv_heads, uint64_t head_dim,
+                                  uint64_t window, float score_scale, float softcap, const uint32_t* visible_ends, float* output);
+int zo_rope_apply_f32(float* data, uint64_t rows, uint64_t columns, uint64_t head_count, uint64_t rotary_dim, uint64_t position,
+                      const float* cosine, const float* sine, uint64_t table_len, int layout, int placement);
+typedef struct {
+    uint64_t kv_lora_rank, qk_rope_head_dim, q_projection_size, kv_projection_size, num_heads;
+} zo_mla_spec;
+int zo_mla_absorbed_q8_history(const zo_mla_spec* spec, const uint16_t* query, uint64_t query_rows, uint64_t query_start,
+                               const uint8_t* latent_codes, const uint16_t* latent_scales, uint64_t latent_group_size, const uint16_t* rope,
+                               uint64_t history_rows, const float* kv_b, const uint32_t* selection, uint64_t width, uint16_t* out_bf16,
+                               float* out_f32, float* weighted_f32);
+}
+
+using namespace zllm_amd;
+
+static int failures = 0;
+
+#define CHECK(cond, ...)                          \
+    do {                                          \
+        if (!(cond)) {                            \
+            printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+            printf(__VA_ARGS__);                  \
+            printf("\n");                         \
+            ++failures;                           \
+        }                                         \
+    } while (0)
+
+static std::vector<float> randn(std::mt19937& rng, size_t n, bool bf16_round)
+{
+    std::normal_distribution<float> dist(0.0f, 1.0f);
+    std::vector<float> out(n);
+    for (auto& x : out) {
+        x = dist(rng);
+        if (bf16_round) {
+            x = zo_bf16_to_f32(zo_f32_to_bf16(x));
+        }
+    }
+    return out;
+}
+
+static void compare(const std::vector<float>& got, const std::vector<float>& want, const char* what)
+{
+    CHECK(got.size() == want.size(), "%s: size %zu vs %zu", what, got.size(), want.size());
+    double max_abs = 0, num = 0, den = 0;
+    for (size_t i = 0; i < got.size() && i < want.size(); ++i) {
+        const double d = (double)got[i] - want[i];
+        max_abs = fmax(max_abs, fabs(d));
+        num += d * d;
+        den += (double)want[i] * want[i];
+        if (!isfinite(got[i])) {
+            max_abs = INFINITY;
+        }
+    }
+    const double rel = den > 0 ? sqrt(num / den) : sqrt(num);
+    printf("%-58s max-abs %.3e rel %.3e\n", what, max_abs, rel);
+    CHECK(max_abs <= 2e-3, "%s: max-abs %.3e > 2e-3", what, max_abs);
+    CHECK(rel <= 1e-2, "%s: relative %.3e > 1e-2", what, rel);
+}
+
+// ---------------------------------------------------------------------------------------------- GQA
+static void test_gqa(const RocmContext& ctx, CausalWindow window, const char* label)
+{
+    std::mt19937 rng(7);
+    GqaSpec spec;
+    spec.num_heads = 16;
+    spec.num_kv_heads = 4;
+    spec.head_dim = 128;
+    spec.window = window;
+    spec.score_scale = 1.0f / sqrtf(128.0f);
+    const size_t kv_cols = spec.num_kv_heads * spec.head_dim, q_cols = spec.num_heads * spec.head_dim;
+    const size_t block = 16, max_tokens = 1024;
+    auto cache_r = RocmKvCache::new_gqa(2, spec.num_kv_heads, spec.head_dim, block, max_tokens);
+    CHECK(cache_r.is_ok(), "cache: %s", cache_r.is_err() ? cache_r.unwrap_err().to_string().c_str() : "");
+    if (cache_r.is_err()) {
+        return;
+    }
+    RocmKvCache cache = cache_r.unwrap();
+    const size_t pool_rows = cache.block_table().size() * block;
+    // the oracle's copy of layer 1's planes, filled by the oracle's quantizer through the same table
+    std::vector<int8_t> k_codes(pool_rows * kv_cols), v_codes(pool_rows * kv_cols);
+    std::vector<uint16_t> k_scales(pool_rows * kv_cols / 64), v_scales(pool_rows * kv_cols / 64);
+    const size_t layer = 1;
+    size_t position = 0;
+    const size_t chunks[] = {300, 200, 1, 1, 37, 1};
+    for (size_t rows : chunks) {
+        const auto q = randn(rng, rows * q_cols, true);
+        const auto k = randn(rng, rows * kv_cols, false);
+        const auto v = randn(rng, rows * kv_cols, false);
+        auto qt = ctx.tensor_from_f32(q, rows, q_cols, DType::BF16);
+        auto kt = ctx.tensor_from_f32(k, rows, kv_cols);
+        auto vt = ctx.tensor_from_f32(v, rows, kv_cols);
+        CHECK(qt.is_ok() && kt.is_ok() && vt.is_ok(), "upload");
+        auto out = ctx.gqa_prefill_attention_cached(cache, layer, position, qt.unwrap(), kt.unwrap(), vt.unwrap(), spec, true);
+        CHECK(out.is_ok(), "%s rows=%zu: %s", label, rows, out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_err()) {
+            return;
+        }
+        auto got = ctx.tensor_to_f32(out.unwrap());
+        CHECK(got.is_ok(), "download");
+        zo_q8g64_append_paged(1, k.data(), k_codes.data(), k_scales.data(), cache.block_table().data(), position, rows, kv_cols, 64, block, 0);
+        zo_q8g64_append_paged(1, v.data(), v_codes.data(), v_scales.data(), cache.block_table().data(), position, rows, kv_cols, 64, block, 0);
+        const size_t total = position + rows;
+        std::vector<float> kd(total * kv_cols), vd(total * kv_cols), want(rows * q_cols);
+        zo_gather_dequant_rows(0, k_codes.data(), k_scales.data(), 1, cache.block_table().data(), block, 0, 0, total, kv_cols, 64, kd.data());
+        zo_gather_dequant_rows(0, v_codes.data(), v_scales.data(), 1, cache.block_table().data(), block, 0, 0, total, kv_cols, 64, vd.data());
+        const int rc = zo_gqa_prefill_at_visible_f32(q.data(), kd.data(), vd.data(), rows, 0, total, position, spec.num_heads, spec.num_kv_heads,
+                                                     spec.head_dim, window.sliding ? window.size : 0, spec.score_scale, 0.0f, nullptr, want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        char what[128];
+        snprintf(what, sizeof(what), "gqa_prefill_attention_cached %s position=%zu rows=%zu", label, position, rows);
+        compare(got.unwrap(), want, what);
+        position = total;
+        CHECK(cache.len(layer) == position, "cache length %zu vs %zu", cache.len(layer), position);
+    }
+    // error behaviour of the reference's body (attention.rs:2213-2229)
+    {
+        const auto q = randn(rng, q_cols, true);
+        const auto k = randn(rng, kv_cols, false);
+        auto qt = ctx.tensor_from_f32(q, 1, q_cols);
+        auto kt = ctx.tensor_from_f32(k, 1, kv_cols);
+        auto stale = ctx.gqa_prefill_attention_cached(cache, layer, position - 1, qt.unwrap(), kt.unwrap(), kt.unwrap(), spec, true);
+        CHECK(stale.is_err() && stale.unwrap_err().kind == BackendError::Kind::Compute, "a stale position must be a Compute error");
+        auto wrong = ctx.gqa_prefill_attention_cached(cache, layer, position, qt.unwrap(), qt.unwrap(), kt.unwrap(), spec, true);
+        CHECK(wrong.is_err() && wrong.unwrap_err().msg.find("shape") != std::string::npos, "a K of the wrong width must be a shape error");
+        auto missing = ctx.gqa_prefill_attention_cached(cache, 9, position, qt.unwrap(), kt.unwrap(), kt.unwrap(), spec, true);
+        CHECK(missing.is_err() && missing.unwrap_err().kind == BackendError::Kind::UnsupportedLayer && missing.unwrap_err().layer == 9,
+              "a layer outside the cache must be UnsupportedLayer");
+        CHECK(cache.len(layer) == position, "failed calls must not move the cache length");
+    }
+}
+
+// ---------------------------------------------------------------------------------------------- MLA
+static void test_mla(const RocmContext& ctx)
+{
+    std::mt19937 rng(11);
+    MlaSpec spec;
+    spec.kv_lora_rank = 512;
+    spec.qk_rope_head_dim = 64;
+    spec.num_heads = 16;
+    spec.q_projection_size = spec.num_heads * 192;  // nope 128 + rope 64
+    spec.kv_projection_size = spec.num_heads * 256; // nope 128 + value 128
+    spec.q_lora_rank = 1536;
+    CHECK(!spec.validate().has_value(), "spec must validate");
+    const size_t block = 64, max_tokens = 700, layer = 0;
+    auto cache_r = RocmKvCache::new_mla(1, 512, 64, block, max_tokens);
+    CHECK(cache_r.is_ok(), "cache");
+    if (cache_r.is_err()) {
+        return;
+    }
+    RocmKvCache cache = cache_r.unwrap();
+    const size_t pool_rows = cache.block_table().size() * block;
+    std::vector<int8_t> ref_codes(pool_rows * 512);
+    std::vector<uint16_t> ref_scales(pool_rows * 8), ref_rope(pool_rows * 64);
+    // rotary tables for 1,024 positions
+    const size_t rotary_dim = 64, half = rotary_dim / 2, table_rows = 1024;
+    std::vector<float> cos(table_rows * half), sin(table_rows * half);
+    for (size_t pos = 0; pos < table_rows; ++pos) {
+        for (size_t i = 0; i < half; ++i) {
+            const float angle = (float)pos * powf(10000.0f, -2.0f * (float)i / (float)rotary_dim);
+            cos[pos * half + i] = cosf(angle);
+            sin[pos * half + i] = sinf(angle);
+        }
+    }
+    // a bulk append of rows whose rope is already rotated, then single-row appends with the rotation fused
+    const size_t bulk = 555, singles = 3;
+    {
+        const auto latent = randn(rng, bulk * 512, false);
+        const auto rope = randn(rng, bulk * 64, false);
+        auto lt = ctx.tensor_from_f32(latent, bulk, 512);
+        auto rt = ctx.tensor_from_f32(rope, bulk, 64);
+        auto done = ctx.append_mla(cache, layer, lt.unwrap(), rt.unwrap());
+        CHECK(done.is_ok(), "append_mla: %s", done.is_err() ? done.unwrap_err().to_string().c_str() : "");
+        zo_q8g64_append_paged(0, latent.data(), ref_codes.data(), ref_scales.data(), cache.block_table().data(), 0, bulk, 512, 64, block, 0);
+        zo_half_append_paged(0, rope.data(), ref_rope.data(), cache.block_table().data(), 0, bulk, 64, block, 0);
+    }
+    for (size_t s = 0; s < singles; ++s) {
+        const size_t position = bulk + s;
+        const auto latent = randn(rng, 512, false);
+        auto rope = randn(rng, 64, false);
+        auto lt = ctx.tensor_from_f32(latent, 1, 512);
+        auto rt = ctx.tensor_from_f32(rope, 1, 64);
+        auto done = ctx.append_mla_rope(cache, layer, lt.unwrap(), rt.unwrap(), rotary_dim, RotaryLayout::SplitHalf, position, cos, sin);
+        CHECK(done.is_ok(), "append_mla_rope: %s", done.is_err() ? done.unwrap_err().to_string().c_str() : "");
+        zo_rope_apply_f32(rope.data(), 1, 64, 1, rotary_dim, position, cos.data(), sin.data(), cos.size(), 0, 1);
+        zo_q8g64_append_paged(0, latent.data(), ref_codes.data(), ref_scales.data(), cache.block_table().data(), position, 1, 512, 64, block, 0);
+        zo_half_append_paged(0, rope.data(), ref_rope.data(), cache.block_table().data(), position, 1, 64, block, 0);
+    }
+    const size_t ctx_len = bulk + singles;
+    CHECK(cache.len(layer) == ctx_len, "cache length %zu", cache.len(layer));
+
+    const size_t q_cols = spec.q_projection_size;
+    const auto q = randn(rng, q_cols, true);
+    std::vector<float> kv_b = randn(rng, spec.kv_projection_size * 512, true);
+    for (auto& w : kv_b) {
+        w *= 0.05f;
+        w = zo_bf16_to_f32(zo_f32_to_bf16(w));
+    }
+    auto qt = ctx.tensor_from_f32(q, 1, q_cols, DType::BF16);
+    auto weight = ctx.prepare_mla_kv_b(kv_b, spec.kv_projection_size, 512);
+    CHECK(qt.is_ok() && weight.is_ok(), "upload");
+    auto out = ctx.mla_decode_attention(qt.unwrap(), cache, weight.unwrap(), layer, ctx_len - 1, spec);
+    CHECK(out.is_ok(), "mla_decode_attention: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+    if (out.is_err()) {
+        return;
+    }
+    auto got = ctx.tensor_to_f32(out.unwrap());
+
+    // oracle on the dense history gathered from ITS planes (the device planes are bit-identical: tests/test_gpu_append.py)
+    std::vector<uint8_t> codes_dense(ctx_len * 512);
+    std::vector<uint16_t> scales_dense(ctx_len * 8), rope_dense(ctx_len * 64), q_bits(q_cols);
+    zo_gather_rows_bytes((const uint8_t*)ref_codes.data(), cache.block_table().data(), block, 0, 0, ctx_len, 512, codes_dense.data());
+    zo_gather_rows_bytes((const uint8_t*)ref_scales.data(), cache.block_table().data(), block, 0, 0, ctx_len, 16, (uint8_t*)scales_dense.data());
+    zo_gather_rows_bytes((const uint8_t*)ref_rope.data(), cache.block_table().data(), block, 0, 0, ctx_len, 128, (uint8_t*)rope_dense.data());
+    for (size_t i = 0; i < q_cols; ++i) {
+        q_bits[i] = zo_f32_to_bf16(q[i]);
+    }
+    zo_mla_spec zs = {512, 64, spec.q_projection_size, spec.kv_projection_size, spec.num_heads};
+    std::vector<float> want(spec.num_heads * spec.value_dim());
+    const int rc = zo_mla_absorbed_q8_history(&zs, q_bits.data(), 1, ctx_len - 1, codes_dense.data(), scales_dense.data(), 64, rope_dense.data(),
+                                              ctx_len, kv_b.data(), nullptr, 0, nullptr, want.data(), nullptr);
+    CHECK(rc == 0, "oracle rc %d", rc);
+    compare(got.unwrap(), want, "mla_decode_attention after append_mla + append_mla_rope");
+
+    auto stale = ctx.mla_decode_attention(qt.unwrap(), cache, weight.unwrap(), layer, ctx_len + 5, spec);
+    CHECK(stale.is_err(), "a position beyond the cache must be an error");
+    MlaSpec bad = spec;
+    bad.q_projection_size += 1;
+    CHECK(bad.validate().has_value(), "inconsistent head dimensions must not validate");
+}
+
+int main()
+{
+    auto ctx = RocmContext::create(0);
+    if (ctx.is_err()) {
+        printf("FAIL context: %s\n", ctx.unwrap_err().to_string().c_str());
+        return 2;
+    }
+    // CausalWindow known answers of the reference's tests (src/attention/gqa.rs:290-330)
+    CHECK(CausalWindow::Full().key_range(5, 10) == std::make_pair((size_t)0, (size_t)6), "full window");
+    CHECK(CausalWindow::Sliding(4).key_range(9, 10) == std::make_pair((size_t)6, (size_t)10), "sliding window");
+    CHECK(CausalWindow::Sliding(4).key_range(1, 10) == std::make_pair((size_t)0, (size_t)2), "sliding window, short history");
+    CHECK(CausalWindow::Sliding(1024).cache_capacity(8192) == 1024 && CausalWindow::Full().cache_capacity(8192) == 8192, "cache capacity");
+    test_gqa(ctx.unwrap(), CausalWindow::Full(), "full");
+    test_gqa(ctx.unwrap(), CausalWindow::Sliding(128), "sliding(128)");
+    test_mla(ctx.unwrap());
+    printf(failures == 0 ? "ALL PASSED\n" : "%d FAILED\n", failures);
+    return failures == 0 ? 0 : 1;
+}

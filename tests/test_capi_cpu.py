@@ -101,3 +101,17 @@ def test_invalid_shapes_are_reported_without_a_gpu(lib):
     assert b"null pointer" in lib.zllm_attn_last_error()
     q8 = capi.Q8AppendArgs()
     assert lib.zllm_attn_q8g64_append(C.byref(q8), None) == -1
+
+
+def test_cpp_host_layer_builds_and_exports_the_backend_methods():
+    """The C++ mirror of the reference's backend traits (zllm_amd/host) is a shared library next to the C ABI."""
+    import os
+    import subprocess
+
+    lib = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "zllm_amd", "libzllm_backend.so")
+    assert os.path.exists(lib), "run __graft_entry__.build()"
+    names = subprocess.run(["nm", "-DC", "--defined-only", lib], capture_output=True, text=True, check=True).stdout
+    for method in ("zllm_amd::RocmContext::gqa_prefill_attention_cached", "zllm_amd::RocmContext::append_mla(",
+                   "zllm_amd::RocmContext::append_mla_rope", "zllm_amd::RocmContext::mla_decode_attention",
+                   "zllm_amd::CausalWindow::key_range", "zllm_amd::RocmKvCache::new_gqa", "zllm_amd::RocmKvCache::new_mla"):
+        assert method in names, method

@@ -1,0 +1,21 @@
+"""Runs the C++ host layer's parity driver (tests/host/backend_parity.cpp): the reference-shaped backend methods
+(gqa_prefill_attention_cached, append_mla, append_mla_rope, mla_decode_attention) over the C ABI, compared with the
+CPU oracle inside the driver, plus their error behaviour.  The binary is built by __graft_entry__.build()."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BINARY = os.path.join(ROOT, "tests", "host", "backend_parity")
+
+
+def test_cpp_backend_mirror_matches_oracle():
+    assert os.path.exists(BINARY), f"{BINARY} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`"
+    done = subprocess.run([BINARY], capture_output=True, text=True, timeout=110)
+    print(done.stdout)
+    print(done.stderr)
+    assert done.returncode == 0, done.stdout[-2000:] + done.stderr[-2000:]
+    assert "ALL PASSED" in done.stdout

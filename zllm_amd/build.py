@@ -46,5 +46,26 @@ def build_library(jobs: int = 4) -> str:
     return LIB
 
 
+BACKEND_LIB = os.path.join(HERE, "libzllm_backend.so")
+HOST_TEST = os.path.join(os.path.dirname(HERE), "tests", "host", "backend_parity")
+
+
+def build_host_layer() -> str:
+    """The C++ host layer above the C ABI (zllm_amd/host) as libzllm_backend.so; needs libzllm_attn.so."""
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared", "-o", BACKEND_LIB,
+           os.path.join(HERE, "host", "rocm_backend.cpp"), "-L" + HERE, "-lzllm_attn", "-Wl,-rpath,$ORIGIN"]
+    subprocess.check_call(cmd)
+    return BACKEND_LIB
+
+
+def build_host_test(oracle_dir: str) -> str:
+    """tests/host/backend_parity: the host layer's parity driver; links the CPU oracle (checker only)."""
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-o", HOST_TEST, HOST_TEST + ".cpp", "-L" + HERE, "-lzllm_backend",
+           "-lzllm_attn", "-L" + oracle_dir, "-lzllm_oracle", "-Wl,-rpath,$ORIGIN/../../zllm_amd", "-Wl,-rpath,$ORIGIN/../../oracle"]
+    subprocess.check_call(cmd)
+    return HOST_TEST
+
+
 if __name__ == "__main__":
     print(build_library())
+    print(build_host_layer())

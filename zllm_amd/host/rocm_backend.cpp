@@ -1,0 +1,656 @@
+// Implementation of the host-side backend mirror over the C ABI.  Device memory comes from hipMalloc here
+// (the C ABI itself never allocates); every attention call runs on the context's stream.
+#include "rocm_backend.hpp"
+
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <numeric>
+
+#include "../../include/zllm_attn.h"
+
+namespace zllm_amd {
+
+namespace {
+
+BackendError compute_error(std::string msg)
+{
+    BackendError e;
+    e.kind = BackendError::Kind::Compute;
+    e.msg = std::move(msg);
+    return e;
+}
+
+BackendError hip_error(const char* what, hipError_t err)
+{
+    return compute_error(std::string(what) + ": " + hipGetErrorString(err));
+}
+
+BackendError abi_error(const char* what, int code)
+{
+    return compute_error(std::string(what) + ": " + zllm_attn_last_error() + " (code " + std::to_string(code) + ")");
+}
+
+uint16_t f32_to_bf16_bits(float value)
+{
+    uint32_t bits;
+    memcpy(&bits, &value, 4);
+    const uint32_t rounding = 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)((bits + rounding) >> 16);
+}
+
+float bf16_bits_to_f32(uint16_t v)
+{
+    const uint32_t bits = (uint32_t)v << 16;
+    float out;
+    memcpy(&out, &bits, 4);
+    return out;
+}
+
+// IEEE binary16 <-> binary32 (round to nearest even), for host-side tensor conversion only
+uint16_t f32_to_f16_bits(float value)
+{
+    const _Float16 h = (_Float16)value;
+    uint16_t out;
+    memcpy(&out, &h, 2);
+    return out;
+}
+
+float f16_bits_to_f32(uint16_t v)
+{
+    _Float16 h;
+    memcpy(&h, &v, 2);
+    return (float)h;
+}
+
+int abi_dtype(DType dtype)
+{
+    return dtype == DType::F32 ? ZLLM_DTYPE_F32 : dtype == DType::BF16 ? ZLLM_DTYPE_BF16 : ZLLM_DTYPE_F16;
+}
+
+} // namespace
+
+std::string BackendError::to_string() const
+{
+    switch (kind) {
+    case Kind::UnsupportedLayer: return "unsupported model layer L" + std::to_string(layer);
+    case Kind::ExpertLoad: return "expert load failed: " + msg;
+    default: return "backend compute failed: " + msg;
+    }
+}
+
+std::pair<size_t, size_t> CausalWindow::key_range(size_t query_position, size_t key_end) const
+{
+    const size_t end = std::min(query_position + 1, key_end);
+    size_t start = 0;
+    if (sliding) {
+        start = query_position + 1 > size ? query_position + 1 - size : 0;
+    }
+    return {std::min(start, end), end};
+}
+
+size_t CausalWindow::cache_capacity(size_t max_sequence_len) const
+{
+    return sliding ? std::min(size, max_sequence_len) : max_sequence_len;
+}
+
+std::optional<std::string> MlaSpec::validate() const
+{
+    if (num_heads == 0 || q_projection_size % num_heads != 0 || kv_projection_size % num_heads != 0) {
+        return "MLA head dimensions invalid: q_proj=" + std::to_string(q_projection_size) + " kv_proj=" + std::to_string(kv_projection_size) +
+               " heads=" + std::to_string(num_heads);
+    }
+    if (qk_rope_head_dim > 0 && (qk_rope_head_dim % 2 != 0 || !isfinite(rope_theta) || rope_theta <= 0.0f)) {
+        return "MLA RoPE parameters invalid: rope_dim=" + std::to_string(qk_rope_head_dim);
+    }
+    if (qk_rope_head_dim > q_head_dim()) {
+        return "MLA rope dim " + std::to_string(qk_rope_head_dim) + " exceeds query head dim " + std::to_string(q_head_dim());
+    }
+    if (qk_nope_dim() > kv_head_dim()) {
+        return "MLA nope dim " + std::to_string(qk_nope_dim()) + " exceeds KV head dim " + std::to_string(kv_head_dim());
+    }
+    return std::nullopt;
+}
+
+size_t dtype_bytes(DType dtype)
+{
+    return dtype == DType::F32 ? 4 : 2;
+}
+
+Result<DeviceBuffer> DeviceBuffer::allocate(size_t bytes)
+{
+    void* raw = nullptr;
+    const hipError_t err = hipMalloc(&raw, std::max<size_t>(bytes, 256));
+    if (err != hipSuccess) {
+        return hip_error("hipMalloc", err);
+    }
+    DeviceBuffer out;
+    out.ptr_ = std::shared_ptr<void>(raw, [](void* p) { (void)hipFree(p); });
+    out.bytes_ = bytes;
+    return out;
+}
+
+// ------------------------------------------------------------------------------------------------ cache
+namespace {
+
+// Pages are handed out in a fixed scrambled order so that the block table is never the identity.
+std::vector<uint32_t> scrambled_pages(size_t pages)
+{
+    std::vector<uint32_t> ids(pages);
+    std::iota(ids.begin(), ids.end(), 0u);
+    uint64_t state = 0x9e3779b97f4a7c15ull;
+    for (size_t i = pages; i > 1; --i) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        std::swap(ids[i - 1], ids[(size_t)((state >> 33) % i)]);
+    }
+    return ids;
+}
+
+} // namespace
+
+Result<RocmKvCache> RocmKvCache::new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens)
+{
+    const size_t cols = num_kv_heads * head_dim;
+    if (layers == 0 || cols == 0 || cols % 64 != 0 || block_tokens == 0 || max_tokens == 0) {
+        return compute_error("Rocm GQA cache: invalid geometry");
+    }
+    RocmKvCache cache;
+    cache.cols_ = cols;
+    cache.block_tokens_ = block_tokens;
+    cache.max_tokens_ = max_tokens;
+    const size_t pages = (max_tokens + block_tokens - 1) / block_tokens;
+    cache.pool_rows_ = pages * block_tokens;
+    cache.table_host_ = scrambled_pages(pages);
+    auto table = DeviceBuffer::allocate(pages * 4);
+    if (table.is_err()) {
+        return table.unwrap_err();
+    }
+    cache.table_ = table.unwrap();
+    hipError_t err = hipMemcpy(cache.table_.data(), cache.table_host_.data(), pages * 4, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        return hip_error("block table upload", err);
+    }
+    for (size_t l = 0; l < layers; ++l) {
+        Layer layer;
+        DeviceBuffer* planes[4] = {&layer.a_codes, &layer.a_scales, &layer.b_codes, &layer.b_scales};
+        const size_t bytes[4] = {cache.pool_rows_ * cols, cache.pool_rows_ * (cols / 64) * 2, cache.pool_rows_ * cols,
+                                 cache.pool_rows_ * (cols / 64) * 2};
+        for (int i = 0; i < 4; ++i) {
+            auto buf = DeviceBuffer::allocate(bytes[i]);
+            if (buf.is_err()) {
+                return buf.unwrap_err();
+            }
+            *planes[i] = buf.unwrap();
+            err = hipMemset(planes[i]->data(), 0, bytes[i]);
+            if (err != hipSuccess) {
+                return hip_error("cache clear", err);
+            }
+        }
+        cache.layers_.push_back(layer);
+        cache.lens_.push_back(0);
+    }
+    return cache;
+}
+
+Result<RocmKvCache> RocmKvCache::new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens)
+{
+    if (layers == 0 || latent_dim == 0 || latent_dim % 64 != 0 || rope_dim == 0 || block_tokens == 0 || max_tokens == 0) {
+        return compute_error("Rocm MLA cache: invalid geometry");
+    }
+    RocmKvCache cache;
+    cache.mla_ = true;
+    cache.cols_ = latent_dim;
+    cache.rope_cols_ = rope_dim;
+    cache.block_tokens_ = block_tokens;
+    cache.max_tokens_ = max_tokens;
+    const size_t pages = (max_tokens + block_tokens - 1) / block_tokens;
+    cache.pool_rows_ = pages * block_tokens;
+    cache.table_host_ = scrambled_pages(pages);
+    auto table = DeviceBuffer::allocate(pages * 4);
+    if (table.is_err()) {
+        return table.unwrap_err();
+    }
+    cache.table_ = table.unwrap();
+    hipError_t err = hipMemcpy(cache.table_.data(), cache.table_host_.data(), pages * 4, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        return hip_error("block table upload", err);
+    }
+    for (size_t l = 0; l < layers; ++l) {
+        Layer layer;
+        DeviceBuffer* planes[3] = {&layer.a_codes, &layer.a_scales, &layer.b_codes};
+        const size_t bytes[3] = {cache.pool_rows_ * latent_dim, cache.pool_rows_ * (latent_dim / 64) * 2, cache.pool_rows_ * rope_dim * 2};
+        for (int i = 0; i < 3; ++i) {
+            auto buf = DeviceBuffer::allocate(bytes[i]);
+            if (buf.is_err()) {
+                return buf.unwrap_err();
+            }
+            *planes[i] = buf.unwrap();
+            err = hipMemset(planes[i]->data(), 0, bytes[i]);
+            if (err != hipSuccess) {
+                return hip_error("cache clear", err);
+            }
+        }
+        cache.layers_.push_back(layer);
+        cache.lens_.push_back(0);
+    }
+    return cache;
+}
+
+// ---------------------------------------------------------------------------------------------- context
+Result<RocmContext> RocmContext::create(int device_id)
+{
+    int cus = 0;
+    const int rc = zllm_attn_init(device_id, &cus);
+    if (rc != 0) {
+        return abi_error("zllm_attn_init", rc);
+    }
+    RocmContext ctx;
+    ctx.device_id_ = device_id;
+    hipError_t err = hipSetDevice(device_id);
+    if (err == hipSuccess) {
+        err = hipStreamCreate(&ctx.stream_); // default priority
+    }
+    if (err != hipSuccess) {
+        return hip_error("stream", err);
+    }
+    return ctx;
+}
+
+Result<Unit> RocmContext::synchronize() const
+{
+    const hipError_t err = hipStreamSynchronize(stream_);
+    if (err != hipSuccess) {
+        return hip_error("hipStreamSynchronize", err);
+    }
+    return Unit{};
+}
+
+Result<RocmTensor> RocmContext::tensor_from_f32(const std::vector<float>& host, size_t rows, size_t cols, DType dtype) const
+{
+    if (host.size() != rows * cols) {
+        return compute_error("tensor_from_f32: data length does not match rows x cols");
+    }
+    auto buf = DeviceBuffer::allocate(rows * cols * dtype_bytes(dtype));
+    if (buf.is_err()) {
+        return buf.unwrap_err();
+    }
+    RocmTensor t;
+    t.device = buf.unwrap();
+    t.rows = rows;
+    t.cols = cols;
+    t.dtype = dtype;
+    hipError_t err;
+    if (dtype == DType::F32) {
+        err = hipMemcpy(t.device.data(), host.data(), host.size() * 4, hipMemcpyHostToDevice);
+    } else {
+        std::vector<uint16_t> half(host.size());
+        for (size_t i = 0; i < host.size(); ++i) {
+            half[i] = dtype == DType::BF16 ? f32_to_bf16_bits(host[i]) : f32_to_f16_bits(host[i]);
+        }
+        err = hipMemcpy(t.device.data(), half.data(), half.size() * 2, hipMemcpyHostToDevice);
+    }
+    if (err != hipSuccess) {
+        return hip_error("tensor upload", err);
+    }
+    return t;
+}
+
+Result<std::vector<float>> RocmContext::tensor_to_f32(const RocmTensor& tensor) const
+{
+    hipError_t err = hipStreamSynchronize(stream_);
+    if (err != hipSuccess) {
+        return hip_error("hipStreamSynchronize", err);
+    }
+    const size_t n = tensor.rows * tensor.cols;
+    std::vector<float> out(n);
+    if (tensor.dtype == DType::F32) {
+        err = hipMemcpy(out.data(), tensor.device.data(), n * 4, hipMemcpyDeviceToHost);
+    } else {
+        std::vector<uint16_t> half(n);
+        err = hipMemcpy(half.data(), tensor.device.data(), n * 2, hipMemcpyDeviceToHost);
+        for (size_t i = 0; i < n; ++i) {
+            out[i] = tensor.dtype == DType::BF16 ? bf16_bits_to_f32(half[i]) : f16_bits_to_f32(half[i]);
+        }
+    }
+    if (err != hipSuccess) {
+        return hip_error("tensor download", err);
+    }
+    return out;
+}
+
+Result<RocmWeight> RocmContext::prepare_mla_kv_b(const std::vector<float>& weight, size_t rows, size_t cols) const
+{
+    auto t = tensor_from_f32(weight, rows, cols, DType::BF16);
+    if (t.is_err()) {
+        return t.unwrap_err();
+    }
+    RocmWeight w;
+    w.device = t.unwrap().device;
+    w.rows = rows;
+    w.cols = cols;
+    return w;
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
+                                                             const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                             bool retain_full_cache) const
+{
+    (void)retain_full_cache;
+    if (spec.num_heads == 0 || spec.num_kv_heads == 0 || spec.head_dim == 0 || spec.num_heads % spec.num_kv_heads != 0) {
+        return compute_error("Rocm GQA spec invalid");
+    }
+    const size_t query_cols = spec.num_heads * spec.head_dim;
+    const size_t kv_cols = spec.num_kv_heads * spec.head_dim;
+    if (query.rows != key.rows || query.rows != value.rows || query.cols != query_cols || key.cols != kv_cols || value.cols != kv_cols) {
+        return compute_error("Rocm GQA cached prefill shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
+                             std::to_string(key.rows) + "," + std::to_string(key.cols) + "] V=[" + std::to_string(value.rows) + "," +
+                             std::to_string(value.cols) + "]");
+    }
+    if (cache.mla_ || layer >= cache.layers_.size() || cache.cols_ != kv_cols) {
+        BackendError e;
+        e.kind = BackendError::Kind::UnsupportedLayer;
+        e.layer = layer;
+        return e;
+    }
+    if (query.rows == 0) {
+        return compute_error("Rocm GQA cached prefill: empty chunk");
+    }
+    // position must be the current cache length (src/backend/rocm/attention.rs:2226-2229)
+    if (cache.lens_[layer] != position) {
+        return compute_error("Rocm GQA L" + std::to_string(layer) + " device cache incomplete: rows=" + std::to_string(cache.lens_[layer]) + "/" +
+                             std::to_string(position));
+    }
+    const size_t total = position + query.rows;
+    if (total > cache.max_tokens_ || total > UINT32_MAX) {
+        return compute_error("Rocm GQA cache position overflow");
+    }
+    RocmKvCache::Layer& planes = cache.layers_[layer];
+    // quantizing append of the chunk's K and V rows (no f32 staging copies)
+    const RocmTensor* sources[2] = {&key, &value};
+    void* codes[2] = {planes.a_codes.data(), planes.b_codes.data()};
+    void* scales[2] = {planes.a_scales.data(), planes.b_scales.data()};
+    for (int i = 0; i < 2; ++i) {
+        zllm_q8_append_args a;
+        memset(&a, 0, sizeof(a));
+        a.src = sources[i]->device.data();
+        a.codes = (int8_t*)codes[i];
+        a.scales = scales[i];
+        a.table = (const uint32_t*)cache.table_.data();
+        a.position = (uint32_t)position;
+        a.rows = (uint32_t)query.rows;
+        a.cols = (uint32_t)kv_cols;
+        a.block_tokens = (uint32_t)cache.block_tokens_;
+        a.src_dtype = abi_dtype(sources[i]->dtype);
+        a.rule = ZLLM_QUANT_METAL_GQA;
+        const int rc = zllm_attn_q8g64_append(&a, stream_);
+        if (rc != 0) {
+            return abi_error("zllm_attn_q8g64_append", rc);
+        }
+    }
+    cache.lens_[layer] = total;
+
+    auto out_buf = DeviceBuffer::allocate(query.rows * query_cols * 4);
+    if (out_buf.is_err()) {
+        return out_buf.unwrap_err();
+    }
+    RocmTensor out;
+    out.device = out_buf.unwrap();
+    out.rows = query.rows;
+    out.cols = query_cols;
+    out.dtype = DType::F32;
+    const size_t table_stride = cache.table_host_.size();
+
+    if (query.rows == 1) {
+        const auto range = spec.window.key_range(position, total);
+        const uint32_t host_meta[2] = {(uint32_t)total, (uint32_t)range.first};
+        auto meta = DeviceBuffer::allocate(8);
+        if (meta.is_err()) {
+            return meta.unwrap_err();
+        }
+        hipError_t err = hipMemcpyAsync(meta.unwrap().data(), host_meta, 8, hipMemcpyHostToDevice, stream_);
+        if (err != hipSuccess) {
+            return hip_error("decode metadata upload", err);
+        }
+        err = hipStreamSynchronize(stream_); // host_meta is a stack array
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+        zllm_gqa_decode_args a;
+        memset(&a, 0, sizeof(a));
+        a.q = query.device.data();
+        a.k_plane = planes.a_codes.data();
+        a.k_scales = planes.a_scales.data();
+        a.v_plane = planes.b_codes.data();
+        a.v_scales = planes.b_scales.data();
+        a.tables = (const uint32_t*)cache.table_.data();
+        a.kv_lens = (const uint32_t*)meta.unwrap().data();
+        a.first_visible = spec.window.sliding ? (const uint32_t*)meta.unwrap().data() + 1 : nullptr;
+        a.out = (float*)out.device.data();
+        a.batch = 1;
+        a.num_heads = (uint32_t)spec.num_heads;
+        a.num_kv_heads = (uint32_t)spec.num_kv_heads;
+        a.head_dim = (uint32_t)spec.head_dim;
+        a.table_stride = (uint32_t)table_stride;
+        a.max_kv_len = (uint32_t)total;
+        a.block_tokens = (uint32_t)cache.block_tokens_;
+        a.score_scale = spec.score_scale;
+        a.kv_format = ZLLM_KV_Q8G64;
+        a.scale_dtype = ZLLM_SCALE_F16;
+        a.q_dtype = abi_dtype(query.dtype);
+        const uint64_t need = zllm_attn_gqa_decode_workspace_bytes(&a);
+        if (need == 0) {
+            return abi_error("zllm_attn_gqa_decode_workspace_bytes", -1);
+        }
+        auto ws = DeviceBuffer::allocate(need);
+        if (ws.is_err()) {
+            return ws.unwrap_err();
+        }
+        a.workspace = ws.unwrap().data();
+        a.workspace_bytes = need;
+        const int rc = zllm_attn_gqa_decode(&a, stream_);
+        if (rc != 0) {
+            return abi_error("zllm_attn_gqa_decode", rc);
+        }
+        err = hipStreamSynchronize(stream_); // the workspace and metadata die with this scope
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+        return out;
+    }
+
+    zllm_gqa_prefill_args a;
+    memset(&a, 0, sizeof(a));
+    a.q = query.device.data();
+    a.k_plane = planes.a_codes.data();
+    a.k_scales = planes.a_scales.data();
+    a.v_plane = planes.b_codes.data();
+    a.v_scales = planes.b_scales.data();
+    a.table = (const uint32_t*)cache.table_.data();
+    a.out = out.device.data();
+    a.rows = (uint32_t)query.rows;
+    a.position = (uint32_t)position;
+    a.window = spec.window.sliding ? (uint32_t)spec.window.size : 0u;
+    a.num_heads = (uint32_t)spec.num_heads;
+    a.num_kv_heads = (uint32_t)spec.num_kv_heads;
+    a.head_dim = (uint32_t)spec.head_dim;
+    a.block_tokens = (uint32_t)cache.block_tokens_;
+    a.score_scale = spec.score_scale;
+    a.kv_format = ZLLM_KV_Q8G64;
+    a.scale_dtype = ZLLM_SCALE_F16;
+    a.q_dtype = abi_dtype(query.dtype);
+    a.out_dtype = ZLLM_DTYPE_F32;
+    const int rc = zllm_attn_gqa_prefill_chunk(&a, stream_);
+    if (rc != 0) {
+        return abi_error("zllm_attn_gqa_prefill_chunk", rc);
+    }
+    return out;
+}
+
+Result<Unit> RocmContext::append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
+                                          RotaryLayout layout, size_t position, const float* cos_dev, const float* sin_dev) const
+{
+    if (!cache.mla_ || layer >= cache.layers_.size()) {
+        BackendError e;
+        e.kind = BackendError::Kind::UnsupportedLayer;
+        e.layer = layer;
+        return e;
+    }
+    if (latent.rows != rope.rows || latent.cols != cache.cols_ || rope.cols != cache.rope_cols_ || latent.dtype != DType::F32 ||
+        rope.dtype != DType::F32) {
+        return compute_error("Rocm MLA append shape mismatch: latent=[" + std::to_string(latent.rows) + "," + std::to_string(latent.cols) + "] rope=[" +
+                             std::to_string(rope.rows) + "," + std::to_string(rope.cols) + "]");
+    }
+    const size_t at = cache.lens_[layer];
+    if (at + latent.rows > cache.max_tokens_) {
+        return compute_error("Rocm MLA cache is full");
+    }
+    RocmKvCache::Layer& planes = cache.layers_[layer];
+    zllm_mla_append_args a;
+    memset(&a, 0, sizeof(a));
+    a.latent = (const float*)latent.device.data();
+    a.k_rope = (const float*)rope.device.data();
+    a.cosine = cos_dev;
+    a.sine = sin_dev;
+    a.latent_codes = (int8_t*)planes.a_codes.data();
+    a.latent_scales = (uint16_t*)planes.a_scales.data();
+    a.rope_cache = (uint16_t*)planes.b_codes.data();
+    a.table = (const uint32_t*)cache.table_.data();
+    a.position = (uint32_t)at;
+    a.rope_position = (uint32_t)position;
+    a.rows = (uint32_t)latent.rows;
+    a.latent_cols = (uint32_t)cache.cols_;
+    a.rope_cols = (uint32_t)cache.rope_cols_;
+    a.rotary_dim = (uint32_t)rotary_dim;
+    a.rotary_layout = layout == RotaryLayout::SplitHalf ? ZLLM_ROTARY_SPLIT_HALF : ZLLM_ROTARY_INTERLEAVED;
+    a.block_tokens = (uint32_t)cache.block_tokens_;
+    const int rc = zllm_attn_mla_append(&a, stream_);
+    if (rc != 0) {
+        return abi_error("zllm_attn_mla_append", rc);
+    }
+    cache.lens_[layer] = at + latent.rows;
+    return Unit{};
+}
+
+Result<Unit> RocmContext::append_mla(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope) const
+{
+    return append_mla_impl(cache, layer, latent, rope, 0, RotaryLayout::SplitHalf, 0, nullptr, nullptr);
+}
+
+Result<Unit> RocmContext::append_mla_rope(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
+                                          RotaryLayout layout, size_t position, const std::vector<float>& cos, const std::vector<float>& sin) const
+{
+    const size_t half = rotary_dim / 2;
+    if (rotary_dim == 0 || rotary_dim % 2 != 0 || rotary_dim > rope.cols || cos.size() != sin.size() ||
+        cos.size() < (position + rope.rows) * half) {
+        return compute_error("Rocm MLA append: rotary tables do not cover position " + std::to_string(position));
+    }
+    auto tables = DeviceBuffer::allocate(cos.size() * 8);
+    if (tables.is_err()) {
+        return tables.unwrap_err();
+    }
+    float* cos_dev = (float*)tables.unwrap().data();
+    float* sin_dev = cos_dev + cos.size();
+    hipError_t err = hipMemcpy(cos_dev, cos.data(), cos.size() * 4, hipMemcpyHostToDevice);
+    if (err == hipSuccess) {
+        err = hipMemcpy(sin_dev, sin.data(), sin.size() * 4, hipMemcpyHostToDevice);
+    }
+    if (err != hipSuccess) {
+        return hip_error("rotary table upload", err);
+    }
+    auto done = append_mla_impl(cache, layer, latent, rope, rotary_dim, layout, position, cos_dev, sin_dev);
+    if (done.is_ok()) {
+        err = hipStreamSynchronize(stream_); // the tables die with this scope
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+    }
+    return done;
+}
+
+Result<RocmTensor> RocmContext::mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
+                                                     size_t position, const MlaSpec& spec) const
+{
+    if (auto bad = spec.validate()) {
+        return compute_error(*bad);
+    }
+    if (!cache.mla_ || layer >= cache.layers_.size()) {
+        BackendError e;
+        e.kind = BackendError::Kind::UnsupportedLayer;
+        e.layer = layer;
+        return e;
+    }
+    if (query.rows != 1 || query.cols != spec.q_projection_size || spec.kv_lora_rank != cache.cols_ || spec.qk_rope_head_dim != cache.rope_cols_ ||
+        kv_b.rows != spec.kv_projection_size || kv_b.cols != spec.kv_lora_rank) {
+        return compute_error("Rocm MLA decode shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] kv_b=[" +
+                             std::to_string(kv_b.rows) + "," + std::to_string(kv_b.cols) + "]");
+    }
+    const size_t ctx = cache.lens_[layer];
+    if (ctx == 0 || position + 1 != ctx) {
+        return compute_error("Rocm MLA L" + std::to_string(layer) + " cache length " + std::to_string(ctx) + " does not match position " +
+                             std::to_string(position));
+    }
+    const size_t out_cols = spec.num_heads * spec.value_dim();
+    auto out_buf = DeviceBuffer::allocate(out_cols * 4);
+    auto meta = DeviceBuffer::allocate(4);
+    if (out_buf.is_err()) {
+        return out_buf.unwrap_err();
+    }
+    if (meta.is_err()) {
+        return meta.unwrap_err();
+    }
+    const uint32_t ctx_u32 = (uint32_t)ctx;
+    hipError_t err = hipMemcpy(meta.unwrap().data(), &ctx_u32, 4, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        return hip_error("decode metadata upload", err);
+    }
+    const RocmKvCache::Layer& planes = cache.layers_[layer];
+    zllm_mla_decode_args a;
+    memset(&a, 0, sizeof(a));
+    a.q = query.device.data();
+    a.kv_b = (const uint16_t*)kv_b.device.data();
+    a.latent_codes = (const int8_t*)planes.a_codes.data();
+    a.latent_scales = (const uint16_t*)planes.a_scales.data();
+    a.rope_cache = (const uint16_t*)planes.b_codes.data();
+    a.tables = (const uint32_t*)cache.table_.data();
+    a.ctx_lens = (const uint32_t*)meta.unwrap().data();
+    a.out = out_buf.unwrap().data();
+    a.batch = 1;
+    a.heads = (uint32_t)spec.num_heads;
+    a.q_head_dim = (uint32_t)spec.q_head_dim();
+    a.kv_head_dim = (uint32_t)spec.kv_head_dim();
+    a.latent_dim = (uint32_t)spec.kv_lora_rank;
+    a.rope_dim = (uint32_t)spec.qk_rope_head_dim;
+    a.table_stride = (uint32_t)cache.table_host_.size();
+    a.max_ctx_len = ctx_u32;
+    a.block_tokens = (uint32_t)cache.block_tokens_;
+    a.q_dtype = abi_dtype(query.dtype);
+    a.out_dtype = ZLLM_DTYPE_F32; // decode rows are written as f32 (src/backend/rocm/attention.rs:17-19)
+    a.out_compact = 1;
+    const uint64_t need = zllm_attn_mla_decode_workspace_bytes(&a);
+    if (need == 0) {
+        return abi_error("zllm_attn_mla_decode_workspace_bytes", -1);
+    }
+    auto ws = DeviceBuffer::allocate(need);
+    if (ws.is_err()) {
+        return ws.unwrap_err();
+    }
+    a.workspace = ws.unwrap().data();
+    a.workspace_bytes = need;
+    const int rc = zllm_attn_mla_decode(&a, stream_);
+    if (rc != 0) {
+        return abi_error("zllm_attn_mla_decode", rc);
+    }
+    err = hipStreamSynchronize(stream_); // workspace and metadata die with this scope
+    if (err != hipSuccess) {
+        return hip_error("hipStreamSynchronize", err);
+    }
+    RocmTensor out;
+    out.device = out_buf.unwrap();
+    out.rows = 1;
+    out.cols = out_cols;
+    out.dtype = DType::F32;
+    return out;
+}
+
+} // namespace zllm_amd

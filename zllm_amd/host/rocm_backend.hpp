@@ -1,0 +1,175 @@
+// Host side of the attention path above the C ABI (include/zllm_attn.h), in C++ because the reference's
+// host side is compiled code (Rust) and no Rust toolchain exists here.  Names, argument meaning and error
+// behaviour follow the reference's backend traits for this path:
+//   GqaPrefillBackend::gqa_prefill_attention_cached   src/backend/mod.rs:1484-1494, ROCm body
+//                                                     src/backend/rocm/attention.rs:2202-2254
+//   DecodeBackend::{append_mla, append_mla_rope,
+//                   mla_decode_attention}             src/backend/mod.rs:1162-1180, attention.rs:1805-1832
+//   CausalWindow::{key_range, cache_capacity}         src/attention/gqa.rs:54-75
+//   GqaSpec / MlaSpec                                 src/attention/gqa.rs:144-168, src/attention/mla.rs:5-70
+//   BackendError                                      src/backend/mod.rs:38-46
+// A cache here belongs to one sequence, as the reference's RocmKvCache does (src/backend/rocm/kv_cache.rs);
+// the batched entry points of the C ABI are the extension a serving loop would use directly.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <memory>
+#include <optional>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace zllm_amd {
+
+struct BackendError {
+    enum class Kind { UnsupportedLayer, ExpertLoad, Compute };
+    Kind kind = Kind::Compute;
+    size_t layer = 0;
+    std::string msg;
+    std::string to_string() const;
+};
+
+// Rust's Result<T, BackendError>: either a value or an error, never both.
+template <class T> class Result {
+  public:
+    Result(T value) : value_(std::move(value)) {}
+    Result(BackendError error) : error_(std::move(error)) {}
+    bool is_ok() const { return value_.has_value(); }
+    bool is_err() const { return !value_.has_value(); }
+    T& unwrap() { return *value_; }
+    const T& unwrap() const { return *value_; }
+    const BackendError& unwrap_err() const { return error_; }
+
+  private:
+    std::optional<T> value_;
+    BackendError error_;
+};
+struct Unit {};
+
+struct CausalWindow {
+    bool sliding = false;
+    size_t size = 0;
+    static CausalWindow Full() { return CausalWindow{}; }
+    static CausalWindow Sliding(size_t size) { return CausalWindow{true, size}; }
+    // [start, end) of the keys a query at `query_position` sees among `key_end` cached keys
+    std::pair<size_t, size_t> key_range(size_t query_position, size_t key_end) const;
+    size_t cache_capacity(size_t max_sequence_len) const;
+};
+
+struct GqaSpec {
+    size_t num_heads = 0, num_kv_heads = 0, head_dim = 0, rope_dim = 0;
+    float rope_theta = 10000.0f;
+    bool use_qk_norm = false;
+    CausalWindow window;
+    float score_scale = 0.0f;
+    bool output_gate = false;
+    size_t group_size() const { return num_heads / num_kv_heads; }
+};
+
+enum class RotaryLayout { SplitHalf, Interleaved };
+
+struct MlaSpec {
+    size_t q_lora_rank = 0, kv_lora_rank = 0, qk_rope_head_dim = 0, q_projection_size = 0, kv_projection_size = 0, num_heads = 0;
+    float rope_theta = 10000.0f;
+    RotaryLayout rotary_layout = RotaryLayout::SplitHalf;
+    std::optional<std::string> validate() const; // message when the dimensions are inconsistent
+    size_t q_head_dim() const { return q_projection_size / num_heads; }
+    size_t qk_nope_dim() const { return q_head_dim() - qk_rope_head_dim; }
+    size_t kv_head_dim() const { return kv_projection_size / num_heads; }
+    size_t value_dim() const { return kv_head_dim() - qk_nope_dim(); }
+    size_t kv_a_out() const { return kv_lora_rank + qk_rope_head_dim; }
+};
+
+enum class DType { F32 = 0, BF16 = 1, F16 = 2 };
+size_t dtype_bytes(DType dtype);
+
+// Device buffer with shared ownership (hipMalloc / hipFree).
+class DeviceBuffer {
+  public:
+    static Result<DeviceBuffer> allocate(size_t bytes);
+    void* data() const { return ptr_.get(); }
+    size_t bytes() const { return bytes_; }
+
+  private:
+    std::shared_ptr<void> ptr_;
+    size_t bytes_ = 0;
+};
+
+// Row-major device tensor (the reference's RocmTensor with a resident device buffer).
+struct RocmTensor {
+    DeviceBuffer device;
+    size_t rows = 0, cols = 0;
+    DType dtype = DType::F32;
+};
+
+// bf16 weight matrix resident on the device (the reference's RocmWeight for kv_b).
+struct RocmWeight {
+    DeviceBuffer device;
+    size_t rows = 0, cols = 0;
+};
+
+enum class KvCacheFormat { F16, Q8g64 };
+
+// Paged KV cache of one sequence: planar code / scale planes per layer plus one block table.
+class RocmKvCache {
+  public:
+    // Q8g64 GQA cache: K codes, K scales (f16), V codes, V scales per layer
+    static Result<RocmKvCache> new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens);
+    // MLA cache: Q8g64 latent (bf16 scales) + bf16 rope per layer
+    static Result<RocmKvCache> new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens);
+    size_t len(size_t layer) const { return layer < lens_.size() ? lens_[layer] : 0; }
+    size_t layers() const { return lens_.size(); }
+    size_t block_tokens() const { return block_tokens_; }
+    size_t max_tokens() const { return max_tokens_; }
+    const std::vector<uint32_t>& block_table() const { return table_host_; }
+
+  private:
+    friend class RocmContext;
+    struct Layer {
+        DeviceBuffer a_codes, a_scales, b_codes, b_scales; // GQA: K, V; MLA: latent codes / scales, rope in b_codes
+    };
+    bool mla_ = false;
+    size_t cols_ = 0, rope_cols_ = 0, block_tokens_ = 0, max_tokens_ = 0, pool_rows_ = 0;
+    std::vector<Layer> layers_;
+    std::vector<size_t> lens_;
+    std::vector<uint32_t> table_host_;
+    DeviceBuffer table_;
+};
+
+class RocmContext {
+  public:
+    static Result<RocmContext> create(int device_id);
+    int device_id() const { return device_id_; }
+    hipStream_t stream() const { return stream_; }
+    Result<Unit> synchronize() const;
+
+    Result<RocmTensor> tensor_from_f32(const std::vector<float>& host, size_t rows, size_t cols, DType dtype = DType::F32) const;
+    Result<std::vector<float>> tensor_to_f32(const RocmTensor& tensor) const;
+    // DecodeBackend::prepare_mla_kv_b: kv_b [heads * kv_head_dim, latent] -> bf16 on the device
+    Result<RocmWeight> prepare_mla_kv_b(const std::vector<float>& weight, size_t rows, size_t cols) const;
+
+    // Appends the chunk's K/V rows at `position` (must equal the layer's cached length), then attends:
+    // one row -> split-KV decode, more rows -> chunked prefill (causal, optional sliding window).
+    // Returns f32 [rows, num_heads * head_dim].  `retain_full_cache` is accepted for signature parity:
+    // this cache always keeps every row.
+    Result<RocmTensor> gqa_prefill_attention_cached(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
+                                                    const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                    bool retain_full_cache) const;
+    Result<Unit> append_mla(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope) const;
+    Result<Unit> append_mla_rope(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
+                                 RotaryLayout layout, size_t position, const std::vector<float>& cos, const std::vector<float>& sin) const;
+    // query [1, heads * q_head_dim]; returns f32 [1, heads * value_dim]
+    Result<RocmTensor> mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
+                                            size_t position, const MlaSpec& spec) const;
+
+  private:
+    Result<Unit> append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
+                                 RotaryLayout layout, size_t position, const float* cos_dev, const float* sin_dev) const;
+    int device_id_ = 0;
+    hipStream_t stream_ = nullptr;
+};
+
+} // namespace zllm_amd
