@@ -1,0 +1,95 @@
+"""Writes the golden fixtures of this directory: small seeded inputs of the attention path and the outputs the
+CPU oracle computes for them (run from the repo root: `python tests/golden/make_fixtures.py`).
+
+The fixtures are data only.  They freeze the oracle's numbers at the time the oracle was pinned against the
+reference's known-answer tests (tests/test_oracle_known_answers.py), so that a later change of the oracle or of a
+kernel shows up as a difference against committed bytes:
+  q8g64_quantizer.npz   128 rows x 256 columns in three magnitude regimes -> codes and scales of the three rules
+  gqa_decode_small.npz  B=3 ragged, 8q/2kv, d=128, 16-token pages -> decode output
+  mla_decode_small.npz  B=2, 4 heads, latent 512 + rope 64 -> output before the final bf16 rounding
+  gqa_prefill_small.npz prefix 200 + chunk 48, 8q/2kv, window 0 and 64 -> chunk outputs
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+import oracle as O  # noqa: E402
+from tests.cases import make_gqa_q8_case, oracle_gqa_decode  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def quantizer():
+    rng = np.random.default_rng(100)
+    x = rng.standard_normal((128, 256)).astype(np.float32)
+    x[32:64] *= 1e-3
+    x[64:96] *= 300.0
+    x[96] = 0.0
+    x[97, :64] = np.float32(127.0)
+    out = {"input": x}
+    table = np.arange(8, dtype=np.uint32)
+    for name, rule, dtype in (("rocm_mla", O.RULE_ROCM_MLA, np.uint16), ("metal_gqa", O.RULE_METAL_GQA, np.uint16),
+                              ("cuda_gqa", O.RULE_CUDA_GQA, np.float32)):
+        codes = np.zeros((128, 256), dtype=np.int8)
+        scales = np.zeros((128, 4), dtype=dtype)
+        O.q8g64_append_paged(rule, x, codes, scales, table, 0, 16)
+        out[name + "_codes"] = codes
+        out[name + "_scales"] = scales
+    np.savez_compressed(os.path.join(HERE, "q8g64_quantizer.npz"), **out)
+
+
+def gqa_decode():
+    case = make_gqa_q8_case(501, [130, 77, 300], 8, 2, 128, outliers=True, q_bf16=True)
+    want = oracle_gqa_decode(case, 0.09)
+    np.savez_compressed(os.path.join(HERE, "gqa_decode_small.npz"), q_bits=case["q_bits"], lens=case["lens"], tables=case["tables"],
+                        score_scale=np.float32(0.09), expected=want, **case["planes"])
+
+
+def mla_decode():
+    from tests.test_gpu_mla_decode import make_mla_case, oracle_mla
+
+    case = make_mla_case(502, [150, 41], 4)
+    want, want_bf16 = oracle_mla(case)
+    np.savez_compressed(os.path.join(HERE, "mla_decode_small.npz"), q_bits=case["q_bits"], kv_b_bits=case["kv_b_bits"], codes=case["codes"],
+                        scales=case["scales"], rope=case["rope"], tables=case["tables"], lens=case["lens"], expected_f32=want,
+                        expected_bf16=want_bf16)
+
+
+def gqa_prefill():
+    rng = np.random.default_rng(503)
+    hq, hkv, d, bt, prefix, chunk = 8, 2, 128, 16, 200, 48
+    cols = hkv * d
+    total = prefix + chunk
+    table = rng.permutation(20)[: (total + bt - 1) // bt].astype(np.uint32)
+    rows = 20 * bt
+    planes = {n: np.zeros((rows, cols if "codes" in n else cols // 64), dtype=np.int8 if "codes" in n else np.uint16)
+              for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    k = rng.standard_normal((total, cols)).astype(np.float32)
+    v = rng.standard_normal((total, cols)).astype(np.float32)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, k, planes["k_codes"], planes["k_scales"], table, 0, bt)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, planes["v_codes"], planes["v_scales"], table, 0, bt)
+    q_bits = O.f32_to_bf16(rng.standard_normal((chunk, hq * d)).astype(np.float32))
+    q = O.bf16_to_f32(q_bits)
+    kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], O.SCALE_F16, table, bt, 0, total, cols)
+    vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], O.SCALE_F16, table, bt, 0, total, cols)
+    out = {}
+    for window in (0, 64):
+        rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=0.0884)
+        assert rc == 0
+        out[f"expected_window_{window}"] = want
+    np.savez_compressed(os.path.join(HERE, "gqa_prefill_small.npz"), q_bits=q_bits, table=table, prefix=np.uint32(prefix),
+                        score_scale=np.float32(0.0884), **planes, **out)
+
+
+if __name__ == "__main__":
+    quantizer()
+    gqa_decode()
+    mla_decode()
+    gqa_prefill()
+    for name in sorted(os.listdir(HERE)):
+        if name.endswith(".npz"):
+            print(name, os.path.getsize(os.path.join(HERE, name)))

@@ -1,0 +1,92 @@
+"""The committed fixtures of tests/golden: the oracle must still reproduce them on the CPU (no drift of the checker),
+and the HIP kernels must match them on a GPU (bit-exact for the quantizer, attention tolerance otherwise)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as O
+from tests.cases import assert_attention_close, to_torch_bf16, upload
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+RULES = (("rocm_mla", O.RULE_ROCM_MLA), ("metal_gqa", O.RULE_METAL_GQA), ("cuda_gqa", O.RULE_CUDA_GQA))
+
+
+def load(name):
+    return np.load(os.path.join(GOLDEN, name), allow_pickle=False)
+
+
+def test_oracle_reproduces_the_quantizer_fixture():
+    g = load("q8g64_quantizer.npz")
+    table = np.arange(8, dtype=np.uint32)
+    for name, rule in RULES:
+        codes = np.zeros_like(g[name + "_codes"])
+        scales = np.zeros_like(g[name + "_scales"])
+        O.q8g64_append_paged(rule, g["input"], codes, scales, table, 0, 16)
+        assert np.array_equal(codes, g[name + "_codes"]), name
+        assert np.array_equal(scales.view(np.uint8), g[name + "_scales"].view(np.uint8)), name
+
+
+def test_oracle_reproduces_the_decode_fixture():
+    g = load("gqa_decode_small.npz")
+    case = dict(q=O.bf16_to_f32(g["q_bits"]), lens=g["lens"], tables=g["tables"], hq=8, hkv=2, d=128, block_tokens=16,
+                scale_dtype=O.SCALE_F16, planes={n: g[n] for n in ("k_codes", "k_scales", "v_codes", "v_scales")})
+    from tests.cases import oracle_gqa_decode
+
+    assert np.array_equal(oracle_gqa_decode(case, float(g["score_scale"])), g["expected"])
+
+
+@pytest.mark.gpu
+def test_append_kernel_matches_the_quantizer_fixture_bit_for_bit():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import ops
+
+    g = load("q8g64_quantizer.npz")
+    table = upload(np.arange(8, dtype=np.uint32))
+    for name, rule in RULES:
+        want_scales = g[name + "_scales"]
+        codes = torch.zeros((128, 256), dtype=torch.int8, device="cuda")
+        scales = torch.zeros(want_scales.shape, dtype=torch.float32 if want_scales.dtype == np.float32 else torch.int16, device="cuda")
+        ops.q8g64_append(upload(g["input"]), codes, scales, table, 0, 16, rule)
+        torch.cuda.synchronize()
+        assert np.array_equal(codes.cpu().numpy(), g[name + "_codes"]), name
+        assert np.array_equal(scales.cpu().numpy().view(np.uint8), want_scales.view(np.uint8)), name
+
+
+@pytest.mark.gpu
+def test_decode_kernel_matches_the_decode_fixture():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import capi, ops
+
+    g = load("gqa_decode_small.npz")
+    out = ops.gqa_decode(to_torch_bf16(g["q_bits"], "cuda"), upload(g["k_codes"]), upload(g["k_scales"]), upload(g["v_codes"]),
+                         upload(g["v_scales"]), upload(g["tables"]), upload(g["lens"]), 8, 2, 128, 16, float(g["score_scale"]),
+                         int(g["lens"].max()), kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16)
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g["expected"], "decode fixture")
+
+
+@pytest.mark.gpu
+def test_mla_kernel_matches_the_mla_fixture():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import ops
+
+    g = load("mla_decode_small.npz")
+    out = ops.mla_decode(to_torch_bf16(g["q_bits"], "cuda"), upload(g["kv_b_bits"]), upload(g["codes"]), upload(g["scales"]), upload(g["rope"]),
+                         upload(g["tables"]), upload(g["lens"]), 4, 192, 256, 512, 64, 16, int(g["lens"].max()))
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g["expected_f32"].reshape(out.shape), "MLA fixture")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [0, 64])
+def test_prefill_kernel_matches_the_prefill_fixture(window):
+    torch = pytest.importorskip("torch")
+    from zllm_amd import capi, ops
+
+    g = load("gqa_prefill_small.npz")
+    out = ops.gqa_prefill_chunk(to_torch_bf16(g["q_bits"], "cuda"), upload(g["k_codes"]), upload(g["k_scales"]), upload(g["v_codes"]),
+                                upload(g["v_scales"]), upload(g["table"]), int(g["prefix"]), 8, 2, 128, 16, float(g["score_scale"]),
+                                window=window, scale_dtype=capi.SCALE_F16)
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g[f"expected_window_{window}"], f"prefill fixture, window {window}")
