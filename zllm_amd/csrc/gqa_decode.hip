@@ -125,15 +125,15 @@ template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(
 // gaps where short sequences end, and one XCD can end up with more live workgroups than CUs).  Every wave
 // finds its item by a prefix sum over the sequences' split counts; ids past the last item exit.
 __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned int item, unsigned int lane, unsigned int& b_out,
-                                             unsigned int& chunk_out)
+                                             unsigned int& chunk_out, unsigned int& len_out, unsigned int& first_out)
 {
     unsigned int base = 0;
     for (unsigned int b0 = 0; b0 < p.batch; b0 += 64u) {
         const unsigned int i = b0 + lane;
-        unsigned int n = 0;
+        unsigned int n = 0, len = 0, first = 0;
         if (i < p.batch) {
-            const unsigned int len = p.kv_lens[i];
-            unsigned int first = p.first_visible != nullptr ? p.first_visible[i] : 0u;
+            len = p.kv_lens[i];
+            first = p.first_visible != nullptr ? p.first_visible[i] : 0u;
             first = min(first, len);
             const unsigned int first_al = first & ~31u;
             n = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
@@ -151,6 +151,8 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
             const unsigned int src = (unsigned int)__builtin_ctzll(hit);
             b_out = b0 + src;
             chunk_out = local - (__builtin_amdgcn_readlane(incl, src) - __builtin_amdgcn_readlane(n, src));
+            len_out = __builtin_amdgcn_readlane(len, src); // already here: no second trip to memory for them
+            first_out = __builtin_amdgcn_readlane(first, src);
             return true;
         }
         base += total;
@@ -162,52 +164,61 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
 // The head's query row is quantized to 15-bit fixed point (step = max|q| / 16256) and split into two
 // signed-byte digits q = 128 * hi + lo, hi in [-127, 127], lo in [-64, 63]: K codes then feed the matrix
 // cores as raw bytes and the integer dot products are exact.
+// Fetching and quantizing are separate so that a kernel can start the fetch, issue other loads, and
+// quantize when the data is needed.
+template <int D> struct QueryRaw {
+    u32x4 v[D / 64][4]; // 16 consecutive elements per scale group: four vectors of f32, or two of 16-bit values
+};
+
 template <int D>
-__device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsigned int b, unsigned int head, bool head_valid,
-                                                  unsigned int j, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64], float& q_step)
+__device__ __forceinline__ QueryRaw<D> fetch_query(const GqaDecodeParams& p, unsigned int b, unsigned int head, bool head_valid, unsigned int j)
+{
+    constexpr int G = D / 64;
+    QueryRaw<D> raw;
+    const size_t q_index = ((size_t)b * p.num_heads + head) * D + j * 16;
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            raw.v[a][w] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    if (head_valid) {
+        if (p.q_dtype == 0) {
+#pragma unroll
+            for (int a = 0; a < G; ++a) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    raw.v[a][w] = *(const u32x4*)((const float*)p.q + q_index + a * 64 + 4 * w);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < G; ++a) {
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    raw.v[a][w] = *(const u32x4*)((const unsigned short*)p.q + q_index + a * 64 + 8 * w);
+                }
+            }
+        }
+    }
+    return raw;
+}
+
+template <int D>
+__device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const QueryRaw<D>& raw, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64],
+                                               float& q_step)
 {
     constexpr int G = D / 64;
     float x[G][16];
-    // 16 consecutive elements per scale group, fetched as whole 16-byte vectors (one round trip, not 32)
-    const size_t q_index = ((size_t)b * p.num_heads + head) * D + j * 16;
-    if (!head_valid) {
 #pragma unroll
-        for (int a = 0; a < G; ++a) {
+    for (int a = 0; a < G; ++a) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                x[a][e] = 0.0f;
-            }
-        }
-    } else if (p.q_dtype == 0) {
-        f32x4 raw[G][4];
-#pragma unroll
-        for (int a = 0; a < G; ++a) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                raw[a][w] = *(const f32x4*)((const float*)p.q + q_index + a * 64 + 4 * w);
-            }
-        }
-#pragma unroll
-        for (int a = 0; a < G; ++a) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                x[a][e] = raw[a][e / 4][e % 4];
-            }
-        }
-    } else {
-        u32x4 raw[G][2];
-#pragma unroll
-        for (int a = 0; a < G; ++a) {
-#pragma unroll
-            for (int w = 0; w < 2; ++w) {
-                raw[a][w] = *(const u32x4*)((const unsigned short*)p.q + q_index + a * 64 + 8 * w);
-            }
-        }
-#pragma unroll
-        for (int a = 0; a < G; ++a) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const unsigned int word = raw[a][e / 8][(e % 8) / 2];
+        for (int e = 0; e < 16; ++e) {
+            if (p.q_dtype == 0) {
+                x[a][e] = __uint_as_float(raw.v[a][e / 4][e % 4]);
+            } else {
+                const unsigned int word = raw.v[a][e / 8][(e % 8) / 2];
                 const unsigned short bits = (unsigned short)((e & 1) ? (word >> 16) : (word & 0xffffu));
                 x[a][e] = p.q_dtype == 1 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
             }
@@ -243,6 +254,14 @@ __device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsi
             qlo[a][w] = (int)lo_word;
         }
     }
+}
+
+template <int D>
+__device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsigned int b, unsigned int head, bool head_valid,
+                                                  unsigned int j, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64], float& q_step)
+{
+    const QueryRaw<D> raw = fetch_query<D>(p, b, head, head_valid, j);
+    quantize_query<D>(p, raw, qhi, qlo, q_step);
 }
 
 // One 32-token step, first half: scores, masking and the online-softmax update.
@@ -362,13 +381,10 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
+    unsigned int b, chunk, len, first;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
         return;
     }
-    const unsigned int len = p.kv_lens[b];
-    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
-    first = min(first, len);
     const unsigned int first_al = first & ~31u;
     const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
     const unsigned int head_in_group = head_block * 16u + m;
@@ -628,13 +644,10 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
+    unsigned int b, chunk, len, first;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
         return;
     }
-    const unsigned int len = p.kv_lens[b];
-    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
-    first = min(first, len);
     const unsigned int first_al = first & ~31u;
     const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
     const unsigned int head_in_group = head_block * 16u + m;
@@ -667,6 +680,8 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
     unsigned int entries0 = p.tables != nullptr ? table[min(first_page + lane, last_page)] : first_page + lane;
     unsigned int entries1 = p.tables != nullptr ? table[min(first_page + 64u + lane, last_page)] : first_page + 64u + lane;
+    // the query fetch rides along with the table loads; it is quantized after the first KV loads are out
+    const QueryRaw<D> q_raw = fetch_query<D>(p, b, head, head_valid, j);
     asm volatile("" : "+v"(entries0), "+v"(entries1)); // their wait happens here, not inside the loop
     auto tile_row = [&](unsigned int T) __attribute__((always_inline)) -> unsigned long long {
         const unsigned int t = min(max(T, lo_tile), hi_tile);
@@ -741,7 +756,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     }
     i32x4 qhi[G], qlo[G];
     float q_step;
-    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
+    quantize_query<D>(p, q_raw, qhi, qlo, q_step);
 
     const float scale_log2 = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_step;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
@@ -840,13 +855,10 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk)) {
+    unsigned int b, chunk, len, first;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
         return;
     }
-    const unsigned int len = p.kv_lens[b];
-    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
-    first = min(first, len);
     const unsigned int first_al = first & ~31u;
     const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
     const unsigned int head_in_group = head_block * 16u + m;
