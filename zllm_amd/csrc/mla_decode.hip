@@ -46,12 +46,15 @@ union Frag {
     bf16x8 b;
 };
 
-// chunk swizzle: eight consecutive rows land in eight different 16-byte columns, and four
-// consecutive rows in four different 32-byte column pairs
+// Chunk swizzle for the 64-bank LDS (256 B per cycle).  A tile row is 72 chunks of 16 B, i.e. 8 chunks past a
+// multiple of 256 B, so the row's parity already selects the upper or lower 128 B of a bank line; XOR-ing
+// row bits 1 and 2 into chunk bits 1 and 2 spreads eight rows over all sixteen 16-byte slots.  Measured with
+// the LDS bank-conflict counter: ds_read_b128 of the K operand (lanes = 16 rows x 4 k-slices) 4.0 cycles and
+// ds_read_b64_tr_b16 of the V operand 2.0 cycles per instruction, both conflict-free (the earlier swizzle,
+// laid out for 32 banks, took 8 and 4).
 __device__ __forceinline__ unsigned int swz(unsigned int row)
 {
-    const unsigned int x = row & 7u;
-    return ((x & 3u) << 1) | (x >> 2);
+    return row & 6u;
 }
 
 __device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned int chunk)
@@ -240,21 +243,26 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's raw items have landed
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
+            // the thread converts codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row: 32 consecutive lanes then
+            // write 512 contiguous bytes per instruction (chunks cc and cc + 32), which the LDS takes without conflicts
             const unsigned int row = t_lo + TROWS * i;
-            const u32x4 codes = *(const u32x4*)(raw_codes + row * kLatent + cc * 16u);
-            u32x4 out[2];
+            const u32x2 half[2] = {*(const u32x2*)(raw_codes + row * kLatent + cc * 8u),
+                                   *(const u32x2*)(raw_codes + row * kLatent + 256u + cc * 8u)};
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const unsigned int word = codes[w];
-                const float c0 = (float)(int)(signed char)(word & 0xffu);
-                const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
-                const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
-                const float c3 = (float)(int)(signed char)(word >> 24);
-                out[w >> 1][(w & 1) * 2] = pack_bf16_trunc(c0, c1);
-                out[w >> 1][(w & 1) * 2 + 1] = pack_bf16_trunc(c2, c3);
+            for (int h = 0; h < 2; ++h) {
+                u32x4 out;
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const unsigned int word = half[h][w];
+                    const float c0 = (float)(int)(signed char)(word & 0xffu);
+                    const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
+                    const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
+                    const float c3 = (float)(int)(signed char)(word >> 24);
+                    out[w * 2] = pack_bf16_trunc(c0, c1);
+                    out[w * 2 + 1] = pack_bf16_trunc(c2, c3);
+                }
+                *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
             }
-            *(u32x4*)(tile + tile_offset(row, cc * 2u)) = out[0];
-            *(u32x4*)(tile + tile_offset(row, cc * 2u + 1u)) = out[1];
         }
         if (has_rope) {
             *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = *(const u32x4*)(raw_rope + tid * 16u);
@@ -440,6 +448,11 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
         unsigned char* nxt = lds + ((step + 1u) & 1u) * kTileBytes;
         const bool more = step + 1 < steps;
         if (more) {
+            // place the wait for the block-table entries (fetched a step ago) before this step's first load
+#pragma unroll
+            for (int i = 0; i <= ITEMS; ++i) {
+                asm volatile("" : "+v"(rows.entry[i]));
+            }
             issue_step(rows, c_start + (step + 1u) * kStepTokens);
             if (step + 2 < steps) {
                 lookup_step(rows, c_start + (step + 2u) * kStepTokens);
@@ -466,6 +479,358 @@ __global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
             *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2b. split-KV partial, role-specialised waves
+// ---------------------------------------------------------------------------------------------
+// Workgroup = (split, block of 64 heads, sequence), eight waves in two roles that run one step apart:
+//   score waves (0..3, 16 heads each): S^T = K.Q^T for all 32 tokens of tile i, online softmax, and hand
+//       the step's probabilities p[32 tokens] and the rescale factor alpha to their value wave through LDS.
+//       The C layout of S^T is the B layout the value wave needs, so the hand-over is lane to lane.
+//   value waves (4..7, the same 16 heads, all 512 output columns): O^T += V^T.P' for tile i - 1.
+// The score work is LDS reads + vector ALU (exp, max), the value work LDS reads + MFMA; with one wave of each
+// role per SIMD the two overlap instead of every wave running the same phase at the same time, and the
+// score exchange between waves of a head tile (a second barrier per step) disappears.  Three tile buffers
+// rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the raw bytes that the
+// global -> LDS loads of the previous iteration brought in).  One LDS-only barrier per step.
+constexpr int kWsTiles = 3;
+
+__global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
+{
+    constexpr int ITEMS = 2;  // staging items per thread: 32 tokens x 32 code chunks over 512 threads
+    constexpr int TROWS = 16; // token rows covered by one pass of the threads
+    __shared__ __align__(16) unsigned char lds[kWsTiles * kTileBytes];
+    __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
+    __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
+    __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
+    __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
+    const unsigned int tid = threadIdx.x;
+    const unsigned int lane = tid & 63u;
+    const unsigned int wave = tid >> 6;
+    const bool value_role = wave >= 4u;
+    const unsigned int hw = wave & 3u;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    const unsigned int chunk = blockIdx.x;
+    const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
+    const unsigned int b = blockIdx.z;
+    const unsigned int len = p.ctx_lens[b];
+    const unsigned long long c_start64 = (unsigned long long)chunk * p.chunk_tokens;
+    const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
+    if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
+        if (head < p.heads && j == 0 && !value_role) {
+            p.stats[rec * 2] = kNegInf;
+            p.stats[rec * 2 + 1] = 0.0f;
+        }
+        return;
+    }
+    const unsigned int c_start = (unsigned int)c_start64;
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int steps = (c_end - c_start + kStepTokens - 1) / kStepTokens;
+    const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
+    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
+
+    // ---- staging (same scheme as mla_partial): loads of the next tile's raw bytes, converted by their owner
+    const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned int cc = tid & 31u;
+    const unsigned int t_lo = tid >> 5;
+    const unsigned int rope_t = (tid >> 3) & 31u;
+    const unsigned int rope_c = tid & 7u;
+    const bool has_rope = tid < 256u;
+    const bool has_scales = tid >= 256u && tid < 256u + kStepTokens;
+    const unsigned int extra_t = has_rope ? rope_t : (tid - 256u) & 31u;
+    unsigned char* const raw_codes = lds_raw;
+    unsigned char* const raw_rope = lds_raw + kRawCodes;
+    unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
+    auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i <= ITEMS; ++i) {
+            const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+            const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+            r.entry[i] = table != nullptr ? table[page] : page;
+        }
+    };
+    auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
+        const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+        if (pow2) {
+            return ((unsigned long long)r.entry[i] << p.block_shift) + (token & (p.block_tokens - 1u));
+        }
+        return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
+    };
+    auto issue_step = [&](const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
+                                             (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
+        }
+        if (has_rope) {
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
+                                             (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+        }
+        if (has_scales) {
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
+                                             (lds_ptr_t)(raw_scales), 16, 0, 0);
+        }
+    };
+    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            // the thread converts codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row: 32 consecutive lanes then
+            // write 512 contiguous bytes per instruction (chunks cc and cc + 32), which the LDS takes without conflicts
+            const unsigned int row = t_lo + TROWS * i;
+            const u32x2 half[2] = {*(const u32x2*)(raw_codes + row * kLatent + cc * 8u),
+                                   *(const u32x2*)(raw_codes + row * kLatent + 256u + cc * 8u)};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                u32x4 out;
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const unsigned int word = half[h][w];
+                    const float c0 = (float)(int)(signed char)(word & 0xffu);
+                    const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
+                    const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
+                    const float c3 = (float)(int)(signed char)(word >> 24);
+                    out[w * 2] = pack_bf16_trunc(c0, c1);
+                    out[w * 2 + 1] = pack_bf16_trunc(c2, c3);
+                }
+                *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
+            }
+        }
+        if (has_rope) {
+            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = *(const u32x4*)(raw_rope + tid * 16u);
+        }
+        if (has_scales) {
+            const u32x4 sc8 = *(const u32x4*)(raw_scales + (tid - 256u) * 16u);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const unsigned int word = sc8[g >> 1];
+                scale_tile[g][tid - 256u] = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+
+    // LDS byte offsets of this lane's fragments (lane part; the rest is compile-time)
+    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ swz(m)) << 4), m * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
+    const unsigned int tr_row = 4u * j + (m >> 2);
+    unsigned int pv_base[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+    }
+
+    StepRows rows;
+    lookup_step(rows, c_start);
+    issue_step(rows, c_start);
+    if (steps > 1) {
+        lookup_step(rows, c_start + kStepTokens);
+    }
+    convert_step(lds, lds_scale[0]);
+    lds_barrier();
+
+    // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile i - 1.
+    auto stage_next = [&](unsigned int i) __attribute__((always_inline)) {
+        if (i + 1 < steps) {
+            // The entries were fetched an iteration ago.  Naming them here places the compiler's wait for them
+            // before the first load of this iteration; left to itself it waits again before every address it
+            // forms from them, i.e. for the load it has just issued.
+            asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]));
+            issue_step(rows, c_start + (i + 1u) * kStepTokens);
+            if (i + 2 < steps) {
+                lookup_step(rows, c_start + (i + 2u) * kStepTokens);
+            }
+        }
+    };
+    auto finish_iteration = [&](unsigned int i) __attribute__((always_inline)) {
+        if (i + 1 < steps) {
+            const unsigned int nb = (i + 1u) % kWsTiles;
+            convert_step(lds + nb * kTileBytes, lds_scale[nb]);
+        }
+        lds_barrier();
+    };
+
+    if (!value_role) {
+        // ================================ score waves ================================
+        Frag qf[18]; // B operand: lane = (head column m, k-slice j); k-step ks covers dims ks*32 + j*8 .. +8
+        {
+            const unsigned short* qa = p.absorbed + ((size_t)b * p.heads + min(head, p.heads - 1u)) * kRowElems;
+#pragma unroll
+            for (int ks = 0; ks < 18; ++ks) {
+                u32x4 v = *(const u32x4*)(qa + ks * 32 + j * 8);
+                if (head >= p.heads) {
+                    v = u32x4{0u, 0u, 0u, 0u};
+                }
+                qf[ks].u = v;
+            }
+        }
+        float run_max = kNegInf, run_sum = 0.0f;
+        const float scale_log2 = p.score_scale * kLog2e;
+        for (unsigned int i = 0; i <= steps; ++i) {
+            stage_next(i);
+            if (i < steps) {
+                const unsigned int tb = i % kWsTiles;
+                const unsigned char* tile = lds + tb * kTileBytes;
+                const float (*scale_tile)[kStepTokens] = lds_scale[tb];
+                const unsigned int t0 = c_start + i * kStepTokens;
+                float sc[8];
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2) {
+                    const unsigned char* kt = tile + t2 * 16 * kRowBytes;
+                    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
+                        Frag kf;
+                        kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
+                        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) { // four independent accumulators at a time
+                        f32x4 d[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int g = half * 4 + u;
+                            Frag k0;
+                            k0.u = *(const u32x4*)(kt + qk_base[0] + g * 128);
+                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int g = half * 4 + u;
+                            Frag k1;
+                            k1.u = *(const u32x4*)(kt + qk_base[1] + g * 128);
+                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int g = half * 4 + u;
+                            const f32x4 gs = *(const f32x4*)(&scale_tile[g][t2 * 16 + 4 * j]);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                s[r] = fmaf(d[u][r], gs[r], s[r]);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const unsigned int token = t0 + 16u * t2 + 4u * j + r;
+                        sc[t2 * 4 + r] = token < len ? s[r] * scale_log2 : kNegInf;
+                    }
+                }
+                // online softmax for this head column; lazy rescaling: the stored maximum only moves when a
+                // score exceeds it by 2^8 (p stays <= 256)
+                float step_max = sc[0];
+#pragma unroll
+                for (int e = 1; e < 8; ++e) {
+                    step_max = fmaxf(step_max, sc[e]);
+                }
+                step_max = wave_max_16x4(step_max);
+                float new_max = run_max;
+                if (step_max > run_max + 8.0f || run_max == kNegInf) {
+                    new_max = fmaxf(run_max, step_max);
+                }
+                const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+                const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max); // 0 on the first step: nothing accumulated yet
+                f32x4 p_lo, p_hi;
+                float step_sum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    p_lo[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+                    p_hi[e] = __builtin_amdgcn_exp2f(sc[4 + e] - safe_max);
+                    step_sum += p_lo[e] + p_hi[e];
+                }
+                run_sum = run_sum * alpha + step_sum;
+                run_max = new_max;
+                float* slot = lds_p[i & 1u][hw][lane];
+                *(f32x4*)(slot) = p_lo;
+                *(f32x4*)(slot + 4) = p_hi;
+                lds_alpha[i & 1u][hw][lane] = alpha;
+            }
+            finish_iteration(i);
+        }
+        const float total = wave_sum_16x4(run_sum);
+        if (head < p.heads && j == 0) {
+            p.stats[rec * 2] = run_max;
+            p.stats[rec * 2 + 1] = total;
+        }
+    } else {
+        // ================================ value waves ================================
+        f32x4 acc[32];
+#pragma unroll
+        for (int t = 0; t < 32; ++t) {
+            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        for (unsigned int i = 0; i <= steps; ++i) {
+            stage_next(i);
+            if (i > 0) {
+                const unsigned int tb = (i - 1u) % kWsTiles;
+                const unsigned char* tile = lds + tb * kTileBytes;
+                const float (*scale_tile)[kStepTokens] = lds_scale[tb];
+                const float* slot = lds_p[(i - 1u) & 1u][hw][lane];
+                const f32x4 p_lo = *(const f32x4*)(slot);
+                const f32x4 p_hi = *(const f32x4*)(slot + 4);
+                const float alpha = lds_alpha[(i - 1u) & 1u][hw][lane];
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int t = 0; t < 32; ++t) {
+                        acc[t] *= alpha;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                // V^T fragments of scale group g + 1 are requested before group g's MFMAs are issued: with the
+                // reads in program order behind each MFMA the wave pays one LDS round trip per tile.
+                union VFrag {
+                    s16x4 s[2];
+                    bf16x8 b;
+                };
+                auto load_group = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int tt = 0; tt < 4; ++tt) {
+                        const unsigned char* at = tile + pv_base[tt] + g * 128;
+                        vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                        vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+                    }
+                };
+                auto scales_of = [&](int g, f32x4& gs0, f32x4& gs1) __attribute__((always_inline)) {
+                    const float* gs_row = scale_tile[g];
+                    gs0 = *(const f32x4*)(gs_row + 4 * j);
+                    gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
+                };
+                VFrag vf[2][4];
+                f32x4 gs0[2], gs1[2];
+                load_group(vf[0], 0);
+                scales_of(0, gs0[0], gs1[0]);
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const int cur = g & 1;
+                    if (g + 1 < 8) {
+                        load_group(vf[cur ^ 1], g + 1);
+                        scales_of(g + 1, gs0[cur ^ 1], gs1[cur ^ 1]);
+                    }
+                    asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
+                    Frag pf; // P'_g = bf16(p * scale_g)
+                    pf.u[0] = pack_bf16_hw(p_lo[0] * gs0[cur][0], p_lo[1] * gs0[cur][1]);
+                    pf.u[1] = pack_bf16_hw(p_lo[2] * gs0[cur][2], p_lo[3] * gs0[cur][3]);
+                    pf.u[2] = pack_bf16_hw(p_hi[0] * gs1[cur][0], p_hi[1] * gs1[cur][1]);
+                    pf.u[3] = pack_bf16_hw(p_hi[2] * gs1[cur][2], p_hi[3] * gs1[cur][3]);
+#pragma unroll
+                    for (int tt = 0; tt < 4; ++tt) {
+                        acc[g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pf.b, acc[g * 4 + tt], 0, 0, 0);
+                    }
+                }
+            }
+            finish_iteration(i);
+        }
+        if (head < p.heads) {
+            float* out = p.partial + rec * kLatent;
+#pragma unroll
+            for (int t = 0; t < 32; ++t) {
+                *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no load may still target this workgroup's LDS at exit
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -542,7 +907,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     }
     if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
-        mla_partial<2><<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
+        mla_partial_ws<<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
         err = hipGetLastError();
         if (err != hipSuccess) {
             return err;
