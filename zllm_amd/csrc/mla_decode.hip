@@ -675,40 +675,55 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 const float (*scale_tile)[kStepTokens] = lds_scale[tb];
                 const unsigned int t0 = c_start + i * kStepTokens;
                 float sc[8];
+                // K fragments are requested one batch (four k-steps) ahead of the MFMAs that use them.
+                // Batch q of a token tile: q = 0..3 -> latent groups {0..3} first k-step, {0..3} second k-step,
+                // {4..7} first, {4..7} second; the two rope k-steps ride along with batch 0.
+                auto load_batch = [&](Frag (&kf)[4], const unsigned char* kt, int q) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        kf[u].u = *(const u32x4*)(kt + qk_base[q & 1] + ((q >> 1) * 4 + u) * 128);
+                    }
+                };
+                Frag kf[2][4], kr[2];
+                load_batch(kf[0], tile, 0);
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) {
                     const unsigned char* kt = tile + t2 * 16 * kRowBytes;
                     f32x4 s = {0.f, 0.f, 0.f, 0.f};
+                    kr[0].u = *(const u32x4*)(kt + qk_base[0] + 8 * 128);
+                    kr[1].u = *(const u32x4*)(kt + qk_base[1] + 8 * 128);
+                    f32x4 d[4];
 #pragma unroll
-                    for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
-                        Frag kf;
-                        kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
-                        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) { // four independent accumulators at a time
-                        f32x4 d[4];
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int g = half * 4 + u;
-                            Frag k0;
-                            k0.u = *(const u32x4*)(kt + qk_base[0] + g * 128);
-                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    for (int q = 0; q < 4; ++q) {
+                        const int cur = q & 1;
+                        if (q + 1 < 4) {
+                            load_batch(kf[cur ^ 1], kt, q + 1);
+                        } else if (t2 == 0) {
+                            load_batch(kf[cur ^ 1], kt + 16 * kRowBytes, 0);
+                        }
+                        asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
+                        if (q == 0) {
+                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[0].b, qf[16].b, s, 0, 0, 0);
+                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[1].b, qf[17].b, s, 0, 0, 0);
                         }
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
-                            const int g = half * 4 + u;
-                            Frag k1;
-                            k1.u = *(const u32x4*)(kt + qk_base[1] + g * 128);
-                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                            const int g = (q >> 1) * 4 + u;
+                            if ((q & 1) == 0) {
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[cur][u].b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                            } else {
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[cur][u].b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                            }
                         }
+                        if ((q & 1) == 1) {
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int g = half * 4 + u;
-                            const f32x4 gs = *(const f32x4*)(&scale_tile[g][t2 * 16 + 4 * j]);
+                            for (int u = 0; u < 4; ++u) {
+                                const int g = (q >> 1) * 4 + u;
+                                const f32x4 gs = *(const f32x4*)(&scale_tile[g][t2 * 16 + 4 * j]);
 #pragma unroll
-                            for (int r = 0; r < 4; ++r) {
-                                s[r] = fmaf(d[u][r], gs[r], s[r]);
+                                for (int r = 0; r < 4; ++r) {
+                                    s[r] = fmaf(d[u][r], gs[r], s[r]);
+                                }
                             }
                         }
                     }
@@ -762,15 +777,17 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
             acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         for (unsigned int i = 0; i <= steps; ++i) {
+            // the hand-over record is requested first: its LDS round trip hides behind the staging work
+            const float* slot = lds_p[(i + 1u) & 1u][hw][lane];
+            const f32x4 p_lo = *(const f32x4*)(slot);
+            const f32x4 p_hi = *(const f32x4*)(slot + 4);
+            const float alpha = lds_alpha[(i + 1u) & 1u][hw][lane];
+            asm volatile("" ::: "memory");
             stage_next(i);
             if (i > 0) {
                 const unsigned int tb = (i - 1u) % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes;
                 const float (*scale_tile)[kStepTokens] = lds_scale[tb];
-                const float* slot = lds_p[(i - 1u) & 1u][hw][lane];
-                const f32x4 p_lo = *(const f32x4*)(slot);
-                const f32x4 p_hi = *(const f32x4*)(slot + 4);
-                const float alpha = lds_alpha[(i - 1u) & 1u][hw][lane];
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
                     for (int t = 0; t < 32; ++t) {
