@@ -38,10 +38,14 @@ union Frag {
     bf16x8 b;
 };
 
+// Chunk swizzle for the 64-bank LDS (256 B per cycle = one tile row).  Row bits 1 and 2 are XOR-ed into chunk
+// bits 1 and 2 and the row's parity into chunk bit 3 (the scale-group half of the row): the LDS serves a
+// 16-byte read instruction sixteen lanes per cycle (eight rows of one k-slice with eight rows of the next),
+// and this keeps those sixteen chunks on sixteen different bank groups; the transposed 8-byte reads of the V
+// operand (thirty-two consecutive lanes per cycle) stay conflict-free as well.
 __device__ __forceinline__ unsigned int swz(unsigned int row)
 {
-    const unsigned int x = row & 7u;
-    return ((x & 3u) << 1) | (x >> 2);
+    return ((row & 1u) << 3) | (row & 6u);
 }
 
 __device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned int chunk)
@@ -59,7 +63,7 @@ __device__ __forceinline__ float soft_tanh(float x)
 }
 
 struct StepRegs {
-    u32x4 codes;           // 16 codes of the thread's plane (K for threads 0..255, V for 256..511)
+    u32x2 codes[2];        // codes 8 cc .. + 8 and 64 + 8 cc .. + 8 of the thread's plane (K: threads 0..255, V: 256..511)
     unsigned int scales;   // two 16-bit scales (groups 0, 1) of the token
 };
 
@@ -141,17 +145,18 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const bool stage_v = tid >= 256u;          // threads 0..255 stage K, 256..511 stage V
     const unsigned int st_token = (tid & 255u) >> 3; // staging: token of the step, 16-code chunk cc
     const unsigned int cc = tid & 7u;
-    const unsigned char* st_codes = (stage_v ? p.v_plane : p.k_plane) + kvh * kD + cc * 16u;
+    const unsigned char* st_codes = (stage_v ? p.v_plane : p.k_plane) + kvh * kD + cc * 8u;
     const unsigned char* st_scales = (stage_v ? p.v_scales : p.k_scales) + kvh * 4u;
     auto load_step = [&](StepRegs& r, unsigned int t0, unsigned int entry) __attribute__((always_inline)) {
         const unsigned long long row = row_from(t0 + st_token, entry);
-        r.codes = *(const u32x4*)(st_codes + row * k_row);
+        r.codes[0] = *(const u32x2*)(st_codes + row * k_row);
+        r.codes[1] = *(const u32x2*)(st_codes + row * k_row + 64u);
         r.scales = *(const unsigned int*)(st_scales + row * s_row);
     };
-    auto convert16 = [&](const u32x4& codes, u32x4& lo, u32x4& hi) __attribute__((always_inline)) {
-        unsigned int out[8];
+    auto convert8 = [&](const u32x2& codes) __attribute__((always_inline)) -> u32x4 {
+        u32x4 out;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < 2; ++w) {
             const unsigned int word = codes[w];
             const float c0 = (float)(int)(signed char)(word & 0xffu);
             const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
@@ -160,15 +165,13 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             out[2 * w] = pack_bf16_trunc(c0, c1);
             out[2 * w + 1] = pack_bf16_trunc(c2, c3);
         }
-        lo = u32x4{out[0], out[1], out[2], out[3]};
-        hi = u32x4{out[4], out[5], out[6], out[7]};
+        return out;
     };
     auto store_step = [&](const StepRegs& r, int buf) __attribute__((always_inline)) {
-        u32x4 lo, hi;
-        convert16(r.codes, lo, hi);
+        // chunks cc and cc + 8: sixteen lanes (two rows x eight chunks) write sixteen different bank groups
         unsigned char* tile = stage_v ? lds_v[buf] : lds_k[buf];
-        *(u32x4*)(tile + tile_offset(st_token, cc * 2u)) = lo;
-        *(u32x4*)(tile + tile_offset(st_token, cc * 2u + 1u)) = hi;
+        *(u32x4*)(tile + tile_offset(st_token, cc)) = convert8(r.codes[0]);
+        *(u32x4*)(tile + tile_offset(st_token, cc + 8u)) = convert8(r.codes[1]);
         if (cc == 0) {
             // K scales carry the score scale (and log2 e) so that the hot loop does not multiply again
             float* dst = stage_v ? &lds_vs[buf][0][0] : &lds_ks[buf][0][0];
@@ -197,12 +200,15 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
     }
 
-    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ swz(m)) << 4), m * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
+    // chunk = g * 8 + half * 4 + j: the low three bits meet row bits 1, 2; the group bit meets the row's parity
+    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ (m & 6u)) << 4), m * kRowBytes + (((4u | j) ^ (m & 6u)) << 4)};
+    const unsigned int qk_group[2] = {(m & 1u) * 128u, 128u - (m & 1u) * 128u};
     const unsigned int tr_row = 4u * j + (m >> 2);
     unsigned int pv_base[4];
+    const unsigned int pv_group[2] = {(tr_row & 1u) * 128u, 128u - (tr_row & 1u) * 128u};
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ (tr_row & 6u)) << 4) + (m & 1u) * 8u;
     }
 
     auto compute_step = [&](int buf, unsigned int t0) __attribute__((always_inline)) {
@@ -219,8 +225,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
                 Frag k0, k1;
-                k0.u = *(const u32x4*)(kt + qk_base[0] + (i * 16 * kRowBytes + g * 128));
-                k1.u = *(const u32x4*)(kt + qk_base[1] + (i * 16 * kRowBytes + g * 128));
+                k0.u = *(const u32x4*)(kt + qk_base[0] + qk_group[g] + i * 16 * kRowBytes);
+                k1.u = *(const u32x4*)(kt + qk_base[1] + qk_group[g] + i * 16 * kRowBytes);
                 const f32x4 gs = *(const f32x4*)(&lds_ks[buf][g][i * 16 + 4 * j]);
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
@@ -321,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt) {
                 const int t = g * 4 + tt;
-                const unsigned char* at = vt + pv_base[tt] + g * 128;
+                const unsigned char* at = vt + pv_base[tt] + pv_group[g];
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
                 const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
                 union {
