@@ -771,27 +771,43 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
         }
     } else {
         // ================================ value waves ================================
-        f32x4 acc[32];
+        // Value wave v = 2 hp + dh owns head tiles 2 hp and 2 hp + 1 and output columns [256 dh, 256 dh + 256):
+        // every V^T fragment it reads from LDS feeds two MFMAs (one per head tile), which halves the LDS traffic
+        // of this stage and doubles the matrix work behind each LDS round trip.
+        const unsigned int hp = hw >> 1;
+        const unsigned int dh = hw & 1u;
+        f32x4 acc[2][16];
 #pragma unroll
-        for (int t = 0; t < 32; ++t) {
-            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ht = 0; ht < 2; ++ht) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                acc[ht][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
         }
         for (unsigned int i = 0; i <= steps; ++i) {
-            // the hand-over record is requested first: its LDS round trip hides behind the staging work
-            const float* slot = lds_p[(i + 1u) & 1u][hw][lane];
-            const f32x4 p_lo = *(const f32x4*)(slot);
-            const f32x4 p_hi = *(const f32x4*)(slot + 4);
-            const float alpha = lds_alpha[(i + 1u) & 1u][hw][lane];
+            // the hand-over records are requested first: their LDS round trip hides behind the staging work
+            f32x4 p_lo[2], p_hi[2];
+            float alpha[2];
+#pragma unroll
+            for (int ht = 0; ht < 2; ++ht) {
+                const float* slot = lds_p[(i + 1u) & 1u][2u * hp + ht][lane];
+                p_lo[ht] = *(const f32x4*)(slot);
+                p_hi[ht] = *(const f32x4*)(slot + 4);
+                alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
+            }
             asm volatile("" ::: "memory");
             stage_next(i);
             if (i > 0) {
                 const unsigned int tb = (i - 1u) % kWsTiles;
-                const unsigned char* tile = lds + tb * kTileBytes;
-                const float (*scale_tile)[kStepTokens] = lds_scale[tb];
-                if (__any(alpha != 1.0f)) {
+                const unsigned char* tile = lds + tb * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
+                const float (*scale_tile)[kStepTokens] = lds_scale[tb] + dh * 4u;
 #pragma unroll
-                    for (int t = 0; t < 32; ++t) {
-                        acc[t] *= alpha;
+                for (int ht = 0; ht < 2; ++ht) {
+                    if (__any(alpha[ht] != 1.0f)) {
+#pragma unroll
+                        for (int t = 0; t < 16; ++t) {
+                            acc[ht][t] *= alpha[ht];
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -819,31 +835,38 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 load_group(vf[0], 0);
                 scales_of(0, gs0[0], gs1[0]);
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
+                for (int g = 0; g < 4; ++g) {
                     const int cur = g & 1;
-                    if (g + 1 < 8) {
+                    if (g + 1 < 4) {
                         load_group(vf[cur ^ 1], g + 1);
                         scales_of(g + 1, gs0[cur ^ 1], gs1[cur ^ 1]);
                     }
                     asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
-                    Frag pf; // P'_g = bf16(p * scale_g)
-                    pf.u[0] = pack_bf16_hw(p_lo[0] * gs0[cur][0], p_lo[1] * gs0[cur][1]);
-                    pf.u[1] = pack_bf16_hw(p_lo[2] * gs0[cur][2], p_lo[3] * gs0[cur][3]);
-                    pf.u[2] = pack_bf16_hw(p_hi[0] * gs1[cur][0], p_hi[1] * gs1[cur][1]);
-                    pf.u[3] = pack_bf16_hw(p_hi[2] * gs1[cur][2], p_hi[3] * gs1[cur][3]);
 #pragma unroll
-                    for (int tt = 0; tt < 4; ++tt) {
-                        acc[g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pf.b, acc[g * 4 + tt], 0, 0, 0);
+                    for (int ht = 0; ht < 2; ++ht) {
+                        Frag pf; // P'_g = bf16(p * scale_g)
+                        pf.u[0] = pack_bf16_hw(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1]);
+                        pf.u[1] = pack_bf16_hw(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3]);
+                        pf.u[2] = pack_bf16_hw(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1]);
+                        pf.u[3] = pack_bf16_hw(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3]);
+#pragma unroll
+                        for (int tt = 0; tt < 4; ++tt) {
+                            acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pf.b, acc[ht][g * 4 + tt], 0, 0, 0);
+                        }
                     }
                 }
             }
             finish_iteration(i);
         }
-        if (head < p.heads) {
-            float* out = p.partial + rec * kLatent;
 #pragma unroll
-            for (int t = 0; t < 32; ++t) {
-                *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
+        for (int ht = 0; ht < 2; ++ht) {
+            const unsigned int out_head = blockIdx.y * 64u + (2u * hp + ht) * 16u + m;
+            if (out_head < p.heads) {
+                float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + dh * 256u;
+#pragma unroll
+                for (int t = 0; t < 16; ++t) {
+                    *(f32x4*)(out + t * 16 + 4 * j) = acc[ht][t];
+                }
             }
         }
     }
