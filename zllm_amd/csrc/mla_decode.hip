@@ -817,12 +817,17 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                     s16x4 s[2];
                     bf16x8 b;
                 };
+                // The transposed reads are written as inline assembly: through the builtin the compiler cannot tell
+                // that they never touch the raw area the global -> LDS loads fill, and it drains those loads
+                // (s_waitcnt vmcnt(0)) in front of the first read of every step.  The price is that their
+                // completion is waited for by hand (lgkmcnt, LDS operations complete in issue order).
+                const unsigned int tile_lds = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)tile;
                 auto load_group = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
 #pragma unroll
                     for (int tt = 0; tt < 4; ++tt) {
-                        const unsigned char* at = tile + pv_base[tt] + g * 128;
-                        vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-                        vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+                        const unsigned int at = tile_lds + pv_base[tt] + g * 128;
+                        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vf[tt].s[0]) : "v"(at));
+                        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vf[tt].s[1]) : "v"(at), "n"(16 * kRowBytes));
                     }
                 };
                 auto scales_of = [&](int g, f32x4& gs0, f32x4& gs1) __attribute__((always_inline)) {
@@ -840,8 +845,17 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                     if (g + 1 < 4) {
                         load_group(vf[cur ^ 1], g + 1);
                         scales_of(g + 1, gs0[cur ^ 1], gs1[cur ^ 1]);
+                        // group g's eight reads are older than the eight just issued
+                        asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1])
+                                     :
+                                     : "memory");
+                    } else {
+                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1])
+                                     :
+                                     : "memory");
                     }
-                    asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
 #pragma unroll
                     for (int ht = 0; ht < 2; ++ht) {
                         Frag pf; // P'_g = bf16(p * scale_g)
