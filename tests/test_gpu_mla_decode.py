@@ -65,7 +65,10 @@ def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None):
     return out
 
 
-@pytest.mark.parametrize("heads,lens", [(128, [700, 2300]), (16, [100]), (64, [1025, 33]), (32, [1])])
+@pytest.mark.parametrize("heads,lens", [(128, [700, 2300]), (16, [100]), (64, [1025, 33]), (32, [1]),
+                                        # one, two and three 32-token steps exactly and off by one; head counts that leave a
+                                        # value wave with one live head tile (40 = 2.5 tiles) or a partial tile (20)
+                                        (40, [31, 32, 33, 64, 65, 96]), (20, [5, 97])])
 def test_mla_decode_matches_oracle(heads, lens):
     case = make_mla_case(heads + len(lens), lens, heads)
     want_f, want_b = oracle_mla(case)

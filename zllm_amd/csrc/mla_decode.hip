@@ -98,12 +98,6 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 // ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
-// Workgroup = (split, block of 64 heads, sequence) with 4 * NDH waves; wave (hw, dh) owns heads
-// [16 hw, 16 hw + 16) and output columns [512 dh / NDH, 512 (dh + 1) / NDH).
-//   NDH = 1: four waves, one per SIMD with the whole 512-register file: 128 accumulator + 72 query
-//            registers leave room to keep many LDS fragment loads in flight; one barrier per step.
-//   NDH = 2: eight waves; the two waves of a head tile split the score work by token tile and exchange
-//            16 x 16 score tiles through LDS (two barriers per step).
 // Workgroup barrier for LDS traffic only.  __syncthreads() also fences the global -> LDS loads in flight
 // (s_waitcnt vmcnt(0)), which would drain the prefetch of the next step at every barrier; the data those
 // loads bring is consumed by the issuing thread alone, after its own explicit wait.
@@ -127,374 +121,19 @@ struct StepRows {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
-template <int NDH>
-__global__ __launch_bounds__(256 * NDH) void mla_partial(MlaDecodeParams p)
-{
-    constexpr int ITEMS = 4 / NDH;      // staging items per thread
-    constexpr int TROWS = 8 * NDH;      // token rows covered by one pass of the threads
-    constexpr int MT = 32 / NDH;        // output M tiles (16 latent columns each) of this wave
-    constexpr int GROUPS = 8 / NDH;     // scale groups among them
-    constexpr int TILES = NDH == 1 ? 2 : 1; // token tiles this wave scores itself
-    constexpr int KSPLIT = NDH == 4 ? 2 : 1; // waves that share one token tile's dot products (by column half)
-    constexpr int QF = 18 / KSPLIT;          // query k-steps held by this wave
-    __shared__ __align__(16) unsigned char lds[2 * kTileBytes];
-    __shared__ __align__(16) float lds_scale[2][8][kStepTokens]; // [buffer][group][token]
-    // raw bytes of the next step, written by global -> LDS loads (no registers held across the MFMA work)
-    __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
-    __shared__ __align__(16) float lds_s[NDH >= 2 ? 4 : 1][2][KSPLIT][16][16]; // [head tile][token tile][column half][token][head]
-    const unsigned int tid = threadIdx.x;
-    const unsigned int lane = tid & 63u;
-    const unsigned int wave = tid >> 6;
-    const unsigned int hw = wave / NDH;
-    const unsigned int dh = wave % NDH;
-    const unsigned int ti = NDH == 4 ? dh >> 1 : dh; // token tile this wave scores (NDH >= 2)
-    const unsigned int kh = NDH == 4 ? dh & 1u : 0u; // column half of the dot products it computes
-    const unsigned int m = lane & 15u;
-    const unsigned int j = lane >> 4;
-    const unsigned int chunk = blockIdx.x;
-    const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
-    const unsigned int b = blockIdx.z;
-    const unsigned int len = p.ctx_lens[b];
-    const unsigned long long c_start64 = (unsigned long long)chunk * p.chunk_tokens;
-    const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
-
-    if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
-        if (head < p.heads && j == 0 && dh == 0) {
-            p.stats[rec * 2] = kNegInf;
-            p.stats[rec * 2 + 1] = 0.0f;
-        }
-        return;
-    }
-    const unsigned int c_start = (unsigned int)c_start64;
-    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
-    const unsigned int steps = (c_end - c_start + kStepTokens - 1) / kStepTokens;
-
-    // ---- Q fragments (B operand): lane = (head column m, k-slice j); k-step ks covers dims
-    //      ks*32 + j*8 .. +8 of the 576-wide absorbed query ------------------------------------
-    // With KSPLIT = 2 a wave keeps the k-steps of its column half only: latent groups 4 kh .. 4 kh + 3
-    // (k-steps 8 kh .. 8 kh + 7) in qf[0..7] and rope k-step 16 + kh in qf[8].
-    Frag qf[QF];
-    {
-        const unsigned short* qa = p.absorbed + ((size_t)b * p.heads + min(head, p.heads - 1u)) * kRowElems;
-#pragma unroll
-        for (int q = 0; q < QF; ++q) {
-            const unsigned int ks = KSPLIT == 1 ? (unsigned int)q : (q < 8 ? 8u * kh + q : 16u + kh);
-            u32x4 v = *(const u32x4*)(qa + ks * 32 + j * 8);
-            if (head >= p.heads) {
-                v = u32x4{0u, 0u, 0u, 0u};
-            }
-            qf[q].u = v;
-        }
-    }
-
-    const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
-    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
-
-    // Cooperative staging, in two halves.
-    //   issue_step:   every thread starts global -> LDS loads of its raw items of the NEXT step: item i = 16 codes
-    //                 of token (tid >> 5) + TROWS * i, chunk cc = tid & 31; threads 0..255 also one 16-byte rope
-    //                 chunk (token tid >> 3); threads 256..287 the eight scales of token tid - 256.
-    //   convert_step: after the MFMA work each thread waits for ITS OWN loads (issued a whole step earlier),
-    //                 reads its raw items back and writes them into the bf16 tile / f32 scale table.
-    // A thread only ever reads raw bytes it loaded itself, so no barrier sits between the two halves.
-    const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const unsigned int cc = tid & 31u;
-    const unsigned int t_lo = tid >> 5;
-    const unsigned int rope_t = (tid >> 3) & 31u;
-    const unsigned int rope_c = tid & 7u;
-    const bool has_rope = tid < 256u;
-    const bool has_scales = tid >= 256u && tid < 256u + kStepTokens;
-    const unsigned int extra_t = has_rope ? rope_t : (tid - 256u) & 31u; // token of the rope / scale item
-    unsigned char* const raw_codes = lds_raw;
-    unsigned char* const raw_rope = lds_raw + kRawCodes;
-    unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
-    auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i <= ITEMS; ++i) {
-            const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
-            const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
-            r.entry[i] = table != nullptr ? table[page] : page;
-        }
-    };
-    auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
-        const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
-        if (pow2) {
-            return ((unsigned long long)r.entry[i] << p.block_shift) + (token & (p.block_tokens - 1u));
-        }
-        return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
-    };
-    auto issue_step = [&](const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            // the wave's 64 lanes cover token rows 2 * wave and 2 * wave + 1 (+ TROWS * i): 1 KiB, contiguous in LDS
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
-                                             (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
-        }
-        if (has_rope) { // waves 0..3: token rows 8 * wave .. + 8 of the rope plane, 128 B each
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
-                                             (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
-        }
-        if (has_scales) { // wave 4, lanes 0..31: the 16 bytes of scales of one token each
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
-                                             (lds_ptr_t)(raw_scales), 16, 0, 0);
-        }
-    };
-    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's raw items have landed
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            // the thread converts codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row: 32 consecutive lanes then
-            // write 512 contiguous bytes per instruction (chunks cc and cc + 32), which the LDS takes without conflicts
-            const unsigned int row = t_lo + TROWS * i;
-            const u32x2 half[2] = {*(const u32x2*)(raw_codes + row * kLatent + cc * 8u),
-                                   *(const u32x2*)(raw_codes + row * kLatent + 256u + cc * 8u)};
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                u32x4 out;
-#pragma unroll
-                for (int w = 0; w < 2; ++w) {
-                    const unsigned int word = half[h][w];
-                    const float c0 = (float)(int)(signed char)(word & 0xffu);
-                    const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
-                    const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
-                    const float c3 = (float)(int)(signed char)(word >> 24);
-                    out[w * 2] = pack_bf16_trunc(c0, c1);
-                    out[w * 2 + 1] = pack_bf16_trunc(c2, c3);
-                }
-                *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
-            }
-        }
-        if (has_rope) {
-            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = *(const u32x4*)(raw_rope + tid * 16u);
-        }
-        if (has_scales) {
-            const u32x4 sc8 = *(const u32x4*)(raw_scales + (tid - 256u) * 16u);
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                const unsigned int word = sc8[g >> 1];
-                scale_tile[g][tid - 256u] = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // raw bytes are in registers before the next loads overwrite them
-    };
-
-    f32x4 acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    float run_max = kNegInf, run_sum = 0.0f;
-    const float scale_log2 = p.score_scale * kLog2e;
-
-    // LDS byte offsets of this lane's fragments, split into a lane part and a compile-time part so
-    // that every read is `base + immediate`:  chunk = (hi << 3) | lo, and only `lo` meets the swizzle.
-    const unsigned int qk_row = (NDH >= 2 ? ti * 16u : 0u) + m;
-    const unsigned int qk_base[2] = {qk_row * kRowBytes + ((j ^ swz(m)) << 4), qk_row * kRowBytes + (((4u | j) ^ swz(m)) << 4)};
-    const unsigned int tr_row = 4u * j + (m >> 2);
-    unsigned int pv_base[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u +
-                     dh * GROUPS * 128u;
-    }
-
-    auto compute_step = [&](const unsigned char* tile, const float (*scale_tile)[kStepTokens], unsigned int t0) __attribute__((always_inline)) {
-        // ---- scores: S^T = sum_g scale_g * (codes_g . qa_g) + rope . q_rope ------------------------------
-        float sc[8];
-#pragma unroll
-        for (int i = 0; i < TILES; ++i) {
-            const unsigned int tile_i = NDH >= 2 ? ti : (unsigned int)i;          // token tile scored here
-            const unsigned char* kt = tile + (NDH >= 2 ? 0 : i * 16 * kRowBytes); // qk_base already holds ti
-            f32x4 s = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (KSPLIT == 1) {
-#pragma unroll
-                for (int ks = 16; ks < 18; ++ks) { // rope columns: unscaled
-                    Frag kf;
-                    kf.u = *(const u32x4*)(kt + qk_base[ks & 1] + (ks >> 1) * 128);
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[ks].b, s, 0, 0, 0);
-                }
-            } else {
-                Frag kf; // rope k-step 16 + kh
-                kf.u = *(const u32x4*)(kt + (kh == 0 ? qk_base[0] : qk_base[1]) + 8 * 128);
-                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.b, qf[8].b, s, 0, 0, 0);
-            }
-#pragma unroll
-            for (int half = 0; half < 2 / KSPLIT; ++half) { // four independent accumulators at a time: no MFMA -> MFMA stalls
-                f32x4 d[4];
-                const unsigned int g0 = KSPLIT == 1 ? half * 4u : kh * 4u; // first scale group of this batch
-                const int q0 = KSPLIT == 1 ? half * 8 : 0;                 // its first query k-step
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    Frag k0;
-                    k0.u = *(const u32x4*)(kt + qk_base[0] + (g0 + u) * 128);
-                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[q0 + 2 * u].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    Frag k1;
-                    k1.u = *(const u32x4*)(kt + qk_base[1] + (g0 + u) * 128);
-                    d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[q0 + 2 * u + 1].b, d[u], 0, 0, 0);
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const f32x4 gs = *(const f32x4*)(&scale_tile[g0 + u][tile_i * 16 + 4 * j]); // one address per 16-lane group
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        s[r] = fmaf(d[u][r], gs[r], s[r]);
-                    }
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if constexpr (NDH >= 2) {
-                    sc[r] = s[r]; // partial or whole dot of (token 16 ti + 4 j + r, head m): exchanged below
-                } else {
-                    const unsigned int token = t0 + 16u * tile_i + 4u * j + r;
-                    sc[i * 4 + r] = token < len ? s[r] * scale_log2 : kNegInf;
-                }
-            }
-        }
-        if constexpr (NDH >= 2) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                lds_s[hw][ti][kh][4 * j + r][m] = sc[r];
-            }
-            lds_barrier();
-            // every wave of the head tile rebuilds the same 32 scores in the same order
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float x = lds_s[hw][t2][0][4 * j + r][m];
-                    if constexpr (KSPLIT == 2) {
-                        x += lds_s[hw][t2][1][4 * j + r][m];
-                    }
-                    const unsigned int token = t0 + 16u * t2 + 4u * j + r;
-                    sc[t2 * 4 + r] = token < len ? x * scale_log2 : kNegInf;
-                }
-            }
-        }
-        // ---- online softmax for this head column ---------------------------------------------------------
-        float step_max = sc[0];
-#pragma unroll
-        for (int e = 1; e < 8; ++e) {
-            step_max = fmaxf(step_max, sc[e]);
-        }
-        step_max = wave_max_16x4(step_max);
-        // lazy rescaling: the stored maximum only moves when a score exceeds it by 2^8 (p stays <= 256)
-        float new_max = run_max;
-        if (step_max > run_max + 8.0f || run_max == kNegInf) {
-            new_max = fmaxf(run_max, step_max);
-        }
-        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-        const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);
-        float pr[8];
-        float step_sum = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            pr[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
-            step_sum += pr[e];
-        }
-        const bool had_mass = run_sum != 0.0f; // nothing accumulated yet -> nothing to rescale
-        run_sum = run_sum * alpha + step_sum;
-        run_max = new_max;
-        __builtin_amdgcn_sched_barrier(0); // keep the (rare) rescale at a point of low register pressure
-        if (__any(alpha != 1.0f && had_mass)) {
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[t] *= alpha;
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- O^T += codes^T . P'_g,  P'_g = bf16(p * scale_g), for this wave's scale groups ----------------
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-            const float* gs_row = scale_tile[dh * GROUPS + g];
-            const f32x4 gs0 = *(const f32x4*)(gs_row + 4 * j);
-            const f32x4 gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
-            Frag pf;
-            pf.u[0] = pack_bf16_hw(pr[0] * gs0[0], pr[1] * gs0[1]);
-            pf.u[1] = pack_bf16_hw(pr[2] * gs0[2], pr[3] * gs0[3]);
-            pf.u[2] = pack_bf16_hw(pr[4] * gs1[0], pr[5] * gs1[1]);
-            pf.u[3] = pack_bf16_hw(pr[6] * gs1[2], pr[7] * gs1[3]);
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
-                const unsigned char* at = tile + pv_base[tt] + g * 128;
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
-                union {
-                    s16x4 s[2];
-                    bf16x8 b;
-                } vf;
-                vf.s[0] = lo;
-                vf.s[1] = hi;
-                acc[g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, pf.b, acc[g * 4 + tt], 0, 0, 0);
-            }
-        }
-    };
-
-    // ---- pipeline: table lookups run two steps ahead, global loads one step ahead of the MFMA work;
-    //      LDS tile double-buffered ---------------------------------------------------------------------
-    StepRows rows;
-    lookup_step(rows, c_start);
-    issue_step(rows, c_start);
-    if (steps > 1) {
-        lookup_step(rows, c_start + kStepTokens);
-    }
-    convert_step(lds, lds_scale[0]);
-    lds_barrier();
-    for (unsigned int step = 0; step < steps; ++step) {
-        unsigned char* cur = lds + (step & 1u) * kTileBytes;
-        unsigned char* nxt = lds + ((step + 1u) & 1u) * kTileBytes;
-        const bool more = step + 1 < steps;
-        if (more) {
-            // place the wait for the block-table entries (fetched a step ago) before this step's first load
-#pragma unroll
-            for (int i = 0; i <= ITEMS; ++i) {
-                asm volatile("" : "+v"(rows.entry[i]));
-            }
-            issue_step(rows, c_start + (step + 1u) * kStepTokens);
-            if (step + 2 < steps) {
-                lookup_step(rows, c_start + (step + 2u) * kStepTokens);
-            }
-        }
-        compute_step(cur, lds_scale[step & 1u], c_start + step * kStepTokens);
-        if (more) {
-            convert_step(nxt, lds_scale[(step + 1u) & 1u]);
-        }
-        lds_barrier();
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no load may still target this workgroup's LDS at exit
-
-    // ---- write un-normalised partials and (max, sum) -------------------------------------------
-    const float total = wave_sum_16x4(run_sum);
-    if (head < p.heads) {
-        if (j == 0 && dh == 0) {
-            p.stats[rec * 2] = run_max;
-            p.stats[rec * 2 + 1] = total;
-        }
-        float* out = p.partial + rec * kLatent + dh * (MT * 16u);
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            *(f32x4*)(out + t * 16 + 4 * j) = acc[t];
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// 2b. split-KV partial, role-specialised waves
-// ---------------------------------------------------------------------------------------------
 // Workgroup = (split, block of 64 heads, sequence), eight waves in two roles that run one step apart:
 //   score waves (0..3, 16 heads each): S^T = K.Q^T for all 32 tokens of tile i, online softmax, and hand
 //       the step's probabilities p[32 tokens] and the rescale factor alpha to their value wave through LDS.
 //       The C layout of S^T is the B layout the value wave needs, so the hand-over is lane to lane.
-//   value waves (4..7, the same 16 heads, all 512 output columns): O^T += V^T.P' for tile i - 1.
+//   value waves (4..7): O^T += V^T.P' for tile i - 1; each owns two head tiles x 256 output columns, so that
+//       every V^T fragment read from LDS feeds two MFMAs.
 // The score work is LDS reads + vector ALU (exp, max), the value work LDS reads + MFMA; with one wave of each
 // role per SIMD the two overlap instead of every wave running the same phase at the same time, and the
 // score exchange between waves of a head tile (a second barrier per step) disappears.  Three tile buffers
 // rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the raw bytes that the
 // global -> LDS loads of the previous iteration brought in).  One LDS-only barrier per step.
 constexpr int kWsTiles = 3;
+constexpr float kLoThreshold = 64.0f; // a probability above 1/64 of its lane's running sum counts as heavy
 
 __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
@@ -505,6 +144,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
     __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
+    __shared__ unsigned int lds_heavy[2][4];             // [parity][head tile]: the step needs the low-order P' term
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
@@ -757,10 +397,17 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 }
                 run_sum = run_sum * alpha + step_sum;
                 run_max = new_max;
+                // P' is one bf16 term (2^-9 relative rounding, random sign) unless some probability of the step is
+                // heavy against its lane's running sum: then the value wave adds the low-order term as well
+                const float p_top = fmaxf(fmaxf(fmaxf(p_lo[0], p_lo[1]), fmaxf(p_lo[2], p_lo[3])), fmaxf(fmaxf(p_hi[0], p_hi[1]), fmaxf(p_hi[2], p_hi[3])));
+                const bool heavy = __any(p_top * kLoThreshold > run_sum);
                 float* slot = lds_p[i & 1u][hw][lane];
                 *(f32x4*)(slot) = p_lo;
                 *(f32x4*)(slot + 4) = p_hi;
                 lds_alpha[i & 1u][hw][lane] = alpha;
+                if (lane == 0) {
+                    lds_heavy[i & 1u][hw] = heavy ? 1u : 0u;
+                }
             }
             finish_iteration(i);
         }
@@ -795,6 +442,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 p_hi[ht] = *(const f32x4*)(slot + 4);
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
+            const bool lo_pass[2] = {lds_heavy[(i + 1u) & 1u][2u * hp] != 0u, lds_heavy[(i + 1u) & 1u][2u * hp + 1u] != 0u};
             asm volatile("" ::: "memory");
             stage_next(i);
             if (i > 0) {
@@ -866,6 +514,19 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 #pragma unroll
                         for (int tt = 0; tt < 4; ++tt) {
                             acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pf.b, acc[ht][g * 4 + tt], 0, 0, 0);
+                        }
+                        if (lo_pass[ht]) { // low-order term: bf16(x - bf16(x))
+                            Frag pl;
+                            unsigned int hi_bits, lo_bits[4];
+                            split_bf16_pair(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1], hi_bits, lo_bits[0]);
+                            split_bf16_pair(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3], hi_bits, lo_bits[1]);
+                            split_bf16_pair(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1], hi_bits, lo_bits[2]);
+                            split_bf16_pair(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3], hi_bits, lo_bits[3]);
+                            pl.u = u32x4{lo_bits[0], lo_bits[1], lo_bits[2], lo_bits[3]};
+#pragma unroll
+                            for (int tt = 0; tt < 4; ++tt) {
+                                acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pl.b, acc[ht][g * 4 + tt], 0, 0, 0);
+                            }
                         }
                     }
                 }
