@@ -4,15 +4,16 @@
 // src/kernel/rocm/hip/attention/paged_mla.rs:3042-3621):
 //   1. mla_absorb:  qa[b, h, 0:512] = bf16(q_nope[b, h, :] . W_kv_b[h, 0:nope, :]),
 //                   qa[b, h, 512:576] = bf16(q_rope[b, h, :])
-//   2. mla_partial: split-KV attention of 128 heads against one shared latent row per token.
-//                   A workgroup owns (split, sequence).  Per 32-token step it converts the latent
-//                   codes ONCE into LDS as bf16 integers (exact) next to the bf16 rope columns and
-//                   the f32 group scales; its four waves (32 heads each) then run
+//   2. mla_partial_ws: split-KV attention of the heads against one shared latent row per token.
+//                   A workgroup owns (split, block of 64 heads, sequence).  Per 32-token step it converts
+//                   the latent codes ONCE into LDS as bf16 integers (exact) next to the bf16 rope columns
+//                   and the f32 group scales.  Four score waves (16 heads each) compute
 //                     S^T[token, head]  = sum_g scale[token, g] * (codes_g[token, :] . qa_g[head, :])
 //                                         + rope[token, :] . q_rope[head, :]     (MFMA 16x16x32 bf16,
 //                                         one accumulator per 64-column group: products are exact)
-//                     online softmax (wave shuffles)
+//                   and the online softmax; four value waves, one step behind, accumulate
 //                     O^T[dim, head]   += codes^T[dim, token] . P'_g[token, head], P'_g = bf16(p * scale_g)
+//                   (plus the low-order half of P'_g when a probability is heavy against the running sum).
 //                   The same row-major tile feeds both products: QK^T reads it with ds_read_b128,
 //                   P.V reads it transposed with ds_read_b64_tr_b16.  A 16-byte XOR swizzle keeps both
 //                   access patterns free of bank conflicts.
