@@ -13,7 +13,6 @@
 //                                         one accumulator per 64-column group: products are exact)
 //                   and the online softmax; four value waves, one step behind, accumulate
 //                     O^T[dim, head]   += codes^T[dim, token] . P'_g[token, head], P'_g = bf16(p * scale_g)
-//                   (plus the low-order half of P'_g when a probability is heavy against the running sum).
 //                   The same row-major tile feeds both products: QK^T reads it with ds_read_b128,
 //                   P.V reads it transposed with ds_read_b64_tr_b16.  A 16-byte XOR swizzle keeps both
 //                   access patterns free of bank conflicts.
@@ -45,7 +44,28 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 union Frag {
     u32x4 u;
     bf16x8 b;
+    f16x8 h;
 };
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// two f32 -> packed f16, round to nearest even (v_cvt_pk_f16_f32)
+__device__ __forceinline__ unsigned int pack_f16_hw(float lo, float hi)
+{
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f32x2{lo, hi}, f16x2));
+}
+
+// Four int8 codes of a word -> four f16 integers (exact), 5 instructions: flipping the sign bits turns a code c
+// into the unsigned byte c + 128; placed under the exponent byte 0x64 it reads as the f16 number 1024 + 128 + c,
+// and one packed subtraction removes the offset.
+__device__ __forceinline__ void codes4_to_f16(unsigned int word, unsigned int& lo, unsigned int& hi)
+{
+    const unsigned int biased = word ^ 0x80808080u;
+    const f16x2 offset = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    lo = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) + offset);
+    hi = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) + offset);
+}
 
 // Chunk swizzle for the 64-bank LDS (256 B per cycle).  A tile row is 72 chunks of 16 B, i.e. 8 chunks past a
 // multiple of 256 B, so the row's parity already selects the upper or lower 128 B of a bank line; XOR-ing
@@ -134,7 +154,6 @@ typedef const __attribute__((address_space(1))) void* global_ptr_t;
 // rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the raw bytes that the
 // global -> LDS loads of the previous iteration brought in).  One LDS-only barrier per step.
 constexpr int kWsTiles = 3;
-constexpr float kLoThreshold = 64.0f; // a probability above 1/64 of its lane's running sum counts as heavy
 
 __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
@@ -145,7 +164,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
     __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
-    __shared__ unsigned int lds_heavy[2][4];             // [parity][head tile]: the step needs the low-order P' term
+    __shared__ float lds_top[kWsTiles];                  // [buffer]: largest group scale of the tile
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
@@ -214,7 +233,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                                              (lds_ptr_t)(raw_scales), 16, 0, 0);
         }
     };
-    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens]) __attribute__((always_inline)) {
+    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
@@ -228,13 +247,10 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 u32x4 out;
 #pragma unroll
                 for (int w = 0; w < 2; ++w) {
-                    const unsigned int word = half[h][w];
-                    const float c0 = (float)(int)(signed char)(word & 0xffu);
-                    const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
-                    const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
-                    const float c3 = (float)(int)(signed char)(word >> 24);
-                    out[w * 2] = pack_bf16_trunc(c0, c1);
-                    out[w * 2 + 1] = pack_bf16_trunc(c2, c3);
+                    unsigned int pair_lo, pair_hi;
+                    codes4_to_f16(half[h][w], pair_lo, pair_hi);
+                    out[w * 2] = pair_lo;
+                    out[w * 2 + 1] = pair_hi;
                 }
                 *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
             }
@@ -244,10 +260,24 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
         }
         if (has_scales) {
             const u32x4 sc8 = *(const u32x4*)(raw_scales + (tid - 256u) * 16u);
+            float top = 0.0f;
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 const unsigned int word = sc8[g >> 1];
-                scale_tile[g][tid - 256u] = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+                const float sg = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+                scale_tile[g][tid - 256u] = sg;
+                top = fmaxf(top, sg);
+            }
+            // largest scale of the step, for the value waves' exponent window: lanes 0..31 of wave 4 hold one token
+            // each; rotate-and-max inside the two 16-lane rows, then one lane of each row
+            top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x128, 0xf, 0xf, false))); // row_ror:8
+            top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x124, 0xf, 0xf, false))); // row_ror:4
+            top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x122, 0xf, 0xf, false))); // row_ror:2
+            top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x121, 0xf, 0xf, false))); // row_ror:1
+            const float both = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
+                                     __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 16)));
+            if (tid == 256u) {
+                *step_top = both;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -268,7 +298,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    convert_step(lds, lds_scale[0]);
+    convert_step(lds, lds_scale[0], &lds_top[0]);
     lds_barrier();
 
     // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile i - 1.
@@ -287,14 +317,19 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     auto finish_iteration = [&](unsigned int i) __attribute__((always_inline)) {
         if (i + 1 < steps) {
             const unsigned int nb = (i + 1u) % kWsTiles;
-            convert_step(lds + nb * kTileBytes, lds_scale[nb]);
+            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb]);
         }
         lds_barrier();
     };
 
     if (!value_role) {
         // ================================ score waves ================================
-        Frag qf[18]; // B operand: lane = (head column m, k-slice j); k-step ks covers dims ks*32 + j*8 .. +8
+        // B operand: lane = (head column m, k-slice j); k-step ks covers dims ks*32 + j*8 .. +8.  The latent part
+        // multiplies f16 codes, so the absorbed query (bf16) is carried as f16 after dividing the head's row by the
+        // power of two of its largest magnitude: exact for every element within 2^-14 of that magnitude, and free
+        // of f16's range limit.  The rope part stays bf16 on both sides.
+        Frag qf[18];
+        float head_pow2 = 1.0f; // the power of two taken out of this head's latent query
         {
             const unsigned short* qa = p.absorbed + ((size_t)b * p.heads + min(head, p.heads - 1u)) * kRowElems;
 #pragma unroll
@@ -305,9 +340,30 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 }
                 qf[ks].u = v;
             }
+            float top = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 16; ++ks) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    top = fmaxf(top, fmaxf(fabsf(__uint_as_float(qf[ks].u[w] << 16)), fabsf(__uint_as_float(qf[ks].u[w] & 0xffff0000u))));
+                }
+            }
+            top = wave_max_16x4(top);
+            const unsigned int top_exp = min(max((__float_as_uint(top) >> 23) & 0xffu, 1u), 253u);
+            head_pow2 = __uint_as_float(top_exp << 23);
+            const float down = __uint_as_float((254u - top_exp) << 23);
+#pragma unroll
+            for (int ks = 0; ks < 16; ++ks) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const unsigned int word = qf[ks].u[w];
+                    qf[ks].u[w] = pack_f16_hw(__uint_as_float(word << 16) * down, __uint_as_float(word & 0xffff0000u) * down);
+                }
+            }
         }
         float run_max = kNegInf, run_sum = 0.0f;
         const float scale_log2 = p.score_scale * kLog2e;
+        const float latent_log2 = scale_log2 * head_pow2;
         for (unsigned int i = 0; i <= steps; ++i) {
             stage_next(i);
             if (i < steps) {
@@ -330,7 +386,8 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) {
                     const unsigned char* kt = tile + t2 * 16 * kRowBytes;
-                    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 s = {0.f, 0.f, 0.f, 0.f};      // latent part, in units of head_pow2
+                    f32x4 s_rope = {0.f, 0.f, 0.f, 0.f}; // rope part
                     kr[0].u = *(const u32x4*)(kt + qk_base[0] + 8 * 128);
                     kr[1].u = *(const u32x4*)(kt + qk_base[1] + 8 * 128);
                     f32x4 d[4];
@@ -344,16 +401,16 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                         }
                         asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
                         if (q == 0) {
-                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[0].b, qf[16].b, s, 0, 0, 0);
-                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[1].b, qf[17].b, s, 0, 0, 0);
+                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[0].b, qf[16].b, s_rope, 0, 0, 0);
+                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[1].b, qf[17].b, s_rope, 0, 0, 0);
                         }
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
                             const int g = (q >> 1) * 4 + u;
                             if ((q & 1) == 0) {
-                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[cur][u].b, qf[2 * g].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[cur][u].h, qf[2 * g].h, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                             } else {
-                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[cur][u].b, qf[2 * g + 1].b, d[u], 0, 0, 0);
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[cur][u].h, qf[2 * g + 1].h, d[u], 0, 0, 0);
                             }
                         }
                         if ((q & 1) == 1) {
@@ -371,7 +428,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const unsigned int token = t0 + 16u * t2 + 4u * j + r;
-                        sc[t2 * 4 + r] = token < len ? s[r] * scale_log2 : kNegInf;
+                        sc[t2 * 4 + r] = token < len ? fmaf(s[r], latent_log2, s_rope[r] * scale_log2) : kNegInf;
                     }
                 }
                 // online softmax for this head column; lazy rescaling: the stored maximum only moves when a
@@ -398,17 +455,10 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 }
                 run_sum = run_sum * alpha + step_sum;
                 run_max = new_max;
-                // P' is one bf16 term (2^-9 relative rounding, random sign) unless some probability of the step is
-                // heavy against its lane's running sum: then the value wave adds the low-order term as well
-                const float p_top = fmaxf(fmaxf(fmaxf(p_lo[0], p_lo[1]), fmaxf(p_lo[2], p_lo[3])), fmaxf(fmaxf(p_hi[0], p_hi[1]), fmaxf(p_hi[2], p_hi[3])));
-                const bool heavy = __any(p_top * kLoThreshold > run_sum);
                 float* slot = lds_p[i & 1u][hw][lane];
                 *(f32x4*)(slot) = p_lo;
                 *(f32x4*)(slot + 4) = p_hi;
                 lds_alpha[i & 1u][hw][lane] = alpha;
-                if (lane == 0) {
-                    lds_heavy[i & 1u][hw] = heavy ? 1u : 0u;
-                }
             }
             finish_iteration(i);
         }
@@ -432,6 +482,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 acc[ht][t] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
+        int window = 0;
         for (unsigned int i = 0; i <= steps; ++i) {
             // the hand-over records are requested first: their LDS round trip hides behind the staging work
             f32x4 p_lo[2], p_hi[2];
@@ -443,13 +494,34 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 p_hi[ht] = *(const f32x4*)(slot + 4);
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
-            const bool lo_pass[2] = {lds_heavy[(i + 1u) & 1u][2u * hp] != 0u, lds_heavy[(i + 1u) & 1u][2u * hp + 1u] != 0u};
+            const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[(i + 2u) % kWsTiles])); // tile i - 1
             asm volatile("" ::: "memory");
             stage_next(i);
             if (i > 0) {
                 const unsigned int tb = (i - 1u) % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
                 const float (*scale_tile)[kStepTokens] = lds_scale[tb] + dh * 4u;
+                // exponent window of P': the accumulators hold sum(P' c) / 2^window with 2^window above the
+                // largest scale seen / 2^7, so p (<= 2^8) * scale / 2^window stays below 2^15; the window only
+                // grows, and the accumulators are rescaled by the power of two it grows by
+                {
+                    const int top_exp = (int)((top_bits >> 23) & 0xffu);
+                    const int need = min(max(top_exp - 133, -96), 112);
+                    if (i == 1u) {
+                        window = need;
+                    } else if (need > window) {
+                        const float shrink = __uint_as_float((unsigned int)(127 - min(need - window, 126)) << 23);
+                        alpha[0] *= shrink;
+                        alpha[1] *= shrink;
+                        window = need;
+                    }
+                    const float into_window = __uint_as_float((unsigned int)(127 - window) << 23);
+#pragma unroll
+                    for (int ht = 0; ht < 2; ++ht) {
+                        p_lo[ht] *= into_window;
+                        p_hi[ht] *= into_window;
+                    }
+                }
 #pragma unroll
                 for (int ht = 0; ht < 2; ++ht) {
                     if (__any(alpha[ht] != 1.0f)) {
@@ -464,7 +536,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 // reads in program order behind each MFMA the wave pays one LDS round trip per tile.
                 union VFrag {
                     s16x4 s[2];
-                    bf16x8 b;
+                    f16x8 h;
                 };
                 // The transposed reads are written as inline assembly: through the builtin the compiler cannot tell
                 // that they never touch the raw area the global -> LDS loads fill, and it drains those loads
@@ -507,27 +579,14 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                     }
 #pragma unroll
                     for (int ht = 0; ht < 2; ++ht) {
-                        Frag pf; // P'_g = bf16(p * scale_g)
-                        pf.u[0] = pack_bf16_hw(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1]);
-                        pf.u[1] = pack_bf16_hw(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3]);
-                        pf.u[2] = pack_bf16_hw(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1]);
-                        pf.u[3] = pack_bf16_hw(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3]);
+                        Frag pf; // P'_g = f16(p * scale_g / 2^window): 2^-12 relative rounding
+                        pf.u[0] = pack_f16_hw(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1]);
+                        pf.u[1] = pack_f16_hw(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3]);
+                        pf.u[2] = pack_f16_hw(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1]);
+                        pf.u[3] = pack_f16_hw(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3]);
 #pragma unroll
                         for (int tt = 0; tt < 4; ++tt) {
-                            acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pf.b, acc[ht][g * 4 + tt], 0, 0, 0);
-                        }
-                        if (lo_pass[ht]) { // low-order term: bf16(x - bf16(x))
-                            Frag pl;
-                            unsigned int hi_bits, lo_bits[4];
-                            split_bf16_pair(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1], hi_bits, lo_bits[0]);
-                            split_bf16_pair(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3], hi_bits, lo_bits[1]);
-                            split_bf16_pair(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1], hi_bits, lo_bits[2]);
-                            split_bf16_pair(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3], hi_bits, lo_bits[3]);
-                            pl.u = u32x4{lo_bits[0], lo_bits[1], lo_bits[2], lo_bits[3]};
-#pragma unroll
-                            for (int tt = 0; tt < 4; ++tt) {
-                                acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[cur][tt].b, pl.b, acc[ht][g * 4 + tt], 0, 0, 0);
-                            }
+                            acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[cur][tt].h, pf.h, acc[ht][g * 4 + tt], 0, 0, 0);
                         }
                     }
                 }
@@ -539,9 +598,10 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
             const unsigned int out_head = blockIdx.y * 64u + (2u * hp + ht) * 16u + m;
             if (out_head < p.heads) {
                 float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + dh * 256u;
+                const float out_of_window = __uint_as_float((unsigned int)(127 + window) << 23);
 #pragma unroll
                 for (int t = 0; t < 16; ++t) {
-                    *(f32x4*)(out + t * 16 + 4 * j) = acc[ht][t];
+                    *(f32x4*)(out + t * 16 + 4 * j) = acc[ht][t] * out_of_window;
                 }
             }
         }
