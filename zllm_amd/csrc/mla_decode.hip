@@ -427,8 +427,14 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                     }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const unsigned int token = t0 + 16u * t2 + 4u * j + r;
-                        sc[t2 * 4 + r] = token < len ? fmaf(s[r], latent_log2, s_rope[r] * scale_log2) : kNegInf;
+                        sc[t2 * 4 + r] = fmaf(s[r], latent_log2, s_rope[r] * scale_log2);
+                    }
+                }
+                if (t0 + kStepTokens > len) { // only the last step of a sequence has tokens to mask
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+                        sc[e] = token < len ? sc[e] : kNegInf;
                     }
                 }
                 // online softmax for this head column; lazy rescaling: the stored maximum only moves when a
@@ -483,6 +489,8 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
             }
         }
         int window = 0;
+        unsigned int value_tile = 0; // buffer of tile i - 1
+        const unsigned int lds_base = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)lds;
         for (unsigned int i = 0; i <= steps; ++i) {
             // the hand-over records are requested first: their LDS round trip hides behind the staging work
             f32x4 p_lo[2], p_hi[2];
@@ -494,13 +502,13 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 p_hi[ht] = *(const f32x4*)(slot + 4);
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
-            const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[(i + 2u) % kWsTiles])); // tile i - 1
+            const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[value_tile])); // tile i - 1
             asm volatile("" ::: "memory");
             stage_next(i);
             if (i > 0) {
-                const unsigned int tb = (i - 1u) % kWsTiles;
-                const unsigned char* tile = lds + tb * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
-                const float (*scale_tile)[kStepTokens] = lds_scale[tb] + dh * 4u;
+                // LDS byte addresses of this step: one register per fragment row, everything else is an immediate
+                const unsigned int tile_lds = lds_base + value_tile * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
+                const float* gs_base = &lds_scale[0][0][0] + value_tile * (8 * kStepTokens) + dh * (4 * kStepTokens) + 4 * j;
                 // exponent window of P': the accumulators hold sum(P' c) / 2^window with 2^window above the
                 // largest scale seen / 2^7, so p (<= 2^8) * scale / 2^window stays below 2^15; the window only
                 // grows, and the accumulators are rescaled by the power of two it grows by
@@ -542,19 +550,17 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                 // that they never touch the raw area the global -> LDS loads fill, and it drains those loads
                 // (s_waitcnt vmcnt(0)) in front of the first read of every step.  The price is that their
                 // completion is waited for by hand (lgkmcnt, LDS operations complete in issue order).
-                const unsigned int tile_lds = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)tile;
+                const unsigned int at[4] = {tile_lds + pv_base[0], tile_lds + pv_base[1], tile_lds + pv_base[2], tile_lds + pv_base[3]};
                 auto load_group = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
 #pragma unroll
                     for (int tt = 0; tt < 4; ++tt) {
-                        const unsigned int at = tile_lds + pv_base[tt] + g * 128;
-                        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vf[tt].s[0]) : "v"(at));
-                        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vf[tt].s[1]) : "v"(at), "n"(16 * kRowBytes));
+                        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vf[tt].s[0]) : "v"(at[tt]), "i"(g * 128));
+                        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vf[tt].s[1]) : "v"(at[tt]), "i"(g * 128 + 16 * kRowBytes));
                     }
                 };
                 auto scales_of = [&](int g, f32x4& gs0, f32x4& gs1) __attribute__((always_inline)) {
-                    const float* gs_row = scale_tile[g];
-                    gs0 = *(const f32x4*)(gs_row + 4 * j);
-                    gs1 = *(const f32x4*)(gs_row + 16 + 4 * j);
+                    gs0 = *(const f32x4*)(gs_base + g * kStepTokens);
+                    gs1 = *(const f32x4*)(gs_base + g * kStepTokens + 16);
                 };
                 VFrag vf[2][4];
                 f32x4 gs0[2], gs1[2];
@@ -590,6 +596,9 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
                         }
                     }
                 }
+            }
+            if (i > 0) {
+                value_tile = value_tile == kWsTiles - 1u ? 0u : value_tile + 1u;
             }
             finish_iteration(i);
         }
