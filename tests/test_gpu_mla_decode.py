@@ -14,13 +14,18 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 
-def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, block_tokens=16, layout="random", w_std=None):
+def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, block_tokens=16, layout="random", w_std=None,
+                  poison=False):
     rng = np.random.default_rng(seed)
     tables, pool_blocks = draw_tables(rng, lens, block_tokens, layout=layout)
     rows = pool_blocks * block_tokens
     codes = np.zeros((rows, latent), dtype=np.int8)
     scales = np.zeros((rows, latent // 64), dtype=np.uint16)
     rope_cache = np.zeros((rows, rope), dtype=np.uint16)
+    if poison:  # rows no sequence has written yet: NaN scales and rope, extreme codes
+        codes[:] = -128
+        scales[:] = 0x7FC0
+        rope_cache[:] = 0x7FC0
     for b, l in enumerate(lens):
         lat = rng.standard_normal((l, latent)).astype(np.float32)
         kr = rng.standard_normal((l, rope)).astype(np.float32)
@@ -111,6 +116,19 @@ def test_mla_page_sizes(block_tokens, layout):
     want_f, _ = oracle_mla(case)
     got = run_mla(case).cpu().numpy()
     assert_attention_close(got, want_f, f"block_tokens={block_tokens}")
+
+
+@pytest.mark.parametrize("block_tokens", [32, 64, 16])
+def test_mla_rows_past_the_end_of_a_page_are_ignored(block_tokens):
+    """A sequence ends in the middle of a page; whatever the rest of the page holds (here NaN scales, NaN rope and
+    the code -128) must not reach the result.  With pages of a multiple of 32 tokens the kernel loads whole
+    32-row steps from a page, so the rows past the end are really read."""
+    lens = [70, 1, 33, 96, 2049]
+    case = make_mla_case(100 + block_tokens, lens, 32, block_tokens=block_tokens, poison=True)
+    want_f, _ = oracle_mla(case)
+    got = run_mla(case).cpu().numpy()
+    assert np.isfinite(got).all()
+    assert_attention_close(got, want_f, f"poisoned tail, block_tokens={block_tokens}")
 
 
 def test_mla_split_invariance_and_zero_query():

@@ -155,7 +155,12 @@ typedef const __attribute__((address_space(1))) void* global_ptr_t;
 // global -> LDS loads of the previous iteration brought in).  One LDS-only barrier per step.
 constexpr int kWsTiles = 3;
 
-__global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
+// ALIGNED: pages hold a multiple of 32 tokens (splits always start at one), so the 32 rows of a step are
+// contiguous in one page: one block-table entry per step, and every global -> LDS load takes a scalar base
+// plus a constant per-lane offset -- no vector address arithmetic in the loop.  Rows past the end of the
+// sequence are then whatever the page holds; their scales are zeroed during conversion and their scores
+// masked, so they contribute exact zeros.
+template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
     constexpr int ITEMS = 2;  // staging items per thread: 32 tokens x 32 code chunks over 512 threads
     constexpr int TROWS = 16; // token rows covered by one pass of the threads
@@ -204,11 +209,16 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     unsigned char* const raw_rope = lds_raw + kRawCodes;
     unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
     auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
+        if constexpr (ALIGNED) {
+            const unsigned int page = pow2 ? t0 >> p.block_shift : t0 / p.block_tokens;
+            r.entry[0] = table != nullptr ? table[page] : page;
+        } else {
 #pragma unroll
-        for (int i = 0; i <= ITEMS; ++i) {
-            const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
-            const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
-            r.entry[i] = table != nullptr ? table[page] : page;
+            for (int i = 0; i <= ITEMS; ++i) {
+                const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+                const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+                r.entry[i] = table != nullptr ? table[page] : page;
+            }
         }
     };
     auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
@@ -219,21 +229,41 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
         return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
     };
     auto issue_step = [&](const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
+        if constexpr (ALIGNED) {
+            const unsigned int entry = __builtin_amdgcn_readfirstlane(rows.entry[0]);
+            const unsigned long long row0 = pow2 ? ((unsigned long long)entry << p.block_shift) + (t0 & (p.block_tokens - 1u))
+                                                 : (unsigned long long)entry * p.block_tokens + t0 % p.block_tokens;
+            const unsigned char* codes = (const unsigned char*)p.latent_codes + (row0 + 2u * wave_u) * kLatent;
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
-                                             (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
-        }
-        if (has_rope) {
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
-                                             (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
-        }
-        if (has_scales) {
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
-                                             (lds_ptr_t)(raw_scales), 16, 0, 0);
+            for (int i = 0; i < ITEMS; ++i) {
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(codes + TROWS * i * kLatent + lane * 16u),
+                                                 (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
+            }
+            if (has_rope) {
+                const unsigned char* rope = (const unsigned char*)p.rope_cache + row0 * (kRope * 2) + wave_u * 1024u;
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(rope + lane * 16u), (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+            }
+            if (has_scales) {
+                const unsigned char* scales = (const unsigned char*)p.latent_scales + row0 * (kLatent / 64 * 2);
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(scales + lane * 16u), (lds_ptr_t)(raw_scales), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
+                                                 (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
+            }
+            if (has_rope) {
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
+                                                 (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+            }
+            if (has_scales) {
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
+                                                 (lds_ptr_t)(raw_scales), 16, 0, 0);
+            }
         }
     };
-    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top) __attribute__((always_inline)) {
+    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top, unsigned int t0) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
@@ -264,7 +294,10 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 const unsigned int word = sc8[g >> 1];
-                const float sg = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+                float sg = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
+                if (t0 + (tid - 256u) >= len) {
+                    sg = 0.0f; // a row past the end: its codes may be anything, its weight is an exact zero
+                }
                 scale_tile[g][tid - 256u] = sg;
                 top = fmaxf(top, sg);
             }
@@ -298,7 +331,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    convert_step(lds, lds_scale[0], &lds_top[0]);
+    convert_step(lds, lds_scale[0], &lds_top[0], c_start);
     lds_barrier();
 
     // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile i - 1.
@@ -307,7 +340,11 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
             // The entries were fetched an iteration ago.  Naming them here places the compiler's wait for them
             // before the first load of this iteration; left to itself it waits again before every address it
             // forms from them, i.e. for the load it has just issued.
-            asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]));
+            if constexpr (ALIGNED) {
+                asm volatile("" : "+v"(rows.entry[0]));
+            } else {
+                asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]));
+            }
             issue_step(rows, c_start + (i + 1u) * kStepTokens);
             if (i + 2 < steps) {
                 lookup_step(rows, c_start + (i + 2u) * kStepTokens);
@@ -317,7 +354,7 @@ __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
     auto finish_iteration = [&](unsigned int i) __attribute__((always_inline)) {
         if (i + 1 < steps) {
             const unsigned int nb = (i + 1u) % kWsTiles;
-            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb]);
+            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + (i + 1u) * kStepTokens);
         }
         lds_barrier();
     };
@@ -692,7 +729,12 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     }
     if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
-        mla_partial_ws<<<dim3(p.max_chunks, (p.heads + 63) / 64, p.batch), dim3(512), 0, stream>>>(p);
+        const dim3 grid(p.max_chunks, (p.heads + 63) / 64, p.batch);
+        if (p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0) {
+            mla_partial_ws<true><<<grid, dim3(512), 0, stream>>>(p);
+        } else {
+            mla_partial_ws<false><<<grid, dim3(512), 0, stream>>>(p);
+        }
         err = hipGetLastError();
         if (err != hipSuccess) {
             return err;
