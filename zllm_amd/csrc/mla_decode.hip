@@ -334,9 +334,14 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
     convert_step(lds, lds_scale[0], &lds_top[0], c_start);
     lds_barrier();
 
-    // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile i - 1.
-    auto stage_next = [&](unsigned int i) __attribute__((always_inline)) {
-        if (i + 1 < steps) {
+    // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile
+    // i - 1.  The roles are half a step out of phase: a score wave requests step i + 1 first, scores tile i (matrix
+    // work) and converts step i + 1 last; a value wave converts step i + 1 first (requested an iteration ago),
+    // requests step i + 2, and accumulates tile i - 1 (matrix work) last.  So the conversion and load-issue work of
+    // one role runs under the matrix work of the other instead of all eight waves queueing at the load unit and
+    // the LDS write port together.
+    auto stage_step = [&](unsigned int n) __attribute__((always_inline)) { // request the raw bytes of step n
+        if (n < steps) {
             // The entries were fetched an iteration ago.  Naming them here places the compiler's wait for them
             // before the first load of this iteration; left to itself it waits again before every address it
             // forms from them, i.e. for the load it has just issued.
@@ -345,18 +350,17 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             } else {
                 asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]));
             }
-            issue_step(rows, c_start + (i + 1u) * kStepTokens);
-            if (i + 2 < steps) {
-                lookup_step(rows, c_start + (i + 2u) * kStepTokens);
+            issue_step(rows, c_start + n * kStepTokens);
+            if (n + 1 < steps) {
+                lookup_step(rows, c_start + (n + 1u) * kStepTokens);
             }
         }
     };
-    auto finish_iteration = [&](unsigned int i) __attribute__((always_inline)) {
-        if (i + 1 < steps) {
-            const unsigned int nb = (i + 1u) % kWsTiles;
-            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + (i + 1u) * kStepTokens);
+    auto convert_to = [&](unsigned int n) __attribute__((always_inline)) { // raw bytes of step n -> tile buffer n % 3
+        if (n < steps) {
+            const unsigned int nb = n % kWsTiles;
+            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + n * kStepTokens);
         }
-        lds_barrier();
     };
 
     if (!value_role) {
@@ -402,7 +406,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
         const float scale_log2 = p.score_scale * kLog2e;
         const float latent_log2 = scale_log2 * head_pow2;
         for (unsigned int i = 0; i <= steps; ++i) {
-            stage_next(i);
+            stage_step(i + 1u);
             if (i < steps) {
                 const unsigned int tb = i % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes;
@@ -503,7 +507,8 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
                 *(f32x4*)(slot + 4) = p_hi;
                 lds_alpha[i & 1u][hw][lane] = alpha;
             }
-            finish_iteration(i);
+            convert_to(i + 1u);
+            lds_barrier();
         }
         const float total = wave_sum_16x4(run_sum);
         if (head < p.heads && j == 0) {
@@ -527,6 +532,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
         }
         int window = 0;
         unsigned int value_tile = 0; // buffer of tile i - 1
+        stage_step(1u);
         const unsigned int lds_base = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)lds;
         for (unsigned int i = 0; i <= steps; ++i) {
             // the hand-over records are requested first: their LDS round trip hides behind the staging work
@@ -541,7 +547,8 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             }
             const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[value_tile])); // tile i - 1
             asm volatile("" ::: "memory");
-            stage_next(i);
+            convert_to(i + 1u);
+            stage_step(i + 2u);
             if (i > 0) {
                 // LDS byte addresses of this step: one register per fragment row, everything else is an immediate
                 const unsigned int tile_lds = lds_base + value_tile * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
@@ -637,7 +644,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             if (i > 0) {
                 value_tile = value_tile == kWsTiles - 1u ? 0u : value_tile + 1u;
             }
-            finish_iteration(i);
+            lds_barrier();
         }
 #pragma unroll
         for (int ht = 0; ht < 2; ++ht) {
