@@ -81,10 +81,29 @@ def run_mla_decode(args):
 
     for _ in range(args.warmup):
         run(0)()
-    ms_step = _wall_ms(run(0), args.steps)
-    ms_events = _event_ms(run(0), args.steps)
+    ms_eager = _wall_ms(run(0), args.steps)
+    # The decode step is replayed from a HIP graph, as the reference replays its decode launches
+    # (src/kernel/rocm/hip/graph.rs): same kernels, same arguments, without per-launch host overhead.  One graph holds
+    # `per_graph` consecutive calls, the way a model step holds one attention call per layer.
+    per_graph = max(g for g in range(1, 17) if args.steps % g == 0)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(0)()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        capture_stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(per_graph):
+            call.stage_mask = 0
+            capi.check(lib.zllm_attn_mla_decode(C.byref(call), capture_stream))
+    replays = args.steps // per_graph
+    for _ in range(max(1, args.warmup // per_graph)):
+        graph.replay()
+    ms_step = _wall_ms(graph.replay, replays) / per_graph
+    ms_events = _event_ms(graph.replay, replays) / per_graph
     stage_ms = {name: _event_ms(run(mask), args.steps) for name, mask in
-                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge", capi.MLA_MERGE), ("project", capi.MLA_PROJECT))}
+                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge_project", capi.MLA_MERGE | capi.MLA_PROJECT))}
     run(0)()
     torch.cuda.synchronize()
     flops = sum(lens) * heads * (2 * (latent + rope) + 2 * latent)  # QK^T over 576 + PV over 512, multiply-add = 2
@@ -102,7 +121,8 @@ def run_mla_decode(args):
         "pct_of_mfma_peak": round(100.0 * tflops_call / MFMA_BF16_PEAK_TFLOPS, 2),
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "effective_kv_gbps": round(kv_bytes / (ms_step * 1e-3) / 1e9, 1),
-        "ms_per_step_events": round(ms_events, 5),
+        "ms_per_step_events": round(ms_events, 5), "ms_per_step_eager": round(ms_eager, 5),
+        "launch": f"hipGraph replay, {per_graph} decode calls (absorb + partial + merge/project each) per graph",
         "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
         "roofline": {"bound": "mfma", "kernel": "mla_partial", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,

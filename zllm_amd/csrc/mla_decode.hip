@@ -665,31 +665,19 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
 // ---------------------------------------------------------------------------------------------
 // 4. project value
 // ---------------------------------------------------------------------------------------------
-// grid = (heads, batch), 256 threads = 4 waves.  A wave works on eight value columns at a time: lane =
-// (column v0 + lane / 8, slice lane % 8 of 64 latent columns); the lane keeps its 64 weighted values in
-// registers, reads its 64 weights as eight 16-byte vectors, and the eight slices are summed with DPP row
-// shifts.  The weight rows of a head are read exactly once, as whole 128-byte lines.
-__global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
+// 256 threads = 4 waves.  A wave works on eight value columns at a time: lane = (column v0 + lane / 8, slice
+// lane % 8 of 64 latent columns); the lane keeps its 64 weighted values in registers, reads its 64 weights as
+// eight 16-byte vectors, and the eight slices are summed with DPP row shifts.  The weight rows of a head are
+// read exactly once, as whole 128-byte lines.
+__device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned int head, unsigned int b, const float (&x)[64])
 {
-    const unsigned int head = blockIdx.x;
-    const unsigned int b = blockIdx.y;
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int wave = threadIdx.x >> 6;
     const unsigned int slice = lane & 7u;
     const unsigned int sub = lane >> 3;
-    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * kLatent + slice * 64u;
     const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 64u;
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     const size_t out_base = ((size_t)b * p.heads + head) * out_stride;
-    float x[64];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const f32x4 t = *(const f32x4*)(weighted + 4 * i);
-        x[4 * i] = t[0];
-        x[4 * i + 1] = t[1];
-        x[4 * i + 2] = t[2];
-        x[4 * i + 3] = t[3];
-    }
     for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
         const unsigned int v = v0 + sub;
         const unsigned int vr = min(v, p.value_dim - 1u);
@@ -721,6 +709,111 @@ __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
     }
 }
 
+// grid = (heads, batch): projection of the merged rows in the workspace (stage run on its own)
+__global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
+{
+    const unsigned int head = blockIdx.x;
+    const unsigned int b = blockIdx.y;
+    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * kLatent + (threadIdx.x & 7u) * 64u;
+    float x[64];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const f32x4 t = *(const f32x4*)(weighted + 4 * i);
+        x[4 * i] = t[0];
+        x[4 * i + 1] = t[1];
+        x[4 * i + 2] = t[2];
+        x[4 * i + 3] = t[3];
+    }
+    project_head(p, head, b, x);
+}
+
+// grid = (heads, batch): split merge and projection in one kernel when both stages run.  The merge is the
+// log-sum-exp combine of the split records (same algebra as the stand-alone merge, base 2): threads =
+// (128 column quads) x (2 split lanes), all loads of a lane issued before any is used; the merged row goes
+// through LDS to the projection's register layout instead of through the workspace.
+__global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
+{
+    const unsigned int head = blockIdx.x;
+    const unsigned int b = blockIdx.y;
+    const unsigned int quad = threadIdx.x & 127u;
+    const unsigned int sl = threadIdx.x >> 7;
+    const unsigned int len = p.ctx_lens[b];
+    const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+    const size_t stat_stride = (size_t)p.heads * 2;
+    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+    const size_t partial_stride = (size_t)p.heads * kLatent;
+    float m = kNegInf, l = 0.0f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned int c0 = sl; c0 < chunks; c0 += 16u) {
+        float cm[8], cl[8];
+        f32x4 part[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const unsigned int c = min(c0 + 2u * u, chunks - 1u);
+            const bool live = c0 + 2u * u < chunks;
+            const float2 st = *(const float2*)(stats + c * stat_stride);
+            cm[u] = live ? st.x : kNegInf;
+            cl[u] = live ? st.y : 0.0f;
+            part[u] = *(const f32x4*)(partial + c * partial_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (cl[u] > 0.0f) {
+                const float nm = fmaxf(m, cm[u]);
+                const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+                const float w = __builtin_amdgcn_exp2f(cm[u] - nm);
+                acc = acc * a + part[u] * w;
+                l = l * a + cl[u] * w;
+                m = nm;
+            }
+        }
+    }
+    __shared__ float other_m[128], other_l[128];
+    __shared__ f32x4 other_acc[128];
+    __shared__ __align__(16) float merged[kLatent];
+    if (sl == 1u) {
+        other_m[quad] = m;
+        other_l[quad] = l;
+        other_acc[quad] = acc;
+    }
+    __syncthreads();
+    if (sl == 0u) {
+        const float om = other_m[quad], ol = other_l[quad];
+        const float gm = fmaxf(m, om);
+        const float safe_g = gm == kNegInf ? 0.0f : gm;
+        float denom = 0.0f;
+        f32x4 total = {0.f, 0.f, 0.f, 0.f};
+        if (l > 0.0f) {
+            const float w = __builtin_amdgcn_exp2f(m - safe_g);
+            denom += l * w;
+            total += acc * w;
+        }
+        if (ol > 0.0f) {
+            const float w = __builtin_amdgcn_exp2f(om - safe_g);
+            denom += ol * w;
+            total += other_acc[quad] * w;
+        }
+        f32x4 result = {0.f, 0.f, 0.f, 0.f};
+        if (denom > 0.0f && denom < __builtin_inff()) {
+            result = total * (1.0f / denom);
+        }
+        *(f32x4*)(merged + quad * 4u) = result;
+    }
+    __syncthreads();
+    float x[64];
+    const float* row = merged + (threadIdx.x & 7u) * 64u;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const f32x4 t = *(const f32x4*)(row + 4 * i);
+        x[4 * i] = t[0];
+        x[4 * i + 1] = t[1];
+        x[4 * i + 2] = t[2];
+        x[4 * i + 3] = t[3];
+    }
+    project_head(p, head, b, x);
+}
+
 } // namespace
 
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
@@ -746,6 +839,10 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         if (err != hipSuccess) {
             return err;
         }
+    }
+    if ((stages & 12u) == 12u) {
+        mla_merge_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        return hipGetLastError();
     }
     if (stages & 4u) {
         // LSE combine into weighted[b, h, 0:512] (f32)
