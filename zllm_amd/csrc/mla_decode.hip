@@ -86,7 +86,7 @@ __device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned i
 // ---------------------------------------------------------------------------------------------
 // 1. absorb
 // ---------------------------------------------------------------------------------------------
-// grid = (heads, batch), 256 threads, thread c owns latent columns c and c + 256.
+// grid = (heads, batch), 256 threads, thread c owns latent columns 2 c and 2 c + 1.
 // The sum runs over k in ascending order with separately rounded multiply and add, the order of
 // the reference's scalar matmul (src/kernel/cpu/mla.rs:712-728); the result is rounded to bf16
 // (mla.rs:1037).
@@ -103,13 +103,27 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
     }
     __syncthreads();
     unsigned short* qa = p.absorbed + ((size_t)b * p.heads + head) * (p.latent_dim + p.rope_dim);
-    const unsigned short* w = p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim;
-    for (unsigned int c = threadIdx.x; c < p.latent_dim; c += 256) {
-        float acc = 0.0f;
-        for (unsigned int k = 0; k < p.nope_dim; ++k) {
-            acc = __fadd_rn(acc, __fmul_rn(q_sh[k], bf16_bits_to_f32(w[(size_t)k * p.latent_dim + c])));
+    // a thread owns two adjacent latent columns: one 4-byte weight load per k, 32 of them requested before the
+    // first is used (the sums themselves stay strictly sequential in k)
+    const unsigned int pairs = p.latent_dim / 2u;
+    const unsigned int* w = (const unsigned int*)(p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim);
+    for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
+        float acc0 = 0.0f, acc1 = 0.0f;
+        for (unsigned int k0 = 0; k0 < p.nope_dim; k0 += 32u) {
+            unsigned int word[32];
+#pragma unroll
+            for (int u = 0; u < 32; ++u) {
+                word[u] = w[(size_t)min(k0 + u, p.nope_dim - 1u) * pairs + c2];
+            }
+#pragma unroll
+            for (int u = 0; u < 32; ++u) {
+                if (k0 + u < p.nope_dim) {
+                    acc0 = __fadd_rn(acc0, __fmul_rn(q_sh[k0 + u], __uint_as_float(word[u] << 16)));
+                    acc1 = __fadd_rn(acc1, __fmul_rn(q_sh[k0 + u], __uint_as_float(word[u] & 0xffff0000u)));
+                }
+            }
         }
-        qa[c] = f32_to_bf16_bits(acc);
+        *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
     }
     for (unsigned int r = threadIdx.x; r < p.rope_dim; r += 256) {
         qa[p.latent_dim + r] = f32_to_bf16_bits(q_sh[p.nope_dim + r]);
