@@ -176,8 +176,10 @@ constexpr int kWsTiles = 3;
 // masked, so they contribute exact zeros.
 template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
-    constexpr int ITEMS = 2;  // staging items per thread: 32 tokens x 32 code chunks over 512 threads
-    constexpr int TROWS = 16; // token rows covered by one pass of the threads
+    // Staging items (token row, 16 codes) per thread: the 32 rows of a step are split 24 : 8 between the score and the
+    // value waves, because the value waves' step is the longer one.  A score thread takes rows r, r + 8 and r + 16,
+    // a value thread row 24 + r, with r = (thread % 256) / 32.
+    constexpr int ITEMS = 3;
     __shared__ __align__(16) unsigned char lds[kWsTiles * kTileBytes];
     __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
     __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
@@ -213,7 +215,10 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
     // ---- staging (same scheme as mla_partial): loads of the next tile's raw bytes, converted by their owner
     const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const unsigned int cc = tid & 31u;
-    const unsigned int t_lo = tid >> 5;
+    const unsigned int t_lo = (tid & 255u) >> 5;
+    const int n_items = value_role ? 1 : 3;
+    const unsigned int row_first = value_role ? 24u + t_lo : t_lo;      // row of item 0; item i is 8 i further on
+    const unsigned int wave_rows = (value_role ? 24u : 0u) + 2u * (wave & 3u); // first row of the wave's item 0
     const unsigned int rope_t = (tid >> 3) & 31u;
     const unsigned int rope_c = tid & 7u;
     const bool has_rope = tid < 256u;
@@ -229,14 +234,16 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
         } else {
 #pragma unroll
             for (int i = 0; i <= ITEMS; ++i) {
-                const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
-                const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
-                r.entry[i] = table != nullptr ? table[page] : page;
+                if (i < n_items || i == ITEMS) {
+                    const unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+                    const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+                    r.entry[i] = table != nullptr ? table[page] : page;
+                }
             }
         }
     };
     auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
-        const unsigned int token = min(t0 + (i < ITEMS ? t_lo + TROWS * i : extra_t), len - 1u);
+        const unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
         if (pow2) {
             return ((unsigned long long)r.entry[i] << p.block_shift) + (token & (p.block_tokens - 1u));
         }
@@ -247,11 +254,14 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             const unsigned int entry = __builtin_amdgcn_readfirstlane(rows.entry[0]);
             const unsigned long long row0 = pow2 ? ((unsigned long long)entry << p.block_shift) + (t0 & (p.block_tokens - 1u))
                                                  : (unsigned long long)entry * p.block_tokens + t0 % p.block_tokens;
-            const unsigned char* codes = (const unsigned char*)p.latent_codes + (row0 + 2u * wave_u) * kLatent;
+            const unsigned int first = __builtin_amdgcn_readfirstlane(wave_rows);
+            const unsigned char* codes = (const unsigned char*)p.latent_codes + (row0 + first) * kLatent;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(codes + TROWS * i * kLatent + lane * 16u),
-                                                 (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
+                if (i < n_items) {
+                    __builtin_amdgcn_global_load_lds((global_ptr_t)(codes + 8 * i * kLatent + lane * 16u),
+                                                     (lds_ptr_t)(raw_codes + (first + 8 * i) * kLatent), 16, 0, 0);
+                }
             }
             if (has_rope) {
                 const unsigned char* rope = (const unsigned char*)p.rope_cache + row0 * (kRope * 2) + wave_u * 1024u;
@@ -262,10 +272,13 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(scales + lane * 16u), (lds_ptr_t)(raw_scales), 16, 0, 0);
             }
         } else {
+            const unsigned int first = __builtin_amdgcn_readfirstlane(wave_rows);
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
-                                                 (lds_ptr_t)(raw_codes + (2u * wave_u + TROWS * i) * kLatent), 16, 0, 0);
+                if (i < n_items) {
+                    __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
+                                                     (lds_ptr_t)(raw_codes + (first + 8 * i) * kLatent), 16, 0, 0);
+                }
             }
             if (has_rope) {
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
@@ -281,9 +294,12 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
+            if (i >= n_items) {
+                break;
+            }
             // the thread converts codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row: 32 consecutive lanes then
             // write 512 contiguous bytes per instruction (chunks cc and cc + 32), which the LDS takes without conflicts
-            const unsigned int row = t_lo + TROWS * i;
+            const unsigned int row = row_first + 8u * i;
             const u32x2 half[2] = {*(const u32x2*)(raw_codes + row * kLatent + cc * 8u),
                                    *(const u32x2*)(raw_codes + row * kLatent + 256u + cc * 8u)};
 #pragma unroll
@@ -339,7 +355,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
         pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
     }
 
-    StepRows rows;
+    StepRows rows = {};
     lookup_step(rows, c_start);
     issue_step(rows, c_start);
     if (steps > 1) {
@@ -362,7 +378,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             if constexpr (ALIGNED) {
                 asm volatile("" : "+v"(rows.entry[0]));
             } else {
-                asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]));
+                asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]), "+v"(rows.entry[3]));
             }
             issue_step(rows, c_start + n * kStepTokens);
             if (n + 1 < steps) {
@@ -427,62 +443,76 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
                 const float (*scale_tile)[kStepTokens] = lds_scale[tb];
                 const unsigned int t0 = c_start + i * kStepTokens;
                 float sc[8];
-                // K fragments are requested one batch (four k-steps) ahead of the MFMAs that use them.
-                // Batch q of a token tile: q = 0..3 -> latent groups {0..3} first k-step, {0..3} second k-step,
-                // {4..7} first, {4..7} second; the two rope k-steps ride along with batch 0.
-                auto load_batch = [&](Frag (&kf)[4], const unsigned char* kt, int q) __attribute__((always_inline)) {
+                // K fragments are requested kAhead batches (of four k-steps) ahead of the MFMAs that use them: an LDS
+                // round trip under load is several batches of matrix work long, and nothing else hides it with two
+                // waves per SIMD.  Batch b of a step: token tile b / 4; q = b % 4 -> latent groups {0..3} first
+                // k-step, {0..3} second k-step, {4..7} first, {4..7} second; the two rope k-steps of a token tile
+                // ride along with its batch 0.
+                constexpr int kRing = 4, kAhead = kRing - 1;
+                Frag kf[kRing][4], kr[2][2];
+                f32x4 gsv[2][4]; // group scales of the odd batches (LDS returns in order: a late scale read would wait
+                                 // for every fragment requested before it)
+                auto load_batch = [&](int bt) __attribute__((always_inline)) {
+                    const unsigned char* kt = tile + (bt >> 2) * 16 * kRowBytes;
+                    const int q = bt & 3;
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        kf[u].u = *(const u32x4*)(kt + qk_base[q & 1] + ((q >> 1) * 4 + u) * 128);
+                        kf[bt % kRing][u].u = *(const u32x4*)(kt + qk_base[q & 1] + ((q >> 1) * 4 + u) * 128);
                     }
-                };
-                Frag kf[2][4], kr[2];
-                load_batch(kf[0], tile, 0);
-#pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2) {
-                    const unsigned char* kt = tile + t2 * 16 * kRowBytes;
-                    f32x4 s = {0.f, 0.f, 0.f, 0.f};      // latent part, in units of head_pow2
-                    f32x4 s_rope = {0.f, 0.f, 0.f, 0.f}; // rope part
-                    kr[0].u = *(const u32x4*)(kt + qk_base[0] + 8 * 128);
-                    kr[1].u = *(const u32x4*)(kt + qk_base[1] + 8 * 128);
-                    f32x4 d[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int cur = q & 1;
-                        if (q + 1 < 4) {
-                            load_batch(kf[cur ^ 1], kt, q + 1);
-                        } else if (t2 == 0) {
-                            load_batch(kf[cur ^ 1], kt + 16 * kRowBytes, 0);
-                        }
-                        asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
-                        if (q == 0) {
-                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[0].b, qf[16].b, s_rope, 0, 0, 0);
-                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[1].b, qf[17].b, s_rope, 0, 0, 0);
-                        }
+                    if (q == 0) {
+                        kr[bt >> 2][0].u = *(const u32x4*)(kt + qk_base[0] + 8 * 128);
+                        kr[bt >> 2][1].u = *(const u32x4*)(kt + qk_base[1] + 8 * 128);
+                    }
+                    if (q & 1) {
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
-                            const int g = (q >> 1) * 4 + u;
-                            if ((q & 1) == 0) {
-                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[cur][u].h, qf[2 * g].h, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                            } else {
-                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[cur][u].h, qf[2 * g + 1].h, d[u], 0, 0, 0);
-                            }
+                            gsv[(bt >> 1) & 1][u] = *(const f32x4*)(&scale_tile[(q >> 1) * 4 + u][(bt >> 2) * 16 + 4 * j]);
                         }
-                        if ((q & 1) == 1) {
+                    }
+                };
 #pragma unroll
-                            for (int u = 0; u < 4; ++u) {
-                                const int g = (q >> 1) * 4 + u;
-                                const f32x4 gs = *(const f32x4*)(&scale_tile[g][t2 * 16 + 4 * j]);
+                for (int bt = 0; bt < kAhead; ++bt) {
+                    load_batch(bt);
+                }
+                f32x4 s = {0.f, 0.f, 0.f, 0.f};      // latent part, in units of head_pow2
+                f32x4 s_rope = {0.f, 0.f, 0.f, 0.f}; // rope part
+                f32x4 d[4];
 #pragma unroll
-                                for (int r = 0; r < 4; ++r) {
-                                    s[r] = fmaf(d[u][r], gs[r], s[r]);
-                                }
+                for (int bt = 0; bt < 8; ++bt) {
+                    const int t2 = bt >> 2, q = bt & 3;
+                    if (bt + kAhead < 8) {
+                        load_batch(bt + kAhead);
+                    }
+                    asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
+                    if (q == 0) {
+                        s = f32x4{0.f, 0.f, 0.f, 0.f};
+                        s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t2][0].b, qf[16].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[t2][1].b, qf[17].b, s_rope, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int g = (q >> 1) * 4 + u;
+                        if ((q & 1) == 0) {
+                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[bt % kRing][u].h, qf[2 * g].h, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        } else {
+                            d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[bt % kRing][u].h, qf[2 * g + 1].h, d[u], 0, 0, 0);
+                        }
+                    }
+                    if ((q & 1) == 1) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const f32x4 gs = gsv[(bt >> 1) & 1][u];
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                s[r] = fmaf(d[u][r], gs[r], s[r]);
                             }
                         }
                     }
+                    if (q == 3) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        sc[t2 * 4 + r] = fmaf(s[r], latent_log2, s_rope[r] * scale_log2);
+                        for (int r = 0; r < 4; ++r) {
+                            sc[t2 * 4 + r] = fmaf(s[r], latent_log2, s_rope[r] * scale_log2);
+                        }
                     }
                 }
                 if (t0 + kStepTokens > len) { // only the last step of a sequence has tokens to mask
