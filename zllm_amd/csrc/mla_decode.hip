@@ -448,7 +448,7 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
                 // waves per SIMD.  Batch b of a step: token tile b / 4; q = b % 4 -> latent groups {0..3} first
                 // k-step, {0..3} second k-step, {4..7} first, {4..7} second; the two rope k-steps of a token tile
                 // ride along with its batch 0.
-                constexpr int kRing = 4, kAhead = kRing - 1;
+                constexpr int kRing = 3, kAhead = kRing - 1;
                 Frag kf[kRing][4], kr[2][2];
                 f32x4 gsv[2][4]; // group scales of the odd batches (LDS returns in order: a late scale read would wait
                                  // for every fragment requested before it)
@@ -591,8 +591,10 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
             }
             const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[value_tile])); // tile i - 1
             asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_setprio(3);
             convert_to(i + 1u);
             stage_step(i + 2u);
+            __builtin_amdgcn_s_setprio(0);
             if (i > 0) {
                 // LDS byte addresses of this step: one register per fragment row, everything else is an immediate
                 const unsigned int tile_lds = lds_base + value_tile * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
