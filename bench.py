@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk", "copy_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration"])
     ap.add_argument("--pool-gib", type=float, default=160.0, help="address span of the paged pool (all four planes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)

@@ -155,9 +155,120 @@ def run_mla_decode(args):
     print(json.dumps(record))
 
 
+def run_gqa_decode_f16(args):
+    """C3: f16 KV cache, B=4, 16q/8kv, d=256, ctx 8192, soft-cap 50; the full layer and the sliding layer (window 1024) are
+    timed as two calls of the same entry point.  `value` is the full layer (268 MB of KV per call)."""
+    import torch
+
+    import oracle as O
+    from zllm_amd import capi, ops
+
+    dev = torch.device("cuda:0")
+    batch, hq, hkv, d, ctx, bt, window, softcap = 4, 16, 8, 256, 8192, 16, 1024, 50.0
+    scale = 1.0 / 16.0  # 1/sqrt(256)
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    blocks_per_seq = ctx // bt
+    pool_blocks = batch * blocks_per_seq * 8  # pages scattered over an 8x larger pool (~2 GiB per plane)
+    rows = pool_blocks * bt
+    k_plane = torch.empty((rows, hkv * d), dtype=torch.float16, device=dev)
+    v_plane = torch.empty((rows, hkv * d), dtype=torch.float16, device=dev)
+    perm = torch.randperm(pool_blocks, generator=gen, device=dev)[: batch * blocks_per_seq].to(torch.int32)
+    tables = perm.view(batch, blocks_per_seq).contiguous()
+    for b in range(batch):
+        idx = (tables[b].long()[:, None] * bt + torch.arange(bt, device=dev)[None, :]).reshape(-1)
+        k_plane[idx] = torch.randn((ctx, hkv * d), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        v_plane[idx] = torch.randn((ctx, hkv * d), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+    q = torch.randn((batch, hq * d), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    lens = [ctx] * batch
+    lens_dev = torch.tensor(lens, dtype=torch.int32, device=dev)
+    first_dev = torch.tensor([ctx - window] * batch, dtype=torch.int32, device=dev)
+    lib = capi.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    results = {}
+    outs = {}
+    for name, first, visible in (("full", None, ctx), ("window", first_dev, window)):
+        call, out, workspace = ops.gqa_decode_args(q, k_plane, None, v_plane, None, tables, lens_dev, hq, hkv, d, bt, scale, ctx,
+                                                   first_visible=first, softcap=softcap, kv_format=capi.KV_F16,
+                                                   total_kv_tokens=visible * batch)
+
+        def launch(stages, call=call):
+            def fn():
+                call.stages = stages
+                capi.check(lib.zllm_attn_gqa_decode(C.byref(call), stream))
+            return fn
+
+        for _ in range(args.warmup):
+            launch(capi.STAGE_ALL)()
+        per_graph = max(g for g in range(1, 17) if args.steps % g == 0)
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            launch(capi.STAGE_ALL)()
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(graph):
+            cap = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for _ in range(per_graph):
+                call.stages = capi.STAGE_ALL
+                capi.check(lib.zllm_attn_gqa_decode(C.byref(call), cap))
+        replays = args.steps // per_graph
+        graph.replay()
+        ms_step = _wall_ms(graph.replay, replays) / per_graph
+        ms_partial = _event_ms(launch(capi.STAGE_PARTIAL), args.steps)
+        launch(capi.STAGE_ALL)()
+        torch.cuda.synchronize()
+        kv_bytes = batch * visible * 2 * hkv * d * 2  # K + V, f16
+        results[name] = {"ms_per_step": ms_step, "kernel_ms": ms_partial, "kv_bytes": kv_bytes}
+        outs[name] = (out.clone(), call, workspace)
+    full, win = results["full"], results["window"]
+    gbps = full["kv_bytes"] / (full["ms_per_step"] * 1e-3) / 1e9
+    achieved = full["kv_bytes"] / (full["kernel_ms"] * 1e-3) / 1e9
+    record = {
+        "metric": "f16-KV GQA decode attn effective KV GB/s (% of HBM peak) at 8K ctx, 1 GPU", "value": round(gbps, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(full["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "C3 f16-KV GQA decode, B=4, 16q/8kv, d=256, ctx 8192, soft-cap 50, score_scale 1/16, 16-token pages; "
+                               "full layer (value) and sliding layer (window 1024)",
+                   "kv_bytes_per_call": full["kv_bytes"], "window_kv_bytes_per_call": win["kv_bytes"], "seed": args.seed},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "tokens_per_s": round(batch / (full["ms_per_step"] * 1e-3), 1),
+        "window_layer": {"ms_per_step": round(win["ms_per_step"], 5), "kernel_ms": round(win["kernel_ms"], 5),
+                         "effective_kv_gbps": round(win["kv_bytes"] / (win["ms_per_step"] * 1e-3) / 1e9, 1),
+                         "kernel_gbps": round(win["kv_bytes"] / (win["kernel_ms"] * 1e-3) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": "gqa_decode_f16_partial", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel_ms": round(full["kernel_ms"], 5)},
+    }
+    if not args.no_cpu_baseline:
+        # CPU oracle on a bounded sample: sequence 0, all heads, both layer kinds
+        threads = O.set_threads(min(len(os.sched_getaffinity(0)), 16))
+        k_rows = ops.gather_rows(k_plane.view(torch.uint8), tables[0], 0, ctx, hkv * d * 2, bt).cpu().numpy().view(np.uint16)
+        v_rows = ops.gather_rows(v_plane.view(torch.uint8), tables[0], 0, ctx, hkv * d * 2, bt).cpu().numpy().view(np.uint16)
+        k_f32 = O.f16_to_f32(k_rows).reshape(ctx, hkv * d)
+        v_f32 = O.f16_to_f32(v_rows).reshape(ctx, hkv * d)
+        q_f32 = q[0:1].float().cpu().numpy()
+        worst = 0.0
+        seconds = 0.0
+        for name, win_size in (("full", 0), ("window", window)):
+            start, end = O.key_range(win_size, ctx - 1, ctx)
+            t0 = time.perf_counter()
+            rc, want = O.gqa_prefill_at_visible(q_f32, k_f32[start:end], v_f32[start:end], start, end, ctx - 1, hq, hkv, d,
+                                                window=win_size, score_scale=scale, softcap=softcap)
+            if name == "full":
+                seconds = time.perf_counter() - t0
+            assert rc == 0
+            worst = max(worst, float(np.abs(outs[name][0][0].cpu().numpy().ravel() - want.ravel()).max()))
+        record["cpu_baseline"] = {"value": round(ctx * 2 * hkv * d * 2 / seconds / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+                                  "sample": f"sequence 0 of the full layer ({ctx} keys, {hq} heads) on dequantised f32 K/V; {seconds:.2f}s"}
+        record["parity_vs_oracle_max_abs"] = worst
+    print(json.dumps(record))
+
+
 def run(args):
     if args.workload == "mla_decode_64k":
         run_mla_decode(args)
+    elif args.workload == "gqa_decode_f16_window":
+        run_gqa_decode_f16(args)
     elif args.workload == "gqa_prefill_chunk":
         from zllm_amd import bench_prefill
 

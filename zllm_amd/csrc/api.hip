@@ -102,6 +102,12 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
     return 0;
 }
 
+// Shortest GQA split: two 32-token steps.  A short visible range (a sliding-window layer, a short context) is
+// latency-bound -- a workgroup walks its steps one memory round trip after the other -- so it is cut into as many
+// splits as there are CUs before the splits are allowed to grow; the partial records this adds are a few percent of
+// the KV bytes even at 64 tokens per split.
+constexpr uint64_t kMinGqaChunk = 64;
+
 void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
     const uint32_t max_waves = zllm::gqa_decode_max_waves(a->head_dim);
@@ -116,12 +122,12 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
         // workgroups that will really run and keep them within one round of the CUs
         const uint64_t slots = (uint64_t)rounds * kComputeUnits / (kvh_blocks * head_blocks) - a->batch;
         uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
-        chunk = align_up(chunk < 256 ? 256 : chunk, 32);
+        chunk = align_up(chunk < kMinGqaChunk ? kMinGqaChunk : chunk, 32);
         *chunk_tokens = (uint32_t)chunk;
         *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
         return;
     }
-    plan_splits(a->max_kv_len, a->max_kv_len, columns, 256, rounds, chunk_tokens, max_chunks);
+    plan_splits(a->max_kv_len, a->max_kv_len, columns, kMinGqaChunk, rounds, chunk_tokens, max_chunks);
 }
 
 int validate_mla_decode(const zllm_mla_decode_args* a)

@@ -876,13 +876,58 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
-    // Q: per-head power-of-two normalisation keeps q inside the f16 range; hi + lo split.
+    // Q: per-head power-of-two normalisation keeps q inside the f16 range; hi + lo split.  The lane's 8 KS elements
+    // (k-step ks -> dims ks*32 + j*8 .. +8) are fetched as 16-byte vectors, all requested before the first is used.
     float q_norm = 1.0f;
+    Frag qhi[KS], qlo[KS];
     {
+        float x[KS][8];
+        const size_t q_index = ((size_t)b * p.num_heads + head) * D + j * 8;
+        if (!head_valid) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[ks][e] = 0.0f;
+                }
+            }
+        } else if (p.q_dtype == 0) {
+            u32x4 raw[KS][2];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                raw[ks][0] = *(const u32x4*)((const float*)p.q + q_index + ks * 32);
+                raw[ks][1] = *(const u32x4*)((const float*)p.q + q_index + ks * 32 + 4);
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[ks][e] = __uint_as_float(raw[ks][e >> 2][e & 3]);
+                }
+            }
+        } else {
+            u32x4 raw[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                raw[ks] = *(const u32x4*)((const unsigned short*)p.q + q_index + ks * 32);
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const unsigned int word = raw[ks][e >> 1];
+                    const unsigned short bits = (unsigned short)((e & 1) ? (word >> 16) : (word & 0xffffu));
+                    x[ks][e] = p.q_dtype == 1 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+                }
+            }
+        }
         float amax = 0.0f;
-        for (int e = 0; e < D / 4; ++e) {
-            const float x = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + j * (D / 4) + e, p.q_dtype) : 0.0f;
-            amax = fmaxf(amax, fabsf(x));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                amax = fmaxf(amax, fabsf(x[ks][e]));
+            }
         }
         amax = wave_max_16x4(amax);
         if (amax > 0.0f && amax < __builtin_inff()) {
@@ -890,16 +935,15 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
             frexpf(amax, &ex);        // amax = f * 2^ex, f in [0.5, 1)
             q_norm = ldexpf(1.0f, -ex); // |q| * q_norm < 1
         }
-    }
-    Frag qhi[KS], qlo[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float x = head_valid ? load_as_f32(p.q, ((size_t)b * p.num_heads + head) * D + ks * 32 + j * 8 + e, p.q_dtype) * q_norm : 0.0f;
-            const _Float16 h = (_Float16)x;
-            qhi[ks].h[e] = h;
-            qlo[ks].h[e] = (_Float16)(x - (float)h);
+            for (int e = 0; e < 8; ++e) {
+                const float scaled = x[ks][e] * q_norm;
+                const _Float16 h = (_Float16)scaled;
+                qhi[ks].h[e] = h;
+                qlo[ks].h[e] = (_Float16)(scaled - (float)h);
+            }
         }
     }
 
