@@ -291,6 +291,14 @@ typedef struct zllm_mla_decode_args {
                                      _PROJECT: run only those stages on the records already in the
                                      workspace (shard exchange, per-stage timing;
                                      cf. paged_mla.rs:3068-3081 per-stage profile) */
+    /* Selected-token (sparse) decode, the `selection` arm of the same launch
+     * (paged_mla.rs:3092-3105,3192-3195; kernel side source.hip:4738-4764): a sequence whose
+     * context is longer than top_k attends only to the tokens selection[b, 0 .. count_b), count_b =
+     * selection_counts[b] when given, else top_k; a sequence with ctx_len <= top_k stays dense.
+     * Entries are token positions (< ctx_len), used in the order given.  NULL = dense. */
+    uint32_t top_k;
+    const uint32_t* selection;        /* [dev] [batch, top_k] or NULL */
+    const uint32_t* selection_counts; /* [dev] [batch] or NULL */
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
 ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);

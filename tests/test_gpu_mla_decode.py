@@ -41,7 +41,9 @@ def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, b
                 latent=latent, block_tokens=block_tokens)
 
 
-def oracle_mla(case, head_subset=None):
+def oracle_mla(case, head_subset=None, selection=None, counts=None):
+    """`selection` [batch, top_k]: the reference's rule (paged_mla/source.hip:4761-4764) -- a sequence longer than top_k
+    attends to its first count listed positions, a shorter one stays dense."""
     spec, bt = case["spec"], case["block_tokens"]
     kv_b = O.bf16_to_f32(case["kv_b_bits"])
     outs_f, outs_b = [], []
@@ -50,14 +52,19 @@ def oracle_mla(case, head_subset=None):
         codes = O.gather_rows_bytes(case["codes"], case["tables"][b], bt, 0, l, case["latent"])
         scales = O.gather_rows_bytes(case["scales"], case["tables"][b], bt, 0, l, case["latent"] // 64 * 2).view(np.uint16)
         rope = O.gather_rows_bytes(case["rope"], case["tables"][b], bt, 0, l, case["rope_dim"] * 2).view(np.uint16)
-        rc, ob, of, _ = O.mla_absorbed_q8_history(spec, case["q_bits"][b:b + 1], 1, l - 1, codes, scales, 64, rope, l, kv_b)
+        sel, width = None, 0
+        if selection is not None and selection.shape[1] < l:
+            width = int(counts[b]) if counts is not None else selection.shape[1]
+            sel = selection[b, :width]
+        rc, ob, of, _ = O.mla_absorbed_q8_history(spec, case["q_bits"][b:b + 1], 1, l - 1, codes, scales, 64, rope, l, kv_b,
+                                                  selection=sel, width=width)
         assert rc == 0
         outs_f.append(of)
         outs_b.append(ob)
     return np.stack(outs_f), np.stack(outs_b)
 
 
-def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None):
+def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, selection=None, counts=None):
     from zllm_amd import ops
 
     out_dtype = out_dtype or torch.float32
@@ -65,7 +72,9 @@ def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None):
     out = ops.mla_decode(q, upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]), upload(case["rope"]),
                          upload(case["tables"]), upload(case["lens"]), case["heads"], case["nope"] + case["rope_dim"],
                          case["nope"] + case["value"], case["latent"], case["rope_dim"], case["block_tokens"],
-                         max_ctx_len or int(case["lens"].max()), out_dtype=out_dtype, out_compact=compact)
+                         max_ctx_len or int(case["lens"].max()), out_dtype=out_dtype, out_compact=compact,
+                         selection=None if selection is None else upload(selection),
+                         selection_counts=None if counts is None else upload(counts))
     torch.cuda.synchronize()
     return out
 
@@ -129,6 +138,48 @@ def test_mla_rows_past_the_end_of_a_page_are_ignored(block_tokens):
     got = run_mla(case).cpu().numpy()
     assert np.isfinite(got).all()
     assert_attention_close(got, want_f, f"poisoned tail, block_tokens={block_tokens}")
+
+
+def draw_selection(rng, lens, top_k, sort):
+    """Per sequence: top_k distinct visible positions (repeats only when the context is shorter than top_k, where the
+    list is ignored anyway)."""
+    sel = np.zeros((len(lens), top_k), dtype=np.uint32)
+    for b, l in enumerate(lens):
+        picks = rng.choice(l, size=top_k, replace=l < top_k)
+        sel[b] = np.sort(picks) if sort else picks
+    return sel
+
+
+@pytest.mark.parametrize("top_k,sort,block_tokens", [(200, False, 16), (2048, True, 64), (33, False, 1), (1, True, 16)])
+def test_mla_selected_tokens(top_k, sort, block_tokens):
+    """The `selection` arm (paged_mla.rs:3092-3105): sequences longer than top_k attend to the listed positions, in
+    list order; shorter ones stay dense.  Lengths straddle top_k on purpose."""
+    rng = np.random.default_rng(500 + top_k)
+    lens = [max(top_k * 3, 40), top_k + 1, max(top_k // 2, 1), 2500]
+    case = make_mla_case(600 + top_k, lens, 32, block_tokens=block_tokens, poison=True)
+    sel = draw_selection(rng, lens, top_k, sort)
+    want_f, _ = oracle_mla(case, selection=sel)
+    got = run_mla(case, selection=sel).cpu().numpy()
+    assert_attention_close(got, want_f, f"top_k={top_k}")
+    dense_f, _ = oracle_mla(case)
+    if top_k > 1:
+        assert np.abs(want_f[0] - dense_f[0]).max() > 1e-3  # the list really changes the long sequences' result
+    np.testing.assert_array_equal(np.abs(want_f[2] - dense_f[2]).max(), 0.0)  # and not the short one's
+
+
+def test_mla_selected_tokens_with_counts_and_repeats():
+    """selection_counts shortens a row's list; a position listed twice counts twice, as in the reference's loop over
+    slots (src/kernel/cpu/mla.rs:582-686)."""
+    rng = np.random.default_rng(77)
+    lens = [1500, 700, 64]
+    top_k = 256
+    case = make_mla_case(78, lens, 16, block_tokens=16)
+    sel = draw_selection(rng, lens, top_k, False)
+    sel[0, 10:20] = sel[0, 0]  # repeats
+    counts = np.array([256, 100, 256], dtype=np.uint32)
+    want_f, _ = oracle_mla(case, selection=sel, counts=counts)
+    got = run_mla(case, selection=sel, counts=counts).cpu().numpy()
+    assert_attention_close(got, want_f, "counts + repeats")
 
 
 def test_mla_split_invariance_and_zero_query():

@@ -274,3 +274,27 @@ def test_mla_zero_query_gives_mean_latent_projection(oracle):
     mean_latent = (codes.astype(np.float64) * 0.03125).mean(0)
     ref = np.stack([kv_b.reshape(H, nope + vd, R)[h, nope:] @ mean_latent for h in range(H)])
     assert rc == 0 and np.abs(out_f.reshape(H, vd) - ref).max() < 1e-3
+
+
+def test_absorbed_q8_selection_equals_dense_attention_over_the_gathered_rows(oracle):
+    """Attention over listed positions is attention over those rows laid out densely in list order: pins the
+    `selected` arm of the absorbed-Q8 oracle (src/kernel/cpu/mla.rs:958-1076) against its dense arm."""
+    rng = np.random.default_rng(11)
+    heads, latent, rope, nope, value, rows, width = 3, 128, 16, 32, 24, 50, 9
+    spec = oracle.MlaSpec(latent, rope, heads * (nope + rope), heads * (nope + value), heads)
+    q = oracle.f32_to_bf16(rng.standard_normal((1, heads * (nope + rope))).astype(np.float32))
+    codes = rng.integers(-127, 128, size=(rows, latent), dtype=np.int8)
+    scales = oracle.f32_to_bf16((rng.random((rows, latent // 64)) * 0.05 + 0.01).astype(np.float32))
+    rope_rows = oracle.f32_to_bf16(rng.standard_normal((rows, rope)).astype(np.float32))
+    kv_b = oracle.bf16_to_f32(oracle.f32_to_bf16((rng.standard_normal((heads * (nope + value), latent)) / 8).astype(np.float32)))
+    sel = rng.choice(rows, size=width, replace=False).astype(np.uint32)
+    rc, _, picked, _ = oracle.mla_absorbed_q8_history(spec, q, 1, rows - 1, codes, scales, 64, rope_rows, rows, kv_b,
+                                                      selection=sel, width=width)
+    assert rc == 0
+    rc, _, dense, _ = oracle.mla_absorbed_q8_history(spec, q, 1, width - 1, codes[sel], scales[sel], 64, rope_rows[sel], width, kv_b)
+    assert rc == 0
+    np.testing.assert_array_equal(picked, dense)
+    # a position at or past the query row is rejected (mla.rs:965-975)
+    bad = sel.copy()
+    bad[0] = rows
+    assert oracle.mla_absorbed_q8_history(spec, q, 1, rows - 1, codes, scales, 64, rope_rows, rows, kv_b, selection=bad, width=width)[0] != 0

@@ -153,6 +153,9 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
     if (a->stage_mask > 15u) {
         return fail(-1, "MLA decode: unknown stage_mask %u", a->stage_mask);
     }
+    if (a->selection != nullptr && a->top_k == 0) {
+        return fail(-1, "MLA decode: a selection needs top_k > 0");
+    }
     return 0;
 }
 
@@ -160,7 +163,9 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
 {
     // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
-    plan_splits(a->max_ctx_len, a->max_ctx_len, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
+    // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
+    const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
+    plan_splits(longest, longest, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {
@@ -484,6 +489,9 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     p.q_dtype = a->q_dtype;
     p.out_dtype = a->out_dtype;
     p.out_compact = a->out_compact;
+    p.selection = a->selection;
+    p.selection_counts = a->selection_counts;
+    p.top_k = a->top_k;
     return hip_status(zllm::launch_mla_decode(p, a->stage_mask, (hipStream_t)stream), "MLA decode launch");
 }
 

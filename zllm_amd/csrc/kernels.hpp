@@ -102,6 +102,9 @@ struct MlaDecodeParams {
     unsigned int chunk_tokens, max_chunks;
     float score_scale;
     int q_dtype, out_dtype, out_compact;
+    const unsigned int* selection;        // [batch][top_k] token positions, or nullptr (dense)
+    const unsigned int* selection_counts; // [batch] or nullptr
+    unsigned int top_k;
 };
 
 // KV heads (= waves) per GQA decode workgroup for a head dimension.

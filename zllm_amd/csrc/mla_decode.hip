@@ -151,6 +151,10 @@ constexpr int kRawScales = kStepTokens * (kLatent / 64) * 2; // 512 B [token][8]
 // scale role (threads 256..287).
 struct StepRows {
     unsigned int entry[kItemsMax + 1];
+    // selected-token mode only: the token positions behind `entry`, and those of the step after (fetched one
+    // step earlier still, so that neither the selection list nor the block table is waited for)
+    unsigned int token[kItemsMax + 1];
+    unsigned int next_token[kItemsMax + 1];
 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -174,8 +178,12 @@ constexpr int kWsTiles = 3;
 // plus a constant per-lane offset -- no vector address arithmetic in the loop.  Rows past the end of the
 // sequence are then whatever the page holds; their scales are zeroed during conversion and their scores
 // masked, so they contribute exact zeros.
-template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
+// SELECTED: the `selection` arm (src/kernel/rocm/hip/attention/paged_mla/source.hip:4738-4764): a sequence longer than
+// top_k attends to the listed token positions only.  The kernel then walks list slots instead of positions -- splits,
+// masks and softmax are over slots -- and only the address of a row goes through the list.
+template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
+    static_assert(!(ALIGNED && SELECTED), "selected rows are not contiguous");
     // Staging items (token row, 16 codes) per thread: the 32 rows of a step are split 24 : 8 between the score and the
     // value waves, because the value waves' step is the longer one.  A score thread takes rows r, r + 8 and r + 16,
     // a value thread row 24 + r, with r = (thread % 256) / 32.
@@ -196,7 +204,14 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
     const unsigned int chunk = blockIdx.x;
     const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
     const unsigned int b = blockIdx.z;
-    const unsigned int len = p.ctx_lens[b];
+    unsigned int len = p.ctx_lens[b]; // keys of this sequence: positions, or list slots when a selection applies
+    const unsigned int* selected = nullptr;
+    if constexpr (SELECTED) {
+        if (p.selection != nullptr && p.top_k < len) {
+            selected = p.selection + (size_t)b * p.top_k;
+            len = p.selection_counts != nullptr ? min(p.selection_counts[b], p.top_k) : p.top_k;
+        }
+    }
     const unsigned long long c_start64 = (unsigned long long)chunk * p.chunk_tokens;
     const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
     if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
@@ -227,6 +242,16 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
     unsigned char* const raw_codes = lds_raw;
     unsigned char* const raw_rope = lds_raw + kRawCodes;
     unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
+    // selected-token mode: positions of the thread's items for the step that starts at slot t0
+    auto fetch_tokens = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i <= ITEMS; ++i) {
+            if (i < n_items || i == ITEMS) {
+                const unsigned int slot = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+                r.next_token[i] = selected != nullptr ? selected[slot] : slot;
+            }
+        }
+    };
     auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
         if constexpr (ALIGNED) {
             const unsigned int page = pow2 ? t0 >> p.block_shift : t0 / p.block_tokens;
@@ -235,15 +260,25 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
 #pragma unroll
             for (int i = 0; i <= ITEMS; ++i) {
                 if (i < n_items || i == ITEMS) {
-                    const unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+                    unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+                    if constexpr (SELECTED) {
+                        token = r.next_token[i]; // fetched a step ago for this t0
+                        r.token[i] = token;
+                    }
                     const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
                     r.entry[i] = table != nullptr ? table[page] : page;
                 }
             }
+            if constexpr (SELECTED) {
+                fetch_tokens(r, t0 + kStepTokens);
+            }
         }
     };
     auto row_of = [&](const StepRows& r, int i, unsigned int t0) __attribute__((always_inline)) -> unsigned long long {
-        const unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+        unsigned int token = min(t0 + (i < ITEMS ? row_first + 8u * i : extra_t), len - 1u);
+        if constexpr (SELECTED) {
+            token = r.token[i];
+        }
         if (pow2) {
             return ((unsigned long long)r.entry[i] << p.block_shift) + (token & (p.block_tokens - 1u));
         }
@@ -356,6 +391,9 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
     }
 
     StepRows rows = {};
+    if constexpr (SELECTED) {
+        fetch_tokens(rows, c_start);
+    }
     lookup_step(rows, c_start);
     issue_step(rows, c_start);
     if (steps > 1) {
@@ -379,6 +417,10 @@ template <bool ALIGNED> __global__ __launch_bounds__(512) void mla_partial_ws(Ml
                 asm volatile("" : "+v"(rows.entry[0]));
             } else {
                 asm volatile("" : "+v"(rows.entry[0]), "+v"(rows.entry[1]), "+v"(rows.entry[2]), "+v"(rows.entry[3]));
+                if constexpr (SELECTED) {
+                    asm volatile("" : "+v"(rows.token[0]), "+v"(rows.token[1]), "+v"(rows.token[2]), "+v"(rows.token[3]),
+                                      "+v"(rows.next_token[0]), "+v"(rows.next_token[1]), "+v"(rows.next_token[2]), "+v"(rows.next_token[3]));
+                }
             }
             issue_step(rows, c_start + n * kStepTokens);
             if (n + 1 < steps) {
@@ -876,10 +918,12 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
         const dim3 grid(p.max_chunks, (p.heads + 63) / 64, p.batch);
-        if (p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0) {
-            mla_partial_ws<true><<<grid, dim3(512), 0, stream>>>(p);
+        if (p.selection != nullptr) {
+            mla_partial_ws<false, true><<<grid, dim3(512), 0, stream>>>(p);
+        } else if (p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0) {
+            mla_partial_ws<true, false><<<grid, dim3(512), 0, stream>>>(p);
         } else {
-            mla_partial_ws<false><<<grid, dim3(512), 0, stream>>>(p);
+            mla_partial_ws<false, false><<<grid, dim3(512), 0, stream>>>(p);
         }
         err = hipGetLastError();
         if (err != hipSuccess) {

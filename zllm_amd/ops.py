@@ -124,7 +124,7 @@ def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, 
 
 def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ctx_lens, heads, q_head_dim,
                     kv_head_dim, latent_dim, rope_dim, block_tokens, max_ctx_len, out_dtype=torch.float32,
-                    out_compact=True, out=None, workspace=None):
+                    out_compact=True, out=None, workspace=None, selection=None, selection_counts=None):
     batch = q.shape[0]
     value_dim = kv_head_dim - (q_head_dim - rope_dim)
     if out is None:
@@ -139,6 +139,9 @@ def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ct
     args.table_stride = 0 if tables is None else tables.shape[1]
     args.max_ctx_len, args.block_tokens = max_ctx_len, block_tokens
     args.q_dtype, args.out_dtype, args.out_compact = _DTYPE[q.dtype], _DTYPE[out_dtype], int(out_compact)
+    if selection is not None:  # [batch, top_k] token positions (uint32 / int32)
+        args.selection, args.top_k = _ptr(selection), selection.shape[1]
+        args.selection_counts = _ptr(selection_counts)
     need = capi.load().zllm_attn_mla_decode_workspace_bytes(C.byref(args))
     if need == 0:
         raise capi.ZllmAttnError(-1, capi.last_error())
