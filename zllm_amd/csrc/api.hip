@@ -165,7 +165,7 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    plan_splits(longest, longest, a->batch * head_blocks, 256, 1, chunk_tokens, max_chunks);
+    plan_splits(longest, longest, a->batch * head_blocks, 64, 1, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {
