@@ -221,6 +221,12 @@ typedef struct zllm_gqa_decode_args {
                                       (cf. try_paged_mla_attention_ct_shard,
                                       paged_mla.rs:3642); ZLLM_STAGE_MERGE combines records
                                       already in the workspace */
+    /* Output gate, the sigmoid_gate step that follows attention in HybridAttention::full
+     * (src/attention/hybrid.rs:79; src/backend/cpu/context.rs:419-432): out *= 1 / (1 + exp(-gate)).
+     * NULL = no gate. */
+    const void* gate;              /* [dev] [rows, gate_cols], gate_dtype */
+    uint32_t gate_cols;            /* num_heads * head_dim, or 1 (one gate per row) */
+    int gate_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
 } zllm_gqa_decode_args;
 ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* args);
 ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);
@@ -252,9 +258,61 @@ typedef struct zllm_gqa_prefill_args {
     float score_scale;
     float softcap;
     int kv_format, scale_dtype, q_dtype, out_dtype;
+    /* Output gate, the sigmoid_gate step that follows attention in HybridAttention::full
+     * (src/attention/hybrid.rs:79; src/backend/cpu/context.rs:419-432): out *= 1 / (1 + exp(-gate)).
+     * NULL = no gate. */
+    const void* gate;              /* [dev] [rows, gate_cols], gate_dtype */
+    uint32_t gate_cols;            /* num_heads * head_dim, or 1 (one gate per row) */
+    int gate_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
 } zllm_gqa_prefill_args;
 ZLLM_API uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* args);
 ZLLM_API int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* args, zllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Pre-attention prologue of a GQA layer.                                     *
+ * ------------------------------------------------------------------------- */
+
+/* One launch for what HybridAttention::full does between the projections and the
+ * attention call (src/attention/hybrid.rs:66-78): per-head RMSNorm of Q and K
+ * (gemma_rmsnorm_heads / rmsnorm_heads, src/kernel/cpu/vae.rs:297-334), RoPE of
+ * both at the row's position (rope_prefix, src/attention/rope.rs:120-164), and
+ * the quantizing page append of K and V (as zllm_attn_q8g64_append).  The
+ * normalise-and-rotate half is what the trait hook
+ * fused_rmsnorm_qkv_head_norm_rope (src/backend/mod.rs:1515-1538) asks of a
+ * backend; the Q/K/V projections stay with the caller's GEMM.
+ * Q comes out as a tensor for zllm_attn_gqa_decode / _prefill_chunk; K and V go
+ * straight into the pages.  Arithmetic is f32 with separately rounded steps
+ * in the reference's order, so Q (f32) and the K/V codes and scales are
+ * bit-exact with the CPU chain norm -> rope -> quantize. */
+typedef struct zllm_gqa_prologue_args {
+    const void* q;             /* [dev] [rows, num_heads * head_dim], src_dtype */
+    const void* k;             /* [dev] [rows, num_kv_heads * head_dim], src_dtype */
+    const void* v;             /* [dev] [rows, num_kv_heads * head_dim], src_dtype */
+    const float* q_norm;       /* [dev] [head_dim] or NULL (no Q norm) */
+    const float* k_norm;       /* [dev] [head_dim] or NULL (no K norm) */
+    const float* cosine;       /* [dev] [rope_table_rows, rotary_dim / 2]; unused when rotary_dim == 0 */
+    const float* sine;
+    void* q_out;               /* [dev] [rows, num_heads * head_dim], q_out_dtype */
+    int8_t* k_codes;           /* [dev] paged planes, as in zllm_q8_append_args */
+    void* k_scales;
+    int8_t* v_codes;
+    void* v_scales;
+    const uint32_t* table;     /* [dev] block table or NULL (identity) */
+    const uint32_t* positions; /* [dev] optional: positions[0] overrides `position` (graph replay) */
+    uint32_t rows, num_heads, num_kv_heads;
+    uint32_t head_dim;         /* multiple of 64, at most 256 */
+    uint32_t rotary_dim;       /* even, <= head_dim; the first rotary_dim columns of a head rotate */
+    uint32_t rope_table_rows;  /* rows of cosine / sine: position + rows must not exceed it */
+    uint32_t position;         /* first row's token position: RoPE angle and page slot */
+    uint32_t block_tokens, ring_capacity;
+    float eps;                 /* RMSNorm epsilon (> 0 when a norm weight is given) */
+    float weight_offset;       /* 1 = Gemma form (1 + weight), 0 = plain */
+    int src_dtype;             /* ZLLM_DTYPE_* of q, k, v */
+    int q_out_dtype;           /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
+    int rule;                  /* ZLLM_QUANT_* of the K/V pages */
+    int split_half;            /* 1 = pairs (i, i + rotary_dim / 2), 0 = interleaved (2 i, 2 i + 1) */
+} zllm_gqa_prologue_args;
+ZLLM_API int zllm_attn_gqa_prologue(const zllm_gqa_prologue_args* args, zllm_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * MLA absorbed decode over the Q8g64 latent cache.                           *

@@ -232,6 +232,27 @@ def rope_apply(data, head_count, rotary_dim, position, cos, sin, layout=0, place
     return rc, data
 
 
+def rmsnorm_heads(x, head_count, head_dim, weight, eps, weight_offset=0.0):
+    """Per-head RMSNorm (weight_offset 1.0 = Gemma form).  x [rows, head_count * head_dim]."""
+    x = _c(x, np.float32)
+    rows = x.size // (head_count * head_dim)
+    w = None if weight is None else _c(weight, np.float32)
+    out = np.zeros_like(x)
+    rc = lib().zo_rmsnorm_heads_f32(_p(x), C.c_uint64(rows), C.c_uint64(head_count), C.c_uint64(head_dim), _p(w),
+                                    C.c_float(eps), C.c_float(weight_offset), _p(out))
+    return rc, out
+
+
+def sigmoid_gate(x, gate):
+    x = _c(x, np.float32)
+    gate = _c(gate, np.float32)
+    rows = x.shape[0]
+    out = np.zeros_like(x)
+    rc = lib().zo_sigmoid_gate_f32(_p(x), _p(gate), C.c_uint64(rows), C.c_uint64(x.size // rows),
+                                   C.c_uint64(gate.size // rows), _p(out))
+    return rc, out
+
+
 # --------------------------------------------------------------------------- MLA
 def mla_reference_attention(query, projected_kv, rope_cache, rope_indices, spec: MlaSpec):
     query = _c(query, np.float32)

@@ -644,6 +644,66 @@ ZO_API int zo_rope_apply_f32(float* data, uint64_t rows, uint64_t columns, uint6
 }
 
 /* ------------------------------------------------------------------------ */
+/* Per-head RMSNorm and the sigmoid output gate                               */
+/* ------------------------------------------------------------------------ */
+
+/* src/kernel/cpu/vae.rs:297-334 (rmsnorm_heads_with), reached from
+ * gemma_rmsnorm_heads / rmsnorm_heads (src/backend/cpu/attention.rs:365-371,
+ * 463-470): out = x * (1 / sqrt(sum(x^2) / head_dim + eps)) * (weight + offset),
+ * offset 1 for the Gemma form, 0 for the plain form; weight NULL = no weight.
+ * The sum of squares runs over eight lane accumulators (element e feeds lane
+ * e % 8, chunks in ascending order) that are then added as the `wide` crate's
+ * f32x8::reduce_add does on AVX -- lanes (l, l + 4), then (0, 2) and (1, 3),
+ * then the two halves -- followed by the tail elements in order.  PARITY
+ * UNPINNED at bit level: `wide` is a third-party dependency (not vendored) and
+ * its reduction order is taken from its published source; the reference's own
+ * tests (src/kernel/cpu/rmsnorm.rs:70-103) hold to 1e-6 / 1e-5 only. */
+ZO_API int zo_rmsnorm_heads_f32(const float* input, uint64_t rows, uint64_t head_count, uint64_t head_dim,
+                                const float* weight, float eps, float weight_offset, float* out)
+{
+    if (head_count == 0 || head_dim == 0 || (weight != NULL && (!isfinite(eps) || eps <= 0.0f))) {
+        return -1;
+    }
+    uint64_t lanes = head_dim / 8 * 8;
+    for (uint64_t unit = 0; unit < rows * head_count; ++unit) {
+        const float* source = input + unit * head_dim;
+        float* target = out + unit * head_dim;
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (uint64_t c = 0; c < lanes; c += 8) {
+            for (int l = 0; l < 8; ++l) {
+                acc[l] += source[c + l] * source[c + l];
+            }
+        }
+        float sum = ((acc[0] + acc[4]) + (acc[2] + acc[6])) + ((acc[1] + acc[5]) + (acc[3] + acc[7]));
+        for (uint64_t c = lanes; c < head_dim; ++c) {
+            sum += source[c] * source[c];
+        }
+        float inverse = 1.0f / sqrtf(sum / (float)head_dim + eps);
+        for (uint64_t c = 0; c < head_dim; ++c) {
+            target[c] = weight != NULL ? source[c] * inverse * (weight[c] + weight_offset) : source[c] * inverse;
+        }
+    }
+    return 0;
+}
+
+/* src/backend/cpu/context.rs:419-432 (sigmoid_gate): out = input / (1 + exp(-gate)),
+ * one gate per element or one per row (gate_cols == 1). */
+ZO_API int zo_sigmoid_gate_f32(const float* input, const float* gate, uint64_t rows, uint64_t cols, uint64_t gate_cols,
+                               float* out)
+{
+    if (gate_cols != 1 && gate_cols != cols) {
+        return -1;
+    }
+    for (uint64_t row = 0; row < rows; ++row) {
+        for (uint64_t c = 0; c < cols; ++c) {
+            float value = gate[row * gate_cols + (gate_cols == 1 ? 0 : c)];
+            out[row * cols + c] = input[row * cols + c] * (1.0f / (1.0f + expf(-value)));
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
 /* MLA attention                                                             */
 /* ------------------------------------------------------------------------ */
 

@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported(lib):
 def test_struct_sizes_follow_the_header():
     # pointers first, then 32-bit fields: natural alignment, no surprises for an FFI binding
     assert C.sizeof(capi.Q8AppendArgs) == 5 * 8 + 7 * 4 + 4
-    assert C.sizeof(capi.GqaDecodeArgs) == 10 * 8 + 8 + 9 * 4 + 2 * 4 + 3 * 4 + 4 + 4  # + tail padding
+    assert C.sizeof(capi.GqaDecodeArgs) == 10 * 8 + 8 + 9 * 4 + 2 * 4 + 3 * 4 + 4 + 4 + 8 + 4 + 4  # + padding, gate fields
     assert C.sizeof(capi.MlaDecodeArgs) == 9 * 8 + 8 + 9 * 4 + 3 * 4 + 4 + 4 + 2 * 8  # stage_mask, top_k, selection pointers
 
 

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 
-def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_capacity=0):
+def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_capacity=0, gate=None):
     from zllm_amd import capi, ops
 
     pl = case["planes"]
@@ -24,9 +24,24 @@ def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_c
     out = ops.gqa_decode(q, upload(pl["k_codes"]), upload(pl["k_scales"]), upload(pl["v_codes"]), upload(pl["v_scales"]),
                          upload(case["tables"]), upload(lens), case["hq"], case["hkv"], case["d"], case["block_tokens"],
                          score_scale, max_kv_len or max(int(lens.max()), 1), first_visible=first, softcap=softcap,
-                         ring_capacity=ring_capacity, kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"])
+                         ring_capacity=ring_capacity, kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"], gate=gate)
     torch.cuda.synchronize()
     return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("per_row,gate_bf16", [(False, False), (True, False), (False, True)])
+def test_decode_output_gate(per_row, gate_bf16):
+    """out * sigmoid(gate) fused into the split merge (src/attention/hybrid.rs:79, src/backend/cpu/context.rs:419-432)."""
+    case = make_gqa_q8_case(91, [700, 33, 2049], 16, 4, 128)
+    rng = np.random.default_rng(92)
+    gate = (rng.standard_normal((3, 1 if per_row else 16 * 128)) * 3).astype(np.float32)
+    if gate_bf16:
+        gate = O.bf16_to_f32(O.f32_to_bf16(gate))
+    dev_gate = to_torch_bf16(O.f32_to_bf16(gate), "cuda") if gate_bf16 else upload(gate)
+    got = run_decode(case, 0.088, gate=dev_gate)
+    rc, want = O.sigmoid_gate(oracle_gqa_decode(case, 0.088), gate)
+    assert rc == 0
+    assert_attention_close(got, want, "gated decode")
 
 
 def test_config1_cpu_oracle_case():

@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
-             out_dtype=None, scale=None, outliers=False):
+             out_dtype=None, scale=None, outliers=False, gate_cols=0):
     from zllm_amd import capi, ops
 
     d = 128
@@ -55,15 +55,26 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     q_bits = O.f32_to_bf16(q)
     q = O.bf16_to_f32(q_bits) if q_bf16 else q
     scale = scale or 1.0 / np.sqrt(d)
+    gate = (rng.standard_normal((chunk, gate_cols)) * 3).astype(np.float32) if gate_cols else None
     out = ops.gqa_prefill_chunk(to_torch_bf16(q_bits, "cuda") if q_bf16 else upload(q), dev["k_codes"], dev["k_scales"], dev["v_codes"],
                                 dev["v_scales"], table, prefix, hq, hkv, d, block_tokens, scale, window=window, softcap=softcap,
-                                scale_dtype=sdt, out_dtype=out_dtype)
+                                scale_dtype=sdt, out_dtype=out_dtype, gate=None if gate is None else upload(gate))
     torch.cuda.synchronize()
     kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, tables[0], block_tokens, 0, total, cols)
     vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, tables[0], block_tokens, 0, total, cols)
     rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
     assert rc == 0
+    if gate is not None:
+        rc, want = O.sigmoid_gate(want, gate)
+        assert rc == 0
     return out, want
+
+
+@pytest.mark.parametrize("gate_cols", [8 * 128, 1])
+def test_prefill_output_gate(gate_cols):
+    """out * sigmoid(gate), one gate per element or per row (src/attention/hybrid.rs:79, src/backend/cpu/context.rs:419-432)."""
+    out, want = run_case(31 + gate_cols, 200, 70, 8, 2, gate_cols=gate_cols)
+    assert_attention_close(out.cpu().numpy(), want, f"gate_cols={gate_cols}")
 
 
 @pytest.mark.parametrize("prefix,chunk,hq,hkv", [(1000, 200, 64, 8), (0, 77, 8, 2), (333, 1, 16, 4), (50, 300, 8, 8), (700, 65, 12, 3),

@@ -206,3 +206,27 @@ def test_q8g64_appends_at_position_offset(oracle):
     assert (codes[:rows] == keep).all()
     deq = codes[rows:].astype(np.float32) * np.repeat(scales[rows:], 64, axis=1)
     assert (np.abs(deq - second) <= np.repeat(scales[rows:], 64, axis=1) / 2 + 1e-6).all()
+
+
+# ---- src/kernel/cpu/rmsnorm.rs:70-86 (Gemma weight reads as 1 + gamma) -----------------------------
+def test_rmsnorm_heads_gemma_weight_is_one_plus_gamma(oracle):
+    x = np.arange(1, 9, dtype=np.float32)
+    w = np.array([[0.0, 0.5, -0.5, 1.0][i % 4] for i in range(8)], dtype=np.float32)
+    rc, plain = oracle.rmsnorm_heads(x[None, :], 1, 8, w, 1.0e-6, 0.0)
+    assert rc == 0
+    rc, gemma = oracle.rmsnorm_heads(x[None, :], 1, 8, w, 1.0e-6, 1.0)
+    assert rc == 0
+    inv = 1.0 / np.sqrt((x.astype(np.float64) ** 2).mean() + 1.0e-6)
+    assert np.abs(plain.ravel() - x * inv * w).max() < 1.0e-6
+    assert np.abs(gemma.ravel() - x * inv * (1.0 + w)).max() < 1.0e-6
+
+
+# ---- src/kernel/cpu/rmsnorm.rs:88-103 (length that is not a multiple of eight: scalar tail) --------
+def test_rmsnorm_heads_scalar_tail(oracle):
+    x = np.arange(1, 12, dtype=np.float32)
+    w = (0.5 + np.arange(11) * 0.1).astype(np.float32)
+    inv = 1.0 / np.sqrt((x.astype(np.float64) ** 2).mean() + 1.0e-6)
+    for offset in (0.0, 1.0):
+        rc, out = oracle.rmsnorm_heads(x[None, :], 1, 11, w, 1.0e-6, offset)
+        assert rc == 0
+        assert np.abs(out.ravel() - x * inv * (offset + w)).max() < 1.0e-5

@@ -298,3 +298,26 @@ def test_absorbed_q8_selection_equals_dense_attention_over_the_gathered_rows(ora
     bad = sel.copy()
     bad[0] = rows
     assert oracle.mla_absorbed_q8_history(spec, q, 1, rows - 1, codes, scales, 64, rope_rows, rows, kv_b, selection=bad, width=width)[0] != 0
+
+
+def test_rmsnorm_heads_and_sigmoid_gate_against_float64(oracle):
+    """Heads are normalised independently (a scaled copy of a head normalises to the same vector), every head of unit
+    weight has mean square 1 - eps-ish, and the gate is the logistic function."""
+    rng = np.random.default_rng(5)
+    rows, heads, dim = 3, 4, 128
+    x = rng.standard_normal((rows, heads * dim)).astype(np.float32)
+    x[:, dim:2 * dim] = 7.5 * x[:, :dim]
+    w = (rng.standard_normal(dim) * 0.1).astype(np.float32)
+    rc, out = oracle.rmsnorm_heads(x, heads, dim, w, 1e-6, 1.0)
+    assert rc == 0
+    x64 = x.astype(np.float64).reshape(rows, heads, dim)
+    want = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * (1.0 + w.astype(np.float64))
+    assert np.abs(out.reshape(rows, heads, dim) - want).max() < 2e-6
+    assert np.abs(out[:, :dim] - out[:, dim:2 * dim]).max() < 5e-6  # eps is not scaled with the head
+    gate = rng.standard_normal((rows, heads * dim)).astype(np.float32) * 4
+    rc, gated = oracle.sigmoid_gate(out, gate)
+    assert rc == 0
+    assert np.abs(gated - out / (1.0 + np.exp(-gate.astype(np.float64)))).max() < 1e-6
+    rc, per_row = oracle.sigmoid_gate(out, gate[:, :1])
+    assert rc == 0
+    assert np.abs(per_row - out / (1.0 + np.exp(-gate[:, :1].astype(np.float64)))).max() < 1e-6

@@ -29,6 +29,15 @@ class Q8AppendArgs(C.Structure):
                 ("src_dtype", _int), ("rule", _int)]
 
 
+class GqaPrologueArgs(C.Structure):
+    _fields_ = [("q", _ptr), ("k", _ptr), ("v", _ptr), ("q_norm", _ptr), ("k_norm", _ptr), ("cosine", _ptr), ("sine", _ptr),
+                ("q_out", _ptr), ("k_codes", _ptr), ("k_scales", _ptr), ("v_codes", _ptr), ("v_scales", _ptr), ("table", _ptr),
+                ("positions", _ptr), ("rows", _u32), ("num_heads", _u32), ("num_kv_heads", _u32), ("head_dim", _u32),
+                ("rotary_dim", _u32), ("rope_table_rows", _u32), ("position", _u32), ("block_tokens", _u32),
+                ("ring_capacity", _u32), ("eps", C.c_float), ("weight_offset", C.c_float), ("src_dtype", _int),
+                ("q_out_dtype", _int), ("rule", _int), ("split_half", _int)]
+
+
 class HalfAppendArgs(C.Structure):
     _fields_ = [("src", _ptr), ("cache", _ptr), ("table", _ptr), ("position", _u32), ("rows", _u32), ("cols", _u32),
                 ("block_tokens", _u32), ("ring_capacity", _u32), ("src_dtype", _int), ("dst_dtype", _int)]
@@ -52,7 +61,7 @@ class GqaDecodeArgs(C.Structure):
                 ("workspace_bytes", _u64), ("batch", _u32), ("num_heads", _u32), ("num_kv_heads", _u32),
                 ("head_dim", _u32), ("table_stride", _u32), ("max_kv_len", _u32), ("total_kv_tokens", _u32),
                 ("block_tokens", _u32), ("ring_capacity", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
-                ("scale_dtype", _int), ("q_dtype", _int), ("stages", _u32)]
+                ("scale_dtype", _int), ("q_dtype", _int), ("stages", _u32), ("gate", _ptr), ("gate_cols", _u32), ("gate_dtype", _int)]
 
 
 class GqaPrefillArgs(C.Structure):
@@ -60,7 +69,8 @@ class GqaPrefillArgs(C.Structure):
                 ("table", _ptr), ("out", _ptr), ("workspace", _ptr), ("workspace_bytes", _u64), ("rows", _u32),
                 ("position", _u32), ("window", _u32), ("num_heads", _u32), ("num_kv_heads", _u32), ("head_dim", _u32),
                 ("block_tokens", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
-                ("scale_dtype", _int), ("q_dtype", _int), ("out_dtype", _int)]
+                ("scale_dtype", _int), ("q_dtype", _int), ("out_dtype", _int), ("gate", _ptr), ("gate_cols", _u32),
+                ("gate_dtype", _int)]
 
 
 class MlaDecodeArgs(C.Structure):
@@ -82,6 +92,7 @@ SYMBOLS = {
     "zllm_kv_ring_write_plan": (_int, [_u64, _u64, _u64, _u64, C.POINTER(_u64)]),
     "zllm_attn_q8g64_append": (_int, [C.POINTER(Q8AppendArgs), _ptr]),
     "zllm_attn_half_append": (_int, [C.POINTER(HalfAppendArgs), _ptr]),
+    "zllm_attn_gqa_prologue": (_int, [C.POINTER(GqaPrologueArgs), _ptr]),
     "zllm_attn_mla_append": (_int, [C.POINTER(MlaAppendArgs), _ptr]),
     "zllm_attn_gather_rows": (_int, [C.POINTER(GatherArgs), _ptr]),
     "zllm_attn_gqa_decode_workspace_bytes": (_u64, [C.POINTER(GqaDecodeArgs)]),

@@ -309,6 +309,41 @@ int zllm_attn_q8g64_append(const zllm_q8_append_args* a, zllm_stream_t stream)
     return hip_status(zllm::launch_q8g64_append(p, (hipStream_t)stream), "Q8g64 append launch");
 }
 
+int zllm_attn_gqa_prologue(const zllm_gqa_prologue_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->q == nullptr || a->k == nullptr || a->v == nullptr || a->q_out == nullptr || a->k_codes == nullptr ||
+        a->k_scales == nullptr || a->v_codes == nullptr || a->v_scales == nullptr) {
+        return fail(-1, "GQA prologue: null pointer");
+    }
+    // shape rules of rmsnorm_heads (src/backend/cpu/attention.rs:463-467) and apply_f32 (src/attention/rope.rs:121-138)
+    if (a->rows == 0 || a->num_heads == 0 || a->num_kv_heads == 0 || a->head_dim == 0 || a->head_dim % ZLLM_GROUP_SIZE != 0 ||
+        a->head_dim > 256 || a->block_tokens == 0) {
+        return fail(-1, "GQA prologue: invalid shape rows=%u heads=%u/%u head_dim=%u block_tokens=%u", a->rows, a->num_heads,
+                    a->num_kv_heads, a->head_dim, a->block_tokens);
+    }
+    if (a->rotary_dim % 2 != 0 || a->rotary_dim > a->head_dim) {
+        return fail(-1, "GQA prologue: rotary_dim=%u must be even and at most head_dim=%u", a->rotary_dim, a->head_dim);
+    }
+    if (a->rotary_dim != 0 && (a->cosine == nullptr || a->sine == nullptr || (uint64_t)a->position + a->rows > a->rope_table_rows)) {
+        return fail(-1, "GQA prologue: RoPE table of %u rows cannot serve position %u + %u rows", a->rope_table_rows, a->position, a->rows);
+    }
+    if ((a->q_norm != nullptr || a->k_norm != nullptr) && !(a->eps > 0.0f && a->eps < INFINITY)) {
+        return fail(-1, "GQA prologue: eps must be finite and positive");
+    }
+    if (a->rule < ZLLM_QUANT_ROCM_MLA || a->rule > ZLLM_QUANT_CUDA_GQA || a->src_dtype < ZLLM_DTYPE_F32 || a->src_dtype > ZLLM_DTYPE_F16 ||
+        (a->q_out_dtype != ZLLM_DTYPE_F32 && a->q_out_dtype != ZLLM_DTYPE_BF16)) {
+        return fail(-1, "GQA prologue: unknown rule %d, src_dtype %d or q_out_dtype %d", a->rule, a->src_dtype, a->q_out_dtype);
+    }
+    if ((uint64_t)a->position + a->rows > 0xffffffffull) {
+        return fail(-1, "GQA prologue: position + rows overflows u32");
+    }
+    zllm::GqaPrologueParams p{a->q, a->k, a->v, a->q_norm, a->k_norm, a->cosine, a->sine, a->q_out, (signed char*)a->k_codes, a->k_scales,
+                              (signed char*)a->v_codes, a->v_scales, a->table, a->positions, a->rows, a->num_heads, a->num_kv_heads,
+                              a->head_dim, a->rotary_dim, a->position, a->block_tokens, a->ring_capacity, a->eps, a->weight_offset,
+                              a->src_dtype, a->q_out_dtype, a->rule, a->split_half};
+    return hip_status(zllm::launch_gqa_prologue(p, (hipStream_t)stream), "GQA prologue launch");
+}
+
 int zllm_attn_half_append(const zllm_half_append_args* a, zllm_stream_t stream)
 {
     if (a == nullptr || a->src == nullptr || a->cache == nullptr) {
@@ -424,6 +459,15 @@ int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
     p.score_scale = a->score_scale;
     p.softcap = a->softcap;
     p.q_dtype = a->q_dtype;
+    if (a->gate != nullptr) {
+        // shape rule of sigmoid_gate (src/backend/cpu/context.rs:420-422)
+        if ((a->gate_cols != 1 && a->gate_cols != a->num_heads * a->head_dim) || (a->gate_dtype != ZLLM_DTYPE_F32 && a->gate_dtype != ZLLM_DTYPE_BF16)) {
+            return fail(-1, "GQA decode: gate_cols=%u must be 1 or %u, gate_dtype f32 or bf16", a->gate_cols, a->num_heads * a->head_dim);
+        }
+        p.gate = a->gate;
+        p.gate_cols = a->gate_cols;
+        p.gate_dtype = a->gate_dtype;
+    }
     return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, a->stages, (hipStream_t)stream), "GQA decode launch");
 }
 
@@ -566,6 +610,14 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
     p.softcap = a->softcap;
     p.q_dtype = a->q_dtype;
     p.out_dtype = a->out_dtype;
+    if (a->gate != nullptr) {
+        if ((a->gate_cols != 1 && a->gate_cols != a->num_heads * a->head_dim) || (a->gate_dtype != ZLLM_DTYPE_F32 && a->gate_dtype != ZLLM_DTYPE_BF16)) {
+            return fail(-1, "GQA prefill: gate_cols=%u must be 1 or %u, gate_dtype f32 or bf16", a->gate_cols, a->num_heads * a->head_dim);
+        }
+        p.gate = a->gate;
+        p.gate_cols = a->gate_cols;
+        p.gate_dtype = a->gate_dtype;
+    }
     return hip_status(zllm::launch_gqa_prefill(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA prefill launch");
 }
 

@@ -6,6 +6,12 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+// Every product and sum in this file is rounded on its own, as in the CPU code these kernels must agree with bit for
+// bit.  Expressions of more than one operation are written with plain operators under this pragma: the __fmul_rn /
+// __fadd_rn intrinsics are ordinary operators compiled in a header where fusing is allowed, so a product and a sum
+// written through them still become one multiply-add.
+#pragma clang fp contract(off)
+
 namespace zllm {
 
 __device__ __forceinline__ float wave_max_all(float v)
@@ -117,8 +123,7 @@ __global__ __launch_bounds__(64) void mla_append_kernel(MlaAppendParams p)
             const float imaginary = p.k_rope[(unsigned long long)row * p.rope_cols + imag_column];
             const float c = p.cosine[(unsigned long long)(rope_position + row) * half + pair];
             const float s = p.sine[(unsigned long long)(rope_position + row) * half + pair];
-            value = column == real_column ? __fsub_rn(__fmul_rn(real, c), __fmul_rn(imaginary, s))
-                                          : __fadd_rn(__fmul_rn(imaginary, c), __fmul_rn(real, s));
+            value = column == real_column ? real * c - imaginary * s : imaginary * c + real * s;
         }
         p.rope_cache[physical * p.rope_cols + column] = f32_to_bf16_bits(value);
         return;
@@ -130,6 +135,112 @@ __global__ __launch_bounds__(64) void mla_append_kernel(MlaAppendParams p)
     const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, 0);
     const signed char code = quantize_lane(value, 0, p.latent_scales, physical * groups_per_row + group, lane);
     p.latent_codes[physical * p.latent_cols + column] = code;
+}
+
+// Pre-attention prologue: one wave per (row, head) of Q, K or V.  The head's values sit one per lane per 64-column
+// group (the layout the quantizer wants); the head goes through LDS once for the sum of squares and once for the
+// rotation partner.
+//   norm   (src/kernel/cpu/vae.rs:297-334): eight accumulators, element e into accumulator e % 8 in ascending order,
+//          added as (l, l + 4), (0, 2) | (1, 3), halves -- lanes 0..7 do exactly that, so the sum has the reference
+//          restatement's bits; then x * (1 / sqrt(sum / d + eps)) * (weight + offset), every step rounded on its own.
+//   rope   (src/attention/rope.rs:120-164): real * cos - imag * sin, imag * cos + real * sin, products rounded
+//          separately.
+//   K, V   quantize_lane + page scatter, as the append kernel.
+template <int GROUPS> __global__ __launch_bounds__(256) void gqa_prologue_kernel(GqaPrologueParams p)
+{
+    __shared__ float head_lds[4][GROUPS * 64];
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int wave = threadIdx.x >> 6;
+    const unsigned int heads_per_row = p.num_heads + 2u * p.num_kv_heads;
+    const unsigned long long unit = (unsigned long long)blockIdx.x * 4u + wave;
+    if (unit >= (unsigned long long)p.rows * heads_per_row) {
+        return;
+    }
+    const unsigned int row = (unsigned int)(unit / heads_per_row);
+    const unsigned int slot = (unsigned int)(unit - (unsigned long long)row * heads_per_row);
+    const unsigned int kind = slot < p.num_heads ? 0u : (slot < p.num_heads + p.num_kv_heads ? 1u : 2u); // Q, K, V
+    const unsigned int head = kind == 0u ? slot : (kind == 1u ? slot - p.num_heads : slot - p.num_heads - p.num_kv_heads);
+    const unsigned int head_count = kind == 0u ? p.num_heads : p.num_kv_heads;
+    const void* src = kind == 0u ? p.q : (kind == 1u ? p.k : p.v);
+    const float* weight = kind == 0u ? p.q_norm : (kind == 1u ? p.k_norm : nullptr);
+    const unsigned int d = GROUPS * 64u;
+    const size_t base = ((size_t)row * head_count + head) * d;
+    const unsigned int position = p.positions != nullptr ? p.positions[0] : p.position;
+    float* lds = head_lds[wave];
+    float x[GROUPS];
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        x[g] = load_as_f32(src, base + g * 64 + lane, p.src_dtype);
+    }
+    if (kind != 2u && weight != nullptr) {
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            lds[g * 64 + lane] = x[g];
+        }
+        __builtin_amdgcn_wave_barrier();
+        float acc = 0.0f;
+        if (lane < 8u) {
+            for (unsigned int c = 0; c < d; c += 8u) {
+                const float value = lds[c + lane];
+                acc = acc + value * value;
+            }
+        }
+        acc = acc + __shfl_xor(acc, 4);
+        acc = acc + __shfl_xor(acc, 2);
+        acc = acc + __shfl_xor(acc, 1);
+        const float sum = __shfl(acc, 0);
+        // sqrtf is correctly rounded (hipcc's default); __fsqrt_rn maps to the native approximation
+        const float inverse = 1.0f / sqrtf(sum / (float)d + p.eps);
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            x[g] = x[g] * inverse * (weight[g * 64 + lane] + p.weight_offset);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (kind != 2u && p.rotary_dim != 0u) {
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            lds[g * 64 + lane] = x[g];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const unsigned int half = p.rotary_dim / 2u;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            const unsigned int column = g * 64u + lane;
+            if (column < p.rotary_dim) {
+                const unsigned int pair = p.split_half ? column % half : column / 2u;
+                const unsigned int real_column = p.split_half ? pair : pair * 2u;
+                const unsigned int imag_column = p.split_half ? half + pair : pair * 2u + 1u;
+                const float real = lds[real_column];
+                const float imaginary = lds[imag_column];
+                const float c = p.cosine[(size_t)(position + row) * half + pair];
+                const float s = p.sine[(size_t)(position + row) * half + pair];
+                x[g] = column == real_column ? real * c - imaginary * s : imaginary * c + real * s;
+            }
+        }
+    }
+    if (kind == 0u) {
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (p.q_out_dtype == 0) {
+                ((float*)p.q_out)[base + g * 64 + lane] = x[g];
+            } else {
+                ((unsigned short*)p.q_out)[base + g * 64 + lane] = f32_to_bf16_bits(x[g]);
+            }
+        }
+        return;
+    }
+    const unsigned int cols = p.num_kv_heads * d;
+    const unsigned int groups_per_row = cols / 64u;
+    const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, p.ring_capacity);
+    signed char* codes = kind == 1u ? p.k_codes : p.v_codes;
+    void* scales = kind == 1u ? p.k_scales : p.v_scales;
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const unsigned int group = head * GROUPS + g;
+        const signed char code = quantize_lane(x[g], p.rule, scales, physical * groups_per_row + group, lane);
+        codes[physical * cols + group * 64u + lane] = code;
+    }
 }
 
 template <typename T> __global__ __launch_bounds__(256) void gather_rows_kernel(GatherParams p, unsigned int units_per_row)
@@ -162,6 +273,20 @@ hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream)
         return hipSuccess;
     }
     half_append_kernel<<<dim3((unsigned int)((elements + 255) / 256)), dim3(256), 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+hipError_t launch_gqa_prologue(const GqaPrologueParams& p, hipStream_t stream)
+{
+    const unsigned long long units = (unsigned long long)p.rows * (p.num_heads + 2u * p.num_kv_heads);
+    const dim3 grid((unsigned int)((units + 3) / 4));
+    switch (p.head_dim / 64u) {
+    case 1: gqa_prologue_kernel<1><<<grid, dim3(256), 0, stream>>>(p); break;
+    case 2: gqa_prologue_kernel<2><<<grid, dim3(256), 0, stream>>>(p); break;
+    case 3: gqa_prologue_kernel<3><<<grid, dim3(256), 0, stream>>>(p); break;
+    case 4: gqa_prologue_kernel<4><<<grid, dim3(256), 0, stream>>>(p); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

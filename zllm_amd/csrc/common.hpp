@@ -75,6 +75,14 @@ __device__ __forceinline__ float load_as_f32(const void* base, size_t index, int
 // Logical token -> physical cache row
 // (src/kernel/rocm/hip/attention/paged_mla/source.hip:46-54), with the optional
 // sliding-window ring applied first (src/kernel/cuda/attention.rs:82-88).
+// out * sigmoid(gate): the output gate of a gated attention layer (src/backend/cpu/context.rs:419-432).
+// `row` indexes the gate's rows, `column` its columns (ignored when the gate has one column).
+__device__ __forceinline__ float gated(float value, const void* gate, unsigned int gate_cols, int gate_dtype, size_t row, unsigned int column)
+{
+    const float g = load_as_f32(gate, row * gate_cols + (gate_cols == 1u ? 0u : column), gate_dtype);
+    return value * (1.0f / (1.0f + __expf(-g)));
+}
+
 __device__ __forceinline__ unsigned long long paged_row(const unsigned int* table, unsigned int token,
                                                         unsigned int block_tokens, unsigned int ring_capacity)
 {

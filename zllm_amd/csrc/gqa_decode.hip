@@ -1192,6 +1192,12 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
         if (denom > 0.0f && denom < __builtin_inff()) {
             result = total * (1.0f / denom);
         }
+        if (p.gate != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                result[e] = gated(result[e], p.gate, p.gate_cols, p.gate_dtype, b, head * p.head_dim + quad * 4u + e);
+            }
+        }
         *(f32x4*)(p.out + ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u) = result;
     }
 }

@@ -385,6 +385,12 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                 v = f32x4{0.f, 0.f, 0.f, 0.f};
             }
             const size_t at = base + t * 16 + 4 * j;
+            if (p.gate != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = gated(v[e], p.gate, p.gate_cols, p.gate_dtype, col_row[ct], col_head[ct] * kD + t * 16 + 4 * j + e);
+                }
+            }
             if (p.out_dtype == 0) {
                 *(f32x4*)((float*)p.out + at) = v;
             } else {

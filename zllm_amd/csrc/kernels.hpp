@@ -16,6 +16,26 @@ struct Q8AppendParams {
     int src_dtype, rule;
 };
 
+struct GqaPrologueParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const float* q_norm;
+    const float* k_norm;
+    const float* cosine;
+    const float* sine;
+    void* q_out;
+    signed char* k_codes;
+    void* k_scales;
+    signed char* v_codes;
+    void* v_scales;
+    const unsigned int* table;
+    const unsigned int* positions;
+    unsigned int rows, num_heads, num_kv_heads, head_dim, rotary_dim, position, block_tokens, ring_capacity;
+    float eps, weight_offset;
+    int src_dtype, q_out_dtype, rule, split_half;
+};
+
 struct HalfAppendParams {
     const void* src;
     unsigned short* cache;
@@ -67,6 +87,9 @@ struct GqaDecodeParams {
     unsigned int chunk_tokens, max_chunks;
     float score_scale, softcap;
     int q_dtype;
+    const void* gate; // optional sigmoid output gate [batch][gate_cols]
+    unsigned int gate_cols;
+    int gate_dtype;
 };
 
 struct GqaPrefillParams {
@@ -82,6 +105,9 @@ struct GqaPrefillParams {
     unsigned int block_tokens, block_shift;
     float score_scale, softcap;
     int q_dtype, out_dtype;
+    const void* gate; // optional sigmoid output gate [rows][gate_cols]
+    unsigned int gate_cols;
+    int gate_dtype;
 };
 
 struct MlaDecodeParams {
@@ -111,6 +137,7 @@ struct MlaDecodeParams {
 unsigned int gqa_decode_max_waves(unsigned int head_dim);
 
 hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream);
+hipError_t launch_gqa_prologue(const GqaPrologueParams& p, hipStream_t stream);
 hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream);
 hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream);
 hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);

@@ -108,6 +108,9 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
     const unsigned int pairs = p.latent_dim / 2u;
     const unsigned int* w = (const unsigned int*)(p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim);
     for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
+        // product and sum rounded separately, as in the CPU code (plain operators: the __fmul_rn / __fadd_rn intrinsics
+        // are ordinary operators from a header compiled with fusing allowed)
+#pragma clang fp contract(off)
         float acc0 = 0.0f, acc1 = 0.0f;
         for (unsigned int k0 = 0; k0 < p.nope_dim; k0 += 32u) {
             unsigned int word[32];
@@ -118,8 +121,8 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 #pragma unroll
             for (int u = 0; u < 32; ++u) {
                 if (k0 + u < p.nope_dim) {
-                    acc0 = __fadd_rn(acc0, __fmul_rn(q_sh[k0 + u], __uint_as_float(word[u] << 16)));
-                    acc1 = __fadd_rn(acc1, __fmul_rn(q_sh[k0 + u], __uint_as_float(word[u] & 0xffff0000u)));
+                    acc0 = acc0 + q_sh[k0 + u] * __uint_as_float(word[u] << 16);
+                    acc1 = acc1 + q_sh[k0 + u] * __uint_as_float(word[u] & 0xffff0000u);
                 }
             }
         }

@@ -42,6 +42,27 @@ def q8g64_append(src, codes, scales, table, position, block_tokens, rule, ring_c
     capi.check(capi.load().zllm_attn_q8g64_append(C.byref(args), _stream()))
 
 
+def gqa_prologue(q, k, v, q_norm, k_norm, cos, sin, k_codes, k_scales, v_codes, v_scales, table, position, num_heads,
+                 num_kv_heads, head_dim, rotary_dim, block_tokens, eps=1e-6, weight_offset=1.0, rule=capi.QUANT_METAL_GQA,
+                 split_half=True, q_out_dtype=torch.float32, ring_capacity=0, positions=None):
+    """Per-head RMSNorm + RoPE of Q and K, Q out as a tensor, K and V quantized into the pages (zllm_attn_gqa_prologue)."""
+    rows = q.shape[0]
+    q_out = torch.empty((rows, num_heads * head_dim), dtype=q_out_dtype, device=q.device)
+    args = capi.GqaPrologueArgs()
+    args.q, args.k, args.v = _ptr(q), _ptr(k), _ptr(v)
+    args.q_norm, args.k_norm, args.cosine, args.sine = _ptr(q_norm), _ptr(k_norm), _ptr(cos), _ptr(sin)
+    args.q_out, args.k_codes, args.k_scales = _ptr(q_out), _ptr(k_codes), _ptr(k_scales)
+    args.v_codes, args.v_scales, args.table, args.positions = _ptr(v_codes), _ptr(v_scales), _ptr(table), _ptr(positions)
+    args.rows, args.num_heads, args.num_kv_heads, args.head_dim = rows, num_heads, num_kv_heads, head_dim
+    args.rotary_dim = rotary_dim
+    args.rope_table_rows = 0 if cos is None else cos.shape[0]
+    args.position, args.block_tokens, args.ring_capacity = position, block_tokens, ring_capacity
+    args.eps, args.weight_offset = eps, weight_offset
+    args.src_dtype, args.q_out_dtype, args.rule, args.split_half = _DTYPE[q.dtype], _DTYPE[q_out_dtype], rule, int(split_half)
+    capi.check(capi.load().zllm_attn_gqa_prologue(C.byref(args), _stream()))
+    return q_out
+
+
 def half_append(src, cache, table, position, block_tokens, ring_capacity=0):
     _dev(src, "src"), _dev(cache, "cache"), _dev(table, "table")
     dst = capi.DTYPE_BF16 if cache.dtype == torch.bfloat16 else capi.DTYPE_F16
@@ -71,7 +92,7 @@ def gather_rows(plane, table, first, count, row_bytes, block_tokens, ring_capaci
 
 def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, num_heads, num_kv_heads, head_dim,
                     block_tokens, score_scale, max_kv_len, first_visible=None, softcap=0.0, ring_capacity=0,
-                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None, total_kv_tokens=0):
+                    kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None, total_kv_tokens=0, gate=None):
     batch = q.shape[0]
     if out is None:
         out = torch.empty((batch, num_heads * head_dim), dtype=torch.float32, device=q.device)
@@ -86,6 +107,8 @@ def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, nu
     args.total_kv_tokens = total_kv_tokens
     args.score_scale, args.softcap = score_scale, softcap
     args.kv_format, args.scale_dtype, args.q_dtype = kv_format, scale_dtype, _DTYPE[q.dtype]
+    if gate is not None:
+        args.gate, args.gate_cols, args.gate_dtype = _ptr(gate), gate.shape[1], _DTYPE[gate.dtype]
     need = capi.load().zllm_attn_gqa_decode_workspace_bytes(C.byref(args))
     if need == 0:
         raise capi.ZllmAttnError(-1, capi.last_error())
@@ -104,7 +127,7 @@ def gqa_decode(*a, **kw):
 
 def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, num_heads, num_kv_heads, head_dim,
                       block_tokens, score_scale, window=0, softcap=0.0, kv_format=capi.KV_Q8G64,
-                      scale_dtype=capi.SCALE_F16, out_dtype=torch.float32):
+                      scale_dtype=capi.SCALE_F16, out_dtype=torch.float32, gate=None):
     rows = q.shape[0]
     out = torch.empty((rows, num_heads * head_dim), dtype=out_dtype, device=q.device)
     args = capi.GqaPrefillArgs()
@@ -115,6 +138,8 @@ def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, 
     args.score_scale, args.softcap = score_scale, softcap
     args.kv_format, args.scale_dtype = kv_format, scale_dtype
     args.q_dtype, args.out_dtype = _DTYPE[q.dtype], _DTYPE[out_dtype]
+    if gate is not None:
+        args.gate, args.gate_cols, args.gate_dtype = _ptr(gate), gate.shape[1], _DTYPE[gate.dtype]
     need = capi.load().zllm_attn_gqa_prefill_workspace_bytes(C.byref(args))
     workspace = torch.empty(max(int(need), 256), dtype=torch.uint8, device=q.device)
     args.workspace, args.workspace_bytes = _ptr(workspace), workspace.numel()
