@@ -179,6 +179,49 @@ typedef struct zllm_gather_args {
 } zllm_gather_args;
 ZLLM_API int zllm_attn_gather_rows(const zllm_gather_args* args, zllm_stream_t stream);
 
+/* Inverse of zllm_attn_gather_rows: plane[paged_row(first + r)] = in[r].  Serves KV snapshot upload
+ * (the restore half of src/backend/rocm/kv_cache.rs:3344-3598: a downloaded layer goes back into
+ * whatever pages the restored sequence owns). */
+typedef struct zllm_scatter_args {
+    void* plane;           /* [dev] */
+    const void* in;        /* [dev] [count, row_bytes] dense */
+    const uint32_t* table; /* [dev] or NULL */
+    uint32_t first, count, row_bytes, block_tokens, ring_capacity;
+} zllm_scatter_args;
+ZLLM_API int zllm_attn_scatter_rows(const zllm_scatter_args* args, zllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * KV snapshot wire format of one MLA layer (host side, no device access).     *
+ * ------------------------------------------------------------------------- */
+
+/* MlaLayerSerde (src/backend/rocm/kv_cache.rs:2067-2083) as write_mla_layer / read_mla_layer
+ * put it on the wire (src/runtime/glm52/rocm_swap.rs:1090-1138; integers are u64 little-endian,
+ * rocm_swap.rs:1145-1153):
+ *   rows, ownership byte (0 Full, 1 BlockParity(0), 2 BlockParity(1), 3 InterleavedPair),
+ *   latent_cols, rope_cols, latent_group_size, len + latent bytes,
+ *   flag byte (+ len + scale bytes when 1), len + rope bytes.
+ * latent_group_size 0 = bf16 latent without scales; otherwise Q8 codes + bf16 scales. */
+typedef struct zllm_mla_layer_record {
+    uint64_t rows;
+    uint32_t ownership;           /* ZLLM_KV_OWNERSHIP_* */
+    uint64_t latent_cols, rope_cols, latent_group_size;
+    const uint8_t* latent;        /* [host] rows * latent_cols (Q8) or * 2 (bf16) bytes */
+    uint64_t latent_bytes;
+    const uint8_t* latent_scales; /* [host] rows * (latent_cols / group) * 2 bytes, or NULL */
+    uint64_t latent_scales_bytes;
+    const uint8_t* rope;          /* [host] rows * rope_cols * 2 bytes */
+    uint64_t rope_bytes;
+} zllm_mla_layer_record;
+enum { ZLLM_KV_OWNERSHIP_FULL = 0, ZLLM_KV_OWNERSHIP_PARITY0 = 1, ZLLM_KV_OWNERSHIP_PARITY1 = 2, ZLLM_KV_OWNERSHIP_INTERLEAVED = 3 };
+/* Bytes write would produce; 0 when the record's lengths do not match its shape. */
+ZLLM_API uint64_t zllm_kv_mla_layer_wire_bytes(const zllm_mla_layer_record* record);
+/* Serialise into out[0 .. capacity); *written = bytes produced.  0 ok, -1 invalid / too small. */
+ZLLM_API int zllm_kv_mla_layer_write(const zllm_mla_layer_record* record, uint8_t* out, uint64_t capacity, uint64_t* written);
+/* Parse one record from in[0 .. len): pointers in *record point into `in`; *consumed = bytes read.
+ * 0 ok, -1 truncated or malformed (same conditions as read_mla_layer's errors), -2 shape and
+ * blob lengths disagree. */
+ZLLM_API int zllm_kv_mla_layer_read(const uint8_t* in, uint64_t len, zllm_mla_layer_record* record, uint64_t* consumed);
+
 /* ------------------------------------------------------------------------- *
  * GQA decode: one query row per sequence, split-KV flash decoding.           *
  * ------------------------------------------------------------------------- */

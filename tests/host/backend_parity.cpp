@@ -250,6 +250,60 @@ static void test_mla(const RocmContext& ctx)
     CHECK(rc == 0, "oracle rc %d", rc);
     compare(got.unwrap(), want, "mla_decode_attention after append_mla + append_mla_rope");
 
+    // session snapshot: download -> wire bytes -> parse -> upload into a second cache (other pages), same result bit for bit
+    {
+        auto layers = ctx.download_layers(cache);
+        CHECK(layers.is_ok(), "download_layers: %s", layers.is_err() ? layers.unwrap_err().to_string().c_str() : "");
+        std::vector<uint8_t> bytes;
+        for (const auto& record : layers.unwrap()) {
+            CHECK(record.has_value() && write_mla_layer(bytes, *record).is_ok(), "write_mla_layer");
+        }
+        const MlaLayerSerde& first = *layers.unwrap()[layer];
+        CHECK(first.rows == ctx_len && first.latent.size() == ctx_len * 512 && memcmp(first.latent.data(), codes_dense.data(), first.latent.size()) == 0 &&
+                  memcmp(first.latent_scales->data(), scales_dense.data(), ctx_len * 16) == 0 && memcmp(first.rope.data(), rope_dense.data(), ctx_len * 128) == 0,
+              "downloaded layer differs from the oracle's dense history");
+        std::vector<std::optional<MlaLayerSerde>> parsed;
+        size_t offset = 0;
+        for (size_t l = 0; l < cache.layers(); ++l) {
+            auto record = read_mla_layer(bytes, offset);
+            CHECK(record.is_ok(), "read_mla_layer: %s", record.is_err() ? record.unwrap_err().to_string().c_str() : "");
+            parsed.push_back(record.unwrap());
+        }
+        CHECK(offset == bytes.size(), "wire bytes left over");
+        auto other = RocmKvCache::new_mla(cache.layers(), 512, 64, 32, 640); // 32-token pages instead of 64
+        CHECK(other.is_ok(), "second cache");
+        auto restored = ctx.upload_layers(other.unwrap(), parsed);
+        CHECK(restored.is_ok() && other.unwrap().len(layer) == ctx_len, "upload_layers");
+        auto again = ctx.mla_decode_attention(qt.unwrap(), other.unwrap(), weight.unwrap(), layer, ctx_len - 1, spec);
+        CHECK(again.is_ok(), "decode on the restored cache");
+        if (again.is_ok()) {
+            auto same = ctx.tensor_to_f32(again.unwrap());
+            CHECK(same.unwrap() == got.unwrap(), "restored cache decodes differently");
+        }
+        std::vector<uint8_t> cut(bytes.begin(), bytes.end() - 1);
+        size_t at = 0;
+        bool failed = false;
+        for (size_t l = 0; l < cache.layers() && !failed; ++l) {
+            failed = read_mla_layer(cut, at).is_err();
+        }
+        CHECK(failed, "a truncated snapshot must be refused");
+        // rollback: the logical length moves back, a stale position is refused, a shorter decode works
+        CHECK(other.unwrap().truncate_layer_rows(layer, ctx_len + 1).is_err(), "truncate beyond the current length");
+        CHECK(other.unwrap().truncate_layer_rows(99, 1).is_err(), "truncate of a layer the cache does not have");
+        CHECK(other.unwrap().truncate_layer_rows(layer, 100).is_ok() && other.unwrap().len(layer) == 100, "truncate_layer_rows");
+        CHECK(ctx.mla_decode_attention(qt.unwrap(), other.unwrap(), weight.unwrap(), layer, ctx_len - 1, spec).is_err(), "stale position after rollback");
+        auto shorter = ctx.mla_decode_attention(qt.unwrap(), other.unwrap(), weight.unwrap(), layer, 99, spec);
+        CHECK(shorter.is_ok(), "decode after rollback");
+        if (shorter.is_ok()) {
+            std::vector<float> want_short(spec.num_heads * spec.value_dim());
+            const int rc2 = zo_mla_absorbed_q8_history(&zs, q_bits.data(), 1, 99, codes_dense.data(), scales_dense.data(), 64, rope_dense.data(), 100,
+                                                       kv_b.data(), nullptr, 0, nullptr, want_short.data(), nullptr);
+            CHECK(rc2 == 0, "oracle rc %d", rc2);
+            compare(ctx.tensor_to_f32(shorter.unwrap()).unwrap(), want_short, "mla_decode_attention after truncate_layer_rows(100)");
+        }
+        CHECK(other.unwrap().truncate_rows(0).is_ok() && other.unwrap().len(layer) == 0, "truncate_rows(0)");
+    }
+
     auto stale = ctx.mla_decode_attention(qt.unwrap(), cache, weight.unwrap(), layer, ctx_len + 5, spec);
     CHECK(stale.is_err(), "a position beyond the cache must be an error");
     MlaSpec bad = spec;

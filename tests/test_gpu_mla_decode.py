@@ -223,3 +223,73 @@ def test_mla_reference_split_test_recipe():
     want_f, _ = oracle_mla(case)
     got = run_mla(case).cpu().numpy()
     assert np.abs(got - want_f).max() <= 5e-3
+
+
+def test_mla_layer_snapshot_round_trip_and_rollback():
+    """Download a layer through its block table (gather), put it on the wire as the reference's MlaLayerSerde record,
+    parse it, upload it into differently placed pages (scatter): decode over the restored cache is bit-identical.  Then
+    rollback as truncate_layer_rows does it (src/backend/rocm/kv_cache.rs:509-586): only the logical length moves, and an
+    append after it overwrites the tail."""
+    import ctypes as C
+
+    from oracle import wire
+    from zllm_amd import capi, ops
+
+    lens = [333]
+    case = make_mla_case(901, lens, 16, block_tokens=16)
+    bt, rows = 16, lens[0]
+    dev = {n: upload(case[n]) for n in ("codes", "scales", "rope")}
+    table = upload(case["tables"][0])
+    row_bytes = {"codes": 512, "scales": 16, "rope": 128}
+    host = {n: ops.gather_rows(dev[n].view(torch.uint8) if dev[n].dtype != torch.uint8 else dev[n], table, 0, rows, row_bytes[n], bt).cpu().numpy().tobytes()
+            for n in dev}
+    record = wire.MlaLayerSerde(rows, "Full", 512, 64, 64, host["codes"], host["scales"], host["rope"])
+    lib = capi.load()
+    keep = []
+    rec = capi.MlaLayerRecord()
+    rec.rows, rec.ownership, rec.latent_cols, rec.rope_cols, rec.latent_group_size = rows, 0, 512, 64, 64
+    for name, field in (("codes", "latent"), ("scales", "latent_scales"), ("rope", "rope")):
+        buf = (C.c_uint8 * len(host[name])).from_buffer_copy(host[name])
+        keep.append(buf)
+        setattr(rec, field, C.cast(buf, C.c_void_p))
+        setattr(rec, field + "_bytes", len(host[name]))
+    need = lib.zllm_kv_mla_layer_wire_bytes(C.byref(rec))
+    out = (C.c_uint8 * need)()
+    written = C.c_uint64(0)
+    assert lib.zllm_kv_mla_layer_write(C.byref(rec), C.cast(out, C.c_void_p), need, C.byref(written)) == 0
+    assert bytes(out) == wire.write_mla_layer(record)  # what the reference's reader would be handed
+    parsed, used = capi.MlaLayerRecord(), C.c_uint64(0)
+    assert lib.zllm_kv_mla_layer_read(C.cast(out, C.c_void_p), need, C.byref(parsed), C.byref(used)) == 0
+    # restore into other pages
+    rng = np.random.default_rng(902)
+    tables2, pool_blocks2 = draw_tables(rng, lens, bt, layout="reversed")
+    pool_rows2 = pool_blocks2 * bt
+    restored = {"codes": torch.zeros((pool_rows2, 512), dtype=torch.uint8, device="cuda"),
+                "scales": torch.zeros((pool_rows2, 16), dtype=torch.uint8, device="cuda"),
+                "rope": torch.zeros((pool_rows2, 128), dtype=torch.uint8, device="cuda")}
+    table2 = upload(tables2[0])
+    for name, field in (("codes", "latent"), ("scales", "latent_scales"), ("rope", "rope")):
+        blob = np.frombuffer(C.string_at(getattr(parsed, field), getattr(parsed, field + "_bytes")), dtype=np.uint8)
+        ops.scatter_rows(restored[name], upload(blob.reshape(rows, row_bytes[name]).copy()), table2, 0, bt)
+    before = run_mla(case).cpu().numpy()
+    case2 = dict(case, codes=restored["codes"].view(torch.int8).cpu().numpy(), scales=restored["scales"].cpu().numpy().view(np.uint16),
+                 rope=restored["rope"].cpu().numpy().view(np.uint16), tables=tables2)
+    after = run_mla(case2).cpu().numpy()
+    assert np.array_equal(before, after)
+    # rollback to 300 rows, then append 10 other rows at position 300: the oracle over 310 rows must agree
+    keep_rows, extra = 300, 10
+    lat = rng.standard_normal((extra, 512)).astype(np.float32)
+    kr = rng.standard_normal((extra, 64)).astype(np.float32)
+    codes_t, scales_t, rope_t = (restored["codes"].view(torch.int8), restored["scales"].view(torch.int16), restored["rope"].view(torch.int16))
+    ops.mla_append(upload(lat), upload(kr), codes_t, scales_t, rope_t, table2, keep_rows, bt)
+    torch.cuda.synchronize()
+    ref = dict(case2)
+    ref["codes"], ref["scales"], ref["rope"] = case2["codes"].copy(), case2["scales"].copy(), case2["rope"].copy()
+    O.q8g64_append_paged(O.RULE_ROCM_MLA, lat, ref["codes"], ref["scales"], tables2[0], keep_rows, bt)
+    O.half_append_paged(0, kr, ref["rope"], tables2[0], keep_rows, bt)
+    ref["lens"] = np.array([keep_rows + extra], dtype=np.uint32)
+    want_f, _ = oracle_mla(ref)
+    live = dict(ref, codes=codes_t.cpu().numpy(), scales=scales_t.cpu().numpy().view(np.uint16), rope=rope_t.cpu().numpy().view(np.uint16))
+    assert np.array_equal(live["codes"], ref["codes"]) and np.array_equal(live["scales"], ref["scales"])
+    got = run_mla(live).cpu().numpy()
+    assert_attention_close(got, want_f, "rollback + append")

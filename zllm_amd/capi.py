@@ -55,6 +55,17 @@ class GatherArgs(C.Structure):
                 ("row_bytes", _u32), ("block_tokens", _u32), ("ring_capacity", _u32)]
 
 
+class ScatterArgs(C.Structure):
+    _fields_ = [("plane", _ptr), ("in_", _ptr), ("table", _ptr), ("first", _u32), ("count", _u32), ("row_bytes", _u32),
+                ("block_tokens", _u32), ("ring_capacity", _u32)]
+
+
+class MlaLayerRecord(C.Structure):
+    _fields_ = [("rows", _u64), ("ownership", _u32), ("latent_cols", _u64), ("rope_cols", _u64), ("latent_group_size", _u64),
+                ("latent", _ptr), ("latent_bytes", _u64), ("latent_scales", _ptr), ("latent_scales_bytes", _u64),
+                ("rope", _ptr), ("rope_bytes", _u64)]
+
+
 class GqaDecodeArgs(C.Structure):
     _fields_ = [("q", _ptr), ("k_plane", _ptr), ("k_scales", _ptr), ("v_plane", _ptr), ("v_scales", _ptr),
                 ("tables", _ptr), ("kv_lens", _ptr), ("first_visible", _ptr), ("out", _ptr), ("workspace", _ptr),
@@ -95,6 +106,10 @@ SYMBOLS = {
     "zllm_attn_gqa_prologue": (_int, [C.POINTER(GqaPrologueArgs), _ptr]),
     "zllm_attn_mla_append": (_int, [C.POINTER(MlaAppendArgs), _ptr]),
     "zllm_attn_gather_rows": (_int, [C.POINTER(GatherArgs), _ptr]),
+    "zllm_attn_scatter_rows": (_int, [C.POINTER(ScatterArgs), _ptr]),
+    "zllm_kv_mla_layer_wire_bytes": (_u64, [C.POINTER(MlaLayerRecord)]),
+    "zllm_kv_mla_layer_write": (_int, [C.POINTER(MlaLayerRecord), _ptr, _u64, C.POINTER(_u64)]),
+    "zllm_kv_mla_layer_read": (_int, [_ptr, _u64, C.POINTER(MlaLayerRecord), C.POINTER(_u64)]),
     "zllm_attn_gqa_decode_workspace_bytes": (_u64, [C.POINTER(GqaDecodeArgs)]),
     "zllm_attn_gqa_decode": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
     "zllm_attn_gqa_prefill_workspace_bytes": (_u64, [C.POINTER(GqaPrefillArgs)]),

@@ -397,6 +397,169 @@ int zllm_attn_gather_rows(const zllm_gather_args* a, zllm_stream_t stream)
     return hip_status(zllm::launch_gather_rows(p, (hipStream_t)stream), "gather rows launch");
 }
 
+int zllm_attn_scatter_rows(const zllm_scatter_args* a, zllm_stream_t stream)
+{
+    if (a == nullptr || a->plane == nullptr || a->in == nullptr) {
+        return fail(-1, "scatter rows: null pointer");
+    }
+    if (a->block_tokens == 0) {
+        return fail(-1, "scatter rows: block_tokens must be non-zero");
+    }
+    zllm::ScatterParams p{a->plane, a->in, a->table, a->first, a->count, a->row_bytes, a->block_tokens, a->ring_capacity};
+    return hip_status(zllm::launch_scatter_rows(p, (hipStream_t)stream), "scatter rows launch");
+}
+
+/* ---- KV snapshot wire format (host) ----------------------------------------------------- */
+
+static bool mla_record_shape_ok(const zllm_mla_layer_record* r)
+{
+    // download_device (src/backend/rocm/kv_cache.rs:3373-3388): Q8 codes are one byte per element with bf16 scales per
+    // group, the bf16 mode has two bytes per element and no scales
+    if (r->ownership > ZLLM_KV_OWNERSHIP_INTERLEAVED) {
+        return false;
+    }
+    if (r->latent_group_size == 0) {
+        return r->latent_scales == nullptr && r->latent_scales_bytes == 0 && r->latent_bytes == r->rows * r->latent_cols * 2 &&
+               r->rope_bytes == r->rows * r->rope_cols * 2;
+    }
+    return r->latent_cols % r->latent_group_size == 0 && r->latent_bytes == r->rows * r->latent_cols &&
+           r->latent_scales != nullptr && r->latent_scales_bytes == r->rows * (r->latent_cols / r->latent_group_size) * 2 &&
+           r->rope_bytes == r->rows * r->rope_cols * 2;
+}
+
+uint64_t zllm_kv_mla_layer_wire_bytes(const zllm_mla_layer_record* r)
+{
+    if (r == nullptr || !mla_record_shape_ok(r)) {
+        return 0;
+    }
+    return 8 + 1 + 3 * 8 + (8 + r->latent_bytes) + 1 + (r->latent_scales != nullptr ? 8 + r->latent_scales_bytes : 0) + (8 + r->rope_bytes);
+}
+
+static uint8_t* put_u64(uint8_t* at, uint64_t value)
+{
+    for (int i = 0; i < 8; ++i) {
+        at[i] = (uint8_t)(value >> (8 * i));
+    }
+    return at + 8;
+}
+
+static uint8_t* put_blob(uint8_t* at, const uint8_t* bytes, uint64_t len)
+{
+    at = put_u64(at, len);
+    if (len != 0) {
+        memcpy(at, bytes, len);
+    }
+    return at + len;
+}
+
+int zllm_kv_mla_layer_write(const zllm_mla_layer_record* r, uint8_t* out, uint64_t capacity, uint64_t* written)
+{
+    const uint64_t need = zllm_kv_mla_layer_wire_bytes(r);
+    if (need == 0 || out == nullptr) {
+        return fail(-1, "MLA layer write: record lengths do not match its shape");
+    }
+    if (capacity < need) {
+        return fail(-1, "MLA layer write: %llu bytes needed, %llu given", (unsigned long long)need, (unsigned long long)capacity);
+    }
+    uint8_t* at = put_u64(out, r->rows);
+    *at++ = (uint8_t)r->ownership;
+    at = put_u64(at, r->latent_cols);
+    at = put_u64(at, r->rope_cols);
+    at = put_u64(at, r->latent_group_size);
+    at = put_blob(at, r->latent, r->latent_bytes);
+    if (r->latent_scales != nullptr) {
+        *at++ = 1;
+        at = put_blob(at, r->latent_scales, r->latent_scales_bytes);
+    } else {
+        *at++ = 0;
+    }
+    at = put_blob(at, r->rope, r->rope_bytes);
+    if (written != nullptr) {
+        *written = (uint64_t)(at - out);
+    }
+    return 0;
+}
+
+namespace {
+struct WireReader {
+    const uint8_t* at;
+    uint64_t remaining;
+    bool ok = true;
+    uint64_t u64()
+    {
+        if (remaining < 8) {
+            ok = false;
+            return 0;
+        }
+        uint64_t value = 0;
+        for (int i = 0; i < 8; ++i) {
+            value |= (uint64_t)at[i] << (8 * i);
+        }
+        at += 8;
+        remaining -= 8;
+        return value;
+    }
+    uint8_t byte()
+    {
+        if (remaining < 1) {
+            ok = false;
+            return 0;
+        }
+        --remaining;
+        return *at++;
+    }
+    const uint8_t* blob(uint64_t* len)
+    {
+        *len = u64();
+        if (!ok || *len > remaining) { // "blob longer than what is left" (rocm_swap.rs:1195-1203)
+            ok = false;
+            return nullptr;
+        }
+        const uint8_t* start = at;
+        at += *len;
+        remaining -= *len;
+        return start;
+    }
+};
+} // namespace
+
+int zllm_kv_mla_layer_read(const uint8_t* in, uint64_t len, zllm_mla_layer_record* r, uint64_t* consumed)
+{
+    if (in == nullptr || r == nullptr) {
+        return fail(-1, "MLA layer read: null pointer");
+    }
+    WireReader reader{in, len};
+    memset(r, 0, sizeof(*r));
+    r->rows = reader.u64();
+    r->ownership = reader.byte();
+    r->latent_cols = reader.u64();
+    r->rope_cols = reader.u64();
+    r->latent_group_size = reader.u64();
+    r->latent = reader.blob(&r->latent_bytes);
+    const uint8_t flag = reader.byte();
+    if (reader.ok && flag > 1) {
+        return fail(-1, "MLA layer read: flag byte %u", flag);
+    }
+    if (flag == 1) {
+        r->latent_scales = reader.blob(&r->latent_scales_bytes);
+    }
+    r->rope = reader.blob(&r->rope_bytes);
+    if (!reader.ok) {
+        return fail(-1, "MLA layer read: record truncated (%llu bytes given)", (unsigned long long)len);
+    }
+    if (r->ownership > ZLLM_KV_OWNERSHIP_INTERLEAVED) {
+        return fail(-1, "MLA layer read: ownership byte %u", r->ownership);
+    }
+    if (consumed != nullptr) {
+        *consumed = len - reader.remaining;
+    }
+    if (!mla_record_shape_ok(r)) {
+        return fail(-2, "MLA layer read: blob lengths do not match rows=%llu latent=%llu rope=%llu group=%llu", (unsigned long long)r->rows,
+                    (unsigned long long)r->latent_cols, (unsigned long long)r->rope_cols, (unsigned long long)r->latent_group_size);
+    }
+    return 0;
+}
+
 /* ---- GQA decode ------------------------------------------------------------------------- */
 
 uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* a)

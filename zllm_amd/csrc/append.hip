@@ -256,6 +256,40 @@ template <typename T> __global__ __launch_bounds__(256) void gather_rows_kernel(
     ((T*)p.out)[index] = ((const T*)p.plane)[physical * units_per_row + unit];
 }
 
+template <typename T> __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterParams p, unsigned int units_per_row)
+{
+    const unsigned long long index = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned long long total = (unsigned long long)p.count * units_per_row;
+    if (index >= total) {
+        return;
+    }
+    const unsigned int row = (unsigned int)(index / units_per_row);
+    const unsigned int unit = (unsigned int)(index - (unsigned long long)row * units_per_row);
+    const unsigned long long physical = paged_row(p.table, p.first + row, p.block_tokens, p.ring_capacity);
+    ((T*)p.plane)[physical * units_per_row + unit] = ((const T*)p.in)[index];
+}
+
+hipError_t launch_scatter_rows(const ScatterParams& p, hipStream_t stream)
+{
+    if (p.count == 0 || p.row_bytes == 0) {
+        return hipSuccess;
+    }
+    const bool aligned16 = p.row_bytes % 16 == 0 && ((uintptr_t)p.plane % 16 == 0) && ((uintptr_t)p.in % 16 == 0);
+    const bool aligned4 = p.row_bytes % 4 == 0 && ((uintptr_t)p.plane % 4 == 0) && ((uintptr_t)p.in % 4 == 0);
+    const unsigned int unit = aligned16 ? 16 : (aligned4 ? 4 : 1);
+    const unsigned int units_per_row = p.row_bytes / unit;
+    const unsigned long long total = (unsigned long long)p.count * units_per_row;
+    const dim3 grid((unsigned int)((total + 255) / 256));
+    if (unit == 16) {
+        scatter_rows_kernel<uint4><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    } else if (unit == 4) {
+        scatter_rows_kernel<unsigned int><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    } else {
+        scatter_rows_kernel<unsigned char><<<grid, dim3(256), 0, stream>>>(p, units_per_row);
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream)
 {
     const unsigned long long groups = (unsigned long long)p.rows * (p.cols / 64u);

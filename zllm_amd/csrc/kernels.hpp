@@ -64,6 +64,13 @@ struct GatherParams {
     unsigned int first, count, row_bytes, block_tokens, ring_capacity;
 };
 
+struct ScatterParams {
+    void* plane;
+    const void* in;
+    const unsigned int* table;
+    unsigned int first, count, row_bytes, block_tokens, ring_capacity;
+};
+
 // Split-KV geometry shared by the partial and merge kernels.
 struct SplitPlan {
     unsigned int chunk_tokens; // tokens per split (multiple of 32)
@@ -137,6 +144,7 @@ struct MlaDecodeParams {
 unsigned int gqa_decode_max_waves(unsigned int head_dim);
 
 hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream);
+hipError_t launch_scatter_rows(const ScatterParams& p, hipStream_t stream);
 hipError_t launch_gqa_prologue(const GqaPrologueParams& p, hipStream_t stream);
 hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream);
 hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream);

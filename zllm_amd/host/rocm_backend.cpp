@@ -237,6 +237,100 @@ Result<RocmKvCache> RocmKvCache::new_mla(size_t layers, size_t latent_dim, size_
     return cache;
 }
 
+Result<Unit> RocmKvCache::truncate_rows(size_t rows)
+{
+    if (rows > max_tokens_) {
+        return compute_error("ROCm KV truncate rows=" + std::to_string(rows) + " exceeds the logical limit " + std::to_string(max_tokens_));
+    }
+    for (size_t layer = 0; layer < lens_.size(); ++layer) {
+        if (rows > lens_[layer]) {
+            return compute_error("L" + std::to_string(layer) + " ROCm KV truncate rows=" + std::to_string(rows) + " exceeds the current length " +
+                                 std::to_string(lens_[layer]));
+        }
+    }
+    for (size_t& len : lens_) {
+        len = rows;
+    }
+    return Unit{};
+}
+
+Result<Unit> RocmKvCache::truncate_layer_rows(size_t layer, size_t rows)
+{
+    if (rows > max_tokens_) {
+        return compute_error("L" + std::to_string(layer) + " ROCm KV truncate rows=" + std::to_string(rows) + " exceeds the logical limit " +
+                             std::to_string(max_tokens_));
+    }
+    if (layer >= lens_.size()) {
+        return BackendError{BackendError::Kind::UnsupportedLayer, layer, ""};
+    }
+    if (rows > lens_[layer]) {
+        return compute_error("L" + std::to_string(layer) + " ROCm KV truncate rows=" + std::to_string(rows) + " exceeds the current length " +
+                             std::to_string(lens_[layer]));
+    }
+    lens_[layer] = rows;
+    return Unit{};
+}
+
+// ---------------------------------------------------------------------------------------------- snapshot wire format
+Result<Unit> write_mla_layer(std::vector<uint8_t>& out, const MlaLayerSerde& layer)
+{
+    zllm_mla_layer_record rec;
+    memset(&rec, 0, sizeof(rec));
+    rec.rows = layer.rows;
+    rec.ownership = (uint32_t)layer.ownership;
+    rec.latent_cols = layer.latent_cols;
+    rec.rope_cols = layer.rope_cols;
+    rec.latent_group_size = layer.latent_group_size;
+    static const uint8_t empty = 0;
+    rec.latent = layer.latent.empty() ? &empty : layer.latent.data();
+    rec.latent_bytes = layer.latent.size();
+    if (layer.latent_scales.has_value()) {
+        rec.latent_scales = layer.latent_scales->empty() ? &empty : layer.latent_scales->data();
+        rec.latent_scales_bytes = layer.latent_scales->size();
+    }
+    rec.rope = layer.rope.empty() ? &empty : layer.rope.data();
+    rec.rope_bytes = layer.rope.size();
+    const uint64_t need = zllm_kv_mla_layer_wire_bytes(&rec);
+    if (need == 0) {
+        return compute_error("GLM cache MLA layer: blob lengths do not match the shape");
+    }
+    const size_t at = out.size();
+    out.resize(at + need);
+    uint64_t written = 0;
+    const int code = zllm_kv_mla_layer_write(&rec, out.data() + at, need, &written);
+    if (code != 0) {
+        out.resize(at);
+        return abi_error("zllm_kv_mla_layer_write", code);
+    }
+    return Unit{};
+}
+
+Result<MlaLayerSerde> read_mla_layer(const std::vector<uint8_t>& in, size_t& offset)
+{
+    if (offset > in.size()) {
+        return compute_error("GLM cache MLA layer: offset past the end");
+    }
+    zllm_mla_layer_record rec;
+    uint64_t used = 0;
+    const int code = zllm_kv_mla_layer_read(in.data() + offset, in.size() - offset, &rec, &used);
+    if (code != 0) {
+        return abi_error("zllm_kv_mla_layer_read", code);
+    }
+    MlaLayerSerde layer;
+    layer.rows = rec.rows;
+    layer.ownership = (RocmKvOwnership)rec.ownership;
+    layer.latent_cols = rec.latent_cols;
+    layer.rope_cols = rec.rope_cols;
+    layer.latent_group_size = rec.latent_group_size;
+    layer.latent.assign(rec.latent, rec.latent + rec.latent_bytes);
+    if (rec.latent_scales != nullptr) {
+        layer.latent_scales = std::vector<uint8_t>(rec.latent_scales, rec.latent_scales + rec.latent_scales_bytes);
+    }
+    layer.rope.assign(rec.rope, rec.rope + rec.rope_bytes);
+    offset += used;
+    return layer;
+}
+
 // ---------------------------------------------------------------------------------------------- context
 Result<RocmContext> RocmContext::create(int device_id)
 {
@@ -651,6 +745,111 @@ Result<RocmTensor> RocmContext::mla_decode_attention(const RocmTensor& query, co
     out.cols = out_cols;
     out.dtype = DType::F32;
     return out;
+}
+
+Result<std::vector<std::optional<MlaLayerSerde>>> RocmContext::download_layers(const RocmKvCache& cache) const
+{
+    if (!cache.mla_) {
+        return compute_error("ROCm KV snapshot: not an MLA cache");
+    }
+    std::vector<std::optional<MlaLayerSerde>> out;
+    for (size_t l = 0; l < cache.layers_.size(); ++l) {
+        const RocmKvCache::Layer& planes = cache.layers_[l];
+        MlaLayerSerde record;
+        record.rows = cache.lens_[l];
+        record.latent_cols = cache.cols_;
+        record.rope_cols = cache.rope_cols_;
+        record.latent_group_size = 64;
+        const size_t row_bytes[3] = {cache.cols_, cache.cols_ / 64 * 2, cache.rope_cols_ * 2};
+        const void* sources[3] = {planes.a_codes.data(), planes.a_scales.data(), planes.b_codes.data()};
+        std::vector<uint8_t> host[3];
+        for (int i = 0; i < 3; ++i) {
+            host[i].resize(record.rows * row_bytes[i]);
+            if (record.rows == 0) {
+                continue;
+            }
+            auto dense = DeviceBuffer::allocate(host[i].size());
+            if (dense.is_err()) {
+                return dense.unwrap_err();
+            }
+            zllm_gather_args g;
+            memset(&g, 0, sizeof(g));
+            g.plane = sources[i];
+            g.out = dense.unwrap().data();
+            g.table = (const uint32_t*)cache.table_.data();
+            g.first = 0;
+            g.count = (uint32_t)record.rows;
+            g.row_bytes = (uint32_t)row_bytes[i];
+            g.block_tokens = (uint32_t)cache.block_tokens_;
+            const int code = zllm_attn_gather_rows(&g, stream_);
+            if (code != 0) {
+                return abi_error("zllm_attn_gather_rows", code);
+            }
+            hipError_t err = hipMemcpyAsync(host[i].data(), dense.unwrap().data(), host[i].size(), hipMemcpyDeviceToHost, stream_);
+            if (err == hipSuccess) {
+                err = hipStreamSynchronize(stream_);
+            }
+            if (err != hipSuccess) {
+                return hip_error("KV snapshot download", err);
+            }
+        }
+        record.latent = std::move(host[0]);
+        record.latent_scales = std::move(host[1]);
+        record.rope = std::move(host[2]);
+        out.push_back(std::move(record));
+    }
+    return out;
+}
+
+Result<Unit> RocmContext::upload_layers(RocmKvCache& cache, const std::vector<std::optional<MlaLayerSerde>>& layers) const
+{
+    if (!cache.mla_ || layers.size() != cache.layers_.size()) {
+        return compute_error("ROCm KV snapshot: layer count " + std::to_string(layers.size()) + " does not match the cache");
+    }
+    for (size_t l = 0; l < layers.size(); ++l) {
+        if (!layers[l].has_value()) {
+            continue;
+        }
+        const MlaLayerSerde& record = *layers[l];
+        if (record.latent_cols != cache.cols_ || record.rope_cols != cache.rope_cols_ || record.latent_group_size != 64 ||
+            !record.latent_scales.has_value() || record.rows > cache.max_tokens_ || record.latent.size() != record.rows * cache.cols_ ||
+            record.latent_scales->size() != record.rows * (cache.cols_ / 64) * 2 || record.rope.size() != record.rows * cache.rope_cols_ * 2) {
+            return compute_error("L" + std::to_string(l) + " ROCm KV snapshot: record shape does not match the cache");
+        }
+        RocmKvCache::Layer& planes = cache.layers_[l];
+        const size_t row_bytes[3] = {cache.cols_, cache.cols_ / 64 * 2, cache.rope_cols_ * 2};
+        void* targets[3] = {planes.a_codes.data(), planes.a_scales.data(), planes.b_codes.data()};
+        const std::vector<uint8_t>* host[3] = {&record.latent, &*record.latent_scales, &record.rope};
+        for (int i = 0; i < 3 && record.rows != 0; ++i) {
+            auto dense = DeviceBuffer::allocate(host[i]->size());
+            if (dense.is_err()) {
+                return dense.unwrap_err();
+            }
+            hipError_t err = hipMemcpyAsync(dense.unwrap().data(), host[i]->data(), host[i]->size(), hipMemcpyHostToDevice, stream_);
+            if (err != hipSuccess) {
+                return hip_error("KV snapshot upload", err);
+            }
+            zllm_scatter_args sc;
+            memset(&sc, 0, sizeof(sc));
+            sc.plane = targets[i];
+            sc.in = dense.unwrap().data();
+            sc.table = (const uint32_t*)cache.table_.data();
+            sc.first = 0;
+            sc.count = (uint32_t)record.rows;
+            sc.row_bytes = (uint32_t)row_bytes[i];
+            sc.block_tokens = (uint32_t)cache.block_tokens_;
+            const int code = zllm_attn_scatter_rows(&sc, stream_);
+            if (code != 0) {
+                return abi_error("zllm_attn_scatter_rows", code);
+            }
+            err = hipStreamSynchronize(stream_);
+            if (err != hipSuccess) {
+                return hip_error("KV snapshot upload", err);
+            }
+        }
+        cache.lens_[l] = record.rows;
+    }
+    return Unit{};
 }
 
 } // namespace zllm_amd

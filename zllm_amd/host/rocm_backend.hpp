@@ -113,6 +113,24 @@ struct RocmWeight {
 
 enum class KvCacheFormat { F16, Q8g64 };
 
+enum class RocmKvOwnership { Full = 0, BlockParity0 = 1, BlockParity1 = 2, InterleavedPair = 3 };
+
+// Host form of one MLA layer for session snapshots (the reference's MlaLayerSerde, src/backend/rocm/kv_cache.rs:2067-2083):
+// plain bytes + shape, no device handles.
+struct MlaLayerSerde {
+    size_t rows = 0;
+    RocmKvOwnership ownership = RocmKvOwnership::Full;
+    size_t latent_cols = 0, rope_cols = 0;
+    size_t latent_group_size = 0;                     // 0 = bf16 latent without scales, else the Q8 group size
+    std::vector<uint8_t> latent;                      // Q8: rows x latent_cols
+    std::optional<std::vector<uint8_t>> latent_scales; // Q8: rows x (latent_cols / group) x 2
+    std::vector<uint8_t> rope;                        // rows x rope_cols x 2 (bf16)
+};
+// write_mla_layer / read_mla_layer (src/runtime/glm52/rocm_swap.rs:1090-1138): `write` appends to `out`; `read` parses one
+// record at `offset` and advances it.
+Result<Unit> write_mla_layer(std::vector<uint8_t>& out, const MlaLayerSerde& layer);
+Result<MlaLayerSerde> read_mla_layer(const std::vector<uint8_t>& in, size_t& offset);
+
 // Paged KV cache of one sequence: planar code / scale planes per layer plus one block table.
 class RocmKvCache {
   public:
@@ -121,6 +139,10 @@ class RocmKvCache {
     // MLA cache: Q8g64 latent (bf16 scales) + bf16 rope per layer
     static Result<RocmKvCache> new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens);
     size_t len(size_t layer) const { return layer < lens_.size() ? lens_[layer] : 0; }
+    // Rollback: only the logical length moves, pages and the kept prefix stay where they are and the next append
+    // overwrites the tail (truncate_rows / truncate_layer_rows, src/backend/rocm/kv_cache.rs:509-586).
+    Result<Unit> truncate_rows(size_t rows);
+    Result<Unit> truncate_layer_rows(size_t layer, size_t rows);
     size_t layers() const { return lens_.size(); }
     size_t block_tokens() const { return block_tokens_; }
     size_t max_tokens() const { return max_tokens_; }
@@ -161,6 +183,10 @@ class RocmContext {
     Result<Unit> append_mla(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope) const;
     Result<Unit> append_mla_rope(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
                                  RotaryLayout layout, size_t position, const std::vector<float>& cos, const std::vector<float>& sin) const;
+    // Session snapshot of an MLA cache (download_layers, src/backend/rocm/kv_cache.rs:3344-3388): every layer's rows
+    // [0, len) gathered through the block table into host bytes; and its inverse, into whatever pages `cache` owns.
+    Result<std::vector<std::optional<MlaLayerSerde>>> download_layers(const RocmKvCache& cache) const;
+    Result<Unit> upload_layers(RocmKvCache& cache, const std::vector<std::optional<MlaLayerSerde>>& layers) const;
     // query [1, heads * q_head_dim]; returns f32 [1, heads * value_dim]
     Result<RocmTensor> mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
                                             size_t position, const MlaSpec& spec) const;

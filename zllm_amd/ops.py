@@ -90,6 +90,12 @@ def gather_rows(plane, table, first, count, row_bytes, block_tokens, ring_capaci
     return out
 
 
+def scatter_rows(plane, rows, table, first, block_tokens, ring_capacity=0):
+    """plane[paged_row(first + r)] = rows[r] (zllm_attn_scatter_rows); `rows` is a dense [count, row_bytes] uint8 tensor."""
+    args = capi.ScatterArgs(_ptr(plane), _ptr(rows), _ptr(table), first, rows.shape[0], rows.shape[1], block_tokens, ring_capacity)
+    capi.check(capi.load().zllm_attn_scatter_rows(C.byref(args), _stream()))
+
+
 def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, num_heads, num_kv_heads, head_dim,
                     block_tokens, score_scale, max_kv_len, first_visible=None, softcap=0.0, ring_capacity=0,
                     kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None, total_kv_tokens=0, gate=None):
