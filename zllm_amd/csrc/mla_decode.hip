@@ -145,9 +145,6 @@ __device__ __forceinline__ void lds_barrier()
 }
 
 constexpr int kItemsMax = 4;
-constexpr int kRawCodes = kStepTokens * kLatent;        // 16 KiB  [token][512] int8
-constexpr int kRawRope = kStepTokens * kRope * 2;       //  4 KiB  [token][64] bf16
-constexpr int kRawScales = kStepTokens * (kLatent / 64) * 2; // 512 B [token][8] bf16
 
 // Block-table entries of a thread's staging items: fetched one step before the loads that use them, so
 // nothing waits on a table -> data chain.  Slot ITEMS belongs to the rope role (threads 0..255) or the
@@ -193,7 +190,6 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     constexpr int ITEMS = 3;
     __shared__ __align__(16) unsigned char lds[kWsTiles * kTileBytes];
     __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
-    __shared__ __align__(16) unsigned char lds_raw[kRawCodes + kRawRope + kRawScales];
     __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
     __shared__ float lds_top[kWsTiles];                  // [buffer]: largest group scale of the tile
@@ -231,20 +227,15 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
     // ---- staging (same scheme as mla_partial): loads of the next tile's raw bytes, converted by their owner
-    const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const unsigned int cc = tid & 31u;
     const unsigned int t_lo = (tid & 255u) >> 5;
     const int n_items = value_role ? 1 : 3;
     const unsigned int row_first = value_role ? 24u + t_lo : t_lo;      // row of item 0; item i is 8 i further on
-    const unsigned int wave_rows = (value_role ? 24u : 0u) + 2u * (wave & 3u); // first row of the wave's item 0
     const unsigned int rope_t = (tid >> 3) & 31u;
     const unsigned int rope_c = tid & 7u;
     const bool has_rope = tid < 256u;
     const bool has_scales = tid >= 256u && tid < 256u + kStepTokens;
     const unsigned int extra_t = has_rope ? rope_t : (tid - 256u) & 31u;
-    unsigned char* const raw_codes = lds_raw;
-    unsigned char* const raw_rope = lds_raw + kRawCodes;
-    unsigned char* const raw_scales = lds_raw + kRawCodes + kRawRope;
     // selected-token mode: positions of the thread's items for the step that starts at slot t0
     auto fetch_tokens = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
 #pragma unroll
@@ -287,77 +278,73 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
         }
         return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
     };
-    auto issue_step = [&](const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
+    // The raw bytes of a step travel through registers: a thread loads its items (16 codes each), its rope piece or its
+    // token's scales with plain 16-byte loads and converts them itself one iteration later, so nothing is waited for
+    // (a load has a whole iteration to land) and the conversion makes no LDS round trip before its writes.
+    struct StageRegs {
+        u32x4 codes[ITEMS];
+        u32x4 extra; // rope piece (threads 0..255) or the token's eight scales (threads 256..287)
+    };
+    auto load_step = [&](StageRegs& regs, const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
         if constexpr (ALIGNED) {
             const unsigned int entry = __builtin_amdgcn_readfirstlane(rows.entry[0]);
             const unsigned long long row0 = pow2 ? ((unsigned long long)entry << p.block_shift) + (t0 & (p.block_tokens - 1u))
                                                  : (unsigned long long)entry * p.block_tokens + t0 % p.block_tokens;
-            const unsigned int first = __builtin_amdgcn_readfirstlane(wave_rows);
-            const unsigned char* codes = (const unsigned char*)p.latent_codes + (row0 + first) * kLatent;
+            const unsigned char* codes = (const unsigned char*)p.latent_codes + row0 * kLatent;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 if (i < n_items) {
-                    __builtin_amdgcn_global_load_lds((global_ptr_t)(codes + 8 * i * kLatent + lane * 16u),
-                                                     (lds_ptr_t)(raw_codes + (first + 8 * i) * kLatent), 16, 0, 0);
+                    regs.codes[i] = *(const u32x4*)(codes + (row_first + 8u * i) * kLatent + cc * 16u);
                 }
             }
             if (has_rope) {
-                const unsigned char* rope = (const unsigned char*)p.rope_cache + row0 * (kRope * 2) + wave_u * 1024u;
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(rope + lane * 16u), (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+                regs.extra = *(const u32x4*)((const unsigned char*)p.rope_cache + row0 * (kRope * 2) + tid * 16u);
             }
             if (has_scales) {
-                const unsigned char* scales = (const unsigned char*)p.latent_scales + row0 * (kLatent / 64 * 2);
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(scales + lane * 16u), (lds_ptr_t)(raw_scales), 16, 0, 0);
+                regs.extra = *(const u32x4*)((const unsigned char*)p.latent_scales + (row0 + (tid - 256u)) * (kLatent / 64 * 2));
             }
         } else {
-            const unsigned int first = __builtin_amdgcn_readfirstlane(wave_rows);
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 if (i < n_items) {
-                    __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u),
-                                                     (lds_ptr_t)(raw_codes + (first + 8 * i) * kLatent), 16, 0, 0);
+                    regs.codes[i] = *(const u32x4*)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u);
                 }
             }
             if (has_rope) {
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u),
-                                                 (lds_ptr_t)(raw_rope + wave_u * 1024u), 16, 0, 0);
+                regs.extra = *(const u32x4*)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u);
             }
             if (has_scales) {
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64)),
-                                                 (lds_ptr_t)(raw_scales), 16, 0, 0);
+                regs.extra = *(const u32x4*)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64));
             }
         }
     };
-    auto convert_step = [&](unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top, unsigned int t0) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    auto convert_step = [&](const StageRegs& regs, unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top, unsigned int t0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
             if (i >= n_items) {
                 break;
             }
-            // the thread converts codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row: 32 consecutive lanes then
-            // write 512 contiguous bytes per instruction (chunks cc and cc + 32), which the LDS takes without conflicts
+            // sixteen codes -> chunks 2 cc and 2 cc + 1 of the row: 32 consecutive lanes write every other 16-byte chunk of
+            // a 1 KiB row per instruction, eight lanes per cycle on distinct banks
             const unsigned int row = row_first + 8u * i;
-            const u32x2 half[2] = {*(const u32x2*)(raw_codes + row * kLatent + cc * 8u),
-                                   *(const u32x2*)(raw_codes + row * kLatent + 256u + cc * 8u)};
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 u32x4 out;
 #pragma unroll
                 for (int w = 0; w < 2; ++w) {
                     unsigned int pair_lo, pair_hi;
-                    codes4_to_f16(half[h][w], pair_lo, pair_hi);
+                    codes4_to_f16(regs.codes[i][h * 2 + w], pair_lo, pair_hi);
                     out[w * 2] = pair_lo;
                     out[w * 2 + 1] = pair_hi;
                 }
-                *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
+                *(u32x4*)(tile + tile_offset(row, 2u * cc + h)) = out;
             }
         }
         if (has_rope) {
-            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = *(const u32x4*)(raw_rope + tid * 16u);
+            *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = regs.extra;
         }
         if (has_scales) {
-            const u32x4 sc8 = *(const u32x4*)(raw_scales + (tid - 256u) * 16u);
+            const u32x4 sc8 = regs.extra;
             float top = 0.0f;
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
@@ -381,7 +368,6 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 *step_top = both;
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
 
     // LDS byte offsets of this lane's fragments (lane part; the rest is compile-time)
@@ -398,11 +384,12 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
         fetch_tokens(rows, c_start);
     }
     lookup_step(rows, c_start);
-    issue_step(rows, c_start);
+    StageRegs staged;
+    load_step(staged, rows, c_start);
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    convert_step(lds, lds_scale[0], &lds_top[0], c_start);
+    convert_step(staged, lds, lds_scale[0], &lds_top[0], c_start);
     lds_barrier();
 
     // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile
@@ -425,7 +412,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                                       "+v"(rows.next_token[0]), "+v"(rows.next_token[1]), "+v"(rows.next_token[2]), "+v"(rows.next_token[3]));
                 }
             }
-            issue_step(rows, c_start + n * kStepTokens);
+            load_step(staged, rows, c_start + n * kStepTokens);
             if (n + 1 < steps) {
                 lookup_step(rows, c_start + (n + 1u) * kStepTokens);
             }
@@ -434,7 +421,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     auto convert_to = [&](unsigned int n) __attribute__((always_inline)) { // raw bytes of step n -> tile buffer n % 3
         if (n < steps) {
             const unsigned int nb = n % kWsTiles;
-            convert_step(lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + n * kStepTokens);
+            convert_step(staged, lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + n * kStepTokens);
         }
     };
 
@@ -480,8 +467,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
         float run_max = kNegInf, run_sum = 0.0f;
         const float scale_log2 = p.score_scale * kLog2e;
         const float latent_log2 = scale_log2 * head_pow2;
+        stage_step(1u);
         for (unsigned int i = 0; i <= steps; ++i) {
-            stage_step(i + 1u);
             if (i < steps) {
                 const unsigned int tb = i % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes;
@@ -597,6 +584,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 lds_alpha[i & 1u][hw][lane] = alpha;
             }
             convert_to(i + 1u);
+            stage_step(i + 2u);
             lds_barrier();
         }
         const float total = wave_sum_16x4(run_sum);
@@ -750,7 +738,6 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             }
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no load may still target this workgroup's LDS at exit
 }
 
 // ---------------------------------------------------------------------------------------------
