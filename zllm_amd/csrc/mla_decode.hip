@@ -192,7 +192,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
     __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
-    __shared__ float lds_top[kWsTiles];                  // [buffer]: largest group scale of the tile
+    __shared__ __align__(16) float lds_top[kWsTiles][4]; // [buffer][value wave]: largest group scale the wave converted
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
@@ -234,8 +234,10 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int rope_t = (tid >> 3) & 31u;
     const unsigned int rope_c = tid & 7u;
     const bool has_rope = tid < 256u;
-    const bool has_scales = tid >= 256u && tid < 256u + kStepTokens;
-    const unsigned int extra_t = has_rope ? rope_t : (tid - 256u) & 31u;
+    const bool has_scales = tid >= 256u; // value-role threads: one (token, group) scale each
+    const unsigned int scale_t = (tid - 256u) >> 3;
+    const unsigned int scale_g = tid & 7u;
+    const unsigned int extra_t = has_rope ? rope_t : scale_t;
     // selected-token mode: positions of the thread's items for the step that starts at slot t0
     auto fetch_tokens = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
 #pragma unroll
@@ -283,7 +285,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     // (a load has a whole iteration to land) and the conversion makes no LDS round trip before its writes.
     struct StageRegs {
         u32x4 codes[ITEMS];
-        u32x4 extra; // rope piece (threads 0..255) or the token's eight scales (threads 256..287)
+        u32x4 extra; // rope piece (threads 0..255); threads 256..511 keep one scale (16 bits) in extra[0]
     };
     auto load_step = [&](StageRegs& regs, const StepRows& rows, unsigned int t0) __attribute__((always_inline)) {
         if constexpr (ALIGNED) {
@@ -301,7 +303,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 regs.extra = *(const u32x4*)((const unsigned char*)p.rope_cache + row0 * (kRope * 2) + tid * 16u);
             }
             if (has_scales) {
-                regs.extra = *(const u32x4*)((const unsigned char*)p.latent_scales + (row0 + (tid - 256u)) * (kLatent / 64 * 2));
+                regs.extra[0] = *(const unsigned short*)((const unsigned char*)p.latent_scales + (row0 + scale_t) * (kLatent / 64 * 2) + scale_g * 2u);
             }
         } else {
 #pragma unroll
@@ -314,7 +316,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 regs.extra = *(const u32x4*)(p.rope_cache + row_of(rows, ITEMS, t0) * kRope + rope_c * 8u);
             }
             if (has_scales) {
-                regs.extra = *(const u32x4*)(p.latent_scales + row_of(rows, ITEMS, t0) * (kLatent / 64));
+                regs.extra[0] = p.latent_scales[row_of(rows, ITEMS, t0) * (kLatent / 64) + scale_g];
             }
         }
     };
@@ -344,28 +346,24 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             *(u32x4*)(tile + tile_offset(rope_t, 64u + rope_c)) = regs.extra;
         }
         if (has_scales) {
-            const u32x4 sc8 = regs.extra;
-            float top = 0.0f;
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                const unsigned int word = sc8[g >> 1];
-                float sg = bf16_bits_to_f32((unsigned short)((g & 1) ? (word >> 16) : (word & 0xffffu)));
-                if (t0 + (tid - 256u) >= len) {
-                    sg = 0.0f; // a row past the end: its codes may be anything, its weight is an exact zero
-                }
-                scale_tile[g][tid - 256u] = sg;
-                top = fmaxf(top, sg);
+            float sg = bf16_bits_to_f32((unsigned short)regs.extra[0]);
+            if (t0 + scale_t >= len) {
+                sg = 0.0f; // a row past the end: its codes may be anything, its weight is an exact zero
             }
-            // largest scale of the step, for the value waves' exponent window: lanes 0..31 of wave 4 hold one token
-            // each; rotate-and-max inside the two 16-lane rows, then one lane of each row
+            scale_tile[scale_g][scale_t] = sg;
+            // largest scale the wave holds, for the value waves' exponent window: rotate-and-max inside the four
+            // 16-lane rows, then one lane of each row
+            float top = sg;
             top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x128, 0xf, 0xf, false))); // row_ror:8
             top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x124, 0xf, 0xf, false))); // row_ror:4
             top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x122, 0xf, 0xf, false))); // row_ror:2
             top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x121, 0xf, 0xf, false))); // row_ror:1
-            const float both = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
-                                     __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 16)));
-            if (tid == 256u) {
-                *step_top = both;
+            const float rows01 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
+                                       __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 16)));
+            const float rows23 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 32)),
+                                       __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 48)));
+            if (lane == 0u) {
+                step_top[hw] = fmaxf(rows01, rows23);
             }
         }
     };
@@ -389,7 +387,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    convert_step(staged, lds, lds_scale[0], &lds_top[0], c_start);
+    convert_step(staged, lds, lds_scale[0], lds_top[0], c_start);
     lds_barrier();
 
     // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile
@@ -421,7 +419,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     auto convert_to = [&](unsigned int n) __attribute__((always_inline)) { // raw bytes of step n -> tile buffer n % 3
         if (n < steps) {
             const unsigned int nb = n % kWsTiles;
-            convert_step(staged, lds + nb * kTileBytes, lds_scale[nb], &lds_top[nb], c_start + n * kStepTokens);
+            convert_step(staged, lds + nb * kTileBytes, lds_scale[nb], lds_top[nb], c_start + n * kStepTokens);
         }
     };
 
@@ -622,7 +620,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 p_hi[ht] = *(const f32x4*)(slot + 4);
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
-            const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(lds_top[value_tile])); // tile i - 1
+            const f32x4 tops = *(const f32x4*)lds_top[value_tile]; // tile i - 1
+            const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3]))));
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_setprio(3);
             convert_to(i + 1u);
