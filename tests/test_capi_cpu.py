@@ -101,6 +101,26 @@ def test_invalid_shapes_are_reported_without_a_gpu(lib):
     assert b"null pointer" in lib.zllm_attn_last_error()
     q8 = capi.Q8AppendArgs()
     assert lib.zllm_attn_q8g64_append(C.byref(q8), None) == -1
+    # MLA decode: shape, selection and alignment errors come back before anything touches a device
+    mla = capi.MlaDecodeArgs()
+    assert lib.zllm_attn_mla_decode(C.byref(mla), None) == -1
+    mla.batch, mla.heads, mla.q_head_dim, mla.kv_head_dim, mla.latent_dim, mla.rope_dim = 1, 16, 192, 256, 512, 64
+    mla.block_tokens, mla.max_ctx_len, mla.q_dtype, mla.out_dtype = 64, 4096, capi.DTYPE_BF16, capi.DTYPE_F32
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) > 0
+    mla.selection, mla.top_k = 0x1000, 0
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) == 0 and b"top_k" in lib.zllm_attn_last_error()
+    mla.top_k = 2048
+    dense = capi.MlaDecodeArgs.from_buffer_copy(mla)
+    dense.selection, dense.top_k = None, 0
+    # a selection bounds every sequence by top_k tokens: fewer splits, smaller workspace
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) < lib.zllm_attn_mla_decode_workspace_bytes(C.byref(dense))
+    for name in ("q", "kv_b", "latent_codes", "latent_scales", "rope_cache", "ctx_lens", "out", "workspace"):
+        setattr(mla, name, 0x10000)
+    mla.workspace_bytes = 1 << 30
+    mla.rope_cache = 0x10008
+    assert lib.zllm_attn_mla_decode(C.byref(mla), None) == -1 and b"aligned" in lib.zllm_attn_last_error()
+    prologue = capi.GqaPrologueArgs()
+    assert lib.zllm_attn_gqa_prologue(C.byref(prologue), None) == -1
 
 
 def test_cpp_host_layer_builds_and_exports_the_backend_methods():

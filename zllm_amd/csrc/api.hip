@@ -656,6 +656,11 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
         a->ctx_lens == nullptr || a->out == nullptr || a->workspace == nullptr) {
         return fail(-1, "MLA decode: null pointer");
     }
+    // the kernels read weights, codes, rope and the workspace as 16-byte vectors
+    if ((((uintptr_t)a->kv_b | (uintptr_t)a->latent_codes | (uintptr_t)a->rope_cache | (uintptr_t)a->workspace) & 15u) != 0 ||
+        (((uintptr_t)a->latent_scales) & 1u) != 0 || (((uintptr_t)a->out | (uintptr_t)a->q) & 3u) != 0) {
+        return fail(-1, "MLA decode: kv_b, latent codes, rope cache and workspace must be 16-byte aligned (q and out 4-byte, scales 2-byte)");
+    }
     zllm::MlaDecodeParams p;
     memset(&p, 0, sizeof(p));
     plan_mla_decode(a, &p.chunk_tokens, &p.max_chunks);
