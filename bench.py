@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "mla_decode_64k", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration"])
     ap.add_argument("--pool-gib", type=float, default=160.0, help="address span of the paged pool (all four planes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -57,6 +57,22 @@ def event_time_ms(fn, steps):
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
+
+
+def event_times_ms(fn, launches):
+    """Per-launch durations (one HIP event pair around each of `launches` back-to-back launches): median and minimum, the
+    reference's bench idiom (src/kernel/rocm/hip/attention/paged_mla.rs:6742-6759)."""
+    import torch
+
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    torch.cuda.synchronize()
+    for start, stop in pairs:
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    times = sorted(start.elapsed_time(stop) for start, stop in pairs)
+    return times[len(times) // 2], times[0]
 
 
 def wall_time_ms(fn, steps):
@@ -166,14 +182,14 @@ def gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, block_tokens, scal
                        f"per pass: dequantize {t_deq / n:.3f}s + f32 attention {t_att / n:.3f}s"), outs
 
 
-def run_gqa_decode(args, ragged):
+def run_gqa_decode(args, ragged, config1=False):
     import torch
 
     from zllm_amd import capi, ops
 
-    hq, hkv, d, bt, batch = 64, 8, 128, 16, 8
+    hq, hkv, d, bt, batch = (16, 4, 128, 16, 1) if config1 else (64, 8, 128, 16, 8)
     rng = np.random.default_rng(args.seed)
-    lens = [int(x) for x in rng.integers(1024, 32769, size=batch)] if ragged else [32768] * batch
+    lens = [int(x) for x in rng.integers(1024, 32769, size=batch)] if ragged else [4096 if config1 else 32768] * batch
     scale = 1.0 / float(np.sqrt(d))
     ops.init(0)
     planes, tables, tables_dev, q, pool = build_gqa_pool(args, lens, hq, hkv, d, bt)
@@ -216,6 +232,7 @@ def run_gqa_decode(args, ragged):
     ms_step = wall_time_ms(graph.replay, replays) / per_graph
     ms_events = event_time_ms(graph.replay, replays) / per_graph
     ms_partial = event_time_ms(partial_only, args.steps)
+    ms_partial_median, ms_partial_min = event_times_ms(partial_only, max(args.steps, 100))
     out.zero_()
     graph.replay()
     torch.cuda.synchronize()
@@ -228,7 +245,8 @@ def run_gqa_decode(args, ragged):
         "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": ("C2 Q8g64 GQA decode, B=8, 64q/8kv, d=128, " + ("ragged L~U[1024,32768]" if ragged else "all L=32768")
+        "config": {"workload": ("C1 Q8g64 GQA decode, B=1, 16q/4kv, d=128, L=4096, 16-token pages (the reference's CPU-runnable case: latency-bound on a GPU)"
+                                if config1 else "C2 Q8g64 GQA decode, B=8, 64q/8kv, d=128, " + ("ragged L~U[1024,32768]" if ragged else "all L=32768")
                                 + ", 16-token pages"),
                    "kv_lens": lens, "kv_bytes_per_call": kv_bytes, "bytes_per_token": bytes_per_token, "seed": args.seed,
                    "pool_bytes": pool["pool_bytes"], "pool_blocks": pool["pool_blocks"], "max_code_plane_offset": pool["max_code_offset"],
@@ -240,8 +258,9 @@ def run_gqa_decode(args, ragged):
         "launch": f"hipGraph replay, {per_graph} decode calls (partial + merge each) per graph",
         "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_dma128", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None if ragged or args.seed != 2 else GQA_32K_TRAFFIC_BYTES,
-                     "kernel_ms": round(ms_partial, 5)},
+                     "traffic": None if ragged or config1 or args.seed != 2 else GQA_32K_TRAFFIC_BYTES,
+                     "kernel_ms": round(ms_partial, 5), "kernel_ms_median": round(ms_partial_median, 5),
+                     "kernel_ms_min": round(ms_partial_min, 5)},
     }
     if not args.no_cpu_baseline:
         cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)
@@ -275,6 +294,8 @@ def main():
         run_gqa_decode(args, ragged=False)
     elif args.workload == "gqa_decode_ragged":
         run_gqa_decode(args, ragged=True)
+    elif args.workload == "gqa_decode_c1":
+        run_gqa_decode(args, ragged=False, config1=True)
     elif args.workload == "copy_calibration":
         run_copy_calibration(args)
     else:
