@@ -190,7 +190,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     constexpr int ITEMS = 3;
     __shared__ __align__(16) unsigned char lds[kWsTiles * kTileBytes];
     __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
-    __shared__ __align__(16) float lds_p[2][4][64][8];   // [parity][head tile][lane][token slot]
+    __shared__ __align__(16) float lds_p[2][4][2][64][4]; // [parity][head tile][token half][lane][4 tokens]: 16-byte slots
+                                                          // of consecutive lanes are contiguous (conflict-free 16-byte reads)
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
     __shared__ __align__(16) float lds_top[kWsTiles][4]; // [buffer][value wave]: largest group scale the wave converted
     const unsigned int tid = threadIdx.x;
@@ -235,8 +236,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int rope_c = tid & 7u;
     const bool has_rope = tid < 256u;
     const bool has_scales = tid >= 256u; // value-role threads: one (token, group) scale each
-    const unsigned int scale_t = (tid - 256u) >> 3;
-    const unsigned int scale_g = tid & 7u;
+    const unsigned int scale_t = (tid - 256u) & 31u; // consecutive lanes write consecutive floats of a group's row
+    const unsigned int scale_g = (tid - 256u) >> 5;
     const unsigned int extra_t = has_rope ? rope_t : scale_t;
     // selected-token mode: positions of the thread's items for the step that starts at slot t0
     auto fetch_tokens = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
@@ -280,8 +281,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
         }
         return (unsigned long long)r.entry[i] * p.block_tokens + token % p.block_tokens;
     };
-    // The raw bytes of a step travel through registers: a thread loads its items (16 codes each), its rope piece or its
-    // token's scales with plain 16-byte loads and converts them itself one iteration later, so nothing is waited for
+    // The raw bytes of a step travel through registers: a thread loads its items (two runs of eight codes each), its rope piece
+    // or one scale with plain loads and converts them itself one iteration later, so nothing is waited for
     // (a load has a whole iteration to land) and the conversion makes no LDS round trip before its writes.
     struct StageRegs {
         u32x4 codes[ITEMS];
@@ -295,8 +296,10 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             const unsigned char* codes = (const unsigned char*)p.latent_codes + row0 * kLatent;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                if (i < n_items) {
-                    regs.codes[i] = *(const u32x4*)(codes + (row_first + 8u * i) * kLatent + cc * 16u);
+                if (i < n_items) { // codes 8 cc .. + 8 and 256 + 8 cc .. + 8 of the row
+                    const unsigned char* at = codes + (row_first + 8u * i) * kLatent + cc * 8u;
+                    const u32x2 lo = *(const u32x2*)(at), hi = *(const u32x2*)(at + 256);
+                    regs.codes[i] = u32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
             }
             if (has_rope) {
@@ -309,7 +312,9 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 if (i < n_items) {
-                    regs.codes[i] = *(const u32x4*)(p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 16u);
+                    const signed char* at = p.latent_codes + row_of(rows, i, t0) * kLatent + cc * 8u;
+                    const u32x2 lo = *(const u32x2*)(at), hi = *(const u32x2*)(at + 256);
+                    regs.codes[i] = u32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
             }
             if (has_rope) {
@@ -326,8 +331,9 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             if (i >= n_items) {
                 break;
             }
-            // sixteen codes -> chunks 2 cc and 2 cc + 1 of the row: 32 consecutive lanes write every other 16-byte chunk of
-            // a 1 KiB row per instruction, eight lanes per cycle on distinct banks
+            // codes 8 cc .. + 8 and 256 + 8 cc .. + 8 -> chunks cc and cc + 32 of the row: 32 consecutive lanes write 512
+            // contiguous bytes per instruction, which the LDS takes without conflicts (chunks 2 cc and 2 cc + 1, the
+            // natural output of one 16-byte load, measured a two-way conflict on every write: sixteen lanes go per cycle)
             const unsigned int row = row_first + 8u * i;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -339,7 +345,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                     out[w * 2] = pair_lo;
                     out[w * 2 + 1] = pair_hi;
                 }
-                *(u32x4*)(tile + tile_offset(row, 2u * cc + h)) = out;
+                *(u32x4*)(tile + tile_offset(row, cc + 32u * h)) = out;
             }
         }
         if (has_rope) {
@@ -576,9 +582,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                 }
                 run_sum = run_sum * alpha + step_sum;
                 run_max = new_max;
-                float* slot = lds_p[i & 1u][hw][lane];
-                *(f32x4*)(slot) = p_lo;
-                *(f32x4*)(slot + 4) = p_hi;
+                *(f32x4*)lds_p[i & 1u][hw][0][lane] = p_lo;
+                *(f32x4*)lds_p[i & 1u][hw][1][lane] = p_hi;
                 lds_alpha[i & 1u][hw][lane] = alpha;
             }
             convert_to(i + 1u);
@@ -615,9 +620,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             float alpha[2];
 #pragma unroll
             for (int ht = 0; ht < 2; ++ht) {
-                const float* slot = lds_p[(i + 1u) & 1u][2u * hp + ht][lane];
-                p_lo[ht] = *(const f32x4*)(slot);
-                p_hi[ht] = *(const f32x4*)(slot + 4);
+                p_lo[ht] = *(const f32x4*)lds_p[(i + 1u) & 1u][2u * hp + ht][0][lane];
+                p_hi[ht] = *(const f32x4*)lds_p[(i + 1u) & 1u][2u * hp + ht][1][lane];
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
             const f32x4 tops = *(const f32x4*)lds_top[value_tile]; // tile i - 1
