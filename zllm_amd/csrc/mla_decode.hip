@@ -136,9 +136,9 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 // ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
-// Workgroup barrier for LDS traffic only.  __syncthreads() also fences the global -> LDS loads in flight
-// (s_waitcnt vmcnt(0)), which would drain the prefetch of the next step at every barrier; the data those
-// loads bring is consumed by the issuing thread alone, after its own explicit wait.
+// Workgroup barrier for LDS traffic only.  __syncthreads() also waits for the global loads in flight
+// (s_waitcnt vmcnt(0)), which would drain the prefetch of the next step at every barrier; what those loads
+// bring is consumed by the issuing thread alone, one iteration later.
 __device__ __forceinline__ void lds_barrier()
 {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -148,7 +148,7 @@ constexpr int kItemsMax = 4;
 
 // Block-table entries of a thread's staging items: fetched one step before the loads that use them, so
 // nothing waits on a table -> data chain.  Slot ITEMS belongs to the rope role (threads 0..255) or the
-// scale role (threads 256..287).
+// scale role (threads 256..511).
 struct StepRows {
     unsigned int entry[kItemsMax + 1];
     // selected-token mode only: the token positions behind `entry`, and those of the step after (fetched one
@@ -157,8 +157,6 @@ struct StepRows {
     unsigned int next_token[kItemsMax + 1];
 };
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
 // Workgroup = (split, block of 64 heads, sequence), eight waves in two roles that run one step apart:
 //   score waves (0..3, 16 heads each): S^T = K.Q^T for all 32 tokens of tile i, online softmax, and hand
@@ -169,12 +167,12 @@ typedef const __attribute__((address_space(1))) void* global_ptr_t;
 // The score work is LDS reads + vector ALU (exp, max), the value work LDS reads + MFMA; with one wave of each
 // role per SIMD the two overlap instead of every wave running the same phase at the same time, and the
 // score exchange between waves of a head tile (a second barrier per step) disappears.  Three tile buffers
-// rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the raw bytes that the
-// global -> LDS loads of the previous iteration brought in).  One LDS-only barrier per step.
+// rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the bytes the threads loaded
+// an iteration ago).  One LDS-only barrier per step.
 constexpr int kWsTiles = 3;
 
 // ALIGNED: pages hold a multiple of 32 tokens (splits always start at one), so the 32 rows of a step are
-// contiguous in one page: one block-table entry per step, and every global -> LDS load takes a scalar base
+// contiguous in one page: one block-table entry per step, and every staging load takes a scalar base
 // plus a constant per-lane offset -- no vector address arithmetic in the loop.  Rows past the end of the
 // sequence are then whatever the page holds; their scales are zeroed during conversion and their scores
 // masked, so they contribute exact zeros.
@@ -227,7 +225,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
-    // ---- staging (same scheme as mla_partial): loads of the next tile's raw bytes, converted by their owner
+    // ---- staging: loads of a later tile's bytes, converted by the thread that loaded them
     const unsigned int cc = tid & 31u;
     const unsigned int t_lo = (tid & 255u) >> 5;
     const int n_items = value_role ? 1 : 3;
@@ -672,10 +670,9 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                     s16x4 s[2];
                     f16x8 h;
                 };
-                // The transposed reads are written as inline assembly: through the builtin the compiler cannot tell
-                // that they never touch the raw area the global -> LDS loads fill, and it drains those loads
-                // (s_waitcnt vmcnt(0)) in front of the first read of every step.  The price is that their
-                // completion is waited for by hand (lgkmcnt, LDS operations complete in issue order).
+                // The transposed reads are written as inline assembly with immediate offsets: one address register per
+                // fragment row serves all four groups, and the waits are placed by hand (lgkmcnt, LDS operations
+                // complete in issue order) exactly one group behind the requests.
                 const unsigned int at[4] = {tile_lds + pv_base[0], tile_lds + pv_base[1], tile_lds + pv_base[2], tile_lds + pv_base[3]};
                 auto load_group = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
 #pragma unroll
