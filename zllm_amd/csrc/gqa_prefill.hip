@@ -324,26 +324,33 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                     }
                 }
             }
+            // all eight V^T fragment reads of the group are requested before the first MFMA, and the low-order pass is one
+            // branch around its own loop: with the reads and the branch inside the tile loop every tile paid an LDS round
+            // trip in front of its four MFMAs
+            union VFrag {
+                s16x4 s[2];
+                bf16x8 b;
+            };
+            VFrag vf[4];
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt) {
-                const int t = g * 4 + tt;
                 const unsigned char* at = vt + pv_base[tt] + pv_group[g];
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
-                union {
-                    s16x4 s[2];
-                    bf16x8 b;
-                } vf;
-                vf.s[0] = lo;
-                vf.s[1] = hi;
+                vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
-                    acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, phi[ct].b, acc[ct][t], 0, 0, 0);
+                    acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[tt].b, phi[ct].b, acc[ct][g * 4 + tt], 0, 0, 0);
                 }
-                if (lo_pass) {
+            }
+            if (lo_pass) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
                     for (int ct = 0; ct < kColTiles; ++ct) {
-                        acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.b, plo[ct].b, acc[ct][t], 0, 0, 0);
+                        acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[tt].b, plo[ct].b, acc[ct][g * 4 + tt], 0, 0, 0);
                     }
                 }
             }
