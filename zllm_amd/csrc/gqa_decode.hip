@@ -124,19 +124,25 @@ template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(
 // a dense numbering spreads the live workgroups of a ragged batch evenly (a [split][sequence] grid leaves
 // gaps where short sequences end, and one XCD can end up with more live workgroups than CUs).  Every wave
 // finds its item by a prefix sum over the sequences' split counts; ids past the last item exit.
+// `span_out` is the split length of the item's sequence: its visible range cut into equal 32-aligned parts (never
+// longer than the planned chunk_tokens), so that a ragged batch has no full-length splits next to short remainders --
+// the longest split sets the kernel's duration.
 __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned int item, unsigned int lane, unsigned int& b_out,
-                                             unsigned int& chunk_out, unsigned int& len_out, unsigned int& first_out)
+                                             unsigned int& chunk_out, unsigned int& len_out, unsigned int& first_out, unsigned int& span_out)
 {
     unsigned int base = 0;
     for (unsigned int b0 = 0; b0 < p.batch; b0 += 64u) {
         const unsigned int i = b0 + lane;
-        unsigned int n = 0, len = 0, first = 0;
+        unsigned int n = 0, len = 0, first = 0, span = p.chunk_tokens;
         if (i < p.batch) {
             len = p.kv_lens[i];
             first = p.first_visible != nullptr ? p.first_visible[i] : 0u;
             first = min(first, len);
             const unsigned int first_al = first & ~31u;
             n = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+            if (n > 0) {
+                span = min(p.chunk_tokens, (((len - first_al + n - 1u) / n) + 31u) & ~31u);
+            }
         }
         unsigned int incl = n; // inclusive prefix sum over the wave
 #pragma unroll
@@ -153,6 +159,7 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
             chunk_out = local - (__builtin_amdgcn_readlane(incl, src) - __builtin_amdgcn_readlane(n, src));
             len_out = __builtin_amdgcn_readlane(len, src); // already here: no second trip to memory for them
             first_out = __builtin_amdgcn_readlane(first, src);
+            span_out = __builtin_amdgcn_readlane(span, src);
             return true;
         }
         base += total;
@@ -381,12 +388,12 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk, len, first;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
+    unsigned int b, chunk, len, first, span;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
-    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * span;
     const unsigned int head_in_group = head_block * 16u + m;
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
@@ -400,7 +407,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         return;
     }
     const unsigned int c_start = (unsigned int)c_start64;
-    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
     i32x4 qhi[G], qlo[G];
@@ -644,12 +651,12 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk, len, first;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
+    unsigned int b, chunk, len, first, span;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
-    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * span;
     const unsigned int head_in_group = head_block * 16u + m;
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
@@ -662,7 +669,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         return;
     }
     const unsigned int c_start = (unsigned int)c_start64;
-    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
     const unsigned int* table = p.tables + (size_t)b * p.table_stride;
@@ -855,12 +862,12 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
     const unsigned int head_block = blockIdx.y / kvh_blocks;
-    unsigned int b, chunk, len, first;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first)) {
+    unsigned int b, chunk, len, first, span;
+    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
-    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * p.chunk_tokens;
+    const unsigned long long c_start64 = (unsigned long long)first_al + (unsigned long long)chunk * span;
     const unsigned int head_in_group = head_block * 16u + m;
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
@@ -873,7 +880,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
         return;
     }
     const unsigned int c_start = (unsigned int)c_start64;
-    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
     // Q: per-head power-of-two normalisation keeps q inside the f16 range; hi + lo split.  The lane's 8 KS elements
