@@ -210,7 +210,11 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             len = p.selection_counts != nullptr ? min(p.selection_counts[b], p.top_k) : p.top_k;
         }
     }
-    const unsigned long long c_start64 = (unsigned long long)chunk * p.chunk_tokens;
+    // the planned split size is an upper bound: the sequence cuts its keys into equal 32-aligned parts, so a ragged
+    // batch has no full-length splits next to short remainders
+    const unsigned int n_splits = min(p.max_chunks, (len + p.chunk_tokens - 1u) / p.chunk_tokens);
+    const unsigned int span = n_splits > 0u ? min(p.chunk_tokens, (((len + n_splits - 1u) / n_splits) + 31u) & ~31u) : p.chunk_tokens;
+    const unsigned long long c_start64 = (unsigned long long)chunk * span;
     const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
     if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
         if (head < p.heads && j == 0 && !value_role) {
@@ -220,7 +224,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
         return;
     }
     const unsigned int c_start = (unsigned int)c_start64;
-    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + p.chunk_tokens);
+    const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + kStepTokens - 1) / kStepTokens;
     const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
