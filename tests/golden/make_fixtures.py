@@ -6,7 +6,9 @@ reference's known-answer tests (tests/test_oracle_known_answers.py), so that a l
 kernel shows up as a difference against committed bytes:
   q8g64_quantizer.npz   128 rows x 256 columns in three magnitude regimes -> codes and scales of the three rules
   gqa_decode_small.npz  B=3 ragged, 8q/2kv, d=128, 16-token pages -> decode output
-  mla_decode_small.npz  B=2, 4 heads, latent 512 + rope 64 -> output before the final bf16 rounding
+  mla_decode_small.npz  B=2, 4 heads, latent 512 + rope 64 -> output before the final bf16 rounding, dense and with a
+                        32-entry token selection per sequence
+  gqa_prologue_small.npz 5 rows, 4q/2kv, d=128: per-head Gemma RMSNorm + split-half RoPE of Q and K, K/V quantized into pages
   gqa_prefill_small.npz prefix 200 + chunk 48, 8q/2kv, window 0 and 64 -> chunk outputs
 """
 import os
@@ -54,9 +56,39 @@ def mla_decode():
 
     case = make_mla_case(502, [150, 41], 4)
     want, want_bf16 = oracle_mla(case)
+    rng = np.random.default_rng(504)
+    selection = np.stack([rng.choice(int(l), size=32, replace=False) for l in case["lens"]]).astype(np.uint32)
+    selected, _ = oracle_mla(case, selection=selection)
     np.savez_compressed(os.path.join(HERE, "mla_decode_small.npz"), q_bits=case["q_bits"], kv_b_bits=case["kv_b_bits"], codes=case["codes"],
                         scales=case["scales"], rope=case["rope"], tables=case["tables"], lens=case["lens"], expected_f32=want,
-                        expected_bf16=want_bf16)
+                        expected_bf16=want_bf16, selection=selection, expected_selected_f32=selected)
+
+
+def gqa_prologue():
+    rng = np.random.default_rng(505)
+    rows, hq, hkv, d, bt, position, rotary, eps = 5, 4, 2, 128, 16, 11, 64, 1e-6
+    q = rng.standard_normal((rows, hq * d)).astype(np.float32) * 2
+    k = rng.standard_normal((rows, hkv * d)).astype(np.float32)
+    v = rng.standard_normal((rows, hkv * d)).astype(np.float32)
+    qw = (rng.standard_normal(d) * 0.2).astype(np.float32)
+    kw = (rng.standard_normal(d) * 0.2).astype(np.float32)
+    half = rotary // 2
+    angles = np.arange(position + rows, dtype=np.float64)[:, None] / 10000.0 ** (np.arange(half, dtype=np.float64)[None, :] / half)
+    cos, sin = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    table = rng.permutation(4)[:2].astype(np.uint32)
+    out = {}
+    for name, x, heads, w in (("q", q, hq, qw), ("k", k, hkv, kw)):
+        rc, normed = O.rmsnorm_heads(x, heads, d, w, eps, 1.0)
+        assert rc == 0
+        rc, rotated = O.rope_apply(normed, heads, rotary, position, cos, sin, layout=0, placement=0)
+        assert rc == 0
+        out[name] = rotated
+    planes = {n: np.zeros((4 * bt, hkv * d if "codes" in n else hkv * d // 64), dtype=np.int8 if "codes" in n else np.uint16)
+              for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    O.q8g64_append_paged(O.RULE_METAL_GQA, out["k"], planes["k_codes"], planes["k_scales"], table, position, bt)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, planes["v_codes"], planes["v_scales"], table, position, bt)
+    np.savez_compressed(os.path.join(HERE, "gqa_prologue_small.npz"), q=q, k=k, v=v, q_norm=qw, k_norm=kw, cos=cos, sin=sin, table=table,
+                        position=np.uint32(position), rotary=np.uint32(rotary), eps=np.float32(eps), expected_q=out["q"], **planes)
 
 
 def gqa_prefill():
@@ -90,6 +122,7 @@ if __name__ == "__main__":
     gqa_decode()
     mla_decode()
     gqa_prefill()
+    gqa_prologue()
     for name in sorted(os.listdir(HERE)):
         if name.endswith(".npz"):
             print(name, os.path.getsize(os.path.join(HERE, name)))

@@ -79,6 +79,44 @@ def test_mla_kernel_matches_the_mla_fixture():
 
 
 @pytest.mark.gpu
+def test_mla_kernel_matches_the_selected_token_fixture():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import ops
+
+    g = load("mla_decode_small.npz")
+    out = ops.mla_decode(to_torch_bf16(g["q_bits"], "cuda"), upload(g["kv_b_bits"]), upload(g["codes"]), upload(g["scales"]), upload(g["rope"]),
+                         upload(g["tables"]), upload(g["lens"]), 4, 192, 256, 512, 64, 16, int(g["lens"].max()), selection=upload(g["selection"]))
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g["expected_selected_f32"].reshape(out.shape), "MLA selected-token fixture")
+
+
+@pytest.mark.gpu
+def test_prologue_kernel_matches_the_prologue_fixture_bit_for_bit():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import ops
+
+    g = load("gqa_prologue_small.npz")
+    dev = {n: torch.zeros(g[n].shape, dtype=torch.int8 if "codes" in n else torch.int16, device="cuda")
+           for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    q_out = ops.gqa_prologue(upload(g["q"]), upload(g["k"]), upload(g["v"]), upload(g["q_norm"]), upload(g["k_norm"]), upload(g["cos"]),
+                             upload(g["sin"]), dev["k_codes"], dev["k_scales"], dev["v_codes"], dev["v_scales"], upload(g["table"]),
+                             int(g["position"]), 4, 2, 128, int(g["rotary"]), 16, eps=float(g["eps"]), weight_offset=1.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(q_out.cpu().numpy().view(np.uint32), g["expected_q"].view(np.uint32))
+    for n in dev:
+        assert np.array_equal(dev[n].cpu().numpy().view(g[n].dtype), g[n]), n
+
+
+def test_oracle_reproduces_the_prologue_fixture():
+    g = load("gqa_prologue_small.npz")
+    rc, normed = O.rmsnorm_heads(g["q"], 4, 128, g["q_norm"], float(g["eps"]), 1.0)
+    assert rc == 0
+    rc, rotated = O.rope_apply(normed, 4, int(g["rotary"]), int(g["position"]), g["cos"], g["sin"], layout=0, placement=0)
+    assert rc == 0
+    assert np.array_equal(rotated.view(np.uint32), g["expected_q"].view(np.uint32))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("window", [0, 64])
 def test_prefill_kernel_matches_the_prefill_fixture(window):
     torch = pytest.importorskip("torch")
