@@ -250,6 +250,30 @@ static void test_mla(const RocmContext& ctx)
     CHECK(rc == 0, "oracle rc %d", rc);
     compare(got.unwrap(), want, "mla_decode_attention after append_mla + append_mla_rope");
 
+    // selected-token decode (DecodeBackend::mla_decode_attention_selected): 64 listed positions out of the context
+    {
+        std::vector<uint32_t> selection;
+        for (uint32_t s = 0; s < 64; ++s) {
+            selection.push_back((uint32_t)((s * 37u + 5u) % ctx_len)); // 37 and ctx_len are coprime here: distinct positions
+        }
+        auto state = ctx.dsa_state_from_selection(selection);
+        CHECK(state.is_ok(), "dsa_state_from_selection");
+        DsaSpec dsa;
+        dsa.top_k = selection.size();
+        auto picked = ctx.mla_decode_attention_selected(qt.unwrap(), cache, weight.unwrap(), layer, ctx_len - 1, spec, dsa, state.unwrap());
+        CHECK(picked.is_ok(), "mla_decode_attention_selected: %s", picked.is_err() ? picked.unwrap_err().to_string().c_str() : "");
+        if (picked.is_ok()) {
+            std::vector<float> want_sel(spec.num_heads * spec.value_dim());
+            const int rc3 = zo_mla_absorbed_q8_history(&zs, q_bits.data(), 1, ctx_len - 1, codes_dense.data(), scales_dense.data(), 64, rope_dense.data(),
+                                                       ctx_len, kv_b.data(), selection.data(), selection.size(), nullptr, want_sel.data(), nullptr);
+            CHECK(rc3 == 0, "oracle rc %d", rc3);
+            compare(ctx.tensor_to_f32(picked.unwrap()).unwrap(), want_sel, "mla_decode_attention_selected, top_k 64");
+        }
+        dsa.top_k = 63;
+        CHECK(ctx.mla_decode_attention_selected(qt.unwrap(), cache, weight.unwrap(), layer, ctx_len - 1, spec, dsa, state.unwrap()).is_err(),
+              "a state of another top_k must be refused");
+    }
+
     // session snapshot: download -> wire bytes -> parse -> upload into a second cache (other pages), same result bit for bit
     {
         auto layers = ctx.download_layers(cache);

@@ -665,6 +665,42 @@ Result<Unit> RocmContext::append_mla_rope(RocmKvCache& cache, size_t layer, cons
 Result<RocmTensor> RocmContext::mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
                                                      size_t position, const MlaSpec& spec) const
 {
+    return mla_decode_impl(query, cache, kv_b, layer, position, spec, nullptr);
+}
+
+Result<RocmTensor> RocmContext::mla_decode_attention_selected(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b,
+                                                              size_t layer, size_t position, const MlaSpec& mla, const DsaSpec& dsa,
+                                                              const RocmDsaState& state) const
+{
+    if (dsa.top_k == 0 || state.top_k != dsa.top_k || state.selection.data() == nullptr) {
+        return compute_error("Rocm MLA selected decode: the DSA state holds " + std::to_string(state.top_k) + " positions, top_k is " +
+                             std::to_string(dsa.top_k));
+    }
+    return mla_decode_impl(query, cache, kv_b, layer, position, mla, &state);
+}
+
+Result<RocmDsaState> RocmContext::dsa_state_from_selection(const std::vector<uint32_t>& selection) const
+{
+    if (selection.empty()) {
+        return compute_error("Rocm DSA state: empty selection");
+    }
+    auto buffer = DeviceBuffer::allocate(selection.size() * 4);
+    if (buffer.is_err()) {
+        return buffer.unwrap_err();
+    }
+    const hipError_t err = hipMemcpy(buffer.unwrap().data(), selection.data(), selection.size() * 4, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        return hip_error("selection upload", err);
+    }
+    RocmDsaState state;
+    state.selection = buffer.unwrap();
+    state.top_k = selection.size();
+    return state;
+}
+
+Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
+                                                size_t position, const MlaSpec& spec, const RocmDsaState* state) const
+{
     if (auto bad = spec.validate()) {
         return compute_error(*bad);
     }
@@ -721,6 +757,10 @@ Result<RocmTensor> RocmContext::mla_decode_attention(const RocmTensor& query, co
     a.q_dtype = abi_dtype(query.dtype);
     a.out_dtype = ZLLM_DTYPE_F32; // decode rows are written as f32 (src/backend/rocm/attention.rs:17-19)
     a.out_compact = 1;
+    if (state != nullptr) {
+        a.selection = (const uint32_t*)state->selection.data();
+        a.top_k = (uint32_t)state->top_k;
+    }
     const uint64_t need = zllm_attn_mla_decode_workspace_bytes(&a);
     if (need == 0) {
         return abi_error("zllm_attn_mla_decode_workspace_bytes", -1);

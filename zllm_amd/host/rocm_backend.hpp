@@ -83,6 +83,11 @@ struct MlaSpec {
     size_t kv_a_out() const { return kv_lora_rank + qk_rope_head_dim; }
 };
 
+// Sparse-attention (DSA) parameters the selected-token decode needs (src/attention/dsa.rs): the list length.
+struct DsaSpec {
+    size_t top_k = 0;
+};
+
 enum class DType { F32 = 0, BF16 = 1, F16 = 2 };
 size_t dtype_bytes(DType dtype);
 
@@ -109,6 +114,14 @@ struct RocmTensor {
 struct RocmWeight {
     DeviceBuffer device;
     size_t rows = 0, cols = 0;
+};
+
+// What the reference's DsaState hands to the selected-token decode: the token positions the indexer chose for the
+// current query row, `top_k` per row, resident on the device.  The indexer itself (scores, radix top-k) is outside
+// this path; a state is built from a list here.
+struct RocmDsaState {
+    DeviceBuffer selection; // u32 [top_k]
+    size_t top_k = 0;
 };
 
 enum class KvCacheFormat { F16, Q8g64 };
@@ -190,8 +203,15 @@ class RocmContext {
     // query [1, heads * q_head_dim]; returns f32 [1, heads * value_dim]
     Result<RocmTensor> mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
                                             size_t position, const MlaSpec& spec) const;
+    // DecodeBackend::mla_decode_attention_selected (src/backend/mod.rs:1227, ROCm body src/backend/rocm/attention.rs:1927-1940):
+    // a context longer than dsa.top_k attends to the positions in `state` only, a shorter one stays dense.
+    Result<RocmTensor> mla_decode_attention_selected(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
+                                                     size_t position, const MlaSpec& mla, const DsaSpec& dsa, const RocmDsaState& state) const;
+    Result<RocmDsaState> dsa_state_from_selection(const std::vector<uint32_t>& selection) const;
 
   private:
+    Result<RocmTensor> mla_decode_impl(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer, size_t position,
+                                       const MlaSpec& spec, const RocmDsaState* state) const;
     Result<Unit> append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
                                  RotaryLayout layout, size_t position, const float* cos_dev, const float* sin_dev) const;
     int device_id_ = 0;
