@@ -44,16 +44,6 @@ union Frag {
     f16x8 h;
 };
 
-// 4 int8 codes in a dword -> two packed bf16 pairs (exact).
-__device__ __forceinline__ u32x2 codes4_to_bf16(unsigned int w)
-{
-    const float c0 = (float)(int)(signed char)(w & 0xffu);
-    const float c1 = (float)(int)(signed char)((w >> 8) & 0xffu);
-    const float c2 = (float)(int)(signed char)((w >> 16) & 0xffu);
-    const float c3 = (float)(int)(signed char)(w >> 24);
-    return u32x2{pack_bf16_trunc(c0, c1), pack_bf16_trunc(c2, c3)};
-}
-
 __device__ __forceinline__ float byte_to_f32(unsigned int w, int e)
 {
     return (float)(int)(signed char)((w >> (8 * e)) & 0xffu);
@@ -73,7 +63,7 @@ __device__ __forceinline__ float fast_tanh(float x)
 template <int G> struct ScaleRow; // G 16-bit scales of one token / KV head
 template <> struct ScaleRow<1> {
     unsigned short v;
-    __device__ __forceinline__ unsigned short get(int a) const { return v; }
+    __device__ __forceinline__ unsigned short get(int) const { return v; }
 };
 template <> struct ScaleRow<2> {
     unsigned int v;
