@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
-             out_dtype=None, scale=None, outliers=False, gate_cols=0):
+             out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0):
     from zllm_amd import capi, ops
 
     d = 128
@@ -25,8 +25,9 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     gain = np.ones(cols, dtype=np.float32)
     if outliers:  # 1 % of the channels carry values eight times larger
         gain[rng.choice(cols, size=max(1, cols // 100), replace=False)] = 8.0
-    k = rng.standard_normal((total, cols)).astype(np.float32) * gain
-    v = rng.standard_normal((total, cols)).astype(np.float32) * gain
+    # q_gain / k_gain / v_gain: a factor, or one factor per token (rows of the chunk for q), for the magnitude tests
+    k = rng.standard_normal((total, cols)).astype(np.float32) * gain * np.reshape(np.asarray(k_gain, dtype=np.float32), (-1, 1))
+    v = rng.standard_normal((total, cols)).astype(np.float32) * gain * np.reshape(np.asarray(v_gain, dtype=np.float32), (-1, 1))
     # the chunk's K/V arrive as bf16 activations
     k[prefix:] = O.bf16_to_f32(O.f32_to_bf16(k[prefix:]))
     v[prefix:] = O.bf16_to_f32(O.f32_to_bf16(v[prefix:]))
@@ -51,7 +52,7 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
         got = ops.gather_rows(dev[n], table, 0, total, planes[n].shape[1] * planes[n].itemsize, block_tokens).cpu().numpy()
         want = O.gather_rows_bytes(planes[n], tables[0], block_tokens, 0, total, planes[n].shape[1] * planes[n].itemsize)
         assert np.array_equal(got, want), n
-    q = rng.standard_normal((chunk, hq * d)).astype(np.float32)
+    q = rng.standard_normal((chunk, hq * d)).astype(np.float32) * np.reshape(np.asarray(q_gain, dtype=np.float32), (-1, 1))
     q_bits = O.f32_to_bf16(q)
     q = O.bf16_to_f32(q_bits) if q_bf16 else q
     scale = scale or 1.0 / np.sqrt(d)
@@ -110,10 +111,53 @@ def test_prefill_softcap_pages_and_outputs():
     out, want = run_case(71, 400, 100, 16, 8, softcap=30.0, block_tokens=64, rule=O.RULE_ROCM_MLA, scale=0.3)
     assert_attention_close(out.cpu().numpy(), want, "softcap + bf16 scales + 64-token pages")
     out, want = run_case(72, 200, 50, 8, 2, block_tokens=1, q_bf16=False)
-    assert_attention_close(out.cpu().numpy(), want, "1-token pages, f32 queries (rounded to bf16 operands)", atol=4e-3)
+    assert_attention_close(out.cpu().numpy(), want, "1-token pages, f32 queries")
     out, want = run_case(73, 200, 50, 8, 2, out_dtype=torch.bfloat16)
     got = out.float().cpu().numpy()
     assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 2e-3
+
+
+def _close_at_scale(out, want, what):
+    """The 2e-3 / 1e-2 bounds, with the absolute one taken relative to the largest expected magnitude."""
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all(), what
+    top = float(np.abs(want).max())
+    assert top > 0
+    return assert_attention_close(got / top, np.asarray(want, dtype=np.float64) / top, what)
+
+
+@pytest.mark.parametrize("rule,exponent", [(O.RULE_ROCM_MLA, 40), (O.RULE_ROCM_MLA, -40), (O.RULE_METAL_GQA, 11), (O.RULE_METAL_GQA, -12)])
+def test_prefill_value_magnitudes(rule, exponent):
+    """V scales far from 1 (the kernel carries P' = p * v_scale as f16 and must keep it in range), uniformly and
+    with the large values first or last in the sequence (the range the kernel tracks grows while it runs)."""
+    total = 600 + 90
+    flat = float(2.0 ** exponent)
+    print("uniform", _close_at_scale(*run_case(41, 600, 90, 8, 2, rule=rule, v_gain=flat), f"v * 2^{exponent}"))
+    first = np.ones(total, dtype=np.float32)
+    first[:40] = 2.0 ** abs(exponent)
+    print("large first", _close_at_scale(*run_case(42, 600, 90, 8, 2, rule=rule, v_gain=first), "large values first"))
+    last = np.ones(total, dtype=np.float32)
+    last[500:] = 2.0 ** abs(exponent)
+    print("large last", _close_at_scale(*run_case(43, 600, 90, 8, 2, rule=rule, v_gain=last), "large values last"))
+    # a single large row in the middle of the prefix, small ones around it
+    spike = np.full(total, 2.0 ** -abs(exponent) if rule == O.RULE_ROCM_MLA else 2.0 ** -6, dtype=np.float32)
+    spike[333] = 1.0
+    print("spike", _close_at_scale(*run_case(44, 600, 90, 8, 2, rule=rule, v_gain=spike), "one large row"))
+
+
+@pytest.mark.parametrize("q_exp,k_exp", [(12, -12), (-14, 14), (20, 0), (0, -20), (-9, -9)])
+def test_prefill_query_and_key_magnitudes(q_exp, k_exp):
+    """Queries and keys far from unit magnitude with the score scale compensating: the kernel multiplies its query
+    tile by a power of two before rounding it to f16 and folds the inverse into the exponent's argument."""
+    scale = float(2.0 ** -(q_exp + k_exp)) / np.sqrt(128)
+    out, want = run_case(50 + q_exp, 500, 70, 8, 2, rule=O.RULE_ROCM_MLA, q_gain=2.0 ** q_exp, k_gain=2.0 ** k_exp, scale=scale, q_bf16=False)
+    print("q/k magnitudes", q_exp, k_exp, assert_attention_close(out.cpu().numpy(), want, f"q 2^{q_exp}, k 2^{k_exp}"))
+    # one row of the chunk much larger than its neighbours inside the same wave's tile (bf16 queries: its scores have a
+    # standard deviation near 180, so any rounding of the operands would move the output)
+    rows = np.ones(70, dtype=np.float32)
+    rows[7] = 2.0 ** 10
+    out, want = run_case(60 + q_exp, 300, 70, 8, 2, q_gain=rows, scale=1.0 / 64)
+    print("one large query row", assert_attention_close(out.cpu().numpy(), want, "one large query row"))
 
 
 def test_prefill_rejects_unsupported_shapes():

@@ -127,6 +127,26 @@ __device__ __forceinline__ void split_bf16_pair(float x0, float x1, unsigned int
     lo = pack_bf16_hw(x0 - h0, x1 - h1);
 }
 
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// two f32 -> packed f16, round to nearest even (v_cvt_pk_f16_f32)
+__device__ __forceinline__ unsigned int pack_f16_hw(float lo, float hi)
+{
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f32x2{lo, hi}, f16x2));
+}
+
+// Four int8 codes of a word -> four f16 integers (exact), 5 instructions: flipping the sign bits turns a code c
+// into the unsigned byte c + 128; placed under the exponent byte 0x64 it reads as the f16 number 1024 + 128 + c,
+// and one packed subtraction removes the offset.
+__device__ __forceinline__ void codes4_to_f16(unsigned int word, unsigned int& lo, unsigned int& hi)
+{
+    const unsigned int biased = word ^ 0x80808080u;
+    const f16x2 offset = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    lo = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) + offset);
+    hi = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) + offset);
+}
+
 // Reductions across the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48): every lane ends up with
 // the result.  v_permlane16_swap / v_permlane32_swap exchange rows inside the vector ALU, so the reduction
 // does not take the round trip through the LDS crossbar that a generic lane shuffle does.

@@ -1,4 +1,4 @@
-// Chunked-prefill GQA attention over a paged Q8g64 KV cache — gfx950, bf16 MFMA.
+// Chunked-prefill GQA attention over a paged Q8g64 KV cache — gfx950, f16 MFMA.
 //
 // T query rows appended at `position` attend the cached prefix plus the chunk itself (causal,
 // optional sliding window).  Replaces the per-(row, head) block attention the reference runs for this
@@ -7,11 +7,17 @@
 // A workgroup (8 waves) owns one KV head and a tile of query rows; its 256 MFMA columns enumerate
 // (row, head-in-group) pairs, 32 per wave, so one K/V tile serves every query head of the group.
 // Two waves share a SIMD, so the LDS and MFMA latencies of one are covered by the other.
-// Per 32-token step the workgroup converts the K and V codes ONCE into LDS as bf16 integers (exact)
+// Per 32-token step the workgroup converts the K and V codes ONCE into LDS as f16 integers (exact)
 // with their f32 group scales beside them; each wave then runs
-//   S^T[token, col]  = sum_g k_scale[token, g] * (Kcodes_g[token, :] . Q_g[col, :])   (MFMA, exact products)
+//   S^T[token, col]  = sum_g k_scale[token, g] * (Kcodes_g[token, :] . Q'_g[col, :])   (f16 MFMA, exact products)
 //   online softmax per column (wave shuffles)
-//   O^T[dim, col]   += Vcodes^T[dim, token] . P'_g[token, col],  P'_g = p * v_scale_g as bf16 hi + lo
+//   O^T[dim, col]   += Vcodes^T[dim, token] . P'_g[token, col],  P'_g = p * v_scale_g as f16 hi (+ lo)
+// The codes stay integers on purpose: a tile of code * scale products rounded to f16 moves single scores by
+// up to 2^-11 of their largest term, which outlier channels turn into output errors above the 2e-3 bound.
+// Q' is the wave's query tile times one power of two (largest magnitude in [2^8, 2^9)), undone in the fused
+// multiply-add that feeds exp2.  P' must stay inside f16 range for any scale a cache can hold: the exponent of
+// the largest V scale met so far (reduced by wave 0 one step ahead of the tile) is subtracted from the softmax
+// reference, so accumulators and running sum carry the same power of two and it cancels in the division.
 // K is read from LDS with ds_read_b128, V transposed with ds_read_b64_tr_b16; a 16-byte XOR swizzle
 // keeps both conflict-free.
 #include "common.hpp"
@@ -21,12 +27,16 @@ namespace zllm {
 
 namespace {
 
+// Fences for the instruction scheduler between the phases of a step (they keep the early LDS requests early).
+#define PREFILL_PHASE_FENCE() __builtin_amdgcn_sched_barrier(0)
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kStep = 32;                 // tokens per step
 constexpr int kD = 128;                   // head_dim handled by this kernel
 constexpr int kRowBytes = kD * 2;         // one token of one KV head as bf16
 constexpr int kTileBytes = kStep * kRowBytes; // 8 KiB
-constexpr float kLoThreshold = 64.0f;       // see the P.V stage
+constexpr float kPBias = 8.0f;            // probabilities are carried as p * 2^8: f16 stays normal down to p = 2^-22
+constexpr float kLoThreshold = 8.0f;      // see the P.V stage
 constexpr int kColTiles = 2;              // 16-column MFMA tiles per wave
 constexpr int kWaves = 256 / (16 * kColTiles);
 constexpr int kThreads = 64 * kWaves;
@@ -35,7 +45,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 union Frag {
     u32x4 u;
-    bf16x8 b;
+    f16x8 h;
 };
 
 // Chunk swizzle for the 64-bank LDS (256 B per cycle = one tile row).  Row bits 1 and 2 are XOR-ed into chunk
@@ -67,6 +77,12 @@ struct StepRegs {
     unsigned int scales;   // two 16-bit scales (groups 0, 1) of the token
 };
 
+// Biased exponent of a (positive) scale, clamped away from the ends of the f32 range.
+__device__ __forceinline__ unsigned int window_exponent(float top)
+{
+    return min(max((__float_as_uint(top) >> 23) & 0xffu, 2u), 252u);
+}
+
 template <int SDT, bool SOFTCAP>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
@@ -74,6 +90,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     __shared__ __align__(16) unsigned char lds_v[2][kTileBytes];
     __shared__ __align__(16) float lds_ks[2][2][kStep]; // [buffer][group][token]
     __shared__ __align__(16) float lds_vs[2][2][kStep];
+    __shared__ __align__(16) float lds_top[2][8];       // [buffer][staging wave]: largest scale the wave converted (4..7: V)
 
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -97,30 +114,52 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const unsigned int steps = (t_end - t_begin + kStep - 1) / kStep;
 
     // ---- this wave's columns and Q fragments -------------------------------------------------
+    // The wave's queries are carried as f16 after a multiplication by one power of two that puts the largest
+    // magnitude of its 32 columns into [2^8, 2^9); the inverse goes into the score factor.
     unsigned int col_row[kColTiles], col_head[kColTiles];
     bool col_valid[kColTiles];
     Frag qf[kColTiles][4];
+    float q_fac;
+    {
+        float qx[kColTiles][4][8];
+        float q_amax = 0.0f;
 #pragma unroll
-    for (int ct = 0; ct < kColTiles; ++ct) {
-        const unsigned int col = wave * (16u * kColTiles) + ct * 16u + m;
-        const unsigned int r = row0 + col / p.group;
-        col_row[ct] = r;
-        col_head[ct] = kvh * p.group + col % p.group;
-        col_valid[ct] = col < cols_used && r < p.rows;
+        for (int ct = 0; ct < kColTiles; ++ct) {
+            const unsigned int col = wave * (16u * kColTiles) + ct * 16u + m;
+            const unsigned int r = row0 + col / p.group;
+            col_row[ct] = r;
+            col_head[ct] = kvh * p.group + col % p.group;
+            col_valid[ct] = col < cols_used && r < p.rows;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            float x[8];
+            for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[e] = col_valid[ct] ? load_as_f32(p.q, ((size_t)r * p.num_heads + col_head[ct]) * kD + ks * 32 + j * 8 + e, p.q_dtype) : 0.0f;
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                qf[ct][ks].u[e] = pack_bf16_hw(x[2 * e], x[2 * e + 1]);
+                for (int e = 0; e < 8; ++e) {
+                    const float x = col_valid[ct] ? load_as_f32(p.q, ((size_t)r * p.num_heads + col_head[ct]) * kD + ks * 32 + j * 8 + e, p.q_dtype) : 0.0f;
+                    qx[ct][ks][e] = x;
+                    q_amax = fmaxf(q_amax, fabsf(x));
+                }
             }
         }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            q_amax = fmaxf(q_amax, __shfl_xor(q_amax, off));
+        }
+        const unsigned int q_exp = min(max((__float_as_uint(q_amax) >> 23) & 0xffu, 16u), 240u);
+        const float q_mul = __uint_as_float((262u - q_exp) << 23); // 2^(127 + 8 - q_exp)
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ++ct) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    qf[ct][ks].u[e] = pack_f16_hw(qx[ct][ks][2 * e] * q_mul, qx[ct][ks][2 * e + 1] * q_mul);
+                }
+            }
+        }
+        q_fac = ldexpf(1.0f, (int)q_exp - 135);
     }
 
+    // scores come out in base-2 units unless the soft cap needs them in natural ones first
     const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
     const float cap_log2 = p.softcap * kLog2e;
@@ -154,31 +193,42 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         r.scales = *(const unsigned int*)(st_scales + row * s_row);
     };
     auto convert8 = [&](const u32x2& codes) __attribute__((always_inline)) -> u32x4 {
-        u32x4 out;
-#pragma unroll
-        for (int w = 0; w < 2; ++w) {
-            const unsigned int word = codes[w];
-            const float c0 = (float)(int)(signed char)(word & 0xffu);
-            const float c1 = (float)(int)(signed char)((word >> 8) & 0xffu);
-            const float c2 = (float)(int)(signed char)((word >> 16) & 0xffu);
-            const float c3 = (float)(int)(signed char)(word >> 24);
-            out[2 * w] = pack_bf16_trunc(c0, c1);
-            out[2 * w + 1] = pack_bf16_trunc(c2, c3);
-        }
-        return out;
+        unsigned int a, b, c, d;
+        codes4_to_f16(codes[0], a, b);
+        codes4_to_f16(codes[1], c, d);
+        return u32x4{a, b, c, d};
     };
     auto store_step = [&](const StepRegs& r, int buf) __attribute__((always_inline)) {
         // chunks cc and cc + 8: sixteen lanes (two rows x eight chunks) write sixteen different bank groups
         unsigned char* tile = stage_v ? lds_v[buf] : lds_k[buf];
         *(u32x4*)(tile + tile_offset(st_token, cc)) = convert8(r.codes[0]);
         *(u32x4*)(tile + tile_offset(st_token, cc + 8u)) = convert8(r.codes[1]);
+        // the eight threads of a token all hold its two scales; K scales carry the score scale (and log2 e) so that
+        // the hot loop does not multiply again
+        const float s0 = scale_bits_to_f32<SDT>((unsigned short)(r.scales & 0xffffu));
+        const float s1 = scale_bits_to_f32<SDT>((unsigned short)(r.scales >> 16));
         if (cc == 0) {
-            // K scales carry the score scale (and log2 e) so that the hot loop does not multiply again
             float* dst = stage_v ? &lds_vs[buf][0][0] : &lds_ks[buf][0][0];
             const float fold = stage_v ? 1.0f : scale_log2;
-            dst[st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales & 0xffffu)) * fold;
-            dst[kStep + st_token] = scale_bits_to_f32<SDT>((unsigned short)(r.scales >> 16)) * fold;
+            dst[st_token] = s0 * fold;
+            dst[kStep + st_token] = s1 * fold;
         }
+        // largest scale of the wave's eight tokens (a row of sixteen lanes holds two)
+        float top = fmaxf(s0, s1);
+        top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x128, 0xf, 0xf, false))); // row_ror:8
+        const float rows01 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
+                                   __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 16)));
+        const float rows23 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 32)),
+                                   __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 48)));
+        if (lane == 0) {
+            lds_top[buf][wave] = fmaxf(rows01, rows23);
+        }
+    };
+    // (biased) exponent of the largest V scale of the tile in `buf`, folded into the running one
+    auto window_of = [&](int buf, unsigned int wv) __attribute__((always_inline)) -> unsigned int {
+        const f32x4 tops = *(const f32x4*)&lds_top[buf][4];
+        const float top = fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3]));
+        return max(wv, (unsigned int)__builtin_amdgcn_readfirstlane(window_exponent(top)));
     };
 
     f32x4 acc[kColTiles][8];
@@ -211,10 +261,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ (tr_row & 6u)) << 4) + (m & 1u) * 8u;
     }
 
-    auto compute_step = [&](int buf, unsigned int t0) __attribute__((always_inline)) {
+    // `v_shift` = 8 - (V window exponent) is added to every score before exp2; `acc_fix` is 2^-(growth of that
+    // window since the last step), 1 almost always.
+    auto compute_step = [&](int buf, unsigned int t0, float v_shift, float acc_fix) __attribute__((always_inline)) {
         const unsigned char* kt = lds_k[buf];
-        const unsigned char* vt = lds_v[buf];
-        // ---- S^T = sum_g k_scale_g * (Kcodes_g . Q_g) -------------------------------------------
+        // ---- S^T = sum_g k_scale_g * (Kcodes_g . Q'_g) ------------------------------------------
         f32x4 s[2][kColTiles];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -231,8 +282,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
                     f32x4 d = {0.f, 0.f, 0.f, 0.f};
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.b, qf[ct][2 * g].b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.b, qf[ct][2 * g + 1].b, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0.h, qf[ct][2 * g].h, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1.h, qf[ct][2 * g + 1].h, d, 0, 0, 0);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         s[i][ct][r] = fmaf(d[r], gs[r], s[i][ct][r]);
@@ -240,21 +291,43 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                 }
             }
         }
+        // The P.V operands that do not depend on the softmax are requested now, so that their LDS round trips pass under
+        // its vector-ALU work: the V^T fragments of scale group 0 and the V scales of both groups.
+        const unsigned char* vt = lds_v[buf];
+        union VFrag {
+            s16x4 s[2];
+            f16x8 h;
+        };
+        auto load_vfrags = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                const unsigned char* at = vt + pv_base[tt] + pv_group[g];
+                vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
+            }
+        };
+        VFrag vf[2][4];
+        f32x4 gsv[2][2];
+        load_vfrags(vf[0], 0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            gsv[g][0] = *(const f32x4*)(&lds_vs[buf][g][4 * j]);
+            gsv[g][1] = *(const f32x4*)(&lds_vs[buf][g][16 + 4 * j]);
+        }
+        PREFILL_PHASE_FENCE();
         // ---- online softmax per column --------------------------------------------------------------
         float pr[kColTiles][8];
-        float alpha[kColTiles];
         bool heavy = false; // some probability of this step is not small against the sum so far
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ++ct) {
             float sc[8];
-            float step_max = kNegInf;
             // only steps that touch a causal or window edge of some column need the per-token masks
             const bool edge = __any(t0 + kStep > vis_hi[ct] || t0 < vis_lo[ct]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 float x = s[e >> 2][ct][e & 3];
                 if constexpr (SOFTCAP) {
-                    x = cap_log2 * soft_tanh(x * inv_cap);
+                    x = cap_log2 * soft_tanh(x * q_fac * inv_cap);
                 }
                 sc[e] = x;
             }
@@ -265,42 +338,42 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                     sc[e] = (token >= vis_lo[ct] && token < vis_hi[ct]) ? sc[e] : kNegInf;
                 }
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                step_max = fmaxf(step_max, sc[e]);
-            }
-            step_max = wave_max_16x4(step_max);
+            // the query's power of two is positive, so maxima are taken first and it rides in the multiply-add
+            const float mult = SOFTCAP ? 1.0f : q_fac;
+            const float lane_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            const float step_max = wave_max_16x4(lane_max) * mult;
             const float new_max = fmaxf(run_max[ct], step_max);
             const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-            alpha[ct] = __builtin_amdgcn_exp2f(run_max[ct] - safe_max);
+            const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max) * acc_fix;
+            const float shift = v_shift - safe_max;
             float step_sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                pr[ct][e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
+                pr[ct][e] = __builtin_amdgcn_exp2f(fmaf(sc[e], mult, shift));
                 step_sum += pr[ct][e];
             }
-            run_sum[ct] = run_sum[ct] * alpha[ct] + step_sum;
+            run_sum[ct] = run_sum[ct] * alpha + step_sum;
             run_max[ct] = new_max;
-            const float p_top = fmaxf(fmaxf(fmaxf(pr[ct][0], pr[ct][1]), fmaxf(pr[ct][2], pr[ct][3])),
-                                      fmaxf(fmaxf(pr[ct][4], pr[ct][5]), fmaxf(pr[ct][6], pr[ct][7])));
+            const float p_top = __builtin_amdgcn_exp2f(fmaf(lane_max, mult, shift)); // the lane's largest probability
             heavy = heavy || p_top * kLoThreshold > run_sum[ct];
-            if (__any(alpha[ct] != 1.0f)) { // the running max settles early in a long prefix
+            if (__any(alpha != 1.0f)) { // the running max settles early in a long prefix
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    acc[ct][t] *= alpha[ct];
+                    acc[ct][t] *= alpha;
                 }
             }
         }
         // ---- O^T += Vcodes^T . P'_g ----------------------------------------------------------------------
-        // P' is carried as bf16 hi + lo (16 significant bits) while any probability of the step weighs more
-        // than 1/64 of its lane's running sum (a lane sums a quarter of the tokens, so < 1/256 of the row's);
-        // below that the hi term's rounding (2^-9 relative, random
-        // sign) moves the normalised output by < 2^-9 / 16 of |v|, so the lo product is skipped.
+        // P' is carried as f16 hi + lo (22 significant bits) while any probability of the step weighs more
+        // than 1/8 of its lane's running sum (a lane sums a quarter of the tokens, so < 1/32 of the row's);
+        // below that the hi term's rounding (2^-12 relative, random sign) moves the normalised output by
+        // < 2^-12 / 32 of |v|, so the lo product is skipped.
         const bool lo_pass = __any(heavy);
+        PREFILL_PHASE_FENCE();
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            const f32x4 gs0 = *(const f32x4*)(&lds_vs[buf][g][4 * j]);
-            const f32x4 gs1 = *(const f32x4*)(&lds_vs[buf][g][16 + 4 * j]);
+            const f32x4 gs0 = gsv[g][0];
+            const f32x4 gs1 = gsv[g][1];
             Frag phi[kColTiles], plo[kColTiles];
 #pragma unroll
             for (int ct = 0; ct < kColTiles; ++ct) {
@@ -308,71 +381,59 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                 for (int e = 0; e < 4; ++e) {
                     const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
                     const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
-                    phi[ct].u[e] = pack_bf16_hw(x0, x1);
+                    phi[ct].u[e] = pack_f16_hw(x0, x1);
                 }
             }
-            if (lo_pass) {
+            if (g == 0) { // group 1's fragments travel while group 0 multiplies
+                load_vfrags(vf[1], 1);
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ++ct) {
+                    acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[g][tt].h, phi[ct].h, acc[ct][g * 4 + tt], 0, 0, 0);
+                }
+            }
+            if (lo_pass) { // rare: one branch around the low-order products
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
                         const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
-                        unsigned int hi, lo;
-                        split_bf16_pair(x0, x1, hi, lo);
-                        plo[ct].u[e] = lo;
+                        const f16x2 hi = __builtin_bit_cast(f16x2, pack_f16_hw(x0, x1));
+                        plo[ct].u[e] = pack_f16_hw(x0 - (float)hi[0], x1 - (float)hi[1]);
                     }
                 }
-            }
-            // all eight V^T fragment reads of the group are requested before the first MFMA, and the low-order pass is one
-            // branch around its own loop: with the reads and the branch inside the tile loop every tile paid an LDS round
-            // trip in front of its four MFMAs
-            union VFrag {
-                s16x4 s[2];
-                bf16x8 b;
-            };
-            VFrag vf[4];
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
-                const unsigned char* at = vt + pv_base[tt] + pv_group[g];
-                vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-                vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
-            }
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
-#pragma unroll
-                for (int ct = 0; ct < kColTiles; ++ct) {
-                    acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[tt].b, phi[ct].b, acc[ct][g * 4 + tt], 0, 0, 0);
-                }
-            }
-            if (lo_pass) {
 #pragma unroll
                 for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
                     for (int ct = 0; ct < kColTiles; ++ct) {
-                        acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[tt].b, plo[ct].b, acc[ct][g * 4 + tt], 0, 0, 0);
+                        acc[ct][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[g][tt].h, plo[ct].h, acc[ct][g * 4 + tt], 0, 0, 0);
                     }
                 }
             }
         }
     };
 
+    // ---- main loop ------------------------------------------------------------------------------------------
     StepRegs regs;
     load_step(regs, t_begin, entry_of(t_begin + st_token));
     unsigned int entry_next = entry_of(t_begin + kStep + st_token);
     store_step(regs, 0);
     __syncthreads();
+    unsigned int wv = 2u; // (biased) exponent of the largest V scale up to the tile being attended
     for (unsigned int step = 0; step < steps; ++step) {
-        const bool more = step + 1 < steps;
-        if (more) {
-            const unsigned int t_next = t_begin + (step + 1u) * kStep;
-            load_step(regs, t_next, entry_next);
-            entry_next = entry_of(t_next + kStep + st_token);
-        }
-        compute_step((int)(step & 1u), t_begin + step * kStep);
-        if (more) {
-            store_step(regs, (int)((step + 1u) & 1u));
-        }
+        const unsigned int t0 = t_begin + step * kStep;
+        const int buf = (int)(step & 1u);
+        // rows past the end of the visible range repeat its last one: the loads stay inside the sequence's pages
+        load_step(regs, t0 + kStep, entry_next);
+        entry_next = entry_of(t0 + 2u * kStep + st_token);
+        const unsigned int wv_now = window_of(buf, wv);
+        const float acc_fix = wv_now != wv ? ldexpf(1.0f, (int)wv - (int)wv_now) : 1.0f;
+        wv = wv_now;
+        compute_step(buf, t0, kPBias + (float)(127 - (int)wv), acc_fix);
+        store_step(regs, buf ^ 1);
         __syncthreads();
     }
 
@@ -383,6 +444,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         if (!col_valid[ct]) {
             continue;
         }
+        // accumulators and sum carry the same power of two (2^8 and the V window), which cancels here
         const float inv = (total > 0.0f && total < __builtin_inff()) ? 1.0f / total : 0.0f;
         const size_t base = ((size_t)col_row[ct] * p.num_heads + col_head[ct]) * kD;
 #pragma unroll

@@ -47,26 +47,6 @@ union Frag {
     f16x8 h;
 };
 
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-// two f32 -> packed f16, round to nearest even (v_cvt_pk_f16_f32)
-__device__ __forceinline__ unsigned int pack_f16_hw(float lo, float hi)
-{
-    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f32x2{lo, hi}, f16x2));
-}
-
-// Four int8 codes of a word -> four f16 integers (exact), 5 instructions: flipping the sign bits turns a code c
-// into the unsigned byte c + 128; placed under the exponent byte 0x64 it reads as the f16 number 1024 + 128 + c,
-// and one packed subtraction removes the offset.
-__device__ __forceinline__ void codes4_to_f16(unsigned int word, unsigned int& lo, unsigned int& hi)
-{
-    const unsigned int biased = word ^ 0x80808080u;
-    const f16x2 offset = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-    lo = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) + offset);
-    hi = __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) + offset);
-}
-
 // Chunk swizzle for the 64-bank LDS (256 B per cycle).  A tile row is 72 chunks of 16 B, i.e. 8 chunks past a
 // multiple of 256 B, so the row's parity already selects the upper or lower 128 B of a bank line; XOR-ing
 // row bits 1 and 2 into chunk bits 1 and 2 spreads eight rows over all sixteen 16-byte slots.  Measured with
