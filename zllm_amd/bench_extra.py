@@ -113,7 +113,7 @@ def run_mla_decode(args):
     record = {
         "metric": "MLA decode attn TFLOP/s (% of bf16 MFMA peak) + tokens/s at 64K ctx, 1 GPU",
         "value": round(tflops_call, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "C4 absorbed MLA decode, B=4, 128 heads, latent 512 Q8g64 + rope 64 bf16, ctx 65536, 64-token pages",
                    "algorithmic_flops_per_call": flops, "kv_bytes_per_call": kv_bytes, "seed": args.seed,

@@ -67,7 +67,7 @@ def run(args):
     record = {
         "metric": "chunked-prefill GQA attn TFLOP/s (% of bf16 MFMA peak), 2048-row chunk on a 50K prefix, 1 GPU",
         "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "C5 chunked prefill GQA, B=1, 2048-row chunk on a 50,000-token Q8g64 prefix, 64q/8kv, d=128, 16-token pages",
                    "algorithmic_flops_per_call": flops, "causal_pairs_per_head": pairs, "seed": args.seed},
