@@ -45,8 +45,9 @@ def draw_tables(rng, lens, block_tokens, pool_blocks=None, layout="random"):
 
 
 def make_gqa_q8_case(seed, lens, hq, hkv, d, block_tokens=16, rule=O.RULE_METAL_GQA, outliers=False, layout="random",
-                     q_bf16=False, pool_blocks=None, q_std=1.0):
-    """K/V ~ N(0,1) (optionally 1 % outlier channels x8), quantized Q8g64 by the oracle into a paged pool."""
+                     q_bf16=False, pool_blocks=None, q_std=1.0, k_gain=1.0, v_gain=1.0):
+    """K/V ~ N(0,1) (optionally 1 % outlier channels x8), quantized Q8g64 by the oracle into a paged pool.
+    k_gain / v_gain: one factor, or one per token of the longest sequence (magnitude tests)."""
     rng = np.random.default_rng(seed)
     lens = [int(l) for l in lens]
     cols = hkv * d
@@ -66,8 +67,10 @@ def make_gqa_q8_case(seed, lens, hq, hkv, d, block_tokens=16, rule=O.RULE_METAL_
         picks = rng.choice(cols, size=max(1, cols // 100), replace=False)
         channel_gain[picks] = 8.0
     for b, length in enumerate(lens):
-        k = rng.standard_normal((length, cols)).astype(np.float32) * channel_gain
-        v = rng.standard_normal((length, cols)).astype(np.float32) * channel_gain
+        kg = np.reshape(np.asarray(k_gain, dtype=np.float32), (-1, 1))
+        vg = np.reshape(np.asarray(v_gain, dtype=np.float32), (-1, 1))
+        k = rng.standard_normal((length, cols)).astype(np.float32) * channel_gain * (kg if kg.shape[0] == 1 else kg[:length])
+        v = rng.standard_normal((length, cols)).astype(np.float32) * channel_gain * (vg if vg.shape[0] == 1 else vg[:length])
         raw_k.append(k)
         raw_v.append(v)
         if length:

@@ -189,7 +189,7 @@ def test_large_pool_exercises_64_bit_offsets():
 
 
 # ---------------------------------------------------------------------------- f16 KV (config 3)
-def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0):
+def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0):
     rng = np.random.default_rng(seed)
     cols = hkv * d
     cap_lens = [min(l, ring_capacity) if ring_capacity else l for l in lens]
@@ -197,11 +197,13 @@ def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0):
     rows = pool_blocks * block_tokens
     planes = {"k": np.zeros((rows, cols), dtype=np.uint16), "v": np.zeros((rows, cols), dtype=np.uint16)}
     for b, l in enumerate(lens):
-        k = rng.standard_normal((l, cols)).astype(np.float32)
-        v = rng.standard_normal((l, cols)).astype(np.float32)
+        kg = np.reshape(np.asarray(k_gain, dtype=np.float32), (-1, 1))
+        vg = np.reshape(np.asarray(v_gain, dtype=np.float32), (-1, 1))
+        k = rng.standard_normal((l, cols)).astype(np.float32) * (kg if kg.shape[0] == 1 else kg[:l])
+        v = rng.standard_normal((l, cols)).astype(np.float32) * (vg if vg.shape[0] == 1 else vg[:l])
         O.half_append_paged(1, k, planes["k"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
         O.half_append_paged(1, v, planes["v"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
-    q = rng.standard_normal((len(lens), hq * d)).astype(np.float32)
+    q = (rng.standard_normal((len(lens), hq * d)) * q_std).astype(np.float32)
     return dict(q=q, q_bits=None, lens=np.array(lens, dtype=np.uint32), tables=tables, planes=planes, hq=hq, hkv=hkv, d=d,
                 block_tokens=block_tokens, scale_dtype=0)
 
@@ -279,3 +281,49 @@ def test_query_dtypes_through_fixed_point_digits(q_kind):
     torch.cuda.synchronize()
     want = oracle_gqa_decode(case, 0.09)
     assert_attention_close(out.cpu().numpy(), want, f"q dtype {q_kind}")
+
+
+def _close_at_scale(got, want, what):
+    """The 2e-3 / 1e-2 bounds, with the absolute one taken relative to the largest expected magnitude."""
+    assert np.isfinite(got).all(), what
+    top = float(np.abs(want).max())
+    assert top > 0
+    return assert_attention_close(got / top, want / top, what)
+
+
+@pytest.mark.parametrize("rule,exponent", [(O.RULE_ROCM_MLA, 40), (O.RULE_ROCM_MLA, -40), (O.RULE_METAL_GQA, 11), (O.RULE_METAL_GQA, -12)])
+def test_q8_value_and_key_magnitudes(rule, exponent):
+    """Scales far from 1 in both 16-bit storage conventions: uniformly, with the large rows first, last, or alone in the
+    middle; keys and queries scaled against a compensating score scale."""
+    lens = [1500, 300, 64]
+    flat = float(2.0 ** exponent)
+    case = make_gqa_q8_case(500, lens, 16, 4, 128, rule=rule, v_gain=flat)
+    print("uniform v", _close_at_scale(run_decode(case, 0.088), oracle_gqa_decode(case, 0.088), f"v * 2^{exponent}"))
+    big = float(2.0 ** abs(exponent))
+    for name, rows in (("large first", slice(0, 40)), ("large last", slice(1400, 1500)), ("spike", slice(700, 701))):
+        gain = np.ones(max(lens), dtype=np.float32)
+        gain[rows] = big
+        case = make_gqa_q8_case(501, lens, 16, 4, 128, rule=rule, v_gain=gain)
+        print(name, _close_at_scale(run_decode(case, 0.088), oracle_gqa_decode(case, 0.088), f"{name}, 2^{abs(exponent)}"))
+    scale = 0.088 / flat
+    case = make_gqa_q8_case(502, lens, 16, 4, 128, rule=rule, k_gain=flat)
+    print("k", assert_attention_close(run_decode(case, scale), oracle_gqa_decode(case, scale), f"k * 2^{exponent}"))
+    case = make_gqa_q8_case(503, lens, 16, 4, 128, rule=rule, q_std=flat)
+    print("q", assert_attention_close(run_decode(case, scale), oracle_gqa_decode(case, scale), f"q * 2^{exponent}"))
+
+
+@pytest.mark.parametrize("exponent", [10, -10])
+def test_f16_kv_magnitudes(exponent):
+    """f16 K/V near the ends of what f16 rows can hold, and queries far from unit size."""
+    lens = [2000, 77]
+    flat = float(2.0 ** exponent)
+    case = make_f16_case(510, lens, 16, 8, 256, v_gain=flat)
+    print("uniform v", _close_at_scale(run_f16(case, 0.0625), oracle_gqa_decode(case, 0.0625, fmt=O.FMT_F16), f"v * 2^{exponent}"))
+    gain = np.full(max(lens), 2.0 ** -abs(exponent), dtype=np.float32)
+    gain[1234] = 2.0 ** abs(exponent)
+    case = make_f16_case(511, lens, 16, 8, 256, v_gain=gain)
+    print("spike", _close_at_scale(run_f16(case, 0.0625), oracle_gqa_decode(case, 0.0625, fmt=O.FMT_F16), "one large row"))
+    case = make_f16_case(512, lens, 16, 8, 256, k_gain=flat)
+    print("k", assert_attention_close(run_f16(case, 0.0625 / flat), oracle_gqa_decode(case, 0.0625 / flat, fmt=O.FMT_F16), f"k * 2^{exponent}"))
+    case = make_f16_case(513, lens, 16, 8, 256, q_std=flat * flat)
+    print("q", assert_attention_close(run_f16(case, 0.0625 / (flat * flat)), oracle_gqa_decode(case, 0.0625 / (flat * flat), fmt=O.FMT_F16), "q"))

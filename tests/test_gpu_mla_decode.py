@@ -15,7 +15,7 @@ torch = pytest.importorskip("torch")
 
 
 def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, block_tokens=16, layout="random", w_std=None,
-                  poison=False):
+                  poison=False, latent_gain=1.0):
     rng = np.random.default_rng(seed)
     tables, pool_blocks = draw_tables(rng, lens, block_tokens, layout=layout)
     rows = pool_blocks * block_tokens
@@ -27,7 +27,9 @@ def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, b
         scales[:] = 0x7FC0
         rope_cache[:] = 0x7FC0
     for b, l in enumerate(lens):
-        lat = rng.standard_normal((l, latent)).astype(np.float32)
+        # latent_gain: one factor, or one per token of the longest sequence (magnitude tests)
+        gain = np.reshape(np.asarray(latent_gain, dtype=np.float32), (-1, 1))
+        lat = rng.standard_normal((l, latent)).astype(np.float32) * (gain if gain.shape[0] == 1 else gain[:l])
         kr = rng.standard_normal((l, rope)).astype(np.float32)
         O.q8g64_append_paged(O.RULE_ROCM_MLA, lat, codes, scales, tables[b], 0, block_tokens)
         O.half_append_paged(0, kr, rope_cache, tables[b], 0, block_tokens)
@@ -138,6 +140,25 @@ def test_mla_rows_past_the_end_of_a_page_are_ignored(block_tokens):
     got = run_mla(case).cpu().numpy()
     assert np.isfinite(got).all()
     assert_attention_close(got, want_f, f"poisoned tail, block_tokens={block_tokens}")
+
+
+@pytest.mark.parametrize("exponent", [30, -30, 12])
+def test_mla_latent_magnitudes(exponent):
+    """Latent rows far from unit magnitude (the kernel carries P' = p * scale as f16 inside an exponent window that follows
+    the largest scale met so far), with kv_b scaled the other way so that scores and outputs keep their size."""
+    heads, lens = 32, [900, 130]
+    flat, w_std = float(2.0 ** exponent), float(2.0 ** -exponent) / np.sqrt(512)
+    case = make_mla_case(300 + exponent, lens, heads, w_std=w_std, latent_gain=flat)
+    want, _ = oracle_mla(case)
+    print("uniform", assert_attention_close(run_mla(case).cpu().numpy(), want, f"latent * 2^{exponent}"))
+    # rows of mixed magnitude: a large row also has large scores, so it takes the whole softmax when it is visible
+    for name, rows in (("large first", slice(0, 20)), ("large last", slice(800, 900)), ("spike", slice(444, 445))):
+        gain = np.full(max(lens), flat, dtype=np.float32)
+        gain[rows] = flat * 64.0
+        case = make_mla_case(310 + exponent, lens, heads, w_std=w_std, latent_gain=gain)
+        want, _ = oracle_mla(case)
+        top = float(np.abs(want).max())  # outputs are 64 times larger here: the absolute bound scales with them
+        print(name, top, assert_attention_close(run_mla(case).cpu().numpy() / top, want / top, f"{name}, 2^{exponent}"))
 
 
 def draw_selection(rng, lens, top_k, sort):
