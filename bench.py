@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration", "read_calibration"])
     ap.add_argument("--pool-gib", type=float, default=160.0, help="address span of the paged pool (all four planes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -262,6 +262,16 @@ def run_gqa_decode(args, ragged, config1=False):
                      "kernel_ms": round(ms_partial, 5), "kernel_ms_median": round(ms_partial_median, 5),
                      "kernel_ms_min": round(ms_partial_min, 5)},
     }
+    if not config1:
+        # what a kernel that only reads the same number of bytes reaches, timed the same way in the same process
+        probe_src = torch.empty(kv_bytes // 16 * 16, dtype=torch.uint8, device="cuda").random_(0, 255)
+        probe_sink = torch.full((1,), 7, dtype=torch.int32, device="cuda")
+        for _ in range(10):
+            ops.stream_read_probe(probe_src, probe_sink)
+        probe_median, probe_min = event_times_ms(lambda: ops.stream_read_probe(probe_src, probe_sink), 100)
+        record["roofline"]["plain_read_of_same_bytes"] = {"kernel_ms_median": round(probe_median, 5), "kernel_ms_min": round(probe_min, 5),
+                                                          "gbps_median": round(probe_src.numel() / (probe_median * 1e-3) / 1e9, 1)}
+        del probe_src
     if not args.no_cpu_baseline:
         cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)
         record["cpu_baseline"] = cpu
@@ -285,6 +295,31 @@ def run_copy_calibration(args):
                       "config": {"workload": "torch uint8 copy_", "bytes_read": n, "bytes_written": n}}))
 
 
+def run_read_calibration(args):
+    """A plain streaming read (16-byte loads, nothing kept) over as many bytes as the headline decode call has KV bytes,
+    and over four times as many: what reading every KV byte once can reach on this device, next to the published peak."""
+    import torch
+
+    from zllm_amd import ops
+
+    kv_bytes = 8 * 32768 * 2112  # config 2, all sequences at 32K
+    sink = torch.full((1,), 7, dtype=torch.int32, device="cuda")
+    results = {}
+    for name, n in (("kv_bytes", kv_bytes), ("four_times", 4 * kv_bytes)):
+        src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+        for _ in range(args.warmup):
+            ops.stream_read_probe(src, sink)
+        med, low = event_times_ms(lambda: ops.stream_read_probe(src, sink), args.steps)
+        results[name] = {"bytes": n, "kernel_ms_median": round(med, 5), "kernel_ms_min": round(low, 5),
+                         "gbps_median": round(n / (med * 1e-3) / 1e9, 1), "gbps_best": round(n / (low * 1e-3) / 1e9, 1)}
+        del src
+    first = results["kv_bytes"]
+    print(json.dumps({"metric": "plain streaming read (ceiling calibration)", "value": first["gbps_median"], "unit": "GB/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["kernel_ms_median"],
+                      "config": {"workload": "zllm_attn_stream_read_probe over the config-2 KV bytes and four times as many", **results},
+                      "frac_of_hbm_peak": round(first["gbps_median"] / HBM_PEAK_GBPS, 4)}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -298,6 +333,8 @@ def main():
         run_gqa_decode(args, ragged=False, config1=True)
     elif args.workload == "copy_calibration":
         run_copy_calibration(args)
+    elif args.workload == "read_calibration":
+        run_read_calibration(args)
     else:
         from zllm_amd import bench_extra
 

@@ -190,6 +190,13 @@ typedef struct zllm_scatter_args {
 } zllm_scatter_args;
 ZLLM_API int zllm_attn_scatter_rows(const zllm_scatter_args* args, zllm_stream_t stream);
 
+/* Measurement aid with no counterpart in the reference: reads `bytes` (a multiple of 16, 16-byte aligned)
+ * of device memory once with plain wide loads and keeps nothing (`sink`: one device word the kernel
+ * never changes in practice).  bench.py times it over a buffer of the decode workload's KV bytes: the
+ * rate it reaches is what "every KV byte read once" can reach on the device at that size, next to the
+ * published HBM peak the roofline fraction is quoted against. */
+ZLLM_API int zllm_attn_stream_read_probe(const void* src, uint64_t bytes, uint32_t* sink, zllm_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * KV snapshot wire format of one MLA layer (host side, no device access).     *
  * ------------------------------------------------------------------------- */

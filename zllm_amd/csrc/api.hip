@@ -409,6 +409,17 @@ int zllm_attn_scatter_rows(const zllm_scatter_args* a, zllm_stream_t stream)
     return hip_status(zllm::launch_scatter_rows(p, (hipStream_t)stream), "scatter rows launch");
 }
 
+int zllm_attn_stream_read_probe(const void* src, uint64_t bytes, uint32_t* sink, zllm_stream_t stream)
+{
+    if (src == nullptr || sink == nullptr) {
+        return fail(-1, "stream read probe: null pointer");
+    }
+    if ((uintptr_t)src % 16 != 0 || bytes % 16 != 0) {
+        return fail(-1, "stream read probe: source and size must be multiples of 16 bytes");
+    }
+    return hip_status(zllm::launch_stream_read(src, bytes, sink, (hipStream_t)stream), "stream read probe launch");
+}
+
 /* ---- KV snapshot wire format (host) ----------------------------------------------------- */
 
 static bool mla_record_shape_ok(const zllm_mla_layer_record* r)

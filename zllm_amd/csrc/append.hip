@@ -335,6 +335,38 @@ hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
+// Measurement aid: streams `n_vec` 16-byte vectors once with plain wide loads and keeps nothing.  The rate it reaches
+// on a buffer of a decode call's KV bytes is the ceiling any kernel that has to read those bytes once can reach.
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, unsigned long long n_vec, unsigned int* sink)
+{
+    const unsigned long long stride = (unsigned long long)gridDim.x * 256u;
+    unsigned long long i = (unsigned long long)blockIdx.x * 256u + threadIdx.x;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (; i + 3u * stride < n_vec; i += 4u * stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            v[u] = __builtin_nontemporal_load(src + i + u * stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            acc ^= v[u];
+        }
+    }
+    for (; i < n_vec; i += stride) {
+        acc ^= __builtin_nontemporal_load(src + i);
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a17c0deu && sink[0] == 0xffffffffu) { // keeps the loads alive; practically never true
+        sink[0] = 0u;
+    }
+}
+
+hipError_t launch_stream_read(const void* src, unsigned long long bytes, unsigned int* sink, hipStream_t stream)
+{
+    stream_read_kernel<<<dim3(2048), dim3(256), 0, stream>>>((const u32x4*)src, bytes / 16u, sink);
+    return hipGetLastError();
+}
+
 hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream)
 {
     if (p.count == 0 || p.row_bytes == 0) {
