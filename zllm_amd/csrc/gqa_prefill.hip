@@ -213,7 +213,10 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             dst[st_token] = s0 * fold;
             dst[kStep + st_token] = s1 * fold;
         }
-        // largest scale of the wave's eight tokens (a row of sixteen lanes holds two)
+        if (!stage_v) {
+            return;
+        }
+        // largest V scale of the wave's eight tokens (a row of sixteen lanes holds two)
         float top = fmaxf(s0, s1);
         top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x128, 0xf, 0xf, false))); // row_ror:8
         const float rows01 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
@@ -340,7 +343,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             }
             // the query's power of two is positive, so maxima are taken first and it rides in the multiply-add
             const float mult = SOFTCAP ? 1.0f : q_fac;
-            const float lane_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            float lane_max = sc[0]; // a chain, so that two comparisons share one instruction
+#pragma unroll
+            for (int e = 1; e < 8; ++e) {
+                lane_max = fmaxf(lane_max, sc[e]);
+            }
             const float step_max = wave_max_16x4(lane_max) * mult;
             const float new_max = fmaxf(run_max[ct], step_max);
             const float safe_max = new_max == kNegInf ? 0.0f : new_max;
@@ -354,7 +361,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             }
             run_sum[ct] = run_sum[ct] * alpha + step_sum;
             run_max[ct] = new_max;
-            const float p_top = __builtin_amdgcn_exp2f(fmaf(lane_max, mult, shift)); // the lane's largest probability
+            float p_top = pr[ct][0]; // the lane's largest probability
+#pragma unroll
+            for (int e = 1; e < 8; ++e) {
+                p_top = fmaxf(p_top, pr[ct][e]);
+            }
             heavy = heavy || p_top * kLoThreshold > run_sum[ct];
             if (__any(alpha != 1.0f)) { // the running max settles early in a long prefix
 #pragma unroll
