@@ -243,15 +243,27 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         }
     }
     float run_max[kColTiles], run_sum[kColTiles];
+    float ref_shift[kColTiles]; // what is added to a scaled score before exp2: bias - V window - running maximum
     unsigned int vis_lo[kColTiles], vis_hi[kColTiles]; // visible tokens [lo, hi) of each column's row
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ++ct) {
         run_max[ct] = kNegInf;
         run_sum[ct] = 0.0f;
+        ref_shift[ct] = kPBias;
         const unsigned int pos = p.position + col_row[ct];
         vis_hi[ct] = col_valid[ct] ? pos + 1u : 0u;
         vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
     }
+
+    // first token some column of the wave cannot see any more / last token some column does not see yet (wave-uniform)
+    unsigned int wave_min_hi = min(vis_hi[0], vis_hi[1]), wave_max_lo = max(vis_lo[0], vis_lo[1]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wave_min_hi = min(wave_min_hi, (unsigned int)__shfl_xor((int)wave_min_hi, off));
+        wave_max_lo = max(wave_max_lo, (unsigned int)__shfl_xor((int)wave_max_lo, off));
+    }
+    wave_min_hi = __builtin_amdgcn_readfirstlane(wave_min_hi);
+    wave_max_lo = __builtin_amdgcn_readfirstlane(wave_max_lo);
 
     // chunk = g * 8 + half * 4 + j: the low three bits meet row bits 1, 2; the group bit meets the row's parity
     const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ (m & 6u)) << 4), m * kRowBytes + (((4u | j) ^ (m & 6u)) << 4)};
@@ -324,8 +336,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ++ct) {
             float sc[8];
-            // only steps that touch a causal or window edge of some column need the per-token masks
-            const bool edge = __any(t0 + kStep > vis_hi[ct] || t0 < vis_lo[ct]);
+            // only steps that touch a causal or window edge of some column of the wave need the per-token masks
+            const bool edge = t0 + kStep > wave_min_hi || t0 < wave_max_lo;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 float x = s[e >> 2][ct][e & 3];
@@ -348,35 +360,37 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             for (int e = 1; e < 8; ++e) {
                 lane_max = fmaxf(lane_max, sc[e]);
             }
-            const float step_max = wave_max_16x4(lane_max) * mult;
-            const float new_max = fmaxf(run_max[ct], step_max);
-            const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-            const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max) * acc_fix;
-            const float shift = v_shift - safe_max;
+            // The reference point of the column (running maximum, V window) moves on few steps of a long prefix, so the
+            // reduction across the wave's rows and the rescaling sit behind a test of the lane's own maximum.
+            if (__any(lane_max * mult > run_max[ct]) || acc_fix != 1.0f) {
+                const float step_max = wave_max_16x4(lane_max) * mult;
+                const float new_max = fmaxf(run_max[ct], step_max);
+                const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+                const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max) * acc_fix;
+                ref_shift[ct] = v_shift - safe_max;
+                run_sum[ct] *= alpha;
+                run_max[ct] = new_max;
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        acc[ct][t] *= alpha;
+                    }
+                }
+            }
+            const float shift = ref_shift[ct];
             float step_sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 pr[ct][e] = __builtin_amdgcn_exp2f(fmaf(sc[e], mult, shift));
                 step_sum += pr[ct][e];
             }
-            run_sum[ct] = run_sum[ct] * alpha + step_sum;
-            run_max[ct] = new_max;
-            float p_top = pr[ct][0]; // the lane's largest probability
-#pragma unroll
-            for (int e = 1; e < 8; ++e) {
-                p_top = fmaxf(p_top, pr[ct][e]);
-            }
-            heavy = heavy || p_top * kLoThreshold > run_sum[ct];
-            if (__any(alpha != 1.0f)) { // the running max settles early in a long prefix
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    acc[ct][t] *= alpha;
-                }
-            }
+            run_sum[ct] += step_sum;
+            // the lane's eight probabilities together bound its largest one
+            heavy = heavy || step_sum * kLoThreshold > run_sum[ct];
         }
         // ---- O^T += Vcodes^T . P'_g ----------------------------------------------------------------------
-        // P' is carried as f16 hi + lo (22 significant bits) while any probability of the step weighs more
-        // than 1/8 of its lane's running sum (a lane sums a quarter of the tokens, so < 1/32 of the row's);
+        // P' is carried as f16 hi + lo (22 significant bits) while the probabilities a lane holds of this step weigh more
+        // than 1/8 of its running sum (a lane sums a quarter of the tokens, so each is < 1/32 of the row's sum);
         // below that the hi term's rounding (2^-12 relative, random sign) moves the normalised output by
         // < 2^-12 / 32 of |v|, so the lo product is skipped.
         const bool lo_pass = __any(heavy);
@@ -434,9 +448,10 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     store_step(regs, 0);
     __syncthreads();
     unsigned int wv = 2u; // (biased) exponent of the largest V scale up to the tile being attended
-    for (unsigned int step = 0; step < steps; ++step) {
+    // `buf` is a literal at every call, so the LDS addresses of a step differ from the other buffer's only in the
+    // instructions' immediate offsets and cost no address arithmetic
+    auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
         const unsigned int t0 = t_begin + step * kStep;
-        const int buf = (int)(step & 1u);
         // rows past the end of the visible range repeat its last one: the loads stay inside the sequence's pages
         load_step(regs, t0 + kStep, entry_next);
         entry_next = entry_of(t0 + 2u * kStep + st_token);
@@ -446,12 +461,27 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         compute_step(buf, t0, kPBias + (float)(127 - (int)wv), acc_fix);
         store_step(regs, buf ^ 1);
         __syncthreads();
+    };
+    unsigned int step = 0;
+    for (; step + 1 < steps; step += 2) {
+        one_step(step, 0);
+        one_step(step + 1u, 1);
+    }
+    if (step < steps) {
+        one_step(step, 0);
     }
 
     // ---- normalise and store ------------------------------------------------------------------------
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ++ct) {
         const float total = wave_sum_16x4(run_sum[ct]);
+        {
+            // recomputed rather than kept: these would sit in registers through the whole main loop
+            const unsigned int col = wave * (16u * kColTiles) + ct * 16u + m;
+            col_row[ct] = row0 + col / p.group;
+            col_head[ct] = kvh * p.group + col % p.group;
+            col_valid[ct] = col < cols_used && col_row[ct] < p.rows;
+        }
         if (!col_valid[ct]) {
             continue;
         }
