@@ -277,8 +277,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     }
 
     // `v_shift` = 8 - (V window exponent) is added to every score before exp2; `acc_fix` is 2^-(growth of that
-    // window since the last step), 1 almost always.
-    auto compute_step = [&](int buf, unsigned int t0, float v_shift, float acc_fix) __attribute__((always_inline)) {
+    // window since the last step): 1 unless `window_moved`.
+    auto compute_step = [&](int buf, unsigned int t0, float v_shift, float acc_fix, bool window_moved) __attribute__((always_inline)) {
         const unsigned char* kt = lds_k[buf];
         // ---- S^T = sum_g k_scale_g * (Kcodes_g . Q'_g) ------------------------------------------
         f32x4 s[2][kColTiles];
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             }
             // The reference point of the column (running maximum, V window) moves on few steps of a long prefix, so the
             // reduction across the wave's rows and the rescaling sit behind a test of the lane's own maximum.
-            if (__any(lane_max * mult > run_max[ct]) || acc_fix != 1.0f) {
+            if (__any(lane_max * mult > run_max[ct]) || window_moved) {
                 const float step_max = wave_max_16x4(lane_max) * mult;
                 const float new_max = fmaxf(run_max[ct], step_max);
                 const float safe_max = new_max == kNegInf ? 0.0f : new_max;
@@ -448,6 +448,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     store_step(regs, 0);
     __syncthreads();
     unsigned int wv = 2u; // (biased) exponent of the largest V scale up to the tile being attended
+    float v_shift = kPBias + 125.0f;
     // `buf` is a literal at every call, so the LDS addresses of a step differ from the other buffer's only in the
     // instructions' immediate offsets and cost no address arithmetic
     auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
@@ -456,9 +457,14 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         load_step(regs, t0 + kStep, entry_next);
         entry_next = entry_of(t0 + 2u * kStep + st_token);
         const unsigned int wv_now = window_of(buf, wv);
-        const float acc_fix = wv_now != wv ? ldexpf(1.0f, (int)wv - (int)wv_now) : 1.0f;
-        wv = wv_now;
-        compute_step(buf, t0, kPBias + (float)(127 - (int)wv), acc_fix);
+        const bool window_moved = wv_now != wv; // rare: a V scale above everything met so far
+        float acc_fix = 1.0f;
+        if (window_moved) {
+            acc_fix = ldexpf(1.0f, (int)wv - (int)wv_now);
+            wv = wv_now;
+            v_shift = kPBias + (float)(127 - (int)wv);
+        }
+        compute_step(buf, t0, v_shift, acc_fix, window_moved);
         store_step(regs, buf ^ 1);
         __syncthreads();
     };
