@@ -451,6 +451,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
             }
         }
         float run_max = kNegInf, run_sum = 0.0f;
+        float neg_ref = 0.0f; // minus the reference the scores are taken against: the running maximum, 0 before the first score
         const float scale_log2 = p.score_scale * kLog2e;
         const float latent_log2 = scale_log2 * head_pow2;
         stage_step(1u);
@@ -529,7 +530,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                     if (q == 3) {
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            sc[t2 * 4 + r] = fmaf(s[r], latent_log2, s_rope[r] * scale_log2);
+                            sc[t2 * 4 + r] = fmaf(s[r], latent_log2, fmaf(s_rope[r], scale_log2, neg_ref)); // relative to the reference
                         }
                     }
                 }
@@ -540,30 +541,43 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
                         sc[e] = token < len ? sc[e] : kNegInf;
                     }
                 }
-                // online softmax for this head column; lazy rescaling: the stored maximum only moves when a
-                // score exceeds it by 2^8 (p stays <= 256)
-                float step_max = sc[0];
+                // Online softmax for this head column with lazy rescaling: the stored maximum (the reference the scores
+                // above are already relative to) only moves when a score exceeds it by 2^8 (p stays <= 256).  On most
+                // steps no lane sees such a score, and the reduction across the wave's rows, the new reference and the
+                // rescaling factor are skipped altogether.
+                float lane_max = sc[0];
 #pragma unroll
                 for (int e = 1; e < 8; ++e) {
-                    step_max = fmaxf(step_max, sc[e]);
+                    lane_max = fmaxf(lane_max, sc[e]);
                 }
-                step_max = wave_max_16x4(step_max);
-                float new_max = run_max;
-                if (step_max > run_max + 8.0f || run_max == kNegInf) {
-                    new_max = fmaxf(run_max, step_max);
+                float alpha = 1.0f;
+                if (__any(lane_max > 8.0f || run_max == kNegInf)) {
+                    const float step_max = wave_max_16x4(lane_max); // relative as well
+                    const float ref = -neg_ref;
+                    float new_max = run_max;
+                    if (step_max > 8.0f || run_max == kNegInf) {
+                        new_max = fmaxf(run_max, ref + step_max);
+                    }
+                    const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+                    alpha = __builtin_amdgcn_exp2f(run_max - safe_max); // 0 on the first step: nothing accumulated yet
+                    const float delta = safe_max - ref;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        sc[e] -= delta;
+                    }
+                    run_max = new_max;
+                    neg_ref = -safe_max;
+                    run_sum *= alpha;
                 }
-                const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-                const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max); // 0 on the first step: nothing accumulated yet
                 f32x4 p_lo, p_hi;
                 float step_sum = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    p_lo[e] = __builtin_amdgcn_exp2f(sc[e] - safe_max);
-                    p_hi[e] = __builtin_amdgcn_exp2f(sc[4 + e] - safe_max);
+                    p_lo[e] = __builtin_amdgcn_exp2f(sc[e]);
+                    p_hi[e] = __builtin_amdgcn_exp2f(sc[4 + e]);
                     step_sum += p_lo[e] + p_hi[e];
                 }
-                run_sum = run_sum * alpha + step_sum;
-                run_max = new_max;
+                run_sum += step_sum;
                 *(f32x4*)lds_p[i & 1u][hw][0][lane] = p_lo;
                 *(f32x4*)lds_p[i & 1u][hw][1][lane] = p_hi;
                 lds_alpha[i & 1u][hw][lane] = alpha;
