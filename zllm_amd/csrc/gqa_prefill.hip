@@ -266,14 +266,25 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     wave_max_lo = __builtin_amdgcn_readfirstlane(wave_max_lo);
 
     // chunk = g * 8 + half * 4 + j: the low three bits meet row bits 1, 2; the group bit meets the row's parity
-    const unsigned int qk_base[2] = {m * kRowBytes + ((j ^ (m & 6u)) << 4), m * kRowBytes + (((4u | j) ^ (m & 6u)) << 4)};
-    const unsigned int qk_group[2] = {(m & 1u) * 128u, 128u - (m & 1u) * 128u};
+    // The byte offsets inside a tile are kept as finished sums, one register per (group, half) or (group, quarter):
+    // formed from their parts inside the loop they cost an addition per LDS read.  The inline assembly hides the
+    // parts from the optimizer, which would otherwise split the sums again to save the registers.
+    unsigned int qk_at[2][2], pv_at[2][4];
     const unsigned int tr_row = 4u * j + (m >> 2);
-    unsigned int pv_base[4];
-    const unsigned int pv_group[2] = {(tr_row & 1u) * 128u, 128u - (tr_row & 1u) * 128u};
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        pv_base[q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ (tr_row & 6u)) << 4) + (m & 1u) * 8u;
+    for (int g = 0; g < 2; ++g) {
+        const unsigned int qk_group = g == 0 ? (m & 1u) * 128u : 128u - (m & 1u) * 128u;
+        const unsigned int pv_group = g == 0 ? (tr_row & 1u) * 128u : 128u - (tr_row & 1u) * 128u;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            qk_at[g][h] = m * kRowBytes + ((((unsigned int)h << 2 | j) ^ (m & 6u)) << 4) + qk_group;
+            asm volatile("" : "+v"(qk_at[g][h]));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            pv_at[g][q] = tr_row * kRowBytes + ((((unsigned int)q << 1 | ((m & 3u) >> 1)) ^ (tr_row & 6u)) << 4) + (m & 1u) * 8u + pv_group;
+            asm volatile("" : "+v"(pv_at[g][q]));
+        }
     }
 
     // `v_shift` = 8 - (V window exponent) is added to every score before exp2; `acc_fix` is 2^-(growth of that
@@ -291,8 +302,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
                 Frag k0, k1;
-                k0.u = *(const u32x4*)(kt + qk_base[0] + qk_group[g] + i * 16 * kRowBytes);
-                k1.u = *(const u32x4*)(kt + qk_base[1] + qk_group[g] + i * 16 * kRowBytes);
+                k0.u = *(const u32x4*)(kt + qk_at[g][0] + i * 16 * kRowBytes);
+                k1.u = *(const u32x4*)(kt + qk_at[g][1] + i * 16 * kRowBytes);
                 const f32x4 gs = *(const f32x4*)(&lds_ks[buf][g][i * 16 + 4 * j]);
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
@@ -316,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         auto load_vfrags = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt) {
-                const unsigned char* at = vt + pv_base[tt] + pv_group[g];
+                const unsigned char* at = vt + pv_at[g][tt];
                 vf[tt].s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
                 vf[tt].s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
             }
