@@ -437,6 +437,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
                     for (int e = 0; e < 4; ++e) {
                         const float x0 = pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]);
                         const float x1 = pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]);
+                        // formed again rather than read back from phi: a bit cast of a vector element (phi[ct].u[e]) picked
+                        // element 0 for every e with this compiler
                         const f16x2 hi = __builtin_bit_cast(f16x2, pack_f16_hw(x0, x1));
                         plo[ct].u[e] = pack_f16_hw(x0 - (float)hi[0], x1 - (float)hi[1]);
                     }
