@@ -16,10 +16,14 @@
 // up to 2^-11 of their largest term, which outlier channels turn into output errors above the 2e-3 bound.
 // Q' is the wave's query tile times one power of two (largest magnitude in [2^8, 2^9)), undone in the fused
 // multiply-add that feeds exp2.  P' must stay inside f16 range for any scale a cache can hold: the exponent of
-// the largest V scale met so far (reduced by wave 0 one step ahead of the tile) is subtracted from the softmax
+// the largest V scale met so far (each V staging wave reduces the scales it converts) is subtracted from the softmax
 // reference, so accumulators and running sum carry the same power of two and it cancels in the division.
 // K is read from LDS with ds_read_b128, V transposed with ds_read_b64_tr_b16; a 16-byte XOR swizzle
 // keeps both conflict-free.
+// The kernel is bound by the vector-ALU instructions it issues, not by the matrix cores, so whatever does not depend on
+// every (token, column) pair stays out of the common path of a step: the tile buffer is a literal (LDS addresses in
+// immediates), edge masks and the low-order P' pass sit behind wave-uniform branches, and a column's reference
+// (running maximum, V window) is only touched when some lane's score passes it.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -33,7 +37,7 @@ namespace {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kStep = 32;                 // tokens per step
 constexpr int kD = 128;                   // head_dim handled by this kernel
-constexpr int kRowBytes = kD * 2;         // one token of one KV head as bf16
+constexpr int kRowBytes = kD * 2;         // one token of one KV head as f16
 constexpr int kTileBytes = kStep * kRowBytes; // 8 KiB
 constexpr float kPBias = 8.0f;            // probabilities are carried as p * 2^8: f16 stays normal down to p = 2^-22
 constexpr float kLoThreshold = 8.0f;      // see the P.V stage
