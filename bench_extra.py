@@ -270,7 +270,7 @@ def run(args):
     elif args.workload == "gqa_decode_f16_window":
         run_gqa_decode_f16(args)
     elif args.workload == "gqa_prefill_chunk":
-        from zllm_amd import bench_prefill
+        import bench_prefill
 
         bench_prefill.run(args)
     else:

@@ -10,7 +10,7 @@ import time
 
 import numpy as np
 
-from .bench_extra import MFMA_BF16_PEAK_TFLOPS, _event_ms, _wall_ms
+from bench_extra import MFMA_BF16_PEAK_TFLOPS, _event_ms, _wall_ms
 
 
 def run(args):

@@ -1,0 +1,108 @@
+// Measurement aids for bench.py: plain read kernels that keep nothing.  They are not part of the attention library
+// (own shared object, libbench_probe.so) and exist to say what "every KV byte read once" can reach on the device.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Streams n_vec 16-byte vectors once, grid-strided, four non-temporal loads in flight per lane.
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, unsigned long long n_vec, unsigned int* sink)
+{
+    const unsigned long long stride = (unsigned long long)gridDim.x * 256u;
+    unsigned long long i = (unsigned long long)blockIdx.x * 256u + threadIdx.x;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (; i + 3u * stride < n_vec; i += 4u * stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            v[u] = __builtin_nontemporal_load(src + i + u * stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            acc ^= v[u];
+        }
+    }
+    for (; i < n_vec; i += stride) {
+        acc ^= __builtin_nontemporal_load(src + i);
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a17c0deu && sink[0] == 0xffffffffu) { // keeps the loads alive; practically never true
+        sink[0] = 0u;
+    }
+}
+
+// The decode kernel's own access pattern without its arithmetic: a workgroup of eight waves walks a run of pages of
+// two code planes (K and V, 16 rows of 1,024 bytes per page, pages scattered through `table`) and their two scale
+// planes (16 rows of 32 bytes).  Wave w reads bytes [128 w, 128 w + 128) of every row -- eight neighbouring lanes
+// fetch one whole 128-byte line with a 16-byte non-temporal load each, eight rows per instruction -- so the eight
+// waves together read whole rows, exactly as the eight KV-head waves of the decode kernel do.  Eight code loads and
+// one scale load are in flight per lane per page.
+__global__ __launch_bounds__(512) void paged_read_kernel(const unsigned char* k_plane, const unsigned char* v_plane,
+                                                         const unsigned char* k_scales, const unsigned char* v_scales,
+                                                         const unsigned int* table, unsigned int pages, unsigned int pages_per_group,
+                                                         unsigned int* sink)
+{
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int wave = threadIdx.x >> 6;
+    const unsigned int first = blockIdx.x * pages_per_group;
+    const unsigned int last = min(first + pages_per_group, pages);
+    const unsigned int lane_off = (lane >> 3) * 1024u + wave * 128u + (lane & 7u) * 16u;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    unsigned int acc_s = 0u;
+    for (unsigned int p = first; p < last; p += 2u) {
+        u32x4 v[2][4];
+        unsigned int s[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const unsigned int page = table[min(p + u, last - 1u)];
+            const unsigned long long base = (unsigned long long)page * 16384u;
+            v[u][0] = __builtin_nontemporal_load((const u32x4*)(k_plane + base + lane_off));
+            v[u][1] = __builtin_nontemporal_load((const u32x4*)(k_plane + base + 8192u + lane_off));
+            v[u][2] = __builtin_nontemporal_load((const u32x4*)(v_plane + base + lane_off));
+            v[u][3] = __builtin_nontemporal_load((const u32x4*)(v_plane + base + 8192u + lane_off));
+            // scale rows: 16 tokens x 32 bytes per plane and page; wave w takes its 4 bytes of each row
+            const unsigned char* sp = (lane >= 32u ? v_scales : k_scales) + (unsigned long long)page * 512u + (lane & 15u) * 32u + wave * 4u;
+            s[u] = *(const unsigned int*)sp;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                acc ^= v[u][w];
+            }
+            acc_s ^= s[u];
+        }
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3] ^ acc_s) == 0x5a17c0deu && sink[0] == 0xffffffffu) {
+        sink[0] = 0u;
+    }
+}
+
+extern "C" {
+
+__attribute__((visibility("default"))) int bench_probe_stream_read(const void* src, uint64_t bytes, uint32_t* sink, void* stream)
+{
+    if (src == nullptr || sink == nullptr || (uintptr_t)src % 16 != 0 || bytes % 16 != 0) {
+        return -1;
+    }
+    stream_read_kernel<<<dim3(2048), dim3(256), 0, (hipStream_t)stream>>>((const u32x4*)src, bytes / 16u, sink);
+    return (int)hipGetLastError();
+}
+
+// `pages` entries of `table` name 16-row pages of planes whose rows are 1,024 bytes (codes) and 32 bytes (scales).
+__attribute__((visibility("default"))) int bench_probe_paged_read(const void* k_plane, const void* v_plane, const void* k_scales,
+                                                                  const void* v_scales, const uint32_t* table, uint32_t pages,
+                                                                  uint32_t workgroups, uint32_t* sink, void* stream)
+{
+    if (k_plane == nullptr || v_plane == nullptr || k_scales == nullptr || v_scales == nullptr || table == nullptr || sink == nullptr ||
+        pages == 0 || workgroups == 0) {
+        return -1;
+    }
+    const uint32_t per_group = (pages + workgroups - 1) / workgroups;
+    const uint32_t groups = (pages + per_group - 1) / per_group;
+    paged_read_kernel<<<dim3(groups), dim3(512), 0, (hipStream_t)stream>>>((const unsigned char*)k_plane, (const unsigned char*)v_plane,
+                                                                             (const unsigned char*)k_scales, (const unsigned char*)v_scales,
+                                                                             table, pages, per_group, sink);
+    return (int)hipGetLastError();
+}
+
+} // extern "C"

@@ -190,13 +190,6 @@ typedef struct zllm_scatter_args {
 } zllm_scatter_args;
 ZLLM_API int zllm_attn_scatter_rows(const zllm_scatter_args* args, zllm_stream_t stream);
 
-/* Measurement aid with no counterpart in the reference: reads `bytes` (a multiple of 16, 16-byte aligned)
- * of device memory once with plain wide loads and keeps nothing (`sink`: one device word the kernel
- * never changes in practice).  bench.py times it over a buffer of the decode workload's KV bytes: the
- * rate it reaches is what "every KV byte read once" can reach on the device at that size, next to the
- * published HBM peak the roofline fraction is quoted against. */
-ZLLM_API int zllm_attn_stream_read_probe(const void* src, uint64_t bytes, uint32_t* sink, zllm_stream_t stream);
-
 /* ------------------------------------------------------------------------- *
  * KV snapshot wire format of one MLA layer (host side, no device access).     *
  * ------------------------------------------------------------------------- */
@@ -255,7 +248,9 @@ typedef struct zllm_gqa_decode_args {
     uint32_t batch;
     uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 256} */
     uint32_t table_stride;         /* entries per sequence in `tables` */
-    uint32_t max_kv_len;           /* host upper bound of kv_lens (sizes the grid) */
+    uint32_t max_kv_len;           /* host upper bound of kv_lens: sizes the grid and the split plan.  A call
+                                      recorded into a HIP graph stays valid only while every kv_lens[b] on the
+                                      device is <= max_kv_len; tokens past the planned splits are not read */
     uint32_t total_kv_tokens;      /* optional host hint: sum of the visible lengths (0 = unknown,
                                       batch * max_kv_len is assumed); only tunes the split size */
     uint32_t block_tokens;
@@ -391,7 +386,10 @@ typedef struct zllm_mla_decode_args {
     uint32_t kv_head_dim;         /* nope + value */
     uint32_t latent_dim;          /* 512 */
     uint32_t rope_dim;            /* 64 */
-    uint32_t table_stride, max_ctx_len, block_tokens;
+    uint32_t table_stride;
+    uint32_t max_ctx_len;         /* host upper bound of ctx_lens (split plan); a recorded graph stays valid
+                                     only while every ctx_lens[b] <= max_ctx_len */
+    uint32_t block_tokens;
     int q_dtype;                  /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
     int out_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
     int out_compact;

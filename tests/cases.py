@@ -45,13 +45,16 @@ def draw_tables(rng, lens, block_tokens, pool_blocks=None, layout="random"):
 
 
 def make_gqa_q8_case(seed, lens, hq, hkv, d, block_tokens=16, rule=O.RULE_METAL_GQA, outliers=False, layout="random",
-                     q_bf16=False, pool_blocks=None, q_std=1.0, k_gain=1.0, v_gain=1.0):
+                     q_bf16=False, pool_blocks=None, q_std=1.0, k_gain=1.0, v_gain=1.0, poison=False, ring_capacity=0):
     """K/V ~ N(0,1) (optionally 1 % outlier channels x8), quantized Q8g64 by the oracle into a paged pool.
-    k_gain / v_gain: one factor, or one per token of the longest sequence (magnitude tests)."""
+    k_gain / v_gain: one factor, or one per token of the longest sequence (magnitude tests).
+    poison: rows no sequence wrote hold NaN scale bits and the code -128 (a pool that was never cleared).
+    ring_capacity: sliding-window storage, token t lives in slot t % ring_capacity of the sequence's pages."""
     rng = np.random.default_rng(seed)
     lens = [int(l) for l in lens]
     cols = hkv * d
-    tables, pool_blocks = draw_tables(rng, lens, block_tokens, pool_blocks, layout)
+    stored = [min(l, ring_capacity) if ring_capacity else l for l in lens]
+    tables, pool_blocks = draw_tables(rng, stored, block_tokens, pool_blocks, layout)
     rows = pool_blocks * block_tokens
     sdt = {O.RULE_ROCM_MLA: O.SCALE_BF16, O.RULE_METAL_GQA: O.SCALE_F16, O.RULE_CUDA_GQA: O.SCALE_F32}[rule]
     scale_np = np.float32 if sdt == O.SCALE_F32 else np.uint16
@@ -61,6 +64,11 @@ def make_gqa_q8_case(seed, lens, hq, hkv, d, block_tokens=16, rule=O.RULE_METAL_
         "v_codes": np.zeros((rows, cols), dtype=np.int8),
         "v_scales": np.zeros((rows, cols // 64), dtype=scale_np),
     }
+    if poison:
+        for name in ("k_codes", "v_codes"):
+            planes[name][:] = -128
+        for name in ("k_scales", "v_scales"):
+            planes[name][:] = np.nan if sdt == O.SCALE_F32 else (0x7FC0 if sdt == O.SCALE_BF16 else 0x7E00)
     raw_k, raw_v = [], []
     channel_gain = np.ones(cols, dtype=np.float32)
     if outliers:
@@ -74,8 +82,8 @@ def make_gqa_q8_case(seed, lens, hq, hkv, d, block_tokens=16, rule=O.RULE_METAL_
         raw_k.append(k)
         raw_v.append(v)
         if length:
-            O.q8g64_append_paged(rule, k, planes["k_codes"], planes["k_scales"], tables[b], 0, block_tokens)
-            O.q8g64_append_paged(rule, v, planes["v_codes"], planes["v_scales"], tables[b], 0, block_tokens)
+            O.q8g64_append_paged(rule, k, planes["k_codes"], planes["k_scales"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
+            O.q8g64_append_paged(rule, v, planes["v_codes"], planes["v_scales"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
     q = (rng.standard_normal((len(lens), hq * d)) * q_std).astype(np.float32)
     q_bits = None
     if q_bf16:

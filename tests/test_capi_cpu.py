@@ -121,8 +121,6 @@ def test_invalid_shapes_are_reported_without_a_gpu(lib):
     assert lib.zllm_attn_mla_decode(C.byref(mla), None) == -1 and b"aligned" in lib.zllm_attn_last_error()
     prologue = capi.GqaPrologueArgs()
     assert lib.zllm_attn_gqa_prologue(C.byref(prologue), None) == -1
-    assert lib.zllm_attn_stream_read_probe(None, 16, None, None) == -1
-    assert lib.zllm_attn_stream_read_probe(0x1008, 16, 0x2000, None) == -1 and b"multiples of 16" in lib.zllm_attn_last_error()
 
 
 def test_cpp_host_layer_builds_and_exports_the_backend_methods():

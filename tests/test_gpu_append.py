@@ -156,17 +156,3 @@ def test_mla_append_bit_exact(layout, rotary_dim):
     assert np.array_equal(codes.cpu().numpy(), ref_codes)
     assert np.array_equal(scales.cpu().numpy().view(np.uint16), ref_scales)
     assert np.array_equal(rope_cache.cpu().numpy().view(np.uint16), ref_rope)
-
-
-def test_stream_read_probe_reads_and_keeps_nothing():
-    """The measurement aid behind bench.py's ceiling figure: runs on any 16-byte multiple and leaves its sink word alone."""
-    from zllm_amd import capi, ops
-
-    sink = torch.full((1,), 7, dtype=torch.int32, device="cuda")
-    for n in (16, 4096 + 16, 3 * (1 << 20)):
-        src = torch.arange(n, dtype=torch.int64, device="cuda").to(torch.uint8)
-        ops.stream_read_probe(src, sink)
-    torch.cuda.synchronize()
-    assert int(sink.item()) == 7
-    with pytest.raises(capi.ZllmAttnError, match="multiples of 16"):
-        ops.stream_read_probe(torch.zeros(40, dtype=torch.uint8, device="cuda"), sink)

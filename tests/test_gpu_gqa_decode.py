@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 
-def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_capacity=0, gate=None):
+def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_capacity=0, gate=None, total_kv_tokens=0):
     from zllm_amd import capi, ops
 
     pl = case["planes"]
@@ -24,7 +24,8 @@ def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_c
     out = ops.gqa_decode(q, upload(pl["k_codes"]), upload(pl["k_scales"]), upload(pl["v_codes"]), upload(pl["v_scales"]),
                          upload(case["tables"]), upload(lens), case["hq"], case["hkv"], case["d"], case["block_tokens"],
                          score_scale, max_kv_len or max(int(lens.max()), 1), first_visible=first, softcap=softcap,
-                         ring_capacity=ring_capacity, kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"], gate=gate)
+                         ring_capacity=ring_capacity, kv_format=capi.KV_Q8G64, scale_dtype=case["scale_dtype"], gate=gate,
+                         total_kv_tokens=total_kv_tokens)
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -189,13 +190,16 @@ def test_large_pool_exercises_64_bit_offsets():
 
 
 # ---------------------------------------------------------------------------- f16 KV (config 3)
-def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0):
+def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0, poison=False):
     rng = np.random.default_rng(seed)
     cols = hkv * d
     cap_lens = [min(l, ring_capacity) if ring_capacity else l for l in lens]
     tables, pool_blocks = draw_tables(rng, cap_lens, block_tokens)
     rows = pool_blocks * block_tokens
     planes = {"k": np.zeros((rows, cols), dtype=np.uint16), "v": np.zeros((rows, cols), dtype=np.uint16)}
+    if poison:  # rows no sequence wrote: f16 NaN
+        planes["k"][:] = 0x7E00
+        planes["v"][:] = 0x7E00
     for b, l in enumerate(lens):
         kg = np.reshape(np.asarray(k_gain, dtype=np.float32), (-1, 1))
         vg = np.reshape(np.asarray(v_gain, dtype=np.float32), (-1, 1))
@@ -327,3 +331,77 @@ def test_f16_kv_magnitudes(exponent):
     print("k", assert_attention_close(run_f16(case, 0.0625 / flat), oracle_gqa_decode(case, 0.0625 / flat, fmt=O.FMT_F16), f"k * 2^{exponent}"))
     case = make_f16_case(513, lens, 16, 8, 256, q_std=flat * flat)
     print("q", assert_attention_close(run_f16(case, 0.0625 / (flat * flat)), oracle_gqa_decode(case, 0.0625 / (flat * flat), fmt=O.FMT_F16), "q"))
+
+
+# ---------------------------------------------------------------------------- pools that were never cleared
+@pytest.mark.parametrize("hq,hkv,d,block_tokens,rule", [(8, 2, 64, 16, O.RULE_METAL_GQA), (16, 4, 128, 16, O.RULE_METAL_GQA),
+                                                       (64, 8, 128, 16, O.RULE_METAL_GQA), (8, 2, 256, 32, O.RULE_ROCM_MLA),
+                                                       (16, 4, 128, 64, O.RULE_ROCM_MLA)])
+@pytest.mark.parametrize("window", [0, 1000])
+def test_q8_rows_outside_the_visible_range_contribute_nothing(hq, hkv, d, block_tokens, rule, window):
+    """The caller owns the pool and need not clear it: the rest of a sequence's last page holds NaN scale bits and the
+    code -128 here.  The fast paths load whole 16-token tiles, so those rows (and, with a window, the rows in front of
+    a first visible token that is not tile-aligned: 2100 - 1000 = 1100 = 68 * 16 + 12) are really read; masked rows
+    must multiply as exact zeros."""
+    lens = [2100, 1, 17, 33, 1023, 4099]
+    case = make_gqa_q8_case(600 + d + block_tokens, lens, hq, hkv, d, block_tokens=block_tokens, rule=rule, poison=True, q_bf16=True)
+    got = run_decode(case, 1.0 / np.sqrt(d), window=window)
+    assert np.isfinite(got).all()
+    assert_attention_close(got, oracle_gqa_decode(case, 1.0 / np.sqrt(d), window=window), f"poisoned pool d={d} window={window}")
+
+
+@pytest.mark.parametrize("d,block_tokens", [(128, 16), (256, 64)])
+@pytest.mark.parametrize("window", [0, 1000])
+def test_f16_rows_outside_the_visible_range_contribute_nothing(d, block_tokens, window):
+    lens = [2100, 1, 17, 33, 1023]
+    case = make_f16_case(700 + d, lens, 16, 8, d, block_tokens=block_tokens, poison=True)
+    got = run_f16(case, 1.0 / np.sqrt(d), window=window)
+    assert np.isfinite(got).all()
+    assert_attention_close(got, oracle_gqa_decode(case, 1.0 / np.sqrt(d), window=window, fmt=O.FMT_F16), f"poisoned f16 pool d={d}")
+
+
+# ---------------------------------------------------------------------------- Q8g64 sliding window stored as a ring
+@pytest.mark.parametrize("d,ring,window,block_tokens", [(128, 1024, 1024, 16), (128, 1000, 1000, 16), (256, 512, 400, 32),
+                                                        (128, 200, 150, 8), (256, 1000, 1000, 16)])
+def test_q8_sliding_window_ring(d, ring, window, block_tokens):
+    """token -> token % capacity before the page lookup (src/kernel/cuda/attention.rs:82-88,108-116): a ring that is a
+    multiple of 16 rows keeps the tile path (per-tile table lookups), any other capacity takes the per-token path; the
+    sequences are longer than the ring, so the visible window wraps."""
+    lens = [3 * ring + 77, ring - 5, ring, 2 * ring + 1]
+    case = make_gqa_q8_case(800 + ring, lens, 16, 4, d, block_tokens=block_tokens, ring_capacity=ring, poison=True)
+    scale = 1.0 / np.sqrt(d)
+    got = run_decode(case, scale, window=window, ring_capacity=ring)
+    want = oracle_gqa_decode(case, scale, window=window, ring_capacity=ring)
+    assert_attention_close(got, want, f"Q8 ring {ring} window {window} d={d}")
+
+
+# ---------------------------------------------------------------------------- the benchmarked shape at its full size
+def _oracle_rows(case, rows, scale):
+    sub = dict(case)
+    sub["lens"] = case["lens"][rows]
+    sub["tables"] = case["tables"][rows]
+    sub["q"] = case["q"][rows]
+    return oracle_gqa_decode(sub, scale)
+
+
+@pytest.mark.parametrize("ragged", [False, True])
+def test_config2_full_size(ragged):
+    """BASELINE config 2 at its own size -- B = 8, 64q/8kv, d = 128, 16-token pages, bf16 queries, outlier channels --
+    every sequence at 32,768 tokens (the kernel instantiation and split plan the bench times) and the ragged draw in
+    [1024, 32768].  The oracle runs on two sequences of the call's output; the zero-query mean is checked on one."""
+    rng = np.random.default_rng(2)
+    lens = [int(x) for x in rng.integers(1024, 32769, size=8)] if ragged else [32768] * 8
+    case = make_gqa_q8_case(2, lens, 64, 8, 128, outliers=True, q_bf16=True)
+    scale = 1.0 / np.sqrt(128.0)
+    got = run_decode(case, scale, total_kv_tokens=sum(lens))  # the bench passes the same hint
+    picks = [0, int(np.argmax(lens)) if ragged else 5]
+    want = _oracle_rows(case, picks, scale)
+    print("config2 full", ragged, assert_attention_close(got[picks], want, f"config 2 full size ragged={ragged}"))
+    case["q"][:] = 0.0
+    case["q_bits"][:] = 0
+    zero = run_decode(case, scale, total_kv_tokens=sum(lens))
+    b = picks[1]
+    v = O.gather_dequant_rows(O.FMT_Q8, case["planes"]["v_codes"], case["planes"]["v_scales"], case["scale_dtype"], case["tables"][b],
+                              16, 0, lens[b], 1024).astype(np.float64)
+    mean = v.reshape(lens[b], 8, 128).mean(0)
+    assert np.abs(zero[b].reshape(64, 128) - np.repeat(mean, 8, axis=0)).max() < 1e-4

@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
-             out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0):
+             out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0, oracle_segments=None):
     from zllm_amd import capi, ops
 
     d = 128
@@ -63,6 +63,16 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     torch.cuda.synchronize()
     kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, tables[0], block_tokens, 0, total, cols)
     vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, tables[0], block_tokens, 0, total, cols)
+    if oracle_segments is not None:
+        # the oracle on a few runs of chunk rows only (a full-size chunk is hours of scalar work): rows [r0, r0 + n) are a
+        # chunk of their own appended at prefix + r0; key_range caps every row at its own position
+        parts = []
+        for r0, n in oracle_segments:
+            rc, part = O.gqa_prefill_at_visible(q[r0:r0 + n], kd, vd, 0, total, prefix + r0, hq, hkv, d, window=window, score_scale=scale,
+                                                softcap=softcap)
+            assert rc == 0
+            parts.append(part)
+        return out, np.concatenate(parts)
     rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
     assert rc == 0
     if gate is not None:
@@ -168,3 +178,13 @@ def test_prefill_rejects_unsupported_shapes():
     q = torch.zeros((1, 64), dtype=torch.float32, device="cuda")
     with pytest.raises(capi.ZllmAttnError, match="head_dim 128"):
         ops.gqa_prefill_chunk(q, z, s, z, s, None, 0, 1, 1, 64, 16, 1.0)
+
+
+def test_prefill_config5_full_size():
+    """BASELINE config 5 at its own size: a 2,048-row chunk on a 50,000-token prefix, 64q/8kv, d = 128, bf16 activations,
+    16-token pages, the chunk quantized into fresh pages by the library.  The oracle runs on the first, a middle and the
+    last eight chunk rows of the full call's output."""
+    segments = [(0, 8), (1020, 8), (2040, 8)]
+    out, want = run_case(5, 50000, 2048, 64, 8, oracle_segments=segments)
+    got = np.concatenate([out[r0:r0 + n].cpu().numpy() for r0, n in segments])
+    print("config5 full", assert_attention_close(got, want, "config 5 full size"))

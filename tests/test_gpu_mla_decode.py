@@ -314,3 +314,37 @@ def test_mla_layer_snapshot_round_trip_and_rollback():
     assert np.array_equal(live["codes"], ref["codes"]) and np.array_equal(live["scales"], ref["scales"])
     got = run_mla(live).cpu().numpy()
     assert_attention_close(got, want_f, "rollback + append")
+
+
+def _oracle_mla_heads(case, b, heads_picked):
+    """The oracle on a few heads of one sequence: heads are independent, so slicing the query and kv_b rows of those heads
+    gives exactly what the full call computes for them."""
+    qd, kd = case["nope"] + case["rope_dim"], case["nope"] + case["value"]
+    q = case["q_bits"][b].reshape(case["heads"], qd)[heads_picked].reshape(1, -1)
+    w = case["kv_b_bits"].reshape(case["heads"], kd, case["latent"])[heads_picked].reshape(-1, case["latent"])
+    n = len(heads_picked)
+    sub = dict(case, q_bits=q, kv_b_bits=w, lens=case["lens"][b:b + 1], tables=case["tables"][b:b + 1], heads=n,
+               spec=O.MlaSpec(case["latent"], case["rope_dim"], n * qd, n * kd, n))
+    want_f, want_b = oracle_mla(sub)
+    return want_f[0].reshape(n, case["value"])
+
+
+@pytest.mark.parametrize("block_tokens", [64, 16])
+def test_config4_full_size(block_tokens):
+    """BASELINE config 4 at its own size: B = 4, 128 heads, 65,536 tokens, with the reference's 64-token pages (the
+    instantiation the bench times: whole 32-row steps from one page) and with 16-token pages (per-row table lookups).
+    The oracle runs on heads 0, 63, 64, 127 -- both 64-head blocks of a workgroup pair, first and last column -- of two
+    sequences sliced out of the full call's output; a zero query at full length must give the projected mean latent."""
+    ctx = 65536
+    case = make_mla_case(4, [ctx, ctx, ctx - 37, ctx], 128, block_tokens=block_tokens)
+    got = run_mla(case).cpu().numpy().reshape(4, 128, 128)
+    picks = [0, 63, 64, 127]
+    for b in (1, 2):
+        want = _oracle_mla_heads(case, b, picks)
+        print("config4 full", block_tokens, b, assert_attention_close(got[b][picks], want, f"config 4 full size, sequence {b}"))
+    case["q_bits"][:] = 0
+    zero = run_mla(case).cpu().numpy().reshape(4, 128, 128)
+    lat = O.gather_dequant_rows(O.FMT_Q8, case["codes"], case["scales"], O.SCALE_BF16, case["tables"][2], block_tokens, 0, ctx - 37, 512)
+    w = O.bf16_to_f32(case["kv_b_bits"]).reshape(128, 256, 512)[:, 128:, :]
+    want = np.einsum("hvc,c->hv", w.astype(np.float64), lat.astype(np.float64).mean(0))
+    assert np.abs(zero[2] - want).max() < 2e-3

@@ -66,6 +66,17 @@ def build_host_test(oracle_dir: str) -> str:
     return HOST_TEST
 
 
+BENCH_PROBE = os.path.join(os.path.dirname(HERE), "libbench_probe.so")
+
+
+def build_bench_probe() -> str:
+    """bench.py's plain-read measurement kernels (bench_probe.hip beside bench.py); not part of the attention library."""
+    cmd = [HIPCC, *FLAGS, "-shared", "-o", BENCH_PROBE, os.path.join(os.path.dirname(HERE), "bench_probe.hip")]
+    subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
+    return BENCH_PROBE
+
+
 if __name__ == "__main__":
     print(build_library())
     print(build_host_layer())
+    print(build_bench_probe())

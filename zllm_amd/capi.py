@@ -107,7 +107,6 @@ SYMBOLS = {
     "zllm_attn_mla_append": (_int, [C.POINTER(MlaAppendArgs), _ptr]),
     "zllm_attn_gather_rows": (_int, [C.POINTER(GatherArgs), _ptr]),
     "zllm_attn_scatter_rows": (_int, [C.POINTER(ScatterArgs), _ptr]),
-    "zllm_attn_stream_read_probe": (_int, [_ptr, _u64, _ptr, _ptr]),
     "zllm_kv_mla_layer_wire_bytes": (_u64, [C.POINTER(MlaLayerRecord)]),
     "zllm_kv_mla_layer_write": (_int, [C.POINTER(MlaLayerRecord), _ptr, _u64, C.POINTER(_u64)]),
     "zllm_kv_mla_layer_read": (_int, [_ptr, _u64, C.POINTER(MlaLayerRecord), C.POINTER(_u64)]),

@@ -141,6 +141,15 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
         return fail(-1, "MLA decode: invalid shape batch=%u heads=%u q_head=%u kv_head=%u rope=%u", a->batch, a->heads, a->q_head_dim,
                     a->kv_head_dim, a->rope_dim);
     }
+    {
+        // project_value writes value_dim columns per head into a slot of stride q_head_dim (strided output) or
+        // value_dim (compact): an empty or overlong value part has nowhere to go
+        const uint32_t value_dim = a->kv_head_dim - (a->q_head_dim - a->rope_dim);
+        if (value_dim == 0 || (!a->out_compact && value_dim > a->q_head_dim)) {
+            return fail(-1, "MLA decode: value_dim=%u must be non-zero and, for strided output, at most q_head_dim=%u", value_dim,
+                        a->q_head_dim);
+        }
+    }
     if (a->latent_dim != 512 || a->rope_dim != 64) {
         return fail(-1, "MLA decode: this build handles latent_dim 512 + rope_dim 64 (got %u + %u)", a->latent_dim, a->rope_dim);
     }
@@ -407,17 +416,6 @@ int zllm_attn_scatter_rows(const zllm_scatter_args* a, zllm_stream_t stream)
     }
     zllm::ScatterParams p{a->plane, a->in, a->table, a->first, a->count, a->row_bytes, a->block_tokens, a->ring_capacity};
     return hip_status(zllm::launch_scatter_rows(p, (hipStream_t)stream), "scatter rows launch");
-}
-
-int zllm_attn_stream_read_probe(const void* src, uint64_t bytes, uint32_t* sink, zllm_stream_t stream)
-{
-    if (src == nullptr || sink == nullptr) {
-        return fail(-1, "stream read probe: null pointer");
-    }
-    if ((uintptr_t)src % 16 != 0 || bytes % 16 != 0) {
-        return fail(-1, "stream read probe: source and size must be multiples of 16 bytes");
-    }
-    return hip_status(zllm::launch_stream_read(src, bytes, sink, (hipStream_t)stream), "stream read probe launch");
 }
 
 /* ---- KV snapshot wire format (host) ----------------------------------------------------- */
@@ -766,6 +764,11 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
     if (a->q == nullptr || a->k_plane == nullptr || a->k_scales == nullptr || a->v_plane == nullptr || a->v_scales == nullptr ||
         a->out == nullptr) {
         return fail(-1, "GQA prefill: null pointer");
+    }
+    // the kernel reads codes as 8-byte vectors and scales as 4-byte words, and stores the output as 16- or 8-byte vectors
+    if ((((uintptr_t)a->q | (uintptr_t)a->k_plane | (uintptr_t)a->v_plane | (uintptr_t)a->out) & 15u) != 0 ||
+        (((uintptr_t)a->k_scales | (uintptr_t)a->v_scales) & 3u) != 0) {
+        return fail(-1, "GQA prefill: q, cache planes and out must be 16-byte aligned (scale planes 4-byte)");
     }
     zllm::GqaPrefillParams p;
     memset(&p, 0, sizeof(p));

@@ -90,51 +90,49 @@ __global__ __launch_bounds__(256) void half_append_kernel(HalfAppendParams p)
     p.cache[physical * p.cols + column] = p.dst_dtype == 1 ? f32_to_bf16_bits(value) : f32_to_f16_bits(value);
 }
 
-// Fused MLA append (semantics of paged_cache_append_mla_body,
-// paged_mla/source.hip:672-758): blocks [0, rows * groups) quantize the latent,
-// the remaining blocks rotate and store k_rope as bf16.  The rotation uses
-// separately rounded products (no fused multiply-add) so results do not depend
-// on the compiler's contraction choices.
-__global__ __launch_bounds__(64) void mla_append_kernel(MlaAppendParams p)
+// Fused MLA append (what paged_cache_append_mla_body computes, paged_mla/source.hip:672-758), laid out the way the
+// prologue kernel below is: one wave per token row, four rows per workgroup.  The wave quantizes the row's latent
+// groups one after the other (a group is one value per lane), then writes the row's rope columns as bf16: the
+// columns in front of the rotary part are copied, and each lane of the rotary part owns whole rotation pairs --
+// it loads the pair and its cos / sin once and stores both rotated values.  Products are rounded on their own
+// (no fused multiply-add), so the bits do not depend on the compiler's contraction choices.
+__global__ __launch_bounds__(256) void mla_append_kernel(MlaAppendParams p)
 {
-    const unsigned int lane = threadIdx.x;
-    const unsigned int groups_per_row = p.latent_cols / 64u;
-    const unsigned int latent_groups = p.rows * groups_per_row;
-    const unsigned int position = p.positions != nullptr ? p.positions[0] : p.position;
-    const unsigned int rope_position = p.positions != nullptr ? p.positions[1] : p.rope_position;
-    if (blockIdx.x >= latent_groups) {
-        const unsigned long long rope_index = (unsigned long long)(blockIdx.x - latent_groups) * 64u + lane;
-        const unsigned long long rope_elements = (unsigned long long)p.rows * p.rope_cols;
-        if (rope_index >= rope_elements) {
-            return;
-        }
-        const unsigned int row = (unsigned int)(rope_index / p.rope_cols);
-        const unsigned int column = (unsigned int)(rope_index - (unsigned long long)row * p.rope_cols);
-        const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, 0);
-        float value = p.k_rope[rope_index];
-        if (p.rotary_dim != 0 && column >= p.rope_cols - p.rotary_dim) {
-            const unsigned int start = p.rope_cols - p.rotary_dim;
-            const unsigned int rotary = column - start;
-            const unsigned int half = p.rotary_dim / 2;
-            const unsigned int pair = p.split_half ? rotary % half : rotary / 2;
-            const unsigned int real_column = p.split_half ? start + pair : start + pair * 2;
-            const unsigned int imag_column = p.split_half ? start + half + pair : real_column + 1;
-            const float real = p.k_rope[(unsigned long long)row * p.rope_cols + real_column];
-            const float imaginary = p.k_rope[(unsigned long long)row * p.rope_cols + imag_column];
-            const float c = p.cosine[(unsigned long long)(rope_position + row) * half + pair];
-            const float s = p.sine[(unsigned long long)(rope_position + row) * half + pair];
-            value = column == real_column ? real * c - imaginary * s : imaginary * c + real * s;
-        }
-        p.rope_cache[physical * p.rope_cols + column] = f32_to_bf16_bits(value);
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= p.rows) {
         return;
     }
-    const unsigned int row = blockIdx.x / groups_per_row;
-    const unsigned int group = blockIdx.x - row * groups_per_row;
-    const unsigned int column = group * 64u + lane;
-    const float value = p.latent[(unsigned long long)row * p.latent_cols + column];
+    const unsigned int position = p.positions != nullptr ? p.positions[0] : p.position;
+    const unsigned int rope_position = p.positions != nullptr ? p.positions[1] : p.rope_position;
     const unsigned long long physical = paged_row(p.table, position + row, p.block_tokens, 0);
-    const signed char code = quantize_lane(value, 0, p.latent_scales, physical * groups_per_row + group, lane);
-    p.latent_codes[physical * p.latent_cols + column] = code;
+
+    const unsigned int groups_per_row = p.latent_cols / 64u;
+    const float* latent_row = p.latent + (unsigned long long)row * p.latent_cols;
+    signed char* code_row = p.latent_codes + physical * p.latent_cols;
+    for (unsigned int group = 0; group < groups_per_row; ++group) {
+        const float value = latent_row[group * 64u + lane];
+        code_row[group * 64u + lane] = quantize_lane(value, 0, p.latent_scales, physical * groups_per_row + group, lane);
+    }
+
+    const float* rope_row = p.k_rope + (unsigned long long)row * p.rope_cols;
+    unsigned short* rope_out = p.rope_cache + physical * p.rope_cols;
+    const unsigned int plain_cols = p.rope_cols - p.rotary_dim; // stored as they are
+    for (unsigned int column = lane; column < plain_cols; column += 64u) {
+        rope_out[column] = f32_to_bf16_bits(rope_row[column]);
+    }
+    const unsigned int pairs = p.rotary_dim / 2u;
+    const float* cos_row = p.cosine + (unsigned long long)(rope_position + row) * pairs;
+    const float* sin_row = p.sine + (unsigned long long)(rope_position + row) * pairs;
+    for (unsigned int i = lane; i < pairs; i += 64u) {
+        // split-half keeps the two members of pair i half a rotary block apart, interleaved keeps them adjacent
+        const unsigned int first = plain_cols + (p.split_half ? i : 2u * i);
+        const unsigned int second = p.split_half ? first + pairs : first + 1u;
+        const float x = rope_row[first], y = rope_row[second];
+        const float cs = cos_row[i], sn = sin_row[i];
+        rope_out[first] = f32_to_bf16_bits(x * cs - y * sn);
+        rope_out[second] = f32_to_bf16_bits(y * cs + x * sn);
+    }
 }
 
 // Pre-attention prologue: one wave per (row, head) of Q, K or V.  The head's values sit one per lane per 64-column
@@ -326,44 +324,10 @@ hipError_t launch_gqa_prologue(const GqaPrologueParams& p, hipStream_t stream)
 
 hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream)
 {
-    const unsigned long long latent_groups = (unsigned long long)p.rows * (p.latent_cols / 64u);
-    const unsigned long long rope_blocks = ((unsigned long long)p.rows * p.rope_cols + 63) / 64;
-    if (latent_groups + rope_blocks == 0) {
+    if (p.rows == 0) {
         return hipSuccess;
     }
-    mla_append_kernel<<<dim3((unsigned int)(latent_groups + rope_blocks)), dim3(64), 0, stream>>>(p);
-    return hipGetLastError();
-}
-
-// Measurement aid: streams `n_vec` 16-byte vectors once with plain wide loads and keeps nothing.  The rate it reaches
-// on a buffer of a decode call's KV bytes is the ceiling any kernel that has to read those bytes once can reach.
-__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, unsigned long long n_vec, unsigned int* sink)
-{
-    const unsigned long long stride = (unsigned long long)gridDim.x * 256u;
-    unsigned long long i = (unsigned long long)blockIdx.x * 256u + threadIdx.x;
-    u32x4 acc = {0u, 0u, 0u, 0u};
-    for (; i + 3u * stride < n_vec; i += 4u * stride) {
-        u32x4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            v[u] = __builtin_nontemporal_load(src + i + u * stride);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            acc ^= v[u];
-        }
-    }
-    for (; i < n_vec; i += stride) {
-        acc ^= __builtin_nontemporal_load(src + i);
-    }
-    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a17c0deu && sink[0] == 0xffffffffu) { // keeps the loads alive; practically never true
-        sink[0] = 0u;
-    }
-}
-
-hipError_t launch_stream_read(const void* src, unsigned long long bytes, unsigned int* sink, hipStream_t stream)
-{
-    stream_read_kernel<<<dim3(2048), dim3(256), 0, stream>>>((const u32x4*)src, bytes / 16u, sink);
+    mla_append_kernel<<<dim3((p.rows + 3u) / 4u), dim3(256), 0, stream>>>(p);
     return hipGetLastError();
 }
 

@@ -363,6 +363,26 @@ __device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const Sca
     }
 }
 
+// A FAST path loads whole 16-token tiles, so on the first and last step of a visible range the rows outside
+// [first, len) are whatever their page holds.  Their probabilities are exact zeros, but 0 * scale is NaN when the
+// stale scale bits read as NaN or infinity, and one NaN in P' poisons every dimension of the head.  Clearing the
+// scale rows of those slots (wave-uniform test, edge steps only) makes them contribute exact zeros.
+template <int G>
+__device__ __forceinline__ void clear_hidden_scale_rows(ScaleRow<G> (&vsr)[8], unsigned int t0, unsigned int j, unsigned int first,
+                                                        unsigned int len)
+{
+    if (t0 >= first && t0 + 32u <= len) {
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+        if (token < first || token >= len) {
+            vsr[e] = ScaleRow<G>{};
+        }
+    }
+}
+
 // NBUF = steps of KV kept in registers: loads run NBUF - 1 steps (32 tokens each) ahead of the MFMA work.
 // With pages scattered over a large pool every page costs an address translation as well as an HBM access,
 // and one step of prefetch leaves the wave waiting ~3.5 us per step.
@@ -551,6 +571,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
         }
         float pr[8];
         qk_softmax_step<G, SDT, SOFTCAP>(s.k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
+        clear_hidden_scale_rows<G>(vsr, t0, j, first, len);
         pv_step<G, SDT>(s.v, vsr, pr, acc);
     };
 
@@ -800,6 +821,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         }
         wait_lds_reads();
         issue_codes(v_base, lds_v, slot, t_next);
+        clear_hidden_scale_rows<G>(vsr, t0, j, first, len);
         pv_step<G, SDT>(v, vsr, pr, acc);
     };
 
@@ -997,7 +1019,21 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     float run_sum = 0.0f;
     const float scale_eff = (p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e) / q_norm;
 
-    auto compute_step = [&](const F16Step<D>& s, unsigned int t0) __attribute__((always_inline)) {
+    auto compute_step = [&](F16Step<D>& s, unsigned int t0) __attribute__((always_inline)) {
+        if (FAST && (t0 < first || t0 + 32u > len)) {
+            // whole tiles are loaded: a slot outside [first, len) holds whatever its page does, and 0 * NaN would
+            // poison the head -- such slots multiply as zeros (edge steps only, wave-uniform test)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+                if (token < first || token >= len) {
+#pragma unroll
+                    for (int u = 0; u < VU; ++u) {
+                        s.v[e][u] = u32x4{0u, 0u, 0u, 0u};
+                    }
+                }
+            }
+        }
         float sc[8];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {

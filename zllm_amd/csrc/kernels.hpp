@@ -149,7 +149,6 @@ hipError_t launch_gqa_prologue(const GqaPrologueParams& p, hipStream_t stream);
 hipError_t launch_half_append(const HalfAppendParams& p, hipStream_t stream);
 hipError_t launch_mla_append(const MlaAppendParams& p, hipStream_t stream);
 hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);
-hipError_t launch_stream_read(const void* src, unsigned long long bytes, unsigned int* sink, hipStream_t stream);
 
 // kv_format: 0 = Q8g64, 1 = f16; scale_dtype: 0 = bf16, 1 = f16 (Q8 only).
 hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream);

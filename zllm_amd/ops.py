@@ -96,11 +96,6 @@ def scatter_rows(plane, rows, table, first, block_tokens, ring_capacity=0):
     capi.check(capi.load().zllm_attn_scatter_rows(C.byref(args), _stream()))
 
 
-def stream_read_probe(buffer, sink):
-    """Reads `buffer` (uint8, a multiple of 16 bytes) once and keeps nothing (zllm_attn_stream_read_probe): a measurement aid."""
-    capi.check(capi.load().zllm_attn_stream_read_probe(_ptr(buffer), buffer.numel() * buffer.element_size(), _ptr(sink), _stream()))
-
-
 def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, num_heads, num_kv_heads, head_dim,
                     block_tokens, score_scale, max_kv_len, first_visible=None, softcap=0.0, ring_capacity=0,
                     kv_format=capi.KV_Q8G64, scale_dtype=capi.SCALE_F16, out=None, workspace=None, total_kv_tokens=0, gate=None):
