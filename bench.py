@@ -61,7 +61,7 @@ def probe_lib():
         lib.bench_probe_stream_read.restype = C.c_int
         lib.bench_probe_stream_read.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
         lib.bench_probe_paged_read.restype = C.c_int
-        lib.bench_probe_paged_read.argtypes = [C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        lib.bench_probe_paged_read.argtypes = [C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         _PROBE = lib
     return _PROBE
 
@@ -74,11 +74,11 @@ def stream_read_probe(buffer, sink):
     assert rc == 0, rc
 
 
-def paged_read_probe(planes, table_flat, workgroups, sink):
+def paged_read_probe(planes, table_flat, workgroups, pages_in_flight, sink):
     import torch
 
     rc = probe_lib().bench_probe_paged_read(planes["k_codes"].data_ptr(), planes["v_codes"].data_ptr(), planes["k_scales"].data_ptr(),
-                                            planes["v_scales"].data_ptr(), table_flat.data_ptr(), table_flat.numel(), workgroups,
+                                            planes["v_scales"].data_ptr(), table_flat.data_ptr(), table_flat.numel(), workgroups, pages_in_flight,
                                             sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0, rc
 
@@ -314,11 +314,14 @@ def run_gqa_decode(args, ragged, config1=False):
         if not ragged:
             # the decode kernel's own access pattern without its arithmetic: same pages, same 128-byte lines per wave
             flat = tables_dev.reshape(-1).contiguous()
-            for _ in range(10):
-                paged_read_probe(planes, flat, 256, probe_sink)
-            paged_median, paged_min = event_times_ms(lambda: paged_read_probe(planes, flat, 256, probe_sink), 100)
-            record["roofline"]["paged_read_of_same_pages"] = {"kernel_ms_median": round(paged_median, 5), "kernel_ms_min": round(paged_min, 5),
-                                                              "gbps_median": round(kv_bytes / (paged_median * 1e-3) / 1e9, 1)}
+            paged = {}
+            for in_flight in (1, 2, 4, 8):  # pages (33 KB each) a workgroup requests before it waits
+                for _ in range(10):
+                    paged_read_probe(planes, flat, 256, in_flight, probe_sink)
+                med, low = event_times_ms(lambda: paged_read_probe(planes, flat, 256, in_flight, probe_sink), 100)
+                paged[f"{in_flight}_pages_in_flight"] = {"kernel_ms_median": round(med, 5), "kernel_ms_min": round(low, 5),
+                                                         "gbps_median": round(kv_bytes / (med * 1e-3) / 1e9, 1)}
+            record["roofline"]["paged_read_of_same_pages"] = paged
     if not args.no_cpu_baseline:
         cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)
         record["cpu_baseline"] = cpu

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, unsi
 // fetch one whole 128-byte line with a 16-byte non-temporal load each, eight rows per instruction -- so the eight
 // waves together read whole rows, exactly as the eight KV-head waves of the decode kernel do.  Eight code loads and
 // one scale load are in flight per lane per page.
-__global__ __launch_bounds__(512) void paged_read_kernel(const unsigned char* k_plane, const unsigned char* v_plane,
+template <int INFLIGHT> __global__ __launch_bounds__(512) void paged_read_kernel(const unsigned char* k_plane, const unsigned char* v_plane,
                                                          const unsigned char* k_scales, const unsigned char* v_scales,
                                                          const unsigned int* table, unsigned int pages, unsigned int pages_per_group,
                                                          unsigned int* sink)
@@ -48,11 +48,11 @@ __global__ __launch_bounds__(512) void paged_read_kernel(const unsigned char* k_
     const unsigned int lane_off = (lane >> 3) * 1024u + wave * 128u + (lane & 7u) * 16u;
     u32x4 acc = {0u, 0u, 0u, 0u};
     unsigned int acc_s = 0u;
-    for (unsigned int p = first; p < last; p += 2u) {
-        u32x4 v[2][4];
-        unsigned int s[2];
+    for (unsigned int p = first; p < last; p += INFLIGHT) {
+        u32x4 v[INFLIGHT][4];
+        unsigned int s[INFLIGHT];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < INFLIGHT; ++u) {
             const unsigned int page = table[min(p + u, last - 1u)];
             const unsigned long long base = (unsigned long long)page * 16384u;
             v[u][0] = __builtin_nontemporal_load((const u32x4*)(k_plane + base + lane_off));
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(512) void paged_read_kernel(const unsigned char* k_
             s[u] = *(const unsigned int*)sp;
         }
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < INFLIGHT; ++u) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 acc ^= v[u][w];
@@ -91,7 +91,7 @@ __attribute__((visibility("default"))) int bench_probe_stream_read(const void* s
 // `pages` entries of `table` name 16-row pages of planes whose rows are 1,024 bytes (codes) and 32 bytes (scales).
 __attribute__((visibility("default"))) int bench_probe_paged_read(const void* k_plane, const void* v_plane, const void* k_scales,
                                                                   const void* v_scales, const uint32_t* table, uint32_t pages,
-                                                                  uint32_t workgroups, uint32_t* sink, void* stream)
+                                                                  uint32_t workgroups, uint32_t pages_in_flight, uint32_t* sink, void* stream)
 {
     if (k_plane == nullptr || v_plane == nullptr || k_scales == nullptr || v_scales == nullptr || table == nullptr || sink == nullptr ||
         pages == 0 || workgroups == 0) {
@@ -99,9 +99,17 @@ __attribute__((visibility("default"))) int bench_probe_paged_read(const void* k_
     }
     const uint32_t per_group = (pages + workgroups - 1) / workgroups;
     const uint32_t groups = (pages + per_group - 1) / per_group;
-    paged_read_kernel<<<dim3(groups), dim3(512), 0, (hipStream_t)stream>>>((const unsigned char*)k_plane, (const unsigned char*)v_plane,
-                                                                             (const unsigned char*)k_scales, (const unsigned char*)v_scales,
-                                                                             table, pages, per_group, sink);
+    const unsigned char *kp = (const unsigned char*)k_plane, *vp = (const unsigned char*)v_plane;
+    const unsigned char *ks = (const unsigned char*)k_scales, *vs = (const unsigned char*)v_scales;
+    const hipStream_t st = (hipStream_t)stream;
+    // pages a workgroup requests before it waits for any of them
+    switch (pages_in_flight) {
+    case 1: paged_read_kernel<1><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    case 2: paged_read_kernel<2><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    case 4: paged_read_kernel<4><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    case 8: paged_read_kernel<8><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    default: return -1;
+    }
     return (int)hipGetLastError();
 }
 
