@@ -276,6 +276,20 @@ typedef struct zllm_gqa_decode_args {
 ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* args);
 ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);
 
+/* zllm_attn_gqa_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher takes its
+ * split records from a pool (src/kernel/rocm/hip/tensor/attention.rs:1031-1046).  Same arguments, same kernels
+ * and the same output bits as zllm_attn_gqa_decode, except that `workspace` / `workspace_bytes` are ignored: the
+ * split records go to an array that is part of the library's device code (zllm_attn_static_scratch_bytes() bytes
+ * on every GPU the library is loaded on, held until the process ends).  A call whose
+ * zllm_attn_gqa_decode_workspace_bytes exceeds that size is rejected (negative return, nothing launched).
+ * Nothing in the array has to survive between calls and nothing in it has to be cleared.  All calls on one GPU
+ * share the one array: calls that overlap on a GPU (two streams, two threads) race and must be serialised by the
+ * caller.  zllm_attn_init(device, ...) looks the array's address up for that device; without it the first call
+ * on a device does (make that call, or the init call, before a capture begins). */
+ZLLM_API uint64_t zllm_attn_static_scratch_bytes(void);
+ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * GQA chunked prefill: T query rows appended at `position`.                  *
  * ------------------------------------------------------------------------- */

@@ -112,6 +112,8 @@ SYMBOLS = {
     "zllm_kv_mla_layer_read": (_int, [_ptr, _u64, C.POINTER(MlaLayerRecord), C.POINTER(_u64)]),
     "zllm_attn_gqa_decode_workspace_bytes": (_u64, [C.POINTER(GqaDecodeArgs)]),
     "zllm_attn_gqa_decode": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
+    "zllm_attn_static_scratch_bytes": (_u64, []),
+    "zllm_attn_gqa_decode_static": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
     "zllm_attn_gqa_prefill_workspace_bytes": (_u64, [C.POINTER(GqaPrefillArgs)]),
     "zllm_attn_gqa_prefill_chunk": (_int, [C.POINTER(GqaPrefillArgs), _ptr]),
     "zllm_attn_mla_decode_workspace_bytes": (_u64, [C.POINTER(MlaDecodeArgs)]),

@@ -8,6 +8,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "kernels.hpp"
 
 namespace {
@@ -33,6 +35,53 @@ int hip_status(hipError_t err, const char* what)
 }
 
 constexpr unsigned int kComputeUnits = 256; // MI355X
+
+} // namespace
+
+// Split records of zllm_attn_gqa_decode_static: one copy of this array lives on every GPU the library's code object
+// is loaded on, from load to process end.  In host code the name below is only a handle for hipGetSymbolAddress --
+// it is never passed to a kernel or a memory call; the device address found for each GPU is.
+constexpr uint64_t kStaticScratchBytes = 16ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_of_device[kMaxDevices];
+
+// Device address of `scratch` on `device`, which must be the current device.  Looked up once per device; two threads
+// racing through the first call find the same address.
+int resolve_static_scratch(int device, void** base)
+{
+    if (device < 0 || device >= kMaxDevices) {
+        return fail(-1, "static scratch: device index %d out of range", device);
+    }
+    void* known = g_scratch_of_device[device].load(std::memory_order_acquire);
+    if (known == nullptr) {
+        void* found = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) {
+            return hip_status(err, "hipGetSymbolAddress(scratch)");
+        }
+        if (found == nullptr) {
+            return fail(-1, "static scratch: no device address on device %d", device);
+        }
+        g_scratch_of_device[device].store(found, std::memory_order_release);
+        known = found;
+    }
+    *base = known;
+    return 0;
+}
+
+int static_scratch_of_current_device(void** base)
+{
+    int device = -1;
+    const hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) {
+        return hip_status(err, "hipGetDevice");
+    }
+    return resolve_static_scratch(device, base);
+}
 
 unsigned int shift_of(unsigned int block_tokens)
 {
@@ -210,7 +259,24 @@ int zllm_attn_init(int device, int* cu_count)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
         return fail(-2, "zllm_attn is built for gfx950 only; device %d is %s", device, prop.gcnArchName);
     }
-    return 0;
+    // the static scratch array of zllm_attn_gqa_decode_static: its address on this device, found with the device current
+    int current = -1;
+    err = hipGetDevice(&current);
+    if (err != hipSuccess) {
+        return hip_status(err, "hipGetDevice");
+    }
+    if (current != device) {
+        err = hipSetDevice(device);
+        if (err != hipSuccess) {
+            return hip_status(err, "hipSetDevice");
+        }
+    }
+    void* base = nullptr;
+    const int found = resolve_static_scratch(device, &base);
+    if (current != device) {
+        (void)hipSetDevice(current);
+    }
+    return found;
 }
 
 const char* zllm_attn_last_error(void)
@@ -582,23 +648,20 @@ uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* a)
     return align_up(rows * a->head_dim * 4, 256) + align_up(rows * 8, 256);
 }
 
-int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
+// The decode call over a workspace that is either the caller's or the library's static array.
+static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint64_t workspace_bytes, zllm_stream_t stream)
 {
-    const int rc = validate_gqa_decode(a);
-    if (rc != 0) {
-        return rc;
-    }
     if (a->q == nullptr || a->k_plane == nullptr || a->v_plane == nullptr || a->kv_lens == nullptr || a->out == nullptr ||
-        a->workspace == nullptr || (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
+        workspace == nullptr || (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
         return fail(-1, "GQA decode: null pointer");
     }
-    if ((((uintptr_t)a->q | (uintptr_t)a->k_plane | (uintptr_t)a->v_plane | (uintptr_t)a->workspace | (uintptr_t)a->out) & 15u) != 0 ||
+    if ((((uintptr_t)a->q | (uintptr_t)a->k_plane | (uintptr_t)a->v_plane | (uintptr_t)workspace | (uintptr_t)a->out) & 15u) != 0 ||
         (((uintptr_t)a->k_scales | (uintptr_t)a->v_scales) & 3u) != 0) {
         return fail(-1, "GQA decode: q, cache planes, out and workspace must be 16-byte aligned (scale planes 4-byte)");
     }
     const uint64_t need = zllm_attn_gqa_decode_workspace_bytes(a);
-    if (a->workspace_bytes < need) {
-        return fail(-1, "GQA decode: workspace %llu bytes, need %llu", (unsigned long long)a->workspace_bytes, (unsigned long long)need);
+    if (workspace_bytes < need) {
+        return fail(-1, "GQA decode: workspace %llu bytes, need %llu", (unsigned long long)workspace_bytes, (unsigned long long)need);
     }
     if (a->tables != nullptr && (uint64_t)a->table_stride * a->block_tokens < a->max_kv_len && a->ring_capacity == 0) {
         return fail(-1, "GQA decode: table_stride=%u pages of %u tokens cannot cover max_kv_len=%u", a->table_stride, a->block_tokens,
@@ -617,8 +680,8 @@ int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
     p.out = a->out;
     plan_gqa_decode(a, &p.chunk_tokens, &p.max_chunks);
     const uint64_t rows = (uint64_t)a->batch * p.max_chunks * a->num_heads;
-    p.partial = (float*)a->workspace;
-    p.stats = (float*)((char*)a->workspace + align_up(rows * a->head_dim * 4, 256));
+    p.partial = (float*)workspace;
+    p.stats = (float*)((char*)workspace + align_up(rows * a->head_dim * 4, 256));
     p.batch = a->batch;
     p.num_heads = a->num_heads;
     p.num_kv_heads = a->num_kv_heads;
@@ -641,6 +704,39 @@ int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
         p.gate_dtype = a->gate_dtype;
     }
     return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, a->stages, (hipStream_t)stream), "GQA decode launch");
+}
+
+int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
+{
+    const int rc = validate_gqa_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    return gqa_decode_over(a, a->workspace, a->workspace_bytes, stream);
+}
+
+uint64_t zllm_attn_static_scratch_bytes(void)
+{
+    return kStaticScratchBytes;
+}
+
+int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* a, zllm_stream_t stream)
+{
+    const int rc = validate_gqa_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    const uint64_t need = zllm_attn_gqa_decode_workspace_bytes(a);
+    if (need > kStaticScratchBytes) {
+        return fail(-1, "GQA decode (static scratch): the split records of this call need %llu bytes, the static array holds %llu",
+                    (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+    }
+    void* base = nullptr;
+    const int found = static_scratch_of_current_device(&base);
+    if (found != 0) {
+        return found;
+    }
+    return gqa_decode_over(a, base, kStaticScratchBytes, stream);
 }
 
 /* ---- MLA decode ------------------------------------------------------------------------- */

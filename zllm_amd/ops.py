@@ -118,6 +118,8 @@ def gqa_decode_args(q, k_plane, k_scales, v_plane, v_scales, tables, kv_lens, nu
     need = capi.load().zllm_attn_gqa_decode_workspace_bytes(C.byref(args))
     if need == 0:
         raise capi.ZllmAttnError(-1, capi.last_error())
+    if workspace is False:  # the static-scratch entry point ignores both fields
+        return args, out, None
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     args.workspace, args.workspace_bytes = _ptr(workspace), workspace.numel()
@@ -128,6 +130,13 @@ def gqa_decode(*a, **kw):
     """Batched GQA decode over the paged cache (zllm_attn_gqa_decode).  Returns f32 [batch, Hq*d]."""
     args, out, workspace = gqa_decode_args(*a, **kw)
     capi.check(capi.load().zllm_attn_gqa_decode(C.byref(args), _stream()))
+    return out
+
+
+def gqa_decode_static(*a, **kw):
+    """zllm_attn_gqa_decode_static: the same call over the library's static device array (no workspace of the caller's)."""
+    args, out, _ = gqa_decode_args(*a, workspace=False, **kw)
+    capi.check(capi.load().zllm_attn_gqa_decode_static(C.byref(args), _stream()))
     return out
 
 
