@@ -377,21 +377,23 @@ ZLLM_API int zllm_attn_gqa_prologue(const zllm_gqa_prologue_args* args, zllm_str
  * MLA absorbed decode over the Q8g64 latent cache.                           *
  * ------------------------------------------------------------------------- */
 
-/* Replaces try_paged_mla_attention_ct_into for query_rows == 1 per sequence
- * (src/kernel/rocm/hip/attention/paged_mla.rs:2870-2914, inner :2917-3634):
+/* Replaces try_paged_mla_attention_ct_into
+ * (src/kernel/rocm/hip/attention/paged_mla.rs:2870-2914, inner :2917-3634), one query row per sequence or a
+ * prefill chunk of `query_rows` rows (the dense prefill arm, kernel mla_paged_dense_latent_f32,
+ * paged_mla/source.hip:3739):
  * absorb (q_nope . W_kv_b[h, 0:nope, :] -> bf16) -> split-KV partial -> LSE
  * merge -> project value (weighted . W_kv_b[h, nope:, :]^T).  Output rows have
  * stride q_head_dim with only the first value_dim entries of each head slot
  * written (src/attention/mla.rs:134) when out_compact == 0, or are compact
  * [batch, heads * value_dim] (src/kernel/cpu/mla.rs:1064-1075) otherwise. */
 typedef struct zllm_mla_decode_args {
-    const void* q;                /* [dev] [batch, heads * q_head_dim], q_dtype */
+    const void* q;                /* [dev] [batch * rows, heads * q_head_dim], q_dtype */
     const uint16_t* kv_b;         /* [dev] bf16 bits [heads * kv_head_dim, latent_dim] */
     const int8_t* latent_codes;   /* [dev] [rows, latent_dim] */
     const uint16_t* latent_scales;/* [dev] bf16 bits [rows, latent_dim / 64] */
     const uint16_t* rope_cache;   /* [dev] bf16 bits [rows, rope_dim] */
     const uint32_t* tables;       /* [dev] [batch, table_stride] */
-    const uint32_t* ctx_lens;     /* [dev] [batch] tokens visible to the query row */
+    const uint32_t* ctx_lens;     /* [dev] [batch] tokens visible to the (last) query row of each sequence */
     void* out;                    /* [dev] out_dtype */
     void* workspace;              /* [dev] */
     uint64_t workspace_bytes;
@@ -417,8 +419,17 @@ typedef struct zllm_mla_decode_args {
      * selection_counts[b] when given, else top_k; a sequence with ctx_len <= top_k stays dense.
      * Entries are token positions (< ctx_len), used in the order given.  NULL = dense. */
     uint32_t top_k;
-    const uint32_t* selection;        /* [dev] [batch, top_k] or NULL */
-    const uint32_t* selection_counts; /* [dev] [batch] or NULL */
+    const uint32_t* selection;        /* [dev] [batch * rows, top_k] or NULL */
+    const uint32_t* selection_counts; /* [dev] [batch * rows] or NULL */
+    /* Query rows per sequence.  0 or 1: a decode step.  T > 1: a prefill chunk -- the last T tokens of every
+     * sequence are its query rows (already appended to the cache), causal inside the chunk: row r sees
+     * ctx_lens[b] - (T - 1 - r) tokens, i.e. position + r + 1 with position = ctx_lens[b] - T
+     * (MlaPrefillBackend::mla_prefill_attention{,_rope}, src/backend/mod.rs:1134-1152; the query_rows > 1 arm of
+     * try_paged_mla_attention_ct_into, src/kernel/rocm/hip/attention/paged_mla.rs:3397-3549; causal rule as in
+     * src/kernel/cpu/mla.rs:958-1018).  q is [batch * T, heads * q_head_dim] and out [batch * T, ...], sequence-major;
+     * a selection holds one list per query row.  The reference returns bf16 for T > 1
+     * (src/backend/rocm/attention.rs:17-19): pass out_dtype = ZLLM_DTYPE_BF16 for that.  batch * T <= 65535. */
+    uint32_t query_rows;
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
 ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);

@@ -348,3 +348,122 @@ def test_config4_full_size(block_tokens):
     w = O.bf16_to_f32(case["kv_b_bits"]).reshape(128, 256, 512)[:, 128:, :]
     want = np.einsum("hvc,c->hv", w.astype(np.float64), lat.astype(np.float64).mean(0))
     assert np.abs(zero[2] - want).max() < 2e-3
+
+
+# ---- prefill chunks: several query rows per sequence --------------------------------------------------------------
+
+def make_mla_chunk_case(seed, lens, rows, heads, **kw):
+    """An MLA case whose sequences end in a chunk of `rows` query rows (already in the cache): queries [batch * rows, ...]."""
+    case = make_mla_case(seed, lens, heads, **kw)
+    rng = np.random.default_rng(seed + 1000)
+    q = rng.standard_normal((len(lens) * rows, heads * (case["nope"] + case["rope_dim"]))).astype(np.float32)
+    case["q_bits"] = O.f32_to_bf16(q)
+    case["rows"] = rows
+    return case
+
+
+def oracle_mla_chunk(case, selection=None):
+    """The oracle's own query_rows > 1 arm (src/kernel/cpu/mla.rs:958-1076): row r of a chunk at query_start sees
+    query_start + r + 1 tokens.  Returns f32 and bf16-bit outputs [batch * rows, heads * value_dim]."""
+    spec, bt, rows = case["spec"], case["block_tokens"], case["rows"]
+    kv_b = O.bf16_to_f32(case["kv_b_bits"])
+    outs_f, outs_b = [], []
+    for b, l in enumerate(case["lens"]):
+        l = int(l)
+        codes = O.gather_rows_bytes(case["codes"], case["tables"][b], bt, 0, l, case["latent"])
+        scales = O.gather_rows_bytes(case["scales"], case["tables"][b], bt, 0, l, case["latent"] // 64 * 2).view(np.uint16)
+        rope = O.gather_rows_bytes(case["rope"], case["tables"][b], bt, 0, l, case["rope_dim"] * 2).view(np.uint16)
+        sel, width = None, 0
+        if selection is not None:
+            sel, width = selection[b * rows:(b + 1) * rows], selection.shape[1]
+        rc, ob, of, _ = O.mla_absorbed_q8_history(spec, case["q_bits"][b * rows:(b + 1) * rows], rows, l - rows, codes, scales, 64,
+                                                  rope, l, kv_b, selection=sel, width=width)
+        assert rc == 0
+        outs_f.append(of.reshape(rows, -1))
+        outs_b.append(ob.reshape(rows, -1))
+    return np.concatenate(outs_f), np.concatenate(outs_b)
+
+
+def run_mla_chunk(case, out_dtype=None, selection=None, compact=True):
+    from zllm_amd import ops
+
+    out = ops.mla_decode(to_torch_bf16(case["q_bits"], "cuda"), upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]),
+                         upload(case["rope"]), upload(case["tables"]), upload(case["lens"]), case["heads"],
+                         case["nope"] + case["rope_dim"], case["nope"] + case["value"], case["latent"], case["rope_dim"],
+                         case["block_tokens"], int(case["lens"].max()), out_dtype=out_dtype or torch.float32, out_compact=compact,
+                         selection=None if selection is None else upload(selection), query_rows=case["rows"])
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("heads,lens,rows,block_tokens", [(16, [40], 8, 16), (128, [700, 300], 5, 16), (32, [1300, 64, 129], 64, 64),
+                                                          (20, [33, 97], 33, 16), (64, [2500], 3, 48)])
+def test_mla_prefill_chunk_matches_oracle(heads, lens, rows, block_tokens):
+    """Chunked MLA prefill: `rows` query rows per sequence, causal inside the chunk, f32 and bf16 output
+    (the reference returns bf16 for more than one row, src/backend/rocm/attention.rs:17-19)."""
+    case = make_mla_chunk_case(heads + rows, lens, rows, heads, block_tokens=block_tokens)
+    want_f, want_b = oracle_mla_chunk(case)
+    got = run_mla_chunk(case).cpu().numpy()
+    print("mla chunk", heads, lens, rows, assert_attention_close(got, want_f, f"MLA chunk heads={heads} lens={lens} rows={rows}"))
+    got_b = run_mla_chunk(case, out_dtype=torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    diff = np.abs(O.bf16_to_f32(got_b).astype(np.float64) - O.bf16_to_f32(want_b))
+    step = np.maximum(np.abs(O.bf16_to_f32(want_b)), 2.0 ** -126) * 2.0 ** -7
+    assert (diff <= step + 2e-3).all()
+
+
+def test_mla_prefill_chunk_rows_equal_single_row_calls():
+    """Row r of a chunk is the decode step of a sequence that ends at that row: same kernels, same bits."""
+    case = make_mla_chunk_case(77, [600, 90], 4, 32)
+    got = run_mla_chunk(case).cpu().numpy()
+    for b, l in enumerate(case["lens"]):
+        for r in range(4):
+            single = dict(case)
+            single["lens"] = np.array([int(l) - 3 + r], dtype=np.uint32)
+            single["tables"] = case["tables"][b:b + 1]
+            single["q_bits"] = case["q_bits"][b * 4 + r:b * 4 + r + 1]
+            one = run_mla(single, max_ctx_len=int(case["lens"].max())).cpu().numpy()
+            assert np.array_equal(one[0], got[b * 4 + r]), (b, r)
+
+
+def test_mla_prefill_chunk_zero_query_is_the_running_mean():
+    """The reference's chunk vector (src/kernel/cpu/mla.rs:1197-1205: zero queries, two rows at position 2 of four
+    tokens whose values are 1/10, 2/20, 3/30, 4/40 -> [2, 20, 2.5, 25]) on this kernel's shape: zero queries make
+    every row the mean of the value projections of the tokens it sees, here 4 tokens and a chunk of 2 rows."""
+    heads = 16
+    case = make_mla_chunk_case(5, [4], 2, heads)
+    case["q_bits"][:] = 0
+    # latent column 0 carries t + 1 and column 64 (another scale group) 10 (t + 1); the value weights pick them out
+    lat = np.zeros((4, 512), dtype=np.float32)
+    lat[:, 0] = [1, 2, 3, 4]
+    lat[:, 64] = [10, 20, 30, 40]
+    case["codes"][:] = 0
+    case["scales"][:] = 0
+    O.q8g64_append_paged(O.RULE_ROCM_MLA, lat, case["codes"], case["scales"], case["tables"][0], 0, case["block_tokens"])
+    w = np.zeros((heads, 256, 512), dtype=np.float32)
+    w[:, 128, 0] = 1.0   # value column 0 <- latent column 0
+    w[:, 129, 64] = 1.0  # value column 1 <- latent column 64
+    case["kv_b_bits"] = O.f32_to_bf16(w.reshape(heads * 256, 512))
+    got = run_mla_chunk(case).cpu().numpy().reshape(2, heads, 128)
+    want_f, _ = oracle_mla_chunk(case)
+    assert_attention_close(got.reshape(2, -1), want_f, "zero-query chunk")
+    # 1, 2, 3 (and 10, 20, 30) are exact in Q8 with these scales up to the bf16 rounding of the scale: compare at 1e-2
+    np.testing.assert_allclose(got[0, :, 0], 2.0, rtol=1e-2)
+    np.testing.assert_allclose(got[0, :, 1], 20.0, rtol=1e-2)
+    np.testing.assert_allclose(got[1, :, 0], 2.5, rtol=1e-2)
+    np.testing.assert_allclose(got[1, :, 1], 25.0, rtol=1e-2)
+    assert (got[:, :, 2:] == 0).all()
+
+
+def test_mla_prefill_chunk_with_per_row_selection():
+    """Selected-token prefill: one list per query row, positions inside the row's causal prefix
+    (src/kernel/cpu/mla.rs:1008-1018)."""
+    rows, top_k = 4, 64
+    case = make_mla_chunk_case(31, [500, 300], rows, 16)
+    rng = np.random.default_rng(32)
+    sel = np.zeros((2 * rows, top_k), dtype=np.uint32)
+    for b, l in enumerate(case["lens"]):
+        for r in range(rows):
+            sel[b * rows + r] = rng.choice(int(l) - rows + r + 1, size=top_k, replace=False)
+    want_f, _ = oracle_mla_chunk(case, selection=sel)
+    got = run_mla_chunk(case, selection=sel).cpu().numpy()
+    assert_attention_close(got, want_f, "selected chunk")

@@ -179,6 +179,12 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     plan_splits(a->max_kv_len, a->max_kv_len, columns, kMinGqaChunk, rounds, chunk_tokens, max_chunks);
 }
 
+// query rows per sequence: 0 and 1 both mean a decode step
+uint32_t mla_query_rows(const zllm_mla_decode_args* a)
+{
+    return a->query_rows == 0 ? 1u : a->query_rows;
+}
+
 int validate_mla_decode(const zllm_mla_decode_args* a)
 {
     if (a == nullptr) {
@@ -214,6 +220,10 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
     if (a->selection != nullptr && a->top_k == 0) {
         return fail(-1, "MLA decode: a selection needs top_k > 0");
     }
+    // query rows over the whole call index the grid's third dimension
+    if ((uint64_t)a->batch * mla_query_rows(a) > 65535u) {
+        return fail(-1, "MLA decode: batch=%u x query_rows=%u exceeds 65535 query rows per call", a->batch, a->query_rows);
+    }
     return 0;
 }
 
@@ -223,7 +233,7 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    plan_splits(longest, longest, a->batch * head_blocks, 64, 1, chunk_tokens, max_chunks);
+    plan_splits(longest, longest, a->batch * mla_query_rows(a) * head_blocks, 64, 1, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {
@@ -233,7 +243,7 @@ struct MlaWorkspace {
 MlaWorkspace mla_workspace(const zllm_mla_decode_args* a, uint32_t max_chunks)
 {
     MlaWorkspace w;
-    const uint64_t rows = (uint64_t)a->batch * a->heads;
+    const uint64_t rows = (uint64_t)a->batch * mla_query_rows(a) * a->heads;
     w.absorbed = 0;
     w.partial = align_up(rows * (a->latent_dim + a->rope_dim) * 2, 256);
     w.stats = w.partial + align_up(rows * max_chunks * a->latent_dim * 4, 256);
@@ -790,7 +800,8 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     p.partial = (float*)(ws + w.partial);
     p.stats = (float*)(ws + w.stats);
     p.weighted = (float*)(ws + w.weighted);
-    p.batch = a->batch;
+    p.query_rows = mla_query_rows(a);
+    p.batch = a->batch * p.query_rows; // the kernels index query rows; a row finds its sequence by division
     p.heads = a->heads;
     p.q_head_dim = a->q_head_dim;
     p.kv_head_dim = a->kv_head_dim;

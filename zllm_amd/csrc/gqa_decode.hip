@@ -1160,7 +1160,12 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     const unsigned int sl = threadIdx.x / quads;
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
-    const unsigned int len = p.kv_lens[b];
+    unsigned int len = p.kv_lens[b];
+    if (p.query_rows > 1u) { // record row b of a multi-row call: its sequence's length less the chunk rows after it
+        const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
+        len = p.kv_lens[b / p.query_rows];
+        len = len > behind ? len - behind : 0u;
+    }
     unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
     first = min(first, len);
     const unsigned int first_al = first & ~31u;

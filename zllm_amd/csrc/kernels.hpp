@@ -97,6 +97,9 @@ struct GqaDecodeParams {
     const void* gate; // optional sigmoid output gate [batch][gate_cols]
     unsigned int gate_cols;
     int gate_dtype;
+    // split merge only: query rows per sequence (0 = 1).  Record row v belongs to sequence v / query_rows and sees
+    // kv_lens[sequence] - (query_rows - 1 - v % query_rows) tokens; `batch` then counts record rows.
+    unsigned int query_rows;
 };
 
 struct GqaPrefillParams {
@@ -138,6 +141,10 @@ struct MlaDecodeParams {
     const unsigned int* selection;        // [batch][top_k] token positions, or nullptr (dense)
     const unsigned int* selection_counts; // [batch] or nullptr
     unsigned int top_k;
+    // Query rows per sequence (>= 1).  With more than one, the last query_rows tokens of a sequence are its query rows
+    // (a prefill chunk, causal inside the chunk): `batch` counts query rows over all sequences, row v belongs to
+    // sequence v / query_rows and sees ctx_lens[sequence] - (query_rows - 1 - v % query_rows) tokens.
+    unsigned int query_rows;
 };
 
 // KV heads (= waves) per GQA decode workgroup for a head dimension.

@@ -63,6 +63,17 @@ __device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned i
     return row * kRowBytes + ((chunk ^ swz(row)) << 4);
 }
 
+// Query row v of the call: its sequence and the number of tokens it sees.  With query_rows > 1 the rows of a
+// sequence are the last query_rows tokens of its context, each seeing everything up to and including itself
+// (src/kernel/cpu/mla.rs:1016-1018: row r of a chunk at query_start sees query_start + r + 1 tokens).
+__device__ __forceinline__ unsigned int visible_tokens(const unsigned int* ctx_lens, unsigned int query_rows, unsigned int v, unsigned int& sequence)
+{
+    sequence = v / query_rows;
+    const unsigned int behind = query_rows - 1u - v % query_rows; // rows of the chunk after this one
+    const unsigned int len = ctx_lens[sequence];
+    return len > behind ? len - behind : 0u;
+}
+
 // ---------------------------------------------------------------------------------------------
 // 1. absorb
 // ---------------------------------------------------------------------------------------------
@@ -181,8 +192,9 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int j = lane >> 4;
     const unsigned int chunk = blockIdx.x;
     const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
-    const unsigned int b = blockIdx.z;
-    unsigned int len = p.ctx_lens[b]; // keys of this sequence: positions, or list slots when a selection applies
+    const unsigned int b = blockIdx.z; // query row of the call (= sequence when every sequence has one row)
+    unsigned int seq;
+    unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq); // keys of this row: positions, or list slots when a selection applies
     const unsigned int* selected = nullptr;
     if constexpr (SELECTED) {
         if (p.selection != nullptr && p.top_k < len) {
@@ -206,7 +218,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int c_start = (unsigned int)c_start64;
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + kStepTokens - 1) / kStepTokens;
-    const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)b * p.table_stride : nullptr;
+    const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)seq * p.table_stride : nullptr;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
     // ---- staging: loads of a later tile's bytes, converted by the thread that loaded them
@@ -813,7 +825,8 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
     const unsigned int b = blockIdx.y;
     const unsigned int quad = threadIdx.x & 127u;
     const unsigned int sl = threadIdx.x >> 7;
-    const unsigned int len = p.ctx_lens[b];
+    unsigned int seq;
+    const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
     const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
     const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
     const size_t stat_stride = (size_t)p.heads * 2;
@@ -935,6 +948,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         mp.head_dim = p.latent_dim;
         mp.chunk_tokens = p.chunk_tokens;
         mp.max_chunks = p.max_chunks;
+        mp.query_rows = p.query_rows;
         err = launch_split_merge(mp, stream);
         if (err != hipSuccess) {
             return err;

@@ -164,12 +164,14 @@ def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, 
 
 def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ctx_lens, heads, q_head_dim,
                     kv_head_dim, latent_dim, rope_dim, block_tokens, max_ctx_len, out_dtype=torch.float32,
-                    out_compact=True, out=None, workspace=None, selection=None, selection_counts=None):
-    batch = q.shape[0]
+                    out_compact=True, out=None, workspace=None, selection=None, selection_counts=None, query_rows=1):
+    """`q` holds every query row of the call, sequence-major: [batch * query_rows, heads * q_head_dim]."""
+    rows = q.shape[0]
+    batch = rows // query_rows
     value_dim = kv_head_dim - (q_head_dim - rope_dim)
     if out is None:
         cols = heads * value_dim if out_compact else heads * q_head_dim
-        out = torch.zeros((batch, cols), dtype=out_dtype, device=q.device)
+        out = torch.zeros((rows, cols), dtype=out_dtype, device=q.device)
     args = capi.MlaDecodeArgs()
     args.q, args.kv_b, args.latent_codes = _ptr(q), _ptr(kv_b), _ptr(latent_codes)
     args.latent_scales, args.rope_cache = _ptr(latent_scales), _ptr(rope_cache)
@@ -179,6 +181,7 @@ def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ct
     args.table_stride = 0 if tables is None else tables.shape[1]
     args.max_ctx_len, args.block_tokens = max_ctx_len, block_tokens
     args.q_dtype, args.out_dtype, args.out_compact = _DTYPE[q.dtype], _DTYPE[out_dtype], int(out_compact)
+    args.query_rows = query_rows
     if selection is not None:  # [batch, top_k] token positions (uint32 / int32)
         args.selection, args.top_k = _ptr(selection), selection.shape[1]
         args.selection_counts = _ptr(selection_counts)
