@@ -298,7 +298,11 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * (src/kernel/rocm/hip/tensor/attention.rs:727-798,
  * src/backend/rocm/attention.rs:2232-2242).  Row r attends logical tokens
  * key_range(position + r, position + rows) of one sequence whose K/V
- * (including the chunk's own rows) are already in the paged cache. */
+ * (including the chunk's own rows) are already in the paged cache.
+ * head_dim 128 over a Q8g64 cache runs the matrix-core chunk kernel and needs no
+ * workspace.  head_dim 64 / 256 and f16 caches run every row as one item of the
+ * split-KV decode kernels (bound by cache bandwidth, not by the matrix cores) and
+ * need zllm_attn_gqa_prefill_workspace_bytes of workspace. */
 typedef struct zllm_gqa_prefill_args {
     const void* q;         /* [dev] [rows, num_heads * head_dim], q_dtype */
     const void* k_plane;   /* [dev] */
@@ -323,6 +327,14 @@ typedef struct zllm_gqa_prefill_args {
     const void* gate;              /* [dev] [rows, gate_cols], gate_dtype */
     uint32_t gate_cols;            /* num_heads * head_dim, or 1 (one gate per row) */
     int gate_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
+    /* Explicit visible ends, the multimodal case in which the rows of a visual block read to the end of their
+     * block (CausalWindow::key_range_with_visible_end, src/attention/gqa.rs:65-68;
+     * gqa_prefill_attention_cached_visible, src/backend/rocm/attention.rs:2256-2316; per-row ranges of
+     * BlockAttentionBackend::block_attention, src/backend/mod.rs:1583-1616): row r attends
+     * [start of key_range(position + r), min(max(position + r + 1, visible_ends[r]), position + rows)).
+     * Absolute token positions.  NULL = causal. */
+    const uint32_t* visible_ends;  /* [dev] [rows] or NULL */
+    uint32_t table_stride;         /* entries in `table` (0 = not stated: the table must cover position + rows) */
 } zllm_gqa_prefill_args;
 ZLLM_API uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* args);
 ZLLM_API int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* args, zllm_stream_t stream);

@@ -11,10 +11,10 @@ torch = pytest.importorskip("torch")
 
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
-             out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0, oracle_segments=None):
+             out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0, oracle_segments=None,
+             d=128, visible_ends=None):
     from zllm_amd import capi, ops
 
-    d = 128
     out_dtype = out_dtype or torch.float32
     rng = np.random.default_rng(seed)
     cols = hkv * d
@@ -59,7 +59,8 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     gate = (rng.standard_normal((chunk, gate_cols)) * 3).astype(np.float32) if gate_cols else None
     out = ops.gqa_prefill_chunk(to_torch_bf16(q_bits, "cuda") if q_bf16 else upload(q), dev["k_codes"], dev["k_scales"], dev["v_codes"],
                                 dev["v_scales"], table, prefix, hq, hkv, d, block_tokens, scale, window=window, softcap=softcap,
-                                scale_dtype=sdt, out_dtype=out_dtype, gate=None if gate is None else upload(gate))
+                                scale_dtype=sdt, out_dtype=out_dtype, gate=None if gate is None else upload(gate),
+                                visible_ends=None if visible_ends is None else upload(np.asarray(visible_ends, dtype=np.uint32)))
     torch.cuda.synchronize()
     kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, tables[0], block_tokens, 0, total, cols)
     vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, tables[0], block_tokens, 0, total, cols)
@@ -73,7 +74,8 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
             assert rc == 0
             parts.append(part)
         return out, np.concatenate(parts)
-    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
+    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap,
+                                        visible_ends=None if visible_ends is None else np.asarray(visible_ends, dtype=np.uint32))
     assert rc == 0
     if gate is not None:
         rc, want = O.sigmoid_gate(want, gate)
@@ -173,11 +175,17 @@ def test_prefill_query_and_key_magnitudes(q_exp, k_exp):
 def test_prefill_rejects_unsupported_shapes():
     from zllm_amd import capi, ops
 
-    z = torch.zeros((16, 64), dtype=torch.int8, device="cuda")
-    s = torch.zeros((16, 1), dtype=torch.int16, device="cuda")
-    q = torch.zeros((1, 64), dtype=torch.float32, device="cuda")
-    with pytest.raises(capi.ZllmAttnError, match="head_dim 128"):
-        ops.gqa_prefill_chunk(q, z, s, z, s, None, 0, 1, 1, 64, 16, 1.0)
+    z = torch.zeros((16, 96), dtype=torch.int8, device="cuda")
+    s = torch.zeros((16, 2), dtype=torch.int16, device="cuda")
+    q = torch.zeros((1, 96), dtype=torch.float32, device="cuda")
+    with pytest.raises(capi.ZllmAttnError, match="head_dim 64 / 128 / 256"):
+        ops.gqa_prefill_chunk(q, z, s, z, s, None, 0, 1, 1, 96, 16, 1.0)
+    with pytest.raises(capi.ZllmAttnError, match="128 / 256 over an f16 cache"):
+        ops.gqa_prefill_chunk(q, z, None, z, None, None, 0, 1, 1, 64, 16, 1.0, kv_format=capi.KV_F16)
+    table = torch.zeros(2, dtype=torch.int32, device="cuda")  # two pages of 16 tokens cannot hold 40 + 8 tokens
+    q8 = torch.zeros((8, 128), dtype=torch.float32, device="cuda")
+    with pytest.raises(capi.ZllmAttnError, match="cannot cover"):
+        ops.gqa_prefill_chunk(q8, z, s, z, s, table, 40, 1, 1, 128, 16, 1.0)
 
 
 def test_prefill_config5_full_size():
@@ -188,3 +196,92 @@ def test_prefill_config5_full_size():
     out, want = run_case(5, 50000, 2048, 64, 8, oracle_segments=segments)
     got = np.concatenate([out[r0:r0 + n].cpu().numpy() for r0, n in segments])
     print("config5 full", assert_attention_close(got, want, "config 5 full size"))
+
+
+# ---- explicit visible ends (multimodal blocks) --------------------------------------------------------------------
+
+def _block_ends(prefix, chunk, block):
+    """Rows of a visual block read to the end of their block: visible end of row r = end of r's block (absolute)."""
+    return [min(prefix + (r // block + 1) * block, prefix + chunk) for r in range(chunk)]
+
+
+@pytest.mark.parametrize("prefix,chunk,hq,hkv,block,window", [(0, 3, 2, 1, 3, 0), (200, 96, 16, 4, 24, 0), (1000, 300, 64, 8, 77, 0),
+                                                              (500, 130, 8, 2, 40, 64)])
+def test_prefill_visible_ends(prefix, chunk, hq, hkv, block, window):
+    """key_range_with_visible_end (src/attention/gqa.rs:65-68): a row sees up to max(its own position + 1, its visible
+    end), the left edge still follows its window.  The first case is the shape of the reference's visual-block vector
+    (src/kernel/cpu/gqa.rs:33-69: three rows that all see the whole block)."""
+    ends = _block_ends(prefix, chunk, block)
+    out, want = run_case(prefix + chunk + block, prefix, chunk, hq, hkv, window=window, visible_ends=ends)
+    assert_attention_close(out.cpu().numpy(), want, f"visible ends block={block}")
+    # not the causal result: the ends must have been used
+    _, causal = run_case(prefix + chunk + block, prefix, chunk, hq, hkv, window=window)
+    assert np.abs(causal - want).max() > 1e-3
+
+
+def test_prefill_visible_ends_reference_vector():
+    """The reference's own known answer (src/kernel/cpu/gqa.rs:33-69): zero queries, three rows that each see the
+    whole three-token block -> every row is the mean of the three values."""
+    from zllm_amd import capi, ops
+
+    d, bt = 128, 16
+    v = np.zeros((3, d), dtype=np.float32)
+    v[:, 0] = [3.0, 6.0, 9.0]  # mean 6 in every row: the [6, 6, 6] of the reference's test
+    k = np.zeros((3, d), dtype=np.float32)
+    planes = {n: np.zeros((bt, d if "codes" in n else d // 64), dtype=np.int8 if "codes" in n else np.uint16)
+              for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    table = np.array([0], dtype=np.uint32)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, k, planes["k_codes"], planes["k_scales"], table, 0, bt)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, planes["v_codes"], planes["v_scales"], table, 0, bt)
+    q = torch.zeros((3, d), dtype=torch.float32, device="cuda")
+    out = ops.gqa_prefill_chunk(q, upload(planes["k_codes"]), upload(planes["k_scales"]), upload(planes["v_codes"]), upload(planes["v_scales"]),
+                                upload(table), 0, 1, 1, d, bt, 1.0, visible_ends=upload(np.array([3, 3, 3], dtype=np.uint32)))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    np.testing.assert_allclose(got[:, 0], [6.0, 6.0, 6.0], rtol=2e-3)
+    assert (got[:, 1:] == 0).all()
+
+
+# ---- other geometries: every chunk row as one item of the split-KV decode kernels ------------------------------------
+
+@pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,block_tokens", [(64, 300, 70, 8, 2, 0, 16), (256, 500, 40, 16, 8, 0, 16),
+                                                                       (256, 700, 33, 4, 1, 128, 64), (64, 0, 50, 4, 4, 0, 4)])
+def test_prefill_head_dim_64_and_256(d, prefix, chunk, hq, hkv, window, block_tokens):
+    out, want = run_case(d + prefix, prefix, chunk, hq, hkv, window=window, d=d, block_tokens=block_tokens)
+    print("prefill d", d, assert_attention_close(out.cpu().numpy(), want, f"head_dim={d}"))
+
+
+def test_prefill_head_dim_256_visible_ends_gate_and_bf16_out():
+    ends = _block_ends(100, 48, 16)
+    out, want = run_case(256, 100, 48, 8, 2, d=256, visible_ends=ends, out_dtype=torch.bfloat16)
+    got = out.float().cpu().numpy()
+    assert np.abs(got - want).max() <= 2e-3 + np.abs(want).max() * 2.0 ** -8
+    out, want = run_case(257, 100, 48, 8, 2, d=256, gate_cols=1)
+    assert_attention_close(out.cpu().numpy(), want, "head_dim 256 gated")
+
+
+@pytest.mark.parametrize("d,prefix,chunk,window,softcap", [(256, 900, 64, 0, 50.0), (256, 1500, 40, 1024, 50.0), (128, 300, 100, 0, 0.0)])
+def test_prefill_f16_kv(d, prefix, chunk, window, softcap):
+    """Chunked prefill over an f16 cache (the config-3 model family prefills too): rows appended as f16, then attended."""
+    from zllm_amd import capi, ops
+
+    hq, hkv, bt = 16, 8, 16
+    rng = np.random.default_rng(d + prefix)
+    total = prefix + chunk
+    cols = hkv * d
+    tables, pool_blocks = draw_tables(rng, [total], bt)
+    k = rng.standard_normal((total, cols)).astype(np.float32)
+    v = rng.standard_normal((total, cols)).astype(np.float32)
+    planes = {"k": np.zeros((pool_blocks * bt, cols), dtype=np.uint16), "v": np.zeros((pool_blocks * bt, cols), dtype=np.uint16)}
+    O.half_append_paged(1, k, planes["k"], tables[0], 0, bt)
+    O.half_append_paged(1, v, planes["v"], tables[0], 0, bt)
+    q = rng.standard_normal((chunk, hq * d)).astype(np.float32)
+    scale = 1.0 / np.sqrt(d)
+    out = ops.gqa_prefill_chunk(upload(q), upload(planes["k"]), None, upload(planes["v"]), None, upload(tables[0]), prefix, hq, hkv, d, bt,
+                                scale, window=window, softcap=softcap, kv_format=capi.KV_F16)
+    torch.cuda.synchronize()
+    kd = O.gather_dequant_rows(O.FMT_F16, planes["k"], None, 0, tables[0], bt, 0, total, cols)
+    vd = O.gather_dequant_rows(O.FMT_F16, planes["v"], None, 0, tables[0], bt, 0, total, cols)
+    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
+    assert rc == 0
+    print("prefill f16", d, assert_attention_close(out.cpu().numpy(), want, f"f16 KV prefill d={d}"))

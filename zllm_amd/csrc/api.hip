@@ -659,7 +659,8 @@ uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* a)
 }
 
 // The decode call over a workspace that is either the caller's or the library's static array.
-static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint64_t workspace_bytes, zllm_stream_t stream)
+static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint64_t workspace_bytes, zllm_stream_t stream,
+                           bool table_shared = false, int out_dtype = ZLLM_DTYPE_F32)
 {
     if (a->q == nullptr || a->k_plane == nullptr || a->v_plane == nullptr || a->kv_lens == nullptr || a->out == nullptr ||
         workspace == nullptr || (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
@@ -698,6 +699,8 @@ static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint6
     p.head_dim = a->head_dim;
     p.group = a->num_heads / a->num_kv_heads;
     p.table_stride = a->table_stride;
+    p.table_shared = table_shared ? 1u : 0u;
+    p.out_dtype = out_dtype;
     p.block_tokens = a->block_tokens;
     p.block_shift = shift_of(a->block_tokens);
     p.ring_capacity = a->ring_capacity;
@@ -834,14 +837,21 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     if (a->rows == 0 || a->num_heads == 0 || a->num_kv_heads == 0 || a->num_heads % a->num_kv_heads != 0) {
         return fail(-1, "GQA prefill: invalid shape rows=%u heads=%u/%u", a->rows, a->num_heads, a->num_kv_heads);
     }
-    if (a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64) {
-        return fail(-1, "GQA prefill: this build handles head_dim 128 over a Q8g64 cache (got dim=%u format=%d)", a->head_dim, a->kv_format);
+    // head dimensions of the reference's block attention that a Q8g64 group divides (tensor/attention.rs:727-745)
+    if (!valid_head_dim(a->head_dim) || (a->kv_format != ZLLM_KV_Q8G64 && a->kv_format != ZLLM_KV_F16) ||
+        (a->kv_format == ZLLM_KV_F16 && a->head_dim == 64)) {
+        return fail(-1, "GQA prefill: head_dim 64 / 128 / 256 over a Q8g64 cache or 128 / 256 over an f16 cache (got dim=%u format=%d)",
+                    a->head_dim, a->kv_format);
     }
     if (a->num_heads / a->num_kv_heads > 256) {
         return fail(-1, "GQA prefill: at most 256 query heads per KV head");
     }
-    if (a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
+    if (a->kv_format == ZLLM_KV_Q8G64 && a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
         return fail(-1, "GQA prefill: Q8g64 scales must be bf16 or f16 (got %d)", a->scale_dtype);
+    }
+    if (a->table != nullptr && a->table_stride != 0 && (uint64_t)a->table_stride * a->block_tokens < (uint64_t)a->position + a->rows) {
+        return fail(-1, "GQA prefill: table_stride=%u pages of %u tokens cannot cover position + rows = %llu", a->table_stride,
+                    a->block_tokens, (unsigned long long)a->position + a->rows);
     }
     if (a->block_tokens == 0 || (uint64_t)a->position + a->rows > 0xffffffffull) {
         return fail(-1, "GQA prefill: block_tokens must be non-zero and position + rows fit u32");
@@ -855,11 +865,58 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     return 0;
 }
 
+// head_dim 128 over Q8g64 runs the matrix-core chunk kernel, which keeps all of its state on chip.  Every other
+// geometry (head_dim 64 / 256, f16 KV) runs each row of the chunk as one item of the split-KV decode kernels: row r is a
+// sequence of position + r + 1 tokens over the same block table.  That route re-reads the KV bytes per row, so it is
+// bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and the split records.
+static bool prefill_rows_as_decode_items(const zllm_gqa_prefill_args* a)
+{
+    return a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64;
+}
+
+static void prefill_decode_args(const zllm_gqa_prefill_args* a, zllm_gqa_decode_args* d)
+{
+    memset(d, 0, sizeof(*d));
+    d->q = a->q;
+    d->k_plane = a->k_plane;
+    d->k_scales = a->k_scales;
+    d->v_plane = a->v_plane;
+    d->v_scales = a->v_scales;
+    d->tables = a->table;
+    d->batch = a->rows;
+    d->num_heads = a->num_heads;
+    d->num_kv_heads = a->num_kv_heads;
+    d->head_dim = a->head_dim;
+    d->max_kv_len = a->position + a->rows;
+    const uint64_t pages = ((uint64_t)a->position + a->rows + a->block_tokens - 1) / a->block_tokens;
+    d->table_stride = a->table_stride != 0 ? a->table_stride : (uint32_t)pages;
+    // sum of the rows' visible lengths (an upper bound when rows carry explicit visible ends): tunes the split size
+    uint64_t total = 0;
+    for (uint32_t r = 0; r < a->rows; ++r) {
+        const uint64_t end = (uint64_t)a->position + r + 1;
+        total += a->visible_ends != nullptr ? (uint64_t)a->position + a->rows : (a->window != 0 && end > a->window ? a->window : end);
+    }
+    d->total_kv_tokens = total > 0xffffffffull ? 0u : (uint32_t)total;
+    d->block_tokens = a->block_tokens;
+    d->score_scale = a->score_scale;
+    d->softcap = a->softcap;
+    d->kv_format = a->kv_format;
+    d->scale_dtype = a->scale_dtype;
+    d->q_dtype = a->q_dtype;
+    d->gate = a->gate;
+    d->gate_cols = a->gate_cols;
+    d->gate_dtype = a->gate_dtype;
+}
+
 uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* a)
 {
-    /* the prefill kernel keeps all of its state on chip */
-    (void)validate_gqa_prefill(a);
-    return 0;
+    if (validate_gqa_prefill(a) != 0 || !prefill_rows_as_decode_items(a)) {
+        return 0; /* the chunk kernel keeps all of its state on chip */
+    }
+    zllm_gqa_decode_args d;
+    prefill_decode_args(a, &d);
+    const uint64_t records = zllm_attn_gqa_decode_workspace_bytes(&d);
+    return records == 0 ? 0 : align_up((uint64_t)a->rows * 8, 256) + records;
 }
 
 int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t stream)
@@ -868,8 +925,8 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
     if (rc != 0) {
         return rc;
     }
-    if (a->q == nullptr || a->k_plane == nullptr || a->k_scales == nullptr || a->v_plane == nullptr || a->v_scales == nullptr ||
-        a->out == nullptr) {
+    if (a->q == nullptr || a->k_plane == nullptr || a->v_plane == nullptr || a->out == nullptr ||
+        (a->kv_format == ZLLM_KV_Q8G64 && (a->k_scales == nullptr || a->v_scales == nullptr))) {
         return fail(-1, "GQA prefill: null pointer");
     }
     // the kernel reads codes as 8-byte vectors and scales as 4-byte words, and stores the output as 16- or 8-byte vectors
@@ -877,8 +934,37 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
         (((uintptr_t)a->k_scales | (uintptr_t)a->v_scales) & 3u) != 0) {
         return fail(-1, "GQA prefill: q, cache planes and out must be 16-byte aligned (scale planes 4-byte)");
     }
+    if (a->gate != nullptr &&
+        ((a->gate_cols != 1 && a->gate_cols != a->num_heads * a->head_dim) || (a->gate_dtype != ZLLM_DTYPE_F32 && a->gate_dtype != ZLLM_DTYPE_BF16))) {
+        return fail(-1, "GQA prefill: gate_cols=%u must be 1 or %u, gate_dtype f32 or bf16", a->gate_cols, a->num_heads * a->head_dim);
+    }
+    if (prefill_rows_as_decode_items(a)) {
+        zllm_gqa_decode_args d;
+        prefill_decode_args(a, &d);
+        if (validate_gqa_decode(&d) != 0) {
+            return -1;
+        }
+        const uint64_t need = zllm_attn_gqa_prefill_workspace_bytes(a);
+        if (a->workspace == nullptr || a->workspace_bytes < need || ((uintptr_t)a->workspace & 15u) != 0) {
+            return fail(-1, "GQA prefill: this geometry needs a 16-byte aligned workspace of %llu bytes (got %llu)", (unsigned long long)need,
+                        (unsigned long long)a->workspace_bytes);
+        }
+        uint32_t* lens = (uint32_t*)a->workspace;
+        uint32_t* first = lens + a->rows;
+        int rc2 = hip_status(zllm::launch_prefill_row_ranges(lens, first, a->visible_ends, a->rows, a->position, a->window, (hipStream_t)stream),
+                             "GQA prefill row ranges launch");
+        if (rc2 != 0) {
+            return rc2;
+        }
+        d.kv_lens = lens;
+        d.first_visible = first;
+        d.out = (float*)a->out;
+        const uint64_t head_bytes = align_up((uint64_t)a->rows * 8, 256);
+        return gqa_decode_over(&d, (char*)a->workspace + head_bytes, a->workspace_bytes - head_bytes, stream, /*table_shared=*/true, a->out_dtype);
+    }
     zllm::GqaPrefillParams p;
     memset(&p, 0, sizeof(p));
+    p.visible_ends = a->visible_ends;
     p.q = a->q;
     p.k_plane = (const unsigned char*)a->k_plane;
     p.k_scales = (const unsigned char*)a->k_scales;

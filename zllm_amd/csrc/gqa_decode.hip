@@ -424,7 +424,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     float q_step; // value of one fixed-point unit of this lane's head
     load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
 
-    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int* table = p.tables + (p.table_shared ? 0 : (size_t)b * p.table_stride);
     const unsigned int k_row = p.num_kv_heads * D;           // bytes per cache row (codes)
     const unsigned int s_row = p.num_kv_heads * G * 2u;      // bytes per scale row
     const unsigned char* k_base = p.k_plane + (size_t)kvh * D;
@@ -683,7 +683,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
-    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int* table = p.tables + (p.table_shared ? 0 : (size_t)b * p.table_stride);
     const unsigned int k_row = p.num_kv_heads * D;
     const unsigned int s_row = p.num_kv_heads * G * 2u;
     const unsigned char* k_base = p.k_plane + (size_t)kvh * D;
@@ -966,7 +966,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
         }
     }
 
-    const unsigned int* table = p.tables + (size_t)b * p.table_stride;
+    const unsigned int* table = p.tables + (p.table_shared ? 0 : (size_t)b * p.table_stride);
     const unsigned int k_row = p.num_kv_heads * D * 2u; // bytes per cache row
     const unsigned char* k_base = p.k_plane + (size_t)kvh * D * 2u;
     const unsigned char* v_base = p.v_plane + (size_t)kvh * D * 2u;
@@ -1236,8 +1236,36 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
                 result[e] = gated(result[e], p.gate, p.gate_cols, p.gate_dtype, b, head * p.head_dim + quad * 4u + e);
             }
         }
-        *(f32x4*)(p.out + ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u) = result;
+        const size_t at = ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u;
+        if (p.out_dtype == 0) {
+            *(f32x4*)(p.out + at) = result;
+        } else if (p.out_dtype == 1) {
+            *(u32x2*)((unsigned short*)p.out + at) = u32x2{pack_bf16_rne(result[0], result[1]), pack_bf16_rne(result[2], result[3])};
+        } else {
+            *(u32x2*)((unsigned short*)p.out + at) = u32x2{(unsigned int)f32_to_f16_bits(result[0]) | ((unsigned int)f32_to_f16_bits(result[1]) << 16),
+                                                            (unsigned int)f32_to_f16_bits(result[2]) | ((unsigned int)f32_to_f16_bits(result[3]) << 16)};
+        }
     }
+}
+
+// Visible ranges of the rows of a prefill chunk, for the route that runs every row as one item of the split-KV
+// decode kernels: lens[r] = end and first[r] = start of key_range(position + r, position + rows), or of
+// key_range_with_visible_end when the row carries an explicit end (src/attention/gqa.rs:54-68).
+__global__ __launch_bounds__(256) void prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends,
+                                                          unsigned int rows, unsigned int position, unsigned int window)
+{
+    const unsigned int r = blockIdx.x * 256u + threadIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    const unsigned int pos = position + r;
+    unsigned int end = pos + 1u;
+    const unsigned int start = (window != 0 && end > window) ? end - window : 0u;
+    if (visible_ends != nullptr) {
+        end = min(max(end, visible_ends[r]), position + rows);
+    }
+    lens[r] = end;
+    first[r] = min(start, end);
 }
 
 template <int D, int SDT>
@@ -1328,6 +1356,13 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_
         return err;
     }
     return launch_split_merge(p, stream);
+}
+
+hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, unsigned int rows,
+                                     unsigned int position, unsigned int window, hipStream_t stream)
+{
+    prefill_row_ranges<<<dim3((rows + 255u) / 256u), dim3(256), 0, stream>>>(lens, first, visible_ends, rows, position, window);
+    return hipGetLastError();
 }
 
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)

@@ -106,9 +106,15 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const unsigned int row0 = blockIdx.x * rows_per_wg;
     const unsigned int cols_used = rows_per_wg * p.group;
 
-    // visible token range of the workgroup: union over its rows of key_range(position + row, kv_end)
+    // visible token range of the workgroup: union over its rows of key_range(position + row, kv_end), or of
+    // key_range_with_visible_end when rows carry an explicit visible end (src/attention/gqa.rs:65-68)
     const unsigned int last_row = min(row0 + rows_per_wg, p.rows) - 1u;
-    const unsigned int t_end = p.position + last_row + 1u;
+    unsigned int t_end = p.position + last_row + 1u;
+    if (p.visible_ends != nullptr) {
+        for (unsigned int r = row0; r <= last_row; ++r) { // uniform over the workgroup: scalar loads
+            t_end = max(t_end, min(p.visible_ends[r], p.position + p.rows));
+        }
+    }
     unsigned int t_begin = 0;
     if (p.window != 0) {
         const unsigned int first_pos = p.position + row0 + 1u;
@@ -255,7 +261,11 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         run_sum[ct] = 0.0f;
         ref_shift[ct] = kPBias;
         const unsigned int pos = p.position + col_row[ct];
-        vis_hi[ct] = col_valid[ct] ? pos + 1u : 0u;
+        unsigned int hi = pos + 1u;
+        if (p.visible_ends != nullptr && col_valid[ct]) { // a row may read past itself, up to the end of the chunk
+            hi = min(max(hi, p.visible_ends[col_row[ct]]), p.position + p.rows);
+        }
+        vis_hi[ct] = col_valid[ct] ? hi : 0u;
         vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
     }
 

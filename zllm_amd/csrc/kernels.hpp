@@ -100,6 +100,8 @@ struct GqaDecodeParams {
     // split merge only: query rows per sequence (0 = 1).  Record row v belongs to sequence v / query_rows and sees
     // kv_lens[sequence] - (query_rows - 1 - v % query_rows) tokens; `batch` then counts record rows.
     unsigned int query_rows;
+    unsigned int table_shared; // 1: every item reads the one table at `tables` (rows of a prefill chunk); table_stride still bounds it
+    int out_dtype;             // split merge: element type of `out` (0 f32, 1 bf16, 2 f16)
 };
 
 struct GqaPrefillParams {
@@ -118,6 +120,7 @@ struct GqaPrefillParams {
     const void* gate; // optional sigmoid output gate [rows][gate_cols]
     unsigned int gate_cols;
     int gate_dtype;
+    const unsigned int* visible_ends; // optional [rows]: row r reads up to max(position + r + 1, visible_ends[r])
 };
 
 struct MlaDecodeParams {
@@ -164,5 +167,8 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
 // LSE combine of split records: uses kv_lens, first_visible, partial, stats, out, batch, num_heads,
 // head_dim, chunk_tokens, max_chunks of the parameter block.
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream);
+// lens[r], first[r] = visible range of row r of a prefill chunk (window 0 = full causal; visible_ends optional)
+hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, unsigned int rows,
+                                     unsigned int position, unsigned int window, hipStream_t stream);
 
 } // namespace zllm
