@@ -274,6 +274,15 @@ typedef struct zllm_gqa_decode_args {
     int gate_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
 } zllm_gqa_decode_args;
 ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* args);
+/* The split plan the call would run with: every sequence's visible range is cut into at most *max_chunks splits of at
+ * most *chunk_tokens tokens (a multiple of 32), so max_chunks * chunk_tokens >= max_kv_len.  It is fixed by the host
+ * arguments alone (the tile / split geometry of try_gqa_decode_cached_f32,
+ * src/kernel/rocm/hip/tensor/attention.rs:1031-1046): a sequence whose kv_lens[b] on the device has grown past
+ * max_kv_len -- a recorded graph replayed too long -- is read up to max_chunks * chunk_tokens tokens only.  A caller
+ * that combines ZLLM_STAGE_PARTIAL records itself indexes them with max_chunks:
+ * partial f32 [batch][max_chunks][num_heads][head_dim] at the start of the workspace, then (max, sum) f32 pairs
+ * [batch][max_chunks][num_heads][2] at the next 256-byte boundary.  0 ok, negative = invalid arguments. */
+ZLLM_API int zllm_attn_gqa_decode_split_plan(const zllm_gqa_decode_args* args, uint32_t* chunk_tokens, uint32_t* max_chunks);
 ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);
 
 /* zllm_attn_gqa_decode for callers that cannot allocate device memory (code under HIP graph capture, tight

@@ -87,7 +87,7 @@ static void compare(const std::vector<float>& got, const std::vector<float>& wan
 }
 
 // ---------------------------------------------------------------------------------------------- GQA
-static void test_gqa(const RocmContext& ctx, CausalWindow window, const char* label)
+static void test_gqa(const RocmContext& ctx, CausalWindow window, const char* label, TablePolicy policy)
 {
     std::mt19937 rng(7);
     GqaSpec spec;
@@ -98,13 +98,16 @@ static void test_gqa(const RocmContext& ctx, CausalWindow window, const char* la
     spec.score_scale = 1.0f / sqrtf(128.0f);
     const size_t kv_cols = spec.num_kv_heads * spec.head_dim, q_cols = spec.num_heads * spec.head_dim;
     const size_t block = 16, max_tokens = 1024;
-    auto cache_r = RocmKvCache::new_gqa(2, spec.num_kv_heads, spec.head_dim, block, max_tokens);
+    auto cache_r = RocmKvCache::new_gqa(2, spec.num_kv_heads, spec.head_dim, block, max_tokens, policy);
     CHECK(cache_r.is_ok(), "cache: %s", cache_r.is_err() ? cache_r.unwrap_err().to_string().c_str() : "");
     if (cache_r.is_err()) {
         return;
     }
     RocmKvCache cache = cache_r.unwrap();
     const size_t pool_rows = cache.block_table().size() * block;
+    // the identity table commits rows as they are needed, the scrambled one commits its pool up front
+    CHECK(cache.committed_rows(1) == (policy == TablePolicy::Identity ? 0 : pool_rows), "rows committed at creation: %zu", cache.committed_rows(1));
+    size_t committed_want = 0;
     // the oracle's copy of layer 1's planes, filled by the oracle's quantizer through the same table
     std::vector<int8_t> k_codes(pool_rows * kv_cols), v_codes(pool_rows * kv_cols);
     std::vector<uint16_t> k_scales(pool_rows * kv_cols / 64), v_scales(pool_rows * kv_cols / 64);
@@ -140,6 +143,12 @@ static void test_gqa(const RocmContext& ctx, CausalWindow window, const char* la
         compare(got.unwrap(), want, what);
         position = total;
         CHECK(cache.len(layer) == position, "cache length %zu vs %zu", cache.len(layer), position);
+        if (policy == TablePolicy::Identity) {
+            // grow-by-doubling in 64-row multiples (src/backend/rocm/mod.rs:303-313), whole pages
+            committed_want = committed_cache_rows(committed_want, total, pool_rows).unwrap();
+            CHECK(cache.committed_rows(layer) == committed_want, "committed rows %zu, rule says %zu", cache.committed_rows(layer), committed_want);
+            CHECK(cache.committed_rows(0) == 0, "a layer nothing was appended to holds no rows");
+        }
     }
     // error behaviour of the reference's body (attention.rs:2213-2229)
     {
@@ -171,7 +180,7 @@ static void test_mla(const RocmContext& ctx)
     spec.q_lora_rank = 1536;
     CHECK(!spec.validate().has_value(), "spec must validate");
     const size_t block = 64, max_tokens = 700, layer = 0;
-    auto cache_r = RocmKvCache::new_mla(1, 512, 64, block, max_tokens);
+    auto cache_r = RocmKvCache::new_mla(1, 512, 64, block, max_tokens, TablePolicy::Scrambled);
     CHECK(cache_r.is_ok(), "cache");
     if (cache_r.is_err()) {
         return;
@@ -335,6 +344,221 @@ static void test_mla(const RocmContext& ctx)
     CHECK(bad.validate().has_value(), "inconsistent head dimensions must not validate");
 }
 
+
+// ---------------------------------------------------------------------------------------------- growth rule, ring, shared KV, visible ends
+static void test_growth_rule()
+{
+    struct Case {
+        size_t current, required, limit, want;
+    };
+    const Case cases[] = {{0, 1, 1000, 64}, {64, 65, 1000, 128}, {128, 129, 200, 200}, {64, 300, 1000, 320}, {100, 50, 1000, 100},
+                          {0, 1000, 1000, 1000}, {512, 513, 8192, 1024}};
+    for (const Case& c : cases) {
+        auto rows = committed_cache_rows(c.current, c.required, c.limit);
+        CHECK(rows.is_ok() && rows.unwrap() == c.want, "committed_cache_rows(%zu, %zu, %zu) = %zu, want %zu", c.current, c.required, c.limit,
+              rows.is_ok() ? rows.unwrap() : (size_t)0, c.want);
+    }
+    CHECK(committed_cache_rows(0, 5, 3).is_err() && committed_cache_rows(0, 0, 3).is_err(), "required outside (0, limit] must be refused");
+}
+
+// A sliding-window layer that keeps a ring of `window` rows (retain_full_cache == false): a chunk longer than the ring at
+// position 0, then decode steps that wrap the ring; the oracle keeps every row and applies the window.
+static void test_gqa_ring(const RocmContext& ctx)
+{
+    std::mt19937 rng(23);
+    GqaSpec spec;
+    spec.num_heads = 8;
+    spec.num_kv_heads = 2;
+    spec.head_dim = 128;
+    spec.window = CausalWindow::Sliding(96);
+    spec.score_scale = 1.0f / sqrtf(128.0f);
+    const size_t kv_cols = spec.num_kv_heads * spec.head_dim, q_cols = spec.num_heads * spec.head_dim;
+    const size_t block = 16, max_tokens = 2048, layer = 0;
+    auto cache_r = RocmKvCache::new_gqa(1, spec.num_kv_heads, spec.head_dim, block, max_tokens);
+    CHECK(cache_r.is_ok(), "ring cache");
+    if (cache_r.is_err()) {
+        return;
+    }
+    RocmKvCache cache = cache_r.unwrap();
+    std::vector<float> all_k, all_v; // the oracle's history: raw rows, quantized through an identity table below
+    size_t position = 0;
+    const size_t chunks[] = {300, 1, 1, 1, 1, 1};
+    for (size_t rows : chunks) {
+        const auto q = randn(rng, rows * q_cols, true);
+        const auto k = randn(rng, rows * kv_cols, false);
+        const auto v = randn(rng, rows * kv_cols, false);
+        auto out = ctx.gqa_prefill_attention_cached(cache, layer, position, ctx.tensor_from_f32(q, rows, q_cols, DType::BF16).unwrap(),
+                                                    ctx.tensor_from_f32(k, rows, kv_cols).unwrap(), ctx.tensor_from_f32(v, rows, kv_cols).unwrap(), spec,
+                                                    false);
+        CHECK(out.is_ok(), "ring rows=%zu: %s", rows, out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_err()) {
+            return;
+        }
+        all_k.insert(all_k.end(), k.begin(), k.end());
+        all_v.insert(all_v.end(), v.begin(), v.end());
+        const size_t total = position + rows;
+        std::vector<int8_t> kc(total * kv_cols), vc(total * kv_cols);
+        std::vector<uint16_t> ks(total * kv_cols / 64), vs(total * kv_cols / 64);
+        zo_q8g64_append_paged(1, all_k.data(), kc.data(), ks.data(), nullptr, 0, total, kv_cols, 64, block, 0);
+        zo_q8g64_append_paged(1, all_v.data(), vc.data(), vs.data(), nullptr, 0, total, kv_cols, 64, block, 0);
+        std::vector<float> kd(total * kv_cols), vd(total * kv_cols), want(rows * q_cols);
+        zo_gather_dequant_rows(0, kc.data(), ks.data(), 1, nullptr, block, 0, 0, total, kv_cols, 64, kd.data());
+        zo_gather_dequant_rows(0, vc.data(), vs.data(), 1, nullptr, block, 0, 0, total, kv_cols, 64, vd.data());
+        const int rc = zo_gqa_prefill_at_visible_f32(q.data(), kd.data(), vd.data(), rows, 0, total, position, spec.num_heads, spec.num_kv_heads,
+                                                     spec.head_dim, 96, spec.score_scale, 0.0f, nullptr, want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        char what[128];
+        snprintf(what, sizeof(what), "gqa_prefill_attention_cached ring(96) position=%zu rows=%zu", position, rows);
+        compare(ctx.tensor_to_f32(out.unwrap()).unwrap(), want, what);
+        position = total;
+    }
+    CHECK(cache.ring_capacity(layer) == 96 && cache.committed_rows(layer) <= 128, "ring of 96 rows in %zu committed rows", cache.committed_rows(layer));
+    // a multi-token chunk at a non-zero position of a draining sliding layer is refused, as on the reference's CPU backend
+    const auto q2 = randn(rng, 2 * q_cols, true);
+    const auto k2 = randn(rng, 2 * kv_cols, false);
+    auto refused = ctx.gqa_prefill_attention_cached(cache, layer, position, ctx.tensor_from_f32(q2, 2, q_cols).unwrap(),
+                                                    ctx.tensor_from_f32(k2, 2, kv_cols).unwrap(), ctx.tensor_from_f32(k2, 2, kv_cols).unwrap(), spec, false);
+    CHECK(refused.is_err() && cache.len(layer) == position, "multi-token chunk on a wrapped ring must be refused and leave the length alone");
+}
+
+// gqa_prefill_attention_cached_from (a layer that shares another layer's K/V) and _visible (explicit visible ends)
+static void test_gqa_shared_and_visible(const RocmContext& ctx)
+{
+    std::mt19937 rng(29);
+    GqaSpec spec;
+    spec.num_heads = 8;
+    spec.num_kv_heads = 2;
+    spec.head_dim = 128;
+    spec.window = CausalWindow::Full();
+    spec.score_scale = 1.0f / sqrtf(128.0f);
+    const size_t kv_cols = spec.num_kv_heads * spec.head_dim, q_cols = spec.num_heads * spec.head_dim;
+    const size_t block = 16, prefix = 150, rows = 48, total = prefix + rows;
+    auto cache_r = RocmKvCache::new_gqa(2, spec.num_kv_heads, spec.head_dim, block, 512, TablePolicy::Scrambled);
+    CHECK(cache_r.is_ok(), "cache");
+    if (cache_r.is_err()) {
+        return;
+    }
+    RocmKvCache cache = cache_r.unwrap();
+    const auto k = randn(rng, total * kv_cols, false);
+    const auto v = randn(rng, total * kv_cols, false);
+    const auto q0 = randn(rng, prefix * q_cols, true);
+    const auto q = randn(rng, rows * q_cols, true);
+    std::vector<float> k_head(k.begin(), k.begin() + prefix * kv_cols), v_head(v.begin(), v.begin() + prefix * kv_cols);
+    std::vector<float> k_tail(k.begin() + prefix * kv_cols, k.end()), v_tail(v.begin() + prefix * kv_cols, v.end());
+    auto first = ctx.gqa_prefill_attention_cached(cache, 1, 0, ctx.tensor_from_f32(q0, prefix, q_cols).unwrap(),
+                                                  ctx.tensor_from_f32(k_head, prefix, kv_cols).unwrap(), ctx.tensor_from_f32(v_head, prefix, kv_cols).unwrap(),
+                                                  spec, true);
+    CHECK(first.is_ok(), "prefix");
+    // rows of a visual block read to the end of their 16-row block
+    std::vector<uint32_t> ends(rows);
+    for (size_t r = 0; r < rows; ++r) {
+        ends[r] = (uint32_t)std::min(prefix + (r / 16 + 1) * 16, total);
+    }
+    auto qt = ctx.tensor_from_f32(q, rows, q_cols);
+    auto seen = ctx.gqa_prefill_attention_cached_visible(cache, 1, prefix, qt.unwrap(), ctx.tensor_from_f32(k_tail, rows, kv_cols).unwrap(),
+                                                         ctx.tensor_from_f32(v_tail, rows, kv_cols).unwrap(), spec, ends, true);
+    CHECK(seen.is_ok(), "visible: %s", seen.is_err() ? seen.unwrap_err().to_string().c_str() : "");
+    std::vector<int8_t> kc(total * kv_cols), vc(total * kv_cols);
+    std::vector<uint16_t> ks(total * kv_cols / 64), vs(total * kv_cols / 64);
+    zo_q8g64_append_paged(1, k.data(), kc.data(), ks.data(), nullptr, 0, total, kv_cols, 64, block, 0);
+    zo_q8g64_append_paged(1, v.data(), vc.data(), vs.data(), nullptr, 0, total, kv_cols, 64, block, 0);
+    std::vector<float> kd(total * kv_cols), vd(total * kv_cols), want(rows * q_cols);
+    zo_gather_dequant_rows(0, kc.data(), ks.data(), 1, nullptr, block, 0, 0, total, kv_cols, 64, kd.data());
+    zo_gather_dequant_rows(0, vc.data(), vs.data(), 1, nullptr, block, 0, 0, total, kv_cols, 64, vd.data());
+    int rc = zo_gqa_prefill_at_visible_f32(q.data(), kd.data(), vd.data(), rows, 0, total, prefix, spec.num_heads, spec.num_kv_heads, spec.head_dim, 0,
+                                           spec.score_scale, 0.0f, ends.data(), want.data());
+    CHECK(rc == 0, "oracle rc %d", rc);
+    if (seen.is_ok()) {
+        compare(ctx.tensor_to_f32(seen.unwrap()).unwrap(), want, "gqa_prefill_attention_cached_visible, 16-row blocks");
+    }
+    // layer 0 shares layer 1's K/V: the same chunk, causal, nothing appended
+    auto shared = ctx.gqa_prefill_attention_cached_from(cache, 1, prefix, qt.unwrap(), spec);
+    CHECK(shared.is_ok(), "cached_from: %s", shared.is_err() ? shared.unwrap_err().to_string().c_str() : "");
+    rc = zo_gqa_prefill_at_visible_f32(q.data(), kd.data(), vd.data(), rows, 0, total, prefix, spec.num_heads, spec.num_kv_heads, spec.head_dim, 0,
+                                       spec.score_scale, 0.0f, nullptr, want.data());
+    CHECK(rc == 0, "oracle rc %d", rc);
+    if (shared.is_ok()) {
+        compare(ctx.tensor_to_f32(shared.unwrap()).unwrap(), want, "gqa_prefill_attention_cached_from layer 1");
+    }
+    CHECK(cache.len(0) == 0 && cache.len(1) == total, "shared-KV attention must not append");
+    CHECK(ctx.gqa_prefill_attention_cached_from(cache, 1, prefix + 1, qt.unwrap(), spec).is_err(), "a source layer shorter than position + rows must be refused");
+    CHECK(ctx.gqa_prefill_attention_cached_from(cache, 7, prefix, qt.unwrap(), spec).is_err(), "a source layer outside the cache must be refused");
+}
+
+// MlaPrefillBackend::mla_prefill_attention: two chunks, each appended and attended causally; bf16 rows for a chunk
+static void test_mla_prefill(const RocmContext& ctx)
+{
+    std::mt19937 rng(31);
+    MlaSpec spec;
+    spec.kv_lora_rank = 512;
+    spec.qk_rope_head_dim = 64;
+    spec.num_heads = 16;
+    spec.q_projection_size = spec.num_heads * 192;
+    spec.kv_projection_size = spec.num_heads * 256;
+    spec.q_lora_rank = 1536;
+    const size_t block = 64, layer = 0;
+    auto cache_r = RocmKvCache::new_mla(1, 512, 64, block, 1024);
+    CHECK(cache_r.is_ok(), "cache");
+    if (cache_r.is_err()) {
+        return;
+    }
+    RocmKvCache cache = cache_r.unwrap();
+    std::vector<float> kv_b = randn(rng, spec.kv_projection_size * 512, true);
+    for (auto& w : kv_b) {
+        w = zo_bf16_to_f32(zo_f32_to_bf16(w * 0.05f));
+    }
+    auto weight = ctx.prepare_mla_kv_b(kv_b, spec.kv_projection_size, 512);
+    std::vector<float> all_latent, all_rope;
+    size_t position = 0;
+    const size_t chunks[] = {90, 37, 1};
+    for (size_t rows : chunks) {
+        const auto q = randn(rng, rows * spec.q_projection_size, true);
+        const auto latent = randn(rng, rows * 512, false);
+        const auto rope = randn(rng, rows * 64, false);
+        auto out = ctx.mla_prefill_attention(ctx.tensor_from_f32(q, rows, spec.q_projection_size, DType::BF16).unwrap(),
+                                             ctx.tensor_from_f32(latent, rows, 512).unwrap(), ctx.tensor_from_f32(rope, rows, 64).unwrap(), weight.unwrap(),
+                                             &cache, layer, spec);
+        CHECK(out.is_ok(), "mla_prefill_attention rows=%zu: %s", rows, out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_err()) {
+            return;
+        }
+        CHECK(out.unwrap().dtype == (rows > 1 ? DType::BF16 : DType::F32), "a chunk comes back as bf16, one row as f32");
+        all_latent.insert(all_latent.end(), latent.begin(), latent.end());
+        all_rope.insert(all_rope.end(), rope.begin(), rope.end());
+        const size_t total = position + rows;
+        std::vector<int8_t> codes(total * 512);
+        std::vector<uint16_t> scales(total * 8), rope_bits(total * 64), q_bits(q.size());
+        zo_q8g64_append_paged(0, all_latent.data(), codes.data(), scales.data(), nullptr, 0, total, 512, 64, block, 0);
+        zo_half_append_paged(0, all_rope.data(), rope_bits.data(), nullptr, 0, total, 64, block, 0);
+        for (size_t i = 0; i < q.size(); ++i) {
+            q_bits[i] = zo_f32_to_bf16(q[i]);
+        }
+        zo_mla_spec zs = {512, 64, spec.q_projection_size, spec.kv_projection_size, spec.num_heads};
+        std::vector<float> want(rows * spec.num_heads * spec.value_dim());
+        const int rc = zo_mla_absorbed_q8_history(&zs, q_bits.data(), rows, position, (const uint8_t*)codes.data(), scales.data(), 64, rope_bits.data(),
+                                                  total, kv_b.data(), nullptr, 0, nullptr, want.data(), nullptr);
+        CHECK(rc == 0, "oracle rc %d", rc);
+        auto got = ctx.tensor_to_f32(out.unwrap()).unwrap();
+        if (rows > 1) { // bf16 rows: within one bf16 step of the oracle's unrounded value, then the attention bound
+            double worst = 0;
+            for (size_t i = 0; i < got.size(); ++i) {
+                worst = fmax(worst, fabs((double)got[i] - want[i]) - fabs((double)want[i]) * 0.0078125);
+            }
+            printf("%-58s worst excess over a bf16 step %.3e\n", "mla_prefill_attention chunk (bf16 rows)", worst);
+            CHECK(worst <= 2e-3, "mla_prefill_attention rows=%zu: %.3e beyond a bf16 step", rows, worst);
+        } else {
+            compare(got, want, "mla_prefill_attention, one row");
+        }
+        position = total;
+        CHECK(cache.len(layer) == position, "cache length %zu vs %zu", cache.len(layer), position);
+    }
+    CHECK(ctx.mla_prefill_attention(ctx.tensor_from_f32(std::vector<float>(spec.q_projection_size), 1, spec.q_projection_size).unwrap(),
+                                    ctx.tensor_from_f32(std::vector<float>(512), 1, 512).unwrap(), ctx.tensor_from_f32(std::vector<float>(64), 1, 64).unwrap(),
+                                    weight.unwrap(), nullptr, layer, spec)
+              .is_err(),
+          "a prefill without a cache must be refused");
+}
+
 int main()
 {
     auto ctx = RocmContext::create(0);
@@ -347,9 +571,14 @@ int main()
     CHECK(CausalWindow::Sliding(4).key_range(9, 10) == std::make_pair((size_t)6, (size_t)10), "sliding window");
     CHECK(CausalWindow::Sliding(4).key_range(1, 10) == std::make_pair((size_t)0, (size_t)2), "sliding window, short history");
     CHECK(CausalWindow::Sliding(1024).cache_capacity(8192) == 1024 && CausalWindow::Full().cache_capacity(8192) == 8192, "cache capacity");
-    test_gqa(ctx.unwrap(), CausalWindow::Full(), "full");
-    test_gqa(ctx.unwrap(), CausalWindow::Sliding(128), "sliding(128)");
+    test_growth_rule();
+    test_gqa(ctx.unwrap(), CausalWindow::Full(), "full", TablePolicy::Scrambled);
+    test_gqa(ctx.unwrap(), CausalWindow::Sliding(128), "sliding(128)", TablePolicy::Scrambled);
+    test_gqa(ctx.unwrap(), CausalWindow::Full(), "full, growing planes", TablePolicy::Identity);
+    test_gqa_ring(ctx.unwrap());
+    test_gqa_shared_and_visible(ctx.unwrap());
     test_mla(ctx.unwrap());
+    test_mla_prefill(ctx.unwrap());
     printf(failures == 0 ? "ALL PASSED\n" : "%d FAILED\n", failures);
     return failures == 0 ? 0 : 1;
 }

@@ -133,5 +133,73 @@ def test_cpp_host_layer_builds_and_exports_the_backend_methods():
     names = subprocess.run(["nm", "-DC", "--defined-only", lib], capture_output=True, text=True, check=True).stdout
     for method in ("zllm_amd::RocmContext::gqa_prefill_attention_cached", "zllm_amd::RocmContext::append_mla(",
                    "zllm_amd::RocmContext::append_mla_rope", "zllm_amd::RocmContext::mla_decode_attention",
-                   "zllm_amd::CausalWindow::key_range", "zllm_amd::RocmKvCache::new_gqa", "zllm_amd::RocmKvCache::new_mla"):
+                   "zllm_amd::CausalWindow::key_range", "zllm_amd::RocmKvCache::new_gqa", "zllm_amd::RocmKvCache::new_mla",
+                   "zllm_amd::RocmContext::gqa_prefill_attention_cached_visible", "zllm_amd::RocmContext::gqa_prefill_attention_cached_from",
+                   "zllm_amd::RocmContext::mla_prefill_attention(", "zllm_amd::RocmContext::mla_prefill_attention_rope",
+                   "zllm_amd::committed_cache_rows"):
         assert method in names, method
+
+
+def test_split_plan_covers_the_host_bound_and_sizes_the_workspace(lib):
+    """The split plan is a function of the host arguments: max_chunks splits of chunk_tokens tokens cover max_kv_len and
+    nothing more, which is the bound a recorded graph stays valid under (a longer kv_lens[b] on the device is read up
+    to max_chunks * chunk_tokens tokens only)."""
+    rng = np.random.default_rng(5)
+    for _ in range(300):
+        args = capi.GqaDecodeArgs()
+        args.batch = int(rng.integers(1, 65))
+        args.num_kv_heads = int(rng.choice([1, 2, 4, 8]))
+        args.num_heads = args.num_kv_heads * int(rng.choice([1, 2, 4, 8, 16]))
+        args.head_dim = int(rng.choice([64, 128, 256]))
+        args.max_kv_len = int(rng.integers(1, 200000))
+        args.block_tokens = int(rng.choice([1, 16, 64]))
+        args.score_scale = 0.1
+        args.kv_format, args.scale_dtype, args.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_F32
+        if rng.random() < 0.5:  # a ragged batch: the hint may only shorten the splits, never drop coverage
+            args.total_kv_tokens = int(rng.integers(1, args.batch * args.max_kv_len + 1) % (1 << 32))
+        chunk, chunks = C.c_uint32(), C.c_uint32()
+        assert lib.zllm_attn_gqa_decode_split_plan(C.byref(args), C.byref(chunk), C.byref(chunks)) == 0
+        assert chunk.value % 32 == 0 and chunk.value >= 64 and chunks.value >= 1
+        assert chunk.value * chunks.value >= args.max_kv_len
+        assert chunk.value * (chunks.value - 1) < args.max_kv_len  # no split lies wholly beyond the bound
+        records = args.batch * chunks.value * args.num_heads
+        align = lambda n: (n + 255) // 256 * 256
+        assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) == align(records * args.head_dim * 4) + align(records * 8)
+    bad = capi.GqaDecodeArgs()
+    assert lib.zllm_attn_gqa_decode_split_plan(C.byref(bad), None, None) == -1
+
+
+def test_prefill_and_mla_argument_checks_without_a_gpu(lib):
+    pre = capi.GqaPrefillArgs()
+    pre.rows, pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens = 8, 8, 2, 128, 16
+    pre.score_scale, pre.kv_format, pre.scale_dtype = 0.1, capi.KV_Q8G64, capi.SCALE_F16
+    for name in ("q", "k_plane", "k_scales", "v_plane", "v_scales", "out"):
+        setattr(pre, name, 0x10000)
+    pre.k_plane = 0x10008  # codes are read as 16-byte vectors
+    assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"aligned" in lib.zllm_attn_last_error()
+    pre.k_plane, pre.k_scales = 0x10000, 0x10002  # scales as 4-byte words
+    assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"aligned" in lib.zllm_attn_last_error()
+    pre.k_scales = 0x10000
+    pre.table, pre.table_stride, pre.position = 0x20000, 3, 48  # 3 pages of 16 tokens < 48 + 8
+    assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"cannot cover" in lib.zllm_attn_last_error()
+    assert lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre)) == 0
+    pre.table_stride = 4
+    pre.head_dim = 256  # this geometry runs its rows through the decode kernels and needs their split records
+    assert lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre)) > 8 * 8
+    assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"workspace" in lib.zllm_attn_last_error()
+    # MLA: value part and query-row limits
+    mla = capi.MlaDecodeArgs()
+    mla.batch, mla.heads, mla.q_head_dim, mla.kv_head_dim, mla.latent_dim, mla.rope_dim = 1, 16, 192, 128, 512, 64
+    mla.block_tokens, mla.max_ctx_len, mla.q_dtype, mla.out_dtype = 64, 4096, capi.DTYPE_BF16, capi.DTYPE_F32
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) == 0 and b"value_dim" in lib.zllm_attn_last_error()  # nope == kv_head_dim
+    mla.kv_head_dim, mla.q_head_dim, mla.rope_dim = 600, 192, 64  # value 472 > q_head_dim with strided output
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) == 0 and b"value_dim" in lib.zllm_attn_last_error()
+    mla.out_compact = 1
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) > 0
+    mla.kv_head_dim = 256
+    mla.batch, mla.query_rows = 40, 2048
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) == 0 and b"65535" in lib.zllm_attn_last_error()
+    mla.batch, mla.query_rows = 2, 64
+    one = capi.MlaDecodeArgs.from_buffer_copy(mla)
+    one.query_rows = 0
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) > lib.zllm_attn_mla_decode_workspace_bytes(C.byref(one)) > 0

@@ -1,6 +1,7 @@
 """Runs the C++ host layer's parity driver (tests/host/backend_parity.cpp): the reference-shaped backend methods
-(gqa_prefill_attention_cached, append_mla, append_mla_rope, mla_decode_attention) over the C ABI, compared with the
-CPU oracle inside the driver, plus their error behaviour.  The binary is built by __graft_entry__.build()."""
+(gqa_prefill_attention_cached and its _visible / _from forms, append_mla, append_mla_rope, mla_decode_attention,
+mla_prefill_attention) over the C ABI, compared with the CPU oracle inside the driver, plus their error behaviour, the
+grow-by-doubling rule of the cache planes and the ring of a sliding-window layer.  The binary is built by __graft_entry__.build()."""
 import os
 import subprocess
 

@@ -111,6 +111,7 @@ SYMBOLS = {
     "zllm_kv_mla_layer_write": (_int, [C.POINTER(MlaLayerRecord), _ptr, _u64, C.POINTER(_u64)]),
     "zllm_kv_mla_layer_read": (_int, [_ptr, _u64, C.POINTER(MlaLayerRecord), C.POINTER(_u64)]),
     "zllm_attn_gqa_decode_workspace_bytes": (_u64, [C.POINTER(GqaDecodeArgs)]),
+    "zllm_attn_gqa_decode_split_plan": (_int, [C.POINTER(GqaDecodeArgs), C.POINTER(_u32), C.POINTER(_u32)]),
     "zllm_attn_gqa_decode": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
     "zllm_attn_static_scratch_bytes": (_u64, []),
     "zllm_attn_gqa_decode_static": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),

@@ -719,6 +719,23 @@ static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint6
     return hip_status(zllm::launch_gqa_decode(p, a->kv_format, a->scale_dtype, a->stages, (hipStream_t)stream), "GQA decode launch");
 }
 
+int zllm_attn_gqa_decode_split_plan(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    const int rc = validate_gqa_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    uint32_t chunk = 0, chunks = 0;
+    plan_gqa_decode(a, &chunk, &chunks);
+    if (chunk_tokens != nullptr) {
+        *chunk_tokens = chunk;
+    }
+    if (max_chunks != nullptr) {
+        *max_chunks = chunks;
+    }
+    return 0;
+}
+
 int zllm_attn_gqa_decode(const zllm_gqa_decode_args* a, zllm_stream_t stream)
 {
     const int rc = validate_gqa_decode(a);

@@ -149,92 +149,136 @@ std::vector<uint32_t> scrambled_pages(size_t pages)
 
 } // namespace
 
-Result<RocmKvCache> RocmKvCache::new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens)
+Result<size_t> committed_cache_rows(size_t current, size_t required, size_t limit)
+{
+    constexpr size_t kBlock = 64; // ROCM_KV_BLOCK_SIZE (src/backend/rocm/mod.rs:301)
+    if (required == 0 || required > limit) {
+        return compute_error("ROCm cache required=" + std::to_string(required) + " exceeds the logical limit " + std::to_string(limit));
+    }
+    if (current >= required) {
+        return current;
+    }
+    const size_t target = std::max(std::max(required, current * 2), kBlock);
+    const size_t aligned = (target + kBlock - 1) / kBlock * kBlock;
+    return std::max(std::min(aligned, limit), required);
+}
+
+void RocmKvCache::plane_row_bytes(size_t (&bytes)[4]) const
+{
+    if (mla_) {
+        bytes[0] = cols_;
+        bytes[1] = cols_ / 64 * 2;
+        bytes[2] = rope_cols_ * 2;
+        bytes[3] = 0;
+    } else {
+        bytes[0] = cols_;
+        bytes[1] = cols_ / 64 * 2;
+        bytes[2] = cols_;
+        bytes[3] = cols_ / 64 * 2;
+    }
+}
+
+Result<RocmKvCache> RocmKvCache::create(bool mla, size_t layers, size_t cols, size_t rope_cols, size_t block_tokens, size_t max_tokens,
+                                        TablePolicy policy)
+{
+    RocmKvCache cache;
+    cache.mla_ = mla;
+    cache.policy_ = policy;
+    cache.cols_ = cols;
+    cache.rope_cols_ = rope_cols;
+    cache.block_tokens_ = block_tokens;
+    cache.max_tokens_ = max_tokens;
+    const size_t pages = (max_tokens + block_tokens - 1) / block_tokens;
+    if (pages > UINT32_MAX) {
+        return compute_error("ROCm KV block ID exceeds u32");
+    }
+    cache.pool_rows_ = pages * block_tokens;
+    // the table is built once, at full capacity: rebuilding it as the cache grows would put an upload and a stream
+    // synchronisation on every page boundary of a decode loop (src/backend/rocm/mod.rs:353-356)
+    if (policy == TablePolicy::Identity) {
+        cache.table_host_.resize(pages);
+        std::iota(cache.table_host_.begin(), cache.table_host_.end(), 0u);
+    } else {
+        cache.table_host_ = scrambled_pages(pages);
+    }
+    auto table = DeviceBuffer::allocate(pages * 4);
+    if (table.is_err()) {
+        return table.unwrap_err();
+    }
+    cache.table_ = table.unwrap();
+    const hipError_t err = hipMemcpy(cache.table_.data(), cache.table_host_.data(), pages * 4, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+        return hip_error("block table upload", err);
+    }
+    cache.layers_.resize(layers);
+    cache.lens_.assign(layers, 0);
+    if (policy == TablePolicy::Scrambled) { // any page may be named from the first append on: commit the pool
+        for (size_t l = 0; l < layers; ++l) {
+            auto done = cache.reserve_rows(l, cache.pool_rows_, nullptr);
+            if (done.is_err()) {
+                return done.unwrap_err();
+            }
+        }
+    }
+    return cache;
+}
+
+Result<Unit> RocmKvCache::reserve_rows(size_t layer, size_t required, hipStream_t stream)
+{
+    Layer& planes = layers_[layer];
+    if (planes.committed_rows >= required) {
+        return Unit{};
+    }
+    auto rows_r = committed_cache_rows(planes.committed_rows, required, pool_rows_);
+    if (rows_r.is_err()) {
+        return rows_r.unwrap_err();
+    }
+    // whole pages: a page's rows are addressed through its table entry
+    const size_t rows = std::min((rows_r.unwrap() + block_tokens_ - 1) / block_tokens_ * block_tokens_, pool_rows_);
+    size_t row_bytes[4];
+    plane_row_bytes(row_bytes);
+    DeviceBuffer* buffers[4] = {&planes.a_codes, &planes.a_scales, &planes.b_codes, &planes.b_scales};
+    for (int i = 0; i < 4; ++i) {
+        if (row_bytes[i] == 0) {
+            continue;
+        }
+        auto grown = DeviceBuffer::allocate(rows * row_bytes[i]);
+        if (grown.is_err()) {
+            return grown.unwrap_err();
+        }
+        if (planes.committed_rows != 0) {
+            // under the identity table the used rows are a prefix of the plane
+            hipError_t err = hipMemcpyAsync(grown.unwrap().data(), buffers[i]->data(), planes.committed_rows * row_bytes[i], hipMemcpyDeviceToDevice, stream);
+            if (err == hipSuccess) {
+                err = hipStreamSynchronize(stream); // the old plane is released below
+            }
+            if (err != hipSuccess) {
+                return hip_error("cache growth copy", err);
+            }
+        }
+        *buffers[i] = grown.unwrap();
+    }
+    planes.committed_rows = rows;
+    return Unit{};
+}
+
+Result<RocmKvCache> RocmKvCache::new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens,
+                                         TablePolicy policy)
 {
     const size_t cols = num_kv_heads * head_dim;
     if (layers == 0 || cols == 0 || cols % 64 != 0 || block_tokens == 0 || max_tokens == 0) {
         return compute_error("Rocm GQA cache: invalid geometry");
     }
-    RocmKvCache cache;
-    cache.cols_ = cols;
-    cache.block_tokens_ = block_tokens;
-    cache.max_tokens_ = max_tokens;
-    const size_t pages = (max_tokens + block_tokens - 1) / block_tokens;
-    cache.pool_rows_ = pages * block_tokens;
-    cache.table_host_ = scrambled_pages(pages);
-    auto table = DeviceBuffer::allocate(pages * 4);
-    if (table.is_err()) {
-        return table.unwrap_err();
-    }
-    cache.table_ = table.unwrap();
-    hipError_t err = hipMemcpy(cache.table_.data(), cache.table_host_.data(), pages * 4, hipMemcpyHostToDevice);
-    if (err != hipSuccess) {
-        return hip_error("block table upload", err);
-    }
-    for (size_t l = 0; l < layers; ++l) {
-        Layer layer;
-        DeviceBuffer* planes[4] = {&layer.a_codes, &layer.a_scales, &layer.b_codes, &layer.b_scales};
-        const size_t bytes[4] = {cache.pool_rows_ * cols, cache.pool_rows_ * (cols / 64) * 2, cache.pool_rows_ * cols,
-                                 cache.pool_rows_ * (cols / 64) * 2};
-        for (int i = 0; i < 4; ++i) {
-            auto buf = DeviceBuffer::allocate(bytes[i]);
-            if (buf.is_err()) {
-                return buf.unwrap_err();
-            }
-            *planes[i] = buf.unwrap();
-            err = hipMemset(planes[i]->data(), 0, bytes[i]);
-            if (err != hipSuccess) {
-                return hip_error("cache clear", err);
-            }
-        }
-        cache.layers_.push_back(layer);
-        cache.lens_.push_back(0);
-    }
-    return cache;
+    return create(false, layers, cols, 0, block_tokens, max_tokens, policy);
 }
 
-Result<RocmKvCache> RocmKvCache::new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens)
+Result<RocmKvCache> RocmKvCache::new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens,
+                                         TablePolicy policy)
 {
     if (layers == 0 || latent_dim == 0 || latent_dim % 64 != 0 || rope_dim == 0 || block_tokens == 0 || max_tokens == 0) {
         return compute_error("Rocm MLA cache: invalid geometry");
     }
-    RocmKvCache cache;
-    cache.mla_ = true;
-    cache.cols_ = latent_dim;
-    cache.rope_cols_ = rope_dim;
-    cache.block_tokens_ = block_tokens;
-    cache.max_tokens_ = max_tokens;
-    const size_t pages = (max_tokens + block_tokens - 1) / block_tokens;
-    cache.pool_rows_ = pages * block_tokens;
-    cache.table_host_ = scrambled_pages(pages);
-    auto table = DeviceBuffer::allocate(pages * 4);
-    if (table.is_err()) {
-        return table.unwrap_err();
-    }
-    cache.table_ = table.unwrap();
-    hipError_t err = hipMemcpy(cache.table_.data(), cache.table_host_.data(), pages * 4, hipMemcpyHostToDevice);
-    if (err != hipSuccess) {
-        return hip_error("block table upload", err);
-    }
-    for (size_t l = 0; l < layers; ++l) {
-        Layer layer;
-        DeviceBuffer* planes[3] = {&layer.a_codes, &layer.a_scales, &layer.b_codes};
-        const size_t bytes[3] = {cache.pool_rows_ * latent_dim, cache.pool_rows_ * (latent_dim / 64) * 2, cache.pool_rows_ * rope_dim * 2};
-        for (int i = 0; i < 3; ++i) {
-            auto buf = DeviceBuffer::allocate(bytes[i]);
-            if (buf.is_err()) {
-                return buf.unwrap_err();
-            }
-            *planes[i] = buf.unwrap();
-            err = hipMemset(planes[i]->data(), 0, bytes[i]);
-            if (err != hipSuccess) {
-                return hip_error("cache clear", err);
-            }
-        }
-        cache.layers_.push_back(layer);
-        cache.lens_.push_back(0);
-    }
-    return cache;
+    return create(true, layers, latent_dim, rope_dim, block_tokens, max_tokens, policy);
 }
 
 Result<Unit> RocmKvCache::truncate_rows(size_t rows)
@@ -332,6 +376,21 @@ Result<MlaLayerSerde> read_mla_layer(const std::vector<uint8_t>& in, size_t& off
 }
 
 // ---------------------------------------------------------------------------------------------- context
+struct RocmContext::Scratch {
+    static constexpr size_t kSlots = 256;
+    hipStream_t stream = nullptr;
+    DeviceBuffer workspace;
+    uint32_t* meta_host = nullptr; // pinned, kSlots records of four u32
+    DeviceBuffer meta_dev;
+    size_t next = 0;
+    ~Scratch()
+    {
+        if (meta_host != nullptr) {
+            (void)hipHostFree(meta_host);
+        }
+    }
+};
+
 Result<RocmContext> RocmContext::create(int device_id)
 {
     int cus = 0;
@@ -348,7 +407,59 @@ Result<RocmContext> RocmContext::create(int device_id)
     if (err != hipSuccess) {
         return hip_error("stream", err);
     }
+    auto scratch = std::make_shared<Scratch>();
+    scratch->stream = ctx.stream_;
+    err = hipHostMalloc((void**)&scratch->meta_host, Scratch::kSlots * 16, hipHostMallocDefault);
+    if (err != hipSuccess) {
+        return hip_error("pinned metadata ring", err);
+    }
+    auto meta = DeviceBuffer::allocate(Scratch::kSlots * 16);
+    if (meta.is_err()) {
+        return meta.unwrap_err();
+    }
+    scratch->meta_dev = meta.unwrap();
+    ctx.scratch_ = scratch;
     return ctx;
+}
+
+Result<void*> RocmContext::workspace(size_t bytes) const
+{
+    Scratch& s = *scratch_;
+    if (bytes > s.workspace.bytes()) {
+        // kernels in flight may still use the old buffer: wait for them before it is released
+        const hipError_t err = hipStreamSynchronize(stream_);
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+        auto grown = DeviceBuffer::allocate(std::max(bytes, s.workspace.bytes() * 2));
+        if (grown.is_err()) {
+            return grown.unwrap_err();
+        }
+        s.workspace = grown.unwrap();
+    }
+    return s.workspace.data();
+}
+
+Result<const uint32_t*> RocmContext::upload_meta(const uint32_t (&values)[4]) const
+{
+    Scratch& s = *scratch_;
+    if (s.next == Scratch::kSlots) {
+        // the ring wrapped: the oldest records may still be read by launches in flight
+        const hipError_t err = hipStreamSynchronize(stream_);
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+        s.next = 0;
+    }
+    uint32_t* host = s.meta_host + 4 * s.next;
+    uint32_t* dev = (uint32_t*)s.meta_dev.data() + 4 * s.next;
+    memcpy(host, values, 16);
+    const hipError_t err = hipMemcpyAsync(dev, host, 16, hipMemcpyHostToDevice, stream_);
+    if (err != hipSuccess) {
+        return hip_error("metadata upload", err);
+    }
+    ++s.next;
+    return (const uint32_t*)dev;
 }
 
 Result<Unit> RocmContext::synchronize() const
@@ -426,55 +537,56 @@ Result<RocmWeight> RocmContext::prepare_mla_kv_b(const std::vector<float>& weigh
     return w;
 }
 
-Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
-                                                             const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
-                                                             bool retain_full_cache) const
+namespace {
+
+// HybridGqaCacheLayout::write_plan (src/kv_cache/mod.rs:440-455) for a layer that keeps `capacity` rows
+struct RingPlan {
+    size_t source_start, token_count;
+};
+
+RingPlan ring_write_plan(size_t capacity, size_t position, size_t count)
 {
-    (void)retain_full_cache;
-    if (spec.num_heads == 0 || spec.num_kv_heads == 0 || spec.head_dim == 0 || spec.num_heads % spec.num_kv_heads != 0) {
-        return compute_error("Rocm GQA spec invalid");
-    }
-    const size_t query_cols = spec.num_heads * spec.head_dim;
-    const size_t kv_cols = spec.num_kv_heads * spec.head_dim;
-    if (query.rows != key.rows || query.rows != value.rows || query.cols != query_cols || key.cols != kv_cols || value.cols != kv_cols) {
-        return compute_error("Rocm GQA cached prefill shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
-                             std::to_string(key.rows) + "," + std::to_string(key.cols) + "] V=[" + std::to_string(value.rows) + "," +
-                             std::to_string(value.cols) + "]");
-    }
-    if (cache.mla_ || layer >= cache.layers_.size() || cache.cols_ != kv_cols) {
-        BackendError e;
-        e.kind = BackendError::Kind::UnsupportedLayer;
-        e.layer = layer;
-        return e;
-    }
-    if (query.rows == 0) {
-        return compute_error("Rocm GQA cached prefill: empty chunk");
-    }
-    // position must be the current cache length (src/backend/rocm/attention.rs:2226-2229)
-    if (cache.lens_[layer] != position) {
-        return compute_error("Rocm GQA L" + std::to_string(layer) + " device cache incomplete: rows=" + std::to_string(cache.lens_[layer]) + "/" +
-                             std::to_string(position));
-    }
-    const size_t total = position + query.rows;
-    if (total > cache.max_tokens_ || total > UINT32_MAX) {
-        return compute_error("Rocm GQA cache position overflow");
-    }
+    const size_t end = position + count;
+    const size_t write_start = std::max(position, end > capacity ? end - capacity : 0);
+    return RingPlan{write_start - position, end - write_start};
+}
+
+BackendError unsupported_layer(size_t layer)
+{
+    BackendError e;
+    e.kind = BackendError::Kind::UnsupportedLayer;
+    e.layer = layer;
+    return e;
+}
+
+} // namespace
+
+Result<Unit> RocmContext::append_gqa_rows(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& key, const RocmTensor& value) const
+{
     RocmKvCache::Layer& planes = cache.layers_[layer];
-    // quantizing append of the chunk's K and V rows (no f32 staging copies)
+    const size_t ring = planes.ring_capacity;
+    const size_t total = position + key.rows;
+    auto reserved = cache.reserve_rows(layer, ring != 0 ? std::min(total, ring) : total, stream_);
+    if (reserved.is_err()) {
+        return reserved.unwrap_err();
+    }
+    // a ring keeps the chunk's last `capacity` rows only
+    const RingPlan plan = ring != 0 ? ring_write_plan(ring, position, key.rows) : RingPlan{0, key.rows};
     const RocmTensor* sources[2] = {&key, &value};
     void* codes[2] = {planes.a_codes.data(), planes.b_codes.data()};
     void* scales[2] = {planes.a_scales.data(), planes.b_scales.data()};
     for (int i = 0; i < 2; ++i) {
         zllm_q8_append_args a;
         memset(&a, 0, sizeof(a));
-        a.src = sources[i]->device.data();
+        a.src = (const char*)sources[i]->device.data() + plan.source_start * sources[i]->cols * dtype_bytes(sources[i]->dtype);
         a.codes = (int8_t*)codes[i];
         a.scales = scales[i];
         a.table = (const uint32_t*)cache.table_.data();
-        a.position = (uint32_t)position;
-        a.rows = (uint32_t)query.rows;
-        a.cols = (uint32_t)kv_cols;
+        a.position = (uint32_t)(position + plan.source_start);
+        a.rows = (uint32_t)plan.token_count;
+        a.cols = (uint32_t)cache.cols_;
         a.block_tokens = (uint32_t)cache.block_tokens_;
+        a.ring_capacity = (uint32_t)ring;
         a.src_dtype = abi_dtype(sources[i]->dtype);
         a.rule = ZLLM_QUANT_METAL_GQA;
         const int rc = zllm_attn_q8g64_append(&a, stream_);
@@ -482,8 +594,16 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
             return abi_error("zllm_attn_q8g64_append", rc);
         }
     }
-    cache.lens_[layer] = total;
+    return Unit{};
+}
 
+// Attention of `query.rows` rows at `position` over the layer's rows [.., position + query.rows), which are in the cache.
+Result<RocmTensor> RocmContext::gqa_attend(const RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query, const GqaSpec& spec,
+                                           const uint32_t* visible_ends_dev) const
+{
+    const RocmKvCache::Layer& planes = cache.layers_[layer];
+    const size_t query_cols = spec.num_heads * spec.head_dim;
+    const size_t total = position + query.rows;
     auto out_buf = DeviceBuffer::allocate(query.rows * query_cols * 4);
     if (out_buf.is_err()) {
         return out_buf.unwrap_err();
@@ -495,20 +615,12 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
     out.dtype = DType::F32;
     const size_t table_stride = cache.table_host_.size();
 
-    if (query.rows == 1) {
+    if (query.rows == 1 && visible_ends_dev == nullptr) {
         const auto range = spec.window.key_range(position, total);
-        const uint32_t host_meta[2] = {(uint32_t)total, (uint32_t)range.first};
-        auto meta = DeviceBuffer::allocate(8);
+        const uint32_t host_meta[4] = {(uint32_t)total, (uint32_t)range.first, 0u, 0u};
+        auto meta = upload_meta(host_meta);
         if (meta.is_err()) {
             return meta.unwrap_err();
-        }
-        hipError_t err = hipMemcpyAsync(meta.unwrap().data(), host_meta, 8, hipMemcpyHostToDevice, stream_);
-        if (err != hipSuccess) {
-            return hip_error("decode metadata upload", err);
-        }
-        err = hipStreamSynchronize(stream_); // host_meta is a stack array
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
         }
         zllm_gqa_decode_args a;
         memset(&a, 0, sizeof(a));
@@ -518,8 +630,8 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
         a.v_plane = planes.b_codes.data();
         a.v_scales = planes.b_scales.data();
         a.tables = (const uint32_t*)cache.table_.data();
-        a.kv_lens = (const uint32_t*)meta.unwrap().data();
-        a.first_visible = spec.window.sliding ? (const uint32_t*)meta.unwrap().data() + 1 : nullptr;
+        a.kv_lens = meta.unwrap();
+        a.first_visible = spec.window.sliding ? meta.unwrap() + 1 : nullptr;
         a.out = (float*)out.device.data();
         a.batch = 1;
         a.num_heads = (uint32_t)spec.num_heads;
@@ -528,6 +640,7 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
         a.table_stride = (uint32_t)table_stride;
         a.max_kv_len = (uint32_t)total;
         a.block_tokens = (uint32_t)cache.block_tokens_;
+        a.ring_capacity = (uint32_t)planes.ring_capacity;
         a.score_scale = spec.score_scale;
         a.kv_format = ZLLM_KV_Q8G64;
         a.scale_dtype = ZLLM_SCALE_F16;
@@ -536,23 +649,21 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
         if (need == 0) {
             return abi_error("zllm_attn_gqa_decode_workspace_bytes", -1);
         }
-        auto ws = DeviceBuffer::allocate(need);
+        auto ws = workspace(need);
         if (ws.is_err()) {
             return ws.unwrap_err();
         }
-        a.workspace = ws.unwrap().data();
+        a.workspace = ws.unwrap();
         a.workspace_bytes = need;
         const int rc = zllm_attn_gqa_decode(&a, stream_);
         if (rc != 0) {
             return abi_error("zllm_attn_gqa_decode", rc);
         }
-        err = hipStreamSynchronize(stream_); // the workspace and metadata die with this scope
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
-        }
         return out;
     }
-
+    if (planes.ring_capacity != 0 && total > planes.ring_capacity) {
+        return compute_error("sliding-window GQA cannot attend a multi-token chunk over a ring that has wrapped");
+    }
     zllm_gqa_prefill_args a;
     memset(&a, 0, sizeof(a));
     a.q = query.device.data();
@@ -561,6 +672,7 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
     a.v_plane = planes.b_codes.data();
     a.v_scales = planes.b_scales.data();
     a.table = (const uint32_t*)cache.table_.data();
+    a.table_stride = (uint32_t)table_stride;
     a.out = out.device.data();
     a.rows = (uint32_t)query.rows;
     a.position = (uint32_t)position;
@@ -574,6 +686,16 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
     a.scale_dtype = ZLLM_SCALE_F16;
     a.q_dtype = abi_dtype(query.dtype);
     a.out_dtype = ZLLM_DTYPE_F32;
+    a.visible_ends = visible_ends_dev;
+    const uint64_t need = zllm_attn_gqa_prefill_workspace_bytes(&a);
+    if (need != 0) {
+        auto ws = workspace(need);
+        if (ws.is_err()) {
+            return ws.unwrap_err();
+        }
+        a.workspace = ws.unwrap();
+        a.workspace_bytes = need;
+    }
     const int rc = zllm_attn_gqa_prefill_chunk(&a, stream_);
     if (rc != 0) {
         return abi_error("zllm_attn_gqa_prefill_chunk", rc);
@@ -581,14 +703,152 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache,
     return out;
 }
 
+Result<RocmTensor> RocmContext::gqa_cached_impl(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query, const RocmTensor& key,
+                                                const RocmTensor& value, const GqaSpec& spec, const std::vector<uint32_t>* visible_ends,
+                                                bool retain_full_cache) const
+{
+    if (spec.num_heads == 0 || spec.num_kv_heads == 0 || spec.head_dim == 0 || spec.num_heads % spec.num_kv_heads != 0) {
+        return compute_error("Rocm GQA spec invalid");
+    }
+    const size_t query_cols = spec.num_heads * spec.head_dim;
+    const size_t kv_cols = spec.num_kv_heads * spec.head_dim;
+    if (query.rows != key.rows || query.rows != value.rows || query.cols != query_cols || key.cols != kv_cols || value.cols != kv_cols) {
+        return compute_error("Rocm GQA cached prefill shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
+                             std::to_string(key.rows) + "," + std::to_string(key.cols) + "] V=[" + std::to_string(value.rows) + "," +
+                             std::to_string(value.cols) + "]");
+    }
+    if (cache.mla_ || layer >= cache.layers_.size() || cache.cols_ != kv_cols) {
+        return unsupported_layer(layer);
+    }
+    if (query.rows == 0) {
+        return compute_error("Rocm GQA cached prefill: empty chunk");
+    }
+    if (visible_ends != nullptr && visible_ends->size() != query.rows) {
+        return compute_error("GQA visible_ends=" + std::to_string(visible_ends->size()) + ", expected " + std::to_string(query.rows));
+    }
+    // position must be the current cache length (src/backend/rocm/attention.rs:2226-2229)
+    if (cache.lens_[layer] != position) {
+        return compute_error("Rocm GQA L" + std::to_string(layer) + " device cache incomplete: rows=" + std::to_string(cache.lens_[layer]) + "/" +
+                             std::to_string(position));
+    }
+    const size_t total = position + query.rows;
+    if (total > cache.max_tokens_ || total > UINT32_MAX) {
+        return compute_error("Rocm GQA cache position overflow");
+    }
+    // a sliding-window layer that need not keep everything keeps a ring of cache_capacity rows
+    const size_t ring = spec.window.sliding && !retain_full_cache ? spec.window.cache_capacity(cache.max_tokens_) : 0;
+    RocmKvCache::Layer& planes = cache.layers_[layer];
+    if (position == 0) {
+        planes.ring_capacity = ring;
+    } else if (planes.ring_capacity != ring) {
+        return compute_error("Rocm GQA L" + std::to_string(layer) + ": the layer was filled with another retention (ring of " +
+                             std::to_string(planes.ring_capacity) + " rows)");
+    }
+    const uint32_t* ends_dev = nullptr;
+    DeviceBuffer ends_buf;
+    if (visible_ends != nullptr) {
+        auto buf = DeviceBuffer::allocate(visible_ends->size() * 4);
+        if (buf.is_err()) {
+            return buf.unwrap_err();
+        }
+        ends_buf = buf.unwrap();
+        const hipError_t err = hipMemcpy(ends_buf.data(), visible_ends->data(), visible_ends->size() * 4, hipMemcpyHostToDevice);
+        if (err != hipSuccess) {
+            return hip_error("visible ends upload", err);
+        }
+        ends_dev = (const uint32_t*)ends_buf.data();
+    }
+    if (ring != 0 && query.rows > 1) {
+        // the reference's CPU backend (src/backend/cpu/attention.rs:401-409): a multi-token chunk on a draining sliding layer
+        // attends to itself at position 0 and is rejected elsewhere
+        if (position != 0) {
+            return compute_error("sliding-window GQA does not take a multi-token prefill at a non-zero position");
+        }
+        if (total > ring) {
+            // the ring cannot hold the whole chunk: attend over a cache of the chunk's own, then keep the tail
+            auto own = RocmKvCache::new_gqa(1, spec.num_kv_heads, spec.head_dim, cache.block_tokens_, total);
+            if (own.is_err()) {
+                return own.unwrap_err();
+            }
+            RocmKvCache chunk_cache = own.unwrap();
+            auto appended = append_gqa_rows(chunk_cache, 0, 0, key, value);
+            if (appended.is_err()) {
+                return appended.unwrap_err();
+            }
+            auto out = gqa_attend(chunk_cache, 0, 0, query, spec, ends_dev);
+            if (out.is_err()) {
+                return out;
+            }
+            auto kept = append_gqa_rows(cache, layer, 0, key, value);
+            if (kept.is_err()) {
+                return kept.unwrap_err();
+            }
+            const hipError_t err = hipStreamSynchronize(stream_); // the chunk's own cache dies with this scope
+            if (err != hipSuccess) {
+                return hip_error("hipStreamSynchronize", err);
+            }
+            cache.lens_[layer] = total;
+            return out;
+        }
+    }
+    auto appended = append_gqa_rows(cache, layer, position, key, value);
+    if (appended.is_err()) {
+        return appended.unwrap_err();
+    }
+    auto out = gqa_attend(cache, layer, position, query, spec, ends_dev);
+    if (out.is_err()) {
+        return out; // the cache length is left alone: the rows written past it are overwritten by the next append
+    }
+    if (ends_dev != nullptr) {
+        const hipError_t err = hipStreamSynchronize(stream_); // the uploaded ends die with this scope
+        if (err != hipSuccess) {
+            return hip_error("hipStreamSynchronize", err);
+        }
+    }
+    cache.lens_[layer] = total;
+    return out;
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_cached(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
+                                                             const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                             bool retain_full_cache) const
+{
+    return gqa_cached_impl(cache, layer, position, query, key, value, spec, nullptr, retain_full_cache);
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_cached_visible(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
+                                                                     const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                                     const std::vector<uint32_t>& visible_ends, bool retain_full_cache) const
+{
+    return gqa_cached_impl(cache, layer, position, query, key, value, spec, &visible_ends, retain_full_cache);
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_cached_from(const RocmKvCache& cache, size_t source_layer, size_t position,
+                                                                  const RocmTensor& query, const GqaSpec& spec) const
+{
+    if (spec.num_heads == 0 || spec.num_kv_heads == 0 || spec.head_dim == 0 || spec.num_heads % spec.num_kv_heads != 0) {
+        return compute_error("Rocm GQA spec invalid");
+    }
+    if (cache.mla_ || source_layer >= cache.layers_.size()) {
+        return unsupported_layer(source_layer);
+    }
+    const size_t required = position + query.rows;
+    // shape rule of the shared-KV path (src/backend/cpu/attention.rs:439-446); a ring or a longer source cannot serve it:
+    // the rows after the chunk would be visible to the kernels' causal ranges only by position, which they respect
+    if (query.rows == 0 || query.cols != spec.num_heads * spec.head_dim || cache.cols_ != spec.num_kv_heads * spec.head_dim ||
+        cache.lens_[source_layer] < required) {
+        return compute_error("GQA shared cache L" + std::to_string(source_layer) + " incomplete: Q=[" + std::to_string(query.rows) + "," +
+                             std::to_string(query.cols) + "], cache rows=" + std::to_string(cache.lens_[source_layer]) +
+                             ", required_rows=" + std::to_string(required));
+    }
+    return gqa_attend(cache, source_layer, position, query, spec, nullptr);
+}
+
 Result<Unit> RocmContext::append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
                                           RotaryLayout layout, size_t position, const float* cos_dev, const float* sin_dev) const
 {
     if (!cache.mla_ || layer >= cache.layers_.size()) {
-        BackendError e;
-        e.kind = BackendError::Kind::UnsupportedLayer;
-        e.layer = layer;
-        return e;
+        return unsupported_layer(layer);
     }
     if (latent.rows != rope.rows || latent.cols != cache.cols_ || rope.cols != cache.rope_cols_ || latent.dtype != DType::F32 ||
         rope.dtype != DType::F32) {
@@ -598,6 +858,10 @@ Result<Unit> RocmContext::append_mla_impl(RocmKvCache& cache, size_t layer, cons
     const size_t at = cache.lens_[layer];
     if (at + latent.rows > cache.max_tokens_) {
         return compute_error("Rocm MLA cache is full");
+    }
+    auto reserved = cache.reserve_rows(layer, at + latent.rows, stream_);
+    if (reserved.is_err()) {
+        return reserved.unwrap_err();
     }
     RocmKvCache::Layer& planes = cache.layers_[layer];
     zllm_mla_append_args a;
@@ -705,34 +969,30 @@ Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const R
         return compute_error(*bad);
     }
     if (!cache.mla_ || layer >= cache.layers_.size()) {
-        BackendError e;
-        e.kind = BackendError::Kind::UnsupportedLayer;
-        e.layer = layer;
-        return e;
+        return unsupported_layer(layer);
     }
-    if (query.rows != 1 || query.cols != spec.q_projection_size || spec.kv_lora_rank != cache.cols_ || spec.qk_rope_head_dim != cache.rope_cols_ ||
+    // `query.rows` query rows that are the last rows of the cache: one for a decode step, a chunk's worth for a prefill
+    if (query.rows == 0 || query.cols != spec.q_projection_size || spec.kv_lora_rank != cache.cols_ || spec.qk_rope_head_dim != cache.rope_cols_ ||
         kv_b.rows != spec.kv_projection_size || kv_b.cols != spec.kv_lora_rank) {
         return compute_error("Rocm MLA decode shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] kv_b=[" +
                              std::to_string(kv_b.rows) + "," + std::to_string(kv_b.cols) + "]");
     }
     const size_t ctx = cache.lens_[layer];
-    if (ctx == 0 || position + 1 != ctx) {
+    if (ctx == 0 || position + query.rows != ctx) {
         return compute_error("Rocm MLA L" + std::to_string(layer) + " cache length " + std::to_string(ctx) + " does not match position " +
                              std::to_string(position));
     }
+    const bool chunk = query.rows > 1;
     const size_t out_cols = spec.num_heads * spec.value_dim();
-    auto out_buf = DeviceBuffer::allocate(out_cols * 4);
-    auto meta = DeviceBuffer::allocate(4);
+    // a decode row is written as f32, the rows of a chunk as bf16 (src/backend/rocm/attention.rs:17-19)
+    auto out_buf = DeviceBuffer::allocate(query.rows * out_cols * (chunk ? 2 : 4));
     if (out_buf.is_err()) {
         return out_buf.unwrap_err();
     }
+    const uint32_t host_meta[4] = {(uint32_t)ctx, 0u, 0u, 0u};
+    auto meta = upload_meta(host_meta);
     if (meta.is_err()) {
         return meta.unwrap_err();
-    }
-    const uint32_t ctx_u32 = (uint32_t)ctx;
-    hipError_t err = hipMemcpy(meta.unwrap().data(), &ctx_u32, 4, hipMemcpyHostToDevice);
-    if (err != hipSuccess) {
-        return hip_error("decode metadata upload", err);
     }
     const RocmKvCache::Layer& planes = cache.layers_[layer];
     zllm_mla_decode_args a;
@@ -743,19 +1003,20 @@ Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const R
     a.latent_scales = (const uint16_t*)planes.a_scales.data();
     a.rope_cache = (const uint16_t*)planes.b_codes.data();
     a.tables = (const uint32_t*)cache.table_.data();
-    a.ctx_lens = (const uint32_t*)meta.unwrap().data();
+    a.ctx_lens = meta.unwrap();
     a.out = out_buf.unwrap().data();
     a.batch = 1;
+    a.query_rows = (uint32_t)query.rows;
     a.heads = (uint32_t)spec.num_heads;
     a.q_head_dim = (uint32_t)spec.q_head_dim();
     a.kv_head_dim = (uint32_t)spec.kv_head_dim();
     a.latent_dim = (uint32_t)spec.kv_lora_rank;
     a.rope_dim = (uint32_t)spec.qk_rope_head_dim;
     a.table_stride = (uint32_t)cache.table_host_.size();
-    a.max_ctx_len = ctx_u32;
+    a.max_ctx_len = (uint32_t)ctx;
     a.block_tokens = (uint32_t)cache.block_tokens_;
     a.q_dtype = abi_dtype(query.dtype);
-    a.out_dtype = ZLLM_DTYPE_F32; // decode rows are written as f32 (src/backend/rocm/attention.rs:17-19)
+    a.out_dtype = chunk ? ZLLM_DTYPE_BF16 : ZLLM_DTYPE_F32;
     a.out_compact = 1;
     if (state != nullptr) {
         a.selection = (const uint32_t*)state->selection.data();
@@ -765,25 +1026,64 @@ Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const R
     if (need == 0) {
         return abi_error("zllm_attn_mla_decode_workspace_bytes", -1);
     }
-    auto ws = DeviceBuffer::allocate(need);
+    auto ws = workspace(need);
     if (ws.is_err()) {
         return ws.unwrap_err();
     }
-    a.workspace = ws.unwrap().data();
+    a.workspace = ws.unwrap();
     a.workspace_bytes = need;
     const int rc = zllm_attn_mla_decode(&a, stream_);
     if (rc != 0) {
         return abi_error("zllm_attn_mla_decode", rc);
     }
-    err = hipStreamSynchronize(stream_); // workspace and metadata die with this scope
-    if (err != hipSuccess) {
-        return hip_error("hipStreamSynchronize", err);
-    }
     RocmTensor out;
     out.device = out_buf.unwrap();
-    out.rows = 1;
+    out.rows = query.rows;
     out.cols = out_cols;
-    out.dtype = DType::F32;
+    out.dtype = chunk ? DType::BF16 : DType::F32;
+    return out;
+}
+
+Result<RocmTensor> RocmContext::mla_prefill_attention(const RocmTensor& query, const RocmTensor& latent, const RocmTensor& k_rope,
+                                                      const RocmWeight& kv_b, RocmKvCache* cache, size_t layer, const MlaSpec& spec) const
+{
+    if (cache == nullptr) {
+        return compute_error("L" + std::to_string(layer) + " ROCm MLA prefill needs a paged cache");
+    }
+    if (query.rows != latent.rows) {
+        return compute_error("Rocm MLA prefill shape mismatch: Q rows=" + std::to_string(query.rows) + " latent rows=" + std::to_string(latent.rows));
+    }
+    const size_t position = cache->len(layer);
+    auto appended = append_mla(*cache, layer, latent, k_rope);
+    if (appended.is_err()) {
+        return appended.unwrap_err();
+    }
+    auto out = mla_decode_impl(query, *cache, kv_b, layer, position, spec, nullptr);
+    if (out.is_err()) {
+        (void)cache->truncate_layer_rows(layer, position); // a failed call leaves the cache length alone
+    }
+    return out;
+}
+
+Result<RocmTensor> RocmContext::mla_prefill_attention_rope(const RocmTensor& query, const RocmTensor& latent, const RocmTensor& k_rope,
+                                                           const RocmWeight& kv_b, RocmKvCache* cache, size_t layer, size_t position,
+                                                           const std::vector<float>& cos, const std::vector<float>& sin, const MlaSpec& spec) const
+{
+    if (cache == nullptr) {
+        return compute_error("L" + std::to_string(layer) + " ROCm MLA prefill needs a paged cache");
+    }
+    if (query.rows != latent.rows) {
+        return compute_error("Rocm MLA prefill shape mismatch: Q rows=" + std::to_string(query.rows) + " latent rows=" + std::to_string(latent.rows));
+    }
+    const size_t before = cache->len(layer);
+    auto appended = append_mla_rope(*cache, layer, latent, k_rope, spec.qk_rope_head_dim, spec.rotary_layout, position, cos, sin);
+    if (appended.is_err()) {
+        return appended.unwrap_err();
+    }
+    auto out = mla_decode_impl(query, *cache, kv_b, layer, before, spec, nullptr);
+    if (out.is_err()) {
+        (void)cache->truncate_layer_rows(layer, before);
+    }
     return out;
 }
 
@@ -855,6 +1155,14 @@ Result<Unit> RocmContext::upload_layers(RocmKvCache& cache, const std::vector<st
             !record.latent_scales.has_value() || record.rows > cache.max_tokens_ || record.latent.size() != record.rows * cache.cols_ ||
             record.latent_scales->size() != record.rows * (cache.cols_ / 64) * 2 || record.rope.size() != record.rows * cache.rope_cols_ * 2) {
             return compute_error("L" + std::to_string(l) + " ROCm KV snapshot: record shape does not match the cache");
+        }
+        if (record.rows != 0) {
+            // the restored rows are committed in one step, at the capacity the growth rule gives for them
+            // (upload_cache_buffer, src/backend/rocm/mod.rs:324-333)
+            auto reserved = cache.reserve_rows(l, record.rows, stream_);
+            if (reserved.is_err()) {
+                return reserved.unwrap_err();
+            }
         }
         RocmKvCache::Layer& planes = cache.layers_[l];
         const size_t row_bytes[3] = {cache.cols_, cache.cols_ / 64 * 2, cache.rope_cols_ * 2};

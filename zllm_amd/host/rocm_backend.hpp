@@ -3,6 +3,8 @@
 // behaviour follow the reference's backend traits for this path:
 //   GqaPrefillBackend::gqa_prefill_attention_cached   src/backend/mod.rs:1484-1494, ROCm body
 //                                                     src/backend/rocm/attention.rs:2202-2254
+//   GqaPrefillBackend::gqa_prefill_attention_cached_{visible,from}   src/backend/mod.rs:1495-1513
+//   MlaPrefillBackend::mla_prefill_attention{,_rope}  src/backend/mod.rs:1134-1152, attention.rs:1732-1764
 //   DecodeBackend::{append_mla, append_mla_rope,
 //                   mla_decode_attention}             src/backend/mod.rs:1162-1180, attention.rs:1805-1832
 //   CausalWindow::{key_range, cache_capacity}         src/attention/gqa.rs:54-75
@@ -126,6 +128,17 @@ struct RocmDsaState {
 
 enum class KvCacheFormat { F16, Q8g64 };
 
+// How a cache hands out pages.  Identity is the reference's policy (block i -> physical block i, one table built at
+// full capacity, src/backend/rocm/mod.rs:335-379): planes then start small and grow by doubling.  Scrambled places
+// the pages in a fixed pseudo-random order over the whole pool, which commits the pool up front; it exists to drive
+// the kernels through a table that is not the identity.
+enum class TablePolicy { Identity, Scrambled };
+
+// Rows a cache plane holds after an append that needs `required` of at most `limit` rows: unchanged when it already
+// holds them, else the larger of `required`, twice `current` and 64, rounded up to 64 rows and capped at `limit`
+// (committed_cache_rows, src/backend/rocm/mod.rs:303-313).
+Result<size_t> committed_cache_rows(size_t current, size_t required, size_t limit);
+
 enum class RocmKvOwnership { Full = 0, BlockParity0 = 1, BlockParity1 = 2, InterleavedPair = 3 };
 
 // Host form of one MLA layer for session snapshots (the reference's MlaLayerSerde, src/backend/rocm/kv_cache.rs:2067-2083):
@@ -148,10 +161,16 @@ Result<MlaLayerSerde> read_mla_layer(const std::vector<uint8_t>& in, size_t& off
 class RocmKvCache {
   public:
     // Q8g64 GQA cache: K codes, K scales (f16), V codes, V scales per layer
-    static Result<RocmKvCache> new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens);
+    static Result<RocmKvCache> new_gqa(size_t layers, size_t num_kv_heads, size_t head_dim, size_t block_tokens, size_t max_tokens,
+                                       TablePolicy policy = TablePolicy::Identity);
     // MLA cache: Q8g64 latent (bf16 scales) + bf16 rope per layer
-    static Result<RocmKvCache> new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens);
+    static Result<RocmKvCache> new_mla(size_t layers, size_t latent_dim, size_t rope_dim, size_t block_tokens, size_t max_tokens,
+                                       TablePolicy policy = TablePolicy::Identity);
     size_t len(size_t layer) const { return layer < lens_.size() ? lens_[layer] : 0; }
+    // rows the layer's planes hold right now (grows with the appends under TablePolicy::Identity)
+    size_t committed_rows(size_t layer) const { return layer < layers_.size() ? layers_[layer].committed_rows : 0; }
+    // 0, or the number of rows a sliding-window layer keeps as a ring (token t in slot t % capacity)
+    size_t ring_capacity(size_t layer) const { return layer < layers_.size() ? layers_[layer].ring_capacity : 0; }
     // Rollback: only the logical length moves, pages and the kept prefix stay where they are and the next append
     // overwrites the tail (truncate_rows / truncate_layer_rows, src/backend/rocm/kv_cache.rs:509-586).
     Result<Unit> truncate_rows(size_t rows);
@@ -165,8 +184,18 @@ class RocmKvCache {
     friend class RocmContext;
     struct Layer {
         DeviceBuffer a_codes, a_scales, b_codes, b_scales; // GQA: K, V; MLA: latent codes / scales, rope in b_codes
+        size_t committed_rows = 0;
+        size_t ring_capacity = 0;
     };
+    static Result<RocmKvCache> create(bool mla, size_t layers, size_t cols, size_t rope_cols, size_t block_tokens, size_t max_tokens,
+                                      TablePolicy policy);
+    // bytes of one row in each of the layer's planes (0 = plane unused)
+    void plane_row_bytes(size_t (&bytes)[4]) const;
+    // make the layer's planes hold `required` rows (grow_cache_buffer, src/backend/rocm/mod.rs:315-322: a larger
+    // buffer, the used prefix copied device to device on `stream`)
+    Result<Unit> reserve_rows(size_t layer, size_t required, hipStream_t stream);
     bool mla_ = false;
+    TablePolicy policy_ = TablePolicy::Identity;
     size_t cols_ = 0, rope_cols_ = 0, block_tokens_ = 0, max_tokens_ = 0, pool_rows_ = 0;
     std::vector<Layer> layers_;
     std::vector<size_t> lens_;
@@ -188,11 +217,28 @@ class RocmContext {
 
     // Appends the chunk's K/V rows at `position` (must equal the layer's cached length), then attends:
     // one row -> split-KV decode, more rows -> chunked prefill (causal, optional sliding window).
-    // Returns f32 [rows, num_heads * head_dim].  `retain_full_cache` is accepted for signature parity:
-    // this cache always keeps every row.
+    // Returns f32 [rows, num_heads * head_dim].  A sliding-window layer appended with retain_full_cache == false keeps
+    // only CausalWindow::cache_capacity rows, as a ring (HybridGqaCacheLayout, src/kv_cache/mod.rs:397-456); such a layer
+    // takes a multi-row chunk at position 0 only, as the reference's CPU backend does (src/backend/cpu/attention.rs:401-409).
+    // The cache length moves only after every launch of the call was accepted.
     Result<RocmTensor> gqa_prefill_attention_cached(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
                                                     const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
                                                     bool retain_full_cache) const;
+    // The same with explicit visible ends per chunk row (multimodal blocks; src/backend/mod.rs:1495-1511).
+    Result<RocmTensor> gqa_prefill_attention_cached_visible(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query,
+                                                            const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                            const std::vector<uint32_t>& visible_ends, bool retain_full_cache) const;
+    // Attention of a layer that shares another layer's K/V (src/backend/mod.rs:1513): nothing is appended, the source
+    // layer must already hold position + rows rows.
+    Result<RocmTensor> gqa_prefill_attention_cached_from(const RocmKvCache& cache, size_t source_layer, size_t position, const RocmTensor& query,
+                                                         const GqaSpec& spec) const;
+    // MlaPrefillBackend: append the chunk, then attend with one query row per chunk row (causal inside the chunk).
+    // Returns bf16 [rows, heads * value_dim] for more than one row, f32 for one (src/backend/rocm/attention.rs:17-19).
+    Result<RocmTensor> mla_prefill_attention(const RocmTensor& query, const RocmTensor& latent, const RocmTensor& k_rope, const RocmWeight& kv_b,
+                                             RocmKvCache* cache, size_t layer, const MlaSpec& spec) const;
+    Result<RocmTensor> mla_prefill_attention_rope(const RocmTensor& query, const RocmTensor& latent, const RocmTensor& k_rope, const RocmWeight& kv_b,
+                                                  RocmKvCache* cache, size_t layer, size_t position, const std::vector<float>& cos,
+                                                  const std::vector<float>& sin, const MlaSpec& spec) const;
     Result<Unit> append_mla(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope) const;
     Result<Unit> append_mla_rope(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
                                  RotaryLayout layout, size_t position, const std::vector<float>& cos, const std::vector<float>& sin) const;
@@ -210,8 +256,21 @@ class RocmContext {
     Result<RocmDsaState> dsa_state_from_selection(const std::vector<uint32_t>& selection) const;
 
   private:
+    // Device scratch of the context's stream, kept between calls: the split-KV workspace (grown when a call needs
+    // more) and a ring of small metadata records (lengths, window starts) that travel host -> device from pinned memory,
+    // so that a call neither allocates nor waits for the stream.
+    struct Scratch;
+    Result<void*> workspace(size_t bytes) const;
+    Result<const uint32_t*> upload_meta(const uint32_t (&values)[4]) const;
+    Result<Unit> append_gqa_rows(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& key, const RocmTensor& value) const;
+    Result<RocmTensor> gqa_attend(const RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query, const GqaSpec& spec,
+                                  const uint32_t* visible_ends_dev) const;
+    Result<RocmTensor> gqa_cached_impl(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query, const RocmTensor& key,
+                                       const RocmTensor& value, const GqaSpec& spec, const std::vector<uint32_t>* visible_ends,
+                                       bool retain_full_cache) const;
     Result<RocmTensor> mla_decode_impl(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer, size_t position,
                                        const MlaSpec& spec, const RocmDsaState* state) const;
+    std::shared_ptr<Scratch> scratch_;
     Result<Unit> append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
                                  RotaryLayout layout, size_t position, const float* cos_dev, const float* sin_dev) const;
     int device_id_ = 0;
