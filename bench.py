@@ -176,9 +176,11 @@ def build_gqa_pool(args, lens, hq, hkv, d, block_tokens):
                                                pool_bytes=pool_rows * bytes_per_row, max_code_offset=span_bytes)
 
 
-def gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, block_tokens, scale, budget_s=12.0):
-    """The CPU oracle (port of the reference's f32 path: dequantize the Q8g64 rows, then causal_head_range per
-    (token, head) task) over the whole batch, repeated until about `budget_s` seconds of CPU work are spent."""
+def gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, block_tokens, scale, budget_s=10.0):
+    """The CPU oracle over the whole batch in the two modes the reference's CPU code has, each repeated until about
+    `budget_s` seconds of CPU work are spent: `value` = dequantize the Q8g64 rows to f32, then causal_head_range per
+    (token, head) task (what its CpuKvCache holds and runs); `direct_q8` = attention straight over the Q8 rows, values
+    formed from the codes on the fly (the way its absorbed MLA path reads the Q8 latent)."""
     import oracle as O
     from zllm_amd import ops
 
@@ -215,9 +217,24 @@ def gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, block_tokens, scal
         t_att += p_att
     median = float(np.median(passes))
     n = len(passes)
+    direct_passes = []
+    direct_out = np.zeros_like(outs)
+    started = time.perf_counter()
+    while time.perf_counter() - started < budget_s or not direct_passes:
+        t0 = time.perf_counter()
+        for b, l in enumerate(lens):
+            rc, out = O.gqa_decode_q8_direct(q_host[b], host[b]["k_codes"], host[b]["k_scales"].view(np.uint16), host[b]["v_codes"],
+                                             host[b]["v_scales"].view(np.uint16), O.SCALE_F16, 0, l, hq, hkv, d, scale)
+            assert rc == 0
+            direct_out[b] = out
+        direct_passes.append(time.perf_counter() - t0)
+    direct_median = float(np.median(direct_passes))
     return dict(value=round(total_bytes / median / 1e9, 3), unit="GB/s", cores=threads, kind="port",
                 sample=f"whole batch ({len(lens)} sequences, all heads), {n} passes in {sum(passes):.1f}s, median pass {median:.3f}s; "
-                       f"per pass: dequantize {t_deq / n:.3f}s + f32 attention {t_att / n:.3f}s"), outs
+                       f"per pass: dequantize {t_deq / n:.3f}s + f32 attention {t_att / n:.3f}s",
+                direct_q8=dict(value=round(total_bytes / direct_median / 1e9, 3), unit="GB/s", cores=threads,
+                               sample=f"same batch, attention straight over the Q8g64 rows: {len(direct_passes)} passes, median pass {direct_median:.3f}s",
+                               max_abs_vs_dequantize_mode=float(np.abs(direct_out - outs).max()))), outs
 
 
 def run_gqa_decode(args, ragged, config1=False):

@@ -208,6 +208,21 @@ def gqa_prefill_at_visible(query, key, value, kv_start, kv_end, position, num_he
     return rc, out
 
 
+def gqa_decode_q8_direct(query, k_codes, k_scales, v_codes, v_scales, scale_dtype, first, length, num_heads, num_kv_heads, head_dim,
+                         score_scale, softcap=0.0):
+    """Decode attention of one sequence straight over dense Q8g64 rows (no f32 K/V): query [Hq*d] f32 -> [Hq*d] f32."""
+    query = _c(query, np.float32).reshape(-1)
+    k_codes = np.ascontiguousarray(k_codes).view(np.int8)
+    v_codes = np.ascontiguousarray(v_codes).view(np.int8)
+    k_scales = np.ascontiguousarray(k_scales)
+    v_scales = np.ascontiguousarray(v_scales)
+    out = np.empty(num_heads * head_dim, dtype=np.float32)
+    rc = lib().zo_gqa_decode_q8_direct(_p(query), _p(k_codes), _p(k_scales), _p(v_codes), _p(v_scales), C.c_int(scale_dtype),
+                                       C.c_uint64(first), C.c_uint64(length), C.c_uint64(num_heads), C.c_uint64(num_kv_heads),
+                                       C.c_uint64(head_dim), C.c_float(score_scale), C.c_float(softcap), _p(out))
+    return rc, out
+
+
 def block_attention(query, key, value, num_heads, num_kv_heads, head_dim, score_scale, visible):
     query = _c(query, np.float32).reshape(-1, num_heads * head_dim)
     key = _c(key, np.float32).reshape(-1, num_kv_heads * head_dim)

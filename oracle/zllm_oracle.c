@@ -15,7 +15,9 @@
  * Parity status:
  *   - pinned: key_range, paged_row, layout arithmetic, ring write plan, bf16 /
  *     f16 conversions, the three Q8g64 quantizer rules, GQA head attention,
- *     MLA reference / absorbed-Q8 attention, RoPE apply.
+ *     MLA reference / absorbed-Q8 attention, RoPE apply; the direct-over-Q8
+ *     GQA decode (the benchmark's second CPU mode) by equality with the pinned
+ *     dequantise-then-f32 routine and by float64 NumPy.
  *   - parity unpinned: the attention-logit soft-cap (the reference has no such
  *     operation; defined here as s <- cap * tanh(s / cap) after the score
  *     scale), and the bit-level float summation order of the reference's SIMD
@@ -566,6 +568,76 @@ ZO_API int zo_gqa_prefill_at_visible_f32(const float* query, const float* key, c
         free(scratch);
     }
     return status;
+}
+
+/* The reference's second CPU mode, applied to a GQA cache: attention straight over the Q8g64 rows, values formed as
+ * (float)code * scale on the fly and nothing materialised in f32, the way absorbed_attention_row_q8_scalar works over
+ * the Q8 latent (src/kernel/cpu/mla.rs:771-829: score pass over the codes, two-pass softmax, weighted sum over the
+ * codes again).  One task per (sequence, head).  k_codes / v_codes are dense rows [len, kv_heads * head_dim] of one
+ * sequence, scales [len, kv_heads * head_dim / 64] in `scale_dtype`; the last row's query sees [first, len).
+ * Same arithmetic as zo_gqa_prefill_at_visible_f32 over the dequantised rows up to the order of the dot product's
+ * partial sums (sequential here, eight lanes there). */
+ZO_API int zo_gqa_decode_q8_direct(const float* query, const int8_t* k_codes, const void* k_scales, const int8_t* v_codes,
+                                   const void* v_scales, int scale_dtype, uint64_t first, uint64_t len, uint64_t num_heads,
+                                   uint64_t num_kv_heads, uint64_t head_dim, float score_scale, float softcap, float* output)
+{
+    if (num_heads == 0 || num_kv_heads == 0 || head_dim == 0 || head_dim % 64 != 0 || num_heads % num_kv_heads != 0 ||
+        !isfinite(score_scale) || score_scale <= 0.0f) {
+        return -1;
+    }
+    uint64_t cols = num_kv_heads * head_dim, groups = cols / 64, group = num_heads / num_kv_heads;
+    uint64_t count = len > first ? len - first : 0;
+#pragma omp parallel
+    {
+        float* scores = (float*)malloc((size_t)(count + 1) * sizeof(float));
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t head = 0; head < (int64_t)num_heads; ++head) {
+            uint64_t kv_head = (uint64_t)head / group;
+            const float* q = query + (uint64_t)head * head_dim;
+            float* out = output + (uint64_t)head * head_dim;
+            float maximum = -INFINITY;
+            for (uint64_t i = 0; i < count; ++i) {
+                uint64_t t = first + i;
+                const int8_t* row = k_codes + t * cols + kv_head * head_dim;
+                float score = 0.0f;
+                for (uint64_t g = 0; g < head_dim / 64; ++g) {
+                    float scale = zo_scale_at(k_scales, t * groups + kv_head * (head_dim / 64) + g, scale_dtype);
+                    for (uint64_t c = 0; c < 64; ++c) {
+                        score += q[g * 64 + c] * ((float)row[g * 64 + c] * scale);
+                    }
+                }
+                score *= score_scale;
+                if (softcap > 0.0f) {
+                    score = softcap * tanhf(score / softcap);
+                }
+                maximum = fmaxf(maximum, score);
+                scores[i] = score;
+            }
+            float denominator = 0.0f;
+            for (uint64_t i = 0; i < count; ++i) {
+                scores[i] = expf(scores[i] - maximum);
+                denominator += scores[i];
+            }
+            for (uint64_t c = 0; c < head_dim; ++c) {
+                out[c] = 0.0f;
+            }
+            if (count != 0 && isfinite(denominator) && denominator != 0.0f) {
+                for (uint64_t i = 0; i < count; ++i) {
+                    uint64_t t = first + i;
+                    float probability = scores[i] / denominator;
+                    const int8_t* row = v_codes + t * cols + kv_head * head_dim;
+                    for (uint64_t g = 0; g < head_dim / 64; ++g) {
+                        float scale = zo_scale_at(v_scales, t * groups + kv_head * (head_dim / 64) + g, scale_dtype);
+                        for (uint64_t c = 0; c < 64; ++c) {
+                            out[g * 64 + c] += probability * ((float)row[g * 64 + c] * scale);
+                        }
+                    }
+                }
+            }
+        }
+        free(scores);
+    }
+    return 0;
 }
 
 /* src/attention/block.rs:67-119 (attention_f32): explicit per-row visible

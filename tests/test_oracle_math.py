@@ -321,3 +321,43 @@ def test_rmsnorm_heads_and_sigmoid_gate_against_float64(oracle):
     rc, per_row = oracle.sigmoid_gate(out, gate[:, :1])
     assert rc == 0
     assert np.abs(per_row - out / (1.0 + np.exp(-gate[:, :1].astype(np.float64)))).max() < 1e-6
+
+
+def test_gqa_decode_direct_over_q8_equals_dequantise_then_f32(oracle):
+    """The second CPU mode (values formed from the codes on the fly, src/kernel/cpu/mla.rs:771-829 style) against the
+    pinned dequantise-then-f32 routine and against float64 NumPy: same products, so they agree to f32 summation order.
+    A dropped scale, a wrong head offset or a shifted visible range would not."""
+    rng = np.random.default_rng(17)
+    for hq, hkv, d, length, first, sdt, rule, softcap in [(8, 2, 128, 300, 0, oracle.SCALE_F16, oracle.RULE_METAL_GQA, 0.0),
+                                                          (4, 4, 64, 77, 13, oracle.SCALE_BF16, oracle.RULE_ROCM_MLA, 0.0),
+                                                          (16, 8, 256, 150, 100, oracle.SCALE_F16, oracle.RULE_METAL_GQA, 50.0)]:
+        cols = hkv * d
+        k = rng.standard_normal((length, cols)).astype(np.float32)
+        v = rng.standard_normal((length, cols)).astype(np.float32)
+        planes = {n: np.zeros((length, cols if "codes" in n else cols // 64), dtype=np.int8 if "codes" in n else np.uint16)
+                  for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+        oracle.q8g64_append_paged(rule, k, planes["k_codes"], planes["k_scales"], None, 0, 1)
+        oracle.q8g64_append_paged(rule, v, planes["v_codes"], planes["v_scales"], None, 0, 1)
+        q = rng.standard_normal(hq * d).astype(np.float32)
+        scale = 1.0 / np.sqrt(d)
+        rc, direct = oracle.gqa_decode_q8_direct(q, planes["k_codes"], planes["k_scales"], planes["v_codes"], planes["v_scales"], sdt, first,
+                                                 length, hq, hkv, d, scale, softcap)
+        assert rc == 0
+        kd = oracle.gather_dequant_rows(oracle.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, None, 1, 0, length, cols)
+        vd = oracle.gather_dequant_rows(oracle.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, None, 1, 0, length, cols)
+        window = length - first if first else 0
+        rc, two_step = oracle.gqa_prefill_at_visible(q[None, :], kd, vd, 0, length, length - 1, hq, hkv, d, window=window, score_scale=scale,
+                                                     softcap=softcap)
+        assert rc == 0
+        np.testing.assert_allclose(direct, two_step[0], rtol=0, atol=2e-6)
+        # float64, from the definition
+        want = np.zeros(hq * d)
+        for h in range(hq):
+            kh = kd[first:, (h // (hq // hkv)) * d:(h // (hq // hkv) + 1) * d].astype(np.float64)
+            vh = vd[first:, (h // (hq // hkv)) * d:(h // (hq // hkv) + 1) * d].astype(np.float64)
+            s = kh @ q[h * d:(h + 1) * d].astype(np.float64) * scale
+            if softcap:
+                s = softcap * np.tanh(s / softcap)
+            p = np.exp(s - s.max())
+            want[h * d:(h + 1) * d] = (p / p.sum()) @ vh
+        np.testing.assert_allclose(direct, want, rtol=0, atol=5e-6)
