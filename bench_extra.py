@@ -155,6 +155,96 @@ def run_mla_decode(args):
     print(json.dumps(record))
 
 
+def run_mla_prefill(args):
+    """Chunked MLA prefill: one sequence, a 512-row chunk appended to a 16,384-token prefix (causal inside the chunk),
+    128 heads, latent 512 Q8g64 + rope 64 bf16, 64-token pages in a random permutation, bf16 queries and bf16 output.
+    Every chunk row runs as one query row of the split-KV kernels over the same pages."""
+    import torch
+
+    import oracle as O
+    from zllm_amd import capi, ops
+
+    dev = "cuda"
+    heads, nope, rope, value, latent, bt, prefix, rows = 128, 128, 64, 128, 512, 64, 16384, 512
+    ctx = prefix + rows
+    ops.init(0)
+    rng = np.random.default_rng(args.seed)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed)
+    need_blocks = (ctx + bt - 1) // bt
+    pool_blocks = need_blocks * 8
+    pool_rows = pool_blocks * bt
+    codes = torch.empty((pool_rows, latent), dtype=torch.int8, device=dev)
+    scales = torch.empty((pool_rows, latent // 64), dtype=torch.int16, device=dev)
+    rope_cache = torch.empty((pool_rows, rope), dtype=torch.int16, device=dev)
+    ids = rng.choice(pool_blocks, size=need_blocks, replace=False).astype(np.uint32).reshape(1, -1)
+    tables = torch.from_numpy(ids.view(np.int32)).to(dev)
+    for pos in range(0, ctx, 2048):
+        n = min(2048, ctx - pos)
+        ops.mla_append(torch.randn((n, latent), generator=gen, device=dev), torch.randn((n, rope), generator=gen, device=dev), codes, scales,
+                       rope_cache, tables[0], pos, bt)
+    q = torch.randn((rows, heads * (nope + rope)), generator=gen, device=dev).to(torch.bfloat16)
+    kv_b = (torch.randn((heads * (nope + value), latent), generator=gen, device=dev) / np.sqrt(latent)).to(torch.bfloat16)
+    lens_dev = torch.tensor([ctx], dtype=torch.int32, device=dev)
+    call, out, workspace = ops.mla_decode_args(q, kv_b, codes, scales, rope_cache, tables, lens_dev, heads, nope + rope, nope + value, latent,
+                                               rope, bt, ctx, out_dtype=torch.bfloat16, out_compact=True, query_rows=rows)
+    lib = capi.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(mask):
+        def fn():
+            call.stage_mask = mask
+            capi.check(lib.zllm_attn_mla_decode(C.byref(call), stream))
+        return fn
+
+    steps, warmup = max(1, args.steps // 10), max(1, args.warmup // 10)
+    for _ in range(warmup):
+        run(0)()
+    ms_step = _event_ms(run(0), steps)
+    stage_ms = {name: _event_ms(run(mask), steps) for name, mask in
+                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge_project", capi.MLA_MERGE | capi.MLA_PROJECT))}
+    run(0)()
+    torch.cuda.synchronize()
+    pairs = rows * prefix + rows * (rows + 1) // 2
+    flops = pairs * heads * (2 * (latent + rope) + 2 * latent)
+    tflops = flops / (ms_step * 1e-3) / 1e12
+    achieved = flops / (stage_ms["partial"] * 1e-3) / 1e12
+    record = {
+        "metric": "MLA chunked prefill attn TFLOP/s (% of bf16 MFMA peak), 1 GPU", "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"absorbed MLA prefill chunk, B=1, {rows} rows on a {prefix}-token prefix, 128 heads, latent 512 Q8g64 + rope 64 bf16, 64-token pages",
+                   "algorithmic_flops_per_call": flops, "seed": args.seed, "workspace_bytes": int(workspace.numel())},
+        "pct_of_mfma_peak": round(100.0 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        "tokens_per_s": round(rows / (ms_step * 1e-3), 1),
+        "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
+        "roofline": {"bound": "mfma", "kernel": "mla_partial_ws", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel_ms": round(stage_ms["partial"], 5)},
+    }
+    if not args.no_cpu_baseline:
+        # CPU oracle on a bounded sample: the last four chunk rows, heads 0..3, over the whole history
+        sample_rows, sample_heads = 4, 4
+        threads = O.set_threads(min(len(os.sched_getaffinity(0)), 16))
+        h_codes = ops.gather_rows(codes, tables[0], 0, ctx, latent, bt).cpu().numpy()
+        h_scales = ops.gather_rows(scales, tables[0], 0, ctx, latent // 64 * 2, bt).cpu().numpy().view(np.uint16)
+        h_rope = ops.gather_rows(rope_cache, tables[0], 0, ctx, rope * 2, bt).cpu().numpy().view(np.uint16)
+        spec = O.MlaSpec(latent, rope, sample_heads * (nope + rope), sample_heads * (nope + value), sample_heads)
+        q_bits = q[rows - sample_rows:].view(torch.int16).cpu().numpy().view(np.uint16)[:, : sample_heads * (nope + rope)]
+        w = kv_b.float().cpu().numpy()[: sample_heads * (nope + value)]
+        t0 = time.perf_counter()
+        rc, _, out_f, _ = O.mla_absorbed_q8_history(spec, np.ascontiguousarray(q_bits), sample_rows, ctx - sample_rows, h_codes, h_scales, 64, h_rope,
+                                                    ctx, w)
+        seconds = time.perf_counter() - t0
+        assert rc == 0
+        cpu_flops = sample_rows * ctx * sample_heads * (2 * (latent + rope) + 2 * latent)
+        record["cpu_baseline"] = {"value": round(cpu_flops / seconds / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                                  "sample": f"last {sample_rows} chunk rows, heads 0..{sample_heads - 1}, {ctx} tokens; {seconds:.2f}s"}
+        got = out[rows - sample_rows:].float().cpu().numpy().reshape(sample_rows, heads, value)[:, :sample_heads].reshape(-1)
+        excess = np.abs(got - out_f) - np.abs(out_f) * 2.0 ** -7  # bf16 output: beyond one bf16 step of the oracle's unrounded value
+        record["parity_vs_oracle_max_abs_beyond_bf16_step"] = float(max(excess.max(), 0.0))
+    print(json.dumps(record))
+
+
 def run_gqa_decode_f16(args):
     """C3: f16 KV cache, B=4, 16q/8kv, d=256, ctx 8192, soft-cap 50; the full layer and the sliding layer (window 1024) are
     timed as two calls of the same entry point.  `value` is the full layer (268 MB of KV per call)."""
@@ -267,6 +357,8 @@ def run_gqa_decode_f16(args):
 def run(args):
     if args.workload == "mla_decode_64k":
         run_mla_decode(args)
+    elif args.workload == "mla_prefill_chunk":
+        run_mla_prefill(args)
     elif args.workload == "gqa_decode_f16_window":
         run_gqa_decode_f16(args)
     elif args.workload == "gqa_prefill_chunk":

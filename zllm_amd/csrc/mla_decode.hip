@@ -124,6 +124,65 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
     }
 }
 
+// The same absorb for a prefill chunk: a workgroup takes R query rows of one head, so a weight word read from memory
+// serves R rows (with one row per workgroup a 2,048-row chunk reads the 16 MiB of absorb weights 2,048 times).  Every
+// row's sum still runs over k in ascending order with separately rounded products: the bits are those of mla_absorb.
+template <int R> __global__ __launch_bounds__(256) void mla_absorb_rows(MlaDecodeParams p)
+{
+    const unsigned int head = blockIdx.x;
+    const unsigned int row0 = blockIdx.y * R;
+    __shared__ float q_sh[R][256]; // the nope part of a head's query (at most 256 columns on this path)
+    for (unsigned int i = threadIdx.x; i < R * p.q_head_dim; i += 256) {
+        const unsigned int r = i / p.q_head_dim, c = i % p.q_head_dim;
+        const unsigned int row = min(row0 + r, p.batch - 1u);
+        const float x = load_as_f32(p.q, ((size_t)row * p.heads + head) * p.q_head_dim + c, p.q_dtype);
+        const float rounded = bf16_bits_to_f32(f32_to_bf16_bits(x));
+        if (c < p.nope_dim) {
+            q_sh[r][c] = rounded;
+        } else if (row0 + r < p.batch) {
+            p.absorbed[((size_t)row * p.heads + head) * (p.latent_dim + p.rope_dim) + p.latent_dim + (c - p.nope_dim)] = f32_to_bf16_bits(rounded);
+        }
+    }
+    __syncthreads();
+    const unsigned int pairs = p.latent_dim / 2u;
+    const unsigned int* w = (const unsigned int*)(p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim);
+    for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
+#pragma clang fp contract(off)
+        float acc0[R], acc1[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            acc0[r] = 0.0f;
+            acc1[r] = 0.0f;
+        }
+        for (unsigned int k0 = 0; k0 < p.nope_dim; k0 += 16u) {
+            unsigned int word[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                word[u] = w[(size_t)min(k0 + u, p.nope_dim - 1u) * pairs + c2];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (k0 + u < p.nope_dim) {
+                    const float w0 = __uint_as_float(word[u] << 16), w1 = __uint_as_float(word[u] & 0xffff0000u);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const float x = q_sh[r][k0 + u];
+                        acc0[r] = acc0[r] + x * w0;
+                        acc1[r] = acc1[r] + x * w1;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (row0 + r < p.batch) {
+                unsigned short* qa = p.absorbed + ((size_t)(row0 + r) * p.heads + head) * (p.latent_dim + p.rope_dim);
+                *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0[r]) | ((unsigned int)f32_to_bf16_bits(acc1[r]) << 16);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
@@ -903,6 +962,107 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
     project_head(p, head, b, x);
 }
 
+// Split merge and projection for a prefill chunk: a workgroup takes R query rows of one head.  A chunk row usually has
+// one or two splits, so each thread folds all splits of its (row, column quad) itself -- two rows at a time over the
+// 256 threads, no exchange between threads -- and writes the merged row to LDS; the projection then reads every weight
+// vector once and applies it to the R merged rows, instead of once per row.
+template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(MlaDecodeParams p)
+{
+    static_assert(R % 2 == 0, "two rows are merged at a time");
+    const unsigned int head = blockIdx.x;
+    const unsigned int row0 = blockIdx.y * R;
+    const unsigned int quad = threadIdx.x & 127u;
+    // a merged row sits in LDS as eight slices of 64 columns, each padded by four floats: the projection's lanes read the
+    // same position of all eight slices at once, which an unpadded row puts on one bank group
+    constexpr unsigned int kSlice = 64 + 4;
+    __shared__ __align__(16) float merged[R][8 * kSlice];
+    for (int r = (int)(threadIdx.x >> 7); r < R; r += 2) {
+        const unsigned int b = min(row0 + r, p.batch - 1u);
+        unsigned int seq;
+        const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
+        const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+        const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+        const size_t stat_stride = (size_t)p.heads * 2;
+        const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+        const size_t partial_stride = (size_t)p.heads * kLatent;
+        float m = kNegInf, l = 0.0f;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (unsigned int c0 = 0; c0 < chunks; c0 += 4u) {
+            float cm[4], cl[4];
+            f32x4 part[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const unsigned int c = min(c0 + u, chunks - 1u);
+                const bool live = c0 + u < chunks;
+                const float2 st = *(const float2*)(stats + c * stat_stride);
+                cm[u] = live ? st.x : kNegInf;
+                cl[u] = live ? st.y : 0.0f;
+                part[u] = *(const f32x4*)(partial + c * partial_stride);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (cl[u] > 0.0f) {
+                    const float nm = fmaxf(m, cm[u]);
+                    const float a = __builtin_amdgcn_exp2f(m - nm);
+                    const float w = __builtin_amdgcn_exp2f(cm[u] - nm);
+                    acc = acc * a + part[u] * w;
+                    l = l * a + cl[u] * w;
+                    m = nm;
+                }
+            }
+        }
+        f32x4 result = {0.f, 0.f, 0.f, 0.f};
+        if (l > 0.0f && l < __builtin_inff()) {
+            result = acc * (1.0f / l);
+        }
+        *(f32x4*)(&merged[r][(quad >> 4) * kSlice + (quad & 15u) * 4u]) = result;
+    }
+    __syncthreads();
+    // projection: lane = (value column v0 + lane / 8, slice lane % 8 of 64 latent columns), as in project_head
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int wave = threadIdx.x >> 6;
+    const unsigned int slice = lane & 7u;
+    const unsigned int sub = lane >> 3;
+    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 64u;
+    const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
+    for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
+        const unsigned int v = v0 + sub;
+        const unsigned int vr = min(v, p.value_dim - 1u);
+        u32x4 raw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 8 * i);
+        }
+        for (int r = 0; r < R; ++r) {
+            const float* x = &merged[r][slice * kSlice];
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const f32x4 x0 = *(const f32x4*)(x + 8 * i), x1 = *(const f32x4*)(x + 8 * i + 4);
+                sum = fmaf(x0[0], __uint_as_float(raw[i][0] << 16), sum);
+                sum = fmaf(x0[1], __uint_as_float(raw[i][0] & 0xffff0000u), sum);
+                sum = fmaf(x0[2], __uint_as_float(raw[i][1] << 16), sum);
+                sum = fmaf(x0[3], __uint_as_float(raw[i][1] & 0xffff0000u), sum);
+                sum = fmaf(x1[0], __uint_as_float(raw[i][2] << 16), sum);
+                sum = fmaf(x1[1], __uint_as_float(raw[i][2] & 0xffff0000u), sum);
+                sum = fmaf(x1[2], __uint_as_float(raw[i][3] << 16), sum);
+                sum = fmaf(x1[3], __uint_as_float(raw[i][3] & 0xffff0000u), sum);
+            }
+            sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x114, 0xf, 0xf, true)); // row_shr:4
+            sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x112, 0xf, 0xf, true)); // row_shr:2
+            sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x111, 0xf, 0xf, true)); // row_shr:1
+            if (slice == 7u && v < p.value_dim && row0 + r < p.batch) {
+                const size_t at = ((size_t)(row0 + r) * p.heads + head) * out_stride + v;
+                if (p.out_dtype == 0) {
+                    ((float*)p.out)[at] = sum;
+                } else {
+                    ((unsigned short*)p.out)[at] = f32_to_bf16_bits(sum);
+                }
+            }
+        }
+    }
+}
+
 } // namespace
 
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
@@ -910,7 +1070,11 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     const unsigned int stages = stage_mask == 0 ? 15u : stage_mask;
     hipError_t err = hipSuccess;
     if (stages & 1u) {
-        mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        if (p.batch >= 16u && p.nope_dim <= 256u) { // a prefill chunk: eight rows share every weight load
+            mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
+        } else {
+            mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        }
         err = hipGetLastError();
         if (err != hipSuccess) {
             return err;
@@ -932,7 +1096,11 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if ((stages & 12u) == 12u) {
-        mla_merge_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        if (p.batch >= 16u) { // a prefill chunk: eight rows share every weight load of the projection
+            mla_merge_project_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
+        } else {
+            mla_merge_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        }
         return hipGetLastError();
     }
     if (stages & 4u) {
