@@ -92,32 +92,55 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
         // the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
         q_sh[i] = bf16_bits_to_f32(f32_to_bf16_bits(x));
     }
-    __syncthreads();
     unsigned short* qa = p.absorbed + ((size_t)b * p.heads + head) * (p.latent_dim + p.rope_dim);
-    // a thread owns two adjacent latent columns: one 4-byte weight load per k, 32 of them requested before the
-    // first is used (the sums themselves stay strictly sequential in k)
+    // a thread owns two adjacent latent columns: one 4-byte weight load per k (the sums themselves stay strictly
+    // sequential in k)
     const unsigned int pairs = p.latent_dim / 2u;
     const unsigned int* w = (const unsigned int*)(p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim);
-    for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
-        // product and sum rounded separately, as in the CPU code (plain operators: the __fmul_rn / __fadd_rn intrinsics
-        // are ordinary operators from a header compiled with fusing allowed)
+    if (pairs == 256u && p.nope_dim == 128u) {
+        // the usual geometry (latent 512, nope 128): all 128 weight words of the thread are requested at once, before the
+        // query has even arrived in LDS -- the kernel is one memory round trip long instead of four
+        const unsigned int c2 = threadIdx.x;
+        unsigned int word[128];
+#pragma unroll
+        for (int k = 0; k < 128; ++k) {
+            word[k] = w[(size_t)k * 256u + c2];
+        }
+        __syncthreads();
+        {
+            // product and sum rounded separately, as in the CPU code
 #pragma clang fp contract(off)
-        float acc0 = 0.0f, acc1 = 0.0f;
-        for (unsigned int k0 = 0; k0 < p.nope_dim; k0 += 32u) {
-            unsigned int word[32];
+            float acc0 = 0.0f, acc1 = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 32; ++u) {
-                word[u] = w[(size_t)min(k0 + u, p.nope_dim - 1u) * pairs + c2];
+            for (int k = 0; k < 128; ++k) {
+                acc0 = acc0 + q_sh[k] * __uint_as_float(word[k] << 16);
+                acc1 = acc1 + q_sh[k] * __uint_as_float(word[k] & 0xffff0000u);
             }
+            *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
+        }
+    } else {
+        __syncthreads();
+        for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
+            // product and sum rounded separately, as in the CPU code (plain operators: the __fmul_rn / __fadd_rn intrinsics
+            // are ordinary operators from a header compiled with fusing allowed)
+#pragma clang fp contract(off)
+            float acc0 = 0.0f, acc1 = 0.0f;
+            for (unsigned int k0 = 0; k0 < p.nope_dim; k0 += 32u) {
+                unsigned int word[32];
 #pragma unroll
-            for (int u = 0; u < 32; ++u) {
-                if (k0 + u < p.nope_dim) {
-                    acc0 = acc0 + q_sh[k0 + u] * __uint_as_float(word[u] << 16);
-                    acc1 = acc1 + q_sh[k0 + u] * __uint_as_float(word[u] & 0xffff0000u);
+                for (int u = 0; u < 32; ++u) {
+                    word[u] = w[(size_t)min(k0 + u, p.nope_dim - 1u) * pairs + c2];
+                }
+#pragma unroll
+                for (int u = 0; u < 32; ++u) {
+                    if (k0 + u < p.nope_dim) {
+                        acc0 = acc0 + q_sh[k0 + u] * __uint_as_float(word[u] << 16);
+                        acc1 = acc1 + q_sh[k0 + u] * __uint_as_float(word[u] & 0xffff0000u);
+                    }
                 }
             }
+            *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
         }
-        *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
     }
     for (unsigned int r = threadIdx.x; r < p.rope_dim; r += 256) {
         qa[p.latent_dim + r] = f32_to_bf16_bits(q_sh[p.nope_dim + r]);
@@ -813,16 +836,17 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
 // 4. project value
 // ---------------------------------------------------------------------------------------------
 // 256 threads = 4 waves.  A wave works on eight value columns at a time: lane = (column v0 + lane / 8, slice
-// lane % 8 of 64 latent columns); the lane keeps its 64 weighted values in registers, reads its 64 weights as
-// eight 16-byte vectors, and the eight slices are summed with DPP row shifts.  The weight rows of a head are
-// read exactly once, as whole 128-byte lines.
+// lane % 8); slice s owns the latent columns 64 i + 8 s .. + 8 for i = 0..7, so that the eight slices of a column
+// fetch one whole 128-byte line of its weight row per load instruction (with 64 consecutive columns per slice every
+// instruction touched 64 different lines: measured, the projection took 12 us of a 16 us kernel).  The lane keeps its
+// 64 weighted values in registers and the eight slices are summed with DPP row shifts.
 __device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned int head, unsigned int b, const float (&x)[64])
 {
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int wave = threadIdx.x >> 6;
     const unsigned int slice = lane & 7u;
     const unsigned int sub = lane >> 3;
-    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 64u;
+    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 8u;
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     const size_t out_base = ((size_t)b * p.heads + head) * out_stride;
     for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
@@ -831,7 +855,7 @@ __device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned 
         u32x4 raw[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 8 * i);
+            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 64 * i);
         }
         float sum = 0.0f;
 #pragma unroll
@@ -861,11 +885,11 @@ __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
-    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * kLatent + (threadIdx.x & 7u) * 64u;
-    float x[64];
+    const float* weighted = p.weighted + ((size_t)b * p.heads + head) * kLatent + (threadIdx.x & 7u) * 8u;
+    float x[64]; // x[8 i + e] = column 64 i + 8 slice + e
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const f32x4 t = *(const f32x4*)(weighted + 4 * i);
+        const f32x4 t = *(const f32x4*)(weighted + 64 * (i >> 1) + 4 * (i & 1));
         x[4 * i] = t[0];
         x[4 * i + 1] = t[1];
         x[4 * i + 2] = t[2];
@@ -877,13 +901,33 @@ __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
 // grid = (heads, batch): split merge and projection in one kernel when both stages run.  The merge is the
 // log-sum-exp combine of the split records (same algebra as the stand-alone merge, base 2): threads =
 // (128 column quads) x (2 split lanes), all loads of a lane issued before any is used; the merged row goes
-// through LDS to the projection's register layout instead of through the workspace.
+// through LDS to the projection's register layout instead of through the workspace.  With the usual value width
+// (128 columns) a thread's weight vectors for all four passes of the projection are requested first of all, so that
+// the kernel is two memory round trips long (sequence length, then records and weights together) instead of seven.
 __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
     const unsigned int quad = threadIdx.x & 127u;
     const unsigned int sl = threadIdx.x >> 7;
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int wave = threadIdx.x >> 6;
+    const unsigned int slice = lane & 7u;
+    const unsigned int sub = lane >> 3;
+    const bool wide = p.value_dim == 128u;
+    u32x4 raw[4][8];
+    const unsigned short* w_head = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 8u;
+    if (wide) {
+        const unsigned short* w = w_head;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            const unsigned int v = wave * 8u + 32u * pass + sub;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                raw[pass][i] = *(const u32x4*)(w + (size_t)v * kLatent + 64 * i);
+            }
+        }
+    }
     unsigned int seq;
     const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
     const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
@@ -893,11 +937,12 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
     const size_t partial_stride = (size_t)p.heads * kLatent;
     float m = kNegInf, l = 0.0f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (unsigned int c0 = sl; c0 < chunks; c0 += 16u) {
-        float cm[8], cl[8];
-        f32x4 part[8];
+    // sixteen records per trip and lane: a sequence of up to 32 splits is one round trip
+    for (unsigned int c0 = sl; c0 < chunks; c0 += 32u) {
+        float cm[16], cl[16];
+        f32x4 part[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 16; ++u) {
             const unsigned int c = min(c0 + 2u * u, chunks - 1u);
             const bool live = c0 + 2u * u < chunks;
             const float2 st = *(const float2*)(stats + c * stat_stride);
@@ -906,7 +951,7 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
             part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 16; ++u) {
             if (cl[u] > 0.0f) {
                 const float nm = fmaxf(m, cm[u]);
                 const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
@@ -949,17 +994,56 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
         *(f32x4*)(merged + quad * 4u) = result;
     }
     __syncthreads();
-    float x[64];
-    const float* row = merged + (threadIdx.x & 7u) * 64u;
+    if (wide) { // the other two passes' weights travel while the merged row is read back
+#pragma unroll
+        for (int pass = 2; pass < 4; ++pass) {
+            const unsigned int v = wave * 8u + 32u * pass + sub;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                raw[pass][i] = *(const u32x4*)(w_head + (size_t)v * kLatent + 64 * i);
+            }
+        }
+    }
+    float x[64]; // x[8 i + e] = column 64 i + 8 slice + e: the eight slices read 256 contiguous bytes at a time
+    const float* row = merged + slice * 8u;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const f32x4 t = *(const f32x4*)(row + 4 * i);
+        const f32x4 t = *(const f32x4*)(row + 64 * (i >> 1) + 4 * (i & 1));
         x[4 * i] = t[0];
         x[4 * i + 1] = t[1];
         x[4 * i + 2] = t[2];
         x[4 * i + 3] = t[3];
     }
-    project_head(p, head, b, x);
+    if (!wide) {
+        project_head(p, head, b, x);
+        return;
+    }
+    // same arithmetic and order as project_head, on the weights fetched at the start
+    const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
+    const size_t out_base = ((size_t)b * p.heads + head) * out_stride;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const unsigned int v = wave * 8u + 32u * pass + sub;
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                sum = fmaf(x[8 * i + 2 * e], __uint_as_float(raw[pass][i][e] << 16), sum);
+                sum = fmaf(x[8 * i + 2 * e + 1], __uint_as_float(raw[pass][i][e] & 0xffff0000u), sum);
+            }
+        }
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x114, 0xf, 0xf, true)); // row_shr:4
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x112, 0xf, 0xf, true)); // row_shr:2
+        sum += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(sum), 0x111, 0xf, 0xf, true)); // row_shr:1
+        if (slice == 7u) {
+            if (p.out_dtype == 0) {
+                ((float*)p.out)[out_base + v] = sum;
+            } else {
+                ((unsigned short*)p.out)[out_base + v] = f32_to_bf16_bits(sum);
+            }
+        }
+    }
 }
 
 // Split merge and projection for a prefill chunk: a workgroup takes R query rows of one head.  A chunk row usually has
@@ -972,10 +1056,7 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
     const unsigned int head = blockIdx.x;
     const unsigned int row0 = blockIdx.y * R;
     const unsigned int quad = threadIdx.x & 127u;
-    // a merged row sits in LDS as eight slices of 64 columns, each padded by four floats: the projection's lanes read the
-    // same position of all eight slices at once, which an unpadded row puts on one bank group
-    constexpr unsigned int kSlice = 64 + 4;
-    __shared__ __align__(16) float merged[R][8 * kSlice];
+    __shared__ __align__(16) float merged[R][kLatent];
     for (int r = (int)(threadIdx.x >> 7); r < R; r += 2) {
         const unsigned int b = min(row0 + r, p.batch - 1u);
         unsigned int seq;
@@ -1015,7 +1096,7 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
         if (l > 0.0f && l < __builtin_inff()) {
             result = acc * (1.0f / l);
         }
-        *(f32x4*)(&merged[r][(quad >> 4) * kSlice + (quad & 15u) * 4u]) = result;
+        *(f32x4*)(&merged[r][quad * 4u]) = result;
     }
     __syncthreads();
     // projection: lane = (value column v0 + lane / 8, slice lane % 8 of 64 latent columns), as in project_head
@@ -1023,7 +1104,7 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
     const unsigned int wave = threadIdx.x >> 6;
     const unsigned int slice = lane & 7u;
     const unsigned int sub = lane >> 3;
-    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 64u;
+    const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 8u;
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
         const unsigned int v = v0 + sub;
@@ -1031,14 +1112,14 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
         u32x4 raw[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 8 * i);
+            raw[i] = *(const u32x4*)(w + (size_t)vr * kLatent + 64 * i);
         }
         for (int r = 0; r < R; ++r) {
-            const float* x = &merged[r][slice * kSlice];
+            const float* x = &merged[r][slice * 8u]; // columns 64 i + 8 slice .. + 8, as the weights
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const f32x4 x0 = *(const f32x4*)(x + 8 * i), x1 = *(const f32x4*)(x + 8 * i + 4);
+                const f32x4 x0 = *(const f32x4*)(x + 64 * i), x1 = *(const f32x4*)(x + 64 * i + 4);
                 sum = fmaf(x0[0], __uint_as_float(raw[i][0] << 16), sum);
                 sum = fmaf(x0[1], __uint_as_float(raw[i][0] & 0xffff0000u), sum);
                 sum = fmaf(x0[2], __uint_as_float(raw[i][1] << 16), sum);
