@@ -405,3 +405,16 @@ def test_config2_full_size(ragged):
                               16, 0, lens[b], 1024).astype(np.float64)
     mean = v.reshape(lens[b], 8, 128).mean(0)
     assert np.abs(zero[b].reshape(64, 128) - np.repeat(mean, 8, axis=0)).max() < 1e-4
+
+
+@pytest.mark.parametrize("d,hq,hkv,lens,block_tokens,window", [(128, 16, 4, [700, 33, 2049], 16, 0), (64, 8, 2, [300, 1], 16, 0),
+                                                              (256, 8, 2, [1500, 97], 64, 128), (128, 8, 8, [555], 4, 0)])
+def test_f32_scale_cache(d, hq, hkv, lens, block_tokens, window):
+    """Q8g64 with f32 scales, the CUDA backend's convention (src/kernel/cuda/attention.rs:331-341, dequantised at :391):
+    the appends write such caches (tests/test_gpu_append.py), the decode kernels read them."""
+    case = make_gqa_q8_case(d + len(lens), lens, hq, hkv, d, block_tokens=block_tokens, rule=O.RULE_CUDA_GQA)
+    assert case["scale_dtype"] == O.SCALE_F32
+    scale = 1.0 / np.sqrt(d)
+    got = run_decode(case, scale, window=window)
+    want = oracle_gqa_decode(case, scale, window=window)
+    print("f32 scales", d, assert_attention_close(got, want, f"f32 scales d={d}"))

@@ -21,7 +21,7 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     total = prefix + chunk
     tables, pool_blocks = draw_tables(rng, [total], block_tokens)
     rows = pool_blocks * block_tokens
-    sdt = O.SCALE_F16 if rule == O.RULE_METAL_GQA else O.SCALE_BF16
+    sdt = {O.RULE_METAL_GQA: O.SCALE_F16, O.RULE_ROCM_MLA: O.SCALE_BF16, O.RULE_CUDA_GQA: O.SCALE_F32}[rule]
     gain = np.ones(cols, dtype=np.float32)
     if outliers:  # 1 % of the channels carry values eight times larger
         gain[rng.choice(cols, size=max(1, cols // 100), replace=False)] = 8.0
@@ -31,7 +31,8 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     # the chunk's K/V arrive as bf16 activations
     k[prefix:] = O.bf16_to_f32(O.f32_to_bf16(k[prefix:]))
     v[prefix:] = O.bf16_to_f32(O.f32_to_bf16(v[prefix:]))
-    planes = {n: np.zeros((rows, cols if "codes" in n else cols // 64), dtype=np.int8 if "codes" in n else np.uint16)
+    planes = {n: np.zeros((rows, cols if "codes" in n else cols // 64),
+                          dtype=np.int8 if "codes" in n else (np.float32 if rule == O.RULE_CUDA_GQA else np.uint16))
               for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
     # prefix already cached (oracle quantizer); host copy of the full cache for the oracle
     O.q8g64_append_paged(rule, k, planes["k_codes"], planes["k_scales"], tables[0], 0, block_tokens)
@@ -285,3 +286,9 @@ def test_prefill_f16_kv(d, prefix, chunk, window, softcap):
     rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
     assert rc == 0
     print("prefill f16", d, assert_attention_close(out.cpu().numpy(), want, f"f16 KV prefill d={d}"))
+
+
+def test_prefill_f32_scale_cache():
+    """A chunk over a cache with f32 scales (CUDA convention): appended by the library, attended through the decode kernels."""
+    out, want = run_case(321, 400, 60, 16, 4, rule=O.RULE_CUDA_GQA)
+    print("prefill f32 scales", assert_attention_close(out.cpu().numpy(), want, "f32-scale prefill"))

@@ -136,8 +136,8 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
     if (a->kv_format != ZLLM_KV_Q8G64 && a->kv_format != ZLLM_KV_F16) {
         return fail(-1, "GQA decode: unknown kv_format %d", a->kv_format);
     }
-    if (a->kv_format == ZLLM_KV_Q8G64 && a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
-        return fail(-1, "GQA decode: Q8g64 scales must be bf16 or f16 (got %d)", a->scale_dtype);
+    if (a->kv_format == ZLLM_KV_Q8G64 && (a->scale_dtype < ZLLM_SCALE_BF16 || a->scale_dtype > ZLLM_SCALE_F32)) {
+        return fail(-1, "GQA decode: Q8g64 scales must be bf16, f16 or f32 (got %d)", a->scale_dtype);
     }
     if (a->kv_format == ZLLM_KV_F16 && a->head_dim == 64) {
         return fail(-1, "GQA decode: f16 KV supports head_dim 128 and 256");
@@ -863,8 +863,8 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     if (a->num_heads / a->num_kv_heads > 256) {
         return fail(-1, "GQA prefill: at most 256 query heads per KV head");
     }
-    if (a->kv_format == ZLLM_KV_Q8G64 && a->scale_dtype != ZLLM_SCALE_BF16 && a->scale_dtype != ZLLM_SCALE_F16) {
-        return fail(-1, "GQA prefill: Q8g64 scales must be bf16 or f16 (got %d)", a->scale_dtype);
+    if (a->kv_format == ZLLM_KV_Q8G64 && (a->scale_dtype < ZLLM_SCALE_BF16 || a->scale_dtype > ZLLM_SCALE_F32)) {
+        return fail(-1, "GQA prefill: Q8g64 scales must be bf16, f16 or f32 (got %d)", a->scale_dtype);
     }
     if (a->table != nullptr && a->table_stride != 0 && (uint64_t)a->table_stride * a->block_tokens < (uint64_t)a->position + a->rows) {
         return fail(-1, "GQA prefill: table_stride=%u pages of %u tokens cannot cover position + rows = %llu", a->table_stride,
@@ -882,13 +882,13 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     return 0;
 }
 
-// head_dim 128 over Q8g64 runs the matrix-core chunk kernel, which keeps all of its state on chip.  Every other
-// geometry (head_dim 64 / 256, f16 KV) runs each row of the chunk as one item of the split-KV decode kernels: row r is a
+// head_dim 128 over Q8g64 with 16-bit scales runs the matrix-core chunk kernel, which keeps all of its state on chip.
+// Every other geometry (head_dim 64 / 256, f16 KV, f32 scales) runs each row of the chunk as one item of the split-KV decode kernels: row r is a
 // sequence of position + r + 1 tokens over the same block table.  That route re-reads the KV bytes per row, so it is
 // bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and the split records.
 static bool prefill_rows_as_decode_items(const zllm_gqa_prefill_args* a)
 {
-    return a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64;
+    return a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64 || a->scale_dtype == ZLLM_SCALE_F32;
 }
 
 static void prefill_decode_args(const zllm_gqa_prefill_args* a, zllm_gqa_decode_args* d)

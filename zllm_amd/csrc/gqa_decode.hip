@@ -78,15 +78,37 @@ template <> struct ScaleRow<4> {
     }
 };
 
+// f32 scales (the CUDA backend's convention, src/kernel/cuda/attention.rs:331-341): G floats per token and KV head.
+template <int G> struct ScaleRowF32 {
+    float v[G];
+    __device__ __forceinline__ float get(int a) const { return v[a]; }
+};
+// Row type and value of a stored scale for a scale dtype (0 bf16, 1 f16, 2 f32).
+template <int G, int SDT> struct ScaleRowOf {
+    typedef ScaleRow<G> type;
+};
+template <int G> struct ScaleRowOf<G, 2> {
+    typedef ScaleRowF32<G> type;
+};
+template <int SDT, class Row> __device__ __forceinline__ float scale_of(const Row& row, int a)
+{
+    if constexpr (SDT == 2) {
+        return row.get(a);
+    } else {
+        return scale_bits_to_f32<SDT>(row.get(a));
+    }
+}
+
 // Everything one wave loads for a 32-token step of a Q8g64 cache.
 //   FAST (pages of >= 16 tokens): the 16 scale rows a 16-lane row needs in a step (2 tiles x 4 token slots x
 //   {K, V}) are loaded one per lane and handed out with DPP row broadcasts — one load instead of sixteen.
 //   Generic: every lane loads the scale rows of its eight token slots itself.
-template <int G, bool FAST> struct Q8Step {
+template <int G, bool FAST, int SDT> struct Q8Step {
+    typedef typename ScaleRowOf<G, SDT>::type Row;
     u32x4 k[2][G];        // K codes: tile i, group a -> 16 codes of the lane's token
     unsigned int v[8][G]; // V codes: token slot s = i*4 + r, group a -> 4 codes (dims a*64 + 4m .. +4)
-    ScaleRow<G> ks[FAST ? 1 : 8]; // FAST: lane x of a row holds scale row (kv = x>>3, tile (x>>2)&1, slot x&3)
-    ScaleRow<G> vs[FAST ? 1 : 8];
+    Row ks[FAST ? 1 : 8]; // FAST: lane x of a row holds scale row (kv = x>>3, tile (x>>2)&1, slot x&3)
+    Row vs[FAST ? 1 : 8];
 };
 
 // lane `n` of each 16-lane row, broadcast to the row (v_mov_b32 row_newbcast)
@@ -265,8 +287,8 @@ __device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsi
 //   k[i][a]   16 K codes of the lane's token of tile i, scale group a (raw bytes = int8 MFMA A operand)
 //   ksr[i*4+r] scale row of token slot (tile i, row 4j + r) -- the C layout of the score tile
 // Leaves the step's probabilities in pr[] (same slots) and rescales acc when the running max moved.
-template <int G, int SDT, bool SOFTCAP>
-__device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const ScaleRow<G> (&ksr)[8], const i32x4 (&qhi)[G],
+template <int G, int SDT, bool SOFTCAP, class Row>
+__device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Row (&ksr)[8], const i32x4 (&qhi)[G],
                                             const i32x4 (&qlo)[G], float scale_log2, float inv_cap, float cap_log2,
                                             unsigned int t0, unsigned int j, unsigned int first, unsigned int len,
                                             float& run_max, float& run_sum, f32x4 (&acc)[G * 4], float (&pr)[8])
@@ -290,7 +312,7 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Sc
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                tile_s[r] = fmaf(d[r], scale_bits_to_f32<SDT>(ksr[i * 4 + r].get(a)), tile_s[r]);
+                tile_s[r] = fmaf(d[r], scale_of<SDT>(ksr[i * 4 + r], a), tile_s[r]);
             }
         }
 #pragma unroll
@@ -331,8 +353,8 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Sc
 
 // Second half: O^T += V^T . P' with P' = p * v_scale split into bf16 hi + lo.
 //   v[i*4+r][a]  4 V codes (dims a*64 + 4m .. +4) of token slot (tile i, row 4j + r)
-template <int G, int SDT>
-__device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const ScaleRow<G> (&vsr)[8], const float (&pr)[8],
+template <int G, int SDT, class Row>
+__device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const Row (&vsr)[8], const float (&pr)[8],
                                     f32x4 (&acc)[G * 4])
 {
     // ---- O^T += V^T . P', P' = p * v_scale split into bf16 hi + lo --------------------
@@ -341,8 +363,8 @@ __device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const Sca
         Frag phi, plo;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float x0 = pr[2 * e] * scale_bits_to_f32<SDT>(vsr[2 * e].get(a));
-            const float x1 = pr[2 * e + 1] * scale_bits_to_f32<SDT>(vsr[2 * e + 1].get(a));
+            const float x0 = pr[2 * e] * scale_of<SDT>(vsr[2 * e], a);
+            const float x1 = pr[2 * e + 1] * scale_of<SDT>(vsr[2 * e + 1], a);
             unsigned int hi, lo;
             split_bf16_pair(x0, x1, hi, lo);
             phi.u[e] = hi;
@@ -367,8 +389,8 @@ __device__ __forceinline__ void pv_step(const unsigned int (&v)[8][G], const Sca
 // [first, len) are whatever their page holds.  Their probabilities are exact zeros, but 0 * scale is NaN when the
 // stale scale bits read as NaN or infinity, and one NaN in P' poisons every dimension of the head.  Clearing the
 // scale rows of those slots (wave-uniform test, edge steps only) makes them contribute exact zeros.
-template <int G>
-__device__ __forceinline__ void clear_hidden_scale_rows(ScaleRow<G> (&vsr)[8], unsigned int t0, unsigned int j, unsigned int first,
+template <int G, class Row>
+__device__ __forceinline__ void clear_hidden_scale_rows(Row (&vsr)[8], unsigned int t0, unsigned int j, unsigned int first,
                                                         unsigned int len)
 {
     if (t0 >= first && t0 + 32u <= len) {
@@ -378,7 +400,7 @@ __device__ __forceinline__ void clear_hidden_scale_rows(ScaleRow<G> (&vsr)[8], u
     for (int e = 0; e < 8; ++e) {
         const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
         if (token < first || token >= len) {
-            vsr[e] = ScaleRow<G>{};
+            vsr[e] = Row{};
         }
     }
 }
@@ -390,6 +412,9 @@ template <int D, int SDT, bool FAST, bool SOFTCAP, int NBUF>
 __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(GqaDecodeParams p)
 {
     constexpr int G = D / 64;           // scale groups per head row
+    typedef typename ScaleRowOf<G, SDT>::type Row;
+    constexpr unsigned int kScaleBytes = SDT == 2 ? 4u : 2u;
+    static_assert(!(FAST && SDT == 2), "f32 scales run the generic path");
     constexpr int MT = D / 16;          // output M tiles
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int m = lane & 15u;  // MFMA row / column index of this lane
@@ -426,11 +451,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
 
     const unsigned int* table = p.tables + (p.table_shared ? 0 : (size_t)b * p.table_stride);
     const unsigned int k_row = p.num_kv_heads * D;           // bytes per cache row (codes)
-    const unsigned int s_row = p.num_kv_heads * G * 2u;      // bytes per scale row
+    const unsigned int s_row = p.num_kv_heads * G * kScaleBytes; // bytes per scale row
     const unsigned char* k_base = p.k_plane + (size_t)kvh * D;
     const unsigned char* v_base = p.v_plane + (size_t)kvh * D;
-    const unsigned char* ks_base = p.k_scales + (size_t)kvh * G * 2u;
-    const unsigned char* vs_base = p.v_scales + (size_t)kvh * G * 2u;
+    const unsigned char* ks_base = p.k_scales + (size_t)kvh * G * kScaleBytes;
+    const unsigned char* vs_base = p.v_scales + (size_t)kvh * G * kScaleBytes;
     const unsigned int block_mask = p.block_tokens - 1u;
     const unsigned int lo_tile = first & ~15u;
     const unsigned int hi_tile = (len - 1u) & ~15u;
@@ -484,7 +509,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     s_off = (4u * j + (sx & 3u)) * s_row;
     const unsigned char* s_plane = sx_value ? vs_base : ks_base;
 
-    auto load_step = [&](Q8Step<G, FAST>& s, unsigned int t0) __attribute__((always_inline)) {
+    auto load_step = [&](Q8Step<G, FAST, SDT>& s, unsigned int t0) __attribute__((always_inline)) {
         if constexpr (FAST) {
             const unsigned long long R0 = tile_row(t0);
             const unsigned long long R1 = tile_row(t0 + 16u);
@@ -506,7 +531,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
                 }
             }
             const unsigned long long Rs = sx_tile1 ? R1 : R0;
-            s.ks[0] = *(const ScaleRow<G>*)(s_plane + Rs * s_row + s_off);
+            s.ks[0] = *(const Row*)(s_plane + Rs * s_row + s_off);
         } else {
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
@@ -524,8 +549,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
                     for (int a = 0; a < G; ++a) {
                         s.v[i * 4 + r][a] = *(const unsigned int*)(vr + a * 64);
                     }
-                    s.ks[i * 4 + r] = *(const ScaleRow<G>*)(ks_base + row * s_row);
-                    s.vs[i * 4 + r] = *(const ScaleRow<G>*)(vs_base + row * s_row);
+                    s.ks[i * 4 + r] = *(const Row*)(ks_base + row * s_row);
+                    s.vs[i * 4 + r] = *(const Row*)(vs_base + row * s_row);
                 }
             }
         }
@@ -542,9 +567,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
     const float cap_log2 = p.softcap * kLog2e;
 
-    auto compute_step = [&](const Q8Step<G, FAST>& s, unsigned int t0) __attribute__((always_inline)) {
+    auto compute_step = [&](const Q8Step<G, FAST, SDT>& s, unsigned int t0) __attribute__((always_inline)) {
         // scale rows of this lane's eight token slots (K then V)
-        ScaleRow<G> ksr[8], vsr[8];
+        Row ksr[8], vsr[8];
         if constexpr (FAST) {
             ksr[0] = row_bcast_scales<G, 0>(s.ks[0]);
             ksr[1] = row_bcast_scales<G, 1>(s.ks[0]);
@@ -576,7 +601,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     };
 
     // ---- software pipeline: loads of steps n+1 .. n+NBUF-1 in flight while step n computes ----------
-    Q8Step<G, FAST> buf[NBUF];
+    Q8Step<G, FAST, SDT> buf[NBUF];
 #pragma unroll
     for (int u = 0; u < NBUF - 1; ++u) {
         if ((unsigned int)u < steps) {
@@ -1301,6 +1326,15 @@ hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block,
 
 template <int D> hipError_t launch_q8_d(const GqaDecodeParams& p, int scale_dtype, bool fast, dim3 grid, dim3 block, hipStream_t stream)
 {
+    if (scale_dtype == 2) {
+        // f32 scales: every lane fetches the scale rows of its token slots itself (the tile paths move 16-bit scales)
+        if (p.softcap > 0.0f) {
+            gqa_decode_q8_partial<D, 2, false, true, 2><<<grid, block, 0, stream>>>(p);
+        } else {
+            gqa_decode_q8_partial<D, 2, false, false, 2><<<grid, block, 0, stream>>>(p);
+        }
+        return hipGetLastError();
+    }
     if (scale_dtype == 0) {
         return launch_q8<D, 0>(p, fast, grid, block, stream);
     }
