@@ -87,7 +87,9 @@ __device__ __forceinline__ unsigned int window_exponent(float top)
     return min(max((__float_as_uint(top) >> 23) & 0xffu, 2u), 252u);
 }
 
-template <int SDT, bool SOFTCAP>
+// POW2: pages of a power-of-two size behind a block table, known at compile time (no run-time choice of the address
+// arithmetic, no division code in the loop).
+template <int SDT, bool SOFTCAP, bool POW2>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
     __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
@@ -175,14 +177,14 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const float cap_log2 = p.softcap * kLog2e;
     const unsigned int k_row = p.num_kv_heads * kD;
     const unsigned int s_row = p.num_kv_heads * 4u; // two 16-bit scales per KV head
-    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
+    const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const unsigned int last_token = t_end - 1u;
     // The block-table entry of a staging thread's token is fetched one step before the data that needs
     // it, so no step waits on a table -> data load chain.
     auto entry_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned int {
         token = min(token, last_token);
         const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
-        return p.table != nullptr ? p.table[page] : page;
+        return (POW2 || p.table != nullptr) ? p.table[page] : page;
     };
     auto row_from = [&](unsigned int token, unsigned int entry) __attribute__((always_inline)) -> unsigned long long {
         token = min(token, last_token);
@@ -561,17 +563,19 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
     const bool cap = p.softcap > 0.0f;
+    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
+    const dim3 block(kThreads);
     if (scale_dtype == 0) {
         if (cap) {
-            gqa_prefill_q8<0, true><<<grid, dim3(kThreads), 0, stream>>>(p);
+            pow2 ? gqa_prefill_q8<0, true, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<0, true, false><<<grid, block, 0, stream>>>(p);
         } else {
-            gqa_prefill_q8<0, false><<<grid, dim3(kThreads), 0, stream>>>(p);
+            pow2 ? gqa_prefill_q8<0, false, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<0, false, false><<<grid, block, 0, stream>>>(p);
         }
     } else {
         if (cap) {
-            gqa_prefill_q8<1, true><<<grid, dim3(kThreads), 0, stream>>>(p);
+            pow2 ? gqa_prefill_q8<1, true, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<1, true, false><<<grid, block, 0, stream>>>(p);
         } else {
-            gqa_prefill_q8<1, false><<<grid, dim3(kThreads), 0, stream>>>(p);
+            pow2 ? gqa_prefill_q8<1, false, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<1, false, false><<<grid, block, 0, stream>>>(p);
         }
     }
     return hipGetLastError();

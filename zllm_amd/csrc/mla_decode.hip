@@ -252,7 +252,9 @@ constexpr int kWsTiles = 3;
 // SELECTED: the `selection` arm (src/kernel/rocm/hip/attention/paged_mla/source.hip:4738-4764): a sequence longer than
 // top_k attends to the listed token positions only.  The kernel then walks list slots instead of positions -- splits,
 // masks and softmax are over slots -- and only the address of a row goes through the list.
-template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
+// POW2: the page size is a power of two and the sequences have block tables, known at compile time: the address
+// arithmetic of a step is then shifts and masks without the run-time choice (and the division code behind it).
+template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
     static_assert(!(ALIGNED && SELECTED), "selected rows are not contiguous");
     // Staging items (token row, 16 codes) per thread: the 32 rows of a step are split 24 : 8 between the score and the
@@ -300,8 +302,8 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     const unsigned int c_start = (unsigned int)c_start64;
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + kStepTokens - 1) / kStepTokens;
-    const unsigned int* table = p.tables != nullptr ? p.tables + (size_t)seq * p.table_stride : nullptr;
-    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
+    const unsigned int* table = (POW2 || p.tables != nullptr) ? p.tables + (size_t)seq * p.table_stride : nullptr;
+    const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
 
     // ---- staging: loads of a later tile's bytes, converted by the thread that loaded them
     const unsigned int cc = tid & 31u;
@@ -328,7 +330,7 @@ template <bool ALIGNED, bool SELECTED> __global__ __launch_bounds__(512) void ml
     auto lookup_step = [&](StepRows& r, unsigned int t0) __attribute__((always_inline)) {
         if constexpr (ALIGNED) {
             const unsigned int page = pow2 ? t0 >> p.block_shift : t0 / p.block_tokens;
-            r.entry[0] = table != nullptr ? table[page] : page;
+            r.entry[0] = (POW2 || table != nullptr) ? table[page] : page;
         } else {
 #pragma unroll
             for (int i = 0; i <= ITEMS; ++i) {
@@ -1167,7 +1169,11 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         if (p.selection != nullptr) {
             mla_partial_ws<false, true><<<grid, dim3(512), 0, stream>>>(p);
         } else if (p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0) {
-            mla_partial_ws<true, false><<<grid, dim3(512), 0, stream>>>(p);
+            if ((p.block_tokens & (p.block_tokens - 1u)) == 0 && p.tables != nullptr) {
+                mla_partial_ws<true, false, true><<<grid, dim3(512), 0, stream>>>(p);
+            } else {
+                mla_partial_ws<true, false><<<grid, dim3(512), 0, stream>>>(p);
+            }
         } else {
             mla_partial_ws<false, false><<<grid, dim3(512), 0, stream>>>(p);
         }
