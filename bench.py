@@ -62,6 +62,8 @@ def probe_lib():
         lib.bench_probe_stream_read.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
         lib.bench_probe_paged_read.restype = C.c_int
         lib.bench_probe_paged_read.argtypes = [C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        lib.bench_probe_paged_read_lds.restype = C.c_int
+        lib.bench_probe_paged_read_lds.argtypes = lib.bench_probe_paged_read.argtypes
         _PROBE = lib
     return _PROBE
 
@@ -74,10 +76,11 @@ def stream_read_probe(buffer, sink):
     assert rc == 0, rc
 
 
-def paged_read_probe(planes, table_flat, workgroups, pages_in_flight, sink):
+def paged_read_probe(planes, table_flat, workgroups, pages_in_flight, sink, through_lds=False):
     import torch
 
-    rc = probe_lib().bench_probe_paged_read(planes["k_codes"].data_ptr(), planes["v_codes"].data_ptr(), planes["k_scales"].data_ptr(),
+    lib = probe_lib()
+    rc = (lib.bench_probe_paged_read_lds if through_lds else lib.bench_probe_paged_read)(planes["k_codes"].data_ptr(), planes["v_codes"].data_ptr(), planes["k_scales"].data_ptr(),
                                             planes["v_scales"].data_ptr(), table_flat.data_ptr(), table_flat.numel(), workgroups, pages_in_flight,
                                             sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0, rc
@@ -338,6 +341,12 @@ def run_gqa_decode(args, ragged, config1=False):
                 med, low = event_times_ms(lambda: paged_read_probe(planes, flat, 256, in_flight, probe_sink), 100)
                 paged[f"{in_flight}_pages_in_flight"] = {"kernel_ms_median": round(med, 5), "kernel_ms_min": round(low, 5),
                                                          "gbps_median": round(kv_bytes / (med * 1e-3) / 1e9, 1)}
+            for in_flight in (1, 2, 4):  # the same walk with the decode kernel's transport (global -> LDS loads)
+                for _ in range(10):
+                    paged_read_probe(planes, flat, 256, in_flight, probe_sink, through_lds=True)
+                med, low = event_times_ms(lambda: paged_read_probe(planes, flat, 256, in_flight, probe_sink, through_lds=True), 100)
+                paged[f"{in_flight}_pages_in_flight_through_lds"] = {"kernel_ms_median": round(med, 5), "kernel_ms_min": round(low, 5),
+                                                                     "gbps_median": round(kv_bytes / (med * 1e-3) / 1e9, 1)}
             record["roofline"]["paged_read_of_same_pages"] = paged
     if not args.no_cpu_baseline:
         cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)

@@ -77,6 +77,56 @@ template <int INFLIGHT> __global__ __launch_bounds__(512) void paged_read_kernel
     }
 }
 
+// The same walk with the decode kernel's transport: global -> LDS loads (no destination registers), each wave into a
+// private region of INFLIGHT pages, then one wait and LDS reads of what arrived.
+typedef __attribute__((address_space(3))) void* probe_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* probe_global_ptr_t;
+
+template <int INFLIGHT> __global__ __launch_bounds__(512) void paged_read_lds_kernel(const unsigned char* k_plane, const unsigned char* v_plane,
+                                                             const unsigned char* k_scales, const unsigned char* v_scales,
+                                                             const unsigned int* table, unsigned int pages, unsigned int pages_per_group,
+                                                             unsigned int* sink)
+{
+    constexpr int kPageBytes = 4 * 1024 + 256; // four code instructions and one scale instruction per page and wave
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[8 * INFLIGHT * kPageBytes];
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned int first = blockIdx.x * pages_per_group;
+    const unsigned int last = min(first + pages_per_group, pages);
+    const unsigned int lane_off = (lane >> 3) * 1024u + wave * 128u + (lane & 7u) * 16u;
+    unsigned char* const mine = lds + wave * (INFLIGHT * kPageBytes);
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    unsigned int acc_s = 0u;
+    for (unsigned int p = first; p < last; p += INFLIGHT) {
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+            const unsigned int page = __builtin_amdgcn_readfirstlane(table[min(p + u, last - 1u)]);
+            const unsigned long long base = (unsigned long long)page * 16384u;
+            unsigned char* const dst = mine + u * kPageBytes;
+            __builtin_amdgcn_global_load_lds((probe_global_ptr_t)(k_plane + base + lane_off), (probe_lds_ptr_t)(dst), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds((probe_global_ptr_t)(k_plane + base + 8192u + lane_off), (probe_lds_ptr_t)(dst + 1024), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds((probe_global_ptr_t)(v_plane + base + lane_off), (probe_lds_ptr_t)(dst + 2048), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds((probe_global_ptr_t)(v_plane + base + 8192u + lane_off), (probe_lds_ptr_t)(dst + 3072), 16, 0, 2);
+            const unsigned char* sp = (lane >= 32u ? v_scales : k_scales) + (unsigned long long)page * 512u + (lane & 15u) * 32u + wave * 4u;
+            __builtin_amdgcn_global_load_lds((probe_global_ptr_t)sp, (probe_lds_ptr_t)(dst + 4096), 4, 0, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+            const unsigned char* src = mine + u * kPageBytes;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                acc ^= *(const u32x4*)(src + w * 1024 + lane * 16u);
+            }
+            acc_s ^= *(const unsigned int*)(src + 4096 + lane * 4u);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the next trip's loads overwrite what was just read
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3] ^ acc_s) == 0x5a17c0deu && sink[0] == 0xffffffffu) {
+        sink[0] = 0u;
+    }
+}
+
 extern "C" {
 
 __attribute__((visibility("default"))) int bench_probe_stream_read(const void* src, uint64_t bytes, uint32_t* sink, void* stream)
@@ -108,6 +158,29 @@ __attribute__((visibility("default"))) int bench_probe_paged_read(const void* k_
     case 2: paged_read_kernel<2><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
     case 4: paged_read_kernel<4><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
     case 8: paged_read_kernel<8><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    default: return -1;
+    }
+    return (int)hipGetLastError();
+}
+
+// Same arguments; the loads go global -> LDS as in the decode kernel.
+__attribute__((visibility("default"))) int bench_probe_paged_read_lds(const void* k_plane, const void* v_plane, const void* k_scales,
+                                                                      const void* v_scales, const uint32_t* table, uint32_t pages,
+                                                                      uint32_t workgroups, uint32_t pages_in_flight, uint32_t* sink, void* stream)
+{
+    if (k_plane == nullptr || v_plane == nullptr || k_scales == nullptr || v_scales == nullptr || table == nullptr || sink == nullptr ||
+        pages == 0 || workgroups == 0) {
+        return -1;
+    }
+    const uint32_t per_group = (pages + workgroups - 1) / workgroups;
+    const uint32_t groups = (pages + per_group - 1) / per_group;
+    const unsigned char *kp = (const unsigned char*)k_plane, *vp = (const unsigned char*)v_plane;
+    const unsigned char *ks = (const unsigned char*)k_scales, *vs = (const unsigned char*)v_scales;
+    const hipStream_t st = (hipStream_t)stream;
+    switch (pages_in_flight) {
+    case 1: paged_read_lds_kernel<1><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    case 2: paged_read_lds_kernel<2><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
+    case 4: paged_read_lds_kernel<4><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
     default: return -1;
     }
     return (int)hipGetLastError();

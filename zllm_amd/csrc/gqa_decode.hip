@@ -687,8 +687,24 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
     const unsigned int head_block = blockIdx.y / kvh_blocks;
+    if (kvh >= p.num_kv_heads) {
+        return;
+    }
+    // The item's place in the batch depends on every sequence's length, which is one trip to memory; the block-table
+    // entries it then needs are a second one before the first row can be requested.  When every sequence fills all
+    // planned splits, item i is split i % max_chunks of sequence i / max_chunks: the entries of that guess are
+    // requested together with the lengths and are kept if the guess turns out right.
+    const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
+    const unsigned int guess_b = min(blockIdx.x / p.max_chunks, p.batch - 1u);
+    const unsigned int guess_page = ((blockIdx.x - guess_b * p.max_chunks) * p.chunk_tokens) >> p.block_shift;
+    const unsigned int* guess_table = p.tables + (p.table_shared ? 0 : (size_t)guess_b * p.table_stride);
+    unsigned int entries0 = 0, entries1 = 0;
+    if (p.tables != nullptr) {
+        entries0 = guess_table[min(guess_page + lane, last_page)];
+        entries1 = guess_table[min(guess_page + 64u + lane, last_page)];
+    }
     unsigned int b, chunk, len, first, span;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    if (!locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -720,9 +736,13 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     // block-table entries of this split: lane i holds entry first_page + i (+ 64); the launcher keeps a
     // split within 128 pages
     const unsigned int first_page = min(max(c_start, lo_tile), hi_tile) >> p.block_shift;
-    const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
-    unsigned int entries0 = p.tables != nullptr ? table[min(first_page + lane, last_page)] : first_page + lane;
-    unsigned int entries1 = p.tables != nullptr ? table[min(first_page + 64u + lane, last_page)] : first_page + 64u + lane;
+    if (p.tables == nullptr) {
+        entries0 = first_page + lane;
+        entries1 = first_page + 64u + lane;
+    } else if (table != guess_table || first_page != guess_page) {
+        entries0 = table[min(first_page + lane, last_page)];
+        entries1 = table[min(first_page + 64u + lane, last_page)];
+    }
     // the query fetch rides along with the table loads; it is quantized after the first KV loads are out
     const QueryRaw<D> q_raw = fetch_query<D>(p, b, head, head_valid, j);
     asm volatile("" : "+v"(entries0), "+v"(entries1)); // their wait happens here, not inside the loop
@@ -808,11 +828,14 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     // Issue order per step n (9 instructions): K(n+2) x4, scales(n+2) x1, [QK, softmax], V(n+2) x4.
     //   K(n), scales(n) complete  <=> at most 13 newer loads outstanding (V(n), K/S/V(n+1))
     //   V(n) complete             <=> at most 14 newer loads outstanding (K/S/V(n+1), K/S(n+2))
-    auto step = [&](auto slot_c, unsigned int n) __attribute__((always_inline)) {
+    // The last two steps of a split request nothing (behind = batches of loads still behind this step's: 2 in the
+    // steady state, then 1, then 0) and wait with the counts that follow from that.
+    auto step = [&](auto slot_c, auto behind_c, unsigned int n) __attribute__((always_inline)) {
         constexpr int slot = decltype(slot_c)::value;
+        constexpr int behind = decltype(behind_c)::value;
         const unsigned int t0 = c_start + n * 32u;
-        const unsigned int t_next = c_start + min(n + 2u, steps - 1u) * 32u; // past the end: re-read the last step
-        wait_vmcnt<13>();
+        const unsigned int t_next = c_start + (n + 2u) * 32u;
+        wait_vmcnt<behind == 0 ? 4 : 13>();
         u32x4 k[2][G];
         ScaleRow<G> ksr[8], vsr[8];
 #pragma unroll
@@ -830,11 +853,13 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
             }
         }
         wait_lds_reads();
-        issue_codes(k_base, lds_k, slot, t_next);
-        issue_scales(slot, t_next);
+        if (behind == 2) {
+            issue_codes(k_base, lds_k, slot, t_next);
+            issue_scales(slot, t_next);
+        }
         float pr[8];
         qk_softmax_step<G, SDT, SOFTCAP>(k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
-        wait_vmcnt<14>();
+        wait_vmcnt<behind == 2 ? 14 : behind == 1 ? 9 : 0>();
         unsigned int v[8][G];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -845,18 +870,33 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
             }
         }
         wait_lds_reads();
-        issue_codes(v_base, lds_v, slot, t_next);
+        if (behind == 2) {
+            issue_codes(v_base, lds_v, slot, t_next);
+        }
         clear_hidden_scale_rows<G>(vsr, t0, j, first, len);
         pv_step<G, SDT>(v, vsr, pr, acc);
     };
+    using slot0 = std::integral_constant<int, 0>;
+    using slot1 = std::integral_constant<int, 1>;
+    using behind0 = std::integral_constant<int, 0>;
+    using behind1 = std::integral_constant<int, 1>;
+    using behind2 = std::integral_constant<int, 2>;
 
     unsigned int n = 0;
-    for (; n + 2u <= steps; n += 2u) {
-        step(std::integral_constant<int, 0>{}, n);
-        step(std::integral_constant<int, 1>{}, n + 1u);
+    for (; n + 4u <= steps; n += 2u) { // both steps have two more behind them
+        step(slot0{}, behind2{}, n);
+        step(slot1{}, behind2{}, n + 1u);
     }
-    if (n < steps) {
-        step(std::integral_constant<int, 0>{}, n);
+    const unsigned int rest = steps - n; // 1 (a one-step split), 2 or 3
+    if (rest == 3u) {
+        step(slot0{}, behind2{}, n);
+        step(slot1{}, behind1{}, n + 1u);
+        step(slot0{}, behind0{}, n + 2u);
+    } else if (rest == 2u) {
+        step(slot0{}, behind1{}, n);
+        step(slot1{}, behind0{}, n + 1u);
+    } else {
+        step(slot0{}, behind1{}, n); // the prologue's second batch (a repeat of the first) is still behind it
     }
     wait_vmcnt<0>(); // no load may still be writing this workgroup's LDS when the wave ends
 
@@ -1204,17 +1244,23 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     float m = kNegInf;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float l = 0.0f;
-    for (unsigned int c0 = sl; c0 < chunks; c0 += 4u * lanes) {
+    // Record addresses are clamped to the planned splits, not to this sequence's own count, so that the first trip's
+    // loads do not wait for the length: what a dead split's record holds is never used.
+    for (unsigned int c0 = sl; c0 == sl || c0 < chunks; c0 += 4u * lanes) {
         float cm[4], cl[4];
         f32x4 part[4];
+        float2 st[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const unsigned int c = min(c0 + u * lanes, chunks - 1u);
-            const bool live = c0 + u * lanes < chunks;
-            const float2 st = *(const float2*)(stats + c * stat_stride);
-            cm[u] = live ? st.x : kNegInf;
-            cl[u] = live ? st.y : 0.0f;
+            const unsigned int c = min(c0 + u * lanes, p.max_chunks - 1u);
+            st[u] = *(const float2*)(stats + c * stat_stride);
             part[u] = *(const f32x4*)(partial + c * partial_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool live = c0 + u * lanes < chunks;
+            cm[u] = live ? st[u].x : kNegInf;
+            cl[u] = live ? st[u].y : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
