@@ -27,9 +27,14 @@ def _event_ms(fn, steps):
 
 
 def _wall_ms(fn, steps):
+    """Wall clock per call over exactly `steps` calls, after 0.1 s of untimed calls: the device needs some milliseconds of
+    work to return to its running clocks after the idle stretch a graph capture leaves."""
     import torch
 
-    torch.cuda.synchronize()
+    started = time.perf_counter()
+    while time.perf_counter() - started < 0.1:
+        fn()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         fn()
@@ -122,7 +127,7 @@ def run_mla_decode(args):
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "effective_kv_gbps": round(kv_bytes / (ms_step * 1e-3) / 1e9, 1),
         "ms_per_step_events": round(ms_events, 5), "ms_per_step_eager": round(ms_eager, 5),
-        "launch": f"hipGraph replay, {per_graph} decode calls (absorb + partial + merge/project each) per graph",
+        "launch": f"hipGraph replay, {per_graph} decode calls (absorb + partial + merge/project each) per graph; 0.1 s of untimed replays before the timed ones",
         "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
         "roofline": {"bound": "mfma", "kernel": "mla_partial", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
