@@ -321,8 +321,14 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Ro
             if constexpr (SOFTCAP) {
                 x = cap_log2 * fast_tanh(x * inv_cap);
             }
-            const unsigned int token = t0 + 16u * i + 4u * j + r;
-            sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;
+            sc[i * 4 + r] = x;
+        }
+    }
+    if (t0 < first || t0 + 32u > len) { // only the first and the last step of a visible range have slots to mask (wave-uniform)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+            sc[e] = (token >= first && token < len) ? sc[e] : kNegInf;
         }
     }
     // ---- online softmax (base 2) -----------------------------------------------------
