@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-Default workload = BASELINE.json configs[1]: Qwen3-style Q8g64 GQA decode, batch 8, 64 query heads /
+Default workload = benchmark configuration 1 (counted from 0): Qwen3-style Q8g64 GQA decode, batch 8, 64 query heads /
 8 KV heads, head_dim 128, every sequence at 32,768 tokens (the "32K ctx" case the metric is quoted
 on), 16-token pages scattered over a large pool, bf16 queries, K/V ~ N(0,1) with 1 % outlier
 channels x8.  One "step" = one decode attention call (split-KV partial + LSE merge) over the batch.

@@ -43,7 +43,7 @@ def _wall_ms(fn, steps):
 
 
 def run_mla_decode(args):
-    """BASELINE.json configs[3]: B=4, 128 heads, latent 512 (Q8g64, bf16 scales) + rope 64 (bf16), ctx 65,536,
+    """benchmark configuration 3 (counted from 0): B=4, 128 heads, latent 512 (Q8g64, bf16 scales) + rope 64 (bf16), ctx 65,536,
     bf16 queries, softmax scale 1/sqrt(192); W_kv_b ~ N(0, 1/512) in bf16; 64-token pages in a random permutation."""
     import torch
 

@@ -1,4 +1,4 @@
-"""bench.py --workload gqa_prefill_chunk: BASELINE.json configs[4] — a 2,048-row chunk appended to a 50,000-token
+"""bench.py --workload gqa_prefill_chunk: benchmark configuration 4 (counted from 0) — a 2,048-row chunk appended to a 50,000-token
 Q8g64 prefix, 64q/8kv, d=128, bf16 Q/K/V, 16-token pages; the chunk's K/V are quantized into fresh pages inside the
 timed step (append + attention), as the path does per chunk."""
 from __future__ import annotations

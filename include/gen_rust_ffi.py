@@ -3,7 +3,7 @@
 constants) to stdout, or into a Markdown file between the markers `<!-- ffi:begin -->` / `<!-- ffi:end -->`:
 
     python include/gen_rust_ffi.py                      # print
-    python include/gen_rust_ffi.py --into INTEGRATION.md
+    python include/gen_rust_ffi.py --into <file.md>
 
 The Rust side follows the conventions of the reference's own FFI layer (src/kernel/rocm/hip/ffi.rs:31-70,357-375):
 `#[repr(C)]` structs, raw pointers, `c_int` status codes, the stream as an opaque pointer.

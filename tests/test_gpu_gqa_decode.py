@@ -46,7 +46,7 @@ def test_decode_output_gate(per_row, gate_bf16):
 
 
 def test_config1_cpu_oracle_case():
-    """BASELINE config 1: B=1, 16q/4kv, d=128, L=4096, f32 q, f16 scales, 16-token pages, random table."""
+    """Benchmark config 1: B=1, 16q/4kv, d=128, L=4096, f32 q, f16 scales, 16-token pages, random table."""
     case = make_gqa_q8_case(1, [4096], 16, 4, 128)
     scale = 1.0 / np.sqrt(128.0)
     got = run_decode(case, scale)
@@ -55,7 +55,7 @@ def test_config1_cpu_oracle_case():
 
 
 def test_config2_shape_ragged_batch_bf16_queries_outliers():
-    """BASELINE config 2 at oracle-sized lengths: B=8, 64q/8kv, ragged, bf16 q, 1 % outlier channels x8."""
+    """Benchmark config 2 at oracle-sized lengths: B=8, 64q/8kv, ragged, bf16 q, 1 % outlier channels x8."""
     rng = np.random.default_rng(2)
     lens = rng.integers(100, 3000, size=8)
     case = make_gqa_q8_case(2, lens, 64, 8, 128, outliers=True, q_bf16=True)
@@ -229,7 +229,7 @@ def run_f16(case, score_scale, window=0, softcap=0.0, ring_capacity=0):
 
 @pytest.mark.parametrize("window,ring", [(0, 0), (1024, 0), (1024, 1024)])
 def test_config3_f16_kv_sliding_window_softcap(window, ring):
-    """BASELINE config 3: B=4, 16q/8kv, d=256, ctx 8192, window 1024 on sliding layers (optionally stored as a
+    """Benchmark config 3: B=4, 16q/8kv, d=256, ctx 8192, window 1024 on sliding layers (optionally stored as a
     1024-row ring), soft-cap 50."""
     case = make_f16_case(3, [8192, 8192, 5000, 8192], 16, 8, 256, ring_capacity=ring)
     scale = 1.0 / 16.0
@@ -386,7 +386,7 @@ def _oracle_rows(case, rows, scale):
 
 @pytest.mark.parametrize("ragged", [False, True])
 def test_config2_full_size(ragged):
-    """BASELINE config 2 at its own size -- B = 8, 64q/8kv, d = 128, 16-token pages, bf16 queries, outlier channels --
+    """Benchmark config 2 at its own size -- B = 8, 64q/8kv, d = 128, 16-token pages, bf16 queries, outlier channels --
     every sequence at 32,768 tokens (the kernel instantiation and split plan the bench times) and the ragged draw in
     [1024, 32768].  The oracle runs on two sequences of the call's output; the zero-query mean is checked on one."""
     rng = np.random.default_rng(2)

@@ -99,7 +99,7 @@ def test_prefill_chunk_matches_oracle(prefix, chunk, hq, hkv):
 
 
 def test_prefill_config5_shape_at_oracle_size():
-    """BASELINE config 5 geometry (64q/8kv, d=128, bf16 activations, 16-token pages, chunk into fresh pages) with a
+    """Benchmark config 5 geometry (64q/8kv, d=128, bf16 activations, 16-token pages, chunk into fresh pages) with a
     3,000-token prefix and a 256-row chunk, which the CPU oracle finishes in seconds."""
     out, want = run_case(5, 3000, 256, 64, 8)
     print("config5-small", assert_attention_close(out.cpu().numpy(), want, "config 5 (small)"))
@@ -190,7 +190,7 @@ def test_prefill_rejects_unsupported_shapes():
 
 
 def test_prefill_config5_full_size():
-    """BASELINE config 5 at its own size: a 2,048-row chunk on a 50,000-token prefix, 64q/8kv, d = 128, bf16 activations,
+    """Benchmark config 5 at its own size: a 2,048-row chunk on a 50,000-token prefix, 64q/8kv, d = 128, bf16 activations,
     16-token pages, the chunk quantized into fresh pages by the library.  The oracle runs on the first, a middle and the
     last eight chunk rows of the full call's output."""
     segments = [(0, 8), (1020, 8), (2040, 8)]

@@ -93,7 +93,7 @@ def test_mla_decode_matches_oracle(heads, lens):
 
 
 def test_mla_decode_config4_shape_at_oracle_size():
-    """BASELINE config 4 geometry (B=4, 128 heads, latent 512 + rope 64, q_head 192, kv_head 256) at a context the
+    """Benchmark config 4 geometry (B=4, 128 heads, latent 512 + rope 64, q_head 192, kv_head 256) at a context the
     scalar oracle finishes in seconds; the full 65,536-token case is covered by the split-invariance property below."""
     case = make_mla_case(4, [4096, 3000, 4096, 257], 128)
     want_f, want_b = oracle_mla(case)
@@ -331,7 +331,7 @@ def _oracle_mla_heads(case, b, heads_picked):
 
 @pytest.mark.parametrize("block_tokens", [64, 16])
 def test_config4_full_size(block_tokens):
-    """BASELINE config 4 at its own size: B = 4, 128 heads, 65,536 tokens, with the reference's 64-token pages (the
+    """Benchmark config 4 at its own size: B = 4, 128 heads, 65,536 tokens, with the reference's 64-token pages (the
     instantiation the bench times: whole 32-row steps from one page) and with 16-token pages (per-row table lookups).
     The oracle runs on heads 0, 63, 64, 127 -- both 64-head blocks of a workgroup pair, first and last column -- of two
     sequences sliced out of the full call's output; a zero query at full length must give the projected mean latent."""

@@ -1,4 +1,4 @@
-"""INTEGRATION.md's Rust binding against include/zllm_attn.h: every structure field by field (name, order, type), every
+"""The Rust binding shown in the integration guide against include/zllm_attn.h: every structure field by field (name, order, type), every
 exported function (name, argument types, return type) and every enum constant.  A binding written from a stale doc
 passes structures of the wrong size, so any difference fails here.  Both sides are parsed in this file, independently
 of the generator that writes the doc's block (include/gen_rust_ffi.py)."""

@@ -140,7 +140,7 @@ def test_bytes_per_token_known_answers(oracle):
     assert oracle.bytes_per_token(0, 0, 4, 4) == 0 and oracle.bytes_per_token(0, 8, 0, 4) == 0
     # src/backend/rocm/kv_cache.rs:3617-3624: 512 + 16 + 128 = 656
     assert oracle.bytes_per_token(0, 512, 64, 64) == 656
-    # BASELINE configs: C1 1,056 B; C2/C5 2,112 B
+    # benchmark configs: C1 1,056 B; C2/C5 2,112 B
     assert oracle.bytes_per_token(1, 4, 128, 64) == 1056
     assert oracle.bytes_per_token(1, 8, 128, 64) == 2112
 
