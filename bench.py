@@ -320,7 +320,7 @@ def run_gqa_decode(args, ragged, config1=False):
     record = {
         "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "int8+bf16", "data": "synthetic",
         "config": {"workload": ("C1 Q8g64 GQA decode, B=1, 16q/4kv, d=128, L=4096, 16-token pages (the reference's CPU-runnable case: latency-bound on a GPU)"
                                 if config1 else "C2 Q8g64 GQA decode, B=8, 64q/8kv, d=128, " + ("ragged L~U[1024,32768]" if ragged else "all L=32768")
                                 + ", 16-token pages"),
