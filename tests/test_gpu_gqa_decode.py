@@ -375,6 +375,25 @@ def test_q8_sliding_window_ring(d, ring, window, block_tokens):
     assert_attention_close(got, want, f"Q8 ring {ring} window {window} d={d}")
 
 
+# ---------------------------------------------------------------------------- every way a split can end
+def test_splits_of_one_to_six_steps():
+    """The head_dim-128 streaming kernel runs its steps in pairs and ends a split with one, two or three steps that
+    request nothing further, each with its own wait counts.  64 sequences with one split plan of 160-token parts
+    (max_kv_len 640) give splits of 1 to 5 steps, alone and behind full parts, with and without a ragged last tile;
+    poisoned pool tails make a step that waited for too little show as NaN or as a wrong row."""
+    lens = [1, 16, 17, 32, 33, 64, 65, 96, 97, 128, 129, 159, 160, 161, 192, 200, 224, 256, 288, 320, 321, 352, 384, 400, 416, 448,
+            479, 480, 481, 512, 544, 576, 600, 608, 639, 640] + [int(x) for x in np.random.default_rng(5).integers(1, 641, size=28)]
+    case = make_gqa_q8_case(905, lens, 16, 8, 128, block_tokens=16, poison=True, q_bf16=True)
+    scale = 1.0 / np.sqrt(128.0)
+    got = run_decode(case, scale, max_kv_len=640)
+    assert np.isfinite(got).all()
+    assert_attention_close(got, oracle_gqa_decode(case, scale), "splits of 1..5 steps")
+    # one long sequence: six-step splits and more, all full
+    case = make_gqa_q8_case(906, [192 * 256], 16, 8, 128, block_tokens=16, q_bf16=True)
+    got = run_decode(case, scale)
+    assert_attention_close(got, oracle_gqa_decode(case, scale), "six-step splits")
+
+
 # ---------------------------------------------------------------------------- the benchmarked shape at its full size
 def _oracle_rows(case, rows, scale):
     sub = dict(case)
