@@ -1,4 +1,4 @@
-// Absorbed MLA decode over the paged Q8g64 latent cache — gfx950, bf16 MFMA.
+// Absorbed MLA decode over the paged Q8g64 latent cache — gfx950, f16 / bf16 MFMA.
 //
 // Stages (the reference's chain absorb -> partial -> merge -> project,
 // src/kernel/rocm/hip/attention/paged_mla.rs:3042-3621):
@@ -6,13 +6,16 @@
 //                   qa[b, h, 512:576] = bf16(q_rope[b, h, :])
 //   2. mla_partial_ws: split-KV attention of the heads against one shared latent row per token.
 //                   A workgroup owns (split, block of 64 heads, sequence).  Per 32-token step it converts
-//                   the latent codes ONCE into LDS as bf16 integers (exact) next to the bf16 rope columns
-//                   and the f32 group scales.  Four score waves (16 heads each) compute
+//                   the latent codes ONCE into LDS as f16 integers (exact) next to the bf16 rope columns,
+//                   the f32 group scales and an f16 copy of them divided by the value side's exponent window.
+//                   Four score waves (16 heads each) compute
 //                     S^T[token, head]  = sum_g scale[token, g] * (codes_g[token, :] . qa_g[head, :])
-//                                         + rope[token, :] . q_rope[head, :]     (MFMA 16x16x32 bf16,
-//                                         one accumulator per 64-column group: products are exact)
+//                                         + rope[token, :] . q_rope[head, :]     (MFMA 16x16x32 f16 on the
+//                                         latent part, bf16 on the rope part; one accumulator per 64-column
+//                                         group: products are exact)
 //                   and the online softmax; four value waves, one step behind, accumulate
-//                     O^T[dim, head]   += codes^T[dim, token] . P'_g[token, head], P'_g = bf16(p * scale_g)
+//                     O^T[dim, head]   += codes^T[dim, token] . P'_g[token, head],
+//                     P'_g = f16(p) * f16(scale_g / 2^window)   (one packed f16 multiply per two tokens)
 //                   The same row-major tile feeds both products: QK^T reads it with ds_read_b128,
 //                   P.V reads it transposed with ds_read_b64_tr_b16.  A 16-byte XOR swizzle keeps both
 //                   access patterns free of bank conflicts.
@@ -243,6 +246,10 @@ struct StepRows {
 // rotate: tile i (scores), tile i - 1 (values), tile i + 1 (being converted from the bytes the threads loaded
 // an iteration ago).  One LDS-only barrier per step.
 constexpr int kWsTiles = 3;
+// The probabilities travel from the score to the value waves as f16 of p * 2^kPShift (p <= 2^8 by the lazy rescaling, so
+// the product stays below 2^13 and p down to 2^-18 keeps f16's full precision); the f16 copy of the scale table carries
+// the inverse, so that P' = p16 * scale16 is one packed multiply per two tokens.
+constexpr int kPShift = 4;
 
 // ALIGNED: pages hold a multiple of 32 tokens (splits always start at one), so the 32 rows of a step are
 // contiguous in one page: one block-table entry per step, and every staging load takes a scalar base
@@ -263,8 +270,11 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
     constexpr int ITEMS = 3;
     __shared__ __align__(16) unsigned char lds[kWsTiles * kTileBytes];
     __shared__ __align__(16) float lds_scale[kWsTiles][8][kStepTokens]; // [buffer][group][token]
-    __shared__ __align__(16) float lds_p[2][4][2][64][4]; // [parity][head tile][token half][lane][4 tokens]: 16-byte slots
-                                                          // of consecutive lanes are contiguous (conflict-free 16-byte reads)
+    __shared__ __align__(16) u32x4 lds_p16[2][4][64]; // [parity][head tile][lane]: the step's probabilities times 2^kPShift as
+                                                      // f16, tokens (4j, 4j+1) (4j+2, 4j+3) (16+4j, ..) (16+4j+2, ..): 16-byte slots
+                                                      // of consecutive lanes are contiguous (conflict-free 16-byte reads)
+    __shared__ __align__(16) _Float16 lds_scale16[kWsTiles][8][kStepTokens]; // [buffer][group][token]: scale / 2^(window + kPShift)
+    __shared__ int lds_win[kWsTiles];                    // the window lds_scale16[buffer] was written for
     __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
     __shared__ __align__(16) float lds_top[kWsTiles][4]; // [buffer][value wave]: largest group scale the wave converted
     const unsigned int tid = threadIdx.x;
@@ -403,7 +413,9 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             }
         }
     };
-    auto convert_step = [&](const StageRegs& regs, unsigned char* tile, float (*scale_tile)[kStepTokens], float* step_top, unsigned int t0) __attribute__((always_inline)) {
+    int window = 0; // value waves: exponent window of P' (see below); the f16 scale table is written for the window of the moment
+    auto convert_step = [&](const StageRegs& regs, unsigned char* tile, float (*scale_tile)[kStepTokens], _Float16 (*scale16_tile)[kStepTokens],
+                            int* table_window, float* step_top, unsigned int t0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
             if (i >= n_items) {
@@ -435,6 +447,12 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                 sg = 0.0f; // a row past the end: its codes may be anything, its weight is an exact zero
             }
             scale_tile[scale_g][scale_t] = sg;
+            // out of the window's range the product overflows to infinity: such a step moves the window, and a table whose
+            // window is not the reader's is not used
+            scale16_tile[scale_g][scale_t] = (_Float16)(sg * __uint_as_float((unsigned int)(127 - kPShift - window) << 23));
+            if (tid == 256u) {
+                *table_window = window;
+            }
             // largest scale the wave holds, for the value waves' exponent window: rotate-and-max inside the four
             // 16-lane rows, then one lane of each row
             float top = sg;
@@ -471,7 +489,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
     if (steps > 1) {
         lookup_step(rows, c_start + kStepTokens);
     }
-    convert_step(staged, lds, lds_scale[0], lds_top[0], c_start);
+    convert_step(staged, lds, lds_scale[0], lds_scale16[0], &lds_win[0], lds_top[0], c_start);
     lds_barrier();
 
     // Both roles run the same number of iterations and barriers: iteration i scores tile i and accumulates tile
@@ -503,7 +521,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
     auto convert_to = [&](unsigned int n) __attribute__((always_inline)) { // raw bytes of step n -> tile buffer n % 3
         if (n < steps) {
             const unsigned int nb = n % kWsTiles;
-            convert_step(staged, lds + nb * kTileBytes, lds_scale[nb], lds_top[nb], c_start + n * kStepTokens);
+            convert_step(staged, lds + nb * kTileBytes, lds_scale[nb], lds_scale16[nb], &lds_win[nb], lds_top[nb], c_start + n * kStepTokens);
         }
     };
 
@@ -548,6 +566,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
         }
         float run_max = kNegInf, run_sum = 0.0f;
         float neg_ref = 0.0f; // minus the reference the scores are taken against: the running maximum, 0 before the first score
+        float neg_ref_shifted = (float)kPShift; // the same plus the hand-over shift: the scores below are log2(p * 2^kPShift)
         const float scale_log2 = p.score_scale * kLog2e;
         const float latent_log2 = scale_log2 * head_pow2;
         stage_step(1u);
@@ -626,7 +645,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                     if (q == 3) {
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            sc[t2 * 4 + r] = fmaf(s[r], latent_log2, fmaf(s_rope[r], scale_log2, neg_ref)); // relative to the reference
+                            sc[t2 * 4 + r] = fmaf(s[r], latent_log2, fmaf(s_rope[r], scale_log2, neg_ref_shifted)); // relative to the reference
                         }
                     }
                 }
@@ -647,8 +666,8 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                     lane_max = fmaxf(lane_max, sc[e]);
                 }
                 float alpha = 1.0f;
-                if (__any(lane_max > 8.0f || run_max == kNegInf)) {
-                    const float step_max = wave_max_16x4(lane_max); // relative as well
+                if (__any(lane_max > 8.0f + (float)kPShift || run_max == kNegInf)) {
+                    const float step_max = wave_max_16x4(lane_max) - (float)kPShift; // relative as well, without the shift
                     const float ref = -neg_ref;
                     float new_max = run_max;
                     if (step_max > 8.0f || run_max == kNegInf) {
@@ -663,6 +682,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                     }
                     run_max = new_max;
                     neg_ref = -safe_max;
+                    neg_ref_shifted = neg_ref + (float)kPShift;
                     run_sum *= alpha;
                 }
                 f32x4 p_lo, p_hi;
@@ -673,16 +693,16 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                     p_hi[e] = __builtin_amdgcn_exp2f(sc[4 + e]);
                     step_sum += p_lo[e] + p_hi[e];
                 }
-                run_sum += step_sum;
-                *(f32x4*)lds_p[i & 1u][hw][0][lane] = p_lo;
-                *(f32x4*)lds_p[i & 1u][hw][1][lane] = p_hi;
+                run_sum += step_sum; // in units of 2^-kPShift, like the probabilities
+                lds_p16[i & 1u][hw][lane] = u32x4{pack_f16_hw(p_lo[0], p_lo[1]), pack_f16_hw(p_lo[2], p_lo[3]),
+                                                 pack_f16_hw(p_hi[0], p_hi[1]), pack_f16_hw(p_hi[2], p_hi[3])};
                 lds_alpha[i & 1u][hw][lane] = alpha;
             }
             convert_to(i + 1u);
             stage_step(i + 2u);
             lds_barrier();
         }
-        const float total = wave_sum_16x4(run_sum);
+        const float total = wave_sum_16x4(run_sum) * (1.0f / (float)(1 << kPShift));
         if (head < p.heads && j == 0) {
             p.stats[rec * 2] = run_max;
             p.stats[rec * 2 + 1] = total;
@@ -702,23 +722,44 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                 acc[ht][t] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
-        int window = 0;
+        // exponent window of P': the accumulators hold sum(P' c) / 2^window with 2^window above the largest scale
+        // seen / 2^7, so p (<= 2^8) * scale / 2^window stays below 2^15; the window only grows, and the accumulators
+        // are rescaled by the power of two it grows by.  It starts at what tile 0 needs, so that the f16 scale table of
+        // every later tile is written for a window its reader still has, unless the scales grew in between.
+        auto window_for = [](unsigned int top_bits) __attribute__((always_inline)) -> int {
+            return min(max((int)((top_bits >> 23) & 0xffu) - 133, -96), 112);
+        };
+        {
+            const f32x4 tops = *(const f32x4*)lds_top[0];
+            window = window_for(__builtin_amdgcn_readfirstlane(__float_as_uint(fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3])))));
+        }
         unsigned int value_tile = 0; // buffer of tile i - 1
         stage_step(1u);
         const unsigned int lds_base = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)lds;
         for (unsigned int i = 0; i <= steps; ++i) {
             // the hand-over records are requested first: their LDS round trip hides behind the staging work
-            f32x4 p_lo[2], p_hi[2];
+            u32x4 p16[2];
             float alpha[2];
 #pragma unroll
             for (int ht = 0; ht < 2; ++ht) {
-                p_lo[ht] = *(const f32x4*)lds_p[(i + 1u) & 1u][2u * hp + ht][0][lane];
-                p_hi[ht] = *(const f32x4*)lds_p[(i + 1u) & 1u][2u * hp + ht][1][lane];
+                p16[ht] = lds_p16[(i + 1u) & 1u][2u * hp + ht][lane];
                 alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
             }
             const f32x4 tops = *(const f32x4*)lds_top[value_tile]; // tile i - 1
             const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3]))));
+            const int table_window = __builtin_amdgcn_readfirstlane(lds_win[value_tile]);
             asm volatile("" ::: "memory");
+            if (i > 0) {
+                // the window moves before this iteration's conversion, so that the table written now is written for it
+                const int need = window_for(top_bits);
+                if (need > window) {
+                    const float shrink = __uint_as_float((unsigned int)(127 - min(need - window, 126)) << 23);
+                    alpha[0] *= shrink;
+                    alpha[1] *= shrink;
+                    window = need;
+                }
+            }
+            const bool table_fits = table_window == window;
             __builtin_amdgcn_s_setprio(3);
             convert_to(i + 1u);
             stage_step(i + 2u);
@@ -726,28 +767,6 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             if (i > 0) {
                 // LDS byte addresses of this step: one register per fragment row, everything else is an immediate
                 const unsigned int tile_lds = lds_base + value_tile * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
-                const float* gs_base = &lds_scale[0][0][0] + value_tile * (8 * kStepTokens) + dh * (4 * kStepTokens) + 4 * j;
-                // exponent window of P': the accumulators hold sum(P' c) / 2^window with 2^window above the
-                // largest scale seen / 2^7, so p (<= 2^8) * scale / 2^window stays below 2^15; the window only
-                // grows, and the accumulators are rescaled by the power of two it grows by
-                {
-                    const int top_exp = (int)((top_bits >> 23) & 0xffu);
-                    const int need = min(max(top_exp - 133, -96), 112);
-                    if (i == 1u) {
-                        window = need;
-                    } else if (need > window) {
-                        const float shrink = __uint_as_float((unsigned int)(127 - min(need - window, 126)) << 23);
-                        alpha[0] *= shrink;
-                        alpha[1] *= shrink;
-                        window = need;
-                    }
-                    const float into_window = __uint_as_float((unsigned int)(127 - window) << 23);
-#pragma unroll
-                    for (int ht = 0; ht < 2; ++ht) {
-                        p_lo[ht] *= into_window;
-                        p_hi[ht] *= into_window;
-                    }
-                }
 #pragma unroll
                 for (int ht = 0; ht < 2; ++ht) {
                     if (__any(alpha[ht] != 1.0f)) {
@@ -766,7 +785,9 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                 };
                 // The transposed reads are written as inline assembly with immediate offsets: one address register per
                 // fragment row serves all four groups, and the waits are placed by hand (lgkmcnt, LDS operations
-                // complete in issue order) exactly one group behind the requests.
+                // complete in issue order) exactly one group behind the requests.  The scale reads are assembly as
+                // well: the compiler does not count the transposed reads, so a wait it places for a scale read of its
+                // own would also wait for every fragment requested since.
                 const unsigned int at[4] = {tile_lds + pv_base[0], tile_lds + pv_base[1], tile_lds + pv_base[2], tile_lds + pv_base[3]};
                 auto load_group = [&](VFrag (&vf)[4], int g) __attribute__((always_inline)) {
 #pragma unroll
@@ -775,41 +796,66 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                         asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vf[tt].s[1]) : "v"(at[tt]), "i"(g * 128 + 16 * kRowBytes));
                     }
                 };
-                auto scales_of = [&](int g, f32x4& gs0, f32x4& gs1) __attribute__((always_inline)) {
-                    gs0 = *(const f32x4*)(gs_base + g * kStepTokens);
-                    gs1 = *(const f32x4*)(gs_base + g * kStepTokens + 16);
-                };
                 VFrag vf[2][4];
-                f32x4 gs0[2], gs1[2];
-                load_group(vf[0], 0);
-                scales_of(0, gs0[0], gs1[0]);
+                if (!table_fits) {
+                    // The f16 table of this tile was written for another window (the first tile of a split, or the scales
+                    // grew since): the wave rewrites the 4 x 32 entries it is about to read from the f32 table.  The other
+                    // value wave of the same column half writes the same values; LDS operations of a wave complete in order.
+                    const float into_window = __uint_as_float((unsigned int)(127 - kPShift - window) << 23);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int cur = g & 1;
-                    if (g + 1 < 4) {
-                        load_group(vf[cur ^ 1], g + 1);
-                        scales_of(g + 1, gs0[cur ^ 1], gs1[cur ^ 1]);
-                        // group g's eight reads are older than the eight just issued
-                        asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
-                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1])
-                                     :
-                                     : "memory");
-                    } else {
-                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
-                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1])
-                                     :
-                                     : "memory");
+                    for (int e = 0; e < 2; ++e) {
+                        const unsigned int idx = lane + 64u * e;
+                        const unsigned int g = 4u * dh + (idx >> 5), t = idx & 31u;
+                        lds_scale16[value_tile][g][t] = (_Float16)(lds_scale[value_tile][g][t] * into_window);
                     }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                }
+                {
+                    // P'_g = p16 * scale16_g: both factors are f16 already (the probabilities from the score wave, the scales
+                    // from the conversion, divided by the window there), one packed multiply per two tokens
+                    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+                    const unsigned int gs16_lds = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const _Float16*)&lds_scale16[0][0][0] +
+                                                  (value_tile * (8 * kStepTokens) + dh * (4 * kStepTokens) + 4 * j) * 2u;
+                    auto scales16_of = [&](int g, u32x2& lo, u32x2& hi) __attribute__((always_inline)) {
+                        asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(lo) : "v"(gs16_lds), "i"(g * kStepTokens * 2));
+                        asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(hi) : "v"(gs16_lds), "i"(g * kStepTokens * 2 + 32));
+                    };
+                    auto pk_mul = [](unsigned int x, unsigned int y) __attribute__((always_inline)) -> unsigned int {
+                        return __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2_t, x) * __builtin_bit_cast(f16x2_t, y));
+                    };
+                    u32x2 gs_lo[2], gs_hi[2];
+                    load_group(vf[0], 0);
+                    scales16_of(0, gs_lo[0], gs_hi[0]);
 #pragma unroll
-                    for (int ht = 0; ht < 2; ++ht) {
-                        Frag pf; // P'_g = f16(p * scale_g / 2^window): 2^-12 relative rounding
-                        pf.u[0] = pack_f16_hw(p_lo[ht][0] * gs0[cur][0], p_lo[ht][1] * gs0[cur][1]);
-                        pf.u[1] = pack_f16_hw(p_lo[ht][2] * gs0[cur][2], p_lo[ht][3] * gs0[cur][3]);
-                        pf.u[2] = pack_f16_hw(p_hi[ht][0] * gs1[cur][0], p_hi[ht][1] * gs1[cur][1]);
-                        pf.u[3] = pack_f16_hw(p_hi[ht][2] * gs1[cur][2], p_hi[ht][3] * gs1[cur][3]);
+                    for (int g = 0; g < 4; ++g) {
+                        const int cur = g & 1;
+                        if (g + 1 < 4) {
+                            load_group(vf[cur ^ 1], g + 1);
+                            scales16_of(g + 1, gs_lo[cur ^ 1], gs_hi[cur ^ 1]);
+                            // group g's ten reads are older than the ten just issued
+                            asm volatile("s_waitcnt lgkmcnt(10)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                         "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
+                                         "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
+                                         :
+                                         : "memory");
+                        } else {
+                            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                         "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
+                                         "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
+                                         :
+                                         : "memory");
+                        }
 #pragma unroll
-                        for (int tt = 0; tt < 4; ++tt) {
-                            acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[cur][tt].h, pf.h, acc[ht][g * 4 + tt], 0, 0, 0);
+                        for (int ht = 0; ht < 2; ++ht) {
+                            Frag pf;
+                            pf.u[0] = pk_mul(p16[ht][0], gs_lo[cur][0]);
+                            pf.u[1] = pk_mul(p16[ht][1], gs_lo[cur][1]);
+                            pf.u[2] = pk_mul(p16[ht][2], gs_hi[cur][0]);
+                            pf.u[3] = pk_mul(p16[ht][3], gs_hi[cur][1]);
+#pragma unroll
+                            for (int tt = 0; tt < 4; ++tt) {
+                                acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[cur][tt].h, pf.h, acc[ht][g * 4 + tt], 0, 0, 0);
+                            }
                         }
                     }
                 }
