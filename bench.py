@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_decode_f16_window", "copy_calibration", "read_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration"])
     ap.add_argument("--pool-gib", type=float, default=256.0, help="address span of the paged pool (all four planes); clipped to 90 %% of free HBM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)

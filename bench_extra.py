@@ -370,5 +370,9 @@ def run(args):
         import bench_prefill
 
         bench_prefill.run(args)
+    elif args.workload == "gqa_prefill_f16":
+        import bench_prefill
+
+        bench_prefill.run_f16(args)
     else:
         raise SystemExit(f"unknown workload {args.workload}")

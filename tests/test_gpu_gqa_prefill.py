@@ -261,31 +261,91 @@ def test_prefill_head_dim_256_visible_ends_gate_and_bf16_out():
     assert_attention_close(out.cpu().numpy(), want, "head_dim 256 gated")
 
 
-@pytest.mark.parametrize("d,prefix,chunk,window,softcap", [(256, 900, 64, 0, 50.0), (256, 1500, 40, 1024, 50.0), (128, 300, 100, 0, 0.0)])
-def test_prefill_f16_kv(d, prefix, chunk, window, softcap):
-    """Chunked prefill over an f16 cache (the config-3 model family prefills too): rows appended as f16, then attended."""
+def run_f16_case(seed, d, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, q_kind="f32", gain=1.0, visible_ends=None,
+                 gate_cols=0, out_dtype=None, scale=None):
+    """A chunk over an f16 cache: rows written by the oracle's f16 append into a pool whose other rows hold f16 NaN, queries
+    as f32 / bf16 / f16; returns (device output as f32 numpy, oracle output)."""
     from zllm_amd import capi, ops
 
-    hq, hkv, bt = 16, 8, 16
-    rng = np.random.default_rng(d + prefix)
+    out_dtype = out_dtype or torch.float32
+    rng = np.random.default_rng(seed)
     total = prefix + chunk
     cols = hkv * d
-    tables, pool_blocks = draw_tables(rng, [total], bt)
-    k = rng.standard_normal((total, cols)).astype(np.float32)
-    v = rng.standard_normal((total, cols)).astype(np.float32)
-    planes = {"k": np.zeros((pool_blocks * bt, cols), dtype=np.uint16), "v": np.zeros((pool_blocks * bt, cols), dtype=np.uint16)}
-    O.half_append_paged(1, k, planes["k"], tables[0], 0, bt)
-    O.half_append_paged(1, v, planes["v"], tables[0], 0, bt)
+    tables, pool_blocks = draw_tables(rng, [total], block_tokens)
+    k = rng.standard_normal((total, cols)).astype(np.float32) * gain
+    v = rng.standard_normal((total, cols)).astype(np.float32) * gain
+    planes = {n: np.full((pool_blocks * block_tokens, cols), 0x7e00, dtype=np.uint16) for n in ("k", "v")}
+    O.half_append_paged(1, k, planes["k"], tables[0], 0, block_tokens)
+    O.half_append_paged(1, v, planes["v"], tables[0], 0, block_tokens)
     q = rng.standard_normal((chunk, hq * d)).astype(np.float32)
-    scale = 1.0 / np.sqrt(d)
-    out = ops.gqa_prefill_chunk(upload(q), upload(planes["k"]), None, upload(planes["v"]), None, upload(tables[0]), prefix, hq, hkv, d, bt,
-                                scale, window=window, softcap=softcap, kv_format=capi.KV_F16)
+    if q_kind == "bf16":
+        q = O.bf16_to_f32(O.f32_to_bf16(q))
+        q_dev = to_torch_bf16(O.f32_to_bf16(q), "cuda")
+    elif q_kind == "f16":
+        q = q.astype(np.float16).astype(np.float32)
+        q_dev = upload(q).to(torch.float16)
+    else:
+        q_dev = upload(q)
+    scale = scale or 1.0 / np.sqrt(d)
+    gate = (rng.standard_normal((chunk, gate_cols)) * 3).astype(np.float32) if gate_cols else None
+    out = ops.gqa_prefill_chunk(q_dev, upload(planes["k"]), None, upload(planes["v"]), None, upload(tables[0]), prefix, hq, hkv, d, block_tokens,
+                                scale, window=window, softcap=softcap, kv_format=capi.KV_F16, out_dtype=out_dtype,
+                                gate=None if gate is None else upload(gate), visible_ends=None if visible_ends is None else upload(visible_ends))
     torch.cuda.synchronize()
-    kd = O.gather_dequant_rows(O.FMT_F16, planes["k"], None, 0, tables[0], bt, 0, total, cols)
-    vd = O.gather_dequant_rows(O.FMT_F16, planes["v"], None, 0, tables[0], bt, 0, total, cols)
-    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap)
+    kd = O.gather_dequant_rows(O.FMT_F16, planes["k"], None, 0, tables[0], block_tokens, 0, total, cols)
+    vd = O.gather_dequant_rows(O.FMT_F16, planes["v"], None, 0, tables[0], block_tokens, 0, total, cols)
+    rc, want = O.gqa_prefill_at_visible(q, kd, vd, 0, total, prefix, hq, hkv, d, window=window, score_scale=scale, softcap=softcap,
+                                        visible_ends=visible_ends)
     assert rc == 0
-    print("prefill f16", d, assert_attention_close(out.cpu().numpy(), want, f"f16 KV prefill d={d}"))
+    if gate is not None:
+        rc, want = O.sigmoid_gate(want.reshape(chunk, -1), gate)
+        assert rc == 0
+    return out.float().cpu().numpy(), want
+
+
+@pytest.mark.parametrize("d,prefix,chunk,window,softcap", [(256, 900, 64, 0, 50.0), (256, 1500, 40, 1024, 50.0), (128, 300, 100, 0, 0.0)])
+def test_prefill_f16_kv(d, prefix, chunk, window, softcap):
+    """Chunked prefill over an f16 cache (the config-3 model family prefills too): head_dim 128 and 256 run a matrix-core
+    kernel of their own; the soft cap is the family's 50."""
+    out, want = run_f16_case(d + prefix, d, prefix, chunk, 16, 8, window=window, softcap=softcap)
+    print("prefill f16", d, assert_attention_close(out, want, f"f16 KV prefill d={d}"))
+
+
+@pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,softcap,block_tokens,q_kind",
+                         [(128, 0, 1, 4, 4, 0, 0.0, 16, "f32"), (256, 0, 300, 16, 8, 0, 50.0, 16, "bf16"), (128, 2000, 130, 48, 3, 0, 0.0, 64, "bf16"),
+                          (256, 1100, 70, 3, 1, 1, 0.0, 1, "f16"), (128, 777, 33, 64, 4, 100, 30.0, 48, "f32"), (256, 640, 129, 128, 1, 0, 0.0, 4, "bf16"),
+                          (128, 31, 2, 2, 2, 40, 0.0, 16, "f16"), (256, 2047, 65, 32, 8, 1024, 50.0, 16, "bf16")])
+def test_prefill_f16_kv_shapes(d, prefix, chunk, hq, hkv, window, softcap, block_tokens, q_kind):
+    """The f16 chunk kernel over group sizes 1 to 128 (one workgroup holds 256 (row, head) pairs at head_dim 128 and 128 at
+    256), pages of 1 to 64 tokens, windows down to one token, chunks that start the sequence, every query type."""
+    out, want = run_f16_case(1000 + prefix + chunk, d, prefix, chunk, hq, hkv, window=window, softcap=softcap, block_tokens=block_tokens, q_kind=q_kind)
+    print("prefill f16 shapes", assert_attention_close(out, want, f"f16 KV prefill d={d} {hq}/{hkv} prefix={prefix} chunk={chunk}"))
+
+
+@pytest.mark.parametrize("d,out_dtype", [(128, torch.bfloat16), (256, torch.float16), (256, torch.float32)])
+def test_prefill_f16_kv_visible_ends_gate_and_output_types(d, out_dtype):
+    prefix, chunk, hq, hkv, block = 500, 90, 16, 4, 24
+    ends = np.array([min(prefix + chunk, prefix + ((r // block) + 1) * block) if r % 5 else 0 for r in range(chunk)], dtype=np.uint32)
+    out, want = run_f16_case(2000 + d, d, prefix, chunk, hq, hkv, visible_ends=ends, gate_cols=hq * d, out_dtype=out_dtype, gain=2.0)
+    step = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[out_dtype]
+    top = max(1.0, float(np.abs(want).max()))
+    assert np.abs(out.astype(np.float64) - want).max() / top <= 2e-3 + step
+
+
+def test_prefill_f16_kv_magnitudes():
+    """Keys and values at 2^6 and 2^-6 of unit scale with the score scale compensating: the query tile's power of two and the
+    2^8 carried by the probabilities keep f16 in range either way."""
+    for gain in (64.0, 1.0 / 64.0):
+        out, want = run_f16_case(3000, 256, 700, 50, 16, 8, gain=gain, scale=1.0 / (np.sqrt(256.0) * gain))
+        top = max(1e-30, float(np.abs(want).max()))
+        assert np.abs(out.astype(np.float64) - want).max() / top <= 2e-3, gain
+
+
+def test_prefill_f16_kv_wide_groups_take_the_decode_route():
+    """More query heads per KV head than a workgroup of the f16 chunk kernel has columns (128 at head_dim 256): the rows run
+    through the decode kernels instead, same results."""
+    out, want = run_f16_case(4000, 256, 300, 5, 160, 1)
+    print("prefill f16 wide group", assert_attention_close(out, want, "f16 KV prefill, 160 heads per KV head"))
 
 
 def test_prefill_f32_scale_cache():

@@ -882,13 +882,18 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     return 0;
 }
 
-// head_dim 128 over Q8g64 with 16-bit scales runs the matrix-core chunk kernel, which keeps all of its state on chip.
-// Every other geometry (head_dim 64 / 256, f16 KV, f32 scales) runs each row of the chunk as one item of the split-KV decode kernels: row r is a
-// sequence of position + r + 1 tokens over the same block table.  That route re-reads the KV bytes per row, so it is
-// bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and the split records.
+// head_dim 128 over Q8g64 with 16-bit scales, and head_dim 128 / 256 over f16 rows, run the matrix-core chunk kernels, which
+// keep all of their state on chip.  Every other geometry (head_dim 64 / 256 over Q8g64, f32 scales, more query heads per
+// KV head than a workgroup of the f16 kernel has columns) runs each row of the chunk as one item of the split-KV decode
+// kernels: row r is a sequence of position + r + 1 tokens over the same block table.  That route re-reads the KV bytes
+// per row, so it is bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and the split
+// records.
 static bool prefill_rows_as_decode_items(const zllm_gqa_prefill_args* a)
 {
-    return a->head_dim != 128 || a->kv_format != ZLLM_KV_Q8G64 || a->scale_dtype == ZLLM_SCALE_F32;
+    if (a->kv_format == ZLLM_KV_F16) {
+        return a->num_heads / a->num_kv_heads > (a->head_dim == 128 ? 256u : 128u);
+    }
+    return a->head_dim != 128 || a->scale_dtype == ZLLM_SCALE_F32;
 }
 
 static void prefill_decode_args(const zllm_gqa_prefill_args* a, zllm_gqa_decode_args* d)

@@ -553,10 +553,430 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// f16 caches (no scales): the same workgroup shape over tiles that are copied, not converted
+// ---------------------------------------------------------------------------------------------
+// K and V rows are f16 as stored (src/kv_cache/mod.rs:179-331), so a tile is the rows themselves and both
+// products are exact f16 MFMAs with f32 accumulation:
+//   S^T[token, col]  = K[token, :] . Q'[col, :]          Q' = the wave's query tile times one power of two, as f16
+//   O^T[dim, col]   += V^T[dim, token] . P[token, col]    P = p * 2^8 as f16 hi (+ lo while the step is heavy)
+// head_dim 128 keeps two 16-column tiles per wave (256 columns per workgroup); head_dim 256 keeps one (128 columns):
+// its accumulators and query fragments fill the registers that the second tile has at 128.
+template <int D> struct F16Prefill {
+    static constexpr int kRow = D * 2;            // bytes of one token of one KV head
+    static constexpr int kTile = kStep * kRow;    // one 32-token tile
+    static constexpr int kChunks = D / 8;         // 16-byte chunks per row
+    static constexpr int kCT = D == 128 ? 2 : 1;  // 16-column MFMA tiles per wave
+    static constexpr int kCols = 8 * 16 * kCT;    // (row, head-in-group) pairs per workgroup
+    static constexpr int kKS = D / 32;            // k-steps of the score product
+    static constexpr int kDT = D / 16;            // 16-dim tiles of the output
+    static constexpr int kLoads = kChunks / 8;    // 16-byte loads per staging thread and step
+};
+
+template <int D, bool SOFTCAP, bool POW2>
+__global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
+{
+    using C = F16Prefill<D>;
+    constexpr int CT = C::kCT;
+    __shared__ __align__(16) unsigned char lds_k[2][C::kTile];
+    __shared__ __align__(16) unsigned char lds_v[2][C::kTile];
+
+    const unsigned int tid = threadIdx.x;
+    const unsigned int lane = tid & 63u;
+    const unsigned int wave = tid >> 6;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    const unsigned int kvh = blockIdx.y;
+    const unsigned int rows_per_wg = max(1u, (unsigned int)C::kCols / p.group);
+    const unsigned int row0 = blockIdx.x * rows_per_wg;
+    const unsigned int cols_used = rows_per_wg * p.group;
+
+    // visible token range of the workgroup, as in gqa_prefill_q8
+    const unsigned int last_row = min(row0 + rows_per_wg, p.rows) - 1u;
+    unsigned int t_end = p.position + last_row + 1u;
+    if (p.visible_ends != nullptr) {
+        for (unsigned int r = row0; r <= last_row; ++r) {
+            t_end = max(t_end, min(p.visible_ends[r], p.position + p.rows));
+        }
+    }
+    unsigned int t_begin = 0;
+    if (p.window != 0) {
+        const unsigned int first_pos = p.position + row0 + 1u;
+        t_begin = first_pos > p.window ? first_pos - p.window : 0u;
+    }
+    t_begin &= ~31u;
+    const unsigned int steps = (t_end - t_begin + kStep - 1) / kStep;
+
+    // ---- this wave's columns and Q fragments (power-of-two normalised f16, as in gqa_prefill_q8) ----
+    unsigned int col_row[CT], col_head[CT];
+    bool col_valid[CT];
+    Frag qf[CT][C::kKS];
+    float q_fac;
+    {
+        float q_amax = 0.0f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const unsigned int col = wave * (16u * CT) + ct * 16u + m;
+            const unsigned int r = row0 + col / p.group;
+            col_row[ct] = r;
+            col_head[ct] = kvh * p.group + col % p.group;
+            col_valid[ct] = col < cols_used && r < p.rows;
+        }
+        // two passes over the query (maximum, then conversion): keeping all of it in f32 would not fit the registers
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+            for (int ks = 0; ks < C::kKS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x = col_valid[ct] ? load_as_f32(p.q, ((size_t)col_row[ct] * p.num_heads + col_head[ct]) * D + ks * 32 + j * 8 + e, p.q_dtype) : 0.0f;
+                    q_amax = fmaxf(q_amax, fabsf(x));
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            q_amax = fmaxf(q_amax, __shfl_xor(q_amax, off));
+        }
+        const unsigned int q_exp = min(max((__float_as_uint(q_amax) >> 23) & 0xffu, 16u), 240u);
+        const float q_mul = __uint_as_float((262u - q_exp) << 23); // 2^(127 + 8 - q_exp)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+            for (int ks = 0; ks < C::kKS; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const size_t at = ((size_t)col_row[ct] * p.num_heads + col_head[ct]) * D + ks * 32 + j * 8 + 2 * e;
+                    const float x0 = col_valid[ct] ? load_as_f32(p.q, at, p.q_dtype) : 0.0f;
+                    const float x1 = col_valid[ct] ? load_as_f32(p.q, at + 1, p.q_dtype) : 0.0f;
+                    qf[ct][ks].u[e] = pack_f16_hw(x0 * q_mul, x1 * q_mul);
+                }
+            }
+        }
+        q_fac = ldexpf(1.0f, (int)q_exp - 135);
+    }
+
+    // score -> exponent of two: natural units first when the soft cap is on
+    const float score_mult = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_fac;
+    const float cap_log2 = p.softcap * kLog2e;
+    const float tanh_arg = SOFTCAP ? score_mult * (2.0f * kLog2e) / p.softcap : 0.0f; // raw product -> 2 y log2(e), y = score / cap
+    const unsigned int k_row = p.num_kv_heads * C::kRow; // bytes of one cache row
+    const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
+    const unsigned int last_token = t_end - 1u;
+    auto entry_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned int {
+        token = min(token, last_token);
+        const unsigned int page = pow2 ? token >> p.block_shift : token / p.block_tokens;
+        return (POW2 || p.table != nullptr) ? p.table[page] : page;
+    };
+    auto row_from = [&](unsigned int token, unsigned int entry) __attribute__((always_inline)) -> unsigned long long {
+        token = min(token, last_token);
+        if (pow2) {
+            return ((unsigned long long)entry << p.block_shift) + (token & (p.block_tokens - 1u));
+        }
+        return (unsigned long long)entry * p.block_tokens + token % p.block_tokens;
+    };
+    // staging: threads 0..255 copy K, 256..511 copy V; a thread owns token (tid % 256) / 8 and the chunks cc, cc + 8, ...
+    const bool stage_v = tid >= 256u;
+    const unsigned int st_token = (tid & 255u) >> 3;
+    const unsigned int cc = tid & 7u;
+    const unsigned char* st_plane = (stage_v ? p.v_plane : p.k_plane) + (size_t)kvh * C::kRow + cc * 16u;
+    struct StageRegs {
+        u32x4 chunk[C::kLoads];
+    };
+    auto load_step = [&](StageRegs& r, unsigned int t0, unsigned int entry) __attribute__((always_inline)) {
+        const unsigned char* at = st_plane + row_from(t0 + st_token, entry) * k_row;
+#pragma unroll
+        for (int u = 0; u < C::kLoads; ++u) {
+            r.chunk[u] = *(const u32x4*)(at + u * 128);
+        }
+    };
+    // chunk c of row r sits at r * kRow + ((c ^ swz(r)) << 4): the swizzle touches chunk bits 1..3 only, so it serves
+    // rows of 16 and of 32 chunks alike (a row is one or two whole lines of the 64 banks)
+    auto store_step = [&](const StageRegs& r, int buf) __attribute__((always_inline)) {
+        unsigned char* tile = stage_v ? lds_v[buf] : lds_k[buf];
+#pragma unroll
+        for (int u = 0; u < C::kLoads; ++u) {
+            *(u32x4*)(tile + st_token * C::kRow + (((cc + 8u * u) ^ swz(st_token)) << 4)) = r.chunk[u];
+        }
+    };
+
+    f32x4 acc[CT][C::kDT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+        for (int t = 0; t < C::kDT; ++t) {
+            acc[ct][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    float run_max[CT], run_sum[CT], ref_shift[CT];
+    unsigned int vis_lo[CT], vis_hi[CT];
+    unsigned int wave_min_hi = 0xffffffffu, wave_max_lo = 0u;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        run_max[ct] = kNegInf;
+        run_sum[ct] = 0.0f;
+        ref_shift[ct] = kPBias;
+        const unsigned int pos = p.position + col_row[ct];
+        unsigned int hi = pos + 1u;
+        if (p.visible_ends != nullptr && col_valid[ct]) {
+            hi = min(max(hi, p.visible_ends[col_row[ct]]), p.position + p.rows);
+        }
+        vis_hi[ct] = col_valid[ct] ? hi : 0u;
+        vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+        wave_min_hi = min(wave_min_hi, vis_hi[ct]);
+        wave_max_lo = max(wave_max_lo, vis_lo[ct]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wave_min_hi = min(wave_min_hi, (unsigned int)__shfl_xor((int)wave_min_hi, off));
+        wave_max_lo = max(wave_max_lo, (unsigned int)__shfl_xor((int)wave_max_lo, off));
+    }
+    wave_min_hi = __builtin_amdgcn_readfirstlane(wave_min_hi);
+    wave_max_lo = __builtin_amdgcn_readfirstlane(wave_max_lo);
+
+    // LDS byte offsets of the lane's fragments as finished sums.  K: chunk 4 ks + j of row m; the swizzle permutes
+    // ks inside a group of four, so four registers serve every k-step (ks / 4 selects 256 bytes further, an immediate).
+    // V: chunk 2 tt + (m & 3) / 2 of row tr_row, 8 bytes in; the swizzle permutes tt inside a group of eight.
+    unsigned int qk_at[4], pv_at[8];
+    const unsigned int tr_row = 4u * j + (m >> 2);
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4) {
+        qk_at[k4] = m * C::kRow + ((((unsigned int)k4 << 2 | j) ^ swz(m)) << 4);
+        asm volatile("" : "+v"(qk_at[k4]));
+    }
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+        pv_at[t8] = tr_row * C::kRow + ((((unsigned int)t8 << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+        asm volatile("" : "+v"(pv_at[t8]));
+    }
+
+    auto compute_step = [&](int buf, unsigned int t0) __attribute__((always_inline)) {
+        const unsigned char* kt = lds_k[buf];
+        const unsigned char* vt = lds_v[buf];
+        // ---- S^T = K . Q' ---------------------------------------------------------------------------
+        f32x4 s[2][CT];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                s[i][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int ks = 0; ks < C::kKS; ++ks) {
+                Frag kf;
+                kf.u = *(const u32x4*)(kt + qk_at[ks & 3] + (ks >> 2) * 256 + i * 16 * C::kRow);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    s[i][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf.h, qf[ct][ks].h, s[i][ct], 0, 0, 0);
+                }
+            }
+        }
+        union VFrag {
+            s16x4 s[2];
+            f16x8 h;
+        };
+        auto load_vfrag = [&](VFrag& vf, int tt) __attribute__((always_inline)) {
+            const unsigned char* at = vt + pv_at[tt & 7] + (tt >> 3) * 256;
+            vf.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+            vf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * C::kRow));
+        };
+        // the first V^T fragments travel under the softmax
+        VFrag vf[2][4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            load_vfrag(vf[0][tt], tt);
+        }
+        PREFILL_PHASE_FENCE();
+        // ---- online softmax per column ----------------------------------------------------------------
+        float pr[CT][8];
+        bool heavy = false;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float sc[8];
+            const bool edge = t0 + kStep > wave_min_hi || t0 < wave_max_lo;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float x = s[e >> 2][ct][e & 3];
+                if constexpr (SOFTCAP) {
+                    // tanh(y) = 1 - 2 / (e^(2y) + 1): its error is a few units of 2^-24 of 1, i.e. of the cap in the score, which
+                    // is all a softmax asks of it (the form cancels for tiny y, but only relative to y); the cap rides in `mult`
+                    const float e2y = __builtin_amdgcn_exp2f(x * tanh_arg);
+                    x = fmaf(-2.0f, __builtin_amdgcn_rcpf(e2y + 1.0f), 1.0f);
+                }
+                sc[e] = x;
+            }
+            if (edge) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const unsigned int token = t0 + 16u * (e >> 2) + 4u * j + (e & 3);
+                    sc[e] = (token >= vis_lo[ct] && token < vis_hi[ct]) ? sc[e] : kNegInf;
+                }
+            }
+            const float mult = SOFTCAP ? cap_log2 : score_mult; // positive: maxima first, the factor rides in the multiply-add
+            float lane_max = sc[0];
+#pragma unroll
+            for (int e = 1; e < 8; ++e) {
+                lane_max = fmaxf(lane_max, sc[e]);
+            }
+            if (__any(lane_max * mult > run_max[ct])) {
+                const float step_max = wave_max_16x4(lane_max) * mult;
+                const float new_max = fmaxf(run_max[ct], step_max);
+                const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+                const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max);
+                ref_shift[ct] = kPBias - safe_max;
+                run_sum[ct] *= alpha;
+                run_max[ct] = new_max;
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int t = 0; t < C::kDT; ++t) {
+                        acc[ct][t] *= alpha;
+                    }
+                }
+            }
+            const float shift = ref_shift[ct];
+            float step_sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                pr[ct][e] = __builtin_amdgcn_exp2f(fmaf(sc[e], mult, shift));
+                step_sum += pr[ct][e];
+            }
+            run_sum[ct] += step_sum;
+            heavy = heavy || step_sum * kLoThreshold > run_sum[ct];
+        }
+        // ---- O^T += V^T . P: f16 hi, and lo while a lane's probabilities of this step weigh more than 1/8 of its sum ----
+        const bool lo_pass = __any(heavy);
+        Frag phi[CT], plo[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                phi[ct].u[e] = pack_f16_hw(pr[ct][2 * e], pr[ct][2 * e + 1]);
+                const f16x2 hi = __builtin_bit_cast(f16x2, pack_f16_hw(pr[ct][2 * e], pr[ct][2 * e + 1]));
+                plo[ct].u[e] = pack_f16_hw(pr[ct][2 * e] - (float)hi[0], pr[ct][2 * e + 1] - (float)hi[1]);
+            }
+        }
+        PREFILL_PHASE_FENCE();
+#pragma unroll
+        for (int q = 0; q < C::kDT / 4; ++q) {
+            if (q + 1 < C::kDT / 4) { // the next four fragments travel while these multiply
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) {
+                    load_vfrag(vf[(q + 1) & 1][tt], (q + 1) * 4 + tt);
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    acc[ct][q * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[q & 1][tt].h, phi[ct].h, acc[ct][q * 4 + tt], 0, 0, 0);
+                }
+            }
+            if (lo_pass) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        acc[ct][q * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[q & 1][tt].h, plo[ct].h, acc[ct][q * 4 + tt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
+    // ---- main loop: the rows of step n + 1 are loaded while step n computes, and stored before the barrier
+    // (requesting them a step earlier still was measured: no change, the loads are not what a step waits for) ----
+    StageRegs regs;
+    load_step(regs, t_begin, entry_of(t_begin + st_token));
+    unsigned int entry_next = entry_of(t_begin + kStep + st_token);
+    store_step(regs, 0);
+    __syncthreads();
+    auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
+        const unsigned int t0 = t_begin + step * kStep;
+        load_step(regs, t0 + kStep, entry_next); // past the end of the range the last row repeats: loads stay inside the pages
+        entry_next = entry_of(t0 + 2u * kStep + st_token);
+        compute_step(buf, t0);
+        store_step(regs, buf ^ 1);
+        __syncthreads();
+    };
+    unsigned int step = 0;
+    for (; step + 1 < steps; step += 2) {
+        one_step(step, 0);
+        one_step(step + 1u, 1);
+    }
+    if (step < steps) {
+        one_step(step, 0);
+    }
+
+    // ---- normalise and store ------------------------------------------------------------------------
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const float total = wave_sum_16x4(run_sum[ct]);
+        const unsigned int col = wave * (16u * CT) + ct * 16u + m;
+        const unsigned int r = row0 + col / p.group;
+        const unsigned int head = kvh * p.group + col % p.group;
+        if (!(col < cols_used && r < p.rows)) {
+            continue;
+        }
+        const float inv = (total > 0.0f && total < __builtin_inff()) ? 1.0f / total : 0.0f; // the 2^8 of P cancels here
+        const size_t base = ((size_t)r * p.num_heads + head) * D;
+#pragma unroll
+        for (int t = 0; t < C::kDT; ++t) {
+            f32x4 v = acc[ct][t] * inv;
+            if (inv == 0.0f) {
+                v = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            const size_t at = base + t * 16 + 4 * j;
+            if (p.gate != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = gated(v[e], p.gate, p.gate_cols, p.gate_dtype, r, head * D + t * 16 + 4 * j + e);
+                }
+            }
+            if (p.out_dtype == 0) {
+                *(f32x4*)((float*)p.out + at) = v;
+            } else {
+                unsigned short* o = (unsigned short*)p.out + at;
+                u32x2 packed;
+                if (p.out_dtype == 1) {
+                    packed = u32x2{pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3])};
+                } else {
+                    packed = u32x2{(unsigned int)f32_to_f16_bits(v[0]) | ((unsigned int)f32_to_f16_bits(v[1]) << 16),
+                                   (unsigned int)f32_to_f16_bits(v[2]) | ((unsigned int)f32_to_f16_bits(v[3]) << 16)};
+                }
+                *(u32x2*)o = packed;
+            }
+        }
+    }
+}
+
+template <int D> static hipError_t launch_prefill_f16(const GqaPrefillParams& p, hipStream_t stream)
+{
+    const unsigned int cols = F16Prefill<D>::kCols;
+    const unsigned int rows_per_wg = p.group >= cols ? 1u : cols / p.group;
+    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
+    const bool cap = p.softcap > 0.0f;
+    const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
+    if (cap) {
+        pow2 ? gqa_prefill_f16<D, true, true><<<grid, dim3(512), 0, stream>>>(p) : gqa_prefill_f16<D, true, false><<<grid, dim3(512), 0, stream>>>(p);
+    } else {
+        pow2 ? gqa_prefill_f16<D, false, true><<<grid, dim3(512), 0, stream>>>(p) : gqa_prefill_f16<D, false, false><<<grid, dim3(512), 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
 } // namespace
 
 hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream)
 {
+    if (kv_format == 1) { // f16 rows
+        if (p.head_dim == 128u) {
+            return launch_prefill_f16<128>(p, stream);
+        }
+        if (p.head_dim == 256u) {
+            return launch_prefill_f16<256>(p, stream);
+        }
+        return hipErrorInvalidValue;
+    }
     if (kv_format != 0 || p.head_dim != (unsigned int)kD) {
         return hipErrorInvalidValue;
     }
