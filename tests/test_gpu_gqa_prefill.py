@@ -341,6 +341,16 @@ def test_prefill_f16_kv_magnitudes():
         assert np.abs(out.astype(np.float64) - want).max() / top <= 2e-3, gain
 
 
+def test_prefill_f16_kv_soft_cap_limit():
+    """An ever larger cap recovers the uncapped result (the caps models use take a cheaper tanh whose error grows with the
+    cap; large caps must not)."""
+    plain, want = run_f16_case(5000, 256, 400, 30, 16, 8)
+    capped, _ = run_f16_case(5000, 256, 400, 30, 16, 8, softcap=1e9)
+    assert_attention_close(capped, want, "f16 KV prefill, cap -> inf")
+    tight, want_tight = run_f16_case(5000, 256, 400, 30, 16, 8, softcap=2.0, scale=1.0)
+    assert_attention_close(tight, want_tight, "f16 KV prefill, cap 2 on large logits")
+
+
 def test_prefill_f16_kv_wide_groups_take_the_decode_route():
     """More query heads per KV head than a workgroup of the f16 chunk kernel has columns (128 at head_dim 256): the rows run
     through the decode kernels instead, same results."""

@@ -60,6 +60,15 @@ __device__ __forceinline__ float fast_tanh(float x)
     return fabsf(x) < 0.1f ? poly : big;
 }
 
+// tanh(y) from t = 2 y log2(e): 1 - 2 / (2^t + 1), five instructions against fifteen.  The form cancels for tiny y: its
+// absolute error is a few units of 2^-24, which the cap multiplies -- 3e-6 of a score under a cap of 50, nothing a softmax
+// sees, but not the limit of an ever larger cap.  Caps up to kSmallCap use it; larger ones take fast_tanh.
+constexpr float kSmallCap = 256.0f;
+__device__ __forceinline__ float tanh_of_exponent(float t)
+{
+    return fmaf(-2.0f, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(t) + 1.0f), 1.0f);
+}
+
 template <int G> struct ScaleRow; // G 16-bit scales of one token / KV head
 template <> struct ScaleRow<1> {
     unsigned short v;
@@ -319,7 +328,7 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Ro
         for (int r = 0; r < 4; ++r) {
             float x = tile_s[r] * scale_log2;
             if constexpr (SOFTCAP) {
-                x = cap_log2 * fast_tanh(x * inv_cap);
+                x = cap_log2 < kSmallCap * kLog2e ? cap_log2 * tanh_of_exponent(x * (inv_cap * 2.0f * kLog2e)) : cap_log2 * fast_tanh(x * inv_cap);
             }
             sc[i * 4 + r] = x;
         }
@@ -1089,6 +1098,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     float run_max = kNegInf;
     float run_sum = 0.0f;
     const float scale_eff = (p.softcap > 0.0f ? p.score_scale : p.score_scale * kLog2e) / q_norm;
+    const float cap_log2 = p.softcap * kLog2e;
+    const float tanh_arg = p.softcap > 0.0f ? scale_eff * (2.0f * kLog2e) / p.softcap : 0.0f; // raw product -> 2 y log2(e), y = score / cap
 
     auto compute_step = [&](F16Step<D>& s, unsigned int t0) __attribute__((always_inline)) {
         if (FAST && (t0 < first || t0 + 32u > len)) {
@@ -1120,7 +1131,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
             for (int r = 0; r < 4; ++r) {
                 float x = d[r] * scale_eff;
                 if (p.softcap > 0.0f) {
-                    x = p.softcap * fast_tanh(x / p.softcap) * kLog2e;
+                    x = p.softcap < kSmallCap ? cap_log2 * tanh_of_exponent(d[r] * tanh_arg) : cap_log2 * fast_tanh(x / p.softcap);
                 }
                 const unsigned int token = t0 + 16u * i + 4u * j + r;
                 sc[i * 4 + r] = (token >= first && token < len) ? x : kNegInf;

@@ -660,6 +660,8 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
     const float score_mult = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_fac;
     const float cap_log2 = p.softcap * kLog2e;
     const float tanh_arg = SOFTCAP ? score_mult * (2.0f * kLog2e) / p.softcap : 0.0f; // raw product -> 2 y log2(e), y = score / cap
+    const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
+    const bool small_cap = p.softcap < 256.0f;
     const unsigned int k_row = p.num_kv_heads * C::kRow; // bytes of one cache row
     const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const unsigned int last_token = t_end - 1u;
@@ -798,10 +800,15 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
             for (int e = 0; e < 8; ++e) {
                 float x = s[e >> 2][ct][e & 3];
                 if constexpr (SOFTCAP) {
-                    // tanh(y) = 1 - 2 / (e^(2y) + 1): its error is a few units of 2^-24 of 1, i.e. of the cap in the score, which
-                    // is all a softmax asks of it (the form cancels for tiny y, but only relative to y); the cap rides in `mult`
-                    const float e2y = __builtin_amdgcn_exp2f(x * tanh_arg);
-                    x = fmaf(-2.0f, __builtin_amdgcn_rcpf(e2y + 1.0f), 1.0f);
+                    // tanh(y) = 1 - 2 / (e^(2y) + 1) for the caps models use: the form cancels for tiny y, and its absolute error,
+                    // a few units of 2^-24, is multiplied by the cap (3e-6 of a score under a cap of 50); larger caps take the
+                    // polynomial-or-exponential form, which keeps the limit of an ever larger cap.  The cap rides in `mult`.
+                    if (small_cap) {
+                        const float e2y = __builtin_amdgcn_exp2f(x * tanh_arg);
+                        x = fmaf(-2.0f, __builtin_amdgcn_rcpf(e2y + 1.0f), 1.0f);
+                    } else {
+                        x = soft_tanh(x * score_mult * inv_cap);
+                    }
                 }
                 sc[e] = x;
             }
