@@ -175,6 +175,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
     const float cap_log2 = p.softcap * kLog2e;
+    const bool small_cap = p.softcap < 256.0f;
+    const float tanh_arg = SOFTCAP ? q_fac * inv_cap * (2.0f * kLog2e) : 0.0f; // scaled score -> 2 y log2(e), y = score / cap
     const unsigned int k_row = p.num_kv_heads * kD;
     const unsigned int s_row = p.num_kv_heads * 4u; // two 16-bit scales per KV head
     const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
@@ -369,7 +371,9 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             for (int e = 0; e < 8; ++e) {
                 float x = s[e >> 2][ct][e & 3];
                 if constexpr (SOFTCAP) {
-                    x = cap_log2 * soft_tanh(x * q_fac * inv_cap);
+                    // caps that models use take the five-instruction form (see gqa_prefill_f16), larger ones the precise one
+                    x = small_cap ? cap_log2 * fmaf(-2.0f, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * tanh_arg) + 1.0f), 1.0f)
+                                  : cap_log2 * soft_tanh(x * q_fac * inv_cap);
                 }
                 sc[e] = x;
             }
