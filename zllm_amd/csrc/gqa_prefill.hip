@@ -1,4 +1,5 @@
-// Chunked-prefill GQA attention over a paged Q8g64 KV cache — gfx950, f16 MFMA.
+// Chunked-prefill GQA attention over a paged KV cache — gfx950, f16 MFMA: gqa_prefill_q8 for Q8g64 caches (head_dim 128,
+// described first), gqa_prefill_f16 for f16 caches (head_dim 128 and 256, further down).
 //
 // T query rows appended at `position` attend the cached prefix plus the chunk itself (causal,
 // optional sliding window).  Replaces the per-(row, head) block attention the reference runs for this
