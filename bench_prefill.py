@@ -150,7 +150,7 @@ def run_f16(args):
         "pct_of_mfma_peak": round(100.0 * g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 2),
         "prefill_tokens_per_s": round(chunk / (g["ms_per_step"] * 1e-3), 1),
         "window_layer": {"ms_per_step": round(results["sliding"]["ms_per_step"], 4), "tflops": round(results["sliding"]["tflops"], 1)},
-        "roofline": {"bound": "mfma", "kernel": "gqa_prefill_f16", "achieved": round(g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "gqa_prefill_tiles", "achieved": round(g["tflops"], 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(g["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel_ms": round(g["ms_per_step"], 4)},
     }
     if not args.no_cpu_baseline:

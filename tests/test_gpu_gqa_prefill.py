@@ -358,6 +358,15 @@ def test_prefill_f16_kv_wide_groups_take_the_decode_route():
     print("prefill f16 wide group", assert_attention_close(out, want, "f16 KV prefill, 160 heads per KV head"))
 
 
+@pytest.mark.parametrize("d,q_bf16", [(256, False), (256, True), (64, False), (64, True)])
+def test_prefill_q8_tiles_and_the_decode_route_agree(d, q_bf16):
+    """head_dim 64 and 256 over Q8g64 run the matrix-core tile kernel, which carries queries as f16 (exact for bf16
+    activations); f32 queries take the decode kernels' route instead, whose query is wider.  Outlier channels
+    and large logits are what separate the two."""
+    out, want = run_case(800 + d, 1200, 96, 16, 4, d=d, q_bf16=q_bf16, outliers=True, scale=0.25 if d == 64 else 0.125)
+    print("prefill q8 tiles", d, q_bf16, assert_attention_close(out.cpu().numpy(), want, f"Q8 prefill d={d} bf16={q_bf16}"))
+
+
 def test_prefill_f32_scale_cache():
     """A chunk over a cache with f32 scales (CUDA convention): appended by the library, attended through the decode kernels."""
     out, want = run_case(321, 400, 60, 16, 4, rule=O.RULE_CUDA_GQA)

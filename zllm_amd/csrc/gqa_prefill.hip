@@ -559,32 +559,46 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 }
 
 // ---------------------------------------------------------------------------------------------
-// f16 caches (no scales): the same workgroup shape over tiles that are copied, not converted
+// The other tile shapes: f16 caches at head_dim 128 / 256, Q8g64 caches at head_dim 64 / 256
 // ---------------------------------------------------------------------------------------------
-// K and V rows are f16 as stored (src/kv_cache/mod.rs:179-331), so a tile is the rows themselves and both
-// products are exact f16 MFMAs with f32 accumulation:
-//   S^T[token, col]  = K[token, :] . Q'[col, :]          Q' = the wave's query tile times one power of two, as f16
-//   O^T[dim, col]   += V^T[dim, token] . P[token, col]    P = p * 2^8 as f16 hi (+ lo while the step is heavy)
-// head_dim 128 keeps two 16-column tiles per wave (256 columns per workgroup); head_dim 256 keeps one (128 columns):
-// its accumulators and query fragments fill the registers that the second tile has at 128.
-template <int D> struct F16Prefill {
-    static constexpr int kRow = D * 2;            // bytes of one token of one KV head
+// The same workgroup as gqa_prefill_q8 over a tile layout that does not depend on the row length: chunk c of row r
+// sits at r * row_bytes + ((c ^ swz(r)) << 4) with the swizzle cut to the row's chunk bits: it touches chunk bits 1..3,
+// so rows of 16 and 32 chunks (one or two whole lines of the 64 banks) take all of it and rows of 8 chunks (half a
+// line: the row's parity already picks the half) take bits 1 and 2.
+//   f16 rows (src/kv_cache/mod.rs:179-331) are copied as stored: S^T = K . Q' is one accumulator, P = p * 2^8 as
+//       f16 hi (+ lo while the step is heavy), no scales and no window.
+//   Q8g64 rows are converted as in gqa_prefill_q8 (exact f16 integers, K scales pre-multiplied by the score scale,
+//       one accumulator per 64-column group, P'_g = p * v_scale_g, the exponent of the largest V scale carried by
+//       the softmax reference).
+// head_dim 64 and 128 keep two 16-column tiles per wave (256 columns per workgroup); head_dim 256 keeps one (128
+// columns): its accumulators and query fragments fill the registers that the second tile has at 128.
+template <int D> struct TileShape {
+    static constexpr int kRow = D * 2;            // bytes of one token of one KV head as f16
     static constexpr int kTile = kStep * kRow;    // one 32-token tile
     static constexpr int kChunks = D / 8;         // 16-byte chunks per row
-    static constexpr int kCT = D == 128 ? 2 : 1;  // 16-column MFMA tiles per wave
+    static constexpr int kCT = D == 256 ? 1 : 2;  // 16-column MFMA tiles per wave
     static constexpr int kCols = 8 * 16 * kCT;    // (row, head-in-group) pairs per workgroup
     static constexpr int kKS = D / 32;            // k-steps of the score product
     static constexpr int kDT = D / 16;            // 16-dim tiles of the output
-    static constexpr int kLoads = kChunks / 8;    // 16-byte loads per staging thread and step
+    static constexpr int kLoads = kChunks / 8;    // staging loads per thread and step (16 bytes of f16, or 8 codes)
+    static constexpr int kG = D / 64;             // Q8g64 scale groups per row
+    __device__ static __forceinline__ unsigned int swizzle(unsigned int row) { return swz(row) & (unsigned int)(kChunks - 1); }
 };
 
-template <int D, bool SOFTCAP, bool POW2>
-__global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
+// KV: 0 = Q8g64 (SDT names the 16-bit scale type), 1 = f16 rows
+template <int D, int KV, int SDT, bool SOFTCAP, bool POW2>
+__global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
 {
-    using C = F16Prefill<D>;
+    using C = TileShape<D>;
     constexpr int CT = C::kCT;
+    constexpr int G = C::kG;
+    constexpr bool Q8 = KV == 0;
+    static_assert(C::kLoads >= 1, "a staging thread owns at least one chunk");
     __shared__ __align__(16) unsigned char lds_k[2][C::kTile];
     __shared__ __align__(16) unsigned char lds_v[2][C::kTile];
+    __shared__ __align__(16) float lds_ks[Q8 ? 2 : 1][Q8 ? G : 1][kStep]; // [buffer][group][token], Q8g64 only
+    __shared__ __align__(16) float lds_vs[Q8 ? 2 : 1][Q8 ? G : 1][kStep];
+    __shared__ __align__(16) float lds_top[2][8];                         // [buffer][staging wave]: largest scale it converted
 
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -661,13 +675,16 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
         q_fac = ldexpf(1.0f, (int)q_exp - 135);
     }
 
-    // score -> exponent of two: natural units first when the soft cap is on
-    const float score_mult = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_fac;
+    // What turns the accumulated product into a score in base-2 units (or, under a soft cap, into natural units first).
+    // Q8g64 tiles carry the score scale in their K scales, f16 tiles do not.
+    const float scale_log2 = SOFTCAP ? p.score_scale : p.score_scale * kLog2e;
+    const float score_mult = Q8 ? q_fac : scale_log2 * q_fac;
     const float cap_log2 = p.softcap * kLog2e;
-    const float tanh_arg = SOFTCAP ? score_mult * (2.0f * kLog2e) / p.softcap : 0.0f; // raw product -> 2 y log2(e), y = score / cap
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
+    const float tanh_arg = SOFTCAP ? score_mult * (2.0f * kLog2e) / p.softcap : 0.0f; // product -> 2 y log2(e), y = score / cap
     const bool small_cap = p.softcap < 256.0f;
-    const unsigned int k_row = p.num_kv_heads * C::kRow; // bytes of one cache row
+    const unsigned int k_row = p.num_kv_heads * (Q8 ? (unsigned int)D : (unsigned int)C::kRow); // bytes of one cache row
+    const unsigned int s_row = p.num_kv_heads * G * 2u;                                         // bytes of one scale row
     const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const unsigned int last_token = t_end - 1u;
     auto entry_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned int {
@@ -682,29 +699,80 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
         }
         return (unsigned long long)entry * p.block_tokens + token % p.block_tokens;
     };
-    // staging: threads 0..255 copy K, 256..511 copy V; a thread owns token (tid % 256) / 8 and the chunks cc, cc + 8, ...
+    // staging: threads 0..255 take K, 256..511 take V; a thread owns token (tid % 256) / 8 and the chunks cc, cc + 8, ...
     const bool stage_v = tid >= 256u;
     const unsigned int st_token = (tid & 255u) >> 3;
     const unsigned int cc = tid & 7u;
-    const unsigned char* st_plane = (stage_v ? p.v_plane : p.k_plane) + (size_t)kvh * C::kRow + cc * 16u;
+    const unsigned char* st_plane = (stage_v ? p.v_plane : p.k_plane) + (size_t)kvh * (Q8 ? D : C::kRow) + cc * (Q8 ? 8u : 16u);
+    const unsigned char* st_scales = Q8 ? (stage_v ? p.v_scales : p.k_scales) + (size_t)kvh * G * 2u : nullptr;
     struct StageRegs {
-        u32x4 chunk[C::kLoads];
+        u32x4 chunk[C::kLoads]; // f16 rows: the chunk as stored; Q8g64: eight codes in the first two words
+        u32x2 scales;           // Q8g64: the token's G 16-bit scales
     };
     auto load_step = [&](StageRegs& r, unsigned int t0, unsigned int entry) __attribute__((always_inline)) {
-        const unsigned char* at = st_plane + row_from(t0 + st_token, entry) * k_row;
+        const unsigned long long row = row_from(t0 + st_token, entry);
+        const unsigned char* at = st_plane + row * k_row;
 #pragma unroll
         for (int u = 0; u < C::kLoads; ++u) {
-            r.chunk[u] = *(const u32x4*)(at + u * 128);
+            if constexpr (Q8) {
+                const u32x2 codes = *(const u32x2*)(at + u * 64);
+                r.chunk[u] = u32x4{codes[0], codes[1], 0u, 0u};
+            } else {
+                r.chunk[u] = *(const u32x4*)(at + u * 128);
+            }
+        }
+        if constexpr (Q8) {
+            const unsigned char* sp = st_scales + row * s_row;
+            if constexpr (G == 1) {
+                r.scales = u32x2{*(const unsigned short*)sp, 0u};
+            } else if constexpr (G == 2) {
+                r.scales = u32x2{*(const unsigned int*)sp, 0u};
+            } else { // the scale planes are only known to be 4-byte aligned
+                r.scales = u32x2{((const unsigned int*)sp)[0], ((const unsigned int*)sp)[1]};
+            }
         }
     };
-    // chunk c of row r sits at r * kRow + ((c ^ swz(r)) << 4): the swizzle touches chunk bits 1..3 only, so it serves
-    // rows of 16 and of 32 chunks alike (a row is one or two whole lines of the 64 banks)
     auto store_step = [&](const StageRegs& r, int buf) __attribute__((always_inline)) {
         unsigned char* tile = stage_v ? lds_v[buf] : lds_k[buf];
 #pragma unroll
         for (int u = 0; u < C::kLoads; ++u) {
-            *(u32x4*)(tile + st_token * C::kRow + (((cc + 8u * u) ^ swz(st_token)) << 4)) = r.chunk[u];
+            u32x4 out = r.chunk[u];
+            if constexpr (Q8) {
+                unsigned int a, b, c, d;
+                codes4_to_f16(r.chunk[u][0], a, b);
+                codes4_to_f16(r.chunk[u][1], c, d);
+                out = u32x4{a, b, c, d};
+            }
+            *(u32x4*)(tile + st_token * C::kRow + (((cc + 8u * u) ^ C::swizzle(st_token)) << 4)) = out;
         }
+        if constexpr (Q8) {
+            // the eight threads of a token all hold its scales; K scales carry the score scale (and log2 e)
+            float top = 0.0f;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float sg = scale_bits_to_f32<SDT>((unsigned short)((r.scales[g >> 1] >> (16 * (g & 1))) & 0xffffu));
+                top = fmaxf(top, sg);
+                if (cc == 0) {
+                    (stage_v ? lds_vs : lds_ks)[buf][g][st_token] = stage_v ? sg : sg * scale_log2;
+                }
+            }
+            if (stage_v) { // largest V scale of the wave's eight tokens (a row of sixteen lanes holds two)
+                top = fmaxf(top, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(top), 0x128, 0xf, 0xf, false))); // row_ror:8
+                const float rows01 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 0)),
+                                           __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 16)));
+                const float rows23 = fmaxf(__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 32)),
+                                           __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(top), 48)));
+                if (lane == 0) {
+                    lds_top[buf][wave] = fmaxf(rows01, rows23);
+                }
+            }
+        }
+    };
+    // (biased) exponent of the largest V scale of the tile in `buf`, folded into the running one (Q8g64 only)
+    auto window_of = [&](int buf, unsigned int wv) __attribute__((always_inline)) -> unsigned int {
+        const f32x4 tops = *(const f32x4*)&lds_top[buf][4];
+        const float top = fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3]));
+        return max(wv, (unsigned int)__builtin_amdgcn_readfirstlane(window_exponent(top)));
     };
 
     f32x4 acc[CT][C::kDT];
@@ -744,23 +812,27 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
     // LDS byte offsets of the lane's fragments as finished sums.  K: chunk 4 ks + j of row m; the swizzle permutes
     // ks inside a group of four, so four registers serve every k-step (ks / 4 selects 256 bytes further, an immediate).
     // V: chunk 2 tt + (m & 3) / 2 of row tr_row, 8 bytes in; the swizzle permutes tt inside a group of eight.
-    unsigned int qk_at[4], pv_at[8];
+    constexpr int kQkRegs = C::kKS < 4 ? C::kKS : 4, kPvRegs = C::kDT < 8 ? C::kDT : 8;
+    unsigned int qk_at[kQkRegs], pv_at[kPvRegs];
     const unsigned int tr_row = 4u * j + (m >> 2);
 #pragma unroll
-    for (int k4 = 0; k4 < 4; ++k4) {
-        qk_at[k4] = m * C::kRow + ((((unsigned int)k4 << 2 | j) ^ swz(m)) << 4);
+    for (int k4 = 0; k4 < kQkRegs; ++k4) {
+        qk_at[k4] = m * C::kRow + ((((unsigned int)k4 << 2 | j) ^ C::swizzle(m)) << 4);
         asm volatile("" : "+v"(qk_at[k4]));
     }
 #pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) {
-        pv_at[t8] = tr_row * C::kRow + ((((unsigned int)t8 << 1 | ((m & 3u) >> 1)) ^ swz(tr_row)) << 4) + (m & 1u) * 8u;
+    for (int t8 = 0; t8 < kPvRegs; ++t8) {
+        pv_at[t8] = tr_row * C::kRow + ((((unsigned int)t8 << 1 | ((m & 3u) >> 1)) ^ C::swizzle(tr_row)) << 4) + (m & 1u) * 8u;
         asm volatile("" : "+v"(pv_at[t8]));
     }
 
-    auto compute_step = [&](int buf, unsigned int t0) __attribute__((always_inline)) {
+    // `v_shift` = 8 - (V window exponent) goes into the softmax reference, `acc_fix` is 2^-(growth of that window since
+    // the last step): 8 and 1 for f16 rows, which have no scales
+    auto compute_step = [&](int buf, unsigned int t0, float v_shift, float acc_fix, bool window_moved) __attribute__((always_inline)) {
         const unsigned char* kt = lds_k[buf];
         const unsigned char* vt = lds_v[buf];
-        // ---- S^T = K . Q' ---------------------------------------------------------------------------
+        const int sbuf = Q8 ? buf : 0;
+        // ---- S^T = K . Q' (one accumulator per scale group for Q8g64 tiles) ------------------------------
         f32x4 s[2][CT];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -768,13 +840,33 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
             for (int ct = 0; ct < CT; ++ct) {
                 s[i][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
+            if constexpr (Q8) {
 #pragma unroll
-            for (int ks = 0; ks < C::kKS; ++ks) {
-                Frag kf;
-                kf.u = *(const u32x4*)(kt + qk_at[ks & 3] + (ks >> 2) * 256 + i * 16 * C::kRow);
+                for (int g = 0; g < G; ++g) {
+                    Frag k0, k1;
+                    k0.u = *(const u32x4*)(kt + qk_at[(2 * g) & 3] + ((2 * g) >> 2) * 256 + i * 16 * C::kRow);
+                    k1.u = *(const u32x4*)(kt + qk_at[(2 * g + 1) & 3] + ((2 * g + 1) >> 2) * 256 + i * 16 * C::kRow);
+                    const f32x4 gs = *(const f32x4*)(&lds_ks[sbuf][g][i * 16 + 4 * j]);
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    s[i][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf.h, qf[ct][ks].h, s[i][ct], 0, 0, 0);
+                    for (int ct = 0; ct < CT; ++ct) {
+                        f32x4 d = {0.f, 0.f, 0.f, 0.f};
+                        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0.h, qf[ct][2 * g].h, d, 0, 0, 0);
+                        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1.h, qf[ct][2 * g + 1].h, d, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            s[i][ct][r] = fmaf(d[r], gs[r], s[i][ct][r]);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < C::kKS; ++ks) {
+                    Frag kf;
+                    kf.u = *(const u32x4*)(kt + qk_at[ks & 3] + (ks >> 2) * 256 + i * 16 * C::kRow);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        s[i][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf.h, qf[ct][ks].h, s[i][ct], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -830,12 +922,12 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
             for (int e = 1; e < 8; ++e) {
                 lane_max = fmaxf(lane_max, sc[e]);
             }
-            if (__any(lane_max * mult > run_max[ct])) {
+            if (__any(lane_max * mult > run_max[ct]) || window_moved) {
                 const float step_max = wave_max_16x4(lane_max) * mult;
                 const float new_max = fmaxf(run_max[ct], step_max);
                 const float safe_max = new_max == kNegInf ? 0.0f : new_max;
-                const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max);
-                ref_shift[ct] = kPBias - safe_max;
+                const float alpha = __builtin_amdgcn_exp2f(run_max[ct] - safe_max) * acc_fix;
+                ref_shift[ct] = v_shift - safe_max;
                 run_sum[ct] *= alpha;
                 run_max[ct] = new_max;
                 if (__any(alpha != 1.0f)) {
@@ -855,21 +947,29 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
             run_sum[ct] += step_sum;
             heavy = heavy || step_sum * kLoThreshold > run_sum[ct];
         }
-        // ---- O^T += V^T . P: f16 hi, and lo while a lane's probabilities of this step weigh more than 1/8 of its sum ----
+        // ---- O^T += V^T . P (Q8g64: P'_g = p * v_scale_g, four output tiles per scale group): f16 hi, and lo while a
+        // lane's probabilities of this step weigh more than 1/8 of its sum ----
         const bool lo_pass = __any(heavy);
-        Frag phi[CT], plo[CT];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                phi[ct].u[e] = pack_f16_hw(pr[ct][2 * e], pr[ct][2 * e + 1]);
-                const f16x2 hi = __builtin_bit_cast(f16x2, pack_f16_hw(pr[ct][2 * e], pr[ct][2 * e + 1]));
-                plo[ct].u[e] = pack_f16_hw(pr[ct][2 * e] - (float)hi[0], pr[ct][2 * e + 1] - (float)hi[1]);
-            }
-        }
         PREFILL_PHASE_FENCE();
 #pragma unroll
         for (int q = 0; q < C::kDT / 4; ++q) {
+            f32x4 gs0 = {1.f, 1.f, 1.f, 1.f}, gs1 = {1.f, 1.f, 1.f, 1.f};
+            if constexpr (Q8) {
+                gs0 = *(const f32x4*)(&lds_vs[sbuf][q][4 * j]);
+                gs1 = *(const f32x4*)(&lds_vs[sbuf][q][16 + 4 * j]);
+            }
+            Frag phi[CT], plo[CT];
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float x0 = Q8 ? pr[ct][2 * e] * (e < 2 ? gs0[2 * e] : gs1[2 * e - 4]) : pr[ct][2 * e];
+                    const float x1 = Q8 ? pr[ct][2 * e + 1] * (e < 2 ? gs0[2 * e + 1] : gs1[2 * e - 3]) : pr[ct][2 * e + 1];
+                    phi[ct].u[e] = pack_f16_hw(x0, x1);
+                    const f16x2 hi = __builtin_bit_cast(f16x2, pack_f16_hw(x0, x1));
+                    plo[ct].u[e] = pack_f16_hw(x0 - (float)hi[0], x1 - (float)hi[1]);
+                }
+            }
             if (q + 1 < C::kDT / 4) { // the next four fragments travel while these multiply
 #pragma unroll
                 for (int tt = 0; tt < 4; ++tt) {
@@ -902,11 +1002,24 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
     unsigned int entry_next = entry_of(t_begin + kStep + st_token);
     store_step(regs, 0);
     __syncthreads();
+    unsigned int wv = 2u; // Q8g64: (biased) exponent of the largest V scale up to the tile being attended
+    float v_shift = Q8 ? kPBias + 125.0f : kPBias;
     auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
         const unsigned int t0 = t_begin + step * kStep;
         load_step(regs, t0 + kStep, entry_next); // past the end of the range the last row repeats: loads stay inside the pages
         entry_next = entry_of(t0 + 2u * kStep + st_token);
-        compute_step(buf, t0);
+        bool window_moved = false;
+        float acc_fix = 1.0f;
+        if constexpr (Q8) {
+            const unsigned int wv_now = window_of(buf, wv);
+            window_moved = wv_now != wv; // rare: a V scale above everything met so far
+            if (window_moved) {
+                acc_fix = ldexpf(1.0f, (int)wv - (int)wv_now);
+                wv = wv_now;
+                v_shift = kPBias + (float)(127 - (int)wv);
+            }
+        }
+        compute_step(buf, t0, v_shift, acc_fix, window_moved);
         store_step(regs, buf ^ 1);
         __syncthreads();
     };
@@ -929,7 +1042,8 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
         if (!(col < cols_used && r < p.rows)) {
             continue;
         }
-        const float inv = (total > 0.0f && total < __builtin_inff()) ? 1.0f / total : 0.0f; // the 2^8 of P cancels here
+        // accumulators and sum carry the same power of two (2^8 and, for Q8g64, the V window), which cancels here
+        const float inv = (total > 0.0f && total < __builtin_inff()) ? 1.0f / total : 0.0f;
         const size_t base = ((size_t)r * p.num_heads + head) * D;
 #pragma unroll
         for (int t = 0; t < C::kDT; ++t) {
@@ -961,17 +1075,19 @@ __global__ __launch_bounds__(512) void gqa_prefill_f16(GqaPrefillParams p)
     }
 }
 
-template <int D> static hipError_t launch_prefill_f16(const GqaPrefillParams& p, hipStream_t stream)
+template <int D, int KV, int SDT> static hipError_t launch_prefill_tiles(const GqaPrefillParams& p, hipStream_t stream)
 {
-    const unsigned int cols = F16Prefill<D>::kCols;
+    const unsigned int cols = TileShape<D>::kCols;
     const unsigned int rows_per_wg = p.group >= cols ? 1u : cols / p.group;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
     const bool cap = p.softcap > 0.0f;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
     if (cap) {
-        pow2 ? gqa_prefill_f16<D, true, true><<<grid, dim3(512), 0, stream>>>(p) : gqa_prefill_f16<D, true, false><<<grid, dim3(512), 0, stream>>>(p);
+        pow2 ? gqa_prefill_tiles<D, KV, SDT, true, true><<<grid, dim3(512), 0, stream>>>(p)
+             : gqa_prefill_tiles<D, KV, SDT, true, false><<<grid, dim3(512), 0, stream>>>(p);
     } else {
-        pow2 ? gqa_prefill_f16<D, false, true><<<grid, dim3(512), 0, stream>>>(p) : gqa_prefill_f16<D, false, false><<<grid, dim3(512), 0, stream>>>(p);
+        pow2 ? gqa_prefill_tiles<D, KV, SDT, false, true><<<grid, dim3(512), 0, stream>>>(p)
+             : gqa_prefill_tiles<D, KV, SDT, false, false><<<grid, dim3(512), 0, stream>>>(p);
     }
     return hipGetLastError();
 }
@@ -982,14 +1098,23 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
 {
     if (kv_format == 1) { // f16 rows
         if (p.head_dim == 128u) {
-            return launch_prefill_f16<128>(p, stream);
+            return launch_prefill_tiles<128, 1, 0>(p, stream);
         }
         if (p.head_dim == 256u) {
-            return launch_prefill_f16<256>(p, stream);
+            return launch_prefill_tiles<256, 1, 0>(p, stream);
         }
         return hipErrorInvalidValue;
     }
-    if (kv_format != 0 || p.head_dim != (unsigned int)kD) {
+    if (kv_format != 0 || scale_dtype > 1) {
+        return hipErrorInvalidValue;
+    }
+    if (p.head_dim == 64u) {
+        return scale_dtype == 0 ? launch_prefill_tiles<64, 0, 0>(p, stream) : launch_prefill_tiles<64, 0, 1>(p, stream);
+    }
+    if (p.head_dim == 256u) {
+        return scale_dtype == 0 ? launch_prefill_tiles<256, 0, 0>(p, stream) : launch_prefill_tiles<256, 0, 1>(p, stream);
+    }
+    if (p.head_dim != (unsigned int)kD) {
         return hipErrorInvalidValue;
     }
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
