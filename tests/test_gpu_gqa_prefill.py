@@ -307,8 +307,9 @@ def run_f16_case(seed, d, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_t
 def test_prefill_f16_kv(d, prefix, chunk, window, softcap):
     """Chunked prefill over an f16 cache (the config-3 model family prefills too): head_dim 128 and 256 run a matrix-core
     kernel of their own; the soft cap is the family's 50."""
-    out, want = run_f16_case(d + prefix, d, prefix, chunk, 16, 8, window=window, softcap=softcap)
-    print("prefill f16", d, assert_attention_close(out, want, f"f16 KV prefill d={d}"))
+    for q_kind in ("bf16", "f32"):  # bf16 activations run the tile kernel, f32 queries the decode kernels' route
+        out, want = run_f16_case(d + prefix, d, prefix, chunk, 16, 8, window=window, softcap=softcap, q_kind=q_kind)
+        print("prefill f16", d, q_kind, assert_attention_close(out, want, f"f16 KV prefill d={d} q={q_kind}"))
 
 
 @pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,softcap,block_tokens,q_kind",
