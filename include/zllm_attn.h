@@ -308,11 +308,11 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * src/backend/rocm/attention.rs:2232-2242).  Row r attends logical tokens
  * key_range(position + r, position + rows) of one sequence whose K/V
  * (including the chunk's own rows) are already in the paged cache.
- * Q8g64 caches with 16-bit scales (head_dim 64 / 128 / 256) and f16 caches
+ * Q8g64 caches (head_dim 64 / 128 / 256, scales of any type) and f16 caches
  * (head_dim 128 / 256) run matrix-core chunk kernels and need no workspace.  What is
- * left -- f32 scales; f32 queries other than over Q8g64 at head_dim 128; more than
- * 128 query heads per KV head at head_dim 256 -- runs every row as one item of the
- * split-KV decode kernels (bound by cache bandwidth, not by the matrix cores) and
+ * left -- f32 queries other than over Q8g64 with 16-bit scales at head_dim 128; more
+ * than 128 query heads per KV head at head_dim 256 -- runs every row as one item of
+ * the split-KV decode kernels (bound by cache bandwidth, not by the matrix cores) and
  * needs zllm_attn_gqa_prefill_workspace_bytes of workspace. */
 typedef struct zllm_gqa_prefill_args {
     const void* q;         /* [dev] [rows, num_heads * head_dim], q_dtype */

@@ -368,7 +368,9 @@ def test_prefill_q8_tiles_and_the_decode_route_agree(d, q_bf16):
     print("prefill q8 tiles", d, q_bf16, assert_attention_close(out.cpu().numpy(), want, f"Q8 prefill d={d} bf16={q_bf16}"))
 
 
-def test_prefill_f32_scale_cache():
-    """A chunk over a cache with f32 scales (CUDA convention): appended by the library, attended through the decode kernels."""
-    out, want = run_case(321, 400, 60, 16, 4, rule=O.RULE_CUDA_GQA)
-    print("prefill f32 scales", assert_attention_close(out.cpu().numpy(), want, "f32-scale prefill"))
+@pytest.mark.parametrize("d,q_bf16", [(128, True), (64, True), (256, True), (128, False)])
+def test_prefill_f32_scale_cache(d, q_bf16):
+    """A chunk over a cache with f32 scales (CUDA convention): appended by the library, attended by the tile kernel (bf16
+    queries) or through the decode kernels (f32 queries)."""
+    out, want = run_case(321 + d, 400, 60, 16, 4, rule=O.RULE_CUDA_GQA, d=d, q_bf16=q_bf16, outliers=True)
+    print("prefill f32 scales", d, q_bf16, assert_attention_close(out.cpu().numpy(), want, f"f32-scale prefill d={d}"))

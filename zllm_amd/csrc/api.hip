@@ -882,22 +882,19 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     return 0;
 }
 
-// Q8g64 caches with 16-bit scales and f16 caches run the matrix-core chunk kernels, which keep all of their state on chip
-// (head_dim 64 / 128 / 256, f16: 128 / 256).  What is left runs each row of the chunk as one item of the split-KV decode
-// kernels (row r is a sequence of position + r + 1 tokens over the same block table): f32 scales; more than 128 query
-// heads per KV head at head_dim 256 (a workgroup has 128 columns there); and f32 queries outside the head_dim-128
-// Q8g64 kernel.  The chunk kernels carry a query as f16, exact for bf16 and f16 activations; an f32 query loses 13 bits,
-// which large logits and outlier channels turn into errors past the 2e-3 bound (measured 2.6e-3 at head_dim 256 and
-// 6e-3 at head_dim 64 with a doubled score scale), and the decode kernels' query is wider.  That route re-reads the KV
-// bytes per row, so it is bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and the
-// split records.
+// Q8g64 caches (scales of any type) and f16 caches run the matrix-core chunk kernels, which keep all of their state on
+// chip (head_dim 64 / 128 / 256, f16: 128 / 256).  What is left runs each row of the chunk as one item of the split-KV
+// decode kernels (row r is a sequence of position + r + 1 tokens over the same block table): more than 128 query heads
+// per KV head at head_dim 256 (a workgroup has 128 columns there), and f32 queries outside gqa_prefill_q8 (head_dim 128,
+// 16-bit scales).  The chunk kernels carry a query as f16, exact for bf16 and f16 activations; an f32 query loses 13
+// bits, which large logits and outlier channels turn into errors past the 2e-3 bound (measured 2.6e-3 at head_dim 256
+// and 6e-3 at head_dim 64 with a doubled score scale), and the decode kernels' query is wider.  That route re-reads the
+// KV bytes per row, so it is bound by the cache bandwidth rather than the matrix cores; it needs the rows' ranges and
+// the split records.
 static bool prefill_rows_as_decode_items(const zllm_gqa_prefill_args* a)
 {
     const bool q8 = a->kv_format == ZLLM_KV_Q8G64;
-    if (q8 && a->scale_dtype == ZLLM_SCALE_F32) {
-        return true;
-    }
-    if (a->q_dtype == ZLLM_DTYPE_F32 && !(q8 && a->head_dim == 128)) {
+    if (a->q_dtype == ZLLM_DTYPE_F32 && !(q8 && a->head_dim == 128 && a->scale_dtype != ZLLM_SCALE_F32)) {
         return true;
     }
     return a->head_dim == 256 && a->num_heads / a->num_kv_heads > 128u;

@@ -585,7 +585,7 @@ template <int D> struct TileShape {
     __device__ static __forceinline__ unsigned int swizzle(unsigned int row) { return swz(row) & (unsigned int)(kChunks - 1); }
 };
 
-// KV: 0 = Q8g64 (SDT names the 16-bit scale type), 1 = f16 rows
+// KV: 0 = Q8g64 (SDT names the scale type: bf16, f16 or f32), 1 = f16 rows
 template <int D, int KV, int SDT, bool SOFTCAP, bool POW2>
 __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
 {
@@ -684,7 +684,8 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     const float tanh_arg = SOFTCAP ? score_mult * (2.0f * kLog2e) / p.softcap : 0.0f; // product -> 2 y log2(e), y = score / cap
     const bool small_cap = p.softcap < 256.0f;
     const unsigned int k_row = p.num_kv_heads * (Q8 ? (unsigned int)D : (unsigned int)C::kRow); // bytes of one cache row
-    const unsigned int s_row = p.num_kv_heads * G * 2u;                                         // bytes of one scale row
+    constexpr unsigned int kScaleBytes = SDT == 2 ? 4u : 2u;
+    const unsigned int s_row = p.num_kv_heads * G * kScaleBytes;                                // bytes of one scale row
     const bool pow2 = POW2 || (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const unsigned int last_token = t_end - 1u;
     auto entry_of = [&](unsigned int token) __attribute__((always_inline)) -> unsigned int {
@@ -704,10 +705,10 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     const unsigned int st_token = (tid & 255u) >> 3;
     const unsigned int cc = tid & 7u;
     const unsigned char* st_plane = (stage_v ? p.v_plane : p.k_plane) + (size_t)kvh * (Q8 ? D : C::kRow) + cc * (Q8 ? 8u : 16u);
-    const unsigned char* st_scales = Q8 ? (stage_v ? p.v_scales : p.k_scales) + (size_t)kvh * G * 2u : nullptr;
+    const unsigned char* st_scales = Q8 ? (stage_v ? p.v_scales : p.k_scales) + (size_t)kvh * G * kScaleBytes : nullptr;
     struct StageRegs {
         u32x4 chunk[C::kLoads]; // f16 rows: the chunk as stored; Q8g64: eight codes in the first two words
-        u32x2 scales;           // Q8g64: the token's G 16-bit scales
+        u32x4 scales;           // Q8g64: the token's G scales (16-bit ones packed two to a word, f32 ones a word each)
     };
     auto load_step = [&](StageRegs& r, unsigned int t0, unsigned int entry) __attribute__((always_inline)) {
         const unsigned long long row = row_from(t0 + st_token, entry);
@@ -722,13 +723,15 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
             }
         }
         if constexpr (Q8) {
-            const unsigned char* sp = st_scales + row * s_row;
-            if constexpr (G == 1) {
-                r.scales = u32x2{*(const unsigned short*)sp, 0u};
-            } else if constexpr (G == 2) {
-                r.scales = u32x2{*(const unsigned int*)sp, 0u};
-            } else { // the scale planes are only known to be 4-byte aligned
-                r.scales = u32x2{((const unsigned int*)sp)[0], ((const unsigned int*)sp)[1]};
+            const unsigned char* sp = st_scales + row * s_row; // the scale planes are only known to be 4-byte aligned
+            r.scales = u32x4{0u, 0u, 0u, 0u};
+            if constexpr (G * kScaleBytes == 2u) {
+                r.scales[0] = *(const unsigned short*)sp;
+            } else {
+#pragma unroll
+                for (unsigned int w = 0; w < G * kScaleBytes / 4u; ++w) {
+                    r.scales[w] = ((const unsigned int*)sp)[w];
+                }
             }
         }
     };
@@ -750,7 +753,12 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
             float top = 0.0f;
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                const float sg = scale_bits_to_f32<SDT>((unsigned short)((r.scales[g >> 1] >> (16 * (g & 1))) & 0xffffu));
+                float sg;
+                if constexpr (SDT == 2) {
+                    sg = __uint_as_float(r.scales[g]);
+                } else {
+                    sg = scale_bits_to_f32<SDT>((unsigned short)((r.scales[g >> 1] >> (16 * (g & 1))) & 0xffffu));
+                }
                 top = fmaxf(top, sg);
                 if (cc == 0) {
                     (stage_v ? lds_vs : lds_ks)[buf][g][st_token] = stage_v ? sg : sg * scale_log2;
@@ -1105,17 +1113,22 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
         }
         return hipErrorInvalidValue;
     }
-    if (kv_format != 0 || scale_dtype > 1) {
+    if (kv_format != 0 || scale_dtype < 0 || scale_dtype > 2) {
         return hipErrorInvalidValue;
     }
     if (p.head_dim == 64u) {
-        return scale_dtype == 0 ? launch_prefill_tiles<64, 0, 0>(p, stream) : launch_prefill_tiles<64, 0, 1>(p, stream);
+        return scale_dtype == 0 ? launch_prefill_tiles<64, 0, 0>(p, stream)
+                                : scale_dtype == 1 ? launch_prefill_tiles<64, 0, 1>(p, stream) : launch_prefill_tiles<64, 0, 2>(p, stream);
     }
     if (p.head_dim == 256u) {
-        return scale_dtype == 0 ? launch_prefill_tiles<256, 0, 0>(p, stream) : launch_prefill_tiles<256, 0, 1>(p, stream);
+        return scale_dtype == 0 ? launch_prefill_tiles<256, 0, 0>(p, stream)
+                                : scale_dtype == 1 ? launch_prefill_tiles<256, 0, 1>(p, stream) : launch_prefill_tiles<256, 0, 2>(p, stream);
     }
     if (p.head_dim != (unsigned int)kD) {
         return hipErrorInvalidValue;
+    }
+    if (scale_dtype == 2) { // f32 scales at head_dim 128: the tile kernel (gqa_prefill_q8 reads 16-bit scales)
+        return launch_prefill_tiles<128, 0, 2>(p, stream);
     }
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
