@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration", "mfma_issue_calibration"])
     ap.add_argument("--pool-gib", type=float, default=256.0, help="address span of the paged pool (all four planes); clipped to 90 %% of free HBM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -64,6 +64,8 @@ def probe_lib():
         lib.bench_probe_paged_read.argtypes = [C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         lib.bench_probe_paged_read_lds.restype = C.c_int
         lib.bench_probe_paged_read_lds.argtypes = lib.bench_probe_paged_read.argtypes
+        lib.bench_probe_mfma_issue.restype = C.c_int
+        lib.bench_probe_mfma_issue.argtypes = [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p]
         _PROBE = lib
     return _PROBE
 
@@ -414,6 +416,41 @@ def run_read_calibration(args):
                       "frac_of_hbm_peak": round(first["gbps_median"] / HBM_PEAK_GBPS, 4)}))
 
 
+def run_mfma_issue_calibration(args):
+    """What one SIMD issues when matrix and vector instructions meet (bench_probe.hip: mfma_issue_kernel): trips of
+    8 MFMAs 16x16x32 f16, of 24 FMAs, of both one after the other and of both interleaved, with one and with two waves
+    per SIMD on every CU.  `value` is the matrix rate of the MFMA-only loop with two waves per SIMD: the rate the
+    device sustains for this instruction, next to the published peak."""
+    import torch
+
+    sink = torch.zeros((1,), dtype=torch.float32, device="cuda")
+    lib = probe_lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    trips = 20000
+    table = {}
+    for waves in (1, 2, 4):
+        for mode, name in enumerate(("mfma8", "fma24", "mfma8_then_fma24", "mfma_fma3_x8", "mfma8_wave_beside_fma24_waves", "mfma4_then_fma12", "mfma_fma3_x4")):
+            if waves == 1 and mode == 4:
+                continue
+            def fn():
+                rc = lib.bench_probe_mfma_issue(mode, waves, cus, trips, sink.data_ptr(), stream)
+                if rc != 0:
+                    raise RuntimeError(f"bench_probe_mfma_issue: {rc}")
+            for _ in range(max(args.warmup, 2)):
+                fn()
+            settle_clocks(fn)
+            med, low = event_times_ms(fn, max(5, min(args.steps, 20)))
+            table[f"{name}_{waves}_per_simd"] = {"ns_per_trip": round(med * 1e6 / trips, 2), "ns_per_trip_min": round(low * 1e6 / trips, 2)}
+    mfma_ns = table["mfma8_2_per_simd"]["ns_per_trip"] / 16.0  # 16 MFMAs per SIMD and trip
+    tflops = 16 * 16 * 32 * 2 / mfma_ns * 4 * cus / 1e3
+    print(json.dumps({"metric": "sustained MFMA 16x16x32 f16 rate (issue calibration)", "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(table["mfma8_2_per_simd"]["ns_per_trip"] * trips / 1e6, 5),
+                      "config": {"workload": "bench_probe_mfma_issue: one workgroup per CU, one and two waves per SIMD", "cus": cus, "trips": trips,
+                                 "ns_per_mfma_two_waves": round(mfma_ns, 3), **table},
+                      "frac_of_mfma_peak": round(tflops / 2500.0, 4)}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -427,6 +464,8 @@ def main():
         run_gqa_decode(args, ragged=False, config1=True)
     elif args.workload == "copy_calibration":
         run_copy_calibration(args)
+    elif args.workload == "mfma_issue_calibration":
+        run_mfma_issue_calibration(args)
     elif args.workload == "read_calibration":
         run_read_calibration(args)
     else:
