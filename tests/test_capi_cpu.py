@@ -169,6 +169,25 @@ def test_split_plan_covers_the_host_bound_and_sizes_the_workspace(lib):
     assert lib.zllm_attn_gqa_decode_split_plan(C.byref(bad), None, None) == -1
 
 
+def test_split_plan_fills_whole_rounds_of_the_compute_units(lib):
+    """A batch that does not divide the 256 CUs must not leave a few workgroups for a round of their own: with uniform
+    lengths the launch's rounds are at least 4/5 full whenever a sequence has keys to spare, and a head_dim-128
+    Q8g64 split stays within the 127 pages whose table entries the page-streaming kernel keeps in registers."""
+    for batch in (1, 2, 3, 5, 7, 8, 12, 13, 24, 31, 48, 64):
+        for max_len in (4096, 16384, 32768, 65536, 131072):
+            args = capi.GqaDecodeArgs()
+            args.batch, args.num_kv_heads, args.num_heads, args.head_dim = batch, 8, 64, 128
+            args.max_kv_len, args.block_tokens, args.score_scale = max_len, 16, 0.1
+            args.kv_format, args.scale_dtype, args.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16
+            chunk, chunks = C.c_uint32(), C.c_uint32()
+            assert lib.zllm_attn_gqa_decode_split_plan(C.byref(args), C.byref(chunk), C.byref(chunks)) == 0
+            groups = batch * chunks.value  # one workgroup per (sequence, split): all eight KV heads ride in it
+            rounds = -(-groups // 256)
+            if chunk.value > 64:  # at the shortest split there are no more keys to spread
+                assert groups >= rounds * 256 * 4 // 5, (batch, max_len, chunk.value, chunks.value)
+            assert chunk.value <= 127 * 16, (batch, max_len, chunk.value)
+
+
 def test_prefill_and_mla_argument_checks_without_a_gpu(lib):
     pre = capi.GqaPrefillArgs()
     pre.rows, pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens = 8, 8, 2, 128, 16

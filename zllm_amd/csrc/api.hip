@@ -102,18 +102,35 @@ bool valid_head_dim(uint32_t d)
     return d == 64 || d == 128 || d == 256;
 }
 
-// Tokens per KV split: one workgroup per CU over the call (a second round would repeat every
-// workgroup's prologue), but splits long enough that the partial write / merge stay a few percent of
-// the KV bytes a split reads.
-void plan_splits(uint64_t total_tokens, uint32_t max_len, uint32_t columns, uint32_t min_chunk, uint32_t rounds, uint32_t* chunk_tokens,
-                 uint32_t* max_chunks)
+// Tokens per KV split.  `units` (sequence, head-block) pairs each cut their keys into the same number of splits, one
+// workgroup per split, and the launch runs in rounds of one workgroup per CU: workgroups beyond the last full round run
+// alone while the other CUs idle, which is what a split count that is merely rounded up costs a batch that does not
+// divide the CU count.  So the candidates are the split counts that fill 1, 2, ... 8 rounds, each priced as
+// rounds x (tokens of a split + what a workgroup's prologue and epilogue cost, about two 32-token steps), and the
+// cheapest is taken, the fewest rounds among equals.  `min_chunk` keeps the partial records and their merge a few
+// percent of the KV bytes a split reads.
+void plan_splits(uint32_t max_len, uint32_t units, uint32_t min_chunk, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
-    // `columns` workgroups run per split; aim at `rounds` workgroups per CU over the whole call
-    const uint64_t target = (uint64_t)rounds * kComputeUnits;
-    uint64_t chunk = (total_tokens * columns + target - 1) / target;
-    chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
-    *chunk_tokens = (uint32_t)chunk;
-    const uint64_t chunks = ((uint64_t)max_len + chunk - 1) / chunk;
+    constexpr uint64_t kFixedTokens = 64;
+    uint64_t best_chunk = align_up(max_len < min_chunk ? min_chunk : max_len, 32); // one split per pair
+    uint64_t best_cost = ~(uint64_t)0;
+    for (uint64_t rounds = 1; rounds <= 8; ++rounds) {
+        const uint64_t per_unit = rounds * kComputeUnits / units;
+        if (per_unit == 0) {
+            continue;
+        }
+        uint64_t chunk = ((uint64_t)max_len + per_unit - 1) / per_unit;
+        chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
+        const uint64_t splits = ((uint64_t)max_len + chunk - 1) / chunk;
+        const uint64_t launched = (splits * units + kComputeUnits - 1) / kComputeUnits;
+        const uint64_t cost = launched * (chunk + kFixedTokens);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best_chunk = chunk;
+        }
+    }
+    *chunk_tokens = (uint32_t)best_chunk;
+    const uint64_t chunks = ((uint64_t)max_len + best_chunk - 1) / best_chunk;
     *max_chunks = (uint32_t)(chunks == 0 ? 1 : chunks);
 }
 
@@ -157,26 +174,46 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
 // the KV bytes even at 64 tokens per split.
 constexpr uint64_t kMinGqaChunk = 64;
 
+// The head_dim-128 Q8g64 kernel that streams pages straight into LDS keeps a split's block-table entries in two
+// registers per lane: a split of at most 127 pages.  A longer split is cut into equal shorter ones (further whole rounds
+// of workgroups), so that a long batch keeps that kernel.
+void cap_split_for_page_registers(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    const bool pow2 = (a->block_tokens & (a->block_tokens - 1u)) == 0;
+    if (a->kv_format != ZLLM_KV_Q8G64 || a->head_dim != 128 || a->scale_dtype == ZLLM_SCALE_F32 || a->ring_capacity != 0 || !pow2 ||
+        a->block_tokens < 16u) {
+        return;
+    }
+    const uint64_t limit = ((uint64_t)127u * a->block_tokens) & ~(uint64_t)31u;
+    if (*chunk_tokens <= limit) {
+        return;
+    }
+    const uint64_t parts = (*chunk_tokens + limit - 1) / limit;
+    const uint64_t chunk = align_up((*chunk_tokens + parts - 1) / parts, 32);
+    *chunk_tokens = (uint32_t)chunk;
+    *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
+}
+
 void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
     const uint32_t max_waves = zllm::gqa_decode_max_waves(a->head_dim);
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
-    const uint32_t rounds = 1u; // workgroups per CU over the call
     const uint32_t columns = a->batch * kvh_blocks * head_blocks;
     const uint64_t uniform_total = (uint64_t)a->batch * a->max_kv_len;
-    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && rounds * kComputeUnits > 2 * columns) {
+    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && kComputeUnits > 2 * columns) {
         // ragged batch: sum_b ceil(len_b / chunk) <= total / chunk + batch, so size the splits for the
         // workgroups that will really run and keep them within one round of the CUs
-        const uint64_t slots = (uint64_t)rounds * kComputeUnits / (kvh_blocks * head_blocks) - a->batch;
+        const uint64_t slots = (uint64_t)kComputeUnits / (kvh_blocks * head_blocks) - a->batch;
         uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
         chunk = align_up(chunk < kMinGqaChunk ? kMinGqaChunk : chunk, 32);
         *chunk_tokens = (uint32_t)chunk;
         *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
-        return;
+    } else {
+        plan_splits(a->max_kv_len, columns, kMinGqaChunk, chunk_tokens, max_chunks);
     }
-    plan_splits(a->max_kv_len, a->max_kv_len, columns, kMinGqaChunk, rounds, chunk_tokens, max_chunks);
+    cap_split_for_page_registers(a, chunk_tokens, max_chunks);
 }
 
 // query rows per sequence: 0 and 1 both mean a decode step
@@ -233,7 +270,7 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    plan_splits(longest, longest, a->batch * mla_query_rows(a) * head_blocks, 64, 1, chunk_tokens, max_chunks);
+    plan_splits(longest, a->batch * mla_query_rows(a) * head_blocks, 64, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {
