@@ -258,6 +258,26 @@ def test_batch_larger_than_a_wave_with_empty_sequences():
     assert not got[[3, 17, 64, 69]].any()
 
 
+@pytest.mark.parametrize("fmt,hq,hkv,d,window", [("q8", 8, 1, 128, 0), ("q8", 16, 2, 128, 100), ("q8", 6, 3, 128, 0), ("q8", 4, 1, 64, 0),
+                                                  ("q8", 8, 2, 64, 33), ("q8", 4, 1, 256, 0), ("q8", 16, 2, 256, 700),
+                                                  ("f16", 8, 1, 128, 0), ("f16", 4, 2, 128, 64), ("f16", 4, 1, 256, 0), ("f16", 32, 2, 256, 500)])
+def test_few_kv_heads_share_a_workgroup(fmt, hq, hkv, d, window):
+    """With one to three KV heads a workgroup runs several (sequence, split) items side by side.  The item count here
+    is not a multiple of the items in a workgroup (the last workgroup has idle waves), one sequence is empty and the
+    lengths cut into different numbers of splits."""
+    lens = [1000, 0, 37, 2049, 515, 3000, 64]
+    if fmt == "q8":
+        case = make_gqa_q8_case(900 + hq + d, lens, hq, hkv, d, outliers=True)
+        got = run_decode(case, 0.09, window=window)
+        want = oracle_gqa_decode(case, 0.09, window=window)
+    else:
+        case = make_f16_case(900 + hq + d, lens, hq, hkv, d)
+        got = run_f16(case, 0.09, window=window)
+        want = oracle_gqa_decode(case, 0.09, window=window, fmt=O.FMT_F16)
+    assert_attention_close(got, want, f"{fmt} {hq}/{hkv} d={d} window={window}")
+    assert not got[1].any()
+
+
 @pytest.mark.parametrize("q_kind", ["f32", "bf16", "f16"])
 def test_query_dtypes_through_fixed_point_digits(q_kind):
     """The kernel quantizes each query row to 15-bit fixed point for the int8 matrix cores; every input

@@ -109,20 +109,22 @@ bool valid_head_dim(uint32_t d)
 // rounds x (tokens of a split + what a workgroup's prologue and epilogue cost, about two 32-token steps), and the
 // cheapest is taken, the fewest rounds among equals.  `min_chunk` keeps the partial records and their merge a few
 // percent of the KV bytes a split reads.
-void plan_splits(uint32_t max_len, uint32_t units, uint32_t min_chunk, uint32_t* chunk_tokens, uint32_t* max_chunks)
+void plan_splits(uint32_t max_len, uint64_t units, uint32_t units_per_group, uint32_t min_chunk, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
+    // `units_per_group` of a pair's splits share one workgroup (GQA decode with few KV heads)
     constexpr uint64_t kFixedTokens = 64;
     uint64_t best_chunk = align_up(max_len < min_chunk ? min_chunk : max_len, 32); // one split per pair
     uint64_t best_cost = ~(uint64_t)0;
     for (uint64_t rounds = 1; rounds <= 8; ++rounds) {
-        const uint64_t per_unit = rounds * kComputeUnits / units;
+        const uint64_t per_unit = rounds * kComputeUnits * units_per_group / units;
         if (per_unit == 0) {
             continue;
         }
         uint64_t chunk = ((uint64_t)max_len + per_unit - 1) / per_unit;
         chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
         const uint64_t splits = ((uint64_t)max_len + chunk - 1) / chunk;
-        const uint64_t launched = (splits * units + kComputeUnits - 1) / kComputeUnits;
+        const uint64_t groups = (splits * units + units_per_group - 1) / units_per_group;
+        const uint64_t launched = (groups + kComputeUnits - 1) / kComputeUnits;
         const uint64_t cost = launched * (chunk + kFixedTokens);
         if (cost < best_cost) {
             best_cost = cost;
@@ -200,18 +202,19 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
     const uint32_t head_blocks = (a->num_heads / a->num_kv_heads + 15) / 16;
-    const uint32_t columns = a->batch * kvh_blocks * head_blocks;
+    const uint32_t items_per_group = zllm::gqa_decode_items_per_group(a->head_dim, a->num_kv_heads);
+    const uint64_t columns = (uint64_t)a->batch * kvh_blocks * head_blocks;
     const uint64_t uniform_total = (uint64_t)a->batch * a->max_kv_len;
-    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && kComputeUnits > 2 * columns) {
+    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && (uint64_t)kComputeUnits * items_per_group > 2 * columns) {
         // ragged batch: sum_b ceil(len_b / chunk) <= total / chunk + batch, so size the splits for the
         // workgroups that will really run and keep them within one round of the CUs
-        const uint64_t slots = (uint64_t)kComputeUnits / (kvh_blocks * head_blocks) - a->batch;
+        const uint64_t slots = (uint64_t)kComputeUnits * items_per_group / (kvh_blocks * head_blocks) - a->batch;
         uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
         chunk = align_up(chunk < kMinGqaChunk ? kMinGqaChunk : chunk, 32);
         *chunk_tokens = (uint32_t)chunk;
         *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
     } else {
-        plan_splits(a->max_kv_len, columns, kMinGqaChunk, chunk_tokens, max_chunks);
+        plan_splits(a->max_kv_len, columns, items_per_group, kMinGqaChunk, chunk_tokens, max_chunks);
     }
     cap_split_for_page_registers(a, chunk_tokens, max_chunks);
 }
@@ -270,7 +273,7 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    plan_splits(longest, a->batch * mla_query_rows(a) * head_blocks, 64, chunk_tokens, max_chunks);
+    plan_splits(longest, (uint64_t)a->batch * mla_query_rows(a) * head_blocks, 1, 64, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {

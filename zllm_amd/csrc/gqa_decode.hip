@@ -140,6 +140,27 @@ template <int G, int N> __device__ __forceinline__ ScaleRow<G> row_bcast_scales(
     return out;
 }
 
+// A workgroup's waves: `items_per_group` work items side by side, each with one wave per KV head of the block (all KV
+// heads when they fit the workgroup).  With one or two KV heads -- a small model, or one GPU's share of the heads -- a
+// workgroup of one item would be one or two waves on a CU, far too few loads in flight; the waves share nothing, so
+// several items ride in one workgroup instead.
+struct WaveItem {
+    unsigned int kvh, head_block, item;
+};
+__device__ __forceinline__ WaveItem wave_item(const GqaDecodeParams& p)
+{
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned int items = max(p.items_per_group, 1u);
+    const unsigned int waves = (blockDim.x >> 6) / items; // per item
+    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
+    const unsigned int sub = wave / waves;
+    WaveItem w;
+    w.kvh = (blockIdx.y % kvh_blocks) * waves + (wave - sub * waves);
+    w.head_block = blockIdx.y / kvh_blocks;
+    w.item = blockIdx.x * items + sub;
+    return w;
+}
+
 // Split-KV work items are numbered densely over the batch: item = (sequence b, split c) with
 // c < splits(b), sequences in order.  Workgroups are handed to the XCDs round-robin by their linear id, so
 // a dense numbering spreads the live workgroups of a ragged batch evenly (a [split][sequence] grid leaves
@@ -434,12 +455,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int m = lane & 15u;  // MFMA row / column index of this lane
     const unsigned int j = lane >> 4;   // k-slice index of this lane
-    const unsigned int waves = blockDim.x >> 6;
-    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
-    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
-    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const WaveItem mine = wave_item(p);
+    const unsigned int kvh = mine.kvh;
+    const unsigned int head_block = mine.head_block;
     unsigned int b, chunk, len, first, span;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -698,10 +718,9 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned int waves = blockDim.x >> 6;
-    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
-    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + wave;
-    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const WaveItem mine = wave_item(p);
+    const unsigned int kvh = mine.kvh;
+    const unsigned int head_block = mine.head_block;
     if (kvh >= p.num_kv_heads) {
         return;
     }
@@ -710,8 +729,8 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     // planned splits, item i is split i % max_chunks of sequence i / max_chunks: the entries of that guess are
     // requested together with the lengths and are kept if the guess turns out right.
     const unsigned int last_page = p.table_stride != 0 ? p.table_stride - 1u : 0u;
-    const unsigned int guess_b = min(blockIdx.x / p.max_chunks, p.batch - 1u);
-    const unsigned int guess_page = ((blockIdx.x - guess_b * p.max_chunks) * p.chunk_tokens) >> p.block_shift;
+    const unsigned int guess_b = min(mine.item / p.max_chunks, p.batch - 1u);
+    const unsigned int guess_page = ((mine.item - guess_b * p.max_chunks) * p.chunk_tokens) >> p.block_shift;
     const unsigned int* guess_table = p.tables + (p.table_shared ? 0 : (size_t)guess_b * p.table_stride);
     unsigned int entries0 = 0, entries1 = 0;
     if (p.tables != nullptr) {
@@ -719,7 +738,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         entries1 = guess_table[min(guess_page + 64u + lane, last_page)];
     }
     unsigned int b, chunk, len, first, span;
-    if (!locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    if (!locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -950,12 +969,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
-    const unsigned int waves = blockDim.x >> 6;
-    const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
-    const unsigned int kvh = (blockIdx.y % kvh_blocks) * waves + (threadIdx.x >> 6);
-    const unsigned int head_block = blockIdx.y / kvh_blocks;
+    const WaveItem mine = wave_item(p);
+    const unsigned int kvh = mine.kvh;
+    const unsigned int head_block = mine.head_block;
     unsigned int b, chunk, len, first, span;
-    if (kvh >= p.num_kv_heads || !locate_split(p, blockIdx.x, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -1263,24 +1281,25 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     float l = 0.0f;
     // Record addresses are clamped to the planned splits, not to this sequence's own count, so that the first trip's
     // loads do not wait for the length: what a dead split's record holds is never used.
-    for (unsigned int c0 = sl; c0 == sl || c0 < chunks; c0 += 4u * lanes) {
-        float cm[4], cl[4];
-        f32x4 part[4];
-        float2 st[4];
+    auto fold = [&](unsigned int c0, auto trip_c) __attribute__((always_inline)) {
+        constexpr int U = decltype(trip_c)::value;
+        float cm[U], cl[U];
+        f32x4 part[U];
+        float2 st[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const unsigned int c = min(c0 + u * lanes, p.max_chunks - 1u);
             st[u] = *(const float2*)(stats + c * stat_stride);
             part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const bool live = c0 + u * lanes < chunks;
             cm[u] = live ? st[u].x : kNegInf;
             cl[u] = live ? st[u].y : 0.0f;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             if (cl[u] > 0.0f) {
                 const float nm = fmaxf(m, cm[u]);
                 const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
@@ -1290,6 +1309,12 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
                 m = nm;
             }
         }
+    };
+    // the first trip runs whatever the split count is; a sequence with many splits (few KV heads: several items share a
+    // workgroup and the splits are short) then takes eight records per trip, a trip being one round trip to memory
+    fold(sl, std::integral_constant<int, 4>{});
+    for (unsigned int c0 = sl + 4u * lanes; c0 < chunks; c0 += 8u * lanes) {
+        fold(c0, std::integral_constant<int, 8>{});
     }
     __shared__ float sm[256];
     __shared__ float sl_sum[256];
@@ -1411,14 +1436,23 @@ unsigned int gqa_decode_max_waves(unsigned int head_dim)
     return head_dim > 128u ? 4u : 8u; // head_dim 256 needs the larger register file share
 }
 
-hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream)
+unsigned int gqa_decode_items_per_group(unsigned int head_dim, unsigned int num_kv_heads)
 {
+    // four waves keep a CU's loads flowing (measured with four KV heads: 5.8 TB/s); more items than that only add
+    // partial records for the merge
+    return num_kv_heads < 4u ? (num_kv_heads == 1u ? 4u : 2u) : 1u;
+}
+
+hipError_t launch_gqa_decode(const GqaDecodeParams& args, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream)
+{
+    GqaDecodeParams p = args;
     const unsigned int max_waves = gqa_decode_max_waves(p.head_dim);
     const unsigned int waves = p.num_kv_heads < max_waves ? p.num_kv_heads : max_waves;
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int head_blocks = (p.group + 15u) / 16u;
-    const dim3 grid(p.max_chunks * p.batch, kvh_blocks * head_blocks, 1);
-    const dim3 block(waves * 64u);
+    p.items_per_group = gqa_decode_items_per_group(p.head_dim, p.num_kv_heads);
+    const dim3 grid((p.max_chunks * p.batch + p.items_per_group - 1u) / p.items_per_group, kvh_blocks * head_blocks, 1);
+    const dim3 block(waves * p.items_per_group * 64u);
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const bool fast = pow2 && p.block_tokens >= 16u && p.ring_capacity % 16u == 0;
     hipError_t err = hipSuccess;

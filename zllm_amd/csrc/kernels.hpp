@@ -102,6 +102,9 @@ struct GqaDecodeParams {
     unsigned int query_rows;
     unsigned int table_shared; // 1: every item reads the one table at `tables` (rows of a prefill chunk); table_stride still bounds it
     int out_dtype;             // split merge: element type of `out` (0 f32, 1 bf16, 2 f16)
+    // partial kernels: (sequence, split) items a workgroup runs side by side, each with one wave per KV head of its block
+    // (0 = 1).  More than one when the KV heads alone would leave the workgroup's waves unused.
+    unsigned int items_per_group;
 };
 
 struct GqaPrefillParams {
@@ -152,6 +155,7 @@ struct MlaDecodeParams {
 
 // KV heads (= waves) per GQA decode workgroup for a head dimension.
 unsigned int gqa_decode_max_waves(unsigned int head_dim);
+unsigned int gqa_decode_items_per_group(unsigned int head_dim, unsigned int num_kv_heads);
 
 hipError_t launch_q8g64_append(const Q8AppendParams& p, hipStream_t stream);
 hipError_t launch_scatter_rows(const ScatterParams& p, hipStream_t stream);
