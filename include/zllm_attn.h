@@ -309,11 +309,16 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * key_range(position + r, position + rows) of one sequence whose K/V
  * (including the chunk's own rows) are already in the paged cache.
  * Q8g64 caches (head_dim 64 / 128 / 256, scales of any type) and f16 caches
- * (head_dim 128 / 256) run matrix-core chunk kernels and need no workspace.  What is
+ * (head_dim 128 / 256) run matrix-core chunk kernels.  A chunk with too few row tiles
+ * for the device -- a short chunk over a long prefix -- is cut into KV splits
+ * (parts of a tile's visible range, combined like a decode call's splits) when the
+ * caller passes zllm_attn_gqa_prefill_workspace_bytes of 16-byte aligned workspace
+ * for their records, and runs unsplit (same results, one workgroup walking the whole
+ * prefix per tile) when it passes none or less.  What is
  * left -- f32 queries other than over Q8g64 with 16-bit scales at head_dim 128; more
  * than 128 query heads per KV head at head_dim 256 -- runs every row as one item of
  * the split-KV decode kernels (bound by cache bandwidth, not by the matrix cores) and
- * needs zllm_attn_gqa_prefill_workspace_bytes of workspace. */
+ * cannot run without that workspace. */
 typedef struct zllm_gqa_prefill_args {
     const void* q;         /* [dev] [rows, num_heads * head_dim], q_dtype */
     const void* k_plane;   /* [dev] */

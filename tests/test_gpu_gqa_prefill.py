@@ -12,7 +12,7 @@ torch = pytest.importorskip("torch")
 
 def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, rule=O.RULE_METAL_GQA, q_bf16=True,
              out_dtype=None, scale=None, outliers=False, gate_cols=0, q_gain=1.0, k_gain=1.0, v_gain=1.0, oracle_segments=None,
-             d=128, visible_ends=None):
+             d=128, visible_ends=None, workspace=True):
     from zllm_amd import capi, ops
 
     out_dtype = out_dtype or torch.float32
@@ -61,7 +61,8 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
     out = ops.gqa_prefill_chunk(to_torch_bf16(q_bits, "cuda") if q_bf16 else upload(q), dev["k_codes"], dev["k_scales"], dev["v_codes"],
                                 dev["v_scales"], table, prefix, hq, hkv, d, block_tokens, scale, window=window, softcap=softcap,
                                 scale_dtype=sdt, out_dtype=out_dtype, gate=None if gate is None else upload(gate),
-                                visible_ends=None if visible_ends is None else upload(np.asarray(visible_ends, dtype=np.uint32)))
+                                visible_ends=None if visible_ends is None else upload(np.asarray(visible_ends, dtype=np.uint32)),
+                                workspace=workspace)
     torch.cuda.synchronize()
     kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], sdt, tables[0], block_tokens, 0, total, cols)
     vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], sdt, tables[0], block_tokens, 0, total, cols)
@@ -82,6 +83,54 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
         rc, want = O.sigmoid_gate(want, gate)
         assert rc == 0
     return out, want
+
+
+@pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,softcap,extra", [
+    (128, 5000, 8, 16, 2, 0, 0.0, ""), (128, 3000, 300, 8, 2, 700, 0.0, ""), (128, 2500, 70, 32, 4, 0, 30.0, "gate"),
+    (128, 4000, 33, 8, 1, 0, 0.0, "bf16out"), (128, 2000, 90, 8, 2, 0, 0.0, "ends"), (64, 3000, 20, 8, 2, 0, 0.0, ""),
+    (256, 3000, 20, 8, 2, 500, 0.0, ""), (128, 2600, 16, 16, 4, 0, 0.0, "f32scales")])
+def test_prefill_kv_splits_and_the_unsplit_kernel_agree(d, prefix, chunk, hq, hkv, window, softcap, extra):
+    """A short chunk over a long prefix is cut into KV splits when the caller brings the workspace for their records (parts
+    of a row tile's visible range, merged like a decode call's splits) and runs unsplit without one: both against the oracle.
+    Covered: row tiles whose range is shorter than the longest (parts beyond their own count stay empty), windows, the soft
+    cap, gates, bf16 output, explicit visible ends, f32 scales, head_dim 64 / 256 and outlier channels (the V window of a
+    split differs from its neighbours')."""
+    kw = dict(window=window, softcap=softcap, outliers=True, d=d)
+    if extra == "gate":
+        kw["gate_cols"] = hq * d
+    if extra == "bf16out":
+        kw["out_dtype"] = torch.bfloat16
+    if extra == "ends":
+        ends = np.arange(prefix + 1, prefix + chunk + 1, dtype=np.uint32)
+        ends[10:40] = prefix + 40  # a block of rows that reads to the end of the block
+        kw["visible_ends"] = ends
+    if extra == "f32scales":
+        kw["rule"] = O.RULE_CUDA_GQA
+    from zllm_amd import capi
+    import ctypes as C
+
+    probe = capi.GqaPrefillArgs()
+    probe.rows, probe.position, probe.window, probe.num_heads, probe.num_kv_heads, probe.head_dim = chunk, prefix, window, hq, hkv, d
+    probe.block_tokens, probe.score_scale, probe.kv_format = 16, 0.1, capi.KV_Q8G64
+    probe.scale_dtype = capi.SCALE_F32 if extra == "f32scales" else capi.SCALE_F16
+    probe.q_dtype = capi.DTYPE_BF16
+    assert capi.load().zllm_attn_gqa_prefill_workspace_bytes(C.byref(probe)) > 0, "this shape is meant to be split"
+    tol = 2.0 ** -8 if extra == "bf16out" else 0.0
+    for workspace in (True, False):
+        out, want = run_case(77 + d + chunk, prefix, chunk, hq, hkv, workspace=workspace, **kw)
+        got = out.float().cpu().numpy()
+        if tol:
+            assert np.abs(got - want).max() <= 2e-3 + tol * max(1.0, float(np.abs(want).max()))
+        else:
+            assert_attention_close(got, want, f"d={d} prefix={prefix} chunk={chunk} {hq}/{hkv} {extra} workspace={workspace}")
+
+
+def test_prefill_f16_kv_splits():
+    for workspace in (True, False):
+        got, want = run_f16_case(5, 256, 4000, 24, 8, 2, softcap=50.0, q_kind="bf16", workspace=workspace)
+        assert_attention_close(got, want, f"f16 split workspace={workspace}")
+        got, want = run_f16_case(6, 128, 3000, 100, 8, 2, window=600, q_kind="f16", workspace=workspace)
+        assert_attention_close(got, want, f"f16 d=128 split workspace={workspace}")
 
 
 @pytest.mark.parametrize("gate_cols", [8 * 128, 1])
@@ -262,7 +311,7 @@ def test_prefill_head_dim_256_visible_ends_gate_and_bf16_out():
 
 
 def run_f16_case(seed, d, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=16, q_kind="f32", gain=1.0, visible_ends=None,
-                 gate_cols=0, out_dtype=None, scale=None):
+                 gate_cols=0, out_dtype=None, scale=None, workspace=True):
     """A chunk over an f16 cache: rows written by the oracle's f16 append into a pool whose other rows hold f16 NaN, queries
     as f32 / bf16 / f16; returns (device output as f32 numpy, oracle output)."""
     from zllm_amd import capi, ops
@@ -290,7 +339,8 @@ def run_f16_case(seed, d, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_t
     gate = (rng.standard_normal((chunk, gate_cols)) * 3).astype(np.float32) if gate_cols else None
     out = ops.gqa_prefill_chunk(q_dev, upload(planes["k"]), None, upload(planes["v"]), None, upload(tables[0]), prefix, hq, hkv, d, block_tokens,
                                 scale, window=window, softcap=softcap, kv_format=capi.KV_F16, out_dtype=out_dtype,
-                                gate=None if gate is None else upload(gate), visible_ends=None if visible_ends is None else upload(visible_ends))
+                                gate=None if gate is None else upload(gate), visible_ends=None if visible_ends is None else upload(visible_ends),
+                                workspace=workspace)
     torch.cuda.synchronize()
     kd = O.gather_dequant_rows(O.FMT_F16, planes["k"], None, 0, tables[0], block_tokens, 0, total, cols)
     vd = O.gather_dequant_rows(O.FMT_F16, planes["v"], None, 0, tables[0], block_tokens, 0, total, cols)

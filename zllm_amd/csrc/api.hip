@@ -922,6 +922,46 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     return 0;
 }
 
+// KV splits of a chunk kernel launch (zllm::GqaPrefillParams::max_chunks).  A workgroup is one row tile of one KV head
+// walking the tile's whole visible range; a short chunk over a long prefix has few such workgroups, so the range is cut
+// as a decode call's is -- whole rounds of the CUs, splits of at least 256 tokens (a workgroup first loads and
+// normalises a tile of queries) -- and the parts meet in the split merge.  The records are
+// rows x splits x heads x head_dim floats: a plan whose records would pass 256 MiB keeps fewer splits.
+void plan_prefill_splits(const zllm_gqa_prefill_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+{
+    const uint32_t group = a->num_heads / a->num_kv_heads;
+    const uint32_t columns = a->head_dim == 256 ? 128u : 256u; // (row, head-in-group) pairs of a workgroup
+    const uint32_t tile_rows = columns / group > 0 ? columns / group : 1u;
+    const uint64_t tiles = ((uint64_t)a->rows + tile_rows - 1) / tile_rows;
+    uint64_t longest = (uint64_t)a->position + a->rows; // keys the last row tile may see
+    if (a->window != 0 && (uint64_t)a->window + tile_rows + 32 < longest) {
+        longest = (uint64_t)a->window + tile_rows + 32;
+    }
+    plan_splits((uint32_t)longest, tiles * a->num_kv_heads, 1, 256, chunk_tokens, max_chunks);
+    const uint64_t record_bytes = (uint64_t)a->rows * a->num_heads * a->head_dim * 4;
+    const uint64_t most = record_bytes == 0 ? 1 : ((uint64_t)256 << 20) / record_bytes;
+    if (*max_chunks > most) {
+        const uint64_t keep = most < 1 ? 1 : most;
+        const uint64_t chunk = align_up((longest + keep - 1) / keep, 32);
+        *chunk_tokens = (uint32_t)chunk;
+        *max_chunks = (uint32_t)((longest + chunk - 1) / chunk);
+    }
+}
+
+struct PrefillSplitRecords {
+    uint64_t partial, stats, total;
+};
+
+PrefillSplitRecords prefill_split_records(const zllm_gqa_prefill_args* a, uint32_t max_chunks)
+{
+    PrefillSplitRecords w;
+    const uint64_t records = (uint64_t)a->rows * max_chunks * a->num_heads;
+    w.partial = 0;
+    w.stats = align_up(records * a->head_dim * 4, 256);
+    w.total = w.stats + align_up(records * 8, 256);
+    return w;
+}
+
 // Q8g64 caches (scales of any type) and f16 caches run the matrix-core chunk kernels, which keep all of their state on
 // chip (head_dim 64 / 128 / 256, f16: 128 / 256).  What is left runs each row of the chunk as one item of the split-KV
 // decode kernels (row r is a sequence of position + r + 1 tokens over the same block table): more than 128 query heads
@@ -976,8 +1016,13 @@ static void prefill_decode_args(const zllm_gqa_prefill_args* a, zllm_gqa_decode_
 
 uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* a)
 {
-    if (validate_gqa_prefill(a) != 0 || !prefill_rows_as_decode_items(a)) {
-        return 0; /* the chunk kernel keeps all of its state on chip */
+    if (validate_gqa_prefill(a) != 0) {
+        return 0;
+    }
+    if (!prefill_rows_as_decode_items(a)) {
+        uint32_t chunk_tokens, max_chunks;
+        plan_prefill_splits(a, &chunk_tokens, &max_chunks);
+        return max_chunks > 1 ? prefill_split_records(a, max_chunks).total : 0; /* unsplit, the chunk kernel keeps all of its state on chip */
     }
     zllm_gqa_decode_args d;
     prefill_decode_args(a, &d);
@@ -1059,7 +1104,38 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
         p.gate_cols = a->gate_cols;
         p.gate_dtype = a->gate_dtype;
     }
-    return hip_status(zllm::launch_gqa_prefill(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA prefill launch");
+    // KV splits when the chunk has too few row tiles for the device and the caller brought the room for their records
+    uint32_t chunk_tokens = 0, max_chunks = 1;
+    plan_prefill_splits(a, &chunk_tokens, &max_chunks);
+    if (max_chunks > 1) {
+        const PrefillSplitRecords w = prefill_split_records(a, max_chunks);
+        if (a->workspace != nullptr && a->workspace_bytes >= w.total && ((uintptr_t)a->workspace & 15u) == 0) {
+            p.partial = (float*)((char*)a->workspace + w.partial);
+            p.stats = (float*)((char*)a->workspace + w.stats);
+            p.chunk_tokens = chunk_tokens;
+            p.max_chunks = max_chunks;
+        }
+    }
+    const int launched = hip_status(zllm::launch_gqa_prefill(p, a->kv_format, a->scale_dtype, (hipStream_t)stream), "GQA prefill launch");
+    if (launched != 0 || p.max_chunks <= 1) {
+        return launched;
+    }
+    zllm::GqaDecodeParams m;
+    memset(&m, 0, sizeof(m));
+    m.out = (float*)a->out;
+    m.out_dtype = a->out_dtype;
+    m.partial = p.partial;
+    m.stats = p.stats;
+    m.batch = a->rows;
+    m.num_heads = a->num_heads;
+    m.head_dim = a->head_dim;
+    m.chunk_tokens = chunk_tokens;
+    m.max_chunks = max_chunks;
+    m.fixed_chunks = max_chunks;
+    m.gate = p.gate;
+    m.gate_cols = p.gate_cols;
+    m.gate_dtype = p.gate_dtype;
+    return hip_status(zllm::launch_split_merge(m, (hipStream_t)stream), "GQA prefill split merge launch");
 }
 
 } // extern "C"

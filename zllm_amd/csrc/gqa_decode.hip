@@ -1260,16 +1260,19 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     const unsigned int sl = threadIdx.x / quads;
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
-    unsigned int len = p.kv_lens[b];
-    if (p.query_rows > 1u) { // record row b of a multi-row call: its sequence's length less the chunk rows after it
-        const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
-        len = p.kv_lens[b / p.query_rows];
-        len = len > behind ? len - behind : 0u;
+    unsigned int chunks = p.fixed_chunks;
+    if (chunks == 0u) {
+        unsigned int len = p.kv_lens[b];
+        if (p.query_rows > 1u) { // record row b of a multi-row call: its sequence's length less the chunk rows after it
+            const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
+            len = p.kv_lens[b / p.query_rows];
+            len = len > behind ? len - behind : 0u;
+        }
+        unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+        first = min(first, len);
+        const unsigned int first_al = first & ~31u;
+        chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     }
-    unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
-    first = min(first, len);
-    const unsigned int first_al = first & ~31u;
-    const unsigned int chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
     const size_t stat_stride = (size_t)p.num_heads * 2;
     const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;

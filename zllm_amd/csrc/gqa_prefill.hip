@@ -88,6 +88,58 @@ __device__ __forceinline__ unsigned int window_exponent(float top)
     return min(max((__float_as_uint(top) >> 23) & 0xffu, 2u), 252u);
 }
 
+// ---- KV splits of a chunk -------------------------------------------------------------------------------------
+// A chunk with few row tiles (a short chunk over a long prefix) leaves most CUs without a workgroup while each
+// workgroup walks the whole prefix.  With p.max_chunks > 1 workgroup z of a row tile attends part z of the tile's
+// visible range [t_begin, t_end) -- equal 32-aligned parts of at most p.chunk_tokens, as the decode kernels cut a
+// sequence -- and writes un-normalised records (sum of p v, running maximum, sum of p) that gqa_decode_merge combines;
+// parts beyond the tile's own count write empty records (maximum -inf, sum 0).
+struct SplitRange {
+    unsigned int begin, end;
+    bool live;
+};
+__device__ __forceinline__ SplitRange split_range(const GqaPrefillParams& p, unsigned int t_begin, unsigned int t_end)
+{
+    SplitRange r = {t_begin, t_end, true};
+    if (p.max_chunks > 1u) {
+        const unsigned int parts = min(p.max_chunks, (t_end - t_begin + p.chunk_tokens - 1u) / p.chunk_tokens);
+        const unsigned int span = (((t_end - t_begin + parts - 1u) / parts) + 31u) & ~31u;
+        const unsigned long long begin = (unsigned long long)t_begin + (unsigned long long)blockIdx.z * span;
+        r.live = blockIdx.z < parts && begin < t_end;
+        r.begin = r.live ? (unsigned int)begin : t_begin;
+        r.end = r.live ? (unsigned int)min((unsigned long long)t_end, begin + span) : t_begin;
+    }
+    return r;
+}
+
+__device__ __forceinline__ void store_empty_record(const GqaPrefillParams& p, unsigned int row, unsigned int head)
+{
+    const size_t rec = ((size_t)row * p.max_chunks + blockIdx.z) * p.num_heads + head;
+    p.stats[rec * 2] = kNegInf;
+    p.stats[rec * 2 + 1] = 0.0f;
+}
+
+// acc and total carry 2^v_shift (the bias that keeps f16 probabilities in range, less the V window): the records are
+// in true units, so that splits with different windows combine
+template <int DT>
+__device__ __forceinline__ void store_split_record(const GqaPrefillParams& p, unsigned int row, unsigned int head, unsigned int j, float run_max,
+                                                   float total, const f32x4 (&acc)[DT], float v_shift)
+{
+    const size_t rec = ((size_t)row * p.max_chunks + blockIdx.z) * p.num_heads + head;
+    const int down = -(int)v_shift;
+    const float fa = ldexpf(1.0f, down / 2), fb = ldexpf(1.0f, down - down / 2); // two factors: 2^down alone may leave f32's range
+    const bool live = total > 0.0f && total < __builtin_inff();
+    if (j == 0) {
+        p.stats[rec * 2] = live ? run_max : kNegInf;
+        p.stats[rec * 2 + 1] = live ? total * fa * fb : 0.0f;
+    }
+    float* out = p.partial + rec * (size_t)(DT * 16) + 4u * j;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        *(f32x4*)(out + t * 16) = acc[t] * fa * fb;
+    }
+}
+
 // POW2: pages of a power-of-two size behind a block table, known at compile time (no run-time choice of the address
 // arithmetic, no division code in the loop).
 template <int SDT, bool SOFTCAP, bool POW2>
@@ -124,7 +176,18 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         t_begin = first_pos > p.window ? first_pos - p.window : 0u;
     }
     t_begin &= ~31u;
-    const unsigned int steps = (t_end - t_begin + kStep - 1) / kStep;
+    const SplitRange part = split_range(p, t_begin, t_end);
+    if (!part.live) {
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ++ct) {
+            const unsigned int col = wave * (16u * kColTiles) + ct * 16u + m;
+            if (col < cols_used && row0 + col / p.group < p.rows && j == 0) {
+                store_empty_record(p, row0 + col / p.group, kvh * p.group + col % p.group);
+            }
+        }
+        return;
+    }
+    const unsigned int steps = (part.end - part.begin + kStep - 1) / kStep;
 
     // ---- this wave's columns and Q fragments -------------------------------------------------
     // The wave's queries are carried as f16 after a multiplication by one power of two that puts the largest
@@ -477,8 +540,8 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 
     // ---- main loop ------------------------------------------------------------------------------------------
     StepRegs regs;
-    load_step(regs, t_begin, entry_of(t_begin + st_token));
-    unsigned int entry_next = entry_of(t_begin + kStep + st_token);
+    load_step(regs, part.begin, entry_of(part.begin + st_token));
+    unsigned int entry_next = entry_of(part.begin + kStep + st_token);
     store_step(regs, 0);
     __syncthreads();
     unsigned int wv = 2u; // (biased) exponent of the largest V scale up to the tile being attended
@@ -486,7 +549,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     // `buf` is a literal at every call, so the LDS addresses of a step differ from the other buffer's only in the
     // instructions' immediate offsets and cost no address arithmetic
     auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
-        const unsigned int t0 = t_begin + step * kStep;
+        const unsigned int t0 = part.begin + step * kStep;
         // rows past the end of the visible range repeat its last one: the loads stay inside the sequence's pages
         load_step(regs, t0 + kStep, entry_next);
         entry_next = entry_of(t0 + 2u * kStep + st_token);
@@ -523,6 +586,10 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             col_valid[ct] = col < cols_used && col_row[ct] < p.rows;
         }
         if (!col_valid[ct]) {
+            continue;
+        }
+        if (p.max_chunks > 1u) {
+            store_split_record<8>(p, col_row[ct], col_head[ct], j, run_max[ct], total, acc[ct], v_shift);
             continue;
         }
         // accumulators and sum carry the same power of two (2^8 and the V window), which cancels here
@@ -624,7 +691,18 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
         t_begin = first_pos > p.window ? first_pos - p.window : 0u;
     }
     t_begin &= ~31u;
-    const unsigned int steps = (t_end - t_begin + kStep - 1) / kStep;
+    const SplitRange part = split_range(p, t_begin, t_end);
+    if (!part.live) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const unsigned int col = wave * (16u * CT) + ct * 16u + m;
+            if (col < cols_used && row0 + col / p.group < p.rows && j == 0) {
+                store_empty_record(p, row0 + col / p.group, kvh * p.group + col % p.group);
+            }
+        }
+        return;
+    }
+    const unsigned int steps = (part.end - part.begin + kStep - 1) / kStep;
 
     // ---- this wave's columns and Q fragments (power-of-two normalised f16, as in gqa_prefill_q8) ----
     unsigned int col_row[CT], col_head[CT];
@@ -1006,14 +1084,14 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     // ---- main loop: the rows of step n + 1 are loaded while step n computes, and stored before the barrier
     // (requesting them a step earlier still was measured: no change, the loads are not what a step waits for) ----
     StageRegs regs;
-    load_step(regs, t_begin, entry_of(t_begin + st_token));
-    unsigned int entry_next = entry_of(t_begin + kStep + st_token);
+    load_step(regs, part.begin, entry_of(part.begin + st_token));
+    unsigned int entry_next = entry_of(part.begin + kStep + st_token);
     store_step(regs, 0);
     __syncthreads();
     unsigned int wv = 2u; // Q8g64: (biased) exponent of the largest V scale up to the tile being attended
     float v_shift = Q8 ? kPBias + 125.0f : kPBias;
     auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
-        const unsigned int t0 = t_begin + step * kStep;
+        const unsigned int t0 = part.begin + step * kStep;
         load_step(regs, t0 + kStep, entry_next); // past the end of the range the last row repeats: loads stay inside the pages
         entry_next = entry_of(t0 + 2u * kStep + st_token);
         bool window_moved = false;
@@ -1048,6 +1126,10 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
         const unsigned int r = row0 + col / p.group;
         const unsigned int head = kvh * p.group + col % p.group;
         if (!(col < cols_used && r < p.rows)) {
+            continue;
+        }
+        if (p.max_chunks > 1u) {
+            store_split_record<C::kDT>(p, r, head, j, run_max[ct], total, acc[ct], v_shift);
             continue;
         }
         // accumulators and sum carry the same power of two (2^8 and, for Q8g64, the V window), which cancels here
@@ -1087,7 +1169,7 @@ template <int D, int KV, int SDT> static hipError_t launch_prefill_tiles(const G
 {
     const unsigned int cols = TileShape<D>::kCols;
     const unsigned int rows_per_wg = p.group >= cols ? 1u : cols / p.group;
-    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
+    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads, p.max_chunks > 1u ? p.max_chunks : 1u);
     const bool cap = p.softcap > 0.0f;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
     if (cap) {
@@ -1131,7 +1213,7 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
         return launch_prefill_tiles<128, 0, 2>(p, stream);
     }
     const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
-    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads);
+    const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg, p.num_kv_heads, p.max_chunks > 1u ? p.max_chunks : 1u);
     const bool cap = p.softcap > 0.0f;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
     const dim3 block(kThreads);

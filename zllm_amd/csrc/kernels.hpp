@@ -105,6 +105,8 @@ struct GqaDecodeParams {
     // partial kernels: (sequence, split) items a workgroup runs side by side, each with one wave per KV head of its block
     // (0 = 1).  More than one when the KV heads alone would leave the workgroup's waves unused.
     unsigned int items_per_group;
+    // split merge only: every record row has this many splits (0: the count follows from kv_lens and first_visible)
+    unsigned int fixed_chunks;
 };
 
 struct GqaPrefillParams {
@@ -124,6 +126,13 @@ struct GqaPrefillParams {
     unsigned int gate_cols;
     int gate_dtype;
     const unsigned int* visible_ends; // optional [rows]: row r reads up to max(position + r + 1, visible_ends[r])
+    // KV splits of a chunk that has too few row tiles for the CUs: workgroup z of a row tile attends part z of the tile's
+    // visible range (equal 32-aligned parts of at most chunk_tokens) and leaves un-normalised records for the split merge:
+    // partial [rows][max_chunks][num_heads][head_dim], stats [rows][max_chunks][num_heads][2] = (max, sum).  max_chunks <= 1:
+    // no splits, the kernel writes `out` itself.
+    float* partial;
+    float* stats;
+    unsigned int chunk_tokens, max_chunks;
 };
 
 struct MlaDecodeParams {
