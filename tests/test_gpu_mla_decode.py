@@ -414,8 +414,9 @@ def test_mla_prefill_chunk_matches_oracle(heads, lens, rows, block_tokens):
 @pytest.mark.parametrize("rows", [4, 11])
 def test_mla_prefill_chunk_rows_equal_single_row_calls(rows):
     """Row r of a chunk is the decode step of a sequence that ends at that row.  With 8 query rows the call runs the
-    decode kernels: same bits.  With 22 it runs the row-batched absorb (same bits by construction) and merge / projection
-    kernels (several rows per weight load; the splits of a row are folded in another order): equal to 1e-6."""
+    decode kernels: same bits.  With 22 it runs absorb and projection on the matrix cores, sixteen rows a workgroup: the
+    f32 sums run in another order, an absorbed query differs from the single-row one by a bf16 step in a few elements
+    out of a million, and the outputs agree to 5e-4."""
     case = make_mla_chunk_case(77, [600, 90], rows, 32)
     got = run_mla_chunk(case).cpu().numpy()
     for b, l in enumerate(case["lens"]):
@@ -428,7 +429,7 @@ def test_mla_prefill_chunk_rows_equal_single_row_calls(rows):
             if rows == 4:
                 assert np.array_equal(one[0], got[b * rows + r]), (b, r)
             else:
-                assert np.abs(one[0] - got[b * rows + r]).max() <= 1e-6, (b, r)
+                assert np.abs(one[0] - got[b * rows + r]).max() <= 5e-4, (b, r)
 
 
 def test_mla_prefill_chunk_zero_query_is_the_running_mean():

@@ -210,6 +210,105 @@ template <int R> __global__ __launch_bounds__(256) void mla_absorb_rows(MlaDecod
 }
 
 // ---------------------------------------------------------------------------------------------
+// absorb and projection on the matrix cores, for calls of sixteen rows and more
+// ---------------------------------------------------------------------------------------------
+// The per-row kernels keep the oracle's summation order and cost a multiply and an add per weight and row on the vector
+// ALU: 28 us of absorb and 23 us of projection for 32 rows, more than the attention between them at short contexts.
+// With sixteen rows a workgroup the two are small GEMMs, (16 x 128).(128 x 512) and (16 x 512).(512 x 128) per head.
+// Products of bf16 values are exact in f32 and only the order of the f32 sum differs from the oracle's, so an absorbed
+// query differs from the bit-exact one by a bf16 step in a few elements out of a million.
+
+// W_k[head] (nope x 512 bf16) lies in LDS as in memory, rows padded by 16 bytes: the sixteen rows a transposed read
+// touches then start in different banks.
+constexpr int kAbsorbRowBytes = kLatent * 2 + 16;
+constexpr int kAbsorbNope = 128;
+
+// absorbed^T[n, row] = sum_k W_k[k, n] q[row, k].  A operand: W_k^T fragments through ds_read_b64_tr_b16 (lane (m, j) gets
+// column n = 16 nt + m at k = 4 j .. 4 j + 3 and 16 + 4 j .. 16 + 4 j + 3 of a 32-k step); B operand: the query row m at
+// the same k.  grid = (heads, workgroups per head), 256 threads; a workgroup stages the head's weights once and takes
+// blocks of sixteen rows in turn; wave w owns latent columns [128 w, 128 w + 128).
+__global__ __launch_bounds__(256) void mla_absorb_mfma(MlaDecodeParams p)
+{
+    __shared__ __align__(16) unsigned char w_lds[kAbsorbNope * kAbsorbRowBytes];
+    const unsigned int head = blockIdx.x;
+    const unsigned int tid = threadIdx.x;
+    const unsigned int lane = tid & 63u;
+    const unsigned int wave = tid >> 6;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    {
+        const unsigned char* w = (const unsigned char*)(p.kv_b + (size_t)head * p.kv_head_dim * kLatent);
+        u32x4 staged[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const unsigned int c = tid + 256u * i; // 16-byte chunk c % 64 of weight row c / 64
+            staged[i] = *(const u32x4*)(w + (size_t)c * 16u);
+        }
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const unsigned int c = tid + 256u * i;
+            *(u32x4*)(w_lds + (c >> 6) * kAbsorbRowBytes + (c & 63u) * 16u) = staged[i];
+        }
+    }
+    __syncthreads();
+    // the staged weights serve every block of sixteen rows this workgroup takes: blocks blockIdx.y, + gridDim.y, ...
+    const unsigned char* frag_at = w_lds + (4u * j + (m >> 2)) * kAbsorbRowBytes + (m & 3u) * 8u;
+    for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
+    const unsigned int row = min(row0 + m, p.batch - 1u);
+    const size_t q_base = ((size_t)row * p.heads + head) * p.q_head_dim;
+    // four consecutive query elements per load, rounded to bf16: the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
+    auto four_as_bf16 = [&](size_t at) __attribute__((always_inline)) -> u32x2 {
+        if (p.q_dtype == 1) {
+            return *(const u32x2*)((const unsigned short*)p.q + at);
+        }
+        if (p.q_dtype == 0) {
+            const f32x4 x = *(const f32x4*)((const float*)p.q + at);
+            return u32x2{pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])};
+        }
+        const u32x2 h = *(const u32x2*)((const unsigned short*)p.q + at);
+        return u32x2{pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[0] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[0] >> 16))),
+                     pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[1] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[1] >> 16)))};
+    };
+    Frag qf[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const u32x2 lo = four_as_bf16(q_base + ks * 32u + 4u * j), hi = four_as_bf16(q_base + ks * 32u + 16u + 4u * j);
+        qf[ks].u = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    }
+    // the rope part of the sixteen rows is a copy: 16 x 64 elements over 256 threads
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned int e = tid + 256u * i;
+        const unsigned int r = row0 + (e >> 6), c = e & 63u;
+        if (r < p.batch) {
+            const float x = load_as_f32(p.q, ((size_t)r * p.heads + head) * p.q_head_dim + kAbsorbNope + c, p.q_dtype);
+            p.absorbed[((size_t)r * p.heads + head) * (kLatent + kRope) + kLatent + c] = f32_to_bf16_bits(x);
+        }
+    }
+    unsigned short* qa = p.absorbed + ((size_t)(row0 + m) * p.heads + head) * (kLatent + kRope) + 4u * j;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const unsigned int nt = wave * 8u + t;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            union {
+                s16x4 s[2];
+                bf16x8 b;
+            } wf;
+            const unsigned char* at = frag_at + ks * 32 * kAbsorbRowBytes + nt * 32u;
+            wf.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+            wf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kAbsorbRowBytes));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, qf[ks].b, acc, 0, 0, 0);
+        }
+        if (row0 + m < p.batch) { // lane (m, j) holds latent columns 16 nt + 4 j .. + 4 of row m
+            *(u32x2*)(qa + nt * 16u) = u32x2{pack_bf16_rne(acc[0], acc[1]), pack_bf16_rne(acc[2], acc[3])};
+        }
+    }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // 2. split-KV partial
 // ---------------------------------------------------------------------------------------------
 // Workgroup barrier for LDS traffic only.  __syncthreads() also waits for the global loads in flight
@@ -1192,7 +1291,159 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
     }
 }
 
+// The split merge of sixteen rows of one head, then out^T[v, row] = sum_c W_v[v, c] merged[row, c] on the matrix cores:
+// A operand: W_v rows straight from memory (a lane's eight consecutive latent columns are 16 bytes); B operand: the merged
+// rows from LDS as bf16 hi + lo (the merged values are f32: two terms keep 16 bits of them).  value_dim <= 128.
+// grid = (heads, workgroups per head), 512 threads; a workgroup takes blocks of sixteen rows in turn.  The merge is a chain of round trips to memory, so it is spread as wide
+// as the workgroup goes: a thread folds the splits of four latent columns of four rows, the four rows' records requested
+// together, four splits a trip.  Wave w then owns value columns [16 w, 16 w + 16).
+constexpr int kMergedStride = kLatent + 4; // floats: sixteen rows' fragments start in different banks
+__global__ __launch_bounds__(512) void mla_merge_project_mfma(MlaDecodeParams p)
+{
+    __shared__ __align__(16) float merged[16][kMergedStride];
+    const unsigned int head = blockIdx.x;
+    const unsigned int tid = threadIdx.x;
+    const unsigned int quad = tid & 127u;
+    const unsigned int lane = tid & 63u;
+    const unsigned int wave = tid >> 6;
+    const unsigned int m = lane & 15u;
+    const unsigned int j = lane >> 4;
+    // the projection's weights travel under the first merge and serve every block of sixteen rows the workgroup takes
+    const unsigned short* w_head = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent;
+    Frag wf[16];
+    {
+        const unsigned int v = min(wave * 16u + m, p.value_dim - 1u);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+            wf[ks].u = *(const u32x4*)(w_head + (size_t)v * kLatent + ks * 32 + 8u * j);
+        }
+    }
+    for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
+    {
+        const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
+        const float* stats[4];
+        const float* partial[4];
+        unsigned int chunks[4];
+        float mx[4], l[4];
+        f32x4 acc[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+            unsigned int seq;
+            const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
+            chunks[u] = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+            stats[u] = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+            partial[u] = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+            mx[u] = kNegInf;
+            l[u] = 0.0f;
+            acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        const size_t stat_stride = (size_t)p.heads * 2;
+        const size_t partial_stride = (size_t)p.heads * kLatent;
+        const unsigned int most = max(max(chunks[0], chunks[1]), max(chunks[2], chunks[3]));
+        if (p.max_chunks == 1u) { // a long chunk leaves one record a row (no KV splits): nothing to fold
+            float2 st[4];
+            f32x4 part[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                st[u] = *(const float2*)stats[u];
+                part[u] = *(const f32x4*)partial[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (chunks[u] > 0u && st[u].y > 0.0f) {
+                    acc[u] = part[u];
+                    l[u] = st[u].y;
+                }
+            }
+        }
+        for (unsigned int c0 = 0; p.max_chunks > 1u && c0 < most; c0 += 4u) {
+            float2 st[4][4];
+            f32x4 part[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const unsigned int c = min(c0 + v, max(chunks[u], 1u) - 1u);
+                    st[u][v] = *(const float2*)(stats[u] + c * stat_stride);
+                    part[u][v] = *(const f32x4*)(partial[u] + c * partial_stride);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const bool live = c0 + v < chunks[u];
+                    const float cl = live ? st[u][v].y : 0.0f;
+                    if (cl > 0.0f) {
+                        const float cm = st[u][v].x;
+                        const float nm = fmaxf(mx[u], cm);
+                        const float a = __builtin_amdgcn_exp2f(mx[u] - nm);
+                        const float w = __builtin_amdgcn_exp2f(cm - nm);
+                        acc[u] = acc[u] * a + part[u][v] * w;
+                        l[u] = l[u] * a + cl * w;
+                        mx[u] = nm;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            f32x4 result = {0.f, 0.f, 0.f, 0.f};
+            if (l[u] > 0.0f && l[u] < __builtin_inff()) {
+                result = acc[u] * (1.0f / l[u]);
+            }
+            *(f32x4*)(&merged[rb + 4u * u][quad * 4u]) = result;
+        }
+    }
+    __syncthreads();
+    // ---- projection
+    const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
+    f32x4 out_acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 16; ++ks) {
+        const float* x = &merged[m][ks * 32 + 8u * j];
+        const f32x4 x0 = *(const f32x4*)x, x1 = *(const f32x4*)(x + 4);
+        Frag hi, lo;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float a0 = x0[2 * e], a1 = x0[2 * e + 1], b0 = x1[2 * e], b1 = x1[2 * e + 1];
+            hi.u[e] = pack_bf16_rne(a0, a1);
+            hi.u[2 + e] = pack_bf16_rne(b0, b1);
+            lo.u[e] = pack_bf16_rne(a0 - __uint_as_float(hi.u[e] << 16), a1 - __uint_as_float(hi.u[e] & 0xffff0000u));
+            lo.u[2 + e] = pack_bf16_rne(b0 - __uint_as_float(hi.u[2 + e] << 16), b1 - __uint_as_float(hi.u[2 + e] & 0xffff0000u));
+        }
+        out_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].b, hi.b, out_acc, 0, 0, 0);
+        out_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].b, lo.b, out_acc, 0, 0, 0);
+    }
+    if (row0 + m < p.batch) { // lane (m, j) holds value columns 16 wave + 4 j .. + 4 of row m
+        const size_t base = ((size_t)(row0 + m) * p.heads + head) * out_stride;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const unsigned int v = wave * 16u + 4u * j + r;
+            if (v < p.value_dim) {
+                if (p.out_dtype == 0) {
+                    ((float*)p.out)[base + v] = out_acc[r];
+                } else {
+                    ((unsigned short*)p.out)[base + v] = f32_to_bf16_bits(out_acc[r]);
+                }
+            }
+        }
+    }
+    __syncthreads(); // the next block's merge overwrites the rows just read
+    }
+}
+
 } // namespace
+
+// Workgroups per head of the matrix-core absorb and projection: every workgroup loads its head's weights once, so a long
+// chunk is covered by about 1,024 workgroups in all, each taking several blocks of sixteen rows.
+static unsigned int row_block_groups(const MlaDecodeParams& p)
+{
+    const unsigned int blocks = (p.batch + 15u) / 16u;
+    const unsigned int per_head = (1024u + p.heads - 1u) / p.heads;
+    return blocks < per_head ? blocks : per_head;
+}
 
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
 {
@@ -1201,7 +1452,9 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     if (stages & 1u) {
         // Eight rows per workgroup share every weight load, and the workgroup then runs eight rows' sums: measured 28 us from
         // 16 rows up to a few hundred, against 13 us (15 rows) to 27 us (32 rows) for one workgroup per row
-        if (p.batch >= 32u && p.nope_dim <= 256u) {
+        if (p.batch >= 16u && p.nope_dim == (unsigned int)kAbsorbNope && (p.q_head_dim & 3u) == 0) { // sixteen rows a workgroup, on the matrix cores
+            mla_absorb_mfma<<<dim3(p.heads, row_block_groups(p)), dim3(256), 0, stream>>>(p);
+        } else if (p.batch >= 32u && p.nope_dim <= 256u) {
             mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
         } else {
             mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
@@ -1231,7 +1484,9 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if ((stages & 12u) == 12u) {
-        if (p.batch >= 16u) { // a prefill chunk: eight rows share every weight load of the projection
+        if (p.batch >= 16u && p.value_dim <= 128u) { // sixteen rows a workgroup, the projection on the matrix cores
+            mla_merge_project_mfma<<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+        } else if (p.batch >= 16u) { // eight rows share every weight load of the projection
             mla_merge_project_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
         } else {
             mla_merge_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
