@@ -384,10 +384,14 @@ def oracle_mla_chunk(case, selection=None):
     return np.concatenate(outs_f), np.concatenate(outs_b)
 
 
-def run_mla_chunk(case, out_dtype=None, selection=None, compact=True):
+def run_mla_chunk(case, out_dtype=None, selection=None, compact=True, q_kind="bf16"):
     from zllm_amd import ops
 
-    out = ops.mla_decode(to_torch_bf16(case["q_bits"], "cuda"), upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]),
+    q = to_torch_bf16(case["q_bits"], "cuda")
+    if q_kind != "bf16":  # the same bf16-representable values carried as f32 or f16 (f16 holds them after a second rounding)
+        q = upload(O.bf16_to_f32(case["q_bits"]))
+        q = q.to(torch.float16) if q_kind == "f16" else q
+    out = ops.mla_decode(q, upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]),
                          upload(case["rope"]), upload(case["tables"]), upload(case["lens"]), case["heads"],
                          case["nope"] + case["rope_dim"], case["nope"] + case["value"], case["latent"], case["rope_dim"],
                          case["block_tokens"], int(case["lens"].max()), out_dtype=out_dtype or torch.float32, out_compact=compact,
@@ -409,6 +413,30 @@ def test_mla_prefill_chunk_matches_oracle(heads, lens, rows, block_tokens):
     diff = np.abs(O.bf16_to_f32(got_b).astype(np.float64) - O.bf16_to_f32(want_b))
     step = np.maximum(np.abs(O.bf16_to_f32(want_b)), 2.0 ** -126) * 2.0 ** -7
     assert (diff <= step + 2e-3).all()
+
+
+def test_mla_batched_decode_on_the_matrix_core_stages():
+    """A decode batch of sixteen rows and more takes the matrix-core absorb and projection (one query row per sequence
+    here; chunks take them through test_mla_prefill_chunk_matches_oracle): 40 ragged sequences, strided and compact
+    output, and the query as bf16 and as f32 (one block of sixteen rows is partly empty: 40 = 2.5 blocks)."""
+    rng = np.random.default_rng(41)
+    lens = [int(x) for x in rng.integers(1, 900, size=40)]
+    case = make_mla_case(41, lens, 32)
+    want_f, want_b = oracle_mla(case)
+    got = run_mla(case).cpu().numpy()
+    print("mla batch 40", assert_attention_close(got.reshape(want_f.shape), want_f, "MLA batch of 40"))
+    got32 = run_mla(case, q_f32=True).cpu().numpy()
+    assert np.array_equal(got, got32)  # the f32 query holds bf16-representable values
+    strided = run_mla(case, compact=False).cpu().numpy().reshape(40, 32, 192)[:, :, :128]
+    assert np.array_equal(strided.reshape(got.shape), got)
+
+
+def test_mla_chunk_query_types_on_the_matrix_core_absorb():
+    case = make_mla_chunk_case(9, [300, 120], 20, 16)
+    want_f, _ = oracle_mla_chunk(case)
+    for q_kind in ("bf16", "f32"):
+        got = run_mla_chunk(case, q_kind=q_kind).cpu().numpy()
+        assert_attention_close(got, want_f, f"MLA chunk q as {q_kind}")
 
 
 @pytest.mark.parametrize("rows", [4, 11])
