@@ -1313,10 +1313,17 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
             }
         }
     };
-    // the first trip runs whatever the split count is; a sequence with many splits (few KV heads: several items share a
-    // workgroup and the splits are short) then takes eight records per trip, a trip being one round trip to memory
-    fold(sl, std::integral_constant<int, 4>{});
-    for (unsigned int c0 = sl + 4u * lanes; c0 < chunks; c0 += 8u * lanes) {
+    // the first trip runs whatever the split count is (its loads do not wait for the length); a trip is one round trip
+    // to memory, so a plan with many short splits (few KV heads, short contexts) takes eight records per trip from the start
+    unsigned int next = sl;
+    if (p.max_chunks > 4u * lanes) {
+        fold(next, std::integral_constant<int, 8>{});
+        next += 8u * lanes;
+    } else {
+        fold(next, std::integral_constant<int, 4>{});
+        next += 4u * lanes;
+    }
+    for (unsigned int c0 = next; c0 < chunks; c0 += 8u * lanes) {
         fold(c0, std::integral_constant<int, 8>{});
     }
     __shared__ float sm[256];
