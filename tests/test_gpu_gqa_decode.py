@@ -270,6 +270,8 @@ def test_few_kv_heads_share_a_workgroup(fmt, hq, hkv, d, window):
         case = make_gqa_q8_case(900 + hq + d, lens, hq, hkv, d, outliers=True)
         got = run_decode(case, 0.09, window=window)
         want = oracle_gqa_decode(case, 0.09, window=window)
+        hinted = run_decode(case, 0.09, window=window, total_kv_tokens=sum(lens))  # the ragged plan counts the shared workgroups too
+        assert_attention_close(hinted, want, f"{fmt} {hq}/{hkv} d={d} window={window} with the token-count hint")
     else:
         case = make_f16_case(900 + hq + d, lens, hq, hkv, d)
         got = run_f16(case, 0.09, window=window)
