@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration", "mfma_issue_calibration"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration", "mfma_issue_calibration", "append_prologue"])
     ap.add_argument("--pool-gib", type=float, default=256.0, help="address span of the paged pool (all four planes); clipped to 90 %% of free HBM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -375,6 +375,71 @@ def run_gqa_decode(args, ragged, config1=False):
     print(json.dumps(record))
 
 
+def run_append_prologue(args):
+    """The steps in front of the attention call on every chunk of a prefill: the quantizing page appends and the fused
+    prologue (per-head RMSNorm + RoPE, Q out, K/V into the pages), at chunk sizes, as bytes moved per second.  `value` is
+    the prologue of a 2,048-row chunk (64 query / 8 KV heads, head_dim 128, bf16 in, bf16 Q out)."""
+    import torch
+
+    from zllm_amd import capi, ops
+
+    ops.init(0)
+    rng = np.random.default_rng(args.seed)
+    dev = "cuda"
+    bt = 16
+    results = {}
+    launches = max(10, min(args.steps, 50))
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        settle_clocks(fn, 0.05)
+        return event_time_ms(fn, launches)
+
+    for rows in (2048, 8192):
+        cols = 1024
+        pool = (rows + bt - 1) // bt * 2 + 64
+        table = torch.from_numpy(rng.choice(pool, size=(rows + bt - 1) // bt + 1, replace=False).astype(np.int32)).to(dev)
+        codes = torch.zeros((pool * bt, cols), dtype=torch.int8, device=dev)
+        scales = torch.zeros((pool * bt, cols // 64), dtype=torch.int16, device=dev)
+        src = torch.randn((rows, cols), device=dev).to(torch.bfloat16)
+        ms = timed(lambda: ops.q8g64_append(src, codes, scales, table, 0, bt, capi.QUANT_METAL_GQA))
+        moved = rows * cols * 2 + rows * cols + rows * cols // 64 * 2
+        results[f"q8g64_append_{rows}_rows_bf16"] = {"ms": round(ms, 5), "bytes": moved, "gbps": round(moved / ms / 1e6, 1)}
+        cache = torch.zeros((pool * bt, cols), dtype=torch.float16, device=dev)
+        ms = timed(lambda: ops.half_append(src, cache, table, 0, bt))
+        moved = rows * cols * 4
+        results[f"half_append_{rows}_rows_bf16"] = {"ms": round(ms, 5), "bytes": moved, "gbps": round(moved / ms / 1e6, 1)}
+        latent = torch.randn((rows, 512), device=dev).to(torch.bfloat16)
+        k_rope = torch.randn((rows, 64), device=dev).to(torch.bfloat16)
+        pool64 = (rows + 63) // 64 * 2 + 8
+        table64 = torch.from_numpy(rng.choice(pool64, size=(rows + 63) // 64 + 1, replace=False).astype(np.int32)).to(dev)
+        lc = torch.zeros((pool64 * 64, 512), dtype=torch.int8, device=dev)
+        ls = torch.zeros((pool64 * 64, 8), dtype=torch.int16, device=dev)
+        rc = torch.zeros((pool64 * 64, 64), dtype=torch.int16, device=dev)
+        latent_f32, rope_f32 = latent.float(), k_rope.float()
+        ms = timed(lambda: ops.mla_append(latent_f32, rope_f32, lc, ls, rc, table64, 0, 64))
+        moved = rows * (576 * 4 + 512 + 16 + 128)
+        results[f"mla_append_{rows}_rows_f32"] = {"ms": round(ms, 5), "bytes": moved, "gbps": round(moved / ms / 1e6, 1)}
+        hq, hkv, d = 64, 8, 128
+        q = torch.randn((rows, hq * d), device=dev).to(torch.bfloat16)
+        k = torch.randn((rows, hkv * d), device=dev).to(torch.bfloat16)
+        v = torch.randn((rows, hkv * d), device=dev).to(torch.bfloat16)
+        qn, kn = torch.ones(d, device=dev), torch.ones(d, device=dev)
+        cos, sin = torch.ones((rows + 8, d // 2), device=dev), torch.zeros((rows + 8, d // 2), device=dev)
+        v_codes, v_scales = torch.zeros_like(codes), torch.zeros_like(scales)
+        ms = timed(lambda: ops.gqa_prologue(q, k, v, qn, kn, cos, sin, codes, scales, v_codes, v_scales, table, 0, hq, hkv, d, d, bt,
+                                            q_out_dtype=torch.bfloat16))
+        moved = rows * (hq * d * 2 * 2 + 2 * hkv * d * 2 + 2 * hkv * d + 2 * (hkv * d // 64) * 2 + d * 4)
+        results[f"gqa_prologue_{rows}_rows_bf16"] = {"ms": round(ms, 5), "bytes": moved, "gbps": round(moved / ms / 1e6, 1)}
+    head = results["gqa_prologue_2048_rows_bf16"]
+    print(json.dumps({"metric": "pre-attention prologue of a 2,048-row chunk, bytes moved per second", "value": head["gbps"], "unit": "GB/s",
+                      "n_gpus": 1, "steps": launches, "warmup": 3, "ms_per_step": head["ms"], "higher_is_better": True, "dtype": "f32",
+                      "data": "synthetic", "config": {"workload": "page appends and fused prologue at chunk sizes", **results},
+                      "roofline": {"bound": "hbm", "kernel": "gqa_prologue_kernel", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                   "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None}}))
+
+
 def run_copy_calibration(args):
     """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters of the
     attention kernels are scaled by (the counters do not report bytes one-to-one on this GPU)."""
@@ -464,6 +529,8 @@ def main():
         run_gqa_decode(args, ragged=False, config1=True)
     elif args.workload == "copy_calibration":
         run_copy_calibration(args)
+    elif args.workload == "append_prologue":
+        run_append_prologue(args)
     elif args.workload == "mfma_issue_calibration":
         run_mfma_issue_calibration(args)
     elif args.workload == "read_calibration":
