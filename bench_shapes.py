@@ -137,7 +137,7 @@ def main():
 
     ops.init(0)
     if args.suite in ("gqa_decode", "all"):
-        gqa_decode_cases(args, [(64, 8, 128)], [(8, 32768), (12, 32768), (5, 65536), (16, 65536), (24, 2048), (3, 8192)])
+        gqa_decode_cases(args, [(64, 8, 128)], [(8, 32768), (12, 32768), (5, 65536), (16, 65536), (24, 2048), (3, 8192), (128, 1024), (512, 2048)])
     if args.suite in ("gqa_heads", "all"):
         gqa_decode_cases(args, [(32, 4, 128), (16, 2, 128), (8, 1, 128), (8, 1, 64), (4, 1, 256)], [(8, 32768), (32, 8192)])
     if args.suite in ("prefill_chunks", "all"):

@@ -1371,6 +1371,82 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     }
 }
 
+// The same combine for plans of at most eight splits (large batches, short contexts): a thread owns four output
+// dimensions of one (head, sequence) and folds the few records itself, 256 / (head_dim / 4) heads a workgroup.  One
+// workgroup of 256 threads per (head, sequence) is mostly idle lanes there, and with hundreds of sequences the launch
+// of tens of thousands of them costs more than the combine (512 sequences x 64 heads, two splits: 37 us, 10 us here).
+__global__ __launch_bounds__(256) void gqa_decode_merge_few(GqaDecodeParams p)
+{
+    const unsigned int quads = p.head_dim / 4u;
+    const unsigned int heads_here = 256u / quads;
+    const unsigned int quad = threadIdx.x % quads;
+    const unsigned int head = blockIdx.x * heads_here + threadIdx.x / quads;
+    const unsigned int b = blockIdx.y;
+    if (head >= p.num_heads) {
+        return;
+    }
+    unsigned int chunks = p.fixed_chunks;
+    if (chunks == 0u) {
+        unsigned int len = p.kv_lens[b];
+        if (p.query_rows > 1u) {
+            const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
+            len = p.kv_lens[b / p.query_rows];
+            len = len > behind ? len - behind : 0u;
+        }
+        unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+        first = min(first, len);
+        const unsigned int first_al = first & ~31u;
+        chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+    }
+    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    const size_t stat_stride = (size_t)p.num_heads * 2;
+    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;
+    const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
+    float m = kNegInf, l = 0.0f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned int c0 = 0; c0 == 0u || c0 < chunks; c0 += 4u) { // the first trip's loads do not wait for the length
+        float2 st[4];
+        f32x4 part[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned int c = min(c0 + u, p.max_chunks - 1u);
+            st[u] = *(const float2*)(stats + c * stat_stride);
+            part[u] = *(const f32x4*)(partial + c * partial_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float cl = c0 + u < chunks ? st[u].y : 0.0f;
+            if (cl > 0.0f) {
+                const float nm = fmaxf(m, st[u].x);
+                const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+                const float w = __builtin_amdgcn_exp2f(st[u].x - nm);
+                acc = acc * a + part[u] * w;
+                l = l * a + cl * w;
+                m = nm;
+            }
+        }
+    }
+    f32x4 result = {0.f, 0.f, 0.f, 0.f};
+    if (l > 0.0f && l < __builtin_inff()) {
+        result = acc * (1.0f / l);
+    }
+    if (p.gate != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            result[e] = gated(result[e], p.gate, p.gate_cols, p.gate_dtype, b, head * p.head_dim + quad * 4u + e);
+        }
+    }
+    const size_t at = ((size_t)b * p.num_heads + head) * p.head_dim + quad * 4u;
+    if (p.out_dtype == 0) {
+        *(f32x4*)(p.out + at) = result;
+    } else if (p.out_dtype == 1) {
+        *(u32x2*)((unsigned short*)p.out + at) = u32x2{pack_bf16_rne(result[0], result[1]), pack_bf16_rne(result[2], result[3])};
+    } else {
+        *(u32x2*)((unsigned short*)p.out + at) = u32x2{(unsigned int)f32_to_f16_bits(result[0]) | ((unsigned int)f32_to_f16_bits(result[1]) << 16),
+                                                        (unsigned int)f32_to_f16_bits(result[2]) | ((unsigned int)f32_to_f16_bits(result[3]) << 16)};
+    }
+}
+
 // Visible ranges of the rows of a prefill chunk, for the route that runs every row as one item of the split-KV
 // decode kernels: lens[r] = end and first[r] = start of key_range(position + r, position + rows), or of
 // key_range_with_visible_end when the row carries an explicit end (src/attention/gqa.rs:54-68).
@@ -1508,7 +1584,13 @@ hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, co
 
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)
 {
-    gqa_decode_merge<<<dim3(p.num_heads, p.batch), dim3(256), 0, stream>>>(p);
+    const unsigned int quads = p.head_dim / 4u;
+    if (p.max_chunks <= 8u && quads <= 256u && 256u % quads == 0u) {
+        const unsigned int heads_here = 256u / quads;
+        gqa_decode_merge_few<<<dim3((p.num_heads + heads_here - 1u) / heads_here, p.batch), dim3(256), 0, stream>>>(p);
+    } else {
+        gqa_decode_merge<<<dim3(p.num_heads, p.batch), dim3(256), 0, stream>>>(p);
+    }
     return hipGetLastError();
 }
 
