@@ -251,8 +251,10 @@ typedef struct zllm_gqa_decode_args {
     uint32_t max_kv_len;           /* host upper bound of kv_lens: sizes the grid and the split plan.  A call
                                       recorded into a HIP graph stays valid only while every kv_lens[b] on the
                                       device is <= max_kv_len; tokens past the planned splits are not read */
-    uint32_t total_kv_tokens;      /* optional host hint: sum of the visible lengths (0 = unknown,
-                                      batch * max_kv_len is assumed); only tunes the split size */
+    uint32_t total_kv_tokens;      /* host hint: sum of the visible lengths (0 = unknown, batch * max_kv_len is
+                                      assumed); only tunes the split size.  Pass it for batches of unequal lengths
+                                      and for sliding windows: planned as if every sequence were max_kv_len long,
+                                      a long sequence among short ones (or a short window) gets few workgroups */
     uint32_t block_tokens;
     uint32_t ring_capacity;        /* 0 or sliding-window ring rows (token % capacity) */
     float score_scale;             /* > 0 */
