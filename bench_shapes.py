@@ -126,6 +126,27 @@ def mla_batch_cases(args):
             flops = batch * ctx * heads * (2 * 576 + 2 * 512)
             print(json.dumps({"suite": "mla_batches", "batch": batch, "heads": heads, "ctx": ctx, "stage_us": stage,
                               "call_tflops": round(flops / stage["call"] / 1e6, 1)}), flush=True)
+    # one long sequence among short ones, with and without the token-count hint
+    batch, lens_host = 32, [65536] + [2048] * 31
+    need = sum(l // bt for l in lens_host)
+    ids = rng.choice(pool, size=need, replace=False).astype(np.uint32)
+    tables_host = np.zeros((batch, 65536 // bt), dtype=np.uint32)
+    at = 0
+    for b, l in enumerate(lens_host):
+        tables_host[b, : l // bt] = ids[at: at + l // bt]
+        at += l // bt
+    tables = torch.from_numpy(tables_host.view(np.int32)).to("cuda")
+    q = torch.randn((batch, heads * (nope + rope)), generator=gen, device="cuda").to(torch.bfloat16)
+    lens = torch.tensor(lens_host, dtype=torch.int32, device="cuda")
+    for label, hint in (("without_hint", 0), ("with_hint", sum(lens_host))):
+        call, out, ws = ops.mla_decode_args(q, kv_b, codes, scales, rope_cache, tables, lens, heads, nope + rope, nope + value, latent, rope, bt,
+                                            65536, total_ctx_tokens=hint)
+
+        def whole():
+            capi.check(lib.zllm_attn_mla_decode(C.byref(call), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+        print(json.dumps({"suite": "mla_batches", "batch": batch, "ctx": "65536 + 31 x 2048", "plan": label, "call_us": round(_time_us(whole, launches=10), 1),
+                          "workspace_mb": round(ws.numel() / 1e6, 1)}), flush=True)
 
 
 def main():

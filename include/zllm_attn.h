@@ -460,6 +460,10 @@ typedef struct zllm_mla_decode_args {
      * a selection holds one list per query row.  The reference returns bf16 for T > 1
      * (src/backend/rocm/attention.rs:17-19): pass out_dtype = ZLLM_DTYPE_BF16 for that.  batch * T <= 65535. */
     uint32_t query_rows;
+    /* Host hint for batches of unequal lengths: the sum of ctx_lens over the sequences (0 = unknown, every sequence is
+     * planned as max_ctx_len long, and a long sequence among short ones gets few workgroups).  Only tunes the split
+     * size; the split records grow with max_ctx_len / split size, which zllm_attn_mla_decode_workspace_bytes reports. */
+    uint32_t total_ctx_tokens;
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
 ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);

@@ -66,7 +66,7 @@ def oracle_mla(case, head_subset=None, selection=None, counts=None):
     return np.stack(outs_f), np.stack(outs_b)
 
 
-def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, selection=None, counts=None):
+def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, selection=None, counts=None, total_ctx_tokens=0):
     from zllm_amd import ops
 
     out_dtype = out_dtype or torch.float32
@@ -76,7 +76,7 @@ def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, s
                          case["nope"] + case["value"], case["latent"], case["rope_dim"], case["block_tokens"],
                          max_ctx_len or int(case["lens"].max()), out_dtype=out_dtype, out_compact=compact,
                          selection=None if selection is None else upload(selection),
-                         selection_counts=None if counts is None else upload(counts))
+                         selection_counts=None if counts is None else upload(counts), total_ctx_tokens=total_ctx_tokens)
     torch.cuda.synchronize()
     return out
 
@@ -413,6 +413,28 @@ def test_mla_prefill_chunk_matches_oracle(heads, lens, rows, block_tokens):
     diff = np.abs(O.bf16_to_f32(got_b).astype(np.float64) - O.bf16_to_f32(want_b))
     step = np.maximum(np.abs(O.bf16_to_f32(want_b)), 2.0 ** -126) * 2.0 ** -7
     assert (diff <= step + 2e-3).all()
+
+
+def test_mla_ragged_batch_with_the_token_count_hint():
+    """One long sequence among short ones: with the sum of the lengths as a hint the plan cuts short splits (the long
+    sequence then has many workgroups), without it every sequence is planned as the longest.  Same results either way."""
+    from zllm_amd import capi
+    import ctypes as C
+
+    lens = [4000, 100, 64, 700, 33, 1]
+    case = make_mla_case(57, lens, 32)
+    want_f, _ = oracle_mla(case)
+    plain = run_mla(case).cpu().numpy()
+    hinted = run_mla(case, total_ctx_tokens=sum(lens)).cpu().numpy()
+    assert_attention_close(plain.reshape(want_f.shape), want_f, "MLA ragged batch")
+    assert_attention_close(hinted.reshape(want_f.shape), want_f, "MLA ragged batch with the hint")
+    args = capi.MlaDecodeArgs()
+    args.batch, args.heads, args.q_head_dim, args.kv_head_dim, args.latent_dim, args.rope_dim = len(lens), 32, 192, 256, 512, 64
+    args.block_tokens, args.max_ctx_len, args.q_dtype, args.out_dtype, args.out_compact = 16, max(lens), capi.DTYPE_BF16, capi.DTYPE_F32, 1
+    lib = capi.load()
+    unhinted_bytes = lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args))
+    args.total_ctx_tokens = sum(lens)
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args)) > unhinted_bytes  # more, shorter splits
 
 
 def test_mla_batched_decode_on_the_matrix_core_stages():

@@ -273,7 +273,26 @@ void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    plan_splits(longest, (uint64_t)a->batch * mla_query_rows(a) * head_blocks, 1, 64, chunk_tokens, max_chunks);
+    const uint64_t per_sequence = (uint64_t)mla_query_rows(a) * head_blocks; // workgroups per split of a sequence
+    const uint64_t uniform_total = (uint64_t)a->batch * a->max_ctx_len;
+    if (a->selection == nullptr && a->total_ctx_tokens != 0 && a->total_ctx_tokens < uniform_total &&
+        kComputeUnits > 2 * a->batch * per_sequence) {
+        // ragged batch, as in plan_gqa_decode: sum_b ceil(len_b / chunk) <= total / chunk + batch.  The records are
+        // [row][max_chunks][head][512] floats: a plan whose records would pass 512 MiB keeps longer splits.
+        const uint64_t slots = kComputeUnits / per_sequence - a->batch;
+        uint64_t chunk = (a->total_ctx_tokens + slots - 1) / slots;
+        chunk = align_up(chunk < 64 ? 64 : chunk, 32);
+        const uint64_t record_bytes = (uint64_t)a->batch * mla_query_rows(a) * a->heads * a->latent_dim * 4;
+        const uint64_t most = ((uint64_t)512 << 20) / record_bytes;
+        const uint64_t fewest_tokens = align_up(((uint64_t)longest + (most < 1 ? 1 : most) - 1) / (most < 1 ? 1 : most), 32);
+        if (chunk < fewest_tokens) {
+            chunk = fewest_tokens;
+        }
+        *chunk_tokens = (uint32_t)chunk;
+        *max_chunks = (uint32_t)(((uint64_t)longest + chunk - 1) / chunk);
+        return;
+    }
+    plan_splits(longest, (uint64_t)a->batch * per_sequence, 1, 64, chunk_tokens, max_chunks);
 }
 
 struct MlaWorkspace {
