@@ -163,6 +163,8 @@ def test_split_plan_covers_the_host_bound_and_sizes_the_workspace(lib):
         assert chunk.value * chunks.value >= args.max_kv_len
         assert chunk.value * (chunks.value - 1) < args.max_kv_len  # no split lies wholly beyond the bound
         records = args.batch * chunks.value * args.num_heads
+        if args.total_kv_tokens:  # a ragged plan never asks for more than 512 MiB of records (plus one split's rounding)
+            assert records * args.head_dim * 4 <= (512 << 20) + args.batch * args.num_heads * args.head_dim * 4
         align = lambda n: (n + 255) // 256 * 256
         assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) == align(records * args.head_dim * 4) + align(records * 8)
     bad = capi.GqaDecodeArgs()

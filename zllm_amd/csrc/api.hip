@@ -211,6 +211,14 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
         const uint64_t slots = (uint64_t)kComputeUnits * items_per_group / (kvh_blocks * head_blocks) - a->batch;
         uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
         chunk = align_up(chunk < kMinGqaChunk ? kMinGqaChunk : chunk, 32);
+        // the records are [sequence][max_chunks][head][head_dim] floats: a plan whose records would pass 512 MiB (one very
+        // long sequence among many short ones) keeps longer splits
+        const uint64_t record_bytes = (uint64_t)a->batch * a->num_heads * a->head_dim * 4;
+        const uint64_t most = ((uint64_t)512 << 20) / record_bytes;
+        const uint64_t fewest_tokens = align_up(((uint64_t)a->max_kv_len + (most < 1 ? 1 : most) - 1) / (most < 1 ? 1 : most), 32);
+        if (chunk < fewest_tokens) {
+            chunk = fewest_tokens;
+        }
         *chunk_tokens = (uint32_t)chunk;
         *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
     } else {
