@@ -1,0 +1,159 @@
+"""Seeded random parity sweeps: every case draws its shape, page size, window, soft cap, scale rule, query type and
+magnitudes from one generator seeded by (sweep, case number), runs the HIP path through the C-ABI and compares with the
+CPU oracle at the tolerance of the fixed cases.  The fixed cases in the other GPU test modules cover the shapes the
+reference tests name; these cover combinations nobody thought to write down (odd group sizes, a window of one token over
+a 48-token page, a 2^-8 value gain with a per-head gate, ...)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from tests.cases import assert_attention_close, make_gqa_q8_case, oracle_gqa_decode
+from tests.test_gpu_gqa_decode import run_decode
+from tests.test_gpu_gqa_prefill import run_case, run_f16_case
+from tests.test_gpu_mla_decode import (draw_selection, make_mla_case, make_mla_chunk_case, oracle_mla, oracle_mla_chunk, run_mla,
+                                       run_mla_chunk)
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+LENGTHS = [0, 1, 15, 16, 17, 31, 32, 33, 64, 100, 255, 256, 257, 700, 1024, 2049, 4100]
+MLA_LENGTHS = [1, 2, 31, 32, 33, 63, 64, 65, 95, 96, 97, 255, 256, 257, 511, 513, 700, 1023, 1025, 2047, 2049, 3000]
+PAGE_SIZES = [1, 4, 16, 16, 64, 48]
+
+
+def pick(rng, values):
+    return values[int(rng.integers(0, len(values)))]
+
+
+def block_ends(rng, prefix, chunk, max_block, keep):
+    """Visible ends in blocks of a random size; about one row in `keep` sees nothing (end 0)."""
+    block = int(rng.integers(1, max_block))
+    return np.array([min(prefix + chunk, prefix + ((r // block) + 1) * block) if rng.integers(0, keep) else 0 for r in range(chunk)],
+                    dtype=np.uint32)
+
+
+def close_at_scale(got, want, what, extra=0.0):
+    """The tolerance applies to outputs of order one: outputs grow with the value gain, so divide by the largest."""
+    want = np.asarray(want, dtype=np.float64)
+    top = max(1.0, float(np.abs(want).max()))
+    return assert_attention_close(np.asarray(got, dtype=np.float64) / top, want / top, what, atol=2e-3 + extra)
+
+
+@pytest.mark.parametrize("it", range(40))
+def test_random_q8_decode(it):
+    rng = np.random.default_rng([101, it])
+    hkv = pick(rng, [1, 2, 4, 8])
+    group = pick(rng, [1, 2, 3, 4, 8, 16])
+    d = pick(rng, [64, 128, 128, 256])
+    lens = [pick(rng, LENGTHS) for _ in range(int(rng.integers(1, 6)))]
+    if max(lens) == 0:
+        lens[0] = 5
+    window = pick(rng, [0, 0, 1, 33, 128, 1024])
+    softcap = pick(rng, [0.0, 0.0, 30.0])
+    what = f"decode {it}: {hkv * group}/{hkv} d={d} lens={lens} window={window} softcap={softcap}"
+    print(what, flush=True)
+    case = make_gqa_q8_case(2000 + it, lens, hkv * group, hkv, d, outliers=bool(it % 2), q_bf16=bool(it % 3 == 0))
+    got = run_decode(case, 0.09, window=window, softcap=softcap)
+    assert_attention_close(got, oracle_gqa_decode(case, 0.09, window=window, softcap=softcap), what)
+
+
+@pytest.mark.parametrize("it", range(48))
+def test_random_q8_prefill_chunk(it):
+    """All three head sizes, the three scale-storage rules, visible ends, gates, K and V gains over 2^-8..2^8."""
+    rng = np.random.default_rng([202, it])
+    d = pick(rng, [64, 128, 128, 256])
+    hkv = pick(rng, [1, 2, 4, 8])
+    hq = hkv * pick(rng, [1, 2, 3, 4, 8, 16])
+    prefix = int(rng.integers(0, 2500))
+    chunk = int(rng.integers(1, 260))
+    window = pick(rng, [0, 0, 0, 1, 33, 200, 1000])
+    softcap = pick(rng, [0.0, 0.0, 30.0, 50.0])
+    bt = pick(rng, PAGE_SIZES)
+    rule = pick(rng, [O.RULE_METAL_GQA, O.RULE_ROCM_MLA, O.RULE_CUDA_GQA])
+    q_bf16 = True if d == 256 else bool(rng.integers(0, 2))
+    scale = pick(rng, [1 / np.sqrt(d), 0.3])
+    v_gain = float(2.0 ** rng.integers(-8, 9))
+    k_gain = float(2.0 ** rng.integers(-3, 4))
+    ends = block_ends(rng, prefix, chunk, 60, 3) if rng.integers(0, 3) == 0 else None
+    gate_cols = pick(rng, [0, 0, 1, hq * d])
+    # f32 queries run row by row through the decode kernels, which need their split records, except at head_dim 128 with
+    # 16-bit scales; every other case may run without a workspace (the unsplit chunk kernel)
+    workspace = bool(rng.integers(0, 4)) or not (q_bf16 or (d == 128 and rule != O.RULE_CUDA_GQA))
+    what = (f"prefill {it}: d={d} {hq}/{hkv} prefix={prefix} chunk={chunk} window={window} softcap={softcap} page={bt} rule={rule} "
+            f"q_bf16={q_bf16} scale={scale:.3f} v_gain={v_gain} k_gain={k_gain} ends={ends is not None} gate_cols={gate_cols} "
+            f"workspace={workspace}")
+    print(what, flush=True)
+    out, want = run_case(7000 + it, prefix, chunk, hq, hkv, window=window, softcap=softcap, block_tokens=bt, rule=rule, q_bf16=q_bf16,
+                         scale=scale / k_gain, outliers=bool(rng.integers(0, 2)), v_gain=v_gain, k_gain=k_gain, d=d, visible_ends=ends,
+                         gate_cols=gate_cols, workspace=workspace)
+    got = out.cpu().numpy().astype(np.float64)
+    want = want.astype(np.float64)
+    top = max(1.0, float(np.abs(want).max())) if v_gain >= 1 else max(1e-30, float(np.abs(want).max()))
+    assert_attention_close(got / top, want / top, what)
+
+
+@pytest.mark.parametrize("it", range(30))
+def test_random_f16_prefill_chunk(it):
+    rng = np.random.default_rng([303, it])
+    d = pick(rng, [128, 256])
+    hkv = pick(rng, [1, 2, 4, 8])
+    hq = hkv * pick(rng, [1, 2, 3, 4, 8, 16])
+    prefix = int(rng.integers(0, 2200))
+    chunk = int(rng.integers(1, 300))
+    window = pick(rng, [0, 0, 1, 40, 700, 1024])
+    softcap = pick(rng, [0.0, 0.0, 50.0, 20.0])
+    bt = pick(rng, PAGE_SIZES)
+    q_kind = pick(rng, ["f32", "bf16", "f16"])
+    gain = float(2.0 ** rng.integers(-3, 4))
+    scale = pick(rng, [1.0 / np.sqrt(d), 0.2])
+    ends = block_ends(rng, prefix, chunk, 70, 4) if rng.integers(0, 3) == 0 else None
+    gate_cols = pick(rng, [0, 0, 1, hq * d])
+    out_dtype = pick(rng, [torch.float32, torch.bfloat16, torch.float16])
+    workspace = bool(rng.integers(0, 4)) or q_kind == "f32"  # f32 queries over an f16 cache need the decode kernels' records
+    what = (f"f16 prefill {it}: d={d} {hq}/{hkv} prefix={prefix} chunk={chunk} window={window} softcap={softcap} page={bt} q={q_kind} "
+            f"gain={gain} ends={ends is not None} gate_cols={gate_cols} out={out_dtype} workspace={workspace}")
+    print(what, flush=True)
+    got, want = run_f16_case(4000 + it, d, prefix, chunk, hq, hkv, window=window, softcap=softcap, block_tokens=bt, q_kind=q_kind, gain=gain,
+                             visible_ends=ends, gate_cols=gate_cols, out_dtype=out_dtype, scale=scale, workspace=workspace)
+    # a 16-bit output rounds once more: half an ulp of the largest output
+    extra = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[out_dtype]
+    close_at_scale(got, want.reshape(got.shape), what, extra)
+
+
+@pytest.mark.parametrize("it", range(45))
+def test_random_mla_decode(it):
+    rng = np.random.default_rng([404, it])
+    heads = pick(rng, [1, 3, 16, 20, 40, 64, 65, 128])
+    bt = pick(rng, [1, 16, 32, 48, 64, 128])
+    batch = pick(rng, [1, 2, 3, 4, 4, 17, 33])  # 16 rows and more take the matrix-core absorb and projection
+    lens = [pick(rng, MLA_LENGTHS) for _ in range(batch)]
+    if heads >= 64 or batch > 4:
+        lens = [min(l, 700) for l in lens]
+    if heads >= 64 and batch > 4:
+        lens = [min(l, 257) for l in lens]
+    selection = None
+    if it % 3 == 0:
+        selection = draw_selection(rng, lens, pick(rng, [1, 7, 32, 100, 300]), bool(it % 2))
+    hint = sum(lens) if (selection is None and rng.integers(0, 2)) else 0
+    what = f"mla {it}: heads={heads} page={bt} lens={lens} top_k={None if selection is None else selection.shape[1]} hint={hint}"
+    print(what, flush=True)
+    case = make_mla_case(1000 + it, lens, heads, block_tokens=bt, poison=bool(it % 2))
+    want, _ = oracle_mla(case, selection=selection)
+    got = run_mla(case, selection=selection, total_ctx_tokens=hint).cpu().numpy()
+    assert_attention_close(got.reshape(want.shape), want, what)
+
+
+@pytest.mark.parametrize("it", range(14))
+def test_random_mla_chunk(it):
+    rng = np.random.default_rng([505, it])
+    heads = pick(rng, [8, 16, 20, 64, 128])
+    rows = pick(rng, [2, 3, 8, 17, 40])
+    lens = [int(rng.integers(rows, 1500)) for _ in range(int(rng.integers(1, 4)))]
+    bt = pick(rng, [16, 64, 48, 1])
+    q_kind = pick(rng, ["bf16", "bf16", "f32"])
+    what = f"mla chunk {it}: heads={heads} lens={lens} rows={rows} page={bt} q={q_kind}"
+    print(what, flush=True)
+    case = make_mla_chunk_case(4000 + it, lens, rows, heads, block_tokens=bt)
+    want, _ = oracle_mla_chunk(case)
+    got = run_mla_chunk(case, q_kind=q_kind).cpu().numpy()
+    assert_attention_close(got.reshape(want.shape), want, what)
