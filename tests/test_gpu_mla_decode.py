@@ -437,6 +437,20 @@ def test_mla_ragged_batch_with_the_token_count_hint():
     assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args)) > unhinted_bytes  # more, shorter splits
 
 
+@pytest.mark.parametrize("heads,lens", [(16, [20000]), (32, [9000, 70]), (64, [17000]), (32, [8300, 8200])])
+def test_mla_few_rows_of_many_splits_take_the_wide_merge(heads, lens):
+    """One or two sequences of few heads are cut into a split per compute unit, 128 or 256 records per (row, head): the
+    merge then runs as eight workgroups per pair, without the sequence lengths (a short sequence beside a long one has
+    records that say "empty"), and the projection as a kernel of its own.  f32 and bf16 output."""
+    case = make_mla_case(91 + heads, lens, heads, block_tokens=64)
+    want_f, want_b = oracle_mla(case)
+    got = run_mla(case).cpu().numpy()
+    print("mla wide merge", heads, lens, assert_attention_close(got.reshape(want_f.shape), want_f, f"MLA heads={heads} lens={lens}"))
+    got_b = run_mla(case, out_dtype=torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    diff = np.abs(O.bf16_to_f32(got_b).astype(np.float64).reshape(want_f.shape) - O.bf16_to_f32(want_b).reshape(want_f.shape))
+    assert (diff <= np.maximum(np.abs(want_f), 2.0 ** -126) * 2.0 ** -7 + 2e-3).all()
+
+
 def test_mla_batched_decode_on_the_matrix_core_stages():
     """A decode batch of sixteen rows and more takes the matrix-core absorb and projection (one query row per sequence
     here; chunks take them through test_mla_prefill_chunk_matches_oracle): 40 ragged sequences, strided and compact

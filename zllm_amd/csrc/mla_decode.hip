@@ -80,17 +80,20 @@ __device__ __forceinline__ unsigned int visible_tokens(const unsigned int* ctx_l
 // ---------------------------------------------------------------------------------------------
 // 1. absorb
 // ---------------------------------------------------------------------------------------------
-// grid = (heads, batch), 256 threads, thread c owns latent columns 2 c and 2 c + 1.
+// grid = (heads, batch, 4), one wave; a thread owns two adjacent latent columns, a workgroup every fourth run of 64
+// column pairs (with the usual 512 columns: one run).  A decode call of one sequence has as many (row, head) pairs as
+// heads, so the weights of a head are fetched by four compute units instead of one: 128 load instructions a wave
+// instead of 512 a compute unit.
 // The sum runs over k in ascending order with separately rounded multiply and add, the order of
 // the reference's scalar matmul (src/kernel/cpu/mla.rs:712-728); the result is rounded to bf16
 // (mla.rs:1037).
-__global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
+__global__ __launch_bounds__(64) void mla_absorb(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
     __shared__ float q_sh[1024];
     const size_t q_base = ((size_t)b * p.heads + head) * p.q_head_dim;
-    for (unsigned int i = threadIdx.x; i < p.q_head_dim; i += 256) {
+    for (unsigned int i = threadIdx.x; i < p.q_head_dim; i += 64) {
         float x = load_as_f32(p.q, q_base + i, p.q_dtype);
         // the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
         q_sh[i] = bf16_bits_to_f32(f32_to_bf16_bits(x));
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
     if (pairs == 256u && p.nope_dim == 128u) {
         // the usual geometry (latent 512, nope 128): all 128 weight words of the thread are requested at once, before the
         // query has even arrived in LDS -- the kernel is one memory round trip long instead of four
-        const unsigned int c2 = threadIdx.x;
+        const unsigned int c2 = blockIdx.z * 64u + threadIdx.x;
         unsigned int word[128];
 #pragma unroll
         for (int k = 0; k < 128; ++k) {
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
         }
     } else {
         __syncthreads();
-        for (unsigned int c2 = threadIdx.x; c2 < pairs; c2 += 256) {
+        for (unsigned int c2 = blockIdx.z * 64u + threadIdx.x; c2 < pairs; c2 += 256) {
             // product and sum rounded separately, as in the CPU code (plain operators: the __fmul_rn / __fadd_rn intrinsics
             // are ordinary operators from a header compiled with fusing allowed)
 #pragma clang fp contract(off)
@@ -145,8 +148,10 @@ __global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
             *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
         }
     }
-    for (unsigned int r = threadIdx.x; r < p.rope_dim; r += 256) {
-        qa[p.latent_dim + r] = f32_to_bf16_bits(q_sh[p.nope_dim + r]);
+    if (blockIdx.z == 0u) {
+        for (unsigned int r = threadIdx.x; r < p.rope_dim; r += 64) {
+            qa[p.latent_dim + r] = f32_to_bf16_bits(q_sh[p.nope_dim + r]);
+        }
     }
 }
 
@@ -987,7 +992,8 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
 // fetch one whole 128-byte line of its weight row per load instruction (with 64 consecutive columns per slice every
 // instruction touched 64 different lines: measured, the projection took 12 us of a 16 us kernel).  The lane keeps its
 // 64 weighted values in registers and the eight slices are summed with DPP row shifts.
-__device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned int head, unsigned int b, const float (&x)[64])
+__device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned int head, unsigned int b, const float (&x)[64],
+                                             unsigned int v_begin, unsigned int v_end)
 {
     const unsigned int lane = threadIdx.x & 63u;
     const unsigned int wave = threadIdx.x >> 6;
@@ -996,7 +1002,7 @@ __device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned 
     const unsigned short* w = p.kv_b + ((size_t)head * p.kv_head_dim + p.nope_dim) * kLatent + slice * 8u;
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     const size_t out_base = ((size_t)b * p.heads + head) * out_stride;
-    for (unsigned int v0 = wave * 8u; v0 < p.value_dim; v0 += 32u) {
+    for (unsigned int v0 = v_begin + wave * 8u; v0 < v_end; v0 += 32u) {
         const unsigned int v = v0 + sub;
         const unsigned int vr = min(v, p.value_dim - 1u);
         u32x4 raw[8];
@@ -1027,7 +1033,8 @@ __device__ __forceinline__ void project_head(const MlaDecodeParams& p, unsigned 
     }
 }
 
-// grid = (heads, batch): projection of the merged rows in the workspace (stage run on its own)
+// grid = (heads, batch, value_dim / 32 rounded up): projection of the merged rows in the workspace, 32 value columns a
+// workgroup -- one pass of project_head, so the kernel is one round trip to memory long (merged row and weights together)
 __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
@@ -1042,7 +1049,7 @@ __global__ __launch_bounds__(256) void mla_project(MlaDecodeParams p)
         x[4 * i + 2] = t[2];
         x[4 * i + 3] = t[3];
     }
-    project_head(p, head, b, x);
+    project_head(p, head, b, x, blockIdx.z * 32u, min(p.value_dim, blockIdx.z * 32u + 32u));
 }
 
 // grid = (heads, batch): split merge and projection in one kernel when both stages run.  The merge is the
@@ -1162,7 +1169,7 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
         x[4 * i + 3] = t[3];
     }
     if (!wide) {
-        project_head(p, head, b, x);
+        project_head(p, head, b, x, 0u, p.value_dim);
         return;
     }
     // same arithmetic and order as project_head, on the weights fetched at the start
@@ -1190,6 +1197,91 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
                 ((unsigned short*)p.out)[out_base + v] = f32_to_bf16_bits(sum);
             }
         }
+    }
+}
+
+// The split merge on its own for a call of few rows with many splits each (one sequence of 32 K tokens is cut into 256
+// splits, one per compute unit): a workgroup per (row, head) folds them in eight dependent round trips, on as many
+// compute units as the call has heads.  Here eight workgroups share a (row, head), each taking a run of 64 latent columns:
+// 256 threads = 16 split lanes x 16 column quads fold sixteen records per lane and trip (256 splits: one round trip, and
+// no wait for the sequence length first: every split of the plan has a record, whose sum says whether it holds
+// anything); the lanes of a quad meet through lane exchanges and LDS.  The merged row goes to the workspace and
+// mla_project reads it from there.  (One kernel for both, the eight runs' products summed by the workgroup that arrives
+// last, was built: the release fence before the arrival counter writes back a level-two cache full of split records, and
+// the kernel took 23 us where the two launches take 10.)  grid = (heads, rows, 8).
+constexpr int kWideParts = 8;
+__global__ __launch_bounds__(256) void mla_merge_wide(MlaDecodeParams p)
+{
+    const unsigned int head = blockIdx.x;
+    const unsigned int b = blockIdx.y;
+    const unsigned int tid = threadIdx.x;
+    const unsigned int quad = tid & 15u;
+    const unsigned int sl = tid >> 4;
+    const unsigned int column = blockIdx.z * 64u + quad * 4u;
+    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+    const size_t stat_stride = (size_t)p.heads * 2;
+    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + column;
+    const size_t partial_stride = (size_t)p.heads * kLatent;
+    float m = kNegInf, l = 0.0f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned int c0 = sl; c0 < p.max_chunks; c0 += 256u) {
+        float cm[16], cl[16];
+        f32x4 part[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const unsigned int c = min(c0 + 16u * u, p.max_chunks - 1u);
+            const bool live = c0 + 16u * u < p.max_chunks;
+            const float2 st = *(const float2*)(stats + c * stat_stride);
+            cm[u] = live ? st.x : kNegInf;
+            cl[u] = live ? st.y : 0.0f;
+            part[u] = *(const f32x4*)(partial + c * partial_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            if (cl[u] > 0.0f) {
+                const float nm = fmaxf(m, cm[u]);
+                const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+                const float w = __builtin_amdgcn_exp2f(cm[u] - nm);
+                acc = acc * a + part[u] * w;
+                l = l * a + cl[u] * w;
+                m = nm;
+            }
+        }
+    }
+    // two partial merges into one; a side that holds nothing has l = 0
+    auto fold = [](float& m, float& l, f32x4& acc, float om, float ol, const f32x4& oacc) __attribute__((always_inline)) {
+        const float nm = fmaxf(l > 0.0f ? m : kNegInf, ol > 0.0f ? om : kNegInf);
+        const float a = l > 0.0f ? __builtin_amdgcn_exp2f(m - nm) : 0.0f;
+        const float w = ol > 0.0f ? __builtin_amdgcn_exp2f(om - nm) : 0.0f;
+        acc = acc * a + oacc * w;
+        l = l * a + ol * w;
+        m = nm;
+    };
+    // the four split lanes of a wave (lanes 16 and 32 apart), then the four waves
+#pragma unroll
+    for (int step = 16; step <= 32; step *= 2) {
+        const float om = __shfl_xor(m, step), ol = __shfl_xor(l, step);
+        const f32x4 oacc = {__shfl_xor(acc[0], step), __shfl_xor(acc[1], step), __shfl_xor(acc[2], step), __shfl_xor(acc[3], step)};
+        fold(m, l, acc, om, ol, oacc);
+    }
+    __shared__ float wave_m[4][16], wave_l[4][16];
+    __shared__ f32x4 wave_acc[4][16];
+    if ((tid & 63u) < 16u) {
+        wave_m[tid >> 6][quad] = m;
+        wave_l[tid >> 6][quad] = l;
+        wave_acc[tid >> 6][quad] = acc;
+    }
+    __syncthreads();
+    if (tid < 16u) {
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            fold(m, l, acc, wave_m[w][quad], wave_l[w][quad], wave_acc[w][quad]);
+        }
+        f32x4 result = {0.f, 0.f, 0.f, 0.f};
+        if (l > 0.0f && l < __builtin_inff()) {
+            result = acc * (1.0f / l);
+        }
+        *(f32x4*)(p.weighted + ((size_t)b * p.heads + head) * kLatent + column) = result;
     }
 }
 
@@ -1446,6 +1538,18 @@ static unsigned int row_block_groups(const MlaDecodeParams& p)
     return blocks < per_head ? blocks : per_head;
 }
 
+// One workgroup per (row, head) folds 32 split records a round trip; the wide merge and the separate projection cost a
+// launch more and read any number of splits in one.  Measured (merge and projection together): one row of 32 heads with 256
+// splits 19.4 -> 8.1 us, of 64 heads 21.1 -> 11.3; two rows of 32 heads with 128 splits 11.8 -> 8.1; one row of 128 heads
+// with 128 splits 13.5 -> 14.7 (no gain: 1,024 workgroups for the merge).
+static bool wide_merge_pays(const MlaDecodeParams& p)
+{
+    if (p.latent_dim != (unsigned int)kLatent) {
+        return false;
+    }
+    return p.max_chunks > 128u || (p.max_chunks > 64u && p.heads * p.batch <= 64u);
+}
+
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
 {
     const unsigned int stages = stage_mask == 0 ? 15u : stage_mask;
@@ -1458,7 +1562,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         } else if (p.batch >= 32u && p.nope_dim <= 256u) {
             mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
         } else {
-            mla_absorb<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+            mla_absorb<<<dim3(p.heads, p.batch, 4), dim3(64), 0, stream>>>(p);
         }
         err = hipGetLastError();
         if (err != hipSuccess) {
@@ -1489,6 +1593,14 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
             mla_merge_project_mfma<<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
         } else if (p.batch >= 16u) { // eight rows share every weight load of the projection
             mla_merge_project_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
+        } else if (wide_merge_pays(p)) {
+            // few rows, each cut into many splits: the merge by eight workgroups per (row, head), then the projection
+            mla_merge_wide<<<dim3(p.heads, p.batch, kWideParts), dim3(256), 0, stream>>>(p);
+            err = hipGetLastError();
+            if (err != hipSuccess) {
+                return err;
+            }
+            mla_project<<<dim3(p.heads, p.batch, (p.value_dim + 31u) / 32u), dim3(256), 0, stream>>>(p);
         } else {
             mla_merge_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
         }
@@ -1514,7 +1626,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if (stages & 8u) {
-        mla_project<<<dim3(p.heads, p.batch), dim3(256), 0, stream>>>(p);
+        mla_project<<<dim3(p.heads, p.batch, (p.value_dim + 31u) / 32u), dim3(256), 0, stream>>>(p);
         err = hipGetLastError();
     }
     return err;
