@@ -22,6 +22,7 @@
 //   3. split merge by log-sum-exp (shared with GQA decode)
 //   4. mla_project: out[b, h, v] = weighted[b, h, :] . W_kv_b[h, nope + v, :]
 #include <string.h>
+#include <type_traits>
 
 #include "common.hpp"
 #include "kernels.hpp"
@@ -365,7 +366,7 @@ constexpr int kPShift = 4;
 // masks and softmax are over slots -- and only the address of a row goes through the list.
 // POW2: the page size is a power of two and the sequences have block tables, known at compile time: the address
 // arithmetic of a step is then shifts and masks without the run-time choice (and the division code behind it).
-template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
+template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> __global__ __launch_bounds__(512) void mla_partial_ws(MlaDecodeParams p)
 {
     static_assert(!(ALIGNED && SELECTED), "selected rows are not contiguous");
     // Staging items (token row, 16 codes) per thread: the 32 rows of a step are split 24 : 8 between the score and the
@@ -379,7 +380,9 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                                                       // of consecutive lanes are contiguous (conflict-free 16-byte reads)
     __shared__ __align__(16) _Float16 lds_scale16[kWsTiles][8][kStepTokens]; // [buffer][group][token]: scale / 2^(window + kPShift)
     __shared__ int lds_win[kWsTiles];                    // the window lds_scale16[buffer] was written for
-    __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]
+    __shared__ __align__(16) float lds_alpha[2][4][64];  // [parity][head tile][lane]; narrow: [parity][2 head tile + token half][lane],
+                                                         // the running maximum the half's probabilities are relative to
+    __shared__ float2 lds_final[2][16];                  // narrow: [head tile][head]: (maximum, sum) of the second token half
     __shared__ __align__(16) float lds_top[kWsTiles][4]; // [buffer][value wave]: largest group scale the wave converted
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -389,7 +392,12 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     const unsigned int chunk = blockIdx.x;
-    const unsigned int head = blockIdx.y * 64u + hw * 16u + m; // this lane's head column
+    // NARROW (a call of at most 32 heads: head tiles 2 and 3 would be empty): the four score waves are two head tiles x
+    // two halves of a step's tokens, each half with its own running maximum and sum, and every value wave takes both
+    // head tiles and a quarter of the columns.
+    const unsigned int score_tile = NARROW ? (hw & 1u) : hw; // head tile of a score wave
+    const unsigned int stream = NARROW ? (hw >> 1) : 0u;     // narrow: which sixteen tokens of a step it scores
+    const unsigned int head = blockIdx.y * 64u + score_tile * 16u + m; // this lane's head column
     const unsigned int b = blockIdx.z; // query row of the call (= sequence when every sequence has one row)
     unsigned int seq;
     unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq); // keys of this row: positions, or list slots when a selection applies
@@ -668,6 +676,8 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                 }
             }
         }
+        // narrow: a head tile past the last head stages and converts like the others and scores nothing
+        const bool tile_live = !NARROW || (unsigned int)__builtin_amdgcn_readfirstlane((int)(score_tile * 16u)) < p.heads;
         float run_max = kNegInf, run_sum = 0.0f;
         float neg_ref = 0.0f; // minus the reference the scores are taken against: the running maximum, 0 before the first score
         float neg_ref_shifted = (float)kPShift; // the same plus the hand-over shift: the scores below are log2(p * 2^kPShift)
@@ -675,6 +685,112 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
         const float latent_log2 = scale_log2 * head_pow2;
         stage_step(1u);
         for (unsigned int i = 0; i <= steps; ++i) {
+            if constexpr (NARROW) {
+                if (i < steps && tile_live) {
+                    // sixteen tokens of the step: four batches of four k-steps (latent groups {0..3} first k-step, {0..3} second,
+                    // {4..7} first, {4..7} second; the rope k-steps ride along with batch 0), fragments requested two batches ahead
+                    const unsigned int tb = i % kWsTiles;
+                    const unsigned char* tile = lds + tb * kTileBytes + stream * (16u * kRowBytes);
+                    const float (*scale_tile)[kStepTokens] = lds_scale[tb];
+                    const unsigned int t0 = c_start + i * kStepTokens + 16u * stream;
+                    constexpr int kRing = 3, kAhead = kRing - 1;
+                    Frag kf[kRing][4], kr[2];
+                    f32x4 gsv[2][4];
+                    auto load_batch = [&](int q) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            kf[q % kRing][u].u = *(const u32x4*)(tile + qk_base[q & 1] + ((q >> 1) * 4 + u) * 128);
+                        }
+                        if (q == 0) {
+                            kr[0].u = *(const u32x4*)(tile + qk_base[0] + 8 * 128);
+                            kr[1].u = *(const u32x4*)(tile + qk_base[1] + 8 * 128);
+                        }
+                        if (q & 1) {
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                gsv[q >> 1][u] = *(const f32x4*)(&scale_tile[(q >> 1) * 4 + u][16u * stream + 4 * j]);
+                            }
+                        }
+                    };
+#pragma unroll
+                    for (int q = 0; q < kAhead; ++q) {
+                        load_batch(q);
+                    }
+                    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 s_rope = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 d[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (q + kAhead < 4) {
+                            load_batch(q + kAhead);
+                        }
+                        asm volatile("" ::: "memory"); // the requests above stay above the MFMAs below
+                        if (q == 0) {
+                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[0].b, qf[16].b, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                            s_rope = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kr[1].b, qf[17].b, s_rope, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int g = (q >> 1) * 4 + u;
+                            if ((q & 1) == 0) {
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[q % kRing][u].h, qf[2 * g].h, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                            } else {
+                                d[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[q % kRing][u].h, qf[2 * g + 1].h, d[u], 0, 0, 0);
+                            }
+                        }
+                        if (q & 1) {
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                const f32x4 gs = gsv[q >> 1][u];
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) {
+                                    s[r] = fmaf(d[u][r], gs[r], s[r]);
+                                }
+                            }
+                        }
+                    }
+                    float sc[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        sc[r] = fmaf(s[r], latent_log2, fmaf(s_rope[r], scale_log2, neg_ref_shifted)); // relative to the reference
+                    }
+                    if (t0 + 16u > len) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            sc[r] = t0 + 4u * j + r < len ? sc[r] : kNegInf;
+                        }
+                    }
+                    // the lazy online softmax of the wide layout; the reference moves to whole numbers, so that the value
+                    // waves bring the two token halves of a head to one reference with exact powers of two
+                    const float lane_max = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+                    if (__any(lane_max > 8.0f + (float)kPShift || run_max == kNegInf)) {
+                        const float step_max = wave_max_16x4(lane_max) - (float)kPShift;
+                        const float ref = -neg_ref;
+                        float new_max = run_max;
+                        if (step_max > 8.0f || run_max == kNegInf) {
+                            new_max = fmaxf(run_max, ceilf(ref + step_max));
+                        }
+                        const float safe_max = new_max == kNegInf ? 0.0f : new_max;
+                        const float delta = safe_max - ref;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            sc[r] -= delta;
+                        }
+                        run_sum *= __builtin_amdgcn_exp2f(run_max - safe_max); // 0 on the first step: nothing accumulated yet
+                        run_max = new_max;
+                        neg_ref = -safe_max;
+                        neg_ref_shifted = neg_ref + (float)kPShift;
+                    }
+                    float pr[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        pr[r] = __builtin_amdgcn_exp2f(sc[r]);
+                    }
+                    run_sum += (pr[0] + pr[1]) + (pr[2] + pr[3]); // in units of 2^-kPShift, like the probabilities
+                    ((u32x2*)&lds_p16[i & 1u][score_tile][lane])[stream] = u32x2{pack_f16_hw(pr[0], pr[1]), pack_f16_hw(pr[2], pr[3])};
+                    lds_alpha[i & 1u][2u * score_tile + stream][lane] = run_max; // -inf: nothing seen yet, the probabilities are zeros
+                }
+            } else
             if (i < steps) {
                 const unsigned int tb = i % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes;
@@ -807,7 +923,27 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             lds_barrier();
         }
         const float total = wave_sum_16x4(run_sum) * (1.0f / (float)(1 << kPShift));
-        if (head < p.heads && j == 0) {
+        if constexpr (NARROW) {
+            // the two token halves of a head become one record: the larger reference (the one the value waves ended on) and
+            // both sums brought to it
+            if (stream == 1u && j == 0u) {
+                lds_final[score_tile][m] = float2{run_max, total};
+            }
+            lds_barrier();
+            if (stream == 0u && head < p.heads && j == 0u) {
+                const float2 other = lds_final[score_tile][m];
+                const float common = fmaxf(run_max, other.x);
+                float sum = 0.0f;
+                if (run_max != kNegInf) {
+                    sum += total * __builtin_amdgcn_exp2f(run_max - common);
+                }
+                if (other.x != kNegInf) {
+                    sum += other.y * __builtin_amdgcn_exp2f(other.x - common);
+                }
+                p.stats[rec * 2] = common;
+                p.stats[rec * 2 + 1] = sum;
+            }
+        } else if (head < p.heads && j == 0) {
             p.stats[rec * 2] = run_max;
             p.stats[rec * 2 + 1] = total;
         }
@@ -816,13 +952,17 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
         // Value wave v = 2 hp + dh owns head tiles 2 hp and 2 hp + 1 and output columns [256 dh, 256 dh + 256):
         // every V^T fragment it reads from LDS feeds two MFMAs (one per head tile), which halves the LDS traffic
         // of this stage and doubles the matrix work behind each LDS round trip.
-        const unsigned int hp = hw >> 1;
-        const unsigned int dh = hw & 1u;
-        f32x4 acc[2][16];
+        // NARROW: every value wave takes head tiles 0 and 1 and a quarter of the columns, [128 v, 128 v + 128).
+        constexpr int GROUPS = NARROW ? 2 : 4; // 64-column scale groups of this wave
+        const unsigned int hp = NARROW ? 0u : hw >> 1;
+        const unsigned int part = NARROW ? hw : hw & 1u; // the wave's run of 64 * GROUPS columns
+        // narrow: sixteen heads or fewer leave the second head tile empty; it is neither rescaled nor multiplied
+        const bool second_tile = !NARROW || __builtin_amdgcn_readfirstlane((int)(p.heads > 16u)) != 0;
+        f32x4 acc[2][GROUPS * 4];
 #pragma unroll
         for (int ht = 0; ht < 2; ++ht) {
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
+            for (int t = 0; t < GROUPS * 4; ++t) {
                 acc[ht][t] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
@@ -837,6 +977,11 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             const f32x4 tops = *(const f32x4*)lds_top[0];
             window = window_for(__builtin_amdgcn_readfirstlane(__float_as_uint(fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3])))));
         }
+        typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+        auto pk_mul = [](unsigned int x, unsigned int y) __attribute__((always_inline)) -> unsigned int {
+            return __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2_t, x) * __builtin_bit_cast(f16x2_t, y));
+        };
+        float common[2] = {kNegInf, kNegInf}; // narrow: the reference a head's accumulators are relative to
         unsigned int value_tile = 0; // buffer of tile i - 1
         stage_step(1u);
         const unsigned int lds_base = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)lds;
@@ -844,15 +989,43 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             // the hand-over records are requested first: their LDS round trip hides behind the staging work
             u32x4 p16[2];
             float alpha[2];
+            float half_ref[2][2];
 #pragma unroll
             for (int ht = 0; ht < 2; ++ht) {
                 p16[ht] = lds_p16[(i + 1u) & 1u][2u * hp + ht][lane];
-                alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
+                if constexpr (NARROW) {
+                    half_ref[ht][0] = lds_alpha[(i + 1u) & 1u][2 * ht][lane];
+                    half_ref[ht][1] = lds_alpha[(i + 1u) & 1u][2 * ht + 1][lane];
+                    alpha[ht] = 1.0f;
+                } else {
+                    alpha[ht] = lds_alpha[(i + 1u) & 1u][2u * hp + ht][lane];
+                }
             }
             const f32x4 tops = *(const f32x4*)lds_top[value_tile]; // tile i - 1
             const unsigned int top_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(fmaxf(fmaxf(tops[0], tops[1]), fmaxf(tops[2], tops[3]))));
             const int table_window = __builtin_amdgcn_readfirstlane(lds_win[value_tile]);
             asm volatile("" ::: "memory");
+            if constexpr (NARROW) {
+                if (i > 0) {
+                    // The two token halves of a head were scored against references of their own (whole numbers, or -inf
+                    // while a half has seen nothing).  The accumulators follow the larger one: they are rescaled when it
+                    // moves, and each half's probabilities are brought to it by an exact power of two (0 for -inf).
+#pragma unroll
+                    for (int ht = 0; ht < 2; ++ht) {
+                        const float ra = half_ref[ht][0], rb = half_ref[ht][1];
+                        const float to = fmaxf(common[ht], fmaxf(ra, rb));
+                        alpha[ht] = to == common[ht] ? 1.0f : __builtin_amdgcn_exp2f(common[ht] - to);
+                        common[ht] = to;
+                        const float fa = ra == kNegInf ? 0.0f : __builtin_amdgcn_exp2f(ra - to);
+                        const float fb = rb == kNegInf ? 0.0f : __builtin_amdgcn_exp2f(rb - to);
+                        const unsigned int fa2 = pack_f16_hw(fa, fa), fb2 = pack_f16_hw(fb, fb);
+                        p16[ht][0] = pk_mul(p16[ht][0], fa2);
+                        p16[ht][1] = pk_mul(p16[ht][1], fa2);
+                        p16[ht][2] = pk_mul(p16[ht][2], fb2);
+                        p16[ht][3] = pk_mul(p16[ht][3], fb2);
+                    }
+                }
+            }
             if (i > 0) {
                 // the window moves before this iteration's conversion, so that the table written now is written for it
                 const int need = window_for(top_bits);
@@ -868,14 +1041,16 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
             convert_to(i + 1u);
             stage_step(i + 2u);
             __builtin_amdgcn_s_setprio(0);
-            if (i > 0) {
+            // O^T += V^T . P' of tile i - 1 for the first HT head tiles of the pair
+            auto accumulate = [&](auto tiles) __attribute__((always_inline)) {
+                constexpr int HT = decltype(tiles)::value;
                 // LDS byte addresses of this step: one register per fragment row, everything else is an immediate
-                const unsigned int tile_lds = lds_base + value_tile * kTileBytes + dh * 4u * 128u; // this wave's four scale groups
+                const unsigned int tile_lds = lds_base + value_tile * kTileBytes + part * (GROUPS * 128u); // this wave's scale groups
 #pragma unroll
-                for (int ht = 0; ht < 2; ++ht) {
+                for (int ht = 0; ht < HT; ++ht) {
                     if (__any(alpha[ht] != 1.0f)) {
 #pragma unroll
-                        for (int t = 0; t < 16; ++t) {
+                        for (int t = 0; t < GROUPS * 4; ++t) {
                             acc[ht][t] *= alpha[ht];
                         }
                     }
@@ -888,7 +1063,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                     f16x8 h;
                 };
                 // The transposed reads are written as inline assembly with immediate offsets: one address register per
-                // fragment row serves all four groups, and the waits are placed by hand (lgkmcnt, LDS operations
+                // fragment row serves all of the wave's groups, and the waits are placed by hand (lgkmcnt, LDS operations
                 // complete in issue order) exactly one group behind the requests.  The scale reads are assembly as
                 // well: the compiler does not count the transposed reads, so a wait it places for a scale read of its
                 // own would also wait for every fragment requested since.
@@ -903,80 +1078,84 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false> __global__ __launch_bo
                 VFrag vf[2][4];
                 if (!table_fits) {
                     // The f16 table of this tile was written for another window (the first tile of a split, or the scales
-                    // grew since): the wave rewrites the 4 x 32 entries it is about to read from the f32 table.  The other
-                    // value wave of the same column half writes the same values; LDS operations of a wave complete in order.
+                    // grew since): the wave rewrites the GROUPS x 32 entries it is about to read from the f32 table.  Another
+                    // value wave with the same columns writes the same values; LDS operations of a wave complete in order.
                     const float into_window = __uint_as_float((unsigned int)(127 - kPShift - window) << 23);
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
+                    for (int e = 0; e < GROUPS / 2; ++e) {
                         const unsigned int idx = lane + 64u * e;
-                        const unsigned int g = 4u * dh + (idx >> 5), t = idx & 31u;
+                        const unsigned int g = GROUPS * part + (idx >> 5), t = idx & 31u;
                         lds_scale16[value_tile][g][t] = (_Float16)(lds_scale[value_tile][g][t] * into_window);
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 }
-                {
-                    // P'_g = p16 * scale16_g: both factors are f16 already (the probabilities from the score wave, the scales
-                    // from the conversion, divided by the window there), one packed multiply per two tokens
-                    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-                    const unsigned int gs16_lds = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const _Float16*)&lds_scale16[0][0][0] +
-                                                  (value_tile * (8 * kStepTokens) + dh * (4 * kStepTokens) + 4 * j) * 2u;
-                    auto scales16_of = [&](int g, u32x2& lo, u32x2& hi) __attribute__((always_inline)) {
-                        asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(lo) : "v"(gs16_lds), "i"(g * kStepTokens * 2));
-                        asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(hi) : "v"(gs16_lds), "i"(g * kStepTokens * 2 + 32));
-                    };
-                    auto pk_mul = [](unsigned int x, unsigned int y) __attribute__((always_inline)) -> unsigned int {
-                        return __builtin_bit_cast(unsigned int, __builtin_bit_cast(f16x2_t, x) * __builtin_bit_cast(f16x2_t, y));
-                    };
-                    u32x2 gs_lo[2], gs_hi[2];
-                    load_group(vf[0], 0);
-                    scales16_of(0, gs_lo[0], gs_hi[0]);
+                // P'_g = p16 * scale16_g: both factors are f16 already (the probabilities from the score wave, the scales
+                // from the conversion, divided by the window there), one packed multiply per two tokens
+                const unsigned int gs16_lds = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) const _Float16*)&lds_scale16[0][0][0] +
+                                              (value_tile * (8 * kStepTokens) + part * (GROUPS * kStepTokens) + 4 * j) * 2u;
+                auto scales16_of = [&](int g, u32x2& lo, u32x2& hi) __attribute__((always_inline)) {
+                    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(lo) : "v"(gs16_lds), "i"(g * kStepTokens * 2));
+                    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(hi) : "v"(gs16_lds), "i"(g * kStepTokens * 2 + 32));
+                };
+                u32x2 gs_lo[2], gs_hi[2];
+                load_group(vf[0], 0);
+                scales16_of(0, gs_lo[0], gs_hi[0]);
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int cur = g & 1;
-                        if (g + 1 < 4) {
-                            load_group(vf[cur ^ 1], g + 1);
-                            scales16_of(g + 1, gs_lo[cur ^ 1], gs_hi[cur ^ 1]);
-                            // group g's ten reads are older than the ten just issued
-                            asm volatile("s_waitcnt lgkmcnt(10)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
-                                         "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
-                                         "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
-                                         :
-                                         : "memory");
-                        } else {
-                            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
-                                         "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
-                                         "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
-                                         :
-                                         : "memory");
-                        }
+                for (int g = 0; g < GROUPS; ++g) {
+                    const int cur = g & 1;
+                    if (g + 1 < GROUPS) {
+                        load_group(vf[cur ^ 1], g + 1);
+                        scales16_of(g + 1, gs_lo[cur ^ 1], gs_hi[cur ^ 1]);
+                        // group g's ten reads are older than the ten just issued
+                        asm volatile("s_waitcnt lgkmcnt(10)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
+                                     "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
+                                     :
+                                     : "memory");
+                    } else {
+                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[cur][0].s[0]), "+v"(vf[cur][0].s[1]), "+v"(vf[cur][1].s[0]), "+v"(vf[cur][1].s[1]),
+                                     "+v"(vf[cur][2].s[0]), "+v"(vf[cur][2].s[1]), "+v"(vf[cur][3].s[0]), "+v"(vf[cur][3].s[1]),
+                                     "+v"(gs_lo[cur]), "+v"(gs_hi[cur])
+                                     :
+                                     : "memory");
+                    }
 #pragma unroll
-                        for (int ht = 0; ht < 2; ++ht) {
-                            Frag pf;
-                            pf.u[0] = pk_mul(p16[ht][0], gs_lo[cur][0]);
-                            pf.u[1] = pk_mul(p16[ht][1], gs_lo[cur][1]);
-                            pf.u[2] = pk_mul(p16[ht][2], gs_hi[cur][0]);
-                            pf.u[3] = pk_mul(p16[ht][3], gs_hi[cur][1]);
+                    for (int ht = 0; ht < HT; ++ht) {
+                        Frag pf;
+                        pf.u[0] = pk_mul(p16[ht][0], gs_lo[cur][0]);
+                        pf.u[1] = pk_mul(p16[ht][1], gs_lo[cur][1]);
+                        pf.u[2] = pk_mul(p16[ht][2], gs_hi[cur][0]);
+                        pf.u[3] = pk_mul(p16[ht][3], gs_hi[cur][1]);
 #pragma unroll
-                            for (int tt = 0; tt < 4; ++tt) {
-                                acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[cur][tt].h, pf.h, acc[ht][g * 4 + tt], 0, 0, 0);
-                            }
+                        for (int tt = 0; tt < 4; ++tt) {
+                            acc[ht][g * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[cur][tt].h, pf.h, acc[ht][g * 4 + tt], 0, 0, 0);
                         }
                     }
                 }
-            }
+            };
             if (i > 0) {
+                // (the one-tile form exists in the narrow layout only: with the wide layout's 32 accumulators a second form
+                // of the block in the same kernel costs 150 spilled registers, and its empty tiles are multiplied and dropped)
+                if (second_tile) {
+                    accumulate(std::integral_constant<int, 2>{});
+                } else {
+                    accumulate(std::integral_constant<int, 1>{});
+                }
                 value_tile = value_tile == kWsTiles - 1u ? 0u : value_tile + 1u;
             }
             lds_barrier();
+        }
+        if constexpr (NARROW) {
+            lds_barrier(); // the score waves exchange their token halves' sums behind this one
         }
 #pragma unroll
         for (int ht = 0; ht < 2; ++ht) {
             const unsigned int out_head = blockIdx.y * 64u + (2u * hp + ht) * 16u + m;
             if (out_head < p.heads) {
-                float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + dh * 256u;
+                float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + part * (GROUPS * 64u);
                 const float out_of_window = __uint_as_float((unsigned int)(127 + window) << 23);
 #pragma unroll
-                for (int t = 0; t < 16; ++t) {
+                for (int t = 0; t < GROUPS * 4; ++t) {
                     *(f32x4*)(out + t * 16 + 4 * j) = acc[ht][t] * out_of_window;
                 }
             }
@@ -1572,16 +1751,17 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
         const dim3 grid(p.max_chunks, (p.heads + 63) / 64, p.batch);
+        const bool narrow = p.heads <= 32u; // two head tiles at most: the score waves split a step's tokens, the value waves the columns four ways
+        const bool aligned = p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0;
+        const bool pow2_tables = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.tables != nullptr;
         if (p.selection != nullptr) {
-            mla_partial_ws<false, true><<<grid, dim3(512), 0, stream>>>(p);
-        } else if (p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0) {
-            if ((p.block_tokens & (p.block_tokens - 1u)) == 0 && p.tables != nullptr) {
-                mla_partial_ws<true, false, true><<<grid, dim3(512), 0, stream>>>(p);
-            } else {
-                mla_partial_ws<true, false><<<grid, dim3(512), 0, stream>>>(p);
-            }
+            (narrow ? mla_partial_ws<false, true, false, true> : mla_partial_ws<false, true>)<<<grid, dim3(512), 0, stream>>>(p);
+        } else if (aligned && pow2_tables) {
+            (narrow ? mla_partial_ws<true, false, true, true> : mla_partial_ws<true, false, true>)<<<grid, dim3(512), 0, stream>>>(p);
+        } else if (aligned) {
+            (narrow ? mla_partial_ws<true, false, false, true> : mla_partial_ws<true, false>)<<<grid, dim3(512), 0, stream>>>(p);
         } else {
-            mla_partial_ws<false, false><<<grid, dim3(512), 0, stream>>>(p);
+            (narrow ? mla_partial_ws<false, false, false, true> : mla_partial_ws<false, false>)<<<grid, dim3(512), 0, stream>>>(p);
         }
         err = hipGetLastError();
         if (err != hipSuccess) {
