@@ -97,7 +97,7 @@ def mla_batch_cases(args):
 
     from zllm_amd import capi, ops
 
-    nope, rope, value, latent, bt = 128, 64, 128, 512, 64
+    rope, latent, bt = 64, 512, 64
     ops.init(0)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(2)
@@ -109,9 +109,9 @@ def mla_batch_cases(args):
     lib = capi.load()
     # 128 heads over batch sizes; then one sequence of 32 and 64 heads at long contexts, the shape of the reference's own
     # split-decode latency test (src/kernel/rocm/hip/attention/paged_mla.rs:6243-6253: a GPU's half of the heads)
-    shapes = [(128, batch, ctx) for batch in (1, 3, 4, 13, 16, 32, 64) for ctx in (2048, 16384)]
-    shapes += [(heads, 1, ctx) for heads in (32, 64) for ctx in (16384, 131072)]
-    for heads, batch, ctx in shapes:
+    shapes = [(128, batch, ctx, 128, 128) for batch in (1, 3, 4, 13, 16, 32, 64) for ctx in (2048, 16384)]
+    shapes += [(heads, 1, ctx, 192, 256) for heads in (32, 64) for ctx in (2048, 16384, 131072)]  # q_head 256, kv_head 448
+    for heads, batch, ctx, nope, value in shapes:
         kv_b = (torch.randn((heads * (nope + value), latent), generator=gen, device="cuda") / np.sqrt(latent)).to(torch.bfloat16)
         need = batch * ctx // bt
         tables = torch.from_numpy(rng.choice(pool, size=need, replace=False).astype(np.uint32).reshape(batch, -1).view(np.int32)).to("cuda")
@@ -127,10 +127,10 @@ def mla_batch_cases(args):
 
         stage = {name: round(_time_us(launch(mask), launches=20), 1) for name, mask in (("absorb", 1), ("partial", 2), ("merge_project", 12), ("call", 0))}
         flops = batch * ctx * heads * (2 * 576 + 2 * 512)
-        print(json.dumps({"suite": "mla_batches", "batch": batch, "heads": heads, "ctx": ctx, "stage_us": stage,
+        print(json.dumps({"suite": "mla_batches", "batch": batch, "heads": heads, "q_head_dim": nope + rope, "kv_head_dim": nope + value, "ctx": ctx, "stage_us": stage,
                           "call_tflops": round(flops / stage["call"] / 1e6, 1)}), flush=True)
     # one long sequence among short ones, with and without the token-count hint
-    heads = 128
+    heads, nope, value = 128, 128, 128
     kv_b = (torch.randn((heads * (nope + value), latent), generator=gen, device="cuda") / np.sqrt(latent)).to(torch.bfloat16)
     batch, lens_host = 32, [65536] + [2048] * 31
     need = sum(l // bt for l in lens_host)

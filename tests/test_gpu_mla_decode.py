@@ -218,11 +218,14 @@ def test_mla_split_invariance_and_zero_query():
     assert np.abs(got - want).max() < 2e-3
 
 
-def test_mla_reference_split_test_recipe():
+@pytest.mark.parametrize("heads,ctx", [(64, 1357), (32, 768), (32, 2048), (32, 16384), (64, 16384)])
+def test_mla_reference_split_test_recipe(heads, ctx):
     """Integer-pattern recipe of `mla_decode_split_matches_serial_and_reports_latency`
-    (src/kernel/rocm/hip/attention/paged_mla.rs:6226-6342): q_head 256, kv_head 448, latent 512, rope 64, 64 heads,
-    128-token identity pages, scales 0x3b80; checked against the CPU oracle at that test's 5e-3 bound."""
-    heads, q_head, kv_head, latent, rope, ctx, bt = 64, 256, 448, 512, 64, 1357, 128
+    (src/kernel/rocm/hip/attention/paged_mla.rs:6226-6342): q_head 256, kv_head 448, latent 512, rope 64, 64 heads and
+    the 32 of a GPU's half, 128-token identity pages, scales 0x3b80, contexts from that test's list; checked against the
+    CPU oracle at that test's 5e-3 bound.  (32 heads run the narrow layout of the partial kernel; 16,384 tokens are cut
+    into a split per compute unit, merged by the wide merge; the value width of 256 takes the projection's general path.)"""
+    q_head, kv_head, latent, rope, bt = 256, 448, 512, 64, 128
     q = np.array([((i % 257) - 128) / 256.0 for i in range(heads * q_head)], dtype=np.float32)
     weight = np.array([(((i * 17) % 127) - 63) / 4096.0 for i in range(heads * kv_head * latent)], dtype=np.float32)
     codes = np.array([((i * 29 + i // latent * 7) % 63 + 1) for i in range(ctx * latent)], dtype=np.uint8).view(np.int8)

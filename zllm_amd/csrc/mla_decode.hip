@@ -81,20 +81,21 @@ __device__ __forceinline__ unsigned int visible_tokens(const unsigned int* ctx_l
 // ---------------------------------------------------------------------------------------------
 // 1. absorb
 // ---------------------------------------------------------------------------------------------
-// grid = (heads, batch, 4), one wave; a thread owns two adjacent latent columns, a workgroup every fourth run of 64
-// column pairs (with the usual 512 columns: one run).  A decode call of one sequence has as many (row, head) pairs as
-// heads, so the weights of a head are fetched by four compute units instead of one: 128 load instructions a wave
-// instead of 512 a compute unit.
+// grid = (heads, batch, z), 256 / z threads, z = 1 or 4; a thread owns two adjacent latent columns, the z workgroups of a
+// (row, head) take the runs of 256 / z column pairs in turn.  A decode call of one sequence has as many (row, head) pairs
+// as heads: with z = 4 the weights of a head are fetched by four compute units, 128 load instructions each, instead of
+// 512 on one (one sequence of 32 heads: 6.7 -> 4.7 us); from a few hundred pairs on the compute units are busy either
+// way and one workgroup per pair is the shorter launch (config 4, 512 pairs: 7.7 against 8.3 us).
 // The sum runs over k in ascending order with separately rounded multiply and add, the order of
 // the reference's scalar matmul (src/kernel/cpu/mla.rs:712-728); the result is rounded to bf16
 // (mla.rs:1037).
-__global__ __launch_bounds__(64) void mla_absorb(MlaDecodeParams p)
+__global__ __launch_bounds__(256) void mla_absorb(MlaDecodeParams p)
 {
     const unsigned int head = blockIdx.x;
     const unsigned int b = blockIdx.y;
     __shared__ float q_sh[1024];
     const size_t q_base = ((size_t)b * p.heads + head) * p.q_head_dim;
-    for (unsigned int i = threadIdx.x; i < p.q_head_dim; i += 64) {
+    for (unsigned int i = threadIdx.x; i < p.q_head_dim; i += blockDim.x) {
         float x = load_as_f32(p.q, q_base + i, p.q_dtype);
         // the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
         q_sh[i] = bf16_bits_to_f32(f32_to_bf16_bits(x));
@@ -104,13 +105,15 @@ __global__ __launch_bounds__(64) void mla_absorb(MlaDecodeParams p)
     // sequential in k)
     const unsigned int pairs = p.latent_dim / 2u;
     const unsigned int* w = (const unsigned int*)(p.kv_b + (size_t)head * p.kv_head_dim * p.latent_dim);
-    if (pairs == 256u && p.nope_dim == 128u) {
-        // the usual geometry (latent 512, nope 128): all 128 weight words of the thread are requested at once, before the
-        // query has even arrived in LDS -- the kernel is one memory round trip long instead of four
-        const unsigned int c2 = blockIdx.z * 64u + threadIdx.x;
-        unsigned int word[128];
+    // the usual geometries (latent 512; nope 128, or 192 as in the reference's own decode test): all weight words of the
+    // thread are requested at once, before the query has even arrived in LDS -- the kernel is one memory round trip long
+    // instead of one per 32 query elements
+    auto one_trip = [&](auto nope) __attribute__((always_inline)) {
+        constexpr int NOPE = decltype(nope)::value;
+        const unsigned int c2 = blockIdx.z * blockDim.x + threadIdx.x;
+        unsigned int word[NOPE];
 #pragma unroll
-        for (int k = 0; k < 128; ++k) {
+        for (int k = 0; k < NOPE; ++k) {
             word[k] = w[(size_t)k * 256u + c2];
         }
         __syncthreads();
@@ -119,15 +122,20 @@ __global__ __launch_bounds__(64) void mla_absorb(MlaDecodeParams p)
 #pragma clang fp contract(off)
             float acc0 = 0.0f, acc1 = 0.0f;
 #pragma unroll
-            for (int k = 0; k < 128; ++k) {
+            for (int k = 0; k < NOPE; ++k) {
                 acc0 = acc0 + q_sh[k] * __uint_as_float(word[k] << 16);
                 acc1 = acc1 + q_sh[k] * __uint_as_float(word[k] & 0xffff0000u);
             }
             *(unsigned int*)(qa + 2u * c2) = (unsigned int)f32_to_bf16_bits(acc0) | ((unsigned int)f32_to_bf16_bits(acc1) << 16);
         }
+    };
+    if (pairs == 256u && p.nope_dim == 128u) {
+        one_trip(std::integral_constant<int, 128>{});
+    } else if (pairs == 256u && p.nope_dim == 192u) {
+        one_trip(std::integral_constant<int, 192>{});
     } else {
         __syncthreads();
-        for (unsigned int c2 = blockIdx.z * 64u + threadIdx.x; c2 < pairs; c2 += 256) {
+        for (unsigned int c2 = blockIdx.z * blockDim.x + threadIdx.x; c2 < pairs; c2 += 256) {
             // product and sum rounded separately, as in the CPU code (plain operators: the __fmul_rn / __fadd_rn intrinsics
             // are ordinary operators from a header compiled with fusing allowed)
 #pragma clang fp contract(off)
@@ -150,7 +158,7 @@ __global__ __launch_bounds__(64) void mla_absorb(MlaDecodeParams p)
         }
     }
     if (blockIdx.z == 0u) {
-        for (unsigned int r = threadIdx.x; r < p.rope_dim; r += 64) {
+        for (unsigned int r = threadIdx.x; r < p.rope_dim; r += blockDim.x) {
             qa[p.latent_dim + r] = f32_to_bf16_bits(q_sh[p.nope_dim + r]);
         }
     }
@@ -1408,12 +1416,16 @@ __global__ __launch_bounds__(256) void mla_merge_wide(MlaDecodeParams p)
         f32x4 part[16];
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
-            const unsigned int c = min(c0 + 16u * u, p.max_chunks - 1u);
-            const bool live = c0 + 16u * u < p.max_chunks;
-            const float2 st = *(const float2*)(stats + c * stat_stride);
-            cm[u] = live ? st.x : kNegInf;
-            cl[u] = live ? st.y : 0.0f;
-            part[u] = *(const f32x4*)(partial + c * partial_stride);
+            const unsigned int c = c0 + 16u * u;
+            cm[u] = kNegInf;
+            cl[u] = 0.0f;
+            part[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (c < p.max_chunks) { // a plan of few splits leaves most of a lane's sixteen requests unmade
+                const float2 st = *(const float2*)(stats + c * stat_stride);
+                cm[u] = st.x;
+                cl[u] = st.y;
+                part[u] = *(const f32x4*)(partial + c * partial_stride);
+            }
         }
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
@@ -1741,7 +1753,8 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         } else if (p.batch >= 32u && p.nope_dim <= 256u) {
             mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
         } else {
-            mla_absorb<<<dim3(p.heads, p.batch, 4), dim3(64), 0, stream>>>(p);
+            const unsigned int z = p.heads * p.batch <= 128u ? 4u : 1u;
+            mla_absorb<<<dim3(p.heads, p.batch, z), dim3(256u / z), 0, stream>>>(p);
         }
         err = hipGetLastError();
         if (err != hipSuccess) {
