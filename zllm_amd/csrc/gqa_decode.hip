@@ -1371,6 +1371,120 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
     }
 }
 
+// The merge for a call of few rows cut into hundreds of splits (one sequence alone on the GPU gets a split per compute
+// unit and KV-head block: 256 or 512 records per head).  One workgroup per (row, head) folds them in four to eight
+// dependent round trips on as many compute units as the call has heads, and a single thread per column quad then walks
+// the split lanes' results in LDS.  Here a workgroup takes 32 columns of a (row, head): 256 threads = 32 split lanes x 8
+// column quads, eight records per lane and trip (256 splits: one round trip, requested before the sequence length is
+// known), the eight lanes of a quad inside a wave meet through lane exchanges and the four waves through LDS.
+// grid = (heads, rows, head_dim / 32).
+__global__ __launch_bounds__(256) void gqa_decode_merge_wide(GqaDecodeParams p)
+{
+    const unsigned int head = blockIdx.x;
+    const unsigned int b = blockIdx.y;
+    const unsigned int quad = threadIdx.x & 7u;
+    const unsigned int sl = threadIdx.x >> 3;
+    const unsigned int column = blockIdx.z * 32u + quad * 4u;
+    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    const size_t stat_stride = (size_t)p.num_heads * 2;
+    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + column;
+    const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
+    // first trip: addresses clamped to the planned splits, so the loads do not wait for the length
+    float2 st[8];
+    f32x4 part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const unsigned int c = min(sl + 32u * u, p.max_chunks - 1u);
+        st[u] = *(const float2*)(stats + c * stat_stride);
+        part[u] = *(const f32x4*)(partial + c * partial_stride);
+    }
+    unsigned int chunks = p.fixed_chunks;
+    if (chunks == 0u) {
+        unsigned int len = p.kv_lens[b];
+        if (p.query_rows > 1u) { // record row b of a multi-row call: its sequence's length less the chunk rows after it
+            const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
+            len = p.kv_lens[b / p.query_rows];
+            len = len > behind ? len - behind : 0u;
+        }
+        unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+        first = min(first, len);
+        const unsigned int first_al = first & ~31u;
+        chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+    }
+    float m = kNegInf, l = 0.0f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned int c0 = sl;; c0 += 256u) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (c0 + 32u * u < chunks && st[u].y > 0.0f) {
+                const float nm = fmaxf(m, st[u].x);
+                const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+                const float w = __builtin_amdgcn_exp2f(st[u].x - nm);
+                acc = acc * a + part[u] * w;
+                l = l * a + st[u].y * w;
+                m = nm;
+            }
+        }
+        if (c0 - sl + 256u >= chunks) { // the same for every thread of the workgroup
+            break;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const unsigned int c = min(c0 + 256u + 32u * u, p.max_chunks - 1u);
+            st[u] = *(const float2*)(stats + c * stat_stride);
+            part[u] = *(const f32x4*)(partial + c * partial_stride);
+        }
+    }
+    // two partial merges into one; a side that holds nothing has l = 0
+    auto fold = [](float& m, float& l, f32x4& acc, float om, float ol, const f32x4& oacc) __attribute__((always_inline)) {
+        const float nm = fmaxf(l > 0.0f ? m : kNegInf, ol > 0.0f ? om : kNegInf);
+        const float a = l > 0.0f ? __builtin_amdgcn_exp2f(m - nm) : 0.0f;
+        const float w = ol > 0.0f ? __builtin_amdgcn_exp2f(om - nm) : 0.0f;
+        acc = acc * a + oacc * w;
+        l = l * a + ol * w;
+        m = nm;
+    };
+#pragma unroll
+    for (int step = 8; step <= 32; step *= 2) {
+        const float om = __shfl_xor(m, step), ol = __shfl_xor(l, step);
+        const f32x4 oacc = {__shfl_xor(acc[0], step), __shfl_xor(acc[1], step), __shfl_xor(acc[2], step), __shfl_xor(acc[3], step)};
+        fold(m, l, acc, om, ol, oacc);
+    }
+    __shared__ float wave_m[4][8], wave_l[4][8];
+    __shared__ f32x4 wave_acc[4][8];
+    if ((threadIdx.x & 63u) < 8u) {
+        wave_m[threadIdx.x >> 6][quad] = m;
+        wave_l[threadIdx.x >> 6][quad] = l;
+        wave_acc[threadIdx.x >> 6][quad] = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x < 8u) {
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            fold(m, l, acc, wave_m[w][quad], wave_l[w][quad], wave_acc[w][quad]);
+        }
+        f32x4 result = {0.f, 0.f, 0.f, 0.f};
+        if (l > 0.0f && l < __builtin_inff()) {
+            result = acc * (1.0f / l);
+        }
+        if (p.gate != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                result[e] = gated(result[e], p.gate, p.gate_cols, p.gate_dtype, b, head * p.head_dim + column + e);
+            }
+        }
+        const size_t at = ((size_t)b * p.num_heads + head) * p.head_dim + column;
+        if (p.out_dtype == 0) {
+            *(f32x4*)(p.out + at) = result;
+        } else if (p.out_dtype == 1) {
+            *(u32x2*)((unsigned short*)p.out + at) = u32x2{pack_bf16_rne(result[0], result[1]), pack_bf16_rne(result[2], result[3])};
+        } else {
+            *(u32x2*)((unsigned short*)p.out + at) = u32x2{(unsigned int)f32_to_f16_bits(result[0]) | ((unsigned int)f32_to_f16_bits(result[1]) << 16),
+                                                            (unsigned int)f32_to_f16_bits(result[2]) | ((unsigned int)f32_to_f16_bits(result[3]) << 16)};
+        }
+    }
+}
+
 // The same combine for plans of at most eight splits (large batches, short contexts): a thread owns four output
 // dimensions of one (head, sequence) and folds the few records itself, 256 / (head_dim / 4) heads a workgroup.  One
 // workgroup of 256 threads per (head, sequence) is mostly idle lanes there, and with hundreds of sequences the launch
@@ -1588,6 +1702,9 @@ hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)
     if (p.max_chunks <= 8u && quads <= 256u && 256u % quads == 0u) {
         const unsigned int heads_here = 256u / quads;
         gqa_decode_merge_few<<<dim3((p.num_heads + heads_here - 1u) / heads_here, p.batch), dim3(256), 0, stream>>>(p);
+    } else if (p.max_chunks > 8u * (256u / quads) && p.head_dim % 32u == 0u && p.num_heads * p.batch <= 512u) {
+        // more splits than one workgroup per (row, head) reads in a round trip, and few such pairs
+        gqa_decode_merge_wide<<<dim3(p.num_heads, p.batch, p.head_dim / 32u), dim3(256), 0, stream>>>(p);
     } else {
         gqa_decode_merge<<<dim3(p.num_heads, p.batch), dim3(256), 0, stream>>>(p);
     }
