@@ -30,6 +30,26 @@ def run_decode(case, score_scale, window=0, softcap=0.0, max_kv_len=None, ring_c
     return out.cpu().numpy()
 
 
+@pytest.mark.parametrize("hq,hkv,d,lens,window,gated", [(64, 8, 128, [9000], 0, False), (16, 2, 128, [20000], 0, True),
+                                                        (32, 4, 128, [9000, 100], 5000, False), (16, 8, 256, [5000], 0, True),
+                                                        (32, 8, 64, [17000], 0, False)])
+def test_one_or_two_long_sequences_take_the_wide_merge(hq, hkv, d, lens, window, gated):
+    """A sequence alone on the GPU is cut into a split per compute unit and KV-head block, 128 to 512 records per head:
+    the merge then runs as head_dim / 32 workgroups per (head, sequence), one round trip for 256 records (20,000 tokens of
+    two KV heads: 313 records, two trips).  With a short sequence beside the long one, a window, and the fused gate."""
+    case = make_gqa_q8_case(70 + hq, lens, hq, hkv, d, outliers=True)
+    gate = dev_gate = None
+    if gated:
+        gate = (np.random.default_rng(71).standard_normal((len(lens), hq * d)) * 3).astype(np.float32)
+        dev_gate = upload(gate)
+    got = run_decode(case, 0.09, window=window, gate=dev_gate)
+    want = oracle_gqa_decode(case, 0.09, window=window)
+    if gated:
+        rc, want = O.sigmoid_gate(want, gate)
+        assert rc == 0
+    print("wide merge", hq, hkv, d, lens, assert_attention_close(got, want, f"{hq}/{hkv} d={d} lens={lens}"))
+
+
 @pytest.mark.parametrize("per_row,gate_bf16", [(False, False), (True, False), (False, True)])
 def test_decode_output_gate(per_row, gate_bf16):
     """out * sigmoid(gate) fused into the split merge (src/attention/hybrid.rs:79, src/backend/cpu/context.rs:419-432)."""
