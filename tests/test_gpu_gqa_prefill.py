@@ -88,7 +88,9 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
 @pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,softcap,extra", [
     (128, 5000, 8, 16, 2, 0, 0.0, ""), (128, 3000, 300, 8, 2, 700, 0.0, ""), (128, 2500, 70, 32, 4, 0, 30.0, "gate"),
     (128, 4000, 33, 8, 1, 0, 0.0, "bf16out"), (128, 2000, 90, 8, 2, 0, 0.0, "ends"), (64, 3000, 20, 8, 2, 0, 0.0, ""),
-    (256, 3000, 20, 8, 2, 500, 0.0, ""), (128, 2600, 16, 16, 4, 0, 0.0, "f32scales")])
+    (256, 3000, 20, 8, 2, 500, 0.0, ""), (128, 2600, 16, 16, 4, 0, 0.0, "f32scales"),
+    # more than 64 splits a row and few rows: the records go through the wide split merge
+    (128, 24000, 8, 16, 2, 0, 0.0, "gate"), (128, 20000, 4, 32, 4, 0, 0.0, "bf16out")])
 def test_prefill_kv_splits_and_the_unsplit_kernel_agree(d, prefix, chunk, hq, hkv, window, softcap, extra):
     """A short chunk over a long prefix is cut into KV splits when the caller brings the workspace for their records (parts
     of a row tile's visible range, merged like a decode call's splits) and runs unsplit without one: both against the oracle.
