@@ -78,13 +78,16 @@ def prefill_chunk_cases(args):
     for name in ("k", "v"):
         rows = torch.randn((total, cols), generator=gen, device="cuda").to(torch.bfloat16)
         ops.q8g64_append(rows, planes[name + "c"], planes[name + "s"], table, 0, bt, capi.QUANT_METAL_GQA)
+    lib = capi.load()
     for prefix in (2048, 32768):
-        for chunk in (1, 8, 64, 256, 512, 2048):
+        for chunk in (1, 2, 4, 8, 64, 256, 512, 2048):
             q = torch.randn((chunk, hq * d), generator=gen, device="cuda").to(torch.bfloat16)
             times = {}
             for label, workspace in (("with_workspace", True), ("without_workspace", False)):
-                times[label] = _time_us(lambda: ops.gqa_prefill_chunk(q, planes["kc"], planes["ks"], planes["vc"], planes["vs"], table, prefix, hq, hkv,
-                                                                        d, bt, 1.0 / float(np.sqrt(d)), workspace=workspace), launches=5)
+                call, out, scratch = ops.gqa_prefill_chunk_args(q, planes["kc"], planes["ks"], planes["vc"], planes["vs"], table, prefix, hq, hkv,
+                                                                d, bt, 1.0 / float(np.sqrt(d)), workspace=workspace)
+                times[label] = _time_us(lambda: capi.check(lib.zllm_attn_gqa_prefill_chunk(C.byref(call), C.c_void_p(torch.cuda.current_stream().cuda_stream))),
+                                        launches=5)
             pairs = sum(prefix + r + 1 for r in range(chunk))
             flops = 4 * d * hq * pairs
             print(json.dumps({"suite": "prefill_chunks", "heads": f"{hq}q/{hkv}kv", "head_dim": d, "prefix": prefix, "chunk_rows": chunk,

@@ -316,11 +316,15 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * (parts of a tile's visible range, combined like a decode call's splits) when the
  * caller passes zllm_attn_gqa_prefill_workspace_bytes of 16-byte aligned workspace
  * for their records, and runs unsplit (same results, one workgroup walking the whole
- * prefix per tile) when it passes none or less.  What is
+ * prefix per tile) when it passes none or less.  A chunk of a few rows (one to four
+ * over a long prefix, up to sixteen over a short one) is a decode step in all but name
+ * -- the reference decodes through this path with one row
+ * (src/backend/rocm/attention.rs:2202-2231) -- and, given that workspace, runs every
+ * row as one item of the split-KV decode kernels.  So does what is
  * left -- f32 queries other than over Q8g64 with 16-bit scales at head_dim 128; more
- * than 128 query heads per KV head at head_dim 256 -- runs every row as one item of
- * the split-KV decode kernels (bound by cache bandwidth, not by the matrix cores) and
- * cannot run without that workspace. */
+ * than 128 query heads per KV head at head_dim 256 -- whatever the number of rows
+ * (bound by cache bandwidth, not by the matrix cores); that cannot run without the
+ * workspace. */
 typedef struct zllm_gqa_prefill_args {
     const void* q;         /* [dev] [rows, num_heads * head_dim], q_dtype */
     const void* k_plane;   /* [dev] */

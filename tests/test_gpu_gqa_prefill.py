@@ -86,11 +86,11 @@ def run_case(seed, prefix, chunk, hq, hkv, window=0, softcap=0.0, block_tokens=1
 
 
 @pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,softcap,extra", [
-    (128, 5000, 8, 16, 2, 0, 0.0, ""), (128, 3000, 300, 8, 2, 700, 0.0, ""), (128, 2500, 70, 32, 4, 0, 30.0, "gate"),
+    (128, 5000, 24, 16, 2, 0, 0.0, ""), (128, 3000, 300, 8, 2, 700, 0.0, ""), (128, 2500, 70, 32, 4, 0, 30.0, "gate"),
     (128, 4000, 33, 8, 1, 0, 0.0, "bf16out"), (128, 2000, 90, 8, 2, 0, 0.0, "ends"), (64, 3000, 20, 8, 2, 0, 0.0, ""),
-    (256, 3000, 20, 8, 2, 500, 0.0, ""), (128, 2600, 16, 16, 4, 0, 0.0, "f32scales"),
+    (256, 3000, 20, 8, 2, 500, 0.0, ""), (128, 2600, 40, 16, 4, 0, 0.0, "f32scales"),
     # more than 64 splits a row and few rows: the records go through the wide split merge
-    (128, 24000, 8, 16, 2, 0, 0.0, "gate"), (128, 20000, 4, 32, 4, 0, 0.0, "bf16out")])
+    (128, 24000, 8, 16, 2, 0, 0.0, "gate"), (128, 20000, 12, 32, 4, 0, 0.0, "bf16out")])
 def test_prefill_kv_splits_and_the_unsplit_kernel_agree(d, prefix, chunk, hq, hkv, window, softcap, extra):
     """A short chunk over a long prefix is cut into KV splits when the caller brings the workspace for their records (parts
     of a row tile's visible range, merged like a decode call's splits) and runs unsplit without one: both against the oracle.
@@ -125,6 +125,28 @@ def test_prefill_kv_splits_and_the_unsplit_kernel_agree(d, prefix, chunk, hq, hk
             assert np.abs(got - want).max() <= 2e-3 + tol * max(1.0, float(np.abs(want).max()))
         else:
             assert_attention_close(got, want, f"d={d} prefix={prefix} chunk={chunk} {hq}/{hkv} {extra} workspace={workspace}")
+
+
+@pytest.mark.parametrize("d,prefix,chunk,hq,hkv,window,extra", [
+    (128, 20000, 1, 32, 8, 0, ""), (128, 5000, 4, 16, 2, 0, "gate"), (128, 3000, 2, 8, 2, 700, "bf16out"),
+    (128, 900, 8, 8, 2, 0, "ends"), (256, 6000, 3, 8, 2, 0, ""), (64, 2000, 5, 8, 2, 0, "")])
+def test_prefill_few_rows_run_as_decode_items(d, prefix, chunk, hq, hkv, window, extra):
+    """A chunk of a few rows is a decode step in all but name (the reference decodes through this entry with one row,
+    src/backend/rocm/attention.rs:2202-2231): with the workspace the call asks for, its rows run as items of the decode
+    kernels; without one, through the chunk kernel.  Both against the oracle, with a gate, a window, explicit visible ends
+    and bf16 output."""
+    kw = dict(window=window, outliers=True, d=d)
+    if extra == "gate":
+        kw["gate_cols"] = hq * d
+    if extra == "bf16out":
+        kw["out_dtype"] = torch.bfloat16
+    if extra == "ends":
+        kw["visible_ends"] = np.array([prefix + 4] * 4 + [0] + [prefix + chunk] * (chunk - 5), dtype=np.uint32)
+    tol = 2.0 ** -8 if extra == "bf16out" else 0.0
+    for workspace in (True, False):
+        out, want = run_case(31 + d + chunk, prefix, chunk, hq, hkv, workspace=workspace, **kw)
+        got = out.float().cpu().numpy()
+        assert np.abs(got - want).max() <= 2e-3 + tol * max(1.0, float(np.abs(want).max())), (workspace, np.abs(got - want).max())
 
 
 def test_prefill_f16_kv_splits():

@@ -1041,20 +1041,46 @@ static void prefill_decode_args(const zllm_gqa_prefill_args* a, zllm_gqa_decode_
     d->gate_dtype = a->gate_dtype;
 }
 
+// Workspace of the route that runs the chunk's rows as items of the decode kernels: the rows' ranges, then the split records
+static uint64_t prefill_decode_route_bytes(const zllm_gqa_prefill_args* a)
+{
+    zllm_gqa_decode_args d;
+    prefill_decode_args(a, &d);
+    const uint64_t records = zllm_attn_gqa_decode_workspace_bytes(&d);
+    return records == 0 ? 0 : align_up((uint64_t)a->rows * 8, 256) + records;
+}
+
+// A chunk of very few rows is a decode step in all but name (the reference decodes through this entry with one row,
+// src/backend/rocm/attention.rs:2202-2231): the chunk kernel would run row tiles that are all but empty.  With the
+// decode route's workspace such a chunk runs as decode items instead, each row re-reading the cache.  Measured on 32
+// query / 8 KV heads of 128 (us, decode items against the chunk kernel with KV splits): one row over 32 K tokens 24 / 71,
+// two 33 / 73, four 56 / 74, eight 104 / 78; eight rows over 2 K tokens 20 / 33 -- about 15 us + 0.34 ns per row and
+// token against 28 us + 1.5 ns per token.
+static bool few_rows_as_decode_items(const zllm_gqa_prefill_args* a)
+{
+    if (a->rows > 16u) {
+        return false;
+    }
+    uint64_t tokens = (uint64_t)a->position + a->rows;
+    if (a->window != 0 && tokens > a->window) {
+        tokens = a->window;
+    }
+    return (uint64_t)a->rows * tokens * 34u < tokens * 150u + 1300000u;
+}
+
 uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* a)
 {
     if (validate_gqa_prefill(a) != 0) {
         return 0;
     }
-    if (!prefill_rows_as_decode_items(a)) {
-        uint32_t chunk_tokens, max_chunks;
-        plan_prefill_splits(a, &chunk_tokens, &max_chunks);
-        return max_chunks > 1 ? prefill_split_records(a, max_chunks).total : 0; /* unsplit, the chunk kernel keeps all of its state on chip */
+    if (prefill_rows_as_decode_items(a)) {
+        return prefill_decode_route_bytes(a);
     }
-    zllm_gqa_decode_args d;
-    prefill_decode_args(a, &d);
-    const uint64_t records = zllm_attn_gqa_decode_workspace_bytes(&d);
-    return records == 0 ? 0 : align_up((uint64_t)a->rows * 8, 256) + records;
+    uint32_t chunk_tokens, max_chunks;
+    plan_prefill_splits(a, &chunk_tokens, &max_chunks);
+    const uint64_t splits = max_chunks > 1 ? prefill_split_records(a, max_chunks).total : 0; /* unsplit, the chunk kernel keeps all of its state on chip */
+    const uint64_t items = few_rows_as_decode_items(a) ? prefill_decode_route_bytes(a) : 0;
+    return splits > items ? splits : items;
 }
 
 int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t stream)
@@ -1076,13 +1102,18 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
         ((a->gate_cols != 1 && a->gate_cols != a->num_heads * a->head_dim) || (a->gate_dtype != ZLLM_DTYPE_F32 && a->gate_dtype != ZLLM_DTYPE_BF16))) {
         return fail(-1, "GQA prefill: gate_cols=%u must be 1 or %u, gate_dtype f32 or bf16", a->gate_cols, a->num_heads * a->head_dim);
     }
-    if (prefill_rows_as_decode_items(a)) {
+    bool as_items = prefill_rows_as_decode_items(a);
+    if (!as_items && few_rows_as_decode_items(a)) {
+        const uint64_t need = prefill_decode_route_bytes(a);
+        as_items = need != 0 && a->workspace != nullptr && a->workspace_bytes >= need && ((uintptr_t)a->workspace & 15u) == 0;
+    }
+    if (as_items) {
         zllm_gqa_decode_args d;
         prefill_decode_args(a, &d);
         if (validate_gqa_decode(&d) != 0) {
             return -1;
         }
-        const uint64_t need = zllm_attn_gqa_prefill_workspace_bytes(a);
+        const uint64_t need = prefill_decode_route_bytes(a);
         if (a->workspace == nullptr || a->workspace_bytes < need || ((uintptr_t)a->workspace & 15u) != 0) {
             return fail(-1, "GQA prefill: this geometry needs a 16-byte aligned workspace of %llu bytes (got %llu)", (unsigned long long)need,
                         (unsigned long long)a->workspace_bytes);

@@ -140,11 +140,11 @@ def gqa_decode_static(*a, **kw):
     return out
 
 
-def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, num_heads, num_kv_heads, head_dim,
-                      block_tokens, score_scale, window=0, softcap=0.0, kv_format=capi.KV_Q8G64,
-                      scale_dtype=capi.SCALE_F16, out_dtype=torch.float32, gate=None, visible_ends=None, workspace=True):
-    """One chunk of causal GQA prefill over the paged cache (zllm_attn_gqa_prefill_chunk).  `workspace=False` passes none:
-    a chunk that would be cut into KV splits then runs unsplit (geometries that need a workspace fail)."""
+def gqa_prefill_chunk_args(q, k_plane, k_scales, v_plane, v_scales, table, position, num_heads, num_kv_heads, head_dim,
+                           block_tokens, score_scale, window=0, softcap=0.0, kv_format=capi.KV_Q8G64,
+                           scale_dtype=capi.SCALE_F16, out_dtype=torch.float32, gate=None, visible_ends=None, workspace=True):
+    """The argument block of zllm_attn_gqa_prefill_chunk, the output tensor and the workspace tensor (None without one):
+    for callers that launch the same call many times."""
     rows = q.shape[0]
     out = torch.empty((rows, num_heads * head_dim), dtype=out_dtype, device=q.device)
     args = capi.GqaPrefillArgs()
@@ -159,10 +159,18 @@ def gqa_prefill_chunk(q, k_plane, k_scales, v_plane, v_scales, table, position, 
         args.gate, args.gate_cols, args.gate_dtype = _ptr(gate), gate.shape[1], _DTYPE[gate.dtype]
     args.visible_ends = _ptr(visible_ends)
     args.table_stride = 0 if table is None else table.numel()
+    scratch = None
     if workspace:
         need = capi.load().zllm_attn_gqa_prefill_workspace_bytes(C.byref(args))
         scratch = torch.empty(max(int(need), 256), dtype=torch.uint8, device=q.device)
         args.workspace, args.workspace_bytes = _ptr(scratch), scratch.numel()
+    return args, out, scratch
+
+
+def gqa_prefill_chunk(*a, **kw):
+    """One chunk of causal GQA prefill over the paged cache (zllm_attn_gqa_prefill_chunk).  `workspace=False` passes none:
+    a chunk that would be cut into KV splits then runs unsplit (geometries that need a workspace fail)."""
+    args, out, _scratch = gqa_prefill_chunk_args(*a, **kw)
     capi.check(capi.load().zllm_attn_gqa_prefill_chunk(C.byref(args), _stream()))
     return out
 
