@@ -169,6 +169,9 @@ def main():
         gqa_decode_cases(args, [(64, 8, 128)], [(8, 32768), (12, 32768), (5, 65536), (16, 65536), (24, 2048), (3, 8192), (128, 1024), (512, 2048)])
     if args.suite in ("gqa_heads", "all"):
         gqa_decode_cases(args, [(32, 4, 128), (16, 2, 128), (8, 1, 128), (8, 1, 64), (4, 1, 256)], [(8, 32768), (32, 8192)])
+        # one sequence alone on the GPU: the reference's embedded engine decodes one request at a time, and its standard
+        # model has 16 query / 2 KV heads of 256 (src/runtime/ornith/mod.rs:709-720)
+        gqa_decode_cases(args, [(16, 2, 256), (64, 8, 128)], [(1, 32768), (1, 131072)])
     if args.suite in ("prefill_chunks", "all"):
         prefill_chunk_cases(args)
     if args.suite in ("mla_batches", "all"):

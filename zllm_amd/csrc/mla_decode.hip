@@ -798,8 +798,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
                     ((u32x2*)&lds_p16[i & 1u][score_tile][lane])[stream] = u32x2{pack_f16_hw(pr[0], pr[1]), pack_f16_hw(pr[2], pr[3])};
                     lds_alpha[i & 1u][2u * score_tile + stream][lane] = run_max; // -inf: nothing seen yet, the probabilities are zeros
                 }
-            } else
-            if (i < steps) {
+            } else if (i < steps) {
                 const unsigned int tb = i % kWsTiles;
                 const unsigned char* tile = lds + tb * kTileBytes;
                 const float (*scale_tile)[kStepTokens] = lds_scale[tb];
