@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     const unsigned int j = lane >> 4;
     const unsigned int kvh = blockIdx.y;
     const unsigned int rows_per_wg = max(1u, 256u / p.group);
-    const unsigned int row0 = blockIdx.x * rows_per_wg;
+    const unsigned int row0 = (gridDim.x - 1u - blockIdx.x) * rows_per_wg; // the row tiles with the longest ranges start first
     const unsigned int cols_used = rows_per_wg * p.group;
 
     // visible token range of the workgroup: union over its rows of key_range(position + row, kv_end), or of
@@ -674,7 +674,7 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     const unsigned int j = lane >> 4;
     const unsigned int kvh = blockIdx.y;
     const unsigned int rows_per_wg = max(1u, (unsigned int)C::kCols / p.group);
-    const unsigned int row0 = blockIdx.x * rows_per_wg;
+    const unsigned int row0 = (gridDim.x - 1u - blockIdx.x) * rows_per_wg; // the row tiles with the longest ranges start first
     const unsigned int cols_used = rows_per_wg * p.group;
 
     // visible token range of the workgroup, as in gqa_prefill_q8
