@@ -957,7 +957,9 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
 void plan_prefill_splits(const zllm_gqa_prefill_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
 {
     const uint32_t group = a->num_heads / a->num_kv_heads;
-    const uint32_t columns = a->head_dim == 256 ? 128u : 256u; // (row, head-in-group) pairs of a workgroup
+    const bool half_tiles = zllm::gqa_prefill_half_tiles(a->rows, a->position, a->window, a->num_heads, a->num_kv_heads, a->head_dim, a->kv_format,
+                                                         a->scale_dtype);
+    const uint32_t columns = a->head_dim == 256 || half_tiles ? 128u : 256u; // (row, head-in-group) pairs of a workgroup
     const uint32_t tile_rows = columns / group > 0 ? columns / group : 1u;
     const uint64_t tiles = ((uint64_t)a->rows + tile_rows - 1) / tile_rows;
     uint64_t longest = (uint64_t)a->position + a->rows; // keys the last row tile may see

@@ -25,6 +25,8 @@
 // every (token, column) pair stays out of the common path of a step: the tile buffer is a literal (LDS addresses in
 // immediates), edge masks and the low-order P' pass sit behind wave-uniform branches, and a column's reference
 // (running maximum, V window) is only touched when some lane's score passes it.
+#include <type_traits>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -45,6 +47,7 @@ constexpr float kLoThreshold = 8.0f;      // see the P.V stage
 constexpr int kColTiles = 2;              // 16-column MFMA tiles per wave
 constexpr int kWaves = 256 / (16 * kColTiles);
 constexpr int kThreads = 64 * kWaves;
+constexpr unsigned long long kComputeUnitsPrefill = 256; // compute units of the device the kernels are tuned for
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -142,9 +145,14 @@ __device__ __forceinline__ void store_split_record(const GqaPrefillParams& p, un
 
 // POW2: pages of a power-of-two size behind a block table, known at compile time (no run-time choice of the address
 // arithmetic, no division code in the loop).
-template <int SDT, bool SOFTCAP, bool POW2>
+// CT: 16-column MFMA tiles per wave.  Two make a workgroup of 256 (row, head-in-group) pairs, in which every K and V^T
+// fragment read from LDS feeds two MFMAs; one makes it 128 pairs, for chunks whose full-size row tiles would be one round
+// of very unequal workgroups (a first chunk: the last tile walks the whole chunk, the first 64 keys) -- twice as many
+// workgroups, handed out longest first, even that out.
+template <int SDT, bool SOFTCAP, bool POW2, int CT = 2>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
+    constexpr int kColTiles = CT; // inside the kernel the name means this instantiation's count
     __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
     __shared__ __align__(16) unsigned char lds_v[2][kTileBytes];
     __shared__ __align__(16) float lds_ks[2][2][kStep]; // [buffer][group][token]
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     // the short tiles of the first ones had finished: a first chunk of 4,096 rows took 495 us instead of 300), and the
     // KV head is the fast index, so that with eight KV heads every XCD reads the cache of one.
     const unsigned int kvh = blockIdx.x % p.num_kv_heads;
-    const unsigned int rows_per_wg = max(1u, 256u / p.group);
+    const unsigned int rows_per_wg = max(1u, (128u * CT) / p.group);
     const unsigned int row0 = (gridDim.x / p.num_kv_heads - 1u - blockIdx.x / p.num_kv_heads) * rows_per_wg;
     const unsigned int cols_used = rows_per_wg * p.group;
 
@@ -342,7 +350,12 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     }
 
     // first token some column of the wave cannot see any more / last token some column does not see yet (wave-uniform)
-    unsigned int wave_min_hi = min(vis_hi[0], vis_hi[1]), wave_max_lo = max(vis_lo[0], vis_lo[1]);
+    unsigned int wave_min_hi = vis_hi[0], wave_max_lo = vis_lo[0];
+#pragma unroll
+    for (int ct = 1; ct < kColTiles; ++ct) {
+        wave_min_hi = min(wave_min_hi, vis_hi[ct]);
+        wave_max_lo = max(wave_max_lo, vis_lo[ct]);
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         wave_min_hi = min(wave_min_hi, (unsigned int)__shfl_xor((int)wave_min_hi, off));
@@ -1192,6 +1205,23 @@ template <int D, int KV, int SDT> static hipError_t launch_prefill_tiles(const G
 
 } // namespace
 
+bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned int window, unsigned int num_heads, unsigned int num_kv_heads,
+                            unsigned int head_dim, int kv_format, int scale_dtype)
+{
+    if (kv_format != 0 || head_dim != (unsigned int)kD || scale_dtype == 2 || num_kv_heads == 0) {
+        return false; // not gqa_prefill_q8's geometry
+    }
+    const unsigned int group = num_heads / num_kv_heads;
+    if (group == 0 || group > 128u || window != 0u) {
+        return false;
+    }
+    const unsigned int full_rows = 256u / group;
+    const unsigned long long full_tiles = ((unsigned long long)rows + full_rows - 1) / full_rows * num_kv_heads;
+    // measured on 32 query / 8 KV heads: 2,048 rows at position 0 140 -> 122 us, 256 rows 40 -> 26 us; at position 1,024
+    // (ranges 1 : 3) the half tiles' dearer steps cost what the evening out gains, 190 -> 200 us
+    return full_tiles <= kComputeUnitsPrefill && (unsigned long long)position * 4u <= rows;
+}
+
 hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream)
 {
     if (kv_format == 1) { // f16 rows
@@ -1220,22 +1250,34 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
     if (scale_dtype == 2) { // f32 scales at head_dim 128: the tile kernel (gqa_prefill_q8 reads 16-bit scales)
         return launch_prefill_tiles<128, 0, 2>(p, stream);
     }
-    const unsigned int rows_per_wg = p.group >= 256u ? 1u : 256u / p.group;
+    const unsigned int full_rows = p.group >= 256u ? 1u : 256u / p.group;
+    const bool halves = gqa_prefill_half_tiles(p.rows, p.position, p.window, p.num_heads, p.num_kv_heads, p.head_dim, kv_format, scale_dtype);
+    const unsigned int rows_per_wg = halves ? (p.group >= 128u ? 1u : 128u / p.group) : full_rows;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg * p.num_kv_heads, 1, p.max_chunks > 1u ? p.max_chunks : 1u);
     const bool cap = p.softcap > 0.0f;
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.table != nullptr;
     const dim3 block(kThreads);
+    auto launch = [&](auto sdt, auto softcap, auto table_pow2) {
+        constexpr int S = decltype(sdt)::value;
+        constexpr bool C = decltype(softcap)::value, P = decltype(table_pow2)::value;
+        if (halves) {
+            gqa_prefill_q8<S, C, P, 1><<<grid, block, 0, stream>>>(p);
+        } else {
+            gqa_prefill_q8<S, C, P, 2><<<grid, block, 0, stream>>>(p);
+        }
+    };
+    using std::integral_constant;
     if (scale_dtype == 0) {
         if (cap) {
-            pow2 ? gqa_prefill_q8<0, true, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<0, true, false><<<grid, block, 0, stream>>>(p);
+            pow2 ? launch(integral_constant<int, 0>{}, std::true_type{}, std::true_type{}) : launch(integral_constant<int, 0>{}, std::true_type{}, std::false_type{});
         } else {
-            pow2 ? gqa_prefill_q8<0, false, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<0, false, false><<<grid, block, 0, stream>>>(p);
+            pow2 ? launch(integral_constant<int, 0>{}, std::false_type{}, std::true_type{}) : launch(integral_constant<int, 0>{}, std::false_type{}, std::false_type{});
         }
     } else {
         if (cap) {
-            pow2 ? gqa_prefill_q8<1, true, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<1, true, false><<<grid, block, 0, stream>>>(p);
+            pow2 ? launch(integral_constant<int, 1>{}, std::true_type{}, std::true_type{}) : launch(integral_constant<int, 1>{}, std::true_type{}, std::false_type{});
         } else {
-            pow2 ? gqa_prefill_q8<1, false, true><<<grid, block, 0, stream>>>(p) : gqa_prefill_q8<1, false, false><<<grid, block, 0, stream>>>(p);
+            pow2 ? launch(integral_constant<int, 1>{}, std::false_type{}, std::true_type{}) : launch(integral_constant<int, 1>{}, std::false_type{}, std::false_type{});
         }
     }
     return hipGetLastError();

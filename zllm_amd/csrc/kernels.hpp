@@ -162,6 +162,13 @@ struct MlaDecodeParams {
     unsigned int query_rows;
 };
 
+// Chunked prefill over Q8g64 with 16-bit scales at head_dim 128: whether the chunk runs row tiles of 128 (row, head) pairs
+// instead of 256.  True for a chunk that is much longer than what lies before it (its row tiles' ranges grow from almost
+// nothing to the whole chunk) when the full-size tiles would be at most one workgroup per compute unit: twice as many
+// workgroups, handed out longest first, even the launch out.  The split planner and the launcher both ask.
+bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned int window, unsigned int num_heads, unsigned int num_kv_heads,
+                            unsigned int head_dim, int kv_format, int scale_dtype);
+
 // KV heads (= waves) per GQA decode workgroup for a head dimension.
 unsigned int gqa_decode_max_waves(unsigned int head_dim);
 unsigned int gqa_decode_items_per_group(unsigned int head_dim, unsigned int num_kv_heads);
