@@ -79,8 +79,8 @@ def prefill_chunk_cases(args):
         rows = torch.randn((total, cols), generator=gen, device="cuda").to(torch.bfloat16)
         ops.q8g64_append(rows, planes[name + "c"], planes[name + "s"], table, 0, bt, capi.QUANT_METAL_GQA)
     lib = capi.load()
-    for prefix in (2048, 32768):
-        for chunk in (1, 2, 4, 8, 64, 256, 512, 2048):
+    for prefix in (0, 2048, 32768):  # position 0: a prompt's first chunk, whose row tiles' ranges grow from nothing
+        for chunk in (1, 2, 4, 8, 64, 256, 512, 2048) if prefix else (128, 512, 2048):
             q = torch.randn((chunk, hq * d), generator=gen, device="cuda").to(torch.bfloat16)
             times = {}
             for label, workspace in (("with_workspace", True), ("without_workspace", False)):
