@@ -1057,7 +1057,7 @@ static uint64_t prefill_decode_route_bytes(const zllm_gqa_prefill_args* a)
 // decode route's workspace such a chunk runs as decode items instead, each row re-reading the cache.  Measured on 32
 // query / 8 KV heads of 128 (us, decode items against the chunk kernel with KV splits): one row over 32 K tokens 24 / 71,
 // two 33 / 73, four 56 / 74, eight 104 / 78; eight rows over 2 K tokens 20 / 33 -- about 15 us + 0.34 ns per row and
-// token against 28 us + 1.5 ns per token.
+// token against 28 us + 1.5 ns per token (0.8 ns with half-size row tiles).
 static bool few_rows_as_decode_items(const zllm_gqa_prefill_args* a)
 {
     if (a->rows > 16u) {
@@ -1067,7 +1067,11 @@ static bool few_rows_as_decode_items(const zllm_gqa_prefill_args* a)
     if (a->window != 0 && tokens > a->window) {
         tokens = a->window;
     }
-    return (uint64_t)a->rows * tokens * 34u < tokens * 150u + 1300000u;
+    // the chunk kernel's half-size row tiles (Q8g64 with 16-bit scales at head_dim 128, a chunk whose pairs fit one) walk
+    // a key in 0.8 ns: eight rows over 32 K tokens 54 us, where they would cost 104 as decode items
+    const bool half_tiles = zllm::gqa_prefill_half_tiles(a->rows, a->position, a->window, a->num_heads, a->num_kv_heads, a->head_dim, a->kv_format,
+                                                         a->scale_dtype);
+    return (uint64_t)a->rows * tokens * 34u < tokens * (half_tiles ? 80u : 150u) + 1300000u;
 }
 
 uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* a)

@@ -1212,7 +1212,13 @@ bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned i
         return false; // not gqa_prefill_q8's geometry
     }
     const unsigned int group = num_heads / num_kv_heads;
-    if (group == 0 || group > 128u || window != 0u) {
+    if (group == 0 || group > 128u) {
+        return false;
+    }
+    if ((unsigned long long)rows * group <= 128u) {
+        return true; // the whole chunk fits a half tile: a full one would be half empty at least
+    }
+    if (window != 0u) {
         return false;
     }
     const unsigned int full_rows = 256u / group;

@@ -163,7 +163,7 @@ struct MlaDecodeParams {
 };
 
 // Chunked prefill over Q8g64 with 16-bit scales at head_dim 128: whether the chunk runs row tiles of 128 (row, head) pairs
-// instead of 256.  True for a chunk that is much longer than what lies before it (its row tiles' ranges grow from almost
+// instead of 256.  True for a chunk whose pairs all fit the smaller tile, and for one that is much longer than what lies before it (its row tiles' ranges grow from almost
 // nothing to the whole chunk) when the full-size tiles would be at most one workgroup per compute unit: twice as many
 // workgroups, handed out longest first, even the launch out.  The split planner and the launcher both ask.
 bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned int window, unsigned int num_heads, unsigned int num_kv_heads,
