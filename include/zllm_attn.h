@@ -316,7 +316,7 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * (parts of a tile's visible range, combined like a decode call's splits) when the
  * caller passes zllm_attn_gqa_prefill_workspace_bytes of 16-byte aligned workspace
  * for their records, and runs unsplit (same results, one workgroup walking the whole
- * prefix per tile) when it passes none or less.  A chunk of a few rows (one to four
+ * prefix per tile) when it passes none or less.  A chunk of a few rows (one to three
  * over a long prefix, up to sixteen over a short one) is a decode step in all but name
  * -- the reference decodes through this path with one row
  * (src/backend/rocm/attention.rs:2202-2231) -- and, given that workspace, runs every
