@@ -149,6 +149,7 @@ struct MlaDecodeParams {
     float* stats;             // [batch][max_chunks][heads][2]
     float* weighted;          // [batch][heads][latent_dim]
     unsigned int batch, heads, q_head_dim, kv_head_dim, latent_dim, rope_dim, nope_dim, value_dim;
+    unsigned int column_split; // mla_absorb_mfma: waves that share a block of sixteen rows (set by the launcher)
     unsigned int table_stride, block_tokens, block_shift;
     unsigned int chunk_tokens, max_chunks;
     float score_scale;

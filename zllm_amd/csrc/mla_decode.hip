@@ -239,86 +239,102 @@ constexpr int kAbsorbNope = 128;
 
 // absorbed^T[n, row] = sum_k W_k[k, n] q[row, k].  A operand: W_k^T fragments through ds_read_b64_tr_b16 (lane (m, j) gets
 // column n = 16 nt + m at k = 4 j .. 4 j + 3 and 16 + 4 j .. 16 + 4 j + 3 of a 32-k step); B operand: the query row m at
-// the same k.  grid = (heads, workgroups per head), 256 threads; a workgroup stages the head's weights once and takes
-// blocks of sixteen rows in turn; wave w owns latent columns [128 w, 128 w + 128).
-__global__ __launch_bounds__(256) void mla_absorb_mfma(MlaDecodeParams p)
+// the same k.  grid = (heads, workgroups per head), 4 or 16 waves; a workgroup stages the head's weights once and its
+// waves take blocks of sixteen rows in turn, a wave (or the 2 to 16 waves that share a block) all 512 latent columns.
+template <int WAVES> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mfma(MlaDecodeParams p)
 {
     __shared__ __align__(16) unsigned char w_lds[kAbsorbNope * kAbsorbRowBytes];
     const unsigned int head = blockIdx.x;
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
     const unsigned int wave = tid >> 6;
+    constexpr unsigned int waves = WAVES;
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     {
         const unsigned char* w = (const unsigned char*)(p.kv_b + (size_t)head * p.kv_head_dim * kLatent);
-        u32x4 staged[32];
+        // 8,192 16-byte chunks (chunk c % 64 of weight row c / 64), all of a thread's requested before any is stored
+        constexpr int kPerThread = kAbsorbNope * 64 / (64 * WAVES);
+        u32x4 staged[kPerThread];
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const unsigned int c = tid + 256u * i; // 16-byte chunk c % 64 of weight row c / 64
+        for (int i = 0; i < kPerThread; ++i) {
+            const unsigned int c = tid + 64u * WAVES * i;
             staged[i] = *(const u32x4*)(w + (size_t)c * 16u);
         }
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const unsigned int c = tid + 256u * i;
+        for (int i = 0; i < kPerThread; ++i) {
+            const unsigned int c = tid + 64u * WAVES * i;
             *(u32x4*)(w_lds + (c >> 6) * kAbsorbRowBytes + (c & 63u) * 16u) = staged[i];
         }
     }
     __syncthreads();
-    // the staged weights serve every block of sixteen rows this workgroup takes: blocks blockIdx.y, + gridDim.y, ...
+    // The staged weights serve every block of sixteen rows the workgroup takes.  The weights leave room for one workgroup
+    // per compute unit, so its waves are all the loads a compute unit has in flight: four waves walking the blocks one
+    // after the other ran the stage at 1.9 TB/s.  Every wave takes blocks of its own, all 512 latent columns of them; when
+    // the workgroup has fewer blocks than waves, 2, 4, 8 or 16 waves share a block and split its columns.
+    const unsigned int share = p.column_split;           // waves per block
+    const unsigned int slots = waves / share;            // blocks the workgroup has in flight
+    const unsigned int tiles = 32u / share;              // 16-column tiles of a wave
+    const unsigned int tile0 = (wave % share) * tiles;
     const unsigned char* frag_at = w_lds + (4u * j + (m >> 2)) * kAbsorbRowBytes + (m & 3u) * 8u;
-    for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
-    const unsigned int row = min(row0 + m, p.batch - 1u);
-    const size_t q_base = ((size_t)row * p.heads + head) * p.q_head_dim;
-    // four consecutive query elements per load, rounded to bf16: the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
-    auto four_as_bf16 = [&](size_t at) __attribute__((always_inline)) -> u32x2 {
-        if (p.q_dtype == 1) {
-            return *(const u32x2*)((const unsigned short*)p.q + at);
-        }
-        if (p.q_dtype == 0) {
-            const f32x4 x = *(const f32x4*)((const float*)p.q + at);
-            return u32x2{pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])};
-        }
-        const u32x2 h = *(const u32x2*)((const unsigned short*)p.q + at);
-        return u32x2{pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[0] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[0] >> 16))),
-                     pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[1] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[1] >> 16)))};
-    };
-    Frag qf[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        const u32x2 lo = four_as_bf16(q_base + ks * 32u + 4u * j), hi = four_as_bf16(q_base + ks * 32u + 16u + 4u * j);
-        qf[ks].u = u32x4{lo[0], lo[1], hi[0], hi[1]};
-    }
-    // the rope part of the sixteen rows is a copy: 16 x 64 elements over 256 threads
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const unsigned int e = tid + 256u * i;
-        const unsigned int r = row0 + (e >> 6), c = e & 63u;
-        if (r < p.batch) {
-            const float x = load_as_f32(p.q, ((size_t)r * p.heads + head) * p.q_head_dim + kAbsorbNope + c, p.q_dtype);
-            p.absorbed[((size_t)r * p.heads + head) * (kLatent + kRope) + kLatent + c] = f32_to_bf16_bits(x);
-        }
-    }
-    unsigned short* qa = p.absorbed + ((size_t)(row0 + m) * p.heads + head) * (kLatent + kRope) + 4u * j;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const unsigned int nt = wave * 8u + t;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned int row0 = (blockIdx.y * slots + wave / share) * 16u; row0 < p.batch; row0 += gridDim.y * slots * 16u) {
+        const unsigned int row = min(row0 + m, p.batch - 1u);
+        const size_t q_base = ((size_t)row * p.heads + head) * p.q_head_dim;
+        // four consecutive query elements per load, rounded to bf16: the oracle takes a bf16 query (src/kernel/cpu/mla.rs:958-961)
+        auto four_as_bf16 = [&](size_t at) __attribute__((always_inline)) -> u32x2 {
+            if (p.q_dtype == 1) {
+                return *(const u32x2*)((const unsigned short*)p.q + at);
+            }
+            if (p.q_dtype == 0) {
+                const f32x4 x = *(const f32x4*)((const float*)p.q + at);
+                return u32x2{pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])};
+            }
+            const u32x2 h = *(const u32x2*)((const unsigned short*)p.q + at);
+            return u32x2{pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[0] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[0] >> 16))),
+                         pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[1] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[1] >> 16)))};
+        };
+        Frag qf[4];
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            union {
-                s16x4 s[2];
-                bf16x8 b;
-            } wf;
-            const unsigned char* at = frag_at + ks * 32 * kAbsorbRowBytes + nt * 32u;
-            wf.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-            wf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kAbsorbRowBytes));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, qf[ks].b, acc, 0, 0, 0);
+            const u32x2 lo = four_as_bf16(q_base + ks * 32u + 4u * j), hi = four_as_bf16(q_base + ks * 32u + 16u + 4u * j);
+            qf[ks].u = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
-        if (row0 + m < p.batch) { // lane (m, j) holds latent columns 16 nt + 4 j .. + 4 of row m
-            *(u32x2*)(qa + nt * 16u) = u32x2{pack_bf16_rne(acc[0], acc[1]), pack_bf16_rne(acc[2], acc[3])};
+        // the rope part of the sixteen rows is a copy: lane = column, one row a pass, the rows dealt out to the block's waves
+        {
+            const unsigned int part = wave % share;
+            float rope_in[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const unsigned int r = min(row0 + i, p.batch - 1u);
+                if ((i & (share - 1u)) == part) {
+                    rope_in[i] = load_as_f32(p.q, ((size_t)r * p.heads + head) * p.q_head_dim + kAbsorbNope + lane, p.q_dtype);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                if ((i & (share - 1u)) == part && row0 + i < p.batch) {
+                    p.absorbed[((size_t)(row0 + i) * p.heads + head) * (kLatent + kRope) + kLatent + lane] = f32_to_bf16_bits(rope_in[i]);
+                }
+            }
         }
-    }
+        unsigned short* qa = p.absorbed + ((size_t)(row0 + m) * p.heads + head) * (kLatent + kRope) + 4u * j;
+        for (unsigned int nt = tile0; nt < tile0 + tiles; ++nt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                union {
+                    s16x4 s[2];
+                    bf16x8 b;
+                } wf;
+                const unsigned char* at = frag_at + ks * 32 * kAbsorbRowBytes + nt * 32u;
+                wf.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
+                wf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kAbsorbRowBytes));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, qf[ks].b, acc, 0, 0, 0);
+            }
+            if (row0 + m < p.batch) { // lane (m, j) holds latent columns 16 nt + 4 j .. + 4 of row m
+                *(u32x2*)(qa + nt * 16u) = u32x2{pack_bf16_rne(acc[0], acc[1]), pack_bf16_rne(acc[2], acc[3])};
+            }
+        }
     }
 }
 
@@ -1579,9 +1595,11 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
 // grid = (heads, workgroups per head), 512 threads; a workgroup takes blocks of sixteen rows in turn.  The merge is a chain of round trips to memory, so it is spread as wide
 // as the workgroup goes: a thread folds the splits of four latent columns of four rows, the four rows' records requested
 // together, four splits a trip.  Wave w then owns value columns [16 w, 16 w + 16).
-// MERGED: the rows were merged by the split-merge kernel and lie in the workspace (p.weighted); the workgroup only projects.
+// MODE 0: the workgroup folds its rows' split records.  MODE 1: the rows were merged by the split-merge kernel and lie in
+// the workspace (p.weighted).  MODE 2: the plan has one record a row (a long chunk without KV splits), which only wants
+// its sum divided out.  Modes 1 and 2 leave the registers for two workgroups per compute unit.
 constexpr int kMergedStride = kLatent + 4; // floats: sixteen rows' fragments start in different banks
-template <bool MERGED> __global__ __launch_bounds__(512) void mla_merge_project_mfma(MlaDecodeParams p)
+template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfma(MlaDecodeParams p)
 {
     __shared__ __align__(16) float merged[16][kMergedStride];
     const unsigned int head = blockIdx.x;
@@ -1601,97 +1619,120 @@ template <bool MERGED> __global__ __launch_bounds__(512) void mla_merge_project_
             wf[ks].u = *(const u32x4*)(w_head + (size_t)v * kLatent + ks * 32 + 8u * j);
         }
     }
-    for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
-    if constexpr (MERGED) {
-        const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
-        f32x4 row[4];
+    // the merged values of this thread's four rows (rb, rb + 4, rb + 8, rb + 12 of the block at row0) and four columns
+    auto fetch_rows = [&](unsigned int row0, f32x4 (&out)[4]) __attribute__((always_inline)) {
+        if constexpr (MODE == 1) {
+            const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
+            f32x4 row[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
-            row[u] = *(const f32x4*)(p.weighted + ((size_t)b * p.heads + head) * kLatent + quad * 4u);
-        }
+            for (int u = 0; u < 4; ++u) {
+                const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+                row[u] = *(const f32x4*)(p.weighted + ((size_t)b * p.heads + head) * kLatent + quad * 4u);
+            }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            *(f32x4*)(&merged[rb + 4u * u][quad * 4u]) = row[u];
-        }
-    } else {
-        const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
-        const float* stats[4];
-        const float* partial[4];
-        unsigned int chunks[4];
-        float mx[4], l[4];
-        f32x4 acc[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
-            unsigned int seq;
-            const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
-            chunks[u] = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
-            stats[u] = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
-            partial[u] = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
-            mx[u] = kNegInf;
-            l[u] = 0.0f;
-            acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-        const size_t stat_stride = (size_t)p.heads * 2;
-        const size_t partial_stride = (size_t)p.heads * kLatent;
-        const unsigned int most = max(max(chunks[0], chunks[1]), max(chunks[2], chunks[3]));
-        if (p.max_chunks == 1u) { // a long chunk leaves one record a row (no KV splits): nothing to fold
+            for (int u = 0; u < 4; ++u) {
+                out[u] = row[u];
+            }
+        } else if constexpr (MODE == 2) {
+            const unsigned int rb = tid >> 7;
             float2 st[4];
             f32x4 part[4];
+            unsigned int len[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                st[u] = *(const float2*)stats[u];
-                part[u] = *(const f32x4*)partial[u];
+                const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+                unsigned int seq;
+                len[u] = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
+                st[u] = *(const float2*)(p.stats + ((size_t)b * p.heads + head) * 2);
+                part[u] = *(const f32x4*)(p.partial + ((size_t)b * p.heads + head) * kLatent + quad * 4u);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                if (chunks[u] > 0u && st[u].y > 0.0f) {
-                    acc[u] = part[u];
-                    l[u] = st[u].y;
+                f32x4 result = {0.f, 0.f, 0.f, 0.f};
+                if (len[u] > 0u && st[u].y > 0.0f && st[u].y < __builtin_inff()) {
+                    result = part[u] * (1.0f / st[u].y);
                 }
+                out[u] = result;
             }
-        }
-        for (unsigned int c0 = 0; p.max_chunks > 1u && c0 < most; c0 += 4u) {
-            float2 st[4][4];
-            f32x4 part[4][4];
+        } else {
+            const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
+            const float* stats[4];
+            const float* partial[4];
+            unsigned int chunks[4];
+            float mx[4], l[4];
+            f32x4 acc[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
+                const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+                unsigned int seq;
+                const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
+                chunks[u] = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+                stats[u] = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+                partial[u] = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+                mx[u] = kNegInf;
+                l[u] = 0.0f;
+                acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            const size_t stat_stride = (size_t)p.heads * 2;
+            const size_t partial_stride = (size_t)p.heads * kLatent;
+            const unsigned int most = max(max(chunks[0], chunks[1]), max(chunks[2], chunks[3]));
+            for (unsigned int c0 = 0; c0 < most; c0 += 4u) {
+                float2 st[4][4];
+                f32x4 part[4][4];
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const unsigned int c = min(c0 + v, max(chunks[u], 1u) - 1u);
-                    st[u][v] = *(const float2*)(stats[u] + c * stat_stride);
-                    part[u][v] = *(const f32x4*)(partial[u] + c * partial_stride);
+                for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const unsigned int c = min(c0 + v, max(chunks[u], 1u) - 1u);
+                        st[u][v] = *(const float2*)(stats[u] + c * stat_stride);
+                        part[u][v] = *(const f32x4*)(partial[u] + c * partial_stride);
+                    }
                 }
-            }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < 4; ++u) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const bool live = c0 + v < chunks[u];
-                    const float cl = live ? st[u][v].y : 0.0f;
-                    if (cl > 0.0f) {
-                        const float cm = st[u][v].x;
-                        const float nm = fmaxf(mx[u], cm);
-                        const float a = __builtin_amdgcn_exp2f(mx[u] - nm);
-                        const float w = __builtin_amdgcn_exp2f(cm - nm);
-                        acc[u] = acc[u] * a + part[u][v] * w;
-                        l[u] = l[u] * a + cl * w;
-                        mx[u] = nm;
+                    for (int v = 0; v < 4; ++v) {
+                        const bool live = c0 + v < chunks[u];
+                        const float cl = live ? st[u][v].y : 0.0f;
+                        if (cl > 0.0f) {
+                            const float cm = st[u][v].x;
+                            const float nm = fmaxf(mx[u], cm);
+                            const float a = __builtin_amdgcn_exp2f(mx[u] - nm);
+                            const float w = __builtin_amdgcn_exp2f(cm - nm);
+                            acc[u] = acc[u] * a + part[u][v] * w;
+                            l[u] = l[u] * a + cl * w;
+                            mx[u] = nm;
+                        }
                     }
                 }
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                f32x4 result = {0.f, 0.f, 0.f, 0.f};
+                if (l[u] > 0.0f && l[u] < __builtin_inff()) {
+                    result = acc[u] * (1.0f / l[u]);
+                }
+                out[u] = result;
+            }
         }
+    };
+    // The next block's rows are requested before the projection of this one, so that the round trips to memory (one for
+    // merged rows, several for split records) run under the matrix work instead of between two barriers: a 2,048-row
+    // chunk of one record a row spent 3 us a block waiting, 408 us in all.
+    f32x4 next_rows[4];
+    fetch_rows(blockIdx.y * 16u, next_rows);
+    for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
+    {
+        const unsigned int rb = tid >> 7;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            f32x4 result = {0.f, 0.f, 0.f, 0.f};
-            if (l[u] > 0.0f && l[u] < __builtin_inff()) {
-                result = acc[u] * (1.0f / l[u]);
-            }
-            *(f32x4*)(&merged[rb + 4u * u][quad * 4u]) = result;
+            *(f32x4*)(&merged[rb + 4u * u][quad * 4u]) = next_rows[u];
         }
     }
     __syncthreads();
+    if (row0 + gridDim.y * 16u < p.batch) {
+        fetch_rows(row0 + gridDim.y * 16u, next_rows);
+    }
     // ---- projection
     const unsigned int out_stride = p.out_compact ? p.value_dim : p.q_head_dim;
     f32x4 out_acc = {0.f, 0.f, 0.f, 0.f};
@@ -1779,7 +1820,21 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         // Eight rows per workgroup share every weight load, and the workgroup then runs eight rows' sums: measured 28 us from
         // 16 rows up to a few hundred, against 13 us (15 rows) to 27 us (32 rows) for one workgroup per row
         if (p.batch >= 16u && p.nope_dim == (unsigned int)kAbsorbNope && (p.q_head_dim & 3u) == 0) { // sixteen rows a workgroup, on the matrix cores
-            mla_absorb_mfma<<<dim3(p.heads, row_block_groups(p)), dim3(256), 0, stream>>>(p);
+            // four waves for a decode batch, sixteen for a chunk (33 against 61 us on 512 rows of 128 heads; on 16 to 64 rows
+            // the larger workgroup costs 4 us); as many waves share a block of sixteen rows as keeps every wave busy
+            MlaDecodeParams q = p;
+            const unsigned int groups = row_block_groups(p);
+            const unsigned int blocks_here = ((p.batch + 15u) / 16u + groups - 1u) / groups;
+            const unsigned int waves = p.batch >= 128u ? 16u : 4u;
+            q.column_split = 1u;
+            while (q.column_split < waves && blocks_here * q.column_split < waves) {
+                q.column_split *= 2u;
+            }
+            if (waves == 16u) {
+                mla_absorb_mfma<16><<<dim3(p.heads, groups), dim3(1024), 0, stream>>>(q);
+            } else {
+                mla_absorb_mfma<4><<<dim3(p.heads, groups), dim3(256), 0, stream>>>(q);
+            }
         } else if (p.batch >= 32u && p.nope_dim <= 256u) {
             mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
         } else {
@@ -1823,9 +1878,14 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
                 if (err != hipSuccess) {
                     return err;
                 }
-                mla_merge_project_mfma<true><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+                mla_merge_project_mfma<1><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+            } else if (p.max_chunks == 1u) {
+                // one record a row: two workgroups fit a compute unit, so twice the workgroups of the usual round
+                const unsigned int blocks = (p.batch + 15u) / 16u;
+                const unsigned int groups = 2u * row_block_groups(p);
+                mla_merge_project_mfma<2><<<dim3(p.heads, groups < blocks ? groups : blocks), dim3(512), 0, stream>>>(p);
             } else {
-                mla_merge_project_mfma<false><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+                mla_merge_project_mfma<0><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
             }
         } else if (p.batch >= 16u) { // eight rows share every weight load of the projection
             mla_merge_project_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
