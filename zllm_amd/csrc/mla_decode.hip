@@ -1598,10 +1598,11 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
 // MODE 0: the workgroup folds its rows' split records.  MODE 1: the rows were merged by the split-merge kernel and lie in
 // the workspace (p.weighted).  MODE 2: the plan has one record a row (a long chunk without KV splits), which only wants
 // its sum divided out.  Modes 1 and 2 leave the registers for two workgroups per compute unit.
-constexpr int kMergedStride = kLatent + 4; // floats: sixteen rows' fragments start in different banks
+constexpr int kMergedStride = kLatent + 8; // bf16 elements: sixteen rows' 16-byte fragments start in different banks
 template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfma(MlaDecodeParams p)
 {
-    __shared__ __align__(16) float merged[16][kMergedStride];
+    // the merged rows as two bf16 terms (value = hi + lo keeps 16 bits of the f32), split once by the thread that merged them
+    __shared__ __align__(16) unsigned short merged_hi[16][kMergedStride], merged_lo[16][kMergedStride];
     const unsigned int head = blockIdx.x;
     const unsigned int tid = threadIdx.x;
     const unsigned int quad = tid & 127u;
@@ -1726,7 +1727,12 @@ template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfm
         const unsigned int rb = tid >> 7;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            *(f32x4*)(&merged[rb + 4u * u][quad * 4u]) = next_rows[u];
+            const f32x4 x = next_rows[u];
+            const u32x2 hi = {pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])};
+            const u32x2 lo = {pack_bf16_rne(x[0] - __uint_as_float(hi[0] << 16), x[1] - __uint_as_float(hi[0] & 0xffff0000u)),
+                              pack_bf16_rne(x[2] - __uint_as_float(hi[1] << 16), x[3] - __uint_as_float(hi[1] & 0xffff0000u))};
+            *(u32x2*)(&merged_hi[rb + 4u * u][quad * 4u]) = hi;
+            *(u32x2*)(&merged_lo[rb + 4u * u][quad * 4u]) = lo;
         }
     }
     __syncthreads();
@@ -1738,17 +1744,9 @@ template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfm
     f32x4 out_acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < 16; ++ks) {
-        const float* x = &merged[m][ks * 32 + 8u * j];
-        const f32x4 x0 = *(const f32x4*)x, x1 = *(const f32x4*)(x + 4);
         Frag hi, lo;
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const float a0 = x0[2 * e], a1 = x0[2 * e + 1], b0 = x1[2 * e], b1 = x1[2 * e + 1];
-            hi.u[e] = pack_bf16_rne(a0, a1);
-            hi.u[2 + e] = pack_bf16_rne(b0, b1);
-            lo.u[e] = pack_bf16_rne(a0 - __uint_as_float(hi.u[e] << 16), a1 - __uint_as_float(hi.u[e] & 0xffff0000u));
-            lo.u[2 + e] = pack_bf16_rne(b0 - __uint_as_float(hi.u[2 + e] << 16), b1 - __uint_as_float(hi.u[2 + e] & 0xffff0000u));
-        }
+        hi.u = *(const u32x4*)(&merged_hi[m][ks * 32 + 8u * j]);
+        lo.u = *(const u32x4*)(&merged_lo[m][ks * 32 + 8u * j]);
         out_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].b, hi.b, out_acc, 0, 0, 0);
         out_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].b, lo.b, out_acc, 0, 0, 0);
     }
