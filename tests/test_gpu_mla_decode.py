@@ -470,6 +470,22 @@ def test_mla_batched_decode_on_the_matrix_core_stages():
     assert np.array_equal(strided.reshape(got.shape), got)
 
 
+def test_mla_matrix_core_stages_at_192_query_and_256_value_columns():
+    """The reference's decode test has 192 query columns next to the rope and 256 value columns
+    (src/kernel/rocm/hip/attention/paged_mla.rs:6226-6233).  The matrix-core absorb then stages half the latent columns
+    a workgroup, and the projection runs sixteen waves: a decode batch of 20 rows (split merge, then projection from
+    merged rows), a chunk of 40 rows (one record a row) and a chunk of 200 rows (sixteen-wave absorb)."""
+    case = make_mla_case(301, [int(x) for x in np.random.default_rng(301).integers(1, 700, size=20)], 16, nope=192, value=256)
+    want_f, _ = oracle_mla(case)
+    got = run_mla(case).cpu().numpy()
+    print("mla 192/256 batch", assert_attention_close(got.reshape(want_f.shape), want_f, "MLA 192/256 batch of 20"))
+    for rows, lens in ((40, [300, 120]), (200, [260])):
+        chunk = make_mla_chunk_case(302 + rows, lens, rows, 16, nope=192, value=256)
+        want_c, _ = oracle_mla_chunk(chunk)
+        got_c = run_mla_chunk(chunk).cpu().numpy()
+        print("mla 192/256 chunk", rows, assert_attention_close(got_c.reshape(want_c.shape), want_c, f"MLA 192/256 chunk of {rows}"))
+
+
 def test_mla_chunk_query_types_on_the_matrix_core_absorb():
     case = make_mla_chunk_case(9, [300, 120], 20, 16)
     want_f, _ = oracle_mla_chunk(case)

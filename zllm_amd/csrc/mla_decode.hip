@@ -232,18 +232,22 @@ template <int R> __global__ __launch_bounds__(256) void mla_absorb_rows(MlaDecod
 // Products of bf16 values are exact in f32 and only the order of the f32 sum differs from the oracle's, so an absorbed
 // query differs from the bit-exact one by a bf16 step in a few elements out of a million.
 
-// W_k[head] (nope x 512 bf16) lies in LDS as in memory, rows padded by 16 bytes: the sixteen rows a transposed read
-// touches then start in different banks.
-constexpr int kAbsorbRowBytes = kLatent * 2 + 16;
-constexpr int kAbsorbNope = 128;
+// W_k[head] (nope rows of bf16) lies in LDS as in memory, rows padded by 16 bytes: the sixteen rows a transposed read
+// touches then start in different banks.  128 query columns x 512 latent columns are 133 KB; 192 query columns (the
+// reference's decode test, src/kernel/rocm/hip/attention/paged_mla.rs:6226-6233) x 256, half the latent columns, 101 KB.
 
 // absorbed^T[n, row] = sum_k W_k[k, n] q[row, k].  A operand: W_k^T fragments through ds_read_b64_tr_b16 (lane (m, j) gets
 // column n = 16 nt + m at k = 4 j .. 4 j + 3 and 16 + 4 j .. 16 + 4 j + 3 of a 32-k step); B operand: the query row m at
 // the same k.  grid = (heads, workgroups per head), 4 or 16 waves; a workgroup stages the head's weights once and its
 // waves take blocks of sixteen rows in turn, a wave (or the 2 to 16 waves that share a block) all 512 latent columns.
-template <int WAVES> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mfma(MlaDecodeParams p)
+// NOPE query columns and COLS latent columns a workgroup: 128 x 512, or 192 x 256 with the two column halves in
+// workgroups of their own (blockIdx.z), which is what fits the LDS.
+template <int WAVES, int NOPE, int COLS> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mfma(MlaDecodeParams p)
 {
-    __shared__ __align__(16) unsigned char w_lds[kAbsorbNope * kAbsorbRowBytes];
+    constexpr int kRowBytes = COLS * 2 + 16; // LDS bytes of one weight row: sixteen rows start in different banks
+    constexpr int kRowChunks = COLS / 8;     // its 16-byte chunks
+    const unsigned int col0 = blockIdx.z * COLS;
+    __shared__ __align__(16) unsigned char w_lds[NOPE * kRowBytes];
     const unsigned int head = blockIdx.x;
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -252,19 +256,21 @@ template <int WAVES> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mf
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
     {
-        const unsigned char* w = (const unsigned char*)(p.kv_b + (size_t)head * p.kv_head_dim * kLatent);
-        // 8,192 16-byte chunks (chunk c % 64 of weight row c / 64), all of a thread's requested before any is stored
-        constexpr int kPerThread = kAbsorbNope * 64 / (64 * WAVES);
+        const unsigned char* w = (const unsigned char*)(p.kv_b + (size_t)head * p.kv_head_dim * kLatent + col0);
+        // NOPE * COLS / 8 16-byte chunks (chunk c % kRowChunks of weight row c / kRowChunks), all of a thread's requested
+        // before any is stored
+        constexpr int kPerThread = NOPE * kRowChunks / (64 * WAVES);
+        static_assert(NOPE * kRowChunks % (64 * WAVES) == 0, "whole chunks per thread");
         u32x4 staged[kPerThread];
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
             const unsigned int c = tid + 64u * WAVES * i;
-            staged[i] = *(const u32x4*)(w + (size_t)c * 16u);
+            staged[i] = *(const u32x4*)(w + (size_t)(c / kRowChunks) * (kLatent * 2) + (c % kRowChunks) * 16u);
         }
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
             const unsigned int c = tid + 64u * WAVES * i;
-            *(u32x4*)(w_lds + (c >> 6) * kAbsorbRowBytes + (c & 63u) * 16u) = staged[i];
+            *(u32x4*)(w_lds + (c / kRowChunks) * kRowBytes + (c % kRowChunks) * 16u) = staged[i];
         }
     }
     __syncthreads();
@@ -274,9 +280,9 @@ template <int WAVES> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mf
     // the workgroup has fewer blocks than waves, 2, 4, 8 or 16 waves share a block and split its columns.
     const unsigned int share = p.column_split;           // waves per block
     const unsigned int slots = waves / share;            // blocks the workgroup has in flight
-    const unsigned int tiles = 32u / share;              // 16-column tiles of a wave
+    const unsigned int tiles = (COLS / 16u) / share;     // 16-column tiles of a wave
     const unsigned int tile0 = (wave % share) * tiles;
-    const unsigned char* frag_at = w_lds + (4u * j + (m >> 2)) * kAbsorbRowBytes + (m & 3u) * 8u;
+    const unsigned char* frag_at = w_lds + (4u * j + (m >> 2)) * kRowBytes + (m & 3u) * 8u;
     for (unsigned int row0 = (blockIdx.y * slots + wave / share) * 16u; row0 < p.batch; row0 += gridDim.y * slots * 16u) {
         const unsigned int row = min(row0 + m, p.batch - 1u);
         const size_t q_base = ((size_t)row * p.heads + head) * p.q_head_dim;
@@ -293,42 +299,42 @@ template <int WAVES> __global__ __launch_bounds__(64 * WAVES) void mla_absorb_mf
             return u32x2{pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[0] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[0] >> 16))),
                          pack_bf16_rne(f16_bits_to_f32((unsigned short)(h[1] & 0xffffu)), f16_bits_to_f32((unsigned short)(h[1] >> 16)))};
         };
-        Frag qf[4];
+        Frag qf[NOPE / 32];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < NOPE / 32; ++ks) {
             const u32x2 lo = four_as_bf16(q_base + ks * 32u + 4u * j), hi = four_as_bf16(q_base + ks * 32u + 16u + 4u * j);
             qf[ks].u = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
         // the rope part of the sixteen rows is a copy: lane = column, one row a pass, the rows dealt out to the block's waves
         {
-            const unsigned int part = wave % share;
+            const unsigned int part = wave % share + share * blockIdx.z; // of share * gridDim.z waves on this block
             float rope_in[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const unsigned int r = min(row0 + i, p.batch - 1u);
-                if ((i & (share - 1u)) == part) {
-                    rope_in[i] = load_as_f32(p.q, ((size_t)r * p.heads + head) * p.q_head_dim + kAbsorbNope + lane, p.q_dtype);
+                if ((i & (share * gridDim.z - 1u)) == part) {
+                    rope_in[i] = load_as_f32(p.q, ((size_t)r * p.heads + head) * p.q_head_dim + NOPE + lane, p.q_dtype);
                 }
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                if ((i & (share - 1u)) == part && row0 + i < p.batch) {
+                if ((i & (share * gridDim.z - 1u)) == part && row0 + i < p.batch) {
                     p.absorbed[((size_t)(row0 + i) * p.heads + head) * (kLatent + kRope) + kLatent + lane] = f32_to_bf16_bits(rope_in[i]);
                 }
             }
         }
-        unsigned short* qa = p.absorbed + ((size_t)(row0 + m) * p.heads + head) * (kLatent + kRope) + 4u * j;
+        unsigned short* qa = p.absorbed + ((size_t)(row0 + m) * p.heads + head) * (kLatent + kRope) + col0 + 4u * j;
         for (unsigned int nt = tile0; nt < tile0 + tiles; ++nt) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
+            for (int ks = 0; ks < NOPE / 32; ++ks) {
                 union {
                     s16x4 s[2];
                     bf16x8 b;
                 } wf;
-                const unsigned char* at = frag_at + ks * 32 * kAbsorbRowBytes + nt * 32u;
+                const unsigned char* at = frag_at + ks * 32 * kRowBytes + nt * 32u;
                 wf.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at));
-                wf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kAbsorbRowBytes));
+                wf.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(at + 16 * kRowBytes));
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.b, qf[ks].b, acc, 0, 0, 0);
             }
             if (row0 + m < p.batch) { // lane (m, j) holds latent columns 16 nt + 4 j .. + 4 of row m
@@ -1599,8 +1605,12 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
 // the workspace (p.weighted).  MODE 2: the plan has one record a row (a long chunk without KV splits), which only wants
 // its sum divided out.  Modes 1 and 2 leave the registers for two workgroups per compute unit.
 constexpr int kMergedStride = kLatent + 8; // bf16 elements: sixteen rows' 16-byte fragments start in different banks
-template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfma(MlaDecodeParams p)
+// WAVES: 8 (value widths up to 128) or 16 (up to 256; modes 1 and 2, whose registers allow 1,024 threads).
+template <int MODE, int WAVES = 8> __global__ __launch_bounds__(64 * WAVES) void mla_merge_project_mfma(MlaDecodeParams p)
 {
+    static_assert(WAVES == 8 || MODE != 0, "the record-folding form needs the registers of 512 threads");
+    constexpr unsigned int RG = WAVES / 2;  // groups of 128 threads: thread group rb takes rows rb, rb + RG, ...
+    constexpr int RPT = 16 / RG;            // rows of a block per thread
     // the merged rows as two bf16 terms (value = hi + lo keeps 16 bits of the f32), split once by the thread that merged them
     __shared__ __align__(16) unsigned short merged_hi[16][kMergedStride], merged_lo[16][kMergedStride];
     const unsigned int head = blockIdx.x;
@@ -1621,34 +1631,34 @@ template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfm
         }
     }
     // the merged values of this thread's four rows (rb, rb + 4, rb + 8, rb + 12 of the block at row0) and four columns
-    auto fetch_rows = [&](unsigned int row0, f32x4 (&out)[4]) __attribute__((always_inline)) {
+    auto fetch_rows = [&](unsigned int row0, f32x4 (&out)[RPT]) __attribute__((always_inline)) {
         if constexpr (MODE == 1) {
-            const unsigned int rb = tid >> 7; // rows rb, rb + 4, rb + 8, rb + 12
-            f32x4 row[4];
+            const unsigned int rb = tid >> 7;
+            f32x4 row[RPT];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+            for (int u = 0; u < RPT; ++u) {
+                const unsigned int b = min(row0 + rb + RG * u, p.batch - 1u);
                 row[u] = *(const f32x4*)(p.weighted + ((size_t)b * p.heads + head) * kLatent + quad * 4u);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < RPT; ++u) {
                 out[u] = row[u];
             }
         } else if constexpr (MODE == 2) {
             const unsigned int rb = tid >> 7;
-            float2 st[4];
-            f32x4 part[4];
-            unsigned int len[4];
+            float2 st[RPT];
+            f32x4 part[RPT];
+            unsigned int len[RPT];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const unsigned int b = min(row0 + rb + 4u * u, p.batch - 1u);
+            for (int u = 0; u < RPT; ++u) {
+                const unsigned int b = min(row0 + rb + RG * u, p.batch - 1u);
                 unsigned int seq;
                 len[u] = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
                 st[u] = *(const float2*)(p.stats + ((size_t)b * p.heads + head) * 2);
                 part[u] = *(const f32x4*)(p.partial + ((size_t)b * p.heads + head) * kLatent + quad * 4u);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < RPT; ++u) {
                 f32x4 result = {0.f, 0.f, 0.f, 0.f};
                 if (len[u] > 0u && st[u].y > 0.0f && st[u].y < __builtin_inff()) {
                     result = part[u] * (1.0f / st[u].y);
@@ -1720,19 +1730,19 @@ template <int MODE> __global__ __launch_bounds__(512) void mla_merge_project_mfm
     // The next block's rows are requested before the projection of this one, so that the round trips to memory (one for
     // merged rows, several for split records) run under the matrix work instead of between two barriers: a 2,048-row
     // chunk of one record a row spent 3 us a block waiting, 408 us in all.
-    f32x4 next_rows[4];
+    f32x4 next_rows[RPT];
     fetch_rows(blockIdx.y * 16u, next_rows);
     for (unsigned int row0 = blockIdx.y * 16u; row0 < p.batch; row0 += gridDim.y * 16u) {
     {
         const unsigned int rb = tid >> 7;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < RPT; ++u) {
             const f32x4 x = next_rows[u];
             const u32x2 hi = {pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])};
             const u32x2 lo = {pack_bf16_rne(x[0] - __uint_as_float(hi[0] << 16), x[1] - __uint_as_float(hi[0] & 0xffff0000u)),
                               pack_bf16_rne(x[2] - __uint_as_float(hi[1] << 16), x[3] - __uint_as_float(hi[1] & 0xffff0000u))};
-            *(u32x2*)(&merged_hi[rb + 4u * u][quad * 4u]) = hi;
-            *(u32x2*)(&merged_lo[rb + 4u * u][quad * 4u]) = lo;
+            *(u32x2*)(&merged_hi[rb + RG * u][quad * 4u]) = hi;
+            *(u32x2*)(&merged_lo[rb + RG * u][quad * 4u]) = lo;
         }
     }
     __syncthreads();
@@ -1817,7 +1827,7 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     if (stages & 1u) {
         // Eight rows per workgroup share every weight load, and the workgroup then runs eight rows' sums: measured 28 us from
         // 16 rows up to a few hundred, against 13 us (15 rows) to 27 us (32 rows) for one workgroup per row
-        if (p.batch >= 16u && p.nope_dim == (unsigned int)kAbsorbNope && (p.q_head_dim & 3u) == 0) { // sixteen rows a workgroup, on the matrix cores
+        if (p.batch >= 16u && (p.nope_dim == 128u || p.nope_dim == 192u) && (p.q_head_dim & 3u) == 0) { // sixteen rows a workgroup, on the matrix cores
             // four waves for a decode batch, sixteen for a chunk (33 against 61 us on 512 rows of 128 heads; on 16 to 64 rows
             // the larger workgroup costs 4 us); as many waves share a block of sixteen rows as keeps every wave busy
             MlaDecodeParams q = p;
@@ -1828,10 +1838,12 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
             while (q.column_split < waves && blocks_here * q.column_split < waves) {
                 q.column_split *= 2u;
             }
-            if (waves == 16u) {
-                mla_absorb_mfma<16><<<dim3(p.heads, groups), dim3(1024), 0, stream>>>(q);
+            if (p.nope_dim == 128u) {
+                waves == 16u ? mla_absorb_mfma<16, 128, 512><<<dim3(p.heads, groups), dim3(1024), 0, stream>>>(q)
+                             : mla_absorb_mfma<4, 128, 512><<<dim3(p.heads, groups), dim3(256), 0, stream>>>(q);
             } else {
-                mla_absorb_mfma<4><<<dim3(p.heads, groups), dim3(256), 0, stream>>>(q);
+                waves == 16u ? mla_absorb_mfma<16, 192, 256><<<dim3(p.heads, groups, 2), dim3(1024), 0, stream>>>(q)
+                             : mla_absorb_mfma<4, 192, 256><<<dim3(p.heads, groups, 2), dim3(256), 0, stream>>>(q);
             }
         } else if (p.batch >= 32u && p.nope_dim <= 256u) {
             mla_absorb_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
@@ -1865,25 +1877,32 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         }
     }
     if ((stages & 12u) == 12u) {
-        if (p.batch >= 16u && p.value_dim <= 128u) { // sixteen rows a workgroup, the projection on the matrix cores
+        // value widths up to 128 run eight waves, up to 256 sixteen (not the record-folding form, whose registers stop at 512 threads)
+        const bool wide_values = p.value_dim > 128u;
+        const bool two_step = p.max_chunks > 1u && p.batch <= 64u;
+        if (p.batch >= 16u && (p.value_dim <= 128u || (p.value_dim <= 256u && (two_step || p.max_chunks == 1u)))) {
+            // sixteen rows a workgroup, the projection on the matrix cores.
             // Up to 64 rows the fused kernel is at most 256 workgroups, each a chain of round trips (lengths, records four
             // splits at a time, projection); the split-merge kernel reads the same records with a thread per (row, head,
             // column quad), and the projection then starts from merged rows: 22.9 -> 18.4 us for 16 rows of 128 heads in 8
             // splits, 29.6 -> 25.7 us for 64 rows.  A long chunk keeps the fused kernel: its merged rows would cross the
             // workspace twice (134 MB each way for 512 rows).
-            if (p.max_chunks > 1u && p.batch <= 64u) {
+            const dim3 grid(p.heads, row_block_groups(p));
+            if (two_step) {
                 err = merge_into_workspace(p, stream);
                 if (err != hipSuccess) {
                     return err;
                 }
-                mla_merge_project_mfma<1><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+                wide_values ? mla_merge_project_mfma<1, 16><<<grid, dim3(1024), 0, stream>>>(p) : mla_merge_project_mfma<1, 8><<<grid, dim3(512), 0, stream>>>(p);
+            } else if (p.max_chunks == 1u && wide_values) {
+                mla_merge_project_mfma<2, 16><<<grid, dim3(1024), 0, stream>>>(p);
             } else if (p.max_chunks == 1u) {
-                // one record a row: two workgroups fit a compute unit, so twice the workgroups of the usual round
+                // one record a row: two workgroups of eight waves fit a compute unit, so twice the workgroups of the usual round
                 const unsigned int blocks = (p.batch + 15u) / 16u;
                 const unsigned int groups = 2u * row_block_groups(p);
-                mla_merge_project_mfma<2><<<dim3(p.heads, groups < blocks ? groups : blocks), dim3(512), 0, stream>>>(p);
+                mla_merge_project_mfma<2, 8><<<dim3(p.heads, groups < blocks ? groups : blocks), dim3(512), 0, stream>>>(p);
             } else {
-                mla_merge_project_mfma<0><<<dim3(p.heads, row_block_groups(p)), dim3(512), 0, stream>>>(p);
+                mla_merge_project_mfma<0, 8><<<grid, dim3(512), 0, stream>>>(p);
             }
         } else if (p.batch >= 16u) { // eight rows share every weight load of the projection
             mla_merge_project_rows<8><<<dim3(p.heads, (p.batch + 7u) / 8u), dim3(256), 0, stream>>>(p);
