@@ -428,7 +428,9 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
     const unsigned int score_tile = NARROW ? (hw & 1u) : hw; // head tile of a score wave
     const unsigned int stream = NARROW ? (hw >> 1) : 0u;     // narrow: which sixteen tokens of a step it scores
     const unsigned int head = blockIdx.y * 64u + score_tile * 16u + m; // this lane's head column
-    const unsigned int b = blockIdx.z; // query row of the call (= sequence when every sequence has one row)
+    // query row of the call (= sequence when every sequence has one row), the last first: the rows of a chunk see more keys
+    // the later they come, and workgroups are handed out in the order of their index
+    const unsigned int b = gridDim.z - 1u - blockIdx.z;
     unsigned int seq;
     unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq); // keys of this row: positions, or list slots when a selection applies
     const unsigned int* selected = nullptr;
