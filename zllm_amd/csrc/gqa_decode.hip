@@ -1702,7 +1702,8 @@ hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)
     if (p.max_chunks <= 8u && quads <= 256u && 256u % quads == 0u) {
         const unsigned int heads_here = 256u / quads;
         gqa_decode_merge_few<<<dim3((p.num_heads + heads_here - 1u) / heads_here, p.batch), dim3(256), 0, stream>>>(p);
-    } else if (p.max_chunks > 8u * (256u / quads) && p.head_dim % 32u == 0u && p.num_heads * p.batch <= 512u) {
+    } else if (p.head_dim % 32u == 0u && ((p.max_chunks > 8u * (256u / quads) && p.num_heads * p.batch <= 512u) ||
+                                          (p.max_chunks > 4u * (256u / quads) && p.num_heads * p.batch <= 256u))) {
         // more splits than one workgroup per (row, head) reads in a round trip, and few such pairs
         gqa_decode_merge_wide<<<dim3(p.num_heads, p.batch, p.head_dim / 32u), dim3(256), 0, stream>>>(p);
     } else {
