@@ -190,6 +190,23 @@ def test_split_plan_fills_whole_rounds_of_the_compute_units(lib):
             assert chunk.value <= 127 * 16, (batch, max_len, chunk.value)
 
 
+def test_prefill_workspace_covers_few_row_chunks_and_kv_splits(lib):
+    """One workspace size serves whichever route the call takes: a chunk of one row over a long prefix runs as a decode
+    item (row ranges + split records), a short chunk is cut into KV splits (records per row and part), a chunk of a
+    workgroup per compute unit and more needs none."""
+    pre = capi.GqaPrefillArgs()
+    pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens = 32, 8, 128, 16
+    pre.score_scale, pre.kv_format, pre.scale_dtype, pre.q_dtype = 0.1, capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16
+    sizes = {}
+    for rows, position in ((1, 32768), (2, 32768), (64, 32768), (2048, 50000), (1, 100)):
+        pre.rows, pre.position = rows, position
+        sizes[rows, position] = lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre))
+    assert sizes[1, 32768] > 256 and sizes[2, 32768] > sizes[1, 32768]  # a row's records beside its ranges
+    assert sizes[64, 32768] >= 64 * 32 * 128 * 4 * 2                     # at least two parts of f32 records a row
+    assert sizes[2048, 50000] == 0
+    assert sizes[1, 100] > 0                                            # still a decode item (its records are small)
+
+
 def test_prefill_and_mla_argument_checks_without_a_gpu(lib):
     pre = capi.GqaPrefillArgs()
     pre.rows, pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens = 8, 8, 2, 128, 16
