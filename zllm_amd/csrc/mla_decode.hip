@@ -792,15 +792,15 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
                             sc[r] = t0 + 4u * j + r < len ? sc[r] : kNegInf;
                         }
                     }
-                    // the lazy online softmax of the wide layout; the reference moves to whole numbers, so that the value
-                    // waves bring the two token halves of a head to one reference with exact powers of two
+                    // the lazy online softmax of the wide layout: the reference is the largest score seen when it last moved, so
+                    // the largest probability of a short or peaked row is exactly 1
                     const float lane_max = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
                     if (__any(lane_max > 8.0f + (float)kPShift || run_max == kNegInf)) {
                         const float step_max = wave_max_16x4(lane_max) - (float)kPShift;
                         const float ref = -neg_ref;
                         float new_max = run_max;
                         if (step_max > 8.0f || run_max == kNegInf) {
-                            new_max = fmaxf(run_max, ceilf(ref + step_max));
+                            new_max = fmaxf(run_max, ref + step_max);
                         }
                         const float safe_max = new_max == kNegInf ? 0.0f : new_max;
                         const float delta = safe_max - ref;
@@ -818,8 +818,13 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
                     for (int r = 0; r < 4; ++r) {
                         pr[r] = __builtin_amdgcn_exp2f(sc[r]);
                     }
-                    run_sum += (pr[0] + pr[1]) + (pr[2] + pr[3]); // in units of 2^-kPShift, like the probabilities
-                    ((u32x2*)&lds_p16[i & 1u][score_tile][lane])[stream] = u32x2{pack_f16_hw(pr[0], pr[1]), pack_f16_hw(pr[2], pr[3])};
+                    // The sum takes the probabilities as the value waves will multiply them, rounded to f16: numerator and
+                    // denominator of a row then carry the same weights.
+                    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+                    const unsigned int p01 = pack_f16_hw(pr[0], pr[1]), p23 = pack_f16_hw(pr[2], pr[3]);
+                    const f16x2_t h01 = __builtin_bit_cast(f16x2_t, p01), h23 = __builtin_bit_cast(f16x2_t, p23);
+                    run_sum += ((float)h01[0] + (float)h01[1]) + ((float)h23[0] + (float)h23[1]); // in units of 2^-kPShift
+                    ((u32x2*)&lds_p16[i & 1u][score_tile][lane])[stream] = u32x2{p01, p23};
                     lds_alpha[i & 1u][2u * score_tile + stream][lane] = run_max; // -inf: nothing seen yet, the probabilities are zeros
                 }
             } else if (i < steps) {
@@ -1038,9 +1043,10 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
             asm volatile("" ::: "memory");
             if constexpr (NARROW) {
                 if (i > 0) {
-                    // The two token halves of a head were scored against references of their own (whole numbers, or -inf
-                    // while a half has seen nothing).  The accumulators follow the larger one: they are rescaled when it
-                    // moves, and each half's probabilities are brought to it by an exact power of two (0 for -inf).
+                    // The two token halves of a head were scored against references of their own (-inf while a half has
+                    // seen nothing).  The accumulators follow the larger one: they are rescaled when it moves, and each
+                    // half's probabilities are brought to it by a factor of at most 1 (exactly 1 for the half that holds
+                    // the larger reference, 0 for -inf).
 #pragma unroll
                     for (int ht = 0; ht < 2; ++ht) {
                         const float ra = half_ref[ht][0], rb = half_ref[ht][1];
