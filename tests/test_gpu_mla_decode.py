@@ -454,6 +454,23 @@ def test_mla_few_rows_of_many_splits_take_the_wide_merge(heads, lens):
     assert (diff <= np.maximum(np.abs(want_f), 2.0 ** -126) * 2.0 ** -7 + 2e-3).all()
 
 
+@pytest.mark.parametrize("heads", [16, 20])
+def test_mla_short_and_peaked_rows_in_the_narrow_layout(heads):
+    """Calls of at most 32 heads score the two token halves of a step in waves of their own.  A row that sees one key, or a
+    few, must come out as precisely as in the wide layout: its largest probability is exactly 1 and numerator and
+    denominator carry the same rounded weights (a reference moved to whole numbers cost these rows half their margin:
+    1.2e-3 to 1.45e-3 against the 2e-3 bound).  Checked at half the usual bound, and a one-key selection at a twentieth of it."""
+    lens = [1, 2, 31, 32, 33, 65, 511]
+    case = make_mla_case(400 + heads, lens, heads, block_tokens=64)
+    want, _ = oracle_mla(case)
+    got = run_mla(case).cpu().numpy()
+    print("mla narrow short rows", heads, assert_attention_close(got.reshape(want.shape), want, f"MLA narrow heads={heads}", atol=1e-3))
+    selection = draw_selection(np.random.default_rng(5), lens, 1, True)
+    want_s, _ = oracle_mla(case, selection=selection)
+    got_s = run_mla(case, selection=selection).cpu().numpy()
+    print("mla narrow one key", heads, assert_attention_close(got_s.reshape(want_s.shape), want_s, f"MLA narrow one key heads={heads}", atol=1e-4))
+
+
 def test_mla_batched_decode_on_the_matrix_core_stages():
     """A decode batch of sixteen rows and more takes the matrix-core absorb and projection (one query row per sequence
     here; chunks take them through test_mla_prefill_chunk_matches_oracle): 40 ragged sequences, strided and compact
