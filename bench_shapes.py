@@ -1,8 +1,9 @@
 """Shape sweeps beside bench.py: the same entry points as the headline workloads over the shapes a serving stack
 produces -- batches that do not divide the CU count, multi-GB batches, one or two KV heads (a GPU's share under tensor
-parallelism), short chunks over long prefixes, MLA decode batches.  One JSON line per case.  These are the cases the
-split planner, the items-per-workgroup rule, the KV splits of the chunk kernels and the matrix-core MLA stages exist
-for; run it after touching any of them.
+parallelism), one sequence alone on the GPU, short chunks over long prefixes and first chunks at position 0, MLA decode
+batches and one-sequence MLA decode at the reference test's head shape.  One JSON line per case.  These are the cases
+the split planner, the items-per-workgroup rule, the wide split merges, the few-rows route, half-size row tiles and KV
+splits of the chunk kernels, and the matrix-core and narrow MLA stages exist for; run it after touching any of them.
 
     python bench_shapes.py [--suite gqa_decode|gqa_heads|prefill_chunks|mla_batches|all] [--pool-gib 40]
 """
