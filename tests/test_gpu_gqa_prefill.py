@@ -149,6 +149,25 @@ def test_prefill_few_rows_run_as_decode_items(d, prefix, chunk, hq, hkv, window,
         assert np.abs(got - want).max() <= 2e-3 + tol * max(1.0, float(np.abs(want).max())), (workspace, np.abs(got - want).max())
 
 
+@pytest.mark.parametrize("prefix,chunk,hq,hkv,extra", [(0, 300, 8, 2, ""), (17, 700, 16, 2, "gate"), (0, 1024, 8, 2, "bf16out"),
+                                                    (40, 200, 32, 4, "softcap"), (0, 33, 8, 1, "")])
+def test_prefill_first_chunks_on_half_size_row_tiles(prefix, chunk, hq, hkv, extra):
+    """A chunk much longer than what lies before it -- a prompt's first chunk -- runs row tiles of 128 (row, head) pairs,
+    handed out longest range first, with or without KV splits on top: against the oracle, with and without a workspace."""
+    kw = dict(outliers=True)
+    if extra == "gate":
+        kw["gate_cols"] = hq * 128
+    if extra == "bf16out":
+        kw["out_dtype"] = torch.bfloat16
+    if extra == "softcap":
+        kw["softcap"] = 30.0
+    tol = 2.0 ** -8 if extra == "bf16out" else 0.0
+    for workspace in (True, False):
+        out, want = run_case(61 + chunk, prefix, chunk, hq, hkv, workspace=workspace, **kw)
+        got = out.float().cpu().numpy()
+        assert np.abs(got - want).max() <= 2e-3 + tol * max(1.0, float(np.abs(want).max())), (workspace, np.abs(got - want).max())
+
+
 def test_prefill_f16_kv_splits():
     for workspace in (True, False):
         got, want = run_f16_case(5, 256, 4000, 24, 8, 2, softcap=50.0, q_kind="bf16", workspace=workspace)
