@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gqa_decode_32k",
-                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "read_calibration", "mfma_issue_calibration", "append_prologue"])
+                    choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "append_prologue"])
     ap.add_argument("--pool-gib", type=float, default=256.0, help="address span of the paged pool (all four planes); clipped to 90 %% of free HBM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
@@ -64,8 +64,6 @@ def probe_lib():
         lib.bench_probe_paged_read.argtypes = [C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         lib.bench_probe_paged_read_lds.restype = C.c_int
         lib.bench_probe_paged_read_lds.argtypes = lib.bench_probe_paged_read.argtypes
-        lib.bench_probe_mfma_issue.restype = C.c_int
-        lib.bench_probe_mfma_issue.argtypes = [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p]
         _PROBE = lib
     return _PROBE
 
@@ -456,66 +454,6 @@ def run_copy_calibration(args):
                       "config": {"workload": "torch uint8 copy_", "bytes_read": n, "bytes_written": n}}))
 
 
-def run_read_calibration(args):
-    """A plain streaming read (16-byte loads, nothing kept) over as many bytes as the headline decode call has KV bytes,
-    and over four times as many: what reading every KV byte once can reach on this device, next to the published peak."""
-    import torch
-
-    from zllm_amd import ops
-
-    kv_bytes = 8 * 32768 * 2112  # config 2, all sequences at 32K
-    sink = torch.full((1,), 7, dtype=torch.int32, device="cuda")
-    results = {}
-    for name, n in (("kv_bytes", kv_bytes), ("four_times", 4 * kv_bytes)):
-        src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
-        for _ in range(args.warmup):
-            stream_read_probe(src, sink)
-        med, low = event_times_ms(lambda: stream_read_probe(src, sink), args.steps)
-        results[name] = {"bytes": n, "kernel_ms_median": round(med, 5), "kernel_ms_min": round(low, 5),
-                         "gbps_median": round(n / (med * 1e-3) / 1e9, 1), "gbps_best": round(n / (low * 1e-3) / 1e9, 1)}
-        del src
-    first = results["kv_bytes"]
-    print(json.dumps({"metric": "plain streaming read (ceiling calibration)", "value": first["gbps_median"], "unit": "GB/s", "n_gpus": 1,
-                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["kernel_ms_median"],
-                      "config": {"workload": "bench_probe_stream_read over the config-2 KV bytes and four times as many", **results},
-                      "frac_of_hbm_peak": round(first["gbps_median"] / HBM_PEAK_GBPS, 4)}))
-
-
-def run_mfma_issue_calibration(args):
-    """What one SIMD issues when matrix and vector instructions meet (bench_probe.hip: mfma_issue_kernel): trips of
-    8 MFMAs 16x16x32 f16, of 24 FMAs, of both one after the other and of both interleaved, with one and with two waves
-    per SIMD on every CU.  `value` is the matrix rate of the MFMA-only loop with two waves per SIMD: the rate the
-    device sustains for this instruction, next to the published peak."""
-    import torch
-
-    sink = torch.zeros((1,), dtype=torch.float32, device="cuda")
-    lib = probe_lib()
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    trips = 20000
-    table = {}
-    for waves in (1, 2, 4):
-        for mode, name in enumerate(("mfma8", "fma24", "mfma8_then_fma24", "mfma_fma3_x8", "mfma8_wave_beside_fma24_waves", "mfma4_then_fma12", "mfma_fma3_x4")):
-            if waves == 1 and mode == 4:
-                continue
-            def fn():
-                rc = lib.bench_probe_mfma_issue(mode, waves, cus, trips, sink.data_ptr(), stream)
-                if rc != 0:
-                    raise RuntimeError(f"bench_probe_mfma_issue: {rc}")
-            for _ in range(max(args.warmup, 2)):
-                fn()
-            settle_clocks(fn)
-            med, low = event_times_ms(fn, max(5, min(args.steps, 20)))
-            table[f"{name}_{waves}_per_simd"] = {"ns_per_trip": round(med * 1e6 / trips, 2), "ns_per_trip_min": round(low * 1e6 / trips, 2)}
-    mfma_ns = table["mfma8_2_per_simd"]["ns_per_trip"] / 16.0  # 16 MFMAs per SIMD and trip
-    tflops = 16 * 16 * 32 * 2 / mfma_ns * 4 * cus / 1e3
-    print(json.dumps({"metric": "sustained MFMA 16x16x32 f16 rate (issue calibration)", "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
-                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(table["mfma8_2_per_simd"]["ns_per_trip"] * trips / 1e6, 5),
-                      "config": {"workload": "bench_probe_mfma_issue: one workgroup per CU, one and two waves per SIMD", "cus": cus, "trips": trips,
-                                 "ns_per_mfma_two_waves": round(mfma_ns, 3), **table},
-                      "frac_of_mfma_peak": round(tflops / 2500.0, 4)}))
-
-
 def main():
     args = parse()
     if args.gpus != 1:
@@ -531,10 +469,6 @@ def main():
         run_copy_calibration(args)
     elif args.workload == "append_prologue":
         run_append_prologue(args)
-    elif args.workload == "mfma_issue_calibration":
-        run_mfma_issue_calibration(args)
-    elif args.workload == "read_calibration":
-        run_read_calibration(args)
     else:
         import bench_extra
 

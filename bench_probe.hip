@@ -127,74 +127,6 @@ template <int INFLIGHT> __global__ __launch_bounds__(512) void paged_read_lds_ke
     }
 }
 
-// What a SIMD issues when matrix and vector instructions meet: a loop trip holds 8 independent MFMAs (16x16x32 f16, own
-// accumulators), or 24 independent FMAs, or both -- one after the other, or one MFMA followed by three FMAs, eight times.
-// One workgroup per CU with one or two waves per SIMD.  The instruction order is fixed by inline assembly.
-typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 probe_f16x8 __attribute__((ext_vector_type(8)));
-#define PROBE_MFMA(k) "v_mfma_f32_16x16x32_f16 %" #k ", %8, %9, %" #k "\n\t"
-#define PROBE_FMA3(a, b, c) \
-    "v_fma_f32 %" #a ", %" #a ", %26, %" #a "\n\tv_fma_f32 %" #b ", %" #b ", %26, %" #b "\n\tv_fma_f32 %" #c ", %" #c ", %26, %" #c "\n\t"
-#define PROBE_OPERANDS                                                                                                                         \
-    : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]), "+v"(a), "+v"(b), "+v"(f[0]), \
-      "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]), "+v"(f[8]), "+v"(f[9]), "+v"(f[10]), "+v"(f[11]),       \
-      "+v"(f[12]), "+v"(f[13]), "+v"(f[14]), "+v"(f[15])                                                                                        \
-    : "v"(c)
-template <int MODE> __global__ __launch_bounds__(1024) void mfma_issue_kernel(float* sink, int trips)
-{
-    probe_f32x4 acc[8];
-    float f[16];
-    probe_f16x8 a, b;
-    for (int i = 0; i < 8; ++i) {
-        acc[i] = probe_f32x4{0.f, 0.f, 0.f, 0.f};
-        a[i] = (_Float16)(threadIdx.x * 0.001f + i);
-        b[i] = (_Float16)(i * 0.5f);
-    }
-    for (int i = 0; i < 16; ++i) {
-        f[i] = (float)(threadIdx.x + i);
-    }
-    const float c = 1.0001f;
-    for (int t = 0; t < trips; ++t) {
-        if (MODE == 0) {
-            asm volatile(PROBE_MFMA(0) PROBE_MFMA(1) PROBE_MFMA(2) PROBE_MFMA(3) PROBE_MFMA(4) PROBE_MFMA(5) PROBE_MFMA(6) PROBE_MFMA(7) PROBE_OPERANDS);
-        } else if (MODE == 1) {
-            asm volatile(PROBE_FMA3(10, 11, 12) PROBE_FMA3(13, 14, 15) PROBE_FMA3(16, 17, 18) PROBE_FMA3(19, 20, 21) PROBE_FMA3(22, 23, 24)
-                             PROBE_FMA3(25, 10, 11) PROBE_FMA3(12, 13, 14) PROBE_FMA3(15, 16, 17) PROBE_OPERANDS);
-        } else if (MODE == 2) {
-            asm volatile(PROBE_MFMA(0) PROBE_MFMA(1) PROBE_MFMA(2) PROBE_MFMA(3) PROBE_MFMA(4) PROBE_MFMA(5) PROBE_MFMA(6) PROBE_MFMA(7)
-                             PROBE_FMA3(10, 11, 12) PROBE_FMA3(13, 14, 15) PROBE_FMA3(16, 17, 18) PROBE_FMA3(19, 20, 21) PROBE_FMA3(22, 23, 24)
-                                 PROBE_FMA3(25, 10, 11) PROBE_FMA3(12, 13, 14) PROBE_FMA3(15, 16, 17) PROBE_OPERANDS);
-        } else if (MODE == 3) {
-            asm volatile(PROBE_MFMA(0) PROBE_FMA3(10, 11, 12) PROBE_MFMA(1) PROBE_FMA3(13, 14, 15) PROBE_MFMA(2) PROBE_FMA3(16, 17, 18) PROBE_MFMA(3)
-                             PROBE_FMA3(19, 20, 21) PROBE_MFMA(4) PROBE_FMA3(22, 23, 24) PROBE_MFMA(5) PROBE_FMA3(25, 10, 11) PROBE_MFMA(6)
-                                 PROBE_FMA3(12, 13, 14) PROBE_MFMA(7) PROBE_FMA3(15, 16, 17) PROBE_OPERANDS);
-        } else if (MODE == 4) { // the kinds apart: the first wave of a SIMD issues the MFMAs, the others the FMAs
-            if (threadIdx.x < 256u) {
-                asm volatile(PROBE_MFMA(0) PROBE_MFMA(1) PROBE_MFMA(2) PROBE_MFMA(3) PROBE_MFMA(4) PROBE_MFMA(5) PROBE_MFMA(6) PROBE_MFMA(7) PROBE_OPERANDS);
-            } else {
-                asm volatile(PROBE_FMA3(10, 11, 12) PROBE_FMA3(13, 14, 15) PROBE_FMA3(16, 17, 18) PROBE_FMA3(19, 20, 21) PROBE_FMA3(22, 23, 24)
-                                 PROBE_FMA3(25, 10, 11) PROBE_FMA3(12, 13, 14) PROBE_FMA3(15, 16, 17) PROBE_OPERANDS);
-            }
-        } else if (MODE == 5) { // half of mode 2 in every wave
-            asm volatile(PROBE_MFMA(0) PROBE_MFMA(1) PROBE_MFMA(2) PROBE_MFMA(3) PROBE_FMA3(10, 11, 12) PROBE_FMA3(13, 14, 15) PROBE_FMA3(16, 17, 18)
-                             PROBE_FMA3(19, 20, 21) PROBE_OPERANDS);
-        } else { // half of mode 3 in every wave
-            asm volatile(PROBE_MFMA(0) PROBE_FMA3(10, 11, 12) PROBE_MFMA(1) PROBE_FMA3(13, 14, 15) PROBE_MFMA(2) PROBE_FMA3(16, 17, 18) PROBE_MFMA(3)
-                             PROBE_FMA3(19, 20, 21) PROBE_OPERANDS);
-        }
-    }
-    float sum = 0.f;
-    for (int i = 0; i < 8; ++i) {
-        sum += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
-    }
-    for (int i = 0; i < 16; ++i) {
-        sum += f[i];
-    }
-    if (sum == 12345.678f) { // keeps the loop alive; practically never true
-        sink[0] = sum;
-    }
-}
-
 extern "C" {
 
 __attribute__((visibility("default"))) int bench_probe_stream_read(const void* src, uint64_t bytes, uint32_t* sink, void* stream)
@@ -250,29 +182,6 @@ __attribute__((visibility("default"))) int bench_probe_paged_read_lds(const void
     case 2: paged_read_lds_kernel<2><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
     case 4: paged_read_lds_kernel<4><<<dim3(groups), dim3(512), 0, st>>>(kp, vp, ks, vs, table, pages, per_group, sink); break;
     default: return -1;
-    }
-    return (int)hipGetLastError();
-}
-
-// mode 0: 8 MFMAs per trip, 1: 24 FMAs, 2: 8 MFMAs then 24 FMAs, 3: (MFMA, 3 FMAs) x 8, 4: the first wave of a SIMD
-// 8 MFMAs and every other wave 24 FMAs, 5 and 6: halves of 2 and 3.  One workgroup per CU (`workgroups` of them),
-// `waves_per_simd` (1, 2 or 4) waves on each of its four SIMDs.
-__attribute__((visibility("default"))) int bench_probe_mfma_issue(uint32_t mode, uint32_t waves_per_simd, uint32_t workgroups, uint32_t trips,
-                                                                  float* sink, void* stream)
-{
-    if (sink == nullptr || mode > 6 || (waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) || workgroups == 0 || trips == 0 || trips > (1u << 24)) {
-        return -1;
-    }
-    const dim3 grid(workgroups), block(256u * waves_per_simd);
-    const hipStream_t st = (hipStream_t)stream;
-    switch (mode) {
-    case 0: mfma_issue_kernel<0><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    case 1: mfma_issue_kernel<1><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    case 2: mfma_issue_kernel<2><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    case 3: mfma_issue_kernel<3><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    case 4: mfma_issue_kernel<4><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    case 5: mfma_issue_kernel<5><<<grid, block, 0, st>>>(sink, (int)trips); break;
-    default: mfma_issue_kernel<6><<<grid, block, 0, st>>>(sink, (int)trips); break;
     }
     return (int)hipGetLastError();
 }

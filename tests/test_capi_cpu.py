@@ -225,6 +225,14 @@ def test_prefill_and_mla_argument_checks_without_a_gpu(lib):
     pre.head_dim = 256  # this geometry runs its rows through the decode kernels and needs their split records
     assert lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre)) > 8 * 8
     assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"workspace" in lib.zllm_attn_last_error()
+    # a chunk whose rows run as decode items is a decode call of that many rows: more than the merge's grid can index is
+    # refused before anything is launched, and so is a decode batch of that size
+    pre.rows, pre.q_dtype, pre.table = 70000, capi.DTYPE_F32, None
+    assert lib.zllm_attn_gqa_prefill_chunk(C.byref(pre), None) == -1 and b"65535" in lib.zllm_attn_last_error()
+    dec = capi.GqaDecodeArgs()
+    dec.batch, dec.num_heads, dec.num_kv_heads, dec.head_dim, dec.block_tokens, dec.max_kv_len = 70000, 8, 2, 128, 16, 64
+    dec.score_scale, dec.kv_format, dec.scale_dtype = 0.1, capi.KV_Q8G64, capi.SCALE_F16
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(dec)) == 0 and b"65535" in lib.zllm_attn_last_error()
     # MLA: value part and query-row limits
     mla = capi.MlaDecodeArgs()
     mla.batch, mla.heads, mla.q_head_dim, mla.kv_head_dim, mla.latent_dim, mla.rope_dim = 1, 16, 192, 128, 512, 64

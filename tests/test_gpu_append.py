@@ -156,3 +156,46 @@ def test_mla_append_bit_exact(layout, rotary_dim):
     assert np.array_equal(codes.cpu().numpy(), ref_codes)
     assert np.array_equal(scales.cpu().numpy().view(np.uint16), ref_scales)
     assert np.array_equal(rope_cache.cpu().numpy().view(np.uint16), ref_rope)
+
+
+@pytest.mark.parametrize("layout,rotary_dim,rows", [(1, 64, 1), (0, 64, 1), (1, 32, 5), (1, 0, 3)])
+def test_mla_append_positions_from_device_memory(layout, rotary_dim, rows):
+    """Graph-replay form of the fused MLA append (paged_cache_append_mla_f32_q8_bf16_indirect, paged_mla/source.hip:787-807,
+    launcher paged_mla.rs:960-1036): the cache row comes from positions[0] and the rope-table row from positions[1], both
+    in device memory; the host-side numbers of the argument block are deliberately wrong and must not be used."""
+    from zllm_amd import ops
+
+    rng = np.random.default_rng(900 + layout + rotary_dim + rows)
+    latent_cols, rope_cols, block = 512, 64, 16
+    pool_rows = 160
+    tables, pool_blocks = draw_tables(rng, [pool_rows], block)
+    pool = pool_blocks * block
+    half = max(rotary_dim // 2, 1)
+    angles = rng.uniform(0, 6.28, size=(pool_rows + 16, half)).astype(np.float32)
+    cos, sin = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    ref_codes = np.zeros((pool, latent_cols), dtype=np.int8)
+    ref_scales = np.zeros((pool, latent_cols // 64), dtype=np.uint16)
+    ref_rope = np.zeros((pool, rope_cols), dtype=np.uint16)
+    codes = torch.zeros((pool, latent_cols), dtype=torch.int8, device="cuda")
+    scales = torch.zeros((pool, latent_cols // 64), dtype=torch.int16, device="cuda")
+    rope_cache = torch.zeros((pool, rope_cols), dtype=torch.int16, device="cuda")
+    table = upload(tables[0])
+    positions = torch.zeros(2, dtype=torch.int32, device="cuda")
+    dev_cos, dev_sin = (upload(cos), upload(sin)) if rotary_dim else (None, None)
+    # three appends through one argument shape; only the device words move (a page boundary is crossed on the way)
+    for position, rope_position in ((13, 13), (13 + rows, 20), (47, 3)):
+        latent = rng.standard_normal((rows, latent_cols)).astype(np.float32)
+        k_rope = rng.standard_normal((rows, rope_cols)).astype(np.float32)
+        O.q8g64_append_paged(O.RULE_ROCM_MLA, latent, ref_codes, ref_scales, tables[0], position, block)
+        rotated = k_rope
+        if rotary_dim:
+            rc, rotated = O.rope_apply(k_rope, 1, rotary_dim, rope_position, cos, sin, layout=0 if layout == 1 else 1, placement=1)
+            assert rc == 0
+        O.half_append_paged(0, rotated, ref_rope, tables[0], position, block)
+        positions.copy_(upload(np.array([position, rope_position], dtype=np.uint32)).view(torch.int32))
+        ops.mla_append(upload(latent), upload(k_rope), codes, scales, rope_cache, table, 99, block, cos=dev_cos, sin=dev_sin,
+                       rotary_dim=rotary_dim, rotary_layout=layout, rope_position=77, positions=positions)
+    torch.cuda.synchronize()
+    assert np.array_equal(codes.cpu().numpy(), ref_codes), "codes differ"
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), ref_scales), "scale bits differ"
+    assert np.array_equal(rope_cache.cpu().numpy().view(np.uint16), ref_rope), "rope bits differ"

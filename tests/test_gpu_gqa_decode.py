@@ -279,8 +279,9 @@ def test_batch_larger_than_a_wave_with_empty_sequences():
 
 
 @pytest.mark.parametrize("fmt,hq,hkv,d,window", [("q8", 8, 1, 128, 0), ("q8", 16, 2, 128, 100), ("q8", 6, 3, 128, 0), ("q8", 4, 1, 64, 0),
-                                                  ("q8", 8, 2, 64, 33), ("q8", 4, 1, 256, 0), ("q8", 16, 2, 256, 700),
-                                                  ("f16", 8, 1, 128, 0), ("f16", 4, 2, 128, 64), ("f16", 4, 1, 256, 0), ("f16", 32, 2, 256, 500)])
+                                                  ("q8", 8, 2, 64, 33), ("q8", 4, 1, 256, 0), ("q8", 16, 2, 256, 700), ("q8", 6, 3, 256, 0),
+                                                  ("f16", 8, 1, 128, 0), ("f16", 4, 2, 128, 64), ("f16", 4, 1, 256, 0), ("f16", 32, 2, 256, 500),
+                                                  ("f16", 6, 3, 256, 0)])
 def test_few_kv_heads_share_a_workgroup(fmt, hq, hkv, d, window):
     """With one to three KV heads a workgroup runs several (sequence, split) items side by side.  The item count here
     is not a multiple of the items in a workgroup (the last workgroup has idle waves), one sequence is empty and the
@@ -298,6 +299,19 @@ def test_few_kv_heads_share_a_workgroup(fmt, hq, hkv, d, window):
         want = oracle_gqa_decode(case, 0.09, window=window, fmt=O.FMT_F16)
     assert_attention_close(got, want, f"{fmt} {hq}/{hkv} d={d} window={window}")
     assert not got[1].any()
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_every_kv_head_count_fits_its_workgroup(d):
+    """One to eight KV heads at every head_dim: waves x items of a workgroup must stay inside the kernels' launch bounds
+    (three KV heads of head_dim 256 once asked for 384 threads of a 256-thread kernel), Q8g64 and f16 rows alike."""
+    for hkv in range(1, 9):
+        lens = [130, 0, 700]
+        case = make_gqa_q8_case(1200 + 10 * d + hkv, lens, 2 * hkv, hkv, d)
+        assert_attention_close(run_decode(case, 0.09), oracle_gqa_decode(case, 0.09), f"q8 {2 * hkv}/{hkv} d={d}")
+        if d != 64:
+            case = make_f16_case(1300 + 10 * d + hkv, lens, 2 * hkv, hkv, d)
+            assert_attention_close(run_f16(case, 0.09), oracle_gqa_decode(case, 0.09, fmt=O.FMT_F16), f"f16 {2 * hkv}/{hkv} d={d}")
 
 
 @pytest.mark.parametrize("q_kind", ["f32", "bf16", "f16"])

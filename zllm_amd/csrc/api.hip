@@ -146,6 +146,11 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
         !valid_head_dim(a->head_dim)) {
         return fail(-1, "GQA decode: invalid shape batch=%u heads=%u/%u dim=%u", a->batch, a->num_heads, a->num_kv_heads, a->head_dim);
     }
+    // the split merge indexes the rows of the call (sequences, or the rows of a prefill chunk that runs as decode items) with
+    // the grid's second dimension
+    if (a->batch > 65535u) {
+        return fail(-1, "GQA decode: batch=%u exceeds 65535 rows per call", a->batch);
+    }
     if (a->block_tokens == 0 || a->max_kv_len == 0) {
         return fail(-1, "GQA decode: block_tokens=%u max_kv_len=%u must be non-zero", a->block_tokens, a->max_kv_len);
     }

@@ -1639,8 +1639,13 @@ unsigned int gqa_decode_max_waves(unsigned int head_dim)
 unsigned int gqa_decode_items_per_group(unsigned int head_dim, unsigned int num_kv_heads)
 {
     // four waves keep a CU's loads flowing (measured with four KV heads: 5.8 TB/s); more items than that only add
-    // partial records for the merge
-    return num_kv_heads < 4u ? (num_kv_heads == 1u ? 4u : 2u) : 1u;
+    // partial records for the merge.  waves x items never passes the kernels' launch bound (gqa_decode_max_waves
+    // waves): three KV heads of head_dim 256 are three of the four waves a workgroup may have, so they run one item.
+    const unsigned int max_waves = gqa_decode_max_waves(head_dim);
+    const unsigned int waves = num_kv_heads < max_waves ? num_kv_heads : max_waves;
+    const unsigned int wanted = num_kv_heads < 4u ? (num_kv_heads == 1u ? 4u : 2u) : 1u;
+    const unsigned int fit = max_waves / waves;
+    return wanted < fit ? wanted : fit;
 }
 
 hipError_t launch_gqa_decode(const GqaDecodeParams& args, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream)
