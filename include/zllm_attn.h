@@ -67,6 +67,11 @@ enum { ZLLM_ROTARY_INTERLEAVED = 0, ZLLM_ROTARY_SPLIT_HALF = 1 };
 enum { ZLLM_STAGE_ALL = 0, ZLLM_STAGE_PARTIAL = 1, ZLLM_STAGE_MERGE = 2 };
 
 enum { ZLLM_MLA_ABSORB = 1, ZLLM_MLA_PARTIAL = 2, ZLLM_MLA_MERGE = 4, ZLLM_MLA_PROJECT = 8 };
+/* OR-ed into zllm_mla_decode_args::stage_mask beside the stage bits (alone = the whole chain): the split-KV partial runs on
+ * its second kernel -- tiles of f16(code * scale) instead of integer codes beside a scale table, 32x32x16 matrix tiles on
+ * the value side -- where the call allows it (dense, more than 32 heads, pages of a multiple of 32 tokens); other calls
+ * run the default kernel.  Same records, same results within the attention tolerance. */
+enum { ZLLM_MLA_WIDE_TILES = 16 };
 
 #define ZLLM_GROUP_SIZE 64 /* src/kv_cache/mod.rs:29 DEFAULT_GROUP_SIZE */
 
@@ -444,7 +449,8 @@ typedef struct zllm_mla_decode_args {
     int out_dtype;                /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
     int out_compact;
     uint32_t stage_mask;          /* 0 = whole chain; else OR of ZLLM_MLA_ABSORB / _PARTIAL / _MERGE /
-                                     _PROJECT: run only those stages on the records already in the
+                                     _PROJECT (and optionally ZLLM_MLA_WIDE_TILES): run only those stages on
+                                     the records already in the
                                      workspace (shard exchange, per-stage timing;
                                      cf. paged_mla.rs:3068-3081 per-stage profile) */
     /* Selected-token (sparse) decode, the `selection` arm of the same launch

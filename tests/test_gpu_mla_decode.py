@@ -66,7 +66,8 @@ def oracle_mla(case, head_subset=None, selection=None, counts=None):
     return np.stack(outs_f), np.stack(outs_b)
 
 
-def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, selection=None, counts=None, total_ctx_tokens=0):
+def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, selection=None, counts=None, total_ctx_tokens=0,
+            wide_tiles=False):
     from zllm_amd import ops
 
     out_dtype = out_dtype or torch.float32
@@ -76,7 +77,8 @@ def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, s
                          case["nope"] + case["value"], case["latent"], case["rope_dim"], case["block_tokens"],
                          max_ctx_len or int(case["lens"].max()), out_dtype=out_dtype, out_compact=compact,
                          selection=None if selection is None else upload(selection),
-                         selection_counts=None if counts is None else upload(counts), total_ctx_tokens=total_ctx_tokens)
+                         selection_counts=None if counts is None else upload(counts), total_ctx_tokens=total_ctx_tokens,
+                         wide_tiles=wide_tiles)
     torch.cuda.synchronize()
     return out
 
@@ -387,7 +389,7 @@ def oracle_mla_chunk(case, selection=None):
     return np.concatenate(outs_f), np.concatenate(outs_b)
 
 
-def run_mla_chunk(case, out_dtype=None, selection=None, compact=True, q_kind="bf16"):
+def run_mla_chunk(case, out_dtype=None, selection=None, compact=True, q_kind="bf16", wide_tiles=False):
     from zllm_amd import ops
 
     q = to_torch_bf16(case["q_bits"], "cuda")
@@ -398,7 +400,7 @@ def run_mla_chunk(case, out_dtype=None, selection=None, compact=True, q_kind="bf
                          upload(case["rope"]), upload(case["tables"]), upload(case["lens"]), case["heads"],
                          case["nope"] + case["rope_dim"], case["nope"] + case["value"], case["latent"], case["rope_dim"],
                          case["block_tokens"], int(case["lens"].max()), out_dtype=out_dtype or torch.float32, out_compact=compact,
-                         selection=None if selection is None else upload(selection), query_rows=case["rows"])
+                         selection=None if selection is None else upload(selection), query_rows=case["rows"], wide_tiles=wide_tiles)
     torch.cuda.synchronize()
     return out
 

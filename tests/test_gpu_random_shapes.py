@@ -141,6 +141,9 @@ def test_random_mla_decode(it):
     want, _ = oracle_mla(case, selection=selection)
     got = run_mla(case, selection=selection, total_ctx_tokens=hint).cpu().numpy()
     assert_attention_close(got.reshape(want.shape), want, what)
+    if heads > 32 and bt % 32 == 0 and selection is None:  # a shape the second split-KV kernel takes
+        wide = run_mla(case, total_ctx_tokens=hint, wide_tiles=True).cpu().numpy()
+        assert_attention_close(wide.reshape(want.shape), want, what + " (wide tiles)")
 
 
 @pytest.mark.parametrize("it", range(14))
@@ -157,3 +160,6 @@ def test_random_mla_chunk(it):
     want, _ = oracle_mla_chunk(case)
     got = run_mla_chunk(case, q_kind=q_kind).cpu().numpy()
     assert_attention_close(got.reshape(want.shape), want, what)
+    if heads > 32 and bt % 32 == 0:
+        wide = run_mla_chunk(case, q_kind=q_kind, wide_tiles=True).cpu().numpy()
+        assert_attention_close(wide.reshape(want.shape), want, what + " (wide tiles)")

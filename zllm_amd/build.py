@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzllm_attn.so")
-SOURCES = ["api.hip", "append.hip", "gqa_decode.hip", "mla_decode.hip", "gqa_prefill.hip"]
+SOURCES = ["api.hip", "append.hip", "gqa_decode.hip", "mla_decode.hip", "mla_partial_x32.hip", "gqa_prefill.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",
@@ -38,7 +38,7 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build_library(jobs: int = 4) -> str:
+def build_library(jobs: int = 6) -> str:
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objects = list(pool.map(_compile, SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objects]

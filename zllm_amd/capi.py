@@ -19,6 +19,7 @@ QUANT_ROCM_MLA, QUANT_METAL_GQA, QUANT_CUDA_GQA = 0, 1, 2
 ROTARY_INTERLEAVED, ROTARY_SPLIT_HALF = 0, 1
 STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
 MLA_ABSORB, MLA_PARTIAL, MLA_MERGE, MLA_PROJECT = 1, 2, 4, 8
+MLA_WIDE_TILES = 16  # OR-ed into stage_mask: the split-KV partial on its second kernel where the call allows it
 
 _u32, _u64, _f32, _int, _ptr = C.c_uint32, C.c_uint64, C.c_float, C.c_int, C.c_void_p
 

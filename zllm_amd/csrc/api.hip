@@ -267,7 +267,7 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
     if ((a->q_dtype != ZLLM_DTYPE_F32 && a->q_dtype != ZLLM_DTYPE_BF16) || (a->out_dtype != ZLLM_DTYPE_F32 && a->out_dtype != ZLLM_DTYPE_BF16)) {
         return fail(-1, "MLA decode: q_dtype / out_dtype must be f32 or bf16");
     }
-    if (a->stage_mask > 15u) {
+    if (a->stage_mask > 31u) {
         return fail(-1, "MLA decode: unknown stage_mask %u", a->stage_mask);
     }
     if (a->selection != nullptr && a->top_k == 0) {

@@ -185,6 +185,9 @@ hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);
 hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream);
 hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream);
+// The split-KV partial on 32x32x16 matrix tiles (mla_partial_x32.hip): which calls it takes, and its launch.
+bool mla_partial_x32_takes(const MlaDecodeParams& p);
+hipError_t launch_mla_partial_x32(const MlaDecodeParams& p, hipStream_t stream);
 // LSE combine of split records: uses kv_lens, first_visible, partial, stats, out, batch, num_heads,
 // head_dim, chunk_tokens, max_chunks of the parameter block.
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream);

@@ -1830,7 +1830,7 @@ static hipError_t merge_into_workspace(const MlaDecodeParams& p, hipStream_t str
 
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream)
 {
-    const unsigned int stages = stage_mask == 0 ? 15u : stage_mask;
+    const unsigned int stages = (stage_mask & 15u) == 0 ? 15u : (stage_mask & 15u);
     hipError_t err = hipSuccess;
     if (stages & 1u) {
         // Eight rows per workgroup share every weight load, and the workgroup then runs eight rows' sums: measured 28 us from
@@ -1870,7 +1870,12 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         const bool narrow = p.heads <= 32u; // two head tiles at most: the score waves split a step's tokens, the value waves the columns four ways
         const bool aligned = p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0;
         const bool pow2_tables = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.tables != nullptr;
-        if (p.selection != nullptr) {
+        if ((stage_mask & 16u) != 0 && mla_partial_x32_takes(p)) { // ZLLM_MLA_WIDE_TILES: the caller asks for the 32x32x16-tile kernel
+            err = launch_mla_partial_x32(p, stream);
+            if (err != hipSuccess) {
+                return err;
+            }
+        } else if (p.selection != nullptr) {
             (narrow ? mla_partial_ws<false, true, false, true> : mla_partial_ws<false, true>)<<<grid, dim3(512), 0, stream>>>(p);
         } else if (aligned && pow2_tables) {
             (narrow ? mla_partial_ws<true, false, true, true> : mla_partial_ws<true, false, true>)<<<grid, dim3(512), 0, stream>>>(p);

@@ -178,7 +178,7 @@ def gqa_prefill_chunk(*a, **kw):
 def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ctx_lens, heads, q_head_dim,
                     kv_head_dim, latent_dim, rope_dim, block_tokens, max_ctx_len, out_dtype=torch.float32,
                     out_compact=True, out=None, workspace=None, selection=None, selection_counts=None, query_rows=1,
-                    total_ctx_tokens=0):
+                    total_ctx_tokens=0, wide_tiles=False):
     """`q` holds every query row of the call, sequence-major: [batch * query_rows, heads * q_head_dim]."""
     rows = q.shape[0]
     batch = rows // query_rows
@@ -197,6 +197,7 @@ def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ct
     args.q_dtype, args.out_dtype, args.out_compact = _DTYPE[q.dtype], _DTYPE[out_dtype], int(out_compact)
     args.query_rows = query_rows
     args.total_ctx_tokens = total_ctx_tokens
+    args.stage_mask = capi.MLA_WIDE_TILES if wide_tiles else 0
     if selection is not None:  # [batch, top_k] token positions (uint32 / int32)
         args.selection, args.top_k = _ptr(selection), selection.shape[1]
         args.selection_counts = _ptr(selection_counts)
