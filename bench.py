@@ -41,6 +41,7 @@ def parse():
                     choices=["gqa_decode_32k", "gqa_decode_ragged", "gqa_decode_c1", "mla_decode_64k", "mla_prefill_chunk", "gqa_prefill_chunk", "gqa_prefill_f16", "gqa_decode_f16_window", "copy_calibration", "append_prologue"])
     ap.add_argument("--pool-gib", type=float, default=256.0, help="address span of the paged pool (all four planes); clipped to 90 %% of free HBM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="default workload only: leave out the other configurations' entries")
     ap.add_argument("--seed", type=int, default=2)
     return ap.parse_args()
 
@@ -142,17 +143,25 @@ def settle_clocks(fn, seconds=CLOCK_SETTLE_S):
         torch.cuda.synchronize()
 
 
-def wall_time_ms(fn, steps):
-    """Wall clock per call over exactly `steps` calls, bracketed by synchronize, after settle_clocks."""
+def wall_time_ms(fn, steps, regions=1):
+    """Wall clock per call over exactly `steps` calls, bracketed by synchronize, after settle_clocks.  With `regions` > 1 the
+    region of `steps` calls is timed that many times back to back and the median region is returned (with the shortest and
+    the longest one beside it)."""
     import torch
 
     settle_clocks(fn)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    times = []
+    for _ in range(regions):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3 / steps)
+    times.sort()
+    if regions == 1:
+        return times[0]
+    return times[len(times) // 2], times[0], times[-1]
 
 
 # ------------------------------------------------------------------------------------------- GQA decode
@@ -315,7 +324,9 @@ def run_gqa_decode(args, ragged, config1=False):
     replays = args.steps // per_graph
     for _ in range(max(1, args.warmup // per_graph)):
         graph.replay()
-    ms_step = wall_time_ms(graph.replay, replays) / per_graph
+    # exactly `steps` calls make one timed region; the region is repeated and the median region is the step time
+    regions = 11
+    ms_step, ms_step_min, ms_step_max = (t / per_graph for t in wall_time_ms(graph.replay, replays, regions=regions))
     ms_events = event_time_ms(graph.replay, replays) / per_graph
     settle_clocks(partial_only)
     ms_partial = event_time_ms(partial_only, args.steps)  # one event pair around `steps` back-to-back launches
@@ -343,10 +354,14 @@ def run_gqa_decode(args, ragged, config1=False):
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "ms_per_step_events": round(ms_events, 5),
         "ms_per_step_eager_launch": round(ms_eager, 5),
-        "launch": f"hipGraph replay, {per_graph} decode calls (partial + merge each) per graph; {CLOCK_SETTLE_S} s of untimed replays before the timed ones",
+        "ms_per_step_regions": {"count": regions, "median": round(ms_step, 5), "min": round(ms_step_min, 5), "max": round(ms_step_max, 5)},
+        "launch": f"hipGraph replay, {per_graph} decode calls (partial + merge each) per graph; {CLOCK_SETTLE_S} s of untimed replays, then {regions} "
+                  f"regions of exactly {args.steps} steps each, bracketed by synchronize: ms_per_step is the median region",
         "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_dma128", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": None if ragged or config1 or args.seed != 2 else GQA_32K_TRAFFIC_BYTES,
+                     "traffic_source": None if ragged or config1 or args.seed != 2 else
+                     "profiles/gqa_decode_q8_dma128__gqa_decode_32k.md: rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload, scaled by a 1 GiB copy; not read in this run",
                      "kernel_ms": round(ms_partial, 5), "kernel_ms_single_launch_median": round(ms_partial_median, 5),
                      "kernel_ms_single_launch_min": round(ms_partial_min, 5)},
     }
@@ -370,7 +385,13 @@ def run_gqa_decode(args, ragged, config1=False):
         cpu, cpu_out = gqa_cpu_baseline(planes, tables_dev, lens, q, hq, hkv, d, bt, scale)
         record["cpu_baseline"] = cpu
         record["parity_vs_oracle_max_abs"] = float(np.abs(out.cpu().numpy() - cpu_out).max())
-    print(json.dumps(record))
+    elif getattr(args, "oracle_sequences", 0):
+        # parity only (no CPU timing): the oracle on the first sequences of the batch
+        n = args.oracle_sequences
+        _, cpu_out = gqa_cpu_baseline(planes, tables_dev[:n], lens[:n], q[:n], hq, hkv, d, bt, scale, budget_s=0.0)
+        record["parity_vs_oracle_max_abs"] = float(np.abs(out[:n].cpu().numpy() - cpu_out).max())
+        record["parity_sample"] = f"first {n} sequences, all heads"
+    return record
 
 
 def run_append_prologue(args):
@@ -431,11 +452,11 @@ def run_append_prologue(args):
         moved = rows * (hq * d * 2 * 2 + 2 * hkv * d * 2 + 2 * hkv * d + 2 * (hkv * d // 64) * 2 + d * 4)
         results[f"gqa_prologue_{rows}_rows_bf16"] = {"ms": round(ms, 5), "bytes": moved, "gbps": round(moved / ms / 1e6, 1)}
     head = results["gqa_prologue_2048_rows_bf16"]
-    print(json.dumps({"metric": "pre-attention prologue of a 2,048-row chunk, bytes moved per second", "value": head["gbps"], "unit": "GB/s",
+    return ({"metric": "pre-attention prologue of a 2,048-row chunk, bytes moved per second", "value": head["gbps"], "unit": "GB/s",
                       "n_gpus": 1, "steps": launches, "warmup": 3, "ms_per_step": head["ms"], "higher_is_better": True, "dtype": "f32",
                       "data": "synthetic", "config": {"workload": "page appends and fused prologue at chunk sizes", **results},
                       "roofline": {"bound": "hbm", "kernel": "gqa_prologue_kernel", "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                   "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None}}))
+                                   "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None}})
 
 
 def run_copy_calibration(args):
@@ -449,9 +470,51 @@ def run_copy_calibration(args):
     for _ in range(args.warmup):
         dst.copy_(src)
     ms = event_time_ms(lambda: dst.copy_(src), args.steps)
-    print(json.dumps({"metric": "device copy (counter calibration)", "value": round(2 * n / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
-                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
-                      "config": {"workload": "torch uint8 copy_", "bytes_read": n, "bytes_written": n}}))
+    return {"metric": "device copy (counter calibration)", "value": round(2 * n / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+            "config": {"workload": "torch uint8 copy_", "bytes_read": n, "bytes_written": n}}
+
+
+def other_configs(args):
+    """The other benchmark configurations in the same process, each replayed or launched at least 100 times and checked
+    against the oracle on a slice: the ragged draw of config 2, config 4 (MLA decode at 64K, the MFMA-bound one) and config 5
+    (the prefill chunk).  Keys per entry: ms_per_step, value + unit, roofline {kernel, achieved, peak, frac, kernel_ms},
+    parity_vs_oracle_max_abs."""
+    import copy
+
+    import torch
+
+    import bench_extra
+
+    def brief(record):
+        keep = ("ms_per_step", "value", "unit", "steps", "pct_of_hbm_peak", "pct_of_mfma_peak", "tokens_per_s", "stage_ms", "parity_vs_oracle_max_abs",
+                "parity_sample", "ms_per_step_regions")
+        out = {k: record[k] for k in keep if k in record}
+        out["workload"] = record["config"]["workload"]
+        out["roofline"] = {k: v for k, v in record["roofline"].items() if k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "kernel_ms",
+                                                                                 "kernel_ms_single_launch_median", "kernel_ms_single_launch_min",
+                                                                                 "second_kernel_wide_tiles")}
+        if "cpu_baseline" in record:
+            out["cpu_baseline"] = {k: record["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind", "sample")}
+        return out
+
+    results = {}
+    sub = copy.copy(args)
+    sub.steps, sub.warmup = max(args.steps, 100), max(args.warmup, 10)
+    sub.no_cpu_baseline, sub.oracle_sequences = True, 2
+    results["gqa_decode_ragged"] = brief(run_gqa_decode(sub, ragged=True))
+    torch.cuda.empty_cache()
+    sub = copy.copy(args)
+    sub.steps, sub.warmup = max(args.steps, 100), max(args.warmup, 10)
+    sub.no_cpu_baseline, sub.oracle_sample_ctx, sub.workload = False, 4096, "mla_decode_64k"
+    results["mla_decode_64k"] = brief(bench_extra.workload_record(sub))
+    torch.cuda.empty_cache()
+    sub = copy.copy(args)
+    sub.steps, sub.warmup = 100, 5
+    sub.no_cpu_baseline, sub.workload = False, "gqa_prefill_chunk"
+    results["gqa_prefill_chunk"] = brief(bench_extra.workload_record(sub))
+    torch.cuda.empty_cache()
+    return results
 
 
 def main():
@@ -460,19 +523,25 @@ def main():
         print("bench.py: this build targets one MI355X; --gpus must be 1 (multi-GPU sharding is design-only)", file=sys.stderr)
         sys.exit(2)
     if args.workload == "gqa_decode_32k":
-        run_gqa_decode(args, ragged=False)
+        import torch
+
+        record = run_gqa_decode(args, ragged=False)
+        if not args.no_other_configs:
+            torch.cuda.empty_cache()
+            record["other_configs"] = other_configs(args)
     elif args.workload == "gqa_decode_ragged":
-        run_gqa_decode(args, ragged=True)
+        record = run_gqa_decode(args, ragged=True)
     elif args.workload == "gqa_decode_c1":
-        run_gqa_decode(args, ragged=False, config1=True)
+        record = run_gqa_decode(args, ragged=False, config1=True)
     elif args.workload == "copy_calibration":
-        run_copy_calibration(args)
+        record = run_copy_calibration(args)
     elif args.workload == "append_prologue":
-        run_append_prologue(args)
+        record = run_append_prologue(args)
     else:
         import bench_extra
 
-        bench_extra.run(args)
+        record = bench_extra.workload_record(args)
+    print(json.dumps(record))
 
 
 if __name__ == "__main__":

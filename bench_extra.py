@@ -108,7 +108,10 @@ def run_mla_decode(args):
     ms_step = _wall_ms(graph.replay, replays) / per_graph
     ms_events = _event_ms(graph.replay, replays) / per_graph
     stage_ms = {name: _event_ms(run(mask), args.steps) for name, mask in
-                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge_project", capi.MLA_MERGE | capi.MLA_PROJECT))}
+                (("absorb", capi.MLA_ABSORB), ("partial", capi.MLA_PARTIAL), ("merge_project", capi.MLA_MERGE | capi.MLA_PROJECT),
+                 # the second split-KV kernel (ZLLM_MLA_WIDE_TILES), not the default: timed beside it
+                 ("partial_wide_tiles", capi.MLA_PARTIAL | capi.MLA_WIDE_TILES))}
+    singles = sorted(_event_ms(run(capi.MLA_PARTIAL), 1) for _ in range(max(args.steps, 100)))
     run(0)()
     torch.cuda.synchronize()
     flops = sum(lens) * heads * (2 * (latent + rope) + 2 * latent)  # QK^T over 576 + PV over 512, multiply-add = 2
@@ -131,12 +134,15 @@ def run_mla_decode(args):
         "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
         "roofline": {"bound": "mfma", "kernel": "mla_partial", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel_ms": round(stage_ms["partial"], 5)},
+                     "kernel_ms": round(stage_ms["partial"], 5), "kernel_ms_single_launch_median": round(singles[len(singles) // 2], 5),
+                     "kernel_ms_single_launch_min": round(singles[0], 5),
+                     "second_kernel_wide_tiles": {"kernel_ms": round(stage_ms["partial_wide_tiles"], 5),
+                                                  "frac": round(flops / (stage_ms["partial_wide_tiles"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}},
     }
     if not args.no_cpu_baseline:
         # CPU oracle (port of mla_attention_absorbed_q8_history) on a bounded sample: sequence 0, the first 8 heads,
-        # the first 16,384 tokens of context.
-        sample_heads, sample_ctx = 8, 16384
+        # the first `sample_ctx` tokens of context.
+        sample_heads, sample_ctx = 8, getattr(args, "oracle_sample_ctx", 16384)
         threads = O.set_threads(min(len(os.sched_getaffinity(0)), 16))
         h_codes = ops.gather_rows(codes, tables[0], 0, sample_ctx, latent, bt).cpu().numpy()
         h_scales = ops.gather_rows(scales, tables[0], 0, sample_ctx, latent // 64 * 2, bt).cpu().numpy().view(np.uint16)
@@ -157,7 +163,7 @@ def run_mla_decode(args):
                                codes, scales, rope_cache, tables[0:1].contiguous(), torch.tensor([sample_ctx], dtype=torch.int32, device=dev),
                                sample_heads, nope + rope, nope + value, latent, rope, bt, sample_ctx)
         record["parity_vs_oracle_max_abs"] = float(np.abs(small.cpu().numpy().ravel() - out_f).max())
-    print(json.dumps(record))
+    return record
 
 
 def run_mla_prefill(args):
@@ -247,7 +253,7 @@ def run_mla_prefill(args):
         got = out[rows - sample_rows:].float().cpu().numpy().reshape(sample_rows, heads, value)[:, :sample_heads].reshape(-1)
         excess = np.abs(got - out_f) - np.abs(out_f) * 2.0 ** -7  # bf16 output: beyond one bf16 step of the oracle's unrounded value
         record["parity_vs_oracle_max_abs_beyond_bf16_step"] = float(max(excess.max(), 0.0))
-    print(json.dumps(record))
+    return record
 
 
 def run_gqa_decode_f16(args):
@@ -356,23 +362,25 @@ def run_gqa_decode_f16(args):
         record["cpu_baseline"] = {"value": round(ctx * 2 * hkv * d * 2 / seconds / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                                   "sample": f"sequence 0 of the full layer ({ctx} keys, {hq} heads) on dequantised f32 K/V; {seconds:.2f}s"}
         record["parity_vs_oracle_max_abs"] = worst
-    print(json.dumps(record))
+    return record
+
+
+def workload_record(args):
+    """The JSON record of one secondary workload."""
+    if args.workload == "mla_decode_64k":
+        return run_mla_decode(args)
+    if args.workload == "mla_prefill_chunk":
+        return run_mla_prefill(args)
+    if args.workload == "gqa_decode_f16_window":
+        return run_gqa_decode_f16(args)
+    import bench_prefill
+
+    if args.workload == "gqa_prefill_chunk":
+        return bench_prefill.run(args)
+    if args.workload == "gqa_prefill_f16":
+        return bench_prefill.run_f16(args)
+    raise SystemExit(f"unknown workload {args.workload}")
 
 
 def run(args):
-    if args.workload == "mla_decode_64k":
-        run_mla_decode(args)
-    elif args.workload == "mla_prefill_chunk":
-        run_mla_prefill(args)
-    elif args.workload == "gqa_decode_f16_window":
-        run_gqa_decode_f16(args)
-    elif args.workload == "gqa_prefill_chunk":
-        import bench_prefill
-
-        bench_prefill.run(args)
-    elif args.workload == "gqa_prefill_f16":
-        import bench_prefill
-
-        bench_prefill.run_f16(args)
-    else:
-        raise SystemExit(f"unknown workload {args.workload}")
+    print(json.dumps(workload_record(args)))

@@ -93,7 +93,7 @@ def run(args):
         record["cpu_baseline"] = {"value": round(4 * d * hq * cpu_pairs / (t2 - t1) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
                                   "sample": f"last {sample} rows of the chunk, all heads, full cache; attention {t2 - t1:.2f}s (+ dequantize {t1 - t0:.2f}s, not counted)"}
         record["parity_vs_oracle_max_abs"] = float(np.abs(result[chunk - sample:].cpu().numpy() - want).max())
-    print(json.dumps(record))
+    return record
 
 
 def run_f16(args):
@@ -167,4 +167,4 @@ def run_f16(args):
         record["cpu_baseline"] = {"value": round(4 * d * hq * cpu_pairs / (t2 - t1) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
                                   "sample": f"last {sample} rows of the chunk, all heads, full cache; attention {t2 - t1:.2f}s"}
         record["parity_vs_oracle_max_abs"] = float(np.abs(result[chunk - sample:].cpu().numpy() - want).max())
-    print(json.dumps(record))
+    return record
