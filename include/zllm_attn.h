@@ -362,6 +362,12 @@ typedef struct zllm_gqa_prefill_args {
      * Absolute token positions.  NULL = causal. */
     const uint32_t* visible_ends;  /* [dev] [rows] or NULL */
     uint32_t table_stride;         /* entries in `table` (0 = not stated: the table must cover position + rows) */
+    /* Explicit row ranges, BlockAttentionSpec::visible (src/attention/block.rs:10-16; the varlen and segment forms of
+     * BlockAttentionBackend::block_attention, src/backend/mod.rs:1582-1617, are ranges too): with visible_starts given,
+     * row r attends exactly the cache rows [visible_starts[r], min(visible_ends[r], position + rows)) -- no causal
+     * rule, no window (window must be 0, visible_ends must be given); an empty range gives a zero row.  `position +
+     * rows` is then only the number of cache rows the call may read. */
+    const uint32_t* visible_starts; /* [dev] [rows] or NULL */
 } zllm_gqa_prefill_args;
 ZLLM_API uint64_t zllm_attn_gqa_prefill_workspace_bytes(const zllm_gqa_prefill_args* args);
 ZLLM_API int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* args, zllm_stream_t stream);

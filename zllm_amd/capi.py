@@ -82,7 +82,7 @@ class GqaPrefillArgs(C.Structure):
                 ("position", _u32), ("window", _u32), ("num_heads", _u32), ("num_kv_heads", _u32), ("head_dim", _u32),
                 ("block_tokens", _u32), ("score_scale", _f32), ("softcap", _f32), ("kv_format", _int),
                 ("scale_dtype", _int), ("q_dtype", _int), ("out_dtype", _int), ("gate", _ptr), ("gate_cols", _u32),
-                ("gate_dtype", _int), ("visible_ends", _ptr), ("table_stride", _u32)]
+                ("gate_dtype", _int), ("visible_ends", _ptr), ("table_stride", _u32), ("visible_starts", _ptr)]
 
 
 class MlaDecodeArgs(C.Structure):

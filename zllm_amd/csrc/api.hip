@@ -951,6 +951,11 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     if (a->q_dtype < ZLLM_DTYPE_F32 || a->q_dtype > ZLLM_DTYPE_F16 || a->out_dtype < ZLLM_DTYPE_F32 || a->out_dtype > ZLLM_DTYPE_F16) {
         return fail(-1, "GQA prefill: unknown q_dtype %d / out_dtype %d", a->q_dtype, a->out_dtype);
     }
+    // explicit row ranges (BlockAttentionSpec::visible, src/attention/block.rs:10-16) come as two arrays and replace the
+    // causal window altogether
+    if (a->visible_starts != nullptr && (a->visible_ends == nullptr || a->window != 0)) {
+        return fail(-1, "GQA prefill: visible_starts needs visible_ends and window == 0 (got window=%u)", a->window);
+    }
     return 0;
 }
 
@@ -1131,7 +1136,7 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
         }
         uint32_t* lens = (uint32_t*)a->workspace;
         uint32_t* first = lens + a->rows;
-        int rc2 = hip_status(zllm::launch_prefill_row_ranges(lens, first, a->visible_ends, a->rows, a->position, a->window, (hipStream_t)stream),
+        int rc2 = hip_status(zllm::launch_prefill_row_ranges(lens, first, a->visible_ends, a->visible_starts, a->rows, a->position, a->window, (hipStream_t)stream),
                              "GQA prefill row ranges launch");
         if (rc2 != 0) {
             return rc2;
@@ -1145,6 +1150,7 @@ int zllm_attn_gqa_prefill_chunk(const zllm_gqa_prefill_args* a, zllm_stream_t st
     zllm::GqaPrefillParams p;
     memset(&p, 0, sizeof(p));
     p.visible_ends = a->visible_ends;
+    p.visible_starts = a->visible_starts;
     p.q = a->q;
     p.k_plane = (const unsigned char*)a->k_plane;
     p.k_scales = (const unsigned char*)a->k_scales;

@@ -1565,7 +1565,8 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_few(GqaDecodeParams p)
 // decode kernels: lens[r] = end and first[r] = start of key_range(position + r, position + rows), or of
 // key_range_with_visible_end when the row carries an explicit end (src/attention/gqa.rs:54-68).
 __global__ __launch_bounds__(256) void prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends,
-                                                          unsigned int rows, unsigned int position, unsigned int window)
+                                                          const unsigned int* visible_starts, unsigned int rows, unsigned int position,
+                                                          unsigned int window)
 {
     const unsigned int r = blockIdx.x * 256u + threadIdx.x;
     if (r >= rows) {
@@ -1574,6 +1575,12 @@ __global__ __launch_bounds__(256) void prefill_row_ranges(unsigned int* lens, un
     const unsigned int pos = position + r;
     unsigned int end = pos + 1u;
     const unsigned int start = (window != 0 && end > window) ? end - window : 0u;
+    if (visible_starts != nullptr) { // an explicit range (BlockAttentionSpec::visible, src/attention/block.rs:10-16): taken as given
+        const unsigned int given_end = min(visible_ends[r], position + rows);
+        lens[r] = given_end;
+        first[r] = min(visible_starts[r], given_end);
+        return;
+    }
     if (visible_ends != nullptr) {
         end = min(max(end, visible_ends[r]), position + rows);
     }
@@ -1694,10 +1701,10 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& args, int kv_format, int sca
     return launch_split_merge(p, stream);
 }
 
-hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, unsigned int rows,
-                                     unsigned int position, unsigned int window, hipStream_t stream)
+hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, const unsigned int* visible_starts,
+                                     unsigned int rows, unsigned int position, unsigned int window, hipStream_t stream)
 {
-    prefill_row_ranges<<<dim3((rows + 255u) / 256u), dim3(256), 0, stream>>>(lens, first, visible_ends, rows, position, window);
+    prefill_row_ranges<<<dim3((rows + 255u) / 256u), dim3(256), 0, stream>>>(lens, first, visible_ends, visible_starts, rows, position, window);
     return hipGetLastError();
 }
 

@@ -177,13 +177,21 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     // key_range_with_visible_end when rows carry an explicit visible end (src/attention/gqa.rs:65-68)
     const unsigned int last_row = min(row0 + rows_per_wg, p.rows) - 1u;
     unsigned int t_end = p.position + last_row + 1u;
-    if (p.visible_ends != nullptr) {
+    unsigned int t_begin = 0;
+    if (p.visible_starts != nullptr) { // explicit ranges (src/attention/block.rs:10-16): the union of the rows' own
+        t_end = 0u;
+        t_begin = 0xffffffffu;
+        for (unsigned int r = row0; r <= last_row; ++r) { // uniform over the workgroup: scalar loads
+            const unsigned int given_end = min(p.visible_ends[r], p.position + p.rows);
+            t_end = max(t_end, given_end);
+            t_begin = min(t_begin, min(p.visible_starts[r], given_end));
+        }
+    } else if (p.visible_ends != nullptr) {
         for (unsigned int r = row0; r <= last_row; ++r) { // uniform over the workgroup: scalar loads
             t_end = max(t_end, min(p.visible_ends[r], p.position + p.rows));
         }
     }
-    unsigned int t_begin = 0;
-    if (p.window != 0) {
+    if (p.window != 0 && p.visible_starts == nullptr) {
         const unsigned int first_pos = p.position + row0 + 1u;
         t_begin = first_pos > p.window ? first_pos - p.window : 0u;
     }
@@ -342,11 +350,15 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
         ref_shift[ct] = kPBias;
         const unsigned int pos = p.position + col_row[ct];
         unsigned int hi = pos + 1u;
-        if (p.visible_ends != nullptr && col_valid[ct]) { // a row may read past itself, up to the end of the chunk
+        unsigned int lo = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+        if (p.visible_starts != nullptr && col_valid[ct]) { // the row's range as given
+            hi = min(p.visible_ends[col_row[ct]], p.position + p.rows);
+            lo = min(p.visible_starts[col_row[ct]], hi);
+        } else if (p.visible_ends != nullptr && col_valid[ct]) { // a row may read past itself, up to the end of the chunk
             hi = min(max(hi, p.visible_ends[col_row[ct]]), p.position + p.rows);
         }
         vis_hi[ct] = col_valid[ct] ? hi : 0u;
-        vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+        vis_lo[ct] = lo;
     }
 
     // first token some column of the wave cannot see any more / last token some column does not see yet (wave-uniform)
@@ -701,13 +713,21 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     // visible token range of the workgroup, as in gqa_prefill_q8
     const unsigned int last_row = min(row0 + rows_per_wg, p.rows) - 1u;
     unsigned int t_end = p.position + last_row + 1u;
-    if (p.visible_ends != nullptr) {
+    unsigned int t_begin = 0;
+    if (p.visible_starts != nullptr) { // explicit ranges (src/attention/block.rs:10-16): the union of the rows' own
+        t_end = 0u;
+        t_begin = 0xffffffffu;
+        for (unsigned int r = row0; r <= last_row; ++r) {
+            const unsigned int given_end = min(p.visible_ends[r], p.position + p.rows);
+            t_end = max(t_end, given_end);
+            t_begin = min(t_begin, min(p.visible_starts[r], given_end));
+        }
+    } else if (p.visible_ends != nullptr) {
         for (unsigned int r = row0; r <= last_row; ++r) {
             t_end = max(t_end, min(p.visible_ends[r], p.position + p.rows));
         }
     }
-    unsigned int t_begin = 0;
-    if (p.window != 0) {
+    if (p.window != 0 && p.visible_starts == nullptr) {
         const unsigned int first_pos = p.position + row0 + 1u;
         t_begin = first_pos > p.window ? first_pos - p.window : 0u;
     }
@@ -900,11 +920,15 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
         ref_shift[ct] = kPBias;
         const unsigned int pos = p.position + col_row[ct];
         unsigned int hi = pos + 1u;
-        if (p.visible_ends != nullptr && col_valid[ct]) {
+        unsigned int lo = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+        if (p.visible_starts != nullptr && col_valid[ct]) { // the row's range as given
+            hi = min(p.visible_ends[col_row[ct]], p.position + p.rows);
+            lo = min(p.visible_starts[col_row[ct]], hi);
+        } else if (p.visible_ends != nullptr && col_valid[ct]) { // a row may read past itself, up to the end of the chunk
             hi = min(max(hi, p.visible_ends[col_row[ct]]), p.position + p.rows);
         }
         vis_hi[ct] = col_valid[ct] ? hi : 0u;
-        vis_lo[ct] = (p.window != 0 && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+        vis_lo[ct] = lo;
         wave_min_hi = min(wave_min_hi, vis_hi[ct]);
         wave_max_lo = max(wave_max_lo, vis_lo[ct]);
     }

@@ -126,6 +126,7 @@ struct GqaPrefillParams {
     unsigned int gate_cols;
     int gate_dtype;
     const unsigned int* visible_ends; // optional [rows]: row r reads up to max(position + r + 1, visible_ends[r])
+    const unsigned int* visible_starts; // optional [rows], with visible_ends: row r reads exactly [visible_starts[r], visible_ends[r])
     // KV splits of a chunk that has too few row tiles for the CUs: workgroup z of a row tile attends part z of the tile's
     // visible range (equal 32-aligned parts of at most chunk_tokens) and leaves un-normalised records for the split merge:
     // partial [rows][max_chunks][num_heads][head_dim], stats [rows][max_chunks][num_heads][2] = (max, sum).  max_chunks <= 1:
@@ -191,8 +192,9 @@ hipError_t launch_mla_partial_x32(const MlaDecodeParams& p, hipStream_t stream);
 // LSE combine of split records: uses kv_lens, first_visible, partial, stats, out, batch, num_heads,
 // head_dim, chunk_tokens, max_chunks of the parameter block.
 hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream);
-// lens[r], first[r] = visible range of row r of a prefill chunk (window 0 = full causal; visible_ends optional)
-hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, unsigned int rows,
+// lens[r], first[r] = visible range of row r of a prefill chunk (window 0 = full causal; visible_ends optional; with
+// visible_starts the range is [visible_starts[r], visible_ends[r]) as given)
+hipError_t launch_prefill_row_ranges(unsigned int* lens, unsigned int* first, const unsigned int* visible_ends, const unsigned int* visible_starts, unsigned int rows,
                                      unsigned int position, unsigned int window, hipStream_t stream);
 
 } // namespace zllm

@@ -142,7 +142,8 @@ def gqa_decode_static(*a, **kw):
 
 def gqa_prefill_chunk_args(q, k_plane, k_scales, v_plane, v_scales, table, position, num_heads, num_kv_heads, head_dim,
                            block_tokens, score_scale, window=0, softcap=0.0, kv_format=capi.KV_Q8G64,
-                           scale_dtype=capi.SCALE_F16, out_dtype=torch.float32, gate=None, visible_ends=None, workspace=True):
+                           scale_dtype=capi.SCALE_F16, out_dtype=torch.float32, gate=None, visible_ends=None, workspace=True,
+                           visible_starts=None):
     """The argument block of zllm_attn_gqa_prefill_chunk, the output tensor and the workspace tensor (None without one):
     for callers that launch the same call many times."""
     rows = q.shape[0]
@@ -158,6 +159,7 @@ def gqa_prefill_chunk_args(q, k_plane, k_scales, v_plane, v_scales, table, posit
     if gate is not None:
         args.gate, args.gate_cols, args.gate_dtype = _ptr(gate), gate.shape[1], _DTYPE[gate.dtype]
     args.visible_ends = _ptr(visible_ends)
+    args.visible_starts = _ptr(visible_starts)
     args.table_stride = 0 if table is None else table.numel()
     scratch = None
     if workspace:
