@@ -29,6 +29,8 @@ int zo_gather_rows_bytes(const uint8_t* plane, const uint32_t* block_table, uint
 int zo_gqa_prefill_at_visible_f32(const float* query, const float* key, const float* value, uint64_t query_tokens, uint64_t kv_start,
                                   uint64_t kv_end, uint64_t position, uint64_t num_heads, uint64_t num_kv_heads, uint64_t head_dim,
                                   uint64_t window, float score_scale, float softcap, const uint32_t* visible_ends, float* output);
+int zo_block_attention_f32(const float* query, const float* key, const float* value, uint64_t query_rows, uint64_t kv_rows, uint64_t num_heads,
+                           uint64_t num_kv_heads, uint64_t head_dim, float score_scale, const uint32_t* visible, float* output);
 int zo_rope_apply_f32(float* data, uint64_t rows, uint64_t columns, uint64_t head_count, uint64_t rotary_dim, uint64_t position,
                       const float* cosine, const float* sine, uint64_t table_len, int layout, int placement);
 typedef struct {
@@ -559,6 +561,269 @@ static void test_mla_prefill(const RocmContext& ctx)
           "a prefill without a cache must be refused");
 }
 
+// Backend::gqa_prefill_attention{,_visible}: a chunk over its own dense K/V, compared with the oracle on the f32 K/V the
+// reference's device path reads (src/backend/rocm/attention.rs:2151-2199) -- the f16 planes in between must stay inside the bound
+static void test_gqa_uncached(const RocmContext& ctx)
+{
+    std::mt19937 rng(41);
+    struct Case {
+        size_t heads, kv_heads, dim, rows;
+        CausalWindow window;
+        DType q_dtype;
+    };
+    const Case cases[] = {{16, 4, 128, 300, CausalWindow::Full(), DType::BF16},
+                          {8, 2, 128, 777, CausalWindow::Sliding(200), DType::F32},
+                          {8, 4, 256, 130, CausalWindow::Full(), DType::BF16},
+                          {4, 1, 128, 1, CausalWindow::Full(), DType::F32}};
+    for (const Case& c : cases) {
+        GqaSpec spec;
+        spec.num_heads = c.heads;
+        spec.num_kv_heads = c.kv_heads;
+        spec.head_dim = c.dim;
+        spec.window = c.window;
+        spec.score_scale = 1.0f / sqrtf((float)c.dim);
+        const size_t q_cols = c.heads * c.dim, kv_cols = c.kv_heads * c.dim;
+        const auto q = randn(rng, c.rows * q_cols, c.q_dtype == DType::BF16);
+        const auto k = randn(rng, c.rows * kv_cols, false);
+        const auto v = randn(rng, c.rows * kv_cols, false);
+        auto qt = ctx.tensor_from_f32(q, c.rows, q_cols, c.q_dtype);
+        auto kt = ctx.tensor_from_f32(k, c.rows, kv_cols);
+        auto vt = ctx.tensor_from_f32(v, c.rows, kv_cols);
+        auto out = ctx.gqa_prefill_attention(qt.unwrap(), kt.unwrap(), vt.unwrap(), spec);
+        CHECK(out.is_ok(), "gqa_prefill_attention: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        std::vector<float> want(c.rows * q_cols);
+        int rc = zo_gqa_prefill_at_visible_f32(q.data(), k.data(), v.data(), c.rows, 0, c.rows, 0, c.heads, c.kv_heads, c.dim,
+                                               c.window.sliding ? c.window.size : 0, spec.score_scale, 0.0f, nullptr, want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        char what[128];
+        snprintf(what, sizeof(what), "gqa_prefill_attention %zux%zu d=%zu rows=%zu%s", c.heads, c.kv_heads, c.dim, c.rows, c.window.sliding ? " sliding" : "");
+        if (out.is_ok()) {
+            compare(ctx.tensor_to_f32(out.unwrap()).unwrap(), want, what);
+        }
+        // right-padded text: the rows of the first 100 tokens (or all) see to the end of that stretch
+        std::vector<uint32_t> ends(c.rows);
+        const size_t text = std::min<size_t>(c.rows, 100);
+        for (size_t r = 0; r < c.rows; ++r) {
+            ends[r] = (uint32_t)(r < text ? text : r + 1);
+        }
+        auto seen = ctx.gqa_prefill_attention_visible(qt.unwrap(), kt.unwrap(), vt.unwrap(), spec, ends);
+        CHECK(seen.is_ok(), "gqa_prefill_attention_visible: %s", seen.is_err() ? seen.unwrap_err().to_string().c_str() : "");
+        rc = zo_gqa_prefill_at_visible_f32(q.data(), k.data(), v.data(), c.rows, 0, c.rows, 0, c.heads, c.kv_heads, c.dim,
+                                           c.window.sliding ? c.window.size : 0, spec.score_scale, 0.0f, ends.data(), want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        snprintf(what, sizeof(what), "gqa_prefill_attention_visible %zux%zu d=%zu rows=%zu", c.heads, c.kv_heads, c.dim, c.rows);
+        if (seen.is_ok()) {
+            compare(ctx.tensor_to_f32(seen.unwrap()).unwrap(), want, what);
+        }
+        ends.pop_back();
+        CHECK(ctx.gqa_prefill_attention_visible(qt.unwrap(), kt.unwrap(), vt.unwrap(), spec, ends).is_err(), "one visible end too few must be refused");
+        CHECK(ctx.gqa_prefill_attention(qt.unwrap(), qt.unwrap(), vt.unwrap(), spec).is_err() || c.heads == c.kv_heads, "a K of the wrong width must be refused");
+    }
+}
+
+// BlockAttentionBackend: the reference's own vectors (src/attention/block.rs:125-141), varlen segments, free ranges, the
+// prefix + suffix form, and the offsets and ranges BlockAttentionSpec refuses
+static void test_block_attention(const RocmContext& ctx)
+{
+    const size_t d = 128;
+    const GqaGeometry one{1, 1, d};
+    {
+        // zero queries: every row is the mean of the values it sees
+        const float values5[] = {2, 4, 6, 20, 40}, values3[] = {2, 6, 10};
+        auto varlen = BlockAttentionSpec::varlen(one, 3, 5, {0, 2, 3}, {0, 3, 5}, 1.0f);
+        CHECK(varlen.is_ok(), "varlen offsets of the reference's test");
+        BlockAttentionSpec free_ranges;
+        free_ranges.geometry = one;
+        free_ranges.score_scale = 1.0f;
+        free_ranges.visible = {{0, 2}, {1, 3}};
+        struct Vec {
+            const float* values;
+            size_t kv_rows, q_rows;
+            const BlockAttentionSpec* spec;
+            float want[3];
+        } vectors[] = {{values5, 5, 3, &varlen.unwrap(), {4, 4, 30}}, {values3, 3, 2, &free_ranges, {4, 8, 0}}};
+        for (const Vec& vec : vectors) {
+            std::vector<float> v(vec.kv_rows * d, 0.0f), zeros_kv(vec.kv_rows * d, 0.0f), zeros_q(vec.q_rows * d, 0.0f);
+            for (size_t r = 0; r < vec.kv_rows; ++r) {
+                v[r * d] = vec.values[r];
+            }
+            auto out = ctx.block_attention(ctx.tensor_from_f32(zeros_q, vec.q_rows, d).unwrap(), ctx.tensor_from_f32(zeros_kv, vec.kv_rows, d).unwrap(),
+                                           ctx.tensor_from_f32(v, vec.kv_rows, d).unwrap(), *vec.spec);
+            CHECK(out.is_ok(), "block_attention vector: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+            if (out.is_ok()) {
+                const auto got = ctx.tensor_to_f32(out.unwrap()).unwrap();
+                for (size_t r = 0; r < vec.q_rows; ++r) {
+                    CHECK(fabsf(got[r * d] - vec.want[r]) <= 2e-3f * vec.want[r], "block vector row %zu: %g, the reference holds %g", r, got[r * d], vec.want[r]);
+                    CHECK(got[r * d + 1] == 0.0f, "block vector row %zu column 1: %g", r, got[r * d + 1]);
+                }
+            }
+        }
+        // the offsets the reference's test refuses
+        const std::vector<size_t> bad[][2] = {{{0, 2}, {0, 5}}, {{0, 0, 3}, {0, 3, 5}}, {{1, 2, 3}, {0, 3, 5}},
+                                              {{0, 4, 3}, {0, 3, 5}}, {{0, 2, 3}, {0, 5}}, {{0, 2, 3}, {0, 5, 5}}};
+        for (const auto& pair : bad) {
+            CHECK(BlockAttentionSpec::varlen(one, 3, 5, pair[0], pair[1], 1.0f).is_err(), "varlen offsets that must be refused");
+        }
+    }
+    std::mt19937 rng(43);
+    const GqaGeometry geometry{8, 2, 128};
+    const size_t q_cols = 8 * 128, kv_cols = 2 * 128;
+    const float scale = 1.0f / sqrtf(128.0f);
+    // isolated sequences packed into one call, query and KV segments of different lengths
+    {
+        const std::vector<size_t> q_off = {0, 1, 40, 340, 357}, kv_off = {0, 700, 733, 1500, 1501};
+        const size_t q_rows = q_off.back(), kv_rows = kv_off.back();
+        auto spec = BlockAttentionSpec::varlen(geometry, q_rows, kv_rows, q_off, kv_off, scale);
+        CHECK(spec.is_ok(), "varlen spec");
+        const auto q = randn(rng, q_rows * q_cols, true);
+        const auto k = randn(rng, kv_rows * kv_cols, false);
+        const auto v = randn(rng, kv_rows * kv_cols, false);
+        std::vector<uint32_t> flat;
+        for (const auto& range : spec.unwrap().visible) {
+            flat.push_back((uint32_t)range.first);
+            flat.push_back((uint32_t)range.second);
+        }
+        std::vector<float> want(q_rows * q_cols);
+        const int rc = zo_block_attention_f32(q.data(), k.data(), v.data(), q_rows, kv_rows, 8, 2, 128, scale, flat.data(), want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        auto qt = ctx.tensor_from_f32(q, q_rows, q_cols, DType::BF16);
+        auto out = ctx.block_attention(qt.unwrap(), ctx.tensor_from_f32(k, kv_rows, kv_cols).unwrap(), ctx.tensor_from_f32(v, kv_rows, kv_cols).unwrap(),
+                                       spec.unwrap());
+        CHECK(out.is_ok(), "block_attention varlen: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_ok()) {
+            compare(ctx.tensor_to_f32(out.unwrap()).unwrap(), want, "block_attention, varlen segments 357 x 1501");
+        }
+        // the same K/V handed over as a resident prefix and a short suffix
+        const size_t cut = 1437;
+        std::vector<float> k_head(k.begin(), k.begin() + cut * kv_cols), k_tail(k.begin() + cut * kv_cols, k.end());
+        std::vector<float> v_head(v.begin(), v.begin() + cut * kv_cols), v_tail(v.begin() + cut * kv_cols, v.end());
+        auto split = ctx.block_attention_prefix_suffix(qt.unwrap(), ctx.tensor_from_f32(k_head, cut, kv_cols, DType::BF16).unwrap(),
+                                                       ctx.tensor_from_f32(v_head, cut, kv_cols, DType::BF16).unwrap(),
+                                                       ctx.tensor_from_f32(k_tail, kv_rows - cut, kv_cols).unwrap(),
+                                                       ctx.tensor_from_f32(v_tail, kv_rows - cut, kv_cols).unwrap(), spec.unwrap());
+        CHECK(split.is_ok(), "block_attention_prefix_suffix: %s", split.is_err() ? split.unwrap_err().to_string().c_str() : "");
+        if (split.is_ok()) {
+            // the prefix arrives as bf16 here (a cache kept in bf16): the oracle reads what the planes hold
+            std::vector<float> k_seen = k, v_seen = v;
+            for (size_t i = 0; i < cut * kv_cols; ++i) {
+                k_seen[i] = zo_bf16_to_f32(zo_f32_to_bf16(k[i]));
+                v_seen[i] = zo_bf16_to_f32(zo_f32_to_bf16(v[i]));
+            }
+            const int rc2 = zo_block_attention_f32(q.data(), k_seen.data(), v_seen.data(), q_rows, kv_rows, 8, 2, 128, scale, flat.data(), want.data());
+            CHECK(rc2 == 0, "oracle rc %d", rc2);
+            compare(ctx.tensor_to_f32(split.unwrap()).unwrap(), want, "block_attention_prefix_suffix, bf16 prefix 1437 + f32 suffix 64");
+        }
+    }
+    // free ranges (not monotone, not causal), one-key rows, more query rows than KV rows
+    {
+        const size_t q_rows = 200, kv_rows = 90;
+        BlockAttentionSpec spec;
+        spec.geometry = geometry;
+        spec.score_scale = scale;
+        std::vector<uint32_t> flat;
+        for (size_t r = 0; r < q_rows; ++r) {
+            const size_t start = rng() % kv_rows;
+            const size_t end = r % 7 == 0 ? start + 1 : start + 1 + rng() % (kv_rows - start);
+            spec.visible.emplace_back(start, end);
+            flat.push_back((uint32_t)start);
+            flat.push_back((uint32_t)end);
+        }
+        const auto q = randn(rng, q_rows * q_cols, false);
+        const auto k = randn(rng, kv_rows * kv_cols, false);
+        const auto v = randn(rng, kv_rows * kv_cols, false);
+        std::vector<float> want(q_rows * q_cols);
+        const int rc = zo_block_attention_f32(q.data(), k.data(), v.data(), q_rows, kv_rows, 8, 2, 128, scale, flat.data(), want.data());
+        CHECK(rc == 0, "oracle rc %d", rc);
+        auto out = ctx.block_attention(ctx.tensor_from_f32(q, q_rows, q_cols).unwrap(), ctx.tensor_from_f32(k, kv_rows, kv_cols).unwrap(),
+                                       ctx.tensor_from_f32(v, kv_rows, kv_cols).unwrap(), spec);
+        CHECK(out.is_ok(), "block_attention free ranges: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_ok()) {
+            compare(ctx.tensor_to_f32(out.unwrap()).unwrap(), want, "block_attention, free ranges, 200 rows over 90 keys");
+        }
+        auto qt = ctx.tensor_from_f32(q, q_rows, q_cols).unwrap(), kt = ctx.tensor_from_f32(k, kv_rows, kv_cols).unwrap();
+        BlockAttentionSpec bad = spec;
+        bad.visible[5] = {7, 7};
+        CHECK(ctx.block_attention(qt, kt, kt, bad).is_err(), "an empty range must be refused");
+        bad.visible[5] = {7, kv_rows + 1};
+        CHECK(ctx.block_attention(qt, kt, kt, bad).is_err(), "a range past the KV rows must be refused");
+        bad = spec;
+        bad.visible.pop_back();
+        CHECK(ctx.block_attention(qt, kt, kt, bad).is_err(), "one range too few must be refused");
+        bad = spec;
+        bad.score_scale = 0.0f;
+        CHECK(ctx.block_attention(qt, kt, kt, bad).is_err(), "a score scale of zero must be refused");
+        CHECK(ctx.block_attention(qt, qt, kt, spec).is_err(), "a K of the wrong width must be refused");
+    }
+}
+
+// A decode loop in steady state: after the first steps the context neither allocates device memory, nor uploads rotary
+// tables again, nor waits for its stream -- outputs come from the pool, tables stay resident, small arrays ride the pinned ring
+static void test_steady_state_counters(const RocmContext& ctx)
+{
+    std::mt19937 rng(47);
+    MlaSpec spec;
+    spec.kv_lora_rank = 512;
+    spec.qk_rope_head_dim = 64;
+    spec.num_heads = 16;
+    spec.q_projection_size = spec.num_heads * 192;
+    spec.kv_projection_size = spec.num_heads * 256;
+    spec.q_lora_rank = 1536;
+    const size_t half = 32, table_rows = 4096;
+    std::vector<float> cos(table_rows * half), sin(table_rows * half);
+    for (size_t pos = 0; pos < table_rows; ++pos) {
+        for (size_t i = 0; i < half; ++i) {
+            const float angle = (float)pos * powf(10000.0f, -2.0f * (float)i / 64.0f);
+            cos[pos * half + i] = cosf(angle);
+            sin[pos * half + i] = sinf(angle);
+        }
+    }
+    auto cache_r = RocmKvCache::new_mla(1, 512, 64, 64, 2048, TablePolicy::Scrambled);
+    CHECK(cache_r.is_ok(), "cache");
+    RocmKvCache cache = cache_r.unwrap();
+    std::vector<float> kv_b = randn(rng, spec.kv_projection_size * 512, true);
+    auto weight = ctx.prepare_mla_kv_b(kv_b, spec.kv_projection_size, 512);
+    auto latent = ctx.tensor_from_f32(randn(rng, 512, false), 1, 512);
+    auto rope = ctx.tensor_from_f32(randn(rng, 64, false), 1, 64);
+    auto query = ctx.tensor_from_f32(randn(rng, spec.q_projection_size, true), 1, spec.q_projection_size, DType::BF16);
+    GqaSpec gqa;
+    gqa.num_heads = 8;
+    gqa.num_kv_heads = 2;
+    gqa.head_dim = 128;
+    gqa.score_scale = 1.0f / sqrtf(128.0f);
+    auto gqa_cache_r = RocmKvCache::new_gqa(1, 2, 128, 16, 2048, TablePolicy::Scrambled);
+    CHECK(gqa_cache_r.is_ok(), "cache");
+    RocmKvCache gqa_cache = gqa_cache_r.unwrap();
+    auto gq = ctx.tensor_from_f32(randn(rng, 8 * 128, true), 1, 8 * 128, DType::BF16);
+    auto gk = ctx.tensor_from_f32(randn(rng, 2 * 128, false), 1, 2 * 128);
+    HostCounters settled;
+    const size_t steps = 150, warm = 20;
+    for (size_t step = 0; step < steps; ++step) {
+        if (step == warm) {
+            settled = ctx.counters();
+        }
+        auto appended = ctx.append_mla_rope(cache, 0, latent.unwrap(), rope.unwrap(), 64, RotaryLayout::SplitHalf, step, cos, sin);
+        CHECK(appended.is_ok(), "append_mla_rope step %zu: %s", step, appended.is_err() ? appended.unwrap_err().to_string().c_str() : "");
+        auto out = ctx.mla_decode_attention(query.unwrap(), cache, weight.unwrap(), 0, step, spec);
+        CHECK(out.is_ok(), "mla_decode_attention step %zu", step);
+        const std::vector<uint32_t> ends = {(uint32_t)(step + 1)};
+        auto gout = ctx.gqa_prefill_attention_cached_visible(gqa_cache, 0, step, gq.unwrap(), gk.unwrap(), gk.unwrap(), gqa, ends, true);
+        CHECK(gout.is_ok(), "gqa decode step %zu: %s", step, gout.is_err() ? gout.unwrap_err().to_string().c_str() : "");
+    }
+    const HostCounters after = ctx.counters();
+    printf("steady state over %zu steps: allocations %zu -> %zu, rope uploads %zu -> %zu, stream waits %zu -> %zu, staged uploads %zu -> %zu\n",
+           steps - warm, settled.device_allocations, after.device_allocations, settled.rope_table_uploads, after.rope_table_uploads,
+           settled.stream_waits, after.stream_waits, settled.staged_uploads, after.staged_uploads);
+    CHECK(after.device_allocations == settled.device_allocations, "a decode loop in steady state must not allocate device memory");
+    // the first call committed 16,384 elements, 512 positions of 32: nothing more to send for positions 20..149
+    CHECK(after.rope_table_uploads == settled.rope_table_uploads && settled.rope_table_uploads >= 1, "rotary tables must stay resident: %zu uploads",
+          after.rope_table_uploads - settled.rope_table_uploads);
+    // 130 steps of two metadata records each: the 256-record ring wraps once
+    CHECK(after.stream_waits - settled.stream_waits <= 1, "a decode loop in steady state must not wait for its stream: %zu waits",
+          after.stream_waits - settled.stream_waits);
+    CHECK(after.staged_uploads - settled.staged_uploads == steps - warm, "visible ends must travel through the pinned ring");
+    CHECK(ctx.synchronize().is_ok(), "synchronize");
+}
+
 int main()
 {
     auto ctx = RocmContext::create(0);
@@ -579,6 +844,9 @@ int main()
     test_gqa_shared_and_visible(ctx.unwrap());
     test_mla(ctx.unwrap());
     test_mla_prefill(ctx.unwrap());
+    test_gqa_uncached(ctx.unwrap());
+    test_block_attention(ctx.unwrap());
+    test_steady_state_counters(ctx.unwrap());
     printf(failures == 0 ? "ALL PASSED\n" : "%d FAILED\n", failures);
     return failures == 0 ? 0 : 1;
 }

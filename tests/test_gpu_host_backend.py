@@ -1,7 +1,9 @@
 """Runs the C++ host layer's parity driver (tests/host/backend_parity.cpp): the reference-shaped backend methods
-(gqa_prefill_attention_cached and its _visible / _from forms, append_mla, append_mla_rope, mla_decode_attention,
-mla_prefill_attention) over the C ABI, compared with the CPU oracle inside the driver, plus their error behaviour, the
-grow-by-doubling rule of the cache planes and the ring of a sliding-window layer.  The binary is built by __graft_entry__.build()."""
+(gqa_prefill_attention and its _visible form over dense K/V, gqa_prefill_attention_cached and its _visible / _from forms,
+block_attention and its prefix + suffix form with the reference's own vectors, append_mla, append_mla_rope,
+mla_decode_attention, mla_prefill_attention) over the C ABI, compared with the CPU oracle inside the driver, plus their
+error behaviour, the grow-by-doubling rule of the cache planes, the ring of a sliding-window layer, and the counters that
+show a decode loop in steady state neither allocating, nor uploading rotary tables again, nor waiting for its stream.  The binary is built by __graft_entry__.build()."""
 import os
 import subprocess
 

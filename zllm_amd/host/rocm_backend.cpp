@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <map>
 #include <numeric>
 
 #include "../../include/zllm_attn.h"
@@ -127,6 +128,14 @@ Result<DeviceBuffer> DeviceBuffer::allocate(size_t bytes)
     }
     DeviceBuffer out;
     out.ptr_ = std::shared_ptr<void>(raw, [](void* p) { (void)hipFree(p); });
+    out.bytes_ = bytes;
+    return out;
+}
+
+DeviceBuffer DeviceBuffer::adopt(std::shared_ptr<void> block, size_t bytes)
+{
+    DeviceBuffer out;
+    out.ptr_ = std::move(block);
     out.bytes_ = bytes;
     return out;
 }
@@ -378,16 +387,57 @@ Result<MlaLayerSerde> read_mla_layer(const std::vector<uint8_t>& in, size_t& off
 // ---------------------------------------------------------------------------------------------- context
 struct RocmContext::Scratch {
     static constexpr size_t kSlots = 256;
+    static constexpr size_t kStageBytes = 1 << 20;       // pinned ring for small arrays
+    static constexpr size_t kPoolKeepBytes = 2ull << 30; // idle blocks kept beyond this are released
     hipStream_t stream = nullptr;
     DeviceBuffer workspace;
     uint32_t* meta_host = nullptr; // pinned, kSlots records of four u32
     DeviceBuffer meta_dev;
     size_t next = 0;
+    uint8_t* stage_host = nullptr; // pinned, kStageBytes
+    size_t stage_next = 0;
+    // idle blocks by capacity; a block is reused for a request of at least half its size
+    std::multimap<size_t, void*> idle;
+    size_t idle_bytes = 0;
+    DeviceBuffer identity;         // u32 [identity_pages]: 0, 1, 2, ...
+    size_t identity_pages = 0;
+    struct RopeTables {
+        const float *cos_host, *sin_host; // identity of the host tables, as the reference keys them
+        size_t host_elements, elements;   // length of the host tables, committed prefix
+        float first, last;                // cos[0] and cos[elements - 1] when committed: a reused address is told apart
+        DeviceBuffer cos, sin;
+    };
+    std::vector<RopeTables> rope;
+    HostCounters counters;
     ~Scratch()
     {
         if (meta_host != nullptr) {
             (void)hipHostFree(meta_host);
         }
+        if (stage_host != nullptr) {
+            (void)hipHostFree(stage_host);
+        }
+        for (auto& block : idle) {
+            (void)hipFree(block.second);
+        }
+    }
+    static size_t size_class(size_t bytes)
+    {
+        // powers of two up to 1 MiB, then multiples of 1 MiB: a decode loop's outputs all land in one class
+        size_t cls = 256;
+        while (cls < bytes && cls < (1u << 20)) {
+            cls *= 2;
+        }
+        return cls >= bytes ? cls : (bytes + (1u << 20) - 1) >> 20 << 20;
+    }
+    void give_back(void* block, size_t capacity)
+    {
+        if (idle_bytes + capacity > kPoolKeepBytes) {
+            (void)hipFree(block);
+            return;
+        }
+        idle.emplace(capacity, block);
+        idle_bytes += capacity;
     }
 };
 
@@ -418,8 +468,169 @@ Result<RocmContext> RocmContext::create(int device_id)
         return meta.unwrap_err();
     }
     scratch->meta_dev = meta.unwrap();
+    err = hipHostMalloc((void**)&scratch->stage_host, Scratch::kStageBytes, hipHostMallocDefault);
+    if (err != hipSuccess) {
+        return hip_error("pinned staging ring", err);
+    }
+    scratch->counters.device_allocations = 1;
     ctx.scratch_ = scratch;
     return ctx;
+}
+
+HostCounters RocmContext::counters() const
+{
+    return scratch_->counters;
+}
+
+Result<Unit> RocmContext::wait_for_stream() const
+{
+    ++scratch_->counters.stream_waits;
+    const hipError_t err = hipStreamSynchronize(stream_);
+    if (err != hipSuccess) {
+        return hip_error("hipStreamSynchronize", err);
+    }
+    return Unit{};
+}
+
+Result<DeviceBuffer> RocmContext::pooled(size_t bytes) const
+{
+    Scratch& s = *scratch_;
+    size_t real = Scratch::size_class(std::max<size_t>(bytes, 1));
+    void* block = nullptr;
+    auto found = s.idle.lower_bound(real);
+    if (found != s.idle.end() && found->first <= real * 2) {
+        block = found->second;
+        real = found->first;
+        s.idle_bytes -= real;
+        s.idle.erase(found);
+    } else {
+        const hipError_t err = hipMalloc(&block, real);
+        if (err != hipSuccess) {
+            return hip_error("hipMalloc", err);
+        }
+        ++s.counters.device_allocations;
+    }
+    // the block returns to the pool of the context that made it; if that is gone, it is released
+    std::weak_ptr<Scratch> home = scratch_;
+    return DeviceBuffer::adopt(std::shared_ptr<void>(block,
+                                                     [home, real](void* p) {
+                                                         if (auto pool = home.lock()) {
+                                                             pool->give_back(p, real);
+                                                         } else {
+                                                             (void)hipFree(p);
+                                                         }
+                                                     }),
+                               bytes);
+}
+
+Result<DeviceBuffer> RocmContext::upload_words(const uint32_t* words, size_t count) const
+{
+    Scratch& s = *scratch_;
+    const size_t bytes = count * 4;
+    auto buffer = pooled(bytes);
+    if (buffer.is_err()) {
+        return buffer;
+    }
+    if (bytes > Scratch::kStageBytes) {
+        // larger than the ring: an ordinary copy, which waits for the stream's earlier work and for itself
+        const hipError_t err = hipMemcpy(buffer.unwrap().data(), words, bytes, hipMemcpyHostToDevice);
+        if (err != hipSuccess) {
+            return hip_error("upload", err);
+        }
+        return buffer;
+    }
+    const size_t aligned = (bytes + 63) / 64 * 64;
+    if (s.stage_next + aligned > Scratch::kStageBytes) {
+        // the ring wrapped: copies still in flight may read its start
+        auto waited = wait_for_stream();
+        if (waited.is_err()) {
+            return waited.unwrap_err();
+        }
+        s.stage_next = 0;
+    }
+    uint8_t* host = s.stage_host + s.stage_next;
+    memcpy(host, words, bytes);
+    const hipError_t err = hipMemcpyAsync(buffer.unwrap().data(), host, bytes, hipMemcpyHostToDevice, stream_);
+    if (err != hipSuccess) {
+        return hip_error("staged upload", err);
+    }
+    s.stage_next += aligned;
+    ++s.counters.staged_uploads;
+    return buffer;
+}
+
+Result<const uint32_t*> RocmContext::identity_table(size_t pages) const
+{
+    Scratch& s = *scratch_;
+    if (pages > s.identity_pages) {
+        const size_t grown = std::max<size_t>(std::max(pages, s.identity_pages * 2), 1024);
+        std::vector<uint32_t> ids(grown);
+        std::iota(ids.begin(), ids.end(), 0u);
+        auto table = pooled(grown * 4);
+        if (table.is_err()) {
+            return table.unwrap_err();
+        }
+        // an ordinary copy: it waits for the stream, so launches that still read the old table are done before it goes
+        const hipError_t err = hipMemcpy(table.unwrap().data(), ids.data(), grown * 4, hipMemcpyHostToDevice);
+        if (err != hipSuccess) {
+            return hip_error("identity table upload", err);
+        }
+        s.identity = table.unwrap();
+        s.identity_pages = grown;
+    }
+    return (const uint32_t*)s.identity.data();
+}
+
+Result<std::pair<const float*, const float*>> RocmContext::resident_rope_tables(const std::vector<float>& cos, const std::vector<float>& sin,
+                                                                                size_t required) const
+{
+    Scratch& s = *scratch_;
+    if (cos.size() != sin.size()) {
+        return compute_error("ROCm RoPE cos=" + std::to_string(cos.size()) + " sin=" + std::to_string(sin.size()) + " differ");
+    }
+    required = std::max<size_t>(required, 1);
+    if (required > cos.size()) {
+        return compute_error("ROCm RoPE needs " + std::to_string(required) + " elements, the tables hold " + std::to_string(cos.size()));
+    }
+    Scratch::RopeTables* entry = nullptr;
+    for (auto& held : s.rope) {
+        if (held.cos_host == cos.data() && held.sin_host == sin.data() && held.host_elements == cos.size()) {
+            entry = &held;
+            break;
+        }
+    }
+    if (entry != nullptr && entry->elements >= required && entry->first == cos[0] && entry->last == cos[entry->elements - 1]) {
+        return std::make_pair((const float*)entry->cos.data(), (const float*)entry->sin.data());
+    }
+    // commit a prefix: at least what is needed, at least twice what was there and 64 KiB, a power of two, never past the table
+    size_t elements = std::max(std::max<size_t>(required, 16384), entry != nullptr ? entry->elements * 2 : 0);
+    size_t pow2 = 1;
+    while (pow2 < elements) {
+        pow2 *= 2;
+    }
+    elements = std::max(std::min(pow2, cos.size()), required);
+    auto cos_dev = pooled(elements * 4);
+    auto sin_dev = pooled(elements * 4);
+    if (cos_dev.is_err() || sin_dev.is_err()) {
+        return cos_dev.is_err() ? cos_dev.unwrap_err() : sin_dev.unwrap_err();
+    }
+    hipError_t err = hipMemcpy(cos_dev.unwrap().data(), cos.data(), elements * 4, hipMemcpyHostToDevice);
+    if (err == hipSuccess) {
+        err = hipMemcpy(sin_dev.unwrap().data(), sin.data(), elements * 4, hipMemcpyHostToDevice);
+    }
+    if (err != hipSuccess) {
+        return hip_error("rotary table upload", err);
+    }
+    ++s.counters.rope_table_uploads;
+    if (entry == nullptr) {
+        if (s.rope.size() == 16) {
+            s.rope.erase(s.rope.begin()); // a model has a handful of tables; the oldest goes first
+        }
+        s.rope.emplace_back();
+        entry = &s.rope.back();
+    }
+    *entry = Scratch::RopeTables{cos.data(), sin.data(), cos.size(), elements, cos[0], cos[elements - 1], cos_dev.unwrap(), sin_dev.unwrap()};
+    return std::make_pair((const float*)entry->cos.data(), (const float*)entry->sin.data());
 }
 
 Result<void*> RocmContext::workspace(size_t bytes) const
@@ -427,14 +638,15 @@ Result<void*> RocmContext::workspace(size_t bytes) const
     Scratch& s = *scratch_;
     if (bytes > s.workspace.bytes()) {
         // kernels in flight may still use the old buffer: wait for them before it is released
-        const hipError_t err = hipStreamSynchronize(stream_);
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
+        auto waited = wait_for_stream();
+        if (waited.is_err()) {
+            return waited.unwrap_err();
         }
         auto grown = DeviceBuffer::allocate(std::max(bytes, s.workspace.bytes() * 2));
         if (grown.is_err()) {
             return grown.unwrap_err();
         }
+        ++s.counters.device_allocations;
         s.workspace = grown.unwrap();
     }
     return s.workspace.data();
@@ -445,9 +657,9 @@ Result<const uint32_t*> RocmContext::upload_meta(const uint32_t (&values)[4]) co
     Scratch& s = *scratch_;
     if (s.next == Scratch::kSlots) {
         // the ring wrapped: the oldest records may still be read by launches in flight
-        const hipError_t err = hipStreamSynchronize(stream_);
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
+        auto waited = wait_for_stream();
+        if (waited.is_err()) {
+            return waited.unwrap_err();
         }
         s.next = 0;
     }
@@ -604,7 +816,7 @@ Result<RocmTensor> RocmContext::gqa_attend(const RocmKvCache& cache, size_t laye
     const RocmKvCache::Layer& planes = cache.layers_[layer];
     const size_t query_cols = spec.num_heads * spec.head_dim;
     const size_t total = position + query.rows;
-    auto out_buf = DeviceBuffer::allocate(query.rows * query_cols * 4);
+    auto out_buf = pooled(query.rows * query_cols * 4);
     if (out_buf.is_err()) {
         return out_buf.unwrap_err();
     }
@@ -744,18 +956,16 @@ Result<RocmTensor> RocmContext::gqa_cached_impl(RocmKvCache& cache, size_t layer
         return compute_error("Rocm GQA L" + std::to_string(layer) + ": the layer was filled with another retention (ring of " +
                              std::to_string(planes.ring_capacity) + " rows)");
     }
+    // the ends travel through the pinned ring into a pooled block, which goes back to the pool when this call
+    // returns and is next written by work queued behind the launches that read it
     const uint32_t* ends_dev = nullptr;
     DeviceBuffer ends_buf;
     if (visible_ends != nullptr) {
-        auto buf = DeviceBuffer::allocate(visible_ends->size() * 4);
+        auto buf = upload_words(visible_ends->data(), visible_ends->size());
         if (buf.is_err()) {
             return buf.unwrap_err();
         }
         ends_buf = buf.unwrap();
-        const hipError_t err = hipMemcpy(ends_buf.data(), visible_ends->data(), visible_ends->size() * 4, hipMemcpyHostToDevice);
-        if (err != hipSuccess) {
-            return hip_error("visible ends upload", err);
-        }
         ends_dev = (const uint32_t*)ends_buf.data();
     }
     if (ring != 0 && query.rows > 1) {
@@ -783,9 +993,9 @@ Result<RocmTensor> RocmContext::gqa_cached_impl(RocmKvCache& cache, size_t layer
             if (kept.is_err()) {
                 return kept.unwrap_err();
             }
-            const hipError_t err = hipStreamSynchronize(stream_); // the chunk's own cache dies with this scope
-            if (err != hipSuccess) {
-                return hip_error("hipStreamSynchronize", err);
+            auto waited = wait_for_stream(); // the chunk's own cache dies with this scope
+            if (waited.is_err()) {
+                return waited.unwrap_err();
             }
             cache.lens_[layer] = total;
             return out;
@@ -798,12 +1008,6 @@ Result<RocmTensor> RocmContext::gqa_cached_impl(RocmKvCache& cache, size_t layer
     auto out = gqa_attend(cache, layer, position, query, spec, ends_dev);
     if (out.is_err()) {
         return out; // the cache length is left alone: the rows written past it are overwritten by the next append
-    }
-    if (ends_dev != nullptr) {
-        const hipError_t err = hipStreamSynchronize(stream_); // the uploaded ends die with this scope
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
-        }
     }
     cache.lens_[layer] = total;
     return out;
@@ -842,6 +1046,304 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_cached_from(const RocmKvCa
                              ", required_rows=" + std::to_string(required));
     }
     return gqa_attend(cache, source_layer, position, query, spec, nullptr);
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_cached_from_visible(const RocmKvCache& cache, size_t source_layer, size_t position,
+                                                                           const RocmTensor& query, const GqaSpec& spec,
+                                                                           const std::vector<uint32_t>& visible_ends) const
+{
+    if (spec.num_heads == 0 || spec.num_kv_heads == 0 || spec.head_dim == 0 || spec.num_heads % spec.num_kv_heads != 0) {
+        return compute_error("Rocm GQA spec invalid");
+    }
+    if (cache.mla_ || source_layer >= cache.layers_.size()) {
+        return unsupported_layer(source_layer);
+    }
+    if (visible_ends.size() != query.rows) {
+        return compute_error("GQA visible_ends=" + std::to_string(visible_ends.size()) + ", expected " + std::to_string(query.rows));
+    }
+    const size_t required = position + query.rows;
+    if (query.rows == 0 || query.cols != spec.num_heads * spec.head_dim || cache.cols_ != spec.num_kv_heads * spec.head_dim ||
+        cache.lens_[source_layer] < required) {
+        return compute_error("GQA shared cache L" + std::to_string(source_layer) + " incomplete: Q=[" + std::to_string(query.rows) + "," +
+                             std::to_string(query.cols) + "], cache rows=" + std::to_string(cache.lens_[source_layer]) +
+                             ", required_rows=" + std::to_string(required));
+    }
+    auto ends = upload_words(visible_ends.data(), visible_ends.size());
+    if (ends.is_err()) {
+        return ends.unwrap_err();
+    }
+    return gqa_attend(cache, source_layer, position, query, spec, (const uint32_t*)ends.unwrap().data());
+}
+
+// ---------------------------------------------------------------------------------------- dense K/V
+std::optional<std::string> GqaGeometry::validate() const
+{
+    if (num_heads == 0 || num_kv_heads == 0 || head_dim == 0 || num_heads % num_kv_heads != 0) {
+        return "GQA geometry invalid: query_heads=" + std::to_string(num_heads) + " kv_heads=" + std::to_string(num_kv_heads) +
+               " head_dim=" + std::to_string(head_dim);
+    }
+    return std::nullopt;
+}
+
+std::optional<std::string> BlockAttentionSpec::validate(size_t query_rows, size_t kv_rows) const
+{
+    if (auto bad = geometry.validate()) {
+        return bad;
+    }
+    if (!isfinite(score_scale) || score_scale <= 0.0f) {
+        return "block attention score_scale=" + std::to_string(score_scale) + " invalid";
+    }
+    if (visible.size() != query_rows) {
+        return "block attention visible=" + std::to_string(visible.size()) + ", expected query_rows=" + std::to_string(query_rows);
+    }
+    for (size_t r = 0; r < visible.size(); ++r) {
+        if (visible[r].first >= visible[r].second || visible[r].second > kv_rows) {
+            return "block attention query=" + std::to_string(r) + " visible range " + std::to_string(visible[r].first) + ".." +
+                   std::to_string(visible[r].second) + " outside KV rows=" + std::to_string(kv_rows);
+        }
+    }
+    return std::nullopt;
+}
+
+BlockAttentionSpec BlockAttentionSpec::full(GqaGeometry geometry, size_t query_rows, size_t kv_rows, float score_scale)
+{
+    BlockAttentionSpec spec;
+    spec.geometry = geometry;
+    spec.score_scale = score_scale;
+    spec.visible.assign(query_rows, std::make_pair((size_t)0, kv_rows));
+    return spec;
+}
+
+Result<BlockAttentionSpec> BlockAttentionSpec::varlen(GqaGeometry geometry, size_t query_rows, size_t kv_rows,
+                                                      const std::vector<size_t>& query_offsets, const std::vector<size_t>& kv_offsets,
+                                                      float score_scale)
+{
+    auto rising = [](const std::vector<size_t>& offsets) {
+        for (size_t i = 1; i < offsets.size(); ++i) {
+            if (offsets[i - 1] >= offsets[i]) {
+                return false;
+            }
+        }
+        return true;
+    };
+    if (query_offsets.size() < 2 || query_offsets.size() != kv_offsets.size() || query_offsets.front() != 0 || kv_offsets.front() != 0 ||
+        query_offsets.back() != query_rows || kv_offsets.back() != kv_rows || !rising(query_offsets) || !rising(kv_offsets)) {
+        return compute_error("varlen attention offsets invalid: Q=" + std::to_string(query_rows) + " KV=" + std::to_string(kv_rows));
+    }
+    BlockAttentionSpec spec;
+    spec.geometry = geometry;
+    spec.score_scale = score_scale;
+    spec.visible.reserve(query_rows);
+    for (size_t i = 1; i < query_offsets.size(); ++i) {
+        spec.visible.insert(spec.visible.end(), query_offsets[i] - query_offsets[i - 1], std::make_pair(kv_offsets[i - 1], kv_offsets[i]));
+    }
+    if (auto bad = spec.validate(query_rows, kv_rows)) {
+        return compute_error(*bad);
+    }
+    return spec;
+}
+
+struct RocmContext::DensePlanes {
+    DeviceBuffer key, value; // f16 [pages * kBlock, cols]
+    const uint32_t* table = nullptr;
+    size_t pages = 0, cols = 0;
+    static constexpr size_t kBlock = 64;
+};
+
+Result<RocmContext::DensePlanes> RocmContext::dense_f16_planes(const std::vector<const RocmTensor*>& keys, const std::vector<const RocmTensor*>& values,
+                                                               size_t cols, size_t cache_rows) const
+{
+    DensePlanes planes;
+    planes.cols = cols;
+    planes.pages = (cache_rows + DensePlanes::kBlock - 1) / DensePlanes::kBlock;
+    if (planes.pages == 0 || planes.pages * DensePlanes::kBlock > UINT32_MAX) {
+        return compute_error("ROCm dense attention: " + std::to_string(cache_rows) + " cache rows");
+    }
+    auto table = identity_table(planes.pages);
+    if (table.is_err()) {
+        return table.unwrap_err();
+    }
+    planes.table = table.unwrap();
+    auto key = pooled(planes.pages * DensePlanes::kBlock * cols * 2);
+    auto value = pooled(planes.pages * DensePlanes::kBlock * cols * 2);
+    if (key.is_err() || value.is_err()) {
+        return key.is_err() ? key.unwrap_err() : value.unwrap_err();
+    }
+    planes.key = key.unwrap();
+    planes.value = value.unwrap();
+    const std::vector<const RocmTensor*>* sources[2] = {&keys, &values};
+    void* targets[2] = {planes.key.data(), planes.value.data()};
+    for (int i = 0; i < 2; ++i) {
+        size_t at = 0;
+        for (const RocmTensor* part : *sources[i]) {
+            if (part->rows == 0) {
+                continue;
+            }
+            zllm_half_append_args a;
+            memset(&a, 0, sizeof(a));
+            a.src = part->device.data();
+            a.cache = targets[i];
+            a.table = planes.table;
+            a.position = (uint32_t)at;
+            a.rows = (uint32_t)part->rows;
+            a.cols = (uint32_t)cols;
+            a.block_tokens = (uint32_t)DensePlanes::kBlock;
+            a.src_dtype = abi_dtype(part->dtype);
+            a.dst_dtype = ZLLM_DTYPE_F16;
+            const int rc = zllm_attn_half_append(&a, stream_);
+            if (rc != 0) {
+                return abi_error("zllm_attn_half_append", rc);
+            }
+            at += part->rows;
+        }
+    }
+    return planes;
+}
+
+// `query.rows` rows at `position` over the planes' rows [0, position + query.rows): causal (with `window`, with visible ends)
+// when `starts_dev` is null, the exact ranges [starts, ends) otherwise.
+Result<RocmTensor> RocmContext::attend_dense(const RocmTensor& query, const DensePlanes& planes, size_t position, const GqaGeometry& geometry,
+                                             float score_scale, size_t window, const uint32_t* starts_dev, const uint32_t* ends_dev) const
+{
+    const size_t query_cols = geometry.num_heads * geometry.head_dim;
+    auto out_buf = pooled(query.rows * query_cols * 4);
+    if (out_buf.is_err()) {
+        return out_buf.unwrap_err();
+    }
+    zllm_gqa_prefill_args a;
+    memset(&a, 0, sizeof(a));
+    a.q = query.device.data();
+    a.k_plane = planes.key.data();
+    a.v_plane = planes.value.data();
+    a.table = planes.table;
+    a.table_stride = (uint32_t)planes.pages;
+    a.out = out_buf.unwrap().data();
+    a.rows = (uint32_t)query.rows;
+    a.position = (uint32_t)position;
+    a.window = (uint32_t)window;
+    a.num_heads = (uint32_t)geometry.num_heads;
+    a.num_kv_heads = (uint32_t)geometry.num_kv_heads;
+    a.head_dim = (uint32_t)geometry.head_dim;
+    a.block_tokens = (uint32_t)DensePlanes::kBlock;
+    a.score_scale = score_scale;
+    a.kv_format = ZLLM_KV_F16;
+    a.scale_dtype = ZLLM_SCALE_F16;
+    a.q_dtype = abi_dtype(query.dtype);
+    a.out_dtype = ZLLM_DTYPE_F32;
+    a.visible_starts = starts_dev;
+    a.visible_ends = ends_dev;
+    const uint64_t need = zllm_attn_gqa_prefill_workspace_bytes(&a);
+    if (need != 0) {
+        auto ws = workspace(need);
+        if (ws.is_err()) {
+            return ws.unwrap_err();
+        }
+        a.workspace = ws.unwrap();
+        a.workspace_bytes = need;
+    }
+    const int rc = zllm_attn_gqa_prefill_chunk(&a, stream_);
+    if (rc != 0) {
+        return abi_error("zllm_attn_gqa_prefill_chunk", rc);
+    }
+    RocmTensor out;
+    out.device = out_buf.unwrap();
+    out.rows = query.rows;
+    out.cols = query_cols;
+    out.dtype = DType::F32;
+    return out;
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec) const
+{
+    const GqaGeometry geometry{spec.num_heads, spec.num_kv_heads, spec.head_dim};
+    if (auto bad = geometry.validate()) {
+        return compute_error(*bad);
+    }
+    const size_t query_cols = spec.num_heads * spec.head_dim, kv_cols = spec.num_kv_heads * spec.head_dim;
+    if (query.rows == 0 || query.rows != key.rows || query.rows != value.rows || query.cols != query_cols || key.cols != kv_cols ||
+        value.cols != kv_cols) {
+        return compute_error("Rocm GQA prefill shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
+                             std::to_string(key.rows) + "," + std::to_string(key.cols) + "] V=[" + std::to_string(value.rows) + "," +
+                             std::to_string(value.cols) + "]");
+    }
+    auto planes = dense_f16_planes({&key}, {&value}, kv_cols, key.rows);
+    if (planes.is_err()) {
+        return planes.unwrap_err();
+    }
+    return attend_dense(query, planes.unwrap(), 0, geometry, spec.score_scale, spec.window.sliding ? spec.window.size : 0, nullptr, nullptr);
+}
+
+Result<RocmTensor> RocmContext::gqa_prefill_attention_visible(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value,
+                                                              const GqaSpec& spec, const std::vector<uint32_t>& visible_ends) const
+{
+    const GqaGeometry geometry{spec.num_heads, spec.num_kv_heads, spec.head_dim};
+    if (auto bad = geometry.validate()) {
+        return compute_error(*bad);
+    }
+    const size_t query_cols = spec.num_heads * spec.head_dim, kv_cols = spec.num_kv_heads * spec.head_dim;
+    if (query.rows == 0 || query.rows != key.rows || query.rows != value.rows || query.cols != query_cols || key.cols != kv_cols ||
+        value.cols != kv_cols || visible_ends.size() != query.rows) {
+        return compute_error("Rocm GQA visible prefill shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
+                             std::to_string(key.rows) + "," + std::to_string(key.cols) + "] V=[" + std::to_string(value.rows) + "," +
+                             std::to_string(value.cols) + "] visible=" + std::to_string(visible_ends.size()));
+    }
+    auto planes = dense_f16_planes({&key}, {&value}, kv_cols, key.rows);
+    if (planes.is_err()) {
+        return planes.unwrap_err();
+    }
+    auto ends = upload_words(visible_ends.data(), visible_ends.size());
+    if (ends.is_err()) {
+        return ends.unwrap_err();
+    }
+    return attend_dense(query, planes.unwrap(), 0, geometry, spec.score_scale, spec.window.sliding ? spec.window.size : 0, nullptr,
+                        (const uint32_t*)ends.unwrap().data());
+}
+
+Result<RocmTensor> RocmContext::block_attention_prefix_suffix(const RocmTensor& query, const RocmTensor& prefix_key, const RocmTensor& prefix_value,
+                                                              const RocmTensor& suffix_key, const RocmTensor& suffix_value,
+                                                              const BlockAttentionSpec& spec) const
+{
+    const size_t kv_rows = prefix_key.rows + suffix_key.rows;
+    if (auto bad = spec.validate(query.rows, kv_rows)) {
+        return compute_error(*bad);
+    }
+    const size_t query_cols = spec.geometry.num_heads * spec.geometry.head_dim, kv_cols = spec.geometry.num_kv_heads * spec.geometry.head_dim;
+    if (query.cols != query_cols || prefix_key.cols != kv_cols || prefix_value.rows != prefix_key.rows || prefix_value.cols != kv_cols ||
+        suffix_key.cols != kv_cols || suffix_value.rows != suffix_key.rows || suffix_value.cols != kv_cols) {
+        return compute_error("ROCm block attention shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
+                             std::to_string(prefix_key.rows) + "+" + std::to_string(suffix_key.rows) + "," + std::to_string(prefix_key.cols) +
+                             "] V=[" + std::to_string(prefix_value.rows) + "+" + std::to_string(suffix_value.rows) + "," +
+                             std::to_string(prefix_value.cols) + "]");
+    }
+    if (kv_rows > UINT32_MAX || query.rows > UINT32_MAX) {
+        return compute_error("ROCm block attention visible range beyond u32");
+    }
+    // the entry point reads no cache row at or past position + rows: put the query rows at the end of whichever is longer
+    const size_t cache_rows = std::max(kv_rows, query.rows);
+    auto planes = dense_f16_planes({&prefix_key, &suffix_key}, {&prefix_value, &suffix_value}, kv_cols, cache_rows);
+    if (planes.is_err()) {
+        return planes.unwrap_err();
+    }
+    std::vector<uint32_t> ranges(2 * query.rows);
+    for (size_t r = 0; r < query.rows; ++r) {
+        ranges[r] = (uint32_t)spec.visible[r].first;
+        ranges[query.rows + r] = (uint32_t)spec.visible[r].second;
+    }
+    auto ranges_dev = upload_words(ranges.data(), ranges.size());
+    if (ranges_dev.is_err()) {
+        return ranges_dev.unwrap_err();
+    }
+    const uint32_t* starts = (const uint32_t*)ranges_dev.unwrap().data();
+    return attend_dense(query, planes.unwrap(), cache_rows - query.rows, spec.geometry, spec.score_scale, 0, starts, starts + query.rows);
+}
+
+Result<RocmTensor> RocmContext::block_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value,
+                                                const BlockAttentionSpec& spec) const
+{
+    RocmTensor none;
+    none.cols = key.cols;
+    none.dtype = key.dtype;
+    return block_attention_prefix_suffix(query, key, value, none, none, spec);
 }
 
 Result<Unit> RocmContext::append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,
@@ -903,27 +1405,11 @@ Result<Unit> RocmContext::append_mla_rope(RocmKvCache& cache, size_t layer, cons
         cos.size() < (position + rope.rows) * half) {
         return compute_error("Rocm MLA append: rotary tables do not cover position " + std::to_string(position));
     }
-    auto tables = DeviceBuffer::allocate(cos.size() * 8);
+    auto tables = resident_rope_tables(cos, sin, (position + rope.rows) * half);
     if (tables.is_err()) {
         return tables.unwrap_err();
     }
-    float* cos_dev = (float*)tables.unwrap().data();
-    float* sin_dev = cos_dev + cos.size();
-    hipError_t err = hipMemcpy(cos_dev, cos.data(), cos.size() * 4, hipMemcpyHostToDevice);
-    if (err == hipSuccess) {
-        err = hipMemcpy(sin_dev, sin.data(), sin.size() * 4, hipMemcpyHostToDevice);
-    }
-    if (err != hipSuccess) {
-        return hip_error("rotary table upload", err);
-    }
-    auto done = append_mla_impl(cache, layer, latent, rope, rotary_dim, layout, position, cos_dev, sin_dev);
-    if (done.is_ok()) {
-        err = hipStreamSynchronize(stream_); // the tables die with this scope
-        if (err != hipSuccess) {
-            return hip_error("hipStreamSynchronize", err);
-        }
-    }
-    return done;
+    return append_mla_impl(cache, layer, latent, rope, rotary_dim, layout, position, tables.unwrap().first, tables.unwrap().second);
 }
 
 Result<RocmTensor> RocmContext::mla_decode_attention(const RocmTensor& query, const RocmKvCache& cache, const RocmWeight& kv_b, size_t layer,
@@ -948,13 +1434,9 @@ Result<RocmDsaState> RocmContext::dsa_state_from_selection(const std::vector<uin
     if (selection.empty()) {
         return compute_error("Rocm DSA state: empty selection");
     }
-    auto buffer = DeviceBuffer::allocate(selection.size() * 4);
+    auto buffer = upload_words(selection.data(), selection.size());
     if (buffer.is_err()) {
         return buffer.unwrap_err();
-    }
-    const hipError_t err = hipMemcpy(buffer.unwrap().data(), selection.data(), selection.size() * 4, hipMemcpyHostToDevice);
-    if (err != hipSuccess) {
-        return hip_error("selection upload", err);
     }
     RocmDsaState state;
     state.selection = buffer.unwrap();
@@ -985,7 +1467,7 @@ Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const R
     const bool chunk = query.rows > 1;
     const size_t out_cols = spec.num_heads * spec.value_dim();
     // a decode row is written as f32, the rows of a chunk as bf16 (src/backend/rocm/attention.rs:17-19)
-    auto out_buf = DeviceBuffer::allocate(query.rows * out_cols * (chunk ? 2 : 4));
+    auto out_buf = pooled(query.rows * out_cols * (chunk ? 2 : 4));
     if (out_buf.is_err()) {
         return out_buf.unwrap_err();
     }

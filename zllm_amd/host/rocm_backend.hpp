@@ -71,6 +71,24 @@ struct GqaSpec {
     size_t group_size() const { return num_heads / num_kv_heads; }
 };
 
+// Head geometry and explicit per-row visible ranges of the model-independent block attention
+// (GqaGeometry, src/attention/gqa.rs:11-37; BlockAttentionSpec, src/attention/block.rs:10-63).
+struct GqaGeometry {
+    size_t num_heads = 0, num_kv_heads = 0, head_dim = 0;
+    std::optional<std::string> validate() const;
+};
+
+struct BlockAttentionSpec {
+    GqaGeometry geometry;
+    float score_scale = 0.0f;
+    std::vector<std::pair<size_t, size_t>> visible; // [start, end) of the KV rows each query row sees
+    std::optional<std::string> validate(size_t query_rows, size_t kv_rows) const;
+    static BlockAttentionSpec full(GqaGeometry geometry, size_t query_rows, size_t kv_rows, float score_scale);
+    // two prefix sums cut the rows into isolated sequences: the rows of query segment i see the KV rows of segment i
+    static Result<BlockAttentionSpec> varlen(GqaGeometry geometry, size_t query_rows, size_t kv_rows, const std::vector<size_t>& query_offsets,
+                                             const std::vector<size_t>& kv_offsets, float score_scale);
+};
+
 enum class RotaryLayout { SplitHalf, Interleaved };
 
 struct MlaSpec {
@@ -93,10 +111,12 @@ struct DsaSpec {
 enum class DType { F32 = 0, BF16 = 1, F16 = 2 };
 size_t dtype_bytes(DType dtype);
 
-// Device buffer with shared ownership (hipMalloc / hipFree).
+// Device buffer with shared ownership.  allocate() is hipMalloc / hipFree; a buffer a RocmContext hands out (outputs,
+// staged uploads, scratch planes) comes from that context's pool and goes back to it when the last owner lets go.
 class DeviceBuffer {
   public:
     static Result<DeviceBuffer> allocate(size_t bytes);
+    static DeviceBuffer adopt(std::shared_ptr<void> block, size_t bytes);
     void* data() const { return ptr_.get(); }
     size_t bytes() const { return bytes_; }
 
@@ -203,9 +223,18 @@ class RocmKvCache {
     DeviceBuffer table_;
 };
 
+// What a context did on the host side so far; a serving loop in steady state moves none of the first three.
+struct HostCounters {
+    size_t device_allocations = 0;  // hipMalloc calls made for pooled buffers, the workspace and resident tables
+    size_t rope_table_uploads = 0;  // uploads of a cos/sin prefix
+    size_t stream_waits = 0;        // hipStreamSynchronize calls made inside attention and append methods
+    size_t staged_uploads = 0;      // small host arrays (visible ends, selections) sent through the pinned ring
+};
+
 class RocmContext {
   public:
     static Result<RocmContext> create(int device_id);
+    HostCounters counters() const;
     int device_id() const { return device_id_; }
     hipStream_t stream() const { return stream_; }
     Result<Unit> synchronize() const;
@@ -215,6 +244,20 @@ class RocmContext {
     // DecodeBackend::prepare_mla_kv_b: kv_b [heads * kv_head_dim, latent] -> bf16 on the device
     Result<RocmWeight> prepare_mla_kv_b(const std::vector<float>& weight, size_t rows, size_t cols) const;
 
+    // Backend::gqa_prefill_attention (src/backend/mod.rs:1477; ROCm body src/backend/rocm/attention.rs:2151-2170): causal
+    // attention of a chunk over its own K/V, nothing cached.  K and V go to dense f16 scratch planes on the way in.
+    Result<RocmTensor> gqa_prefill_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec) const;
+    // The same with a visible end per row (right-padded text encoders; src/backend/mod.rs:1479-1482).
+    Result<RocmTensor> gqa_prefill_attention_visible(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value, const GqaSpec& spec,
+                                                     const std::vector<uint32_t>& visible_ends) const;
+    // BlockAttentionBackend::block_attention (src/backend/mod.rs:1582-1584; ROCm body src/backend/rocm/attention.rs:118-144):
+    // query and KV lengths differ, every query row sees exactly its range.  Returns f32 [query.rows, num_heads * head_dim].
+    Result<RocmTensor> block_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value, const BlockAttentionSpec& spec) const;
+    // block_attention_prefix_suffix (src/backend/mod.rs:1601-1616): the KV rows are a resident prefix followed by this
+    // step's short suffix; the two are written one behind the other into the scratch planes, never concatenated on the host.
+    Result<RocmTensor> block_attention_prefix_suffix(const RocmTensor& query, const RocmTensor& prefix_key, const RocmTensor& prefix_value,
+                                                     const RocmTensor& suffix_key, const RocmTensor& suffix_value,
+                                                     const BlockAttentionSpec& spec) const;
     // Appends the chunk's K/V rows at `position` (must equal the layer's cached length), then attends:
     // one row -> split-KV decode, more rows -> chunked prefill (causal, optional sliding window).
     // Returns f32 [rows, num_heads * head_dim].  A sliding-window layer appended with retain_full_cache == false keeps
@@ -232,6 +275,10 @@ class RocmContext {
     // layer must already hold position + rows rows.
     Result<RocmTensor> gqa_prefill_attention_cached_from(const RocmKvCache& cache, size_t source_layer, size_t position, const RocmTensor& query,
                                                          const GqaSpec& spec) const;
+    // The shared-KV form with visible ends (visual blocks on a shared layer; src/backend/mod.rs:1575-1578).
+    Result<RocmTensor> gqa_prefill_attention_cached_from_visible(const RocmKvCache& cache, size_t source_layer, size_t position,
+                                                                 const RocmTensor& query, const GqaSpec& spec,
+                                                                 const std::vector<uint32_t>& visible_ends) const;
     // MlaPrefillBackend: append the chunk, then attend with one query row per chunk row (causal inside the chunk).
     // Returns bf16 [rows, heads * value_dim] for more than one row, f32 for one (src/backend/rocm/attention.rs:17-19).
     Result<RocmTensor> mla_prefill_attention(const RocmTensor& query, const RocmTensor& latent, const RocmTensor& k_rope, const RocmWeight& kv_b,
@@ -257,11 +304,29 @@ class RocmContext {
 
   private:
     // Device scratch of the context's stream, kept between calls: the split-KV workspace (grown when a call needs
-    // more) and a ring of small metadata records (lengths, window starts) that travel host -> device from pinned memory,
-    // so that a call neither allocates nor waits for the stream.
+    // more), a ring of small metadata records (lengths, window starts) and a ring for small arrays (visible ends,
+    // selections) that travel host -> device from pinned memory, a pool that output tensors and scratch planes are
+    // taken from and returned to, an identity block table and the cos/sin tables already on the device -- so that a
+    // call in steady state neither allocates nor waits for the stream.  Blocks are reused in stream order: everything
+    // the context launches runs on its one stream, so a block that went back to the pool is next written by work
+    // queued behind its last reader.
     struct Scratch;
     Result<void*> workspace(size_t bytes) const;
     Result<const uint32_t*> upload_meta(const uint32_t (&values)[4]) const;
+    Result<DeviceBuffer> pooled(size_t bytes) const;
+    Result<DeviceBuffer> upload_words(const uint32_t* words, size_t count) const;
+    Result<const uint32_t*> identity_table(size_t pages) const;
+    // cos/sin of a model live on the device once per host table (keyed like the reference's table cache,
+    // src/backend/rocm/compressed_sparse.rs:20-36,323-348): the committed prefix doubles as positions arrive
+    Result<std::pair<const float*, const float*>> resident_rope_tables(const std::vector<float>& cos, const std::vector<float>& sin,
+                                                                       size_t required) const;
+    Result<Unit> wait_for_stream() const;
+    // dense rows -> f16 scratch planes [pages * 64, cols] behind the identity table; `parts` are written one behind the other
+    struct DensePlanes;
+    Result<DensePlanes> dense_f16_planes(const std::vector<const RocmTensor*>& keys, const std::vector<const RocmTensor*>& values, size_t cols,
+                                         size_t cache_rows) const;
+    Result<RocmTensor> attend_dense(const RocmTensor& query, const DensePlanes& planes, size_t position, const GqaGeometry& geometry,
+                                    float score_scale, size_t window, const uint32_t* starts_dev, const uint32_t* ends_dev) const;
     Result<Unit> append_gqa_rows(RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& key, const RocmTensor& value) const;
     Result<RocmTensor> gqa_attend(const RocmKvCache& cache, size_t layer, size_t position, const RocmTensor& query, const GqaSpec& spec,
                                   const uint32_t* visible_ends_dev) const;
