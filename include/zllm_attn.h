@@ -256,10 +256,14 @@ typedef struct zllm_gqa_decode_args {
     uint32_t max_kv_len;           /* host upper bound of kv_lens: sizes the grid and the split plan.  A call
                                       recorded into a HIP graph stays valid only while every kv_lens[b] on the
                                       device is <= max_kv_len; tokens past the planned splits are not read */
-    uint32_t total_kv_tokens;      /* host hint: sum of the visible lengths (0 = unknown, batch * max_kv_len is
-                                      assumed); only tunes the split size.  Pass it for batches of unequal lengths
-                                      and for sliding windows: planned as if every sequence were max_kv_len long,
-                                      a long sequence among short ones (or a short window) gets few workgroups */
+    uint32_t total_kv_tokens;      /* host bound: sum of the visible lengths (0 = unknown, batch * max_kv_len is
+                                      assumed).  Pass it for batches of unequal lengths and for sliding windows:
+                                      planned as if every sequence were max_kv_len long, a long sequence among short
+                                      ones (or a short window) gets few workgroups.  With it the splits are sized for
+                                      the tokens there are and the split records for the splits there are (see
+                                      zllm_attn_gqa_decode_record_layout), so it must not be below the real sum --
+                                      like max_kv_len it has to hold for every replay of a recorded call.  Splits
+                                      beyond the records it sized are dropped (wrong output, nothing out of bounds) */
     uint32_t block_tokens;
     uint32_t ring_capacity;        /* 0 or sliding-window ring rows (token % capacity) */
     float score_scale;             /* > 0 */
@@ -285,11 +289,26 @@ ZLLM_API uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_arg
  * most *chunk_tokens tokens (a multiple of 32), so max_chunks * chunk_tokens >= max_kv_len.  It is fixed by the host
  * arguments alone (the tile / split geometry of try_gqa_decode_cached_f32,
  * src/kernel/rocm/hip/tensor/attention.rs:1031-1046): a sequence whose kv_lens[b] on the device has grown past
- * max_kv_len -- a recorded graph replayed too long -- is read up to max_chunks * chunk_tokens tokens only.  A caller
- * that combines ZLLM_STAGE_PARTIAL records itself indexes them with max_chunks:
- * partial f32 [batch][max_chunks][num_heads][head_dim] at the start of the workspace, then (max, sum) f32 pairs
- * [batch][max_chunks][num_heads][2] at the next 256-byte boundary.  0 ok, negative = invalid arguments. */
+ * max_kv_len -- a recorded graph replayed too long -- is read up to max_chunks * chunk_tokens tokens only.
+ * 0 ok, negative = invalid arguments. */
 ZLLM_API int zllm_attn_gqa_decode_split_plan(const zllm_gqa_decode_args* args, uint32_t* chunk_tokens, uint32_t* max_chunks);
+/* Where a call's split records lie in its workspace, for a caller that combines ZLLM_STAGE_PARTIAL records itself
+ * (the reference sizes its records per launch the same way, src/kernel/rocm/hip/attention/paged_mla.rs:2987-2994,
+ * 3248-3257): partial f32 [record_rows][heads][width] at partial_offset (width = head_dim for GQA, latent_dim for MLA),
+ * (max, sum) f32 pairs [record_rows][heads][2] at stats_offset.  Split c of record group g (a sequence; for MLA calls
+ * with query_rows > 1, a query row) is row g * max_chunks + c when dense == 0 -- a plan for equal lengths -- and row
+ * first_rows[g] + c when dense == 1: a ragged plan numbers its records over the live splits only, in group order, so the
+ * workspace grows with the tokens there are and not with batch x longest sequence; first_rows is u32 [groups] at
+ * first_rows_offset, written by the partial stage (entries of groups without splits are not written). */
+typedef struct zllm_split_record_layout {
+    uint64_t record_rows;
+    uint64_t partial_offset;
+    uint64_t stats_offset;
+    uint64_t first_rows_offset; /* 0 when dense == 0 */
+    uint32_t chunk_tokens, max_chunks;
+    uint32_t dense;
+} zllm_split_record_layout;
+ZLLM_API int zllm_attn_gqa_decode_record_layout(const zllm_gqa_decode_args* args, zllm_split_record_layout* layout);
 ZLLM_API int zllm_attn_gqa_decode(const zllm_gqa_decode_args* args, zllm_stream_t stream);
 
 /* zllm_attn_gqa_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
@@ -476,12 +495,16 @@ typedef struct zllm_mla_decode_args {
      * a selection holds one list per query row.  The reference returns bf16 for T > 1
      * (src/backend/rocm/attention.rs:17-19): pass out_dtype = ZLLM_DTYPE_BF16 for that.  batch * T <= 65535. */
     uint32_t query_rows;
-    /* Host hint for batches of unequal lengths: the sum of ctx_lens over the sequences (0 = unknown, every sequence is
-     * planned as max_ctx_len long, and a long sequence among short ones gets few workgroups).  Only tunes the split
-     * size; the split records grow with max_ctx_len / split size, which zllm_attn_mla_decode_workspace_bytes reports. */
+    /* Host bound for batches of unequal lengths: the sum of ctx_lens over the sequences (0 = unknown, every sequence is
+     * planned as max_ctx_len long, and a long sequence among short ones gets few workgroups).  With it the splits are
+     * sized for the tokens there are and the split records for the splits there are (zllm_attn_mla_decode_record_layout),
+     * so it must not be below the real sum -- like max_ctx_len it has to hold for every replay of a recorded call;
+     * splits beyond the records it sized are dropped (wrong output, nothing out of bounds). */
     uint32_t total_ctx_tokens;
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
+/* The record layout of a call, as zllm_attn_gqa_decode_record_layout gives it for GQA; record groups are query rows. */
+ZLLM_API int zllm_attn_mla_decode_record_layout(const zllm_mla_decode_args* args, zllm_split_record_layout* layout);
 ZLLM_API int zllm_attn_mla_decode(const zllm_mla_decode_args* args, zllm_stream_t stream);
 
 #ifdef __cplusplus

@@ -162,13 +162,48 @@ def test_split_plan_covers_the_host_bound_and_sizes_the_workspace(lib):
         assert chunk.value % 32 == 0 and chunk.value >= 64 and chunks.value >= 1
         assert chunk.value * chunks.value >= args.max_kv_len
         assert chunk.value * (chunks.value - 1) < args.max_kv_len  # no split lies wholly beyond the bound
-        records = args.batch * chunks.value * args.num_heads
-        if args.total_kv_tokens:  # a ragged plan never asks for more than 512 MiB of records (plus one split's rounding)
-            assert records * args.head_dim * 4 <= (512 << 20) + args.batch * args.num_heads * args.head_dim * 4
+        # the record layout: [sequence][max_chunks] rows for a plan of equal lengths; a ragged plan numbers its records over
+        # the live splits, so their bytes follow the tokens there are and not batch x longest sequence
+        layout = capi.SplitRecordLayout()
+        assert lib.zllm_attn_gqa_decode_record_layout(C.byref(args), C.byref(layout)) == 0
+        assert (layout.chunk_tokens, layout.max_chunks) == (chunk.value, chunks.value)
         align = lambda n: (n + 255) // 256 * 256
-        assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) == align(records * args.head_dim * 4) + align(records * 8)
+        if layout.dense:
+            assert args.total_kv_tokens and layout.record_rows < args.batch * chunks.value
+            assert layout.record_rows == args.total_kv_tokens // chunk.value + 2 * args.batch
+            # every sequence's splits fit: sum of ceil((len + 31) / chunk) over any lengths that add up to the total
+            assert layout.record_rows >= -(-args.total_kv_tokens // chunk.value) + args.batch
+        else:
+            assert layout.record_rows == args.batch * chunks.value and layout.first_rows_offset == 0
+        records = layout.record_rows * args.num_heads
+        assert layout.partial_offset == 0 and layout.stats_offset == align(records * args.head_dim * 4)
+        size = layout.stats_offset + align(records * 8)
+        if layout.dense:
+            assert layout.first_rows_offset == size
+            size += align(args.batch * 4)
+        assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(args)) == size
     bad = capi.GqaDecodeArgs()
     assert lib.zllm_attn_gqa_decode_split_plan(C.byref(bad), None, None) == -1
+    assert lib.zllm_attn_gqa_decode_record_layout(C.byref(bad), C.byref(capi.SplitRecordLayout())) == -1
+
+
+def test_ragged_mla_records_follow_the_tokens_not_the_longest_sequence(lib):
+    """One 1M-token context among 31 of 2,000 tokens: records numbered over the live splits stay a few MiB where
+    [row][max_chunks] rows would take most of a gigabyte; a plan of equal lengths keeps the rows that need no lookup."""
+    args = capi.MlaDecodeArgs()
+    args.batch, args.heads, args.q_head_dim, args.kv_head_dim = 32, 64, 192, 256
+    args.latent_dim, args.rope_dim, args.block_tokens = 512, 64, 64
+    args.max_ctx_len, args.total_ctx_tokens = 1 << 20, (1 << 20) + 31 * 2000
+    args.q_dtype, args.out_dtype = capi.DTYPE_BF16, capi.DTYPE_F32
+    layout = capi.SplitRecordLayout()
+    assert lib.zllm_attn_mla_decode_record_layout(C.byref(args), C.byref(layout)) == 0
+    assert layout.dense == 1 and layout.record_rows == args.total_ctx_tokens // layout.chunk_tokens + args.batch
+    assert layout.record_rows < 400 and layout.max_chunks * layout.chunk_tokens >= args.max_ctx_len
+    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args)) < 64 << 20
+    assert args.batch * layout.max_chunks * args.heads * 512 * 4 > 512 << 20  # what the rows by sequence would have taken
+    args.total_ctx_tokens = 0
+    assert lib.zllm_attn_mla_decode_record_layout(C.byref(args), C.byref(layout)) == 0
+    assert layout.dense == 0 and layout.first_rows_offset == 0 and layout.record_rows == args.batch * layout.max_chunks
 
 
 def test_split_plan_fills_whole_rounds_of_the_compute_units(lib):

@@ -437,9 +437,11 @@ def test_mla_ragged_batch_with_the_token_count_hint():
     args.batch, args.heads, args.q_head_dim, args.kv_head_dim, args.latent_dim, args.rope_dim = len(lens), 32, 192, 256, 512, 64
     args.block_tokens, args.max_ctx_len, args.q_dtype, args.out_dtype, args.out_compact = 16, max(lens), capi.DTYPE_BF16, capi.DTYPE_F32, 1
     lib = capi.load()
-    unhinted_bytes = lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args))
+    plain_plan, hinted_plan = capi.SplitRecordLayout(), capi.SplitRecordLayout()
+    assert lib.zllm_attn_mla_decode_record_layout(C.byref(args), C.byref(plain_plan)) == 0
     args.total_ctx_tokens = sum(lens)
-    assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(args)) > unhinted_bytes  # more, shorter splits
+    assert lib.zllm_attn_mla_decode_record_layout(C.byref(args), C.byref(hinted_plan)) == 0
+    assert hinted_plan.chunk_tokens < plain_plan.chunk_tokens and hinted_plan.dense == 1  # more, shorter splits; records over the live ones
 
 
 @pytest.mark.parametrize("heads,lens", [(16, [20000]), (32, [9000, 70]), (64, [17000]), (32, [8300, 8200])])

@@ -85,6 +85,11 @@ class GqaPrefillArgs(C.Structure):
                 ("gate_dtype", _int), ("visible_ends", _ptr), ("table_stride", _u32), ("visible_starts", _ptr)]
 
 
+class SplitRecordLayout(C.Structure):
+    _fields_ = [("record_rows", _u64), ("partial_offset", _u64), ("stats_offset", _u64), ("first_rows_offset", _u64),
+                ("chunk_tokens", _u32), ("max_chunks", _u32), ("dense", _u32)]
+
+
 class MlaDecodeArgs(C.Structure):
     _fields_ = [("q", _ptr), ("kv_b", _ptr), ("latent_codes", _ptr), ("latent_scales", _ptr), ("rope_cache", _ptr),
                 ("tables", _ptr), ("ctx_lens", _ptr), ("out", _ptr), ("workspace", _ptr), ("workspace_bytes", _u64),
@@ -114,12 +119,14 @@ SYMBOLS = {
     "zllm_kv_mla_layer_read": (_int, [_ptr, _u64, C.POINTER(MlaLayerRecord), C.POINTER(_u64)]),
     "zllm_attn_gqa_decode_workspace_bytes": (_u64, [C.POINTER(GqaDecodeArgs)]),
     "zllm_attn_gqa_decode_split_plan": (_int, [C.POINTER(GqaDecodeArgs), C.POINTER(_u32), C.POINTER(_u32)]),
+    "zllm_attn_gqa_decode_record_layout": (_int, [C.POINTER(GqaDecodeArgs), C.POINTER(SplitRecordLayout)]),
     "zllm_attn_gqa_decode": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
     "zllm_attn_static_scratch_bytes": (_u64, []),
     "zllm_attn_gqa_decode_static": (_int, [C.POINTER(GqaDecodeArgs), _ptr]),
     "zllm_attn_gqa_prefill_workspace_bytes": (_u64, [C.POINTER(GqaPrefillArgs)]),
     "zllm_attn_gqa_prefill_chunk": (_int, [C.POINTER(GqaPrefillArgs), _ptr]),
     "zllm_attn_mla_decode_workspace_bytes": (_u64, [C.POINTER(MlaDecodeArgs)]),
+    "zllm_attn_mla_decode_record_layout": (_int, [C.POINTER(MlaDecodeArgs), C.POINTER(SplitRecordLayout)]),
     "zllm_attn_mla_decode": (_int, [C.POINTER(MlaDecodeArgs), _ptr]),
 }
 

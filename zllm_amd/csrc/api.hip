@@ -34,7 +34,29 @@ int hip_status(hipError_t err, const char* what)
     return (int)err;
 }
 
-constexpr unsigned int kComputeUnits = 256; // MI355X
+// Compute units of the current device, asked once per device; 256 (MI355X) where there is no device to ask, so that the
+// host-only planning calls still answer.
+unsigned int compute_units()
+{
+    constexpr int kKnown = 64;
+    static std::atomic<unsigned int> known[kKnown];
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kKnown) {
+        (void)hipGetLastError();
+        return 256u;
+    }
+    unsigned int units = known[device].load(std::memory_order_relaxed);
+    if (units == 0u) {
+        int count = 0;
+        if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) {
+            (void)hipGetLastError();
+            return 256u;
+        }
+        units = (unsigned int)count;
+        known[device].store(units, std::memory_order_relaxed);
+    }
+    return units;
+}
 
 } // namespace
 
@@ -113,10 +135,11 @@ void plan_splits(uint32_t max_len, uint64_t units, uint32_t units_per_group, uin
 {
     // `units_per_group` of a pair's splits share one workgroup (GQA decode with few KV heads)
     constexpr uint64_t kFixedTokens = 64;
+    const uint64_t cus = compute_units();
     uint64_t best_chunk = align_up(max_len < min_chunk ? min_chunk : max_len, 32); // one split per pair
     uint64_t best_cost = ~(uint64_t)0;
     for (uint64_t rounds = 1; rounds <= 8; ++rounds) {
-        const uint64_t per_unit = rounds * kComputeUnits * units_per_group / units;
+        const uint64_t per_unit = rounds * cus * units_per_group / units;
         if (per_unit == 0) {
             continue;
         }
@@ -124,7 +147,7 @@ void plan_splits(uint32_t max_len, uint64_t units, uint32_t units_per_group, uin
         chunk = align_up(chunk < min_chunk ? min_chunk : chunk, 32);
         const uint64_t splits = ((uint64_t)max_len + chunk - 1) / chunk;
         const uint64_t groups = (splits * units + units_per_group - 1) / units_per_group;
-        const uint64_t launched = (groups + kComputeUnits - 1) / kComputeUnits;
+        const uint64_t launched = (groups + cus - 1) / cus;
         const uint64_t cost = launched * (chunk + kFixedTokens);
         if (cost < best_cost) {
             best_cost = cost;
@@ -201,8 +224,20 @@ void cap_split_for_page_registers(const zllm_gqa_decode_args* a, uint32_t* chunk
     *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
 }
 
-void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+// Rows of the split record arrays.  A plan made for equal lengths keeps [sequence][max_chunks] rows, which a workgroup
+// and the merge address without reading anything.  A ragged plan (total_kv_tokens given and below batch x max_kv_len) numbers
+// its records like its work items, densely over the live splits: sequence b has ceil((len_b - first_b rounded down to 32) /
+// chunk_tokens) of them, so total / chunk_tokens + 2 x batch rows hold them all, however long the longest sequence is.
+struct GqaSplitPlan {
+    uint32_t chunk_tokens, max_chunks;
+    uint64_t record_rows;
+    bool dense;
+};
+
+GqaSplitPlan plan_gqa_decode(const zllm_gqa_decode_args* a)
 {
+    GqaSplitPlan plan;
+    const uint64_t cus = compute_units();
     const uint32_t max_waves = zllm::gqa_decode_max_waves(a->head_dim);
     const uint32_t waves = a->num_kv_heads < max_waves ? a->num_kv_heads : max_waves;
     const uint32_t kvh_blocks = (a->num_kv_heads + waves - 1) / waves;
@@ -210,26 +245,44 @@ void plan_gqa_decode(const zllm_gqa_decode_args* a, uint32_t* chunk_tokens, uint
     const uint32_t items_per_group = zllm::gqa_decode_items_per_group(a->head_dim, a->num_kv_heads);
     const uint64_t columns = (uint64_t)a->batch * kvh_blocks * head_blocks;
     const uint64_t uniform_total = (uint64_t)a->batch * a->max_kv_len;
-    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && (uint64_t)kComputeUnits * items_per_group > 2 * columns) {
+    plan.dense = false;
+    if (a->total_kv_tokens != 0 && a->total_kv_tokens < uniform_total && cus * items_per_group > 2 * columns) {
         // ragged batch: sum_b ceil(len_b / chunk) <= total / chunk + batch, so size the splits for the
         // workgroups that will really run and keep them within one round of the CUs
-        const uint64_t slots = (uint64_t)kComputeUnits * items_per_group / (kvh_blocks * head_blocks) - a->batch;
+        const uint64_t slots = cus * items_per_group / (kvh_blocks * head_blocks) - a->batch;
         uint64_t chunk = (a->total_kv_tokens + slots - 1) / slots;
         chunk = align_up(chunk < kMinGqaChunk ? kMinGqaChunk : chunk, 32);
-        // the records are [sequence][max_chunks][head][head_dim] floats: a plan whose records would pass 512 MiB (one very
-        // long sequence among many short ones) keeps longer splits
-        const uint64_t record_bytes = (uint64_t)a->batch * a->num_heads * a->head_dim * 4;
-        const uint64_t most = ((uint64_t)512 << 20) / record_bytes;
-        const uint64_t fewest_tokens = align_up(((uint64_t)a->max_kv_len + (most < 1 ? 1 : most) - 1) / (most < 1 ? 1 : most), 32);
-        if (chunk < fewest_tokens) {
-            chunk = fewest_tokens;
-        }
-        *chunk_tokens = (uint32_t)chunk;
-        *max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
+        plan.chunk_tokens = (uint32_t)chunk;
+        plan.max_chunks = (uint32_t)((a->max_kv_len + chunk - 1) / chunk);
+        plan.dense = true;
     } else {
-        plan_splits(a->max_kv_len, columns, items_per_group, kMinGqaChunk, chunk_tokens, max_chunks);
+        plan_splits(a->max_kv_len, columns, items_per_group, kMinGqaChunk, &plan.chunk_tokens, &plan.max_chunks);
     }
-    cap_split_for_page_registers(a, chunk_tokens, max_chunks);
+    cap_split_for_page_registers(a, &plan.chunk_tokens, &plan.max_chunks);
+    plan.record_rows = (uint64_t)a->batch * plan.max_chunks;
+    if (plan.dense) {
+        const uint64_t live = a->total_kv_tokens / plan.chunk_tokens + 2ull * a->batch;
+        if (live < plan.record_rows) {
+            plan.record_rows = live;
+        } else {
+            plan.dense = false; // nothing to save: keep the rows that need no lookup
+        }
+    }
+    return plan;
+}
+
+struct GqaWorkspace {
+    uint64_t stats, first_rows, total;
+};
+
+GqaWorkspace gqa_workspace(const zllm_gqa_decode_args* a, const GqaSplitPlan& plan)
+{
+    GqaWorkspace w;
+    const uint64_t rows = plan.record_rows * a->num_heads;
+    w.stats = align_up(rows * a->head_dim * 4, 256);
+    w.first_rows = w.stats + align_up(rows * 8, 256);
+    w.total = w.first_rows + (plan.dense ? align_up((uint64_t)a->batch * 4, 256) : 0);
+    return w;
 }
 
 // query rows per sequence: 0 and 1 both mean a decode step
@@ -280,47 +333,64 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
     return 0;
 }
 
-void plan_mla_decode(const zllm_mla_decode_args* a, uint32_t* chunk_tokens, uint32_t* max_chunks)
+struct MlaSplitPlan {
+    uint32_t chunk_tokens, max_chunks;
+    uint64_t record_rows; // rows of the record arrays
+    bool dense;           // numbered over the live splits (see GqaSplitPlan)
+};
+
+MlaSplitPlan plan_mla_decode(const zllm_mla_decode_args* a)
 {
+    MlaSplitPlan plan;
     // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
     const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
-    const uint64_t per_sequence = (uint64_t)mla_query_rows(a) * head_blocks; // workgroups per split of a sequence
+    const uint64_t query_rows = mla_query_rows(a);
+    const uint64_t per_sequence = query_rows * head_blocks; // workgroups per split of a sequence
+    const uint64_t cus = compute_units();
     const uint64_t uniform_total = (uint64_t)a->batch * a->max_ctx_len;
-    if (a->selection == nullptr && a->total_ctx_tokens != 0 && a->total_ctx_tokens < uniform_total &&
-        kComputeUnits > 2 * a->batch * per_sequence) {
-        // ragged batch, as in plan_gqa_decode: sum_b ceil(len_b / chunk) <= total / chunk + batch.  The records are
-        // [row][max_chunks][head][512] floats: a plan whose records would pass 512 MiB keeps longer splits.
-        const uint64_t slots = kComputeUnits / per_sequence - a->batch;
+    plan.dense = false;
+    if (a->selection == nullptr && a->total_ctx_tokens != 0 && a->total_ctx_tokens < uniform_total && cus > 2 * a->batch * per_sequence) {
+        // ragged batch, as in plan_gqa_decode: sum_b ceil(len_b / chunk) <= total / chunk + batch
+        const uint64_t slots = cus / per_sequence - a->batch;
         uint64_t chunk = (a->total_ctx_tokens + slots - 1) / slots;
         chunk = align_up(chunk < 64 ? 64 : chunk, 32);
-        const uint64_t record_bytes = (uint64_t)a->batch * mla_query_rows(a) * a->heads * a->latent_dim * 4;
-        const uint64_t most = ((uint64_t)512 << 20) / record_bytes;
-        const uint64_t fewest_tokens = align_up(((uint64_t)longest + (most < 1 ? 1 : most) - 1) / (most < 1 ? 1 : most), 32);
-        if (chunk < fewest_tokens) {
-            chunk = fewest_tokens;
-        }
-        *chunk_tokens = (uint32_t)chunk;
-        *max_chunks = (uint32_t)(((uint64_t)longest + chunk - 1) / chunk);
-        return;
+        plan.chunk_tokens = (uint32_t)chunk;
+        plan.max_chunks = (uint32_t)(((uint64_t)longest + chunk - 1) / chunk);
+        plan.dense = true;
+    } else {
+        plan_splits(longest, (uint64_t)a->batch * per_sequence, 1, 64, &plan.chunk_tokens, &plan.max_chunks);
     }
-    plan_splits(longest, (uint64_t)a->batch * per_sequence, 1, 64, chunk_tokens, max_chunks);
+    const uint64_t rows = (uint64_t)a->batch * query_rows;
+    plan.record_rows = rows * plan.max_chunks;
+    if (plan.dense) {
+        // every query row of a sequence sees at most the sequence's tokens: query_rows x (total / chunk) + one per row
+        const uint64_t live = query_rows * (a->total_ctx_tokens / plan.chunk_tokens) + rows;
+        if (live < plan.record_rows && live <= UINT32_MAX) {
+            plan.record_rows = live;
+        } else {
+            plan.dense = false;
+        }
+    }
+    return plan;
 }
 
 struct MlaWorkspace {
-    uint64_t absorbed, partial, stats, weighted, total;
+    uint64_t absorbed, partial, stats, weighted, first_rows, total;
 };
 
-MlaWorkspace mla_workspace(const zllm_mla_decode_args* a, uint32_t max_chunks)
+MlaWorkspace mla_workspace(const zllm_mla_decode_args* a, const MlaSplitPlan& plan)
 {
     MlaWorkspace w;
     const uint64_t rows = (uint64_t)a->batch * mla_query_rows(a) * a->heads;
+    const uint64_t records = plan.record_rows * a->heads;
     w.absorbed = 0;
     w.partial = align_up(rows * (a->latent_dim + a->rope_dim) * 2, 256);
-    w.stats = w.partial + align_up(rows * max_chunks * a->latent_dim * 4, 256);
-    w.weighted = w.stats + align_up(rows * max_chunks * 8, 256);
-    w.total = w.weighted + align_up(rows * a->latent_dim * 4, 256);
+    w.stats = w.partial + align_up(records * a->latent_dim * 4, 256);
+    w.weighted = w.stats + align_up(records * 8, 256);
+    w.first_rows = w.weighted + align_up(rows * a->latent_dim * 4, 256);
+    w.total = w.first_rows + (plan.dense ? align_up((uint64_t)a->batch * mla_query_rows(a) * 4, 256) : 0);
     return w;
 }
 
@@ -724,10 +794,7 @@ uint64_t zllm_attn_gqa_decode_workspace_bytes(const zllm_gqa_decode_args* a)
     if (validate_gqa_decode(a) != 0) {
         return 0;
     }
-    uint32_t chunk_tokens, max_chunks;
-    plan_gqa_decode(a, &chunk_tokens, &max_chunks);
-    const uint64_t rows = (uint64_t)a->batch * max_chunks * a->num_heads;
-    return align_up(rows * a->head_dim * 4, 256) + align_up(rows * 8, 256);
+    return gqa_workspace(a, plan_gqa_decode(a)).total;
 }
 
 // The decode call over a workspace that is either the caller's or the library's static array.
@@ -761,10 +828,16 @@ static int gqa_decode_over(const zllm_gqa_decode_args* a, void* workspace, uint6
     p.kv_lens = a->kv_lens;
     p.first_visible = a->first_visible;
     p.out = a->out;
-    plan_gqa_decode(a, &p.chunk_tokens, &p.max_chunks);
-    const uint64_t rows = (uint64_t)a->batch * p.max_chunks * a->num_heads;
+    const GqaSplitPlan plan = plan_gqa_decode(a);
+    const GqaWorkspace layout = gqa_workspace(a, plan);
+    p.chunk_tokens = plan.chunk_tokens;
+    p.max_chunks = plan.max_chunks;
     p.partial = (float*)workspace;
-    p.stats = (float*)((char*)workspace + align_up(rows * a->head_dim * 4, 256));
+    p.stats = (float*)((char*)workspace + layout.stats);
+    if (plan.dense) {
+        p.record_rows = (unsigned int)plan.record_rows;
+        p.first_rows = (unsigned int*)((char*)workspace + layout.first_rows);
+    }
     p.batch = a->batch;
     p.num_heads = a->num_heads;
     p.num_kv_heads = a->num_kv_heads;
@@ -797,14 +870,34 @@ int zllm_attn_gqa_decode_split_plan(const zllm_gqa_decode_args* a, uint32_t* chu
     if (rc != 0) {
         return rc;
     }
-    uint32_t chunk = 0, chunks = 0;
-    plan_gqa_decode(a, &chunk, &chunks);
+    const GqaSplitPlan plan = plan_gqa_decode(a);
     if (chunk_tokens != nullptr) {
-        *chunk_tokens = chunk;
+        *chunk_tokens = plan.chunk_tokens;
     }
     if (max_chunks != nullptr) {
-        *max_chunks = chunks;
+        *max_chunks = plan.max_chunks;
     }
+    return 0;
+}
+
+int zllm_attn_gqa_decode_record_layout(const zllm_gqa_decode_args* a, zllm_split_record_layout* out)
+{
+    const int rc = validate_gqa_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    if (out == nullptr) {
+        return fail(-1, "GQA decode record layout: null output");
+    }
+    const GqaSplitPlan plan = plan_gqa_decode(a);
+    const GqaWorkspace layout = gqa_workspace(a, plan);
+    out->record_rows = plan.record_rows;
+    out->partial_offset = 0;
+    out->stats_offset = layout.stats;
+    out->first_rows_offset = plan.dense ? layout.first_rows : 0;
+    out->chunk_tokens = plan.chunk_tokens;
+    out->max_chunks = plan.max_chunks;
+    out->dense = plan.dense ? 1u : 0u;
     return 0;
 }
 
@@ -848,9 +941,28 @@ uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* a)
     if (validate_mla_decode(a) != 0) {
         return 0;
     }
-    uint32_t chunk_tokens, max_chunks;
-    plan_mla_decode(a, &chunk_tokens, &max_chunks);
-    return mla_workspace(a, max_chunks).total;
+    return mla_workspace(a, plan_mla_decode(a)).total;
+}
+
+int zllm_attn_mla_decode_record_layout(const zllm_mla_decode_args* a, zllm_split_record_layout* out)
+{
+    const int rc = validate_mla_decode(a);
+    if (rc != 0) {
+        return rc;
+    }
+    if (out == nullptr) {
+        return fail(-1, "MLA decode record layout: null output");
+    }
+    const MlaSplitPlan plan = plan_mla_decode(a);
+    const MlaWorkspace w = mla_workspace(a, plan);
+    out->record_rows = plan.record_rows;
+    out->partial_offset = w.partial;
+    out->stats_offset = w.stats;
+    out->first_rows_offset = plan.dense ? w.first_rows : 0;
+    out->chunk_tokens = plan.chunk_tokens;
+    out->max_chunks = plan.max_chunks;
+    out->dense = plan.dense ? 1u : 0u;
+    return 0;
 }
 
 int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
@@ -870,8 +982,10 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     }
     zllm::MlaDecodeParams p;
     memset(&p, 0, sizeof(p));
-    plan_mla_decode(a, &p.chunk_tokens, &p.max_chunks);
-    const MlaWorkspace w = mla_workspace(a, p.max_chunks);
+    const MlaSplitPlan plan = plan_mla_decode(a);
+    p.chunk_tokens = plan.chunk_tokens;
+    p.max_chunks = plan.max_chunks;
+    const MlaWorkspace w = mla_workspace(a, plan);
     if (a->workspace_bytes < w.total) {
         return fail(-1, "MLA decode: workspace %llu bytes, need %llu", (unsigned long long)a->workspace_bytes, (unsigned long long)w.total);
     }
@@ -892,6 +1006,10 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     p.partial = (float*)(ws + w.partial);
     p.stats = (float*)(ws + w.stats);
     p.weighted = (float*)(ws + w.weighted);
+    if (plan.dense) {
+        p.record_rows = (unsigned int)plan.record_rows;
+        p.first_rows = (unsigned int*)(ws + w.first_rows);
+    }
     p.query_rows = mla_query_rows(a);
     p.batch = a->batch * p.query_rows; // the kernels index query rows; a row finds its sequence by division
     p.heads = a->heads;

@@ -169,9 +169,16 @@ __device__ __forceinline__ WaveItem wave_item(const GqaDecodeParams& p)
 // `span_out` is the split length of the item's sequence: its visible range cut into equal 32-aligned parts (never
 // longer than the planned chunk_tokens), so that a ragged batch has no full-length splits next to short remainders --
 // the longest split sets the kernel's duration.
+// `row_out` is the item's row in the split record arrays: sequence x max_chunks + split, or, when the records are numbered
+// densely, the item number itself -- the first split of a sequence then leaves its row in first_rows for the merge, and an
+// item past the rows the host sized (a total_kv_tokens hint below the real sum) is dropped rather than written out of bounds.
 __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned int item, unsigned int lane, unsigned int& b_out,
-                                             unsigned int& chunk_out, unsigned int& len_out, unsigned int& first_out, unsigned int& span_out)
+                                             unsigned int& chunk_out, unsigned int& len_out, unsigned int& first_out, unsigned int& span_out,
+                                             unsigned int& row_out)
 {
+    if (p.record_rows != 0u && item >= p.record_rows) {
+        return false;
+    }
     unsigned int base = 0;
     for (unsigned int b0 = 0; b0 < p.batch; b0 += 64u) {
         const unsigned int i = b0 + lane;
@@ -202,6 +209,13 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
             len_out = __builtin_amdgcn_readlane(len, src); // already here: no second trip to memory for them
             first_out = __builtin_amdgcn_readlane(first, src);
             span_out = __builtin_amdgcn_readlane(span, src);
+            row_out = b_out * p.max_chunks + chunk_out;
+            if (p.record_rows != 0u) {
+                row_out = item;
+                if (chunk_out == 0u && lane == 0u) {
+                    p.first_rows[b_out] = item; // every wave of the split writes the same number
+                }
+            }
             return true;
         }
         base += total;
@@ -458,8 +472,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const WaveItem mine = wave_item(p);
     const unsigned int kvh = mine.kvh;
     const unsigned int head_block = mine.head_block;
-    unsigned int b, chunk, len, first, span;
-    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    unsigned int b, chunk, len, first, span, row;
+    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span, row)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -468,7 +482,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
 
-    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    const size_t stat_index = ((size_t)row * p.num_heads + head) * 2;
     if (c_start64 >= len) {
         if (head_valid && j == 0) {
             p.stats[stat_index] = kNegInf;
@@ -669,7 +683,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             p.stats[stat_index] = run_max;
             p.stats[stat_index + 1] = total;
         }
-        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
+        float* out = p.partial + ((size_t)row * p.num_heads + head) * D;
         // tile (a, e), register r holds dim a*64 + 16*j + 4*r + e
 #pragma unroll
         for (int a = 0; a < G; ++a) {
@@ -737,8 +751,8 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         entries0 = guess_table[min(guess_page + lane, last_page)];
         entries1 = guess_table[min(guess_page + 64u + lane, last_page)];
     }
-    unsigned int b, chunk, len, first, span;
-    if (!locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    unsigned int b, chunk, len, first, span, row;
+    if (!locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span, row)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -746,7 +760,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
     const unsigned int head_in_group = head_block * 16u + m;
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
-    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    const size_t stat_index = ((size_t)row * p.num_heads + head) * 2;
     if (c_start64 >= len) {
         if (head_valid && j == 0) {
             p.stats[stat_index] = kNegInf;
@@ -940,7 +954,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
             p.stats[stat_index] = run_max;
             p.stats[stat_index + 1] = total;
         }
-        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
+        float* out = p.partial + ((size_t)row * p.num_heads + head) * D;
 #pragma unroll
         for (int a = 0; a < G; ++a) {
 #pragma unroll
@@ -972,8 +986,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const WaveItem mine = wave_item(p);
     const unsigned int kvh = mine.kvh;
     const unsigned int head_block = mine.head_block;
-    unsigned int b, chunk, len, first, span;
-    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span)) {
+    unsigned int b, chunk, len, first, span, row;
+    if (kvh >= p.num_kv_heads || !locate_split(p, mine.item, threadIdx.x & 63u, b, chunk, len, first, span, row)) {
         return;
     }
     const unsigned int first_al = first & ~31u;
@@ -981,7 +995,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
     const unsigned int head_in_group = head_block * 16u + m;
     const bool head_valid = head_in_group < p.group;
     const unsigned int head = kvh * p.group + head_in_group;
-    const size_t stat_index = (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * 2;
+    const size_t stat_index = ((size_t)row * p.num_heads + head) * 2;
     if (c_start64 >= len) {
         if (head_valid && j == 0) {
             p.stats[stat_index] = kNegInf;
@@ -1234,7 +1248,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
             p.stats[stat_index] = run_max;
             p.stats[stat_index + 1] = total;
         }
-        float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.num_heads + head) * D;
+        float* out = p.partial + ((size_t)row * p.num_heads + head) * D;
         // tile t, register r holds dim (4*j + r) * (D/16) + t ; undo the P scaling
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
@@ -1243,6 +1257,21 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_f16_partial(Gq
                 out[(4 * j + r) * (D / 16) + t] = acc[t][r] * (1.0f / kPScale);
             }
         }
+    }
+}
+
+// Where a merge finds the records of record group `b`: `base` is its first row, `last` the largest split index whose
+// address may be formed (loads are issued before the split count is known and clamped to it).  Densely numbered records
+// start at the row the group's first split left in first_rows; a group without splits never wrote its entry, so what is
+// read there is clamped into the arrays and never used.
+__device__ __forceinline__ void merge_rows(const GqaDecodeParams& p, unsigned int b, size_t& base, unsigned int& last)
+{
+    base = (size_t)b * p.max_chunks;
+    last = p.max_chunks - 1u;
+    if (p.record_rows != 0u) {
+        const unsigned int first = min(p.first_rows[b], p.record_rows - 1u);
+        base = first;
+        last = min(last, p.record_rows - 1u - first);
     }
 }
 
@@ -1273,9 +1302,12 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
         const unsigned int first_al = first & ~31u;
         chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     }
-    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    size_t base;
+    unsigned int last;
+    merge_rows(p, b, base, last);
+    const float* stats = p.stats + (base * p.num_heads + head) * 2;
     const size_t stat_stride = (size_t)p.num_heads * 2;
-    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;
+    const float* partial = p.partial + (base * p.num_heads + head) * p.head_dim + quad * 4u;
     const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
 
     // single pass, four splits per trip with all eight loads issued before any is used
@@ -1291,7 +1323,7 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
         float2 st[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const unsigned int c = min(c0 + u * lanes, p.max_chunks - 1u);
+            const unsigned int c = min(c0 + u * lanes, last);
             st[u] = *(const float2*)(stats + c * stat_stride);
             part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
@@ -1385,16 +1417,19 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_wide(GqaDecodeParams p)
     const unsigned int quad = threadIdx.x & 7u;
     const unsigned int sl = threadIdx.x >> 3;
     const unsigned int column = blockIdx.z * 32u + quad * 4u;
-    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    size_t base;
+    unsigned int last;
+    merge_rows(p, b, base, last);
+    const float* stats = p.stats + (base * p.num_heads + head) * 2;
     const size_t stat_stride = (size_t)p.num_heads * 2;
-    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + column;
+    const float* partial = p.partial + (base * p.num_heads + head) * p.head_dim + column;
     const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
     // first trip: addresses clamped to the planned splits, so the loads do not wait for the length
     float2 st[8];
     f32x4 part[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        const unsigned int c = min(sl + 32u * u, p.max_chunks - 1u);
+        const unsigned int c = min(sl + 32u * u, last);
         st[u] = *(const float2*)(stats + c * stat_stride);
         part[u] = *(const f32x4*)(partial + c * partial_stride);
     }
@@ -1430,7 +1465,7 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_wide(GqaDecodeParams p)
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const unsigned int c = min(c0 + 256u + 32u * u, p.max_chunks - 1u);
+            const unsigned int c = min(c0 + 256u + 32u * u, last);
             st[u] = *(const float2*)(stats + c * stat_stride);
             part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
@@ -1512,9 +1547,12 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_few(GqaDecodeParams p)
         const unsigned int first_al = first & ~31u;
         chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     }
-    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.num_heads + head) * 2;
+    size_t base;
+    unsigned int last;
+    merge_rows(p, b, base, last);
+    const float* stats = p.stats + (base * p.num_heads + head) * 2;
     const size_t stat_stride = (size_t)p.num_heads * 2;
-    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.num_heads + head) * p.head_dim + quad * 4u;
+    const float* partial = p.partial + (base * p.num_heads + head) * p.head_dim + quad * 4u;
     const size_t partial_stride = (size_t)p.num_heads * p.head_dim;
     float m = kNegInf, l = 0.0f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -1523,7 +1561,7 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_few(GqaDecodeParams p)
         f32x4 part[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const unsigned int c = min(c0 + u, p.max_chunks - 1u);
+            const unsigned int c = min(c0 + u, last);
             st[u] = *(const float2*)(stats + c * stat_stride);
             part[u] = *(const f32x4*)(partial + c * partial_stride);
         }
@@ -1663,7 +1701,9 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& args, int kv_format, int sca
     const unsigned int kvh_blocks = (p.num_kv_heads + waves - 1) / waves;
     const unsigned int head_blocks = (p.group + 15u) / 16u;
     p.items_per_group = gqa_decode_items_per_group(p.head_dim, p.num_kv_heads);
-    const dim3 grid((p.max_chunks * p.batch + p.items_per_group - 1u) / p.items_per_group, kvh_blocks * head_blocks, 1);
+    // densely numbered records are sized for the live splits: no workgroups beyond them
+    const unsigned int items = p.record_rows != 0u ? p.record_rows : p.max_chunks * p.batch;
+    const dim3 grid((items + p.items_per_group - 1u) / p.items_per_group, kvh_blocks * head_blocks, 1);
     const dim3 block(waves * p.items_per_group * 64u);
     const bool pow2 = (p.block_tokens & (p.block_tokens - 1u)) == 0;
     const bool fast = pow2 && p.block_tokens >= 16u && p.ring_capacity % 16u == 0;

@@ -87,8 +87,13 @@ struct GqaDecodeParams {
     const unsigned int* kv_lens;
     const unsigned int* first_visible;
     float* out;
-    float* partial; // [batch][max_chunks][num_heads][head_dim]
-    float* stats;   // [batch][max_chunks][num_heads][2] = (max, sum)
+    float* partial; // [record row][num_heads][head_dim]
+    float* stats;   // [record row][num_heads][2] = (max, sum)
+    // Record rows.  record_rows == 0: row = sequence * max_chunks + split.  Otherwise the records are numbered like the
+    // work items, densely over the live splits: row = first_rows[sequence] + split, `record_rows` rows in all; the
+    // partial kernel writes first_rows, the merge reads it.
+    unsigned int* first_rows;
+    unsigned int record_rows;
     unsigned int batch, num_heads, num_kv_heads, head_dim, group;
     unsigned int table_stride, block_tokens, block_shift, ring_capacity;
     unsigned int chunk_tokens, max_chunks;
@@ -146,8 +151,13 @@ struct MlaDecodeParams {
     const unsigned int* ctx_lens;
     void* out;
     unsigned short* absorbed; // bf16 [batch][heads][latent_dim + rope_dim] (absorbed nope | q_rope)
-    float* partial;           // [batch][max_chunks][heads][latent_dim]
-    float* stats;             // [batch][max_chunks][heads][2]
+    float* partial;           // [record row][heads][latent_dim]
+    float* stats;             // [record row][heads][2]
+    // Record rows.  record_rows == 0: row = query row * max_chunks + split, and the partial grid is (split, head block,
+    // query row).  Otherwise records and work items are numbered densely over the live splits (grid = (item, head block)):
+    // row = first_rows[query row] + split; the partial kernel writes first_rows, the merges read it.
+    unsigned int* first_rows;
+    unsigned int record_rows;
     float* weighted;          // [batch][heads][latent_dim]
     unsigned int batch, heads, q_head_dim, kv_head_dim, latent_dim, rope_dim, nope_dim, value_dim;
     unsigned int column_split; // mla_absorb_mfma: waves that share a block of sixteen rows (set by the launcher)

@@ -26,6 +26,7 @@
 
 #include "common.hpp"
 #include "kernels.hpp"
+#include "mla_rows.hpp"
 
 namespace zllm {
 
@@ -65,17 +66,6 @@ __device__ __forceinline__ unsigned int swz(unsigned int row)
 __device__ __forceinline__ unsigned int tile_offset(unsigned int row, unsigned int chunk)
 {
     return row * kRowBytes + ((chunk ^ swz(row)) << 4);
-}
-
-// Query row v of the call: its sequence and the number of tokens it sees.  With query_rows > 1 the rows of a
-// sequence are the last query_rows tokens of its context, each seeing everything up to and including itself
-// (src/kernel/cpu/mla.rs:1016-1018: row r of a chunk at query_start sees query_start + r + 1 tokens).
-__device__ __forceinline__ unsigned int visible_tokens(const unsigned int* ctx_lens, unsigned int query_rows, unsigned int v, unsigned int& sequence)
-{
-    sequence = v / query_rows;
-    const unsigned int behind = query_rows - 1u - v % query_rows; // rows of the chunk after this one
-    const unsigned int len = ctx_lens[sequence];
-    return len > behind ? len - behind : 0u;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -421,16 +411,20 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
     const unsigned int hw = wave & 3u;
     const unsigned int m = lane & 15u;
     const unsigned int j = lane >> 4;
-    const unsigned int chunk = blockIdx.x;
+    // the split and the query row this workgroup works on: grid coordinates, or looked up from the dense item number.
+    // Query rows run the last first: the rows of a chunk see more keys the later they come, and workgroups are handed
+    // out in the order of their index
+    unsigned int chunk = blockIdx.x;
+    unsigned int b = gridDim.z - 1u - blockIdx.z;
+    if (p.record_rows != 0u && !mla_locate_split(p, blockIdx.x, lane, b, chunk)) {
+        return;
+    }
     // NARROW (a call of at most 32 heads: head tiles 2 and 3 would be empty): the four score waves are two head tiles x
     // two halves of a step's tokens, each half with its own running maximum and sum, and every value wave takes both
     // head tiles and a quarter of the columns.
     const unsigned int score_tile = NARROW ? (hw & 1u) : hw; // head tile of a score wave
     const unsigned int stream = NARROW ? (hw >> 1) : 0u;     // narrow: which sixteen tokens of a step it scores
     const unsigned int head = blockIdx.y * 64u + score_tile * 16u + m; // this lane's head column
-    // query row of the call (= sequence when every sequence has one row), the last first: the rows of a chunk see more keys
-    // the later they come, and workgroups are handed out in the order of their index
-    const unsigned int b = gridDim.z - 1u - blockIdx.z;
     unsigned int seq;
     unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq); // keys of this row: positions, or list slots when a selection applies
     const unsigned int* selected = nullptr;
@@ -445,7 +439,8 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
     const unsigned int n_splits = min(p.max_chunks, (len + p.chunk_tokens - 1u) / p.chunk_tokens);
     const unsigned int span = n_splits > 0u ? min(p.chunk_tokens, (((len + n_splits - 1u) / n_splits) + 31u) & ~31u) : p.chunk_tokens;
     const unsigned long long c_start64 = (unsigned long long)chunk * span;
-    const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
+    const size_t row = p.record_rows != 0u ? (size_t)blockIdx.x : (size_t)b * p.max_chunks + chunk;
+    const size_t rec = row * p.heads + head;
     if (c_start64 >= len) { // empty split: (max, sum) = (-inf, 0), merge skips it
         if (head < p.heads && j == 0 && !value_role) {
             p.stats[rec * 2] = kNegInf;
@@ -1189,7 +1184,7 @@ template <bool ALIGNED, bool SELECTED, bool POW2 = false, bool NARROW = false> _
         for (int ht = 0; ht < 2; ++ht) {
             const unsigned int out_head = blockIdx.y * 64u + (2u * hp + ht) * 16u + m;
             if (out_head < p.heads) {
-                float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + part * (GROUPS * 64u);
+                float* out = p.partial + (row * p.heads + out_head) * kLatent + part * (GROUPS * 64u);
                 const float out_of_window = __uint_as_float((unsigned int)(127 + window) << 23);
 #pragma unroll
                 for (int t = 0; t < GROUPS * 4; ++t) {
@@ -1300,10 +1295,11 @@ __global__ __launch_bounds__(256) void mla_merge_project(MlaDecodeParams p)
     }
     unsigned int seq;
     const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
-    const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
-    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+    unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+    const size_t base = mla_merge_base(p, b, chunks);
+    const float* stats = p.stats + (base * p.heads + head) * 2;
     const size_t stat_stride = (size_t)p.heads * 2;
-    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+    const float* partial = p.partial + (base * p.heads + head) * kLatent + quad * 4u;
     const size_t partial_stride = (size_t)p.heads * kLatent;
     float m = kNegInf, l = 0.0f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -1434,13 +1430,22 @@ __global__ __launch_bounds__(256) void mla_merge_wide(MlaDecodeParams p)
     const unsigned int quad = tid & 15u;
     const unsigned int sl = tid >> 4;
     const unsigned int column = blockIdx.z * 64u + quad * 4u;
-    const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+    // every planned split has a record (an empty one says so) when the rows are [query row][max_chunks]; densely numbered
+    // rows hold live splits only, so there the row's own count bounds the walk
+    unsigned int limit = p.max_chunks;
+    if (p.record_rows != 0u) {
+        unsigned int seq;
+        const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
+        limit = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+    }
+    const size_t base = mla_merge_base(p, b, limit);
+    const float* stats = p.stats + (base * p.heads + head) * 2;
     const size_t stat_stride = (size_t)p.heads * 2;
-    const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + column;
+    const float* partial = p.partial + (base * p.heads + head) * kLatent + column;
     const size_t partial_stride = (size_t)p.heads * kLatent;
     float m = kNegInf, l = 0.0f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (unsigned int c0 = sl; c0 < p.max_chunks; c0 += 256u) {
+    for (unsigned int c0 = sl; c0 < limit; c0 += 256u) {
         float cm[16], cl[16];
         f32x4 part[16];
 #pragma unroll
@@ -1449,7 +1454,7 @@ __global__ __launch_bounds__(256) void mla_merge_wide(MlaDecodeParams p)
             cm[u] = kNegInf;
             cl[u] = 0.0f;
             part[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (c < p.max_chunks) { // a plan of few splits leaves most of a lane's sixteen requests unmade
+            if (c < limit) { // a plan of few splits leaves most of a lane's sixteen requests unmade
                 const float2 st = *(const float2*)(stats + c * stat_stride);
                 cm[u] = st.x;
                 cl[u] = st.y;
@@ -1520,10 +1525,11 @@ template <int R> __global__ __launch_bounds__(256) void mla_merge_project_rows(M
         const unsigned int b = min(row0 + r, p.batch - 1u);
         unsigned int seq;
         const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
-        const unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
-        const float* stats = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
+        unsigned int chunks = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
+        const size_t base = mla_merge_base(p, b, chunks);
+        const float* stats = p.stats + (base * p.heads + head) * 2;
         const size_t stat_stride = (size_t)p.heads * 2;
-        const float* partial = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+        const float* partial = p.partial + (base * p.heads + head) * kLatent + quad * 4u;
         const size_t partial_stride = (size_t)p.heads * kLatent;
         float m = kNegInf, l = 0.0f;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -1686,8 +1692,9 @@ template <int MODE, int WAVES = 8> __global__ __launch_bounds__(64 * WAVES) void
                 unsigned int seq;
                 const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
                 chunks[u] = (unsigned int)min((unsigned long long)p.max_chunks, ((unsigned long long)len + p.chunk_tokens - 1u) / p.chunk_tokens);
-                stats[u] = p.stats + ((size_t)b * p.max_chunks * p.heads + head) * 2;
-                partial[u] = p.partial + ((size_t)b * p.max_chunks * p.heads + head) * kLatent + quad * 4u;
+                const size_t base = mla_merge_base(p, b, chunks[u]);
+                stats[u] = p.stats + (base * p.heads + head) * 2;
+                partial[u] = p.partial + (base * p.heads + head) * kLatent + quad * 4u;
                 mx[u] = kNegInf;
                 l[u] = 0.0f;
                 acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1825,6 +1832,8 @@ static hipError_t merge_into_workspace(const MlaDecodeParams& p, hipStream_t str
     mp.chunk_tokens = p.chunk_tokens;
     mp.max_chunks = p.max_chunks;
     mp.query_rows = p.query_rows;
+    mp.record_rows = p.record_rows;
+    mp.first_rows = p.first_rows;
     return launch_split_merge(mp, stream);
 }
 
@@ -1866,7 +1875,8 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
     }
     if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
-        const dim3 grid(p.max_chunks, (p.heads + 63) / 64, p.batch);
+        // densely numbered records are sized for the live splits: one workgroup per item and head block
+        const dim3 grid = p.record_rows != 0u ? dim3(p.record_rows, (p.heads + 63) / 64, 1) : dim3(p.max_chunks, (p.heads + 63) / 64, p.batch);
         const bool narrow = p.heads <= 32u; // two head tiles at most: the score waves split a step's tokens, the value waves the columns four ways
         const bool aligned = p.block_tokens % kStepTokens == 0 && p.chunk_tokens % kStepTokens == 0;
         const bool pow2_tables = (p.block_tokens & (p.block_tokens - 1u)) == 0 && p.tables != nullptr;

@@ -23,6 +23,7 @@
 
 #include "common.hpp"
 #include "kernels.hpp"
+#include "mla_rows.hpp"
 
 namespace zllm {
 
@@ -85,14 +86,6 @@ __device__ __forceinline__ float pair_sum(float v)
     return __uint_as_float(s.x) + __uint_as_float(s.y);
 }
 
-__device__ __forceinline__ unsigned int visible_tokens(const unsigned int* ctx_lens, unsigned int query_rows, unsigned int v, unsigned int& sequence)
-{
-    sequence = v / query_rows;
-    const unsigned int behind = query_rows - 1u - v % query_rows;
-    const unsigned int len = ctx_lens[sequence];
-    return len > behind ? len - behind : 0u;
-}
-
 
 // Sixteen codes of one scale group -> sixteen f16 values code * factor: the 16-byte chunks 2 k and 2 k + 1 of a tile row.
 __device__ __forceinline__ void convert_run(const u32x4& codes, _Float16 f, unsigned char* tile, unsigned int row, unsigned int k)
@@ -134,8 +127,13 @@ __global__ __launch_bounds__(512) void mla_partial_x32(MlaDecodeParams p)
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned int n32 = lane & 31u;
     const unsigned int half = lane >> 5;
-    const unsigned int chunk = blockIdx.x;
-    const unsigned int b = gridDim.z - 1u - blockIdx.z; // rows of a chunk see more keys the later they come: longest first
+    // grid coordinates, or looked up from the dense item number when the records are numbered that way
+    unsigned int chunk = blockIdx.x;
+    unsigned int b = gridDim.z - 1u - blockIdx.z; // rows of a chunk see more keys the later they come: longest first
+    if (p.record_rows != 0u && !mla_locate_split(p, blockIdx.x, lane, b, chunk)) {
+        return;
+    }
+    const size_t row = p.record_rows != 0u ? (size_t)blockIdx.x : (size_t)b * p.max_chunks + chunk;
     unsigned int seq;
     const unsigned int len = visible_tokens(p.ctx_lens, p.query_rows, b, seq);
     const unsigned int n_splits = min(p.max_chunks, (len + p.chunk_tokens - 1u) / p.chunk_tokens);
@@ -147,7 +145,7 @@ __global__ __launch_bounds__(512) void mla_partial_x32(MlaDecodeParams p)
         if (score_role && half == 0u) {
             const unsigned int head = blockIdx.y * 64u + wave * 32u + n32;
             if (head < p.heads) {
-                const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
+                const size_t rec = row * p.heads + head;
                 p.stats[rec * 2] = kNegInf;
                 p.stats[rec * 2 + 1] = 0.0f;
             }
@@ -574,7 +572,7 @@ __global__ __launch_bounds__(512) void mla_partial_x32(MlaDecodeParams p)
             const float total = wave_sum_16x4(run_sum[H]) * (1.0f / (float)(1 << kPShift));
             const unsigned int head = head0 + 16u * H;
             if (head < p.heads && j4 == 0u) {
-                const size_t rec = ((size_t)b * p.max_chunks + chunk) * p.heads + head;
+                const size_t rec = row * p.heads + head;
                 p.stats[rec * 2] = run_max[H];
                 p.stats[rec * 2 + 1] = total;
             }
@@ -762,7 +760,7 @@ __global__ __launch_bounds__(512) void mla_partial_x32(MlaDecodeParams p)
             const int window = lds_window[ht];
             // acc = sum p 2^kPShift v / 2^(window - 127)
             const float up = __uint_as_float((unsigned int)min(max(window - kPShift, 1), 253) << 23);
-            float* out = p.partial + (((size_t)b * p.max_chunks + chunk) * p.heads + out_head) * kLatent + 128u * v + 4u * half;
+            float* out = p.partial + (row * p.heads + out_head) * kLatent + 128u * v + 4u * half;
 #pragma unroll
             for (int ct = 0; ct < 4; ++ct) {
 #pragma unroll
@@ -785,7 +783,7 @@ bool mla_partial_x32_takes(const MlaDecodeParams& p)
 
 hipError_t launch_mla_partial_x32(const MlaDecodeParams& p, hipStream_t stream)
 {
-    const dim3 grid(p.max_chunks, (p.heads + 63) / 64, p.batch);
+    const dim3 grid = p.record_rows != 0u ? dim3(p.record_rows, (p.heads + 63) / 64, 1) : dim3(p.max_chunks, (p.heads + 63) / 64, p.batch);
     mla_partial_x32<<<grid, dim3(512), 0, stream>>>(p);
     return hipGetLastError();
 }
