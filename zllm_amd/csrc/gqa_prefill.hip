@@ -153,11 +153,24 @@ template <int SDT, bool SOFTCAP, bool POW2, int CT = 2>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
     constexpr int kColTiles = CT; // inside the kernel the name means this instantiation's count
-    __shared__ __align__(16) unsigned char lds_k[2][kTileBytes];
-    __shared__ __align__(16) unsigned char lds_v[2][kTileBytes];
-    __shared__ __align__(16) float lds_ks[2][2][kStep]; // [buffer][group][token]
-    __shared__ __align__(16) float lds_vs[2][2][kStep];
-    __shared__ __align__(16) float lds_top[2][8];       // [buffer][staging wave]: largest scale the wave converted (4..7: V)
+    // Four tile buffers: a pass of the main loop attends two 32-token tiles (buffers 2 s and 2 s + 1) while the next two
+    // are loaded, converted and stored into the other pair, with one barrier per 64 tokens.
+    // One block, the small arrays first: every address a step forms is then a register (the lane's part) plus an
+    // immediate below 64 KiB (the buffer's part), which is as far as an LDS instruction's offset field reaches.
+    struct Lds {
+        float ks[4][2][kStep]; // [buffer][group][token]
+        float vs[4][2][kStep];
+        float top[4][8];       // [buffer][staging wave]: largest scale the wave converted (4..7: V)
+        unsigned char k[4][kTileBytes];
+        unsigned char v[4][kTileBytes];
+    };
+    static_assert(offsetof(Lds, v) + 4 * kTileBytes <= 65536 + 2048 + 128, "tile buffers must stay within reach of LDS offsets");
+    __shared__ __align__(16) Lds lds;
+    auto& lds_k = lds.k;
+    auto& lds_v = lds.v;
+    auto& lds_ks = lds.ks;
+    auto& lds_vs = lds.vs;
+    auto& lds_top = lds.top;
 
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -572,16 +585,15 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
     load_step(regs, part.begin, entry_of(part.begin + st_token));
     unsigned int entry_next = entry_of(part.begin + kStep + st_token);
     store_step(regs, 0);
+    load_step(regs, part.begin + kStep, entry_next); // past the range: its last row again
+    entry_next = entry_of(part.begin + 2u * kStep + st_token);
+    store_step(regs, 1);
     __syncthreads();
     unsigned int wv = 2u; // (biased) exponent of the largest V scale up to the tile being attended
     float v_shift = kPBias + 125.0f;
-    // `buf` is a literal at every call, so the LDS addresses of a step differ from the other buffer's only in the
+    // `buf` is a literal at every call, so the LDS addresses of a step differ from the other buffers' only in the
     // instructions' immediate offsets and cost no address arithmetic
-    auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
-        const unsigned int t0 = part.begin + step * kStep;
-        // rows past the end of the visible range repeat its last one: the loads stay inside the sequence's pages
-        load_step(regs, t0 + kStep, entry_next);
-        entry_next = entry_of(t0 + 2u * kStep + st_token);
+    auto attend_tile = [&](unsigned int t0, int buf) __attribute__((always_inline)) {
         const unsigned int wv_now = window_of(buf, wv);
         const bool window_moved = wv_now != wv; // rare: a V scale above everything met so far
         float acc_fix = 1.0f;
@@ -591,16 +603,36 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             v_shift = kPBias + (float)(127 - (int)wv);
         }
         compute_step(buf, t0, v_shift, acc_fix, window_moved);
-        store_step(regs, buf ^ 1);
+    };
+    // Tiles `step` and `step + 1` are in the buffers of `set`; the two after them travel, one at a time through the same
+    // registers, into the other pair, which nobody reads before the barrier.
+    auto two_steps = [&](unsigned int step, int set) __attribute__((always_inline)) {
+        const unsigned int t0 = part.begin + step * kStep;
+        // rows past the end of the visible range repeat its last one: the loads stay inside the sequence's pages
+        load_step(regs, t0 + 2u * kStep, entry_next);
+        entry_next = entry_of(t0 + 3u * kStep + st_token);
+        attend_tile(t0, 2 * set);
+        store_step(regs, 2 * (set ^ 1));
+        PREFILL_PHASE_FENCE(); // the two tiles are attended one after the other: interleaved, their operands do not fit the registers
+        load_step(regs, t0 + 3u * kStep, entry_next);
+        entry_next = entry_of(t0 + 4u * kStep + st_token);
+        attend_tile(t0 + kStep, 2 * set + 1);
+        store_step(regs, 2 * (set ^ 1) + 1);
         __syncthreads();
     };
     unsigned int step = 0;
-    for (; step + 1 < steps; step += 2) {
-        one_step(step, 0);
-        one_step(step + 1u, 1);
+    for (; step + 4 <= steps; step += 4) {
+        two_steps(step, 0);
+        two_steps(step + 2u, 1);
     }
-    if (step < steps) {
-        one_step(step, 0);
+    if (step + 2 <= steps) {
+        two_steps(step, 0);
+        step += 2;
+        if (step < steps) { // the odd tile at the end sits in the first buffer of the other pair
+            attend_tile(part.begin + step * kStep, 2);
+        }
+    } else if (step < steps) {
+        attend_tile(part.begin + step * kStep, 0);
     }
 
     // ---- normalise and store ------------------------------------------------------------------------
