@@ -452,7 +452,7 @@ ZLLM_API int zllm_attn_gqa_prologue(const zllm_gqa_prologue_args* args, zllm_str
  * [batch, heads * value_dim] (src/kernel/cpu/mla.rs:1064-1075) otherwise. */
 typedef struct zllm_mla_decode_args {
     const void* q;                /* [dev] [batch * rows, heads * q_head_dim], q_dtype */
-    const uint16_t* kv_b;         /* [dev] bf16 bits [heads * kv_head_dim, latent_dim] */
+    const uint16_t* kv_b;         /* [dev] bf16 bits [heads * kv_head_dim, latent_dim]; another form with kv_b_bits */
     const int8_t* latent_codes;   /* [dev] [rows, latent_dim] */
     const uint16_t* latent_scales;/* [dev] bf16 bits [rows, latent_dim / 64] */
     const uint16_t* rope_cache;   /* [dev] bf16 bits [rows, rope_dim] */
@@ -464,8 +464,8 @@ typedef struct zllm_mla_decode_args {
     uint32_t batch, heads;
     uint32_t q_head_dim;          /* nope + rope */
     uint32_t kv_head_dim;         /* nope + value */
-    uint32_t latent_dim;          /* 512 */
-    uint32_t rope_dim;            /* 64 */
+    uint32_t latent_dim;          /* a multiple of 64 up to 1024; 512 runs the matrix-core kernels */
+    uint32_t rope_dim;            /* even, up to 256; 64 runs the matrix-core kernels */
     uint32_t table_stride;
     uint32_t max_ctx_len;         /* host upper bound of ctx_lens (split plan); a recorded graph stays valid
                                      only while every ctx_lens[b] <= max_ctx_len */
@@ -501,6 +501,17 @@ typedef struct zllm_mla_decode_args {
      * so it must not be below the real sum -- like max_ctx_len it has to hold for every replay of a recorded call;
      * splits beyond the records it sized are dropped (wrong output, nothing out of bounds). */
     uint32_t total_ctx_tokens;
+    /* kv_b in the other forms the reference's weight loader reads (paged_weight,
+     * src/kernel/rocm/hip/attention/paged_mla/source.hip:2-26; W8A16 / W4A16 of ct_mla_weight,
+     * src/backend/rocm/attention.rs:181-192).  kv_b_bits 0 or 16: bf16 at kv_b.  32: f32 at kv_b.  8 / 4: codes at kv_b,
+     * packed low bits first into 32-bit words, ceil(latent_dim / (32 / bits)) words a row; element = (code - 128) or
+     * (code - 8) times kv_b_scales[row * (latent_dim / kv_b_group) + column / kv_b_group], scales of kv_b_scale_dtype
+     * (ZLLM_SCALE_*).  Only the absorb and projection stages read kv_b: with any form but bf16 those two run on the
+     * vector ALUs, f32 throughout. */
+    const void* kv_b_scales;      /* [dev] or NULL */
+    uint32_t kv_b_bits;
+    uint32_t kv_b_group;          /* columns per scale; divides latent_dim */
+    int kv_b_scale_dtype;
 } zllm_mla_decode_args;
 ZLLM_API uint64_t zllm_attn_mla_decode_workspace_bytes(const zllm_mla_decode_args* args);
 /* The record layout of a call, as zllm_attn_gqa_decode_record_layout gives it for GQA; record groups are query rows. */

@@ -33,7 +33,8 @@ def test_struct_sizes_follow_the_header():
     # pointers first, then 32-bit fields: natural alignment, no surprises for an FFI binding
     assert C.sizeof(capi.Q8AppendArgs) == 5 * 8 + 7 * 4 + 4
     assert C.sizeof(capi.GqaDecodeArgs) == 10 * 8 + 8 + 9 * 4 + 2 * 4 + 3 * 4 + 4 + 4 + 8 + 4 + 4  # + padding, gate fields
-    assert C.sizeof(capi.MlaDecodeArgs) == 9 * 8 + 8 + 9 * 4 + 3 * 4 + 4 + 4 + 2 * 8 + 4 + 4  # stage_mask, top_k, selection pointers, query_rows + padding
+    # stage_mask, top_k, selection pointers, query_rows, total_ctx_tokens; then the kv_b scales pointer, three 32-bit fields + padding
+    assert C.sizeof(capi.MlaDecodeArgs) == 9 * 8 + 8 + 9 * 4 + 3 * 4 + 4 + 4 + 2 * 8 + 4 + 4 + 8 + 3 * 4 + 4
 
 
 def test_key_range_known_answers(lib):

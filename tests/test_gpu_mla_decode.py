@@ -43,11 +43,62 @@ def make_mla_case(seed, lens, heads, nope=128, rope=64, value=128, latent=512, b
                 latent=latent, block_tokens=block_tokens)
 
 
+def weights_f32(case):
+    """kv_b as the oracle takes it: the f32 values of whatever form the device reads (bf16 unless the case says otherwise)."""
+    return case["kv_b_f32"] if "kv_b_f32" in case else O.bf16_to_f32(case["kv_b_bits"])
+
+
+def weight_args(case):
+    """(device tensor of kv_b, keyword arguments naming its form) for ops.mla_decode: bf16, or what set_weight_form left."""
+    if "kv_b_form" not in case:
+        return upload(case["kv_b_bits"]), {}
+    form = case["kv_b_form"]
+    kw = dict(kv_b_bits=form["bits"])
+    if form["bits"] in (4, 8):
+        kw.update(kv_b_scales=upload(form["scales"]), kv_b_group=form["group"], kv_b_scale_dtype=form["scale_dtype"])
+    return upload(form["data"]), kw
+
+
+def set_weight_form(case, bits, group=128, scale_dtype=O.SCALE_BF16):
+    """Re-express the case's kv_b as f32 (bits 32) or as 8- / 4-bit codes with a scale per row and `group` columns, the
+    W8A16 / W4A16 layout of paged_weight (src/kernel/rocm/hip/attention/paged_mla/source.hip:2-26): codes packed low
+    bits first into 32-bit words, value = (code - 128 | code - 8) * scale.  The oracle gets the values the codes stand for."""
+    w = O.bf16_to_f32(case["kv_b_bits"]).astype(np.float32)
+    rows, cols = w.shape
+    if bits == 32:
+        rng = np.random.default_rng(rows + cols)
+        w = (w * (1.0 + 1e-3 * rng.standard_normal(w.shape))).astype(np.float32)  # not bf16-representable any more
+        case["kv_b_form"], case["kv_b_f32"] = dict(bits=32, data=w), w
+        return case
+    top = 127 if bits == 8 else 7
+    grouped = w.reshape(rows, cols // group, group)
+    scale = np.abs(grouped).max(axis=2) / top
+    scale[scale == 0] = 1.0
+    if scale_dtype == O.SCALE_BF16:
+        stored = O.f32_to_bf16(scale.astype(np.float32))
+        scale = O.bf16_to_f32(stored)
+    elif scale_dtype == O.SCALE_F16:
+        stored = scale.astype(np.float16).view(np.uint16)
+        scale = stored.view(np.float16).astype(np.float32)
+    else:
+        stored = scale.astype(np.float32)
+        scale = stored
+    centred = np.clip(np.rint(grouped / scale[:, :, None]), -top - 1, top).astype(np.int32)
+    codes = (centred + (128 if bits == 8 else 8)).astype(np.uint32).reshape(rows, cols)
+    per_word = 32 // bits
+    words = np.zeros((rows, cols // per_word), dtype=np.uint32)
+    for i in range(per_word):
+        words |= codes[:, i::per_word] << np.uint32(i * bits)
+    case["kv_b_form"] = dict(bits=bits, data=words, scales=np.ascontiguousarray(stored), group=group, scale_dtype=scale_dtype)
+    case["kv_b_f32"] = (centred.astype(np.float32) * scale[:, :, None].astype(np.float32)).reshape(rows, cols)
+    return case
+
+
 def oracle_mla(case, head_subset=None, selection=None, counts=None):
     """`selection` [batch, top_k]: the reference's rule (paged_mla/source.hip:4761-4764) -- a sequence longer than top_k
     attends to its first count listed positions, a shorter one stays dense."""
     spec, bt = case["spec"], case["block_tokens"]
-    kv_b = O.bf16_to_f32(case["kv_b_bits"])
+    kv_b = weights_f32(case)
     outs_f, outs_b = [], []
     for b, l in enumerate(case["lens"]):
         l = int(l)
@@ -72,13 +123,14 @@ def run_mla(case, out_dtype=None, compact=True, q_f32=False, max_ctx_len=None, s
 
     out_dtype = out_dtype or torch.float32
     q = upload(O.bf16_to_f32(case["q_bits"])) if q_f32 else to_torch_bf16(case["q_bits"], "cuda")
-    out = ops.mla_decode(q, upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]), upload(case["rope"]),
+    kv_b, weight_kw = weight_args(case)
+    out = ops.mla_decode(q, kv_b, upload(case["codes"]), upload(case["scales"]), upload(case["rope"]),
                          upload(case["tables"]), upload(case["lens"]), case["heads"], case["nope"] + case["rope_dim"],
                          case["nope"] + case["value"], case["latent"], case["rope_dim"], case["block_tokens"],
                          max_ctx_len or int(case["lens"].max()), out_dtype=out_dtype, out_compact=compact,
                          selection=None if selection is None else upload(selection),
                          selection_counts=None if counts is None else upload(counts), total_ctx_tokens=total_ctx_tokens,
-                         wide_tiles=wide_tiles)
+                         wide_tiles=wide_tiles, **weight_kw)
     torch.cuda.synchronize()
     return out
 
@@ -371,7 +423,7 @@ def oracle_mla_chunk(case, selection=None):
     """The oracle's own query_rows > 1 arm (src/kernel/cpu/mla.rs:958-1076): row r of a chunk at query_start sees
     query_start + r + 1 tokens.  Returns f32 and bf16-bit outputs [batch * rows, heads * value_dim]."""
     spec, bt, rows = case["spec"], case["block_tokens"], case["rows"]
-    kv_b = O.bf16_to_f32(case["kv_b_bits"])
+    kv_b = weights_f32(case)
     outs_f, outs_b = [], []
     for b, l in enumerate(case["lens"]):
         l = int(l)
@@ -396,11 +448,13 @@ def run_mla_chunk(case, out_dtype=None, selection=None, compact=True, q_kind="bf
     if q_kind != "bf16":  # the same bf16-representable values carried as f32 or f16 (f16 holds them after a second rounding)
         q = upload(O.bf16_to_f32(case["q_bits"]))
         q = q.to(torch.float16) if q_kind == "f16" else q
-    out = ops.mla_decode(q, upload(case["kv_b_bits"]), upload(case["codes"]), upload(case["scales"]),
+    kv_b, weight_kw = weight_args(case)
+    out = ops.mla_decode(q, kv_b, upload(case["codes"]), upload(case["scales"]),
                          upload(case["rope"]), upload(case["tables"]), upload(case["lens"]), case["heads"],
                          case["nope"] + case["rope_dim"], case["nope"] + case["value"], case["latent"], case["rope_dim"],
                          case["block_tokens"], int(case["lens"].max()), out_dtype=out_dtype or torch.float32, out_compact=compact,
-                         selection=None if selection is None else upload(selection), query_rows=case["rows"], wide_tiles=wide_tiles)
+                         selection=None if selection is None else upload(selection), query_rows=case["rows"], wide_tiles=wide_tiles,
+                         **weight_kw)
     torch.cuda.synchronize()
     return out
 

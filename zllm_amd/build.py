@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzllm_attn.so")
-SOURCES = ["api.hip", "append.hip", "gqa_decode.hip", "mla_decode.hip", "mla_partial_x32.hip", "gqa_prefill.hip"]
+SOURCES = ["api.hip", "append.hip", "gqa_decode.hip", "mla_decode.hip", "mla_partial_x32.hip", "mla_generic.hip", "gqa_prefill.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",

@@ -97,7 +97,8 @@ class MlaDecodeArgs(C.Structure):
                 ("rope_dim", _u32), ("table_stride", _u32), ("max_ctx_len", _u32), ("block_tokens", _u32),
                 ("q_dtype", _int), ("out_dtype", _int), ("out_compact", _int), ("stage_mask", _u32),
                 ("top_k", _u32), ("selection", _ptr), ("selection_counts", _ptr), ("query_rows", _u32),
-                ("total_ctx_tokens", _u32)]
+                ("total_ctx_tokens", _u32), ("kv_b_scales", _ptr), ("kv_b_bits", _u32), ("kv_b_group", _u32),
+                ("kv_b_scale_dtype", _int)]
 
 
 # every symbol include/zllm_attn.h declares: name -> (restype, argtypes)

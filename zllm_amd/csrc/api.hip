@@ -311,8 +311,19 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
                         a->q_head_dim);
         }
     }
-    if (a->latent_dim != 512 || a->rope_dim != 64) {
-        return fail(-1, "MLA decode: this build handles latent_dim 512 + rope_dim 64 (got %u + %u)", a->latent_dim, a->rope_dim);
+    // latent rows are Q8g64 (a scale per 64 columns); a lane of the vector-ALU kernels owns up to 16 latent and 4 rope columns
+    if (a->latent_dim == 0 || a->latent_dim % 64u != 0 || a->latent_dim > 1024u || a->rope_dim % 2u != 0 || a->rope_dim > 256u) {
+        return fail(-1, "MLA decode: latent_dim must be a multiple of 64 up to 1024 and rope_dim even up to 256 (got %u + %u)", a->latent_dim,
+                    a->rope_dim);
+    }
+    if (a->kv_b_bits != 0u && a->kv_b_bits != 16u && a->kv_b_bits != 32u && a->kv_b_bits != 8u && a->kv_b_bits != 4u) {
+        return fail(-1, "MLA decode: kv_b_bits must be 0 / 16 (bf16), 32 (f32), 8 or 4 (got %u)", a->kv_b_bits);
+    }
+    if ((a->kv_b_bits == 8u || a->kv_b_bits == 4u) &&
+        (a->kv_b_scales == nullptr || a->kv_b_group == 0u || a->latent_dim % a->kv_b_group != 0 || a->kv_b_scale_dtype < ZLLM_SCALE_BF16 ||
+         a->kv_b_scale_dtype > ZLLM_SCALE_F32)) {
+        return fail(-1, "MLA decode: %u-bit kv_b needs scales, a group size that divides latent_dim=%u (got %u) and a scale dtype", a->kv_b_bits,
+                    a->latent_dim, a->kv_b_group);
     }
     if (a->block_tokens == 0 || a->max_ctx_len == 0) {
         return fail(-1, "MLA decode: block_tokens=%u max_ctx_len=%u must be non-zero", a->block_tokens, a->max_ctx_len);
@@ -343,7 +354,8 @@ MlaSplitPlan plan_mla_decode(const zllm_mla_decode_args* a)
 {
     MlaSplitPlan plan;
     // one workgroup per CU: the partial kernel owns a whole CU (LDS tile + 512 registers per lane)
-    const uint32_t head_blocks = (a->heads + 63) / 64; // 64 heads per workgroup
+    // 64 heads per workgroup; the vector-ALU kernel of the other latent / rope widths runs one head per workgroup
+    const uint32_t head_blocks = a->latent_dim == 512u && a->rope_dim == 64u ? (a->heads + 63) / 64 : a->heads;
     // with a selection no sequence attends to more than top_k tokens (shorter contexts stay dense)
     const uint32_t longest = a->selection != nullptr && a->top_k < a->max_ctx_len ? a->top_k : a->max_ctx_len;
     const uint64_t query_rows = mla_query_rows(a);
@@ -1030,6 +1042,10 @@ int zllm_attn_mla_decode(const zllm_mla_decode_args* a, zllm_stream_t stream)
     p.selection = a->selection;
     p.selection_counts = a->selection_counts;
     p.top_k = a->top_k;
+    p.kv_b_scales = a->kv_b_scales;
+    p.kv_b_bits = a->kv_b_bits == 0u ? 16u : a->kv_b_bits;
+    p.kv_b_group = a->kv_b_group;
+    p.kv_b_scale_dtype = a->kv_b_scale_dtype;
     return hip_status(zllm::launch_mla_decode(p, a->stage_mask, (hipStream_t)stream), "MLA decode launch");
 }
 

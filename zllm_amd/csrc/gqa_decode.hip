@@ -1302,6 +1302,9 @@ __global__ __launch_bounds__(256) void gqa_decode_merge(GqaDecodeParams p)
         const unsigned int first_al = first & ~31u;
         chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
     }
+    if (sl >= lanes) {
+        chunks = 0u; // a width whose quads do not divide the workgroup leaves its last threads without a share
+    }
     size_t base;
     unsigned int last;
     merge_rows(p, b, base, last);

@@ -168,6 +168,11 @@ struct MlaDecodeParams {
     const unsigned int* selection;        // [batch][top_k] token positions, or nullptr (dense)
     const unsigned int* selection_counts; // [batch] or nullptr
     unsigned int top_k;
+    // kv_b [heads * kv_head_dim, latent_dim] in another form than bf16 (mla_generic.hip): bits 32 = f32, 8 / 4 = codes in
+    // 32-bit words with a scale per row and `kv_b_group` columns; 16 = bf16 at `kv_b`
+    const void* kv_b_scales;
+    unsigned int kv_b_bits, kv_b_group;
+    int kv_b_scale_dtype;
     // Query rows per sequence (>= 1).  With more than one, the last query_rows tokens of a sequence are its query rows
     // (a prefill chunk, causal inside the chunk): `batch` counts query rows over all sequences, row v belongs to
     // sequence v / query_rows and sees ctx_lens[sequence] - (query_rows - 1 - v % query_rows) tokens.
@@ -196,6 +201,10 @@ hipError_t launch_gather_rows(const GatherParams& p, hipStream_t stream);
 hipError_t launch_gqa_decode(const GqaDecodeParams& p, int kv_format, int scale_dtype, unsigned int stages, hipStream_t stream);
 hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scale_dtype, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, hipStream_t stream);
+// The vector-ALU kernels for latent / rope widths other than 512 / 64 and for kv_b in other forms than bf16 (mla_generic.hip).
+hipError_t launch_mla_absorb_any(const MlaDecodeParams& p, hipStream_t stream);
+hipError_t launch_mla_partial_any(const MlaDecodeParams& p, hipStream_t stream);
+hipError_t launch_mla_project_any(const MlaDecodeParams& p, hipStream_t stream);
 // The split-KV partial on 32x32x16 matrix tiles (mla_partial_x32.hip): which calls it takes, and its launch.
 bool mla_partial_x32_takes(const MlaDecodeParams& p);
 hipError_t launch_mla_partial_x32(const MlaDecodeParams& p, hipStream_t stream);

@@ -1841,7 +1841,16 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
 {
     const unsigned int stages = (stage_mask & 15u) == 0 ? 15u : (stage_mask & 15u);
     hipError_t err = hipSuccess;
-    if (stages & 1u) {
+    // what the matrix-core kernels are built for; anything else runs the vector-ALU kernels of mla_generic.hip -- all
+    // stages for other widths, absorb and projection (the stages that read kv_b) for other weight forms
+    const bool usual_widths = p.latent_dim == (unsigned int)kLatent && p.rope_dim == 64u;
+    const bool bf16_weights = p.kv_b_bits == 16u;
+    if ((stages & 1u) && !(usual_widths && bf16_weights)) {
+        err = launch_mla_absorb_any(p, stream);
+        if (err != hipSuccess) {
+            return err;
+        }
+    } else if (stages & 1u) {
         // Eight rows per workgroup share every weight load, and the workgroup then runs eight rows' sums: measured 28 us from
         // 16 rows up to a few hundred, against 13 us (15 rows) to 27 us (32 rows) for one workgroup per row
         if (p.batch >= 16u && (p.nope_dim == 128u || p.nope_dim == 192u) && (p.q_head_dim & 3u) == 0) { // sixteen rows a workgroup, on the matrix cores
@@ -1873,7 +1882,12 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
             return err;
         }
     }
-    if (stages & 2u) {
+    if ((stages & 2u) && !usual_widths) {
+        err = launch_mla_partial_any(p, stream);
+        if (err != hipSuccess) {
+            return err;
+        }
+    } else if (stages & 2u) {
         // eight waves per workgroup measured 1.7x faster than four (261 vs 446 us on the 64K-context case)
         // densely numbered records are sized for the live splits: one workgroup per item and head block
         const dim3 grid = p.record_rows != 0u ? dim3(p.record_rows, (p.heads + 63) / 64, 1) : dim3(p.max_chunks, (p.heads + 63) / 64, p.batch);
@@ -1898,6 +1912,15 @@ hipError_t launch_mla_decode(const MlaDecodeParams& p, unsigned int stage_mask, 
         if (err != hipSuccess) {
             return err;
         }
+    }
+    if (!(usual_widths && bf16_weights)) {
+        if (stages & 4u) {
+            err = merge_into_workspace(p, stream);
+            if (err != hipSuccess) {
+                return err;
+            }
+        }
+        return (stages & 8u) ? launch_mla_project_any(p, stream) : hipSuccess;
     }
     if ((stages & 12u) == 12u) {
         // value widths up to 128 run eight waves, up to 256 sixteen (not the record-folding form, whose registers stop at 512 threads)

@@ -180,8 +180,9 @@ def gqa_prefill_chunk(*a, **kw):
 def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ctx_lens, heads, q_head_dim,
                     kv_head_dim, latent_dim, rope_dim, block_tokens, max_ctx_len, out_dtype=torch.float32,
                     out_compact=True, out=None, workspace=None, selection=None, selection_counts=None, query_rows=1,
-                    total_ctx_tokens=0, wide_tiles=False):
-    """`q` holds every query row of the call, sequence-major: [batch * query_rows, heads * q_head_dim]."""
+                    total_ctx_tokens=0, wide_tiles=False, kv_b_bits=0, kv_b_scales=None, kv_b_group=0, kv_b_scale_dtype=capi.SCALE_BF16):
+    """`q` holds every query row of the call, sequence-major: [batch * query_rows, heads * q_head_dim].
+    `kv_b` is bf16 unless kv_b_bits says f32 (32) or packed 8- / 4-bit codes with `kv_b_scales` per `kv_b_group` columns."""
     rows = q.shape[0]
     batch = rows // query_rows
     value_dim = kv_head_dim - (q_head_dim - rope_dim)
@@ -200,6 +201,7 @@ def mla_decode_args(q, kv_b, latent_codes, latent_scales, rope_cache, tables, ct
     args.query_rows = query_rows
     args.total_ctx_tokens = total_ctx_tokens
     args.stage_mask = capi.MLA_WIDE_TILES if wide_tiles else 0
+    args.kv_b_bits, args.kv_b_scales, args.kv_b_group, args.kv_b_scale_dtype = kv_b_bits, _ptr(kv_b_scales), kv_b_group, kv_b_scale_dtype
     if selection is not None:  # [batch, top_k] token positions (uint32 / int32)
         args.selection, args.top_k = _ptr(selection), selection.shape[1]
         args.selection_counts = _ptr(selection_counts)
