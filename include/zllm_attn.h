@@ -251,7 +251,7 @@ typedef struct zllm_gqa_decode_args {
     void* workspace;               /* [dev] zllm_attn_gqa_decode_workspace_bytes */
     uint64_t workspace_bytes;
     uint32_t batch;
-    uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 256} */
+    uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 192, 256}; f16 caches 128 / 256 */
     uint32_t table_stride;         /* entries per sequence in `tables` */
     uint32_t max_kv_len;           /* host upper bound of kv_lens: sizes the grid and the split plan.  A call
                                       recorded into a HIP graph stays valid only while every kv_lens[b] on the
@@ -346,7 +346,7 @@ ZLLM_API int zllm_attn_gqa_decode_static(const zllm_gqa_decode_args* args, zllm_
  * (src/backend/rocm/attention.rs:2202-2231) -- and, given that workspace, runs every
  * row as one item of the split-KV decode kernels.  So does what is
  * left -- f32 queries other than over Q8g64 with 16-bit scales at head_dim 128; more
- * than 128 query heads per KV head at head_dim 256 -- whatever the number of rows
+ * than 128 query heads per KV head at head_dim 256; head_dim 192 -- whatever the number of rows
  * (bound by cache bandwidth, not by the matrix cores); that cannot run without the
  * workspace. */
 typedef struct zllm_gqa_prefill_args {

@@ -105,7 +105,8 @@ def test_edge_lengths(lens):
             assert (got[b] == 0).all()  # nothing visible -> zeros, never NaN
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(8, 8, 128), (32, 1, 128), (40, 2, 128), (12, 3, 128), (8, 2, 64), (8, 2, 256), (64, 16, 128)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 8, 128), (32, 1, 128), (40, 2, 128), (12, 3, 128), (8, 2, 64), (8, 2, 256), (64, 16, 128),
+                                      (8, 2, 192), (12, 3, 192), (40, 1, 192), (16, 8, 192)])
 def test_head_geometries(hq, hkv, d):
     case = make_gqa_q8_case(hq * 7 + d, [600, 90], hq, hkv, d)
     got = run_decode(case, 1.0 / np.sqrt(d))
@@ -493,3 +494,36 @@ def test_f32_scale_cache(d, hq, hkv, lens, block_tokens, window):
     got = run_decode(case, scale, window=window)
     want = oracle_gqa_decode(case, scale, window=window)
     print("f32 scales", d, assert_attention_close(got, want, f"f32 scales d={d}"))
+
+
+@pytest.mark.parametrize("rule,page,window,softcap,gated", [(O.RULE_METAL_GQA, 16, 0, 0.0, False), (O.RULE_ROCM_MLA, 64, 500, 0.0, True),
+                                                            (O.RULE_CUDA_GQA, 1, 0, 30.0, False), (O.RULE_METAL_GQA, 48, 37, 50.0, True)])
+def test_head_dim_192(rule, page, window, softcap, gated):
+    """Three Q8g64 groups a head (the reference takes any head_dim up to 256, src/kernel/rocm/hip/tensor/attention.rs:1022):
+    bf16, f16 and f32 scales, pages of 1 to 64 tokens, sliding windows, the soft cap, the fused gate, an empty sequence,
+    lengths that cut into different numbers of splits, with and without the token-count hint."""
+    lens = [3000, 0, 33, 1, 700, 64, 2049]
+    case = make_gqa_q8_case(192 + page, lens, 16, 4, 192, block_tokens=page, rule=rule, outliers=True, poison=True)
+    gate = None
+    if gated:
+        gate = np.random.default_rng(5).standard_normal((len(lens), 16 * 192)).astype(np.float32)
+    scale = 1.0 / np.sqrt(192.0)
+    want = oracle_gqa_decode(case, scale, window=window, softcap=softcap)
+    if gate is not None:
+        rc, want = O.sigmoid_gate(want.reshape(len(lens), -1), gate)
+        assert rc == 0
+    got = run_decode(case, scale, window=window, softcap=softcap, gate=None if gate is None else upload(gate))
+    assert_attention_close(got, want.reshape(got.shape), f"d=192 rule={rule} page={page} window={window} cap={softcap}")
+    visible = [min(l, window) if window else l for l in lens]
+    hinted = run_decode(case, scale, window=window, softcap=softcap, gate=None if gate is None else upload(gate), total_kv_tokens=sum(visible))
+    assert_attention_close(hinted, want.reshape(got.shape), "d=192 with the token-count hint")
+    assert (got[1] == 0).all()
+
+
+def test_head_dim_192_over_f16_is_refused():
+    from zllm_amd import capi
+
+    case = make_f16_case(7, [100], 8, 2, 128)
+    case["d"] = 192
+    with pytest.raises(capi.ZllmAttnError, match="f16 KV supports head_dim 128 and 256"):
+        run_f16(case, 0.1)

@@ -271,7 +271,7 @@ def test_prefill_rejects_unsupported_shapes():
     z = torch.zeros((16, 96), dtype=torch.int8, device="cuda")
     s = torch.zeros((16, 2), dtype=torch.int16, device="cuda")
     q = torch.zeros((1, 96), dtype=torch.float32, device="cuda")
-    with pytest.raises(capi.ZllmAttnError, match="head_dim 64 / 128 / 256"):
+    with pytest.raises(capi.ZllmAttnError, match="head_dim 64 / 128 / 192 / 256"):
         ops.gqa_prefill_chunk(q, z, s, z, s, None, 0, 1, 1, 96, 16, 1.0)
     with pytest.raises(capi.ZllmAttnError, match="128 / 256 over an f16 cache"):
         ops.gqa_prefill_chunk(q, z, None, z, None, None, 0, 1, 1, 64, 16, 1.0, kv_format=capi.KV_F16)
@@ -467,3 +467,22 @@ def test_prefill_f32_scale_cache(d, q_bf16):
     queries) or through the decode kernels (f32 queries)."""
     out, want = run_case(321 + d, 400, 60, 16, 4, rule=O.RULE_CUDA_GQA, d=d, q_bf16=q_bf16, outliers=True)
     print("prefill f32 scales", d, q_bf16, assert_attention_close(out.cpu().numpy(), want, f"f32-scale prefill d={d}"))
+
+
+@pytest.mark.parametrize("prefix,chunk,hq,hkv,window,q_bf16,rule", [(700, 40, 16, 4, 0, True, O.RULE_METAL_GQA), (0, 130, 8, 2, 0, False, O.RULE_ROCM_MLA),
+                                                                   (2500, 1, 12, 3, 0, True, O.RULE_METAL_GQA), (900, 64, 8, 1, 300, True, O.RULE_CUDA_GQA)])
+def test_head_dim_192_chunks_run_as_decode_items(prefix, chunk, hq, hkv, window, q_bf16, rule):
+    """A chunk at head_dim 192 (three Q8g64 groups a head) has no matrix-core chunk kernel: its rows run as items of the
+    split-KV decode kernels, whatever their number; f32 and bf16 output, visible ends, and no workspace -> refused."""
+    from zllm_amd import capi
+
+    out, want = run_case(192 + chunk, prefix, chunk, hq, hkv, window=window, d=192, q_bf16=q_bf16, rule=rule, outliers=True)
+    print("d=192 chunk", prefix, chunk, assert_attention_close(out.cpu().numpy(), want, f"d=192 prefix={prefix} chunk={chunk} window={window}"))
+    if window == 0 and chunk > 1:
+        total = prefix + chunk
+        ends = np.minimum((np.arange(chunk) // 16 + 1) * 16 + prefix, total).astype(np.uint32)
+        out, want = run_case(192 + chunk, prefix, chunk, hq, hkv, d=192, q_bf16=q_bf16, rule=rule, visible_ends=ends, out_dtype=torch.bfloat16)
+        got = out.float().cpu().numpy()
+        assert np.abs(got - want).max() <= 2e-3 + np.abs(want).max() * 2.0 ** -8
+    with pytest.raises(capi.ZllmAttnError, match="needs a 16-byte aligned workspace"):
+        run_case(192 + chunk, prefix, chunk, hq, hkv, window=window, d=192, q_bf16=q_bf16, rule=rule, workspace=False)

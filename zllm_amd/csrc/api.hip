@@ -119,9 +119,10 @@ uint64_t align_up(uint64_t value, uint64_t to)
     return (value + to - 1) / to * to;
 }
 
+// head dimensions that Q8g64 groups divide, up to the reference's limit of 256 (tensor/attention.rs:1022)
 bool valid_head_dim(uint32_t d)
 {
-    return d == 64 || d == 128 || d == 256;
+    return d == 64 || d == 128 || d == 192 || d == 256;
 }
 
 // Tokens per KV split.  `units` (sequence, head-block) pairs each cut their keys into the same number of splits, one
@@ -186,7 +187,7 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
     if (a->kv_format == ZLLM_KV_Q8G64 && (a->scale_dtype < ZLLM_SCALE_BF16 || a->scale_dtype > ZLLM_SCALE_F32)) {
         return fail(-1, "GQA decode: Q8g64 scales must be bf16, f16 or f32 (got %d)", a->scale_dtype);
     }
-    if (a->kv_format == ZLLM_KV_F16 && a->head_dim == 64) {
+    if (a->kv_format == ZLLM_KV_F16 && a->head_dim != 128 && a->head_dim != 256) {
         return fail(-1, "GQA decode: f16 KV supports head_dim 128 and 256");
     }
     if (a->q_dtype < ZLLM_DTYPE_F32 || a->q_dtype > ZLLM_DTYPE_F16) {
@@ -1062,8 +1063,8 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
     }
     // head dimensions of the reference's block attention that a Q8g64 group divides (tensor/attention.rs:727-745)
     if (!valid_head_dim(a->head_dim) || (a->kv_format != ZLLM_KV_Q8G64 && a->kv_format != ZLLM_KV_F16) ||
-        (a->kv_format == ZLLM_KV_F16 && a->head_dim == 64)) {
-        return fail(-1, "GQA prefill: head_dim 64 / 128 / 256 over a Q8g64 cache or 128 / 256 over an f16 cache (got dim=%u format=%d)",
+        (a->kv_format == ZLLM_KV_F16 && a->head_dim != 128 && a->head_dim != 256)) {
+        return fail(-1, "GQA prefill: head_dim 64 / 128 / 192 / 256 over a Q8g64 cache or 128 / 256 over an f16 cache (got dim=%u format=%d)",
                     a->head_dim, a->kv_format);
     }
     if (a->num_heads / a->num_kv_heads > 256) {
@@ -1149,6 +1150,9 @@ static bool prefill_rows_as_decode_items(const zllm_gqa_prefill_args* a)
     const bool q8 = a->kv_format == ZLLM_KV_Q8G64;
     if (a->q_dtype == ZLLM_DTYPE_F32 && !(q8 && a->head_dim == 128 && a->scale_dtype != ZLLM_SCALE_F32)) {
         return true;
+    }
+    if (a->head_dim == 192) {
+        return true; // no chunk kernel is built for three scale groups a head
     }
     return a->head_dim == 256 && a->num_heads / a->num_kv_heads > 128u;
 }

@@ -78,6 +78,10 @@ template <> struct ScaleRow<2> {
     unsigned int v;
     __device__ __forceinline__ unsigned short get(int a) const { return (unsigned short)(a == 0 ? (v & 0xffffu) : (v >> 16)); }
 };
+template <> struct ScaleRow<3> { // head_dim 192: three 16-bit words, two-byte aligned
+    unsigned short v[3];
+    __device__ __forceinline__ unsigned short get(int a) const { return v[a]; }
+};
 template <> struct ScaleRow<4> {
     u32x2 v;
     __device__ __forceinline__ unsigned short get(int a) const
@@ -1644,13 +1648,17 @@ hipError_t launch_q8(const GqaDecodeParams& p, bool fast, dim3 grid, dim3 block,
             return hipGetLastError();
         }
     }
-    if (fast) {
-        if (cap) {
-            gqa_decode_q8_partial<D, SDT, true, true, 2><<<grid, block, 0, stream>>>(p);
-        } else {
-            gqa_decode_q8_partial<D, SDT, true, false, 2><<<grid, block, 0, stream>>>(p);
+    if constexpr (D != 192) { // three scale words a row do not travel as one register: head_dim 192 loads them per token
+        if (fast) {
+            if (cap) {
+                gqa_decode_q8_partial<D, SDT, true, true, 2><<<grid, block, 0, stream>>>(p);
+            } else {
+                gqa_decode_q8_partial<D, SDT, true, false, 2><<<grid, block, 0, stream>>>(p);
+            }
+            return hipGetLastError();
         }
-    } else {
+    }
+    {
         if (cap) {
             gqa_decode_q8_partial<D, SDT, false, true, 2><<<grid, block, 0, stream>>>(p);
         } else {
@@ -1717,6 +1725,7 @@ hipError_t launch_gqa_decode(const GqaDecodeParams& args, int kv_format, int sca
         switch (p.head_dim) {
         case 64: err = launch_q8_d<64>(p, scale_dtype, fast, grid, block, stream); break;
         case 128: err = launch_q8_d<128>(p, scale_dtype, fast, grid, block, stream); break;
+        case 192: err = launch_q8_d<192>(p, scale_dtype, fast, grid, block, stream); break;
         case 256: err = launch_q8_d<256>(p, scale_dtype, fast, grid, block, stream); break;
         default: return hipErrorInvalidValue;
         }
