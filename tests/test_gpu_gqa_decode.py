@@ -210,6 +210,64 @@ def test_large_pool_exercises_64_bit_offsets():
     assert_attention_close(out, want, "far pool")
 
 
+def test_pages_spread_over_64_gib_give_the_compact_pool_bits():
+    """Config 2's geometry with every sequence's pages drawn from all over a 64 GiB code plane (the span the benchmark's
+    pool has per plane and more than a serving pool hands one sequence), beside the same rows in a compact pool: where a
+    page lies changes no bit of the output, and both meet the oracle."""
+    from zllm_amd import capi, ops
+
+    hq, hkv, d, bt = 64, 8, 128, 16
+    cols = hkv * d
+    lens = [8192, 3000, 8192, 1025]
+    rng = np.random.default_rng(64)
+    blocks = [(l + bt - 1) // bt for l in lens]
+    stride = max(blocks)
+    far_blocks = (64 << 30) // (cols * bt)
+    far_ids = rng.choice(far_blocks, size=sum(blocks), replace=False).astype(np.uint32)
+    far_ids[0], far_ids[-1] = far_blocks - 1, 0  # both ends of the plane are in use
+    near_ids = rng.permutation(sum(blocks)).astype(np.uint32)
+    q_bits = O.f32_to_bf16(rng.standard_normal((len(lens), hq * d)).astype(np.float32))
+    rows = [(rng.standard_normal((l, cols)).astype(np.float32), rng.standard_normal((l, cols)).astype(np.float32)) for l in lens]
+    torch.cuda.empty_cache()
+    outs = {}
+    for name, ids, pool_blocks in (("near", near_ids, sum(blocks)), ("far", far_ids, far_blocks)):
+        tables = np.zeros((len(lens), stride), dtype=np.uint32)
+        at = 0
+        for b, n in enumerate(blocks):
+            tables[b, :n] = ids[at:at + n]
+            at += n
+        kc = torch.empty((pool_blocks * bt, cols), dtype=torch.int8, device="cuda")
+        vc = torch.empty((pool_blocks * bt, cols), dtype=torch.int8, device="cuda")
+        ks = torch.empty((pool_blocks * bt, cols // 64), dtype=torch.int16, device="cuda")
+        vs = torch.empty((pool_blocks * bt, cols // 64), dtype=torch.int16, device="cuda")
+        tbl = upload(tables)
+        for b, (k, v) in enumerate(rows):
+            ops.q8g64_append(upload(k), kc, ks, tbl[b], 0, bt, capi.QUANT_METAL_GQA)
+            ops.q8g64_append(upload(v), vc, vs, tbl[b], 0, bt, capi.QUANT_METAL_GQA)
+        out = ops.gqa_decode(to_torch_bf16(q_bits, "cuda"), kc, ks, vc, vs, tbl, upload(np.array(lens, dtype=np.uint32)), hq, hkv, d, bt,
+                             0.088, max(lens))
+        torch.cuda.synchronize()
+        outs[name] = out.cpu().numpy()
+        if name == "far":
+            assert int(tables.max()) * bt * cols >= (64 << 30) - bt * cols
+        del kc, vc, ks, vs
+        torch.cuda.empty_cache()
+    assert np.array_equal(outs["near"], outs["far"])
+    q = O.bf16_to_f32(q_bits)
+    for b, (k, v) in enumerate(rows):
+        l = lens[b]
+        codes = np.zeros((blocks[b] * bt, cols), dtype=np.int8)
+        kscale = np.zeros((blocks[b] * bt, cols // 64), dtype=np.uint16)
+        vcodes, vscale = codes.copy(), kscale.copy()
+        O.q8g64_append_paged(O.RULE_METAL_GQA, k, codes, kscale, None, 0, bt)
+        O.q8g64_append_paged(O.RULE_METAL_GQA, v, vcodes, vscale, None, 0, bt)
+        kd = O.gather_dequant_rows(O.FMT_Q8, codes, kscale, O.SCALE_F16, None, bt, 0, l, cols)
+        vd = O.gather_dequant_rows(O.FMT_Q8, vcodes, vscale, O.SCALE_F16, None, bt, 0, l, cols)
+        rc, want = O.gqa_prefill_at_visible(q[b:b + 1], kd, vd, 0, l, l - 1, hq, hkv, d, score_scale=0.088)
+        assert rc == 0
+        assert_attention_close(outs["far"][b:b + 1], want, f"pages over 64 GiB, sequence {b}")
+
+
 # ---------------------------------------------------------------------------- f16 KV (config 3)
 def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0, poison=False):
     rng = np.random.default_rng(seed)
