@@ -824,6 +824,84 @@ static void test_steady_state_counters(const RocmContext& ctx)
     CHECK(ctx.synchronize().is_ok(), "synchronize");
 }
 
+// MLA at another latent / rope width with kv_b as W8A16 and W4A16 codes (RocmQuantizedWeight, src/backend/rocm/attention.rs:181-192):
+// the oracle gets the f32 values the codes stand for
+static void test_mla_other_widths_and_quantized_weights(const RocmContext& ctx)
+{
+    std::mt19937 rng(53);
+    struct Case {
+        size_t latent, rope, nope, value, heads, rows;
+        unsigned bits;
+        size_t group;
+    };
+    const Case cases[] = {{128, 32, 64, 64, 6, 300, 8, 64}, {512, 64, 128, 128, 16, 700, 8, 128}, {512, 64, 128, 128, 8, 200, 4, 32}, {256, 128, 32, 96, 3, 90, 16, 0}};
+    for (const Case& c : cases) {
+        MlaSpec spec;
+        spec.kv_lora_rank = c.latent;
+        spec.qk_rope_head_dim = c.rope;
+        spec.num_heads = c.heads;
+        spec.q_projection_size = c.heads * (c.nope + c.rope);
+        spec.kv_projection_size = c.heads * (c.nope + c.value);
+        spec.q_lora_rank = 64;
+        CHECK(!spec.validate().has_value(), "spec must validate");
+        auto cache_r = RocmKvCache::new_mla(1, c.latent, c.rope, 16, 1024, TablePolicy::Scrambled);
+        CHECK(cache_r.is_ok(), "cache: %s", cache_r.is_err() ? cache_r.unwrap_err().to_string().c_str() : "");
+        if (cache_r.is_err()) {
+            return;
+        }
+        RocmKvCache cache = cache_r.unwrap();
+        const auto latent = randn(rng, c.rows * c.latent, false);
+        const auto rope = randn(rng, c.rows * c.rope, false);
+        auto appended = ctx.append_mla(cache, 0, ctx.tensor_from_f32(latent, c.rows, c.latent).unwrap(), ctx.tensor_from_f32(rope, c.rows, c.rope).unwrap());
+        CHECK(appended.is_ok(), "append_mla: %s", appended.is_err() ? appended.unwrap_err().to_string().c_str() : "");
+        std::vector<float> kv_b = randn(rng, spec.kv_projection_size * c.latent, true);
+        for (auto& w : kv_b) {
+            w = zo_bf16_to_f32(zo_f32_to_bf16(w * 0.05f));
+        }
+        auto weight = c.bits == 16 ? ctx.prepare_mla_kv_b(kv_b, spec.kv_projection_size, c.latent)
+                                   : ctx.prepare_mla_kv_b_quantized(kv_b, spec.kv_projection_size, c.latent, c.bits, c.group);
+        CHECK(weight.is_ok(), "weight: %s", weight.is_err() ? weight.unwrap_err().to_string().c_str() : "");
+        if (weight.is_err()) {
+            return;
+        }
+        std::vector<float> seen = kv_b;
+        if (c.bits != 16) {
+            auto values = ctx.dequantized_kv_b(weight.unwrap());
+            CHECK(values.is_ok(), "dequantized_kv_b");
+            seen = values.unwrap();
+            double worst = 0;
+            for (size_t i = 0; i < seen.size(); ++i) {
+                worst = fmax(worst, fabs((double)seen[i] - kv_b[i]));
+            }
+            CHECK(worst < (c.bits == 8 ? 2e-3 : 3e-2), "the codes are %.3e from the weights", worst);
+        }
+        const auto q = randn(rng, spec.q_projection_size, true);
+        auto out = ctx.mla_decode_attention(ctx.tensor_from_f32(q, 1, spec.q_projection_size, DType::BF16).unwrap(), cache, weight.unwrap(), 0,
+                                            c.rows - 1, spec);
+        CHECK(out.is_ok(), "mla_decode_attention: %s", out.is_err() ? out.unwrap_err().to_string().c_str() : "");
+        if (out.is_err()) {
+            return;
+        }
+        std::vector<int8_t> codes(c.rows * c.latent);
+        std::vector<uint16_t> scales(c.rows * c.latent / 64), rope_bits(c.rows * c.rope), q_bits(q.size());
+        zo_q8g64_append_paged(0, latent.data(), codes.data(), scales.data(), nullptr, 0, c.rows, c.latent, 64, 16, 0);
+        zo_half_append_paged(0, rope.data(), rope_bits.data(), nullptr, 0, c.rows, c.rope, 16, 0);
+        for (size_t i = 0; i < q.size(); ++i) {
+            q_bits[i] = zo_f32_to_bf16(q[i]);
+        }
+        zo_mla_spec zs = {c.latent, c.rope, spec.q_projection_size, spec.kv_projection_size, c.heads};
+        std::vector<float> want(c.heads * c.value);
+        const int rc = zo_mla_absorbed_q8_history(&zs, q_bits.data(), 1, c.rows - 1, (const uint8_t*)codes.data(), scales.data(), 64, rope_bits.data(),
+                                                  c.rows, seen.data(), nullptr, 0, nullptr, want.data(), nullptr);
+        CHECK(rc == 0, "oracle rc %d", rc);
+        char what[128];
+        snprintf(what, sizeof(what), "mla_decode_attention latent=%zu rope=%zu kv_b %u-bit", c.latent, c.rope, c.bits);
+        compare(ctx.tensor_to_f32(out.unwrap()).unwrap(), want, what);
+    }
+    CHECK(ctx.prepare_mla_kv_b_quantized(std::vector<float>(64 * 128), 64, 128, 8, 48).is_err(), "a group that does not divide the columns must be refused");
+    CHECK(ctx.prepare_mla_kv_b_quantized(std::vector<float>(64 * 128), 64, 128, 5, 64).is_err(), "five-bit codes must be refused");
+}
+
 int main()
 {
     auto ctx = RocmContext::create(0);
@@ -846,6 +924,7 @@ int main()
     test_mla_prefill(ctx.unwrap());
     test_gqa_uncached(ctx.unwrap());
     test_block_attention(ctx.unwrap());
+    test_mla_other_widths_and_quantized_weights(ctx.unwrap());
     test_steady_state_counters(ctx.unwrap());
     printf(failures == 0 ? "ALL PASSED\n" : "%d FAILED\n", failures);
     return failures == 0 ? 0 : 1;

@@ -749,6 +749,81 @@ Result<RocmWeight> RocmContext::prepare_mla_kv_b(const std::vector<float>& weigh
     return w;
 }
 
+Result<RocmWeight> RocmContext::prepare_mla_kv_b_quantized(const std::vector<float>& weight, size_t rows, size_t cols, unsigned bits,
+                                                           size_t group_size) const
+{
+    if ((bits != 8 && bits != 4) || group_size == 0 || cols % group_size != 0 || weight.size() != rows * cols || cols % (32 / bits) != 0) {
+        return compute_error("prepare_mla_kv_b_quantized: bits=" + std::to_string(bits) + " group=" + std::to_string(group_size) + " for [" +
+                             std::to_string(rows) + "," + std::to_string(cols) + "]");
+    }
+    const int top = bits == 8 ? 127 : 7, offset = bits == 8 ? 128 : 8;
+    const size_t per_word = 32 / bits, words_per_row = cols / per_word, groups = cols / group_size;
+    std::vector<uint32_t> words(rows * words_per_row, 0u);
+    std::vector<uint16_t> scale_bits(rows * groups);
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t g = 0; g < groups; ++g) {
+            float largest = 0.0f;
+            for (size_t c = g * group_size; c < (g + 1) * group_size; ++c) {
+                largest = std::max(largest, fabsf(weight[r * cols + c]));
+            }
+            const uint16_t stored = f32_to_bf16_bits(largest > 0.0f ? largest / (float)top : 1.0f);
+            const float scale = bf16_bits_to_f32(stored);
+            scale_bits[r * groups + g] = stored;
+            for (size_t c = g * group_size; c < (g + 1) * group_size; ++c) {
+                const int code = std::max(-top - 1, std::min(top, (int)lrintf(weight[r * cols + c] / scale))) + offset;
+                words[r * words_per_row + c / per_word] |= (uint32_t)code << ((c % per_word) * bits);
+            }
+        }
+    }
+    RocmWeight w;
+    w.rows = rows;
+    w.cols = cols;
+    w.bits = bits;
+    w.group_size = group_size;
+    w.scale_dtype = DType::BF16;
+    auto codes = DeviceBuffer::allocate(words.size() * 4);
+    auto scales = DeviceBuffer::allocate(scale_bits.size() * 2);
+    if (codes.is_err() || scales.is_err()) {
+        return codes.is_err() ? codes.unwrap_err() : scales.unwrap_err();
+    }
+    hipError_t err = hipMemcpy(codes.unwrap().data(), words.data(), words.size() * 4, hipMemcpyHostToDevice);
+    if (err == hipSuccess) {
+        err = hipMemcpy(scales.unwrap().data(), scale_bits.data(), scale_bits.size() * 2, hipMemcpyHostToDevice);
+    }
+    if (err != hipSuccess) {
+        return hip_error("weight upload", err);
+    }
+    w.device = codes.unwrap();
+    w.scales = scales.unwrap();
+    return w;
+}
+
+Result<std::vector<float>> RocmContext::dequantized_kv_b(const RocmWeight& weight) const
+{
+    if (weight.bits != 8 && weight.bits != 4) {
+        return compute_error("dequantized_kv_b: the weight holds no codes");
+    }
+    const size_t per_word = 32 / weight.bits, words_per_row = weight.cols / per_word, groups = weight.cols / weight.group_size;
+    std::vector<uint32_t> words(weight.rows * words_per_row);
+    std::vector<uint16_t> scale_bits(weight.rows * groups);
+    hipError_t err = hipMemcpy(words.data(), weight.device.data(), words.size() * 4, hipMemcpyDeviceToHost);
+    if (err == hipSuccess) {
+        err = hipMemcpy(scale_bits.data(), weight.scales.data(), scale_bits.size() * 2, hipMemcpyDeviceToHost);
+    }
+    if (err != hipSuccess) {
+        return hip_error("weight download", err);
+    }
+    const int offset = weight.bits == 8 ? 128 : 8;
+    std::vector<float> out(weight.rows * weight.cols);
+    for (size_t r = 0; r < weight.rows; ++r) {
+        for (size_t c = 0; c < weight.cols; ++c) {
+            const uint32_t code = (words[r * words_per_row + c / per_word] >> ((c % per_word) * weight.bits)) & ((1u << weight.bits) - 1u);
+            out[r * weight.cols + c] = (float)((int)code - offset) * bf16_bits_to_f32(scale_bits[r * groups + c / weight.group_size]);
+        }
+    }
+    return out;
+}
+
 namespace {
 
 // HybridGqaCacheLayout::write_plan (src/kv_cache/mod.rs:440-455) for a layer that keeps `capacity` rows
@@ -1503,6 +1578,12 @@ Result<RocmTensor> RocmContext::mla_decode_impl(const RocmTensor& query, const R
     if (state != nullptr) {
         a.selection = (const uint32_t*)state->selection.data();
         a.top_k = (uint32_t)state->top_k;
+    }
+    if (kv_b.bits != 16) {
+        a.kv_b_bits = kv_b.bits;
+        a.kv_b_scales = kv_b.scales.data();
+        a.kv_b_group = (uint32_t)kv_b.group_size;
+        a.kv_b_scale_dtype = kv_b.scale_dtype == DType::F32 ? ZLLM_SCALE_F32 : (kv_b.scale_dtype == DType::F16 ? ZLLM_SCALE_F16 : ZLLM_SCALE_BF16);
     }
     const uint64_t need = zllm_attn_mla_decode_workspace_bytes(&a);
     if (need == 0) {

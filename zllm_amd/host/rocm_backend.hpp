@@ -132,10 +132,16 @@ struct RocmTensor {
     DType dtype = DType::F32;
 };
 
-// bf16 weight matrix resident on the device (the reference's RocmWeight for kv_b).
+// kv_b resident on the device (the reference's RocmWeight): bf16, or the W8A16 / W4A16 form of RocmQuantizedWeight
+// (src/backend/rocm/attention.rs:181-192) -- codes packed low bits first into 32-bit words, a scale per row and
+// `group_size` columns.
 struct RocmWeight {
     DeviceBuffer device;
     size_t rows = 0, cols = 0;
+    unsigned bits = 16;       // 16 bf16, 32 f32, 8 / 4 codes
+    DeviceBuffer scales;      // 8 / 4 bits only
+    size_t group_size = 0;
+    DType scale_dtype = DType::BF16;
 };
 
 // What the reference's DsaState hands to the selected-token decode: the token positions the indexer chose for the
@@ -243,6 +249,12 @@ class RocmContext {
     Result<std::vector<float>> tensor_to_f32(const RocmTensor& tensor) const;
     // DecodeBackend::prepare_mla_kv_b: kv_b [heads * kv_head_dim, latent] -> bf16 on the device
     Result<RocmWeight> prepare_mla_kv_b(const std::vector<float>& weight, size_t rows, size_t cols) const;
+    // The same weight quantized on the way in: 8- or 4-bit codes with one bf16 scale per row and `group_size` columns
+    // (scale = largest magnitude of the group / 127 or / 7, rounded to bf16; code = round(value / scale) + 128 or + 8).
+    Result<RocmWeight> prepare_mla_kv_b_quantized(const std::vector<float>& weight, size_t rows, size_t cols, unsigned bits,
+                                                  size_t group_size) const;
+    // What a quantized weight's codes stand for, as f32 [rows, cols] (for callers that check against a CPU reference).
+    Result<std::vector<float>> dequantized_kv_b(const RocmWeight& weight) const;
 
     // Backend::gqa_prefill_attention (src/backend/mod.rs:1477; ROCm body src/backend/rocm/attention.rs:2151-2170): causal
     // attention of a chunk over its own K/V, nothing cached.  K and V go to dense f16 scratch planes on the way in.
