@@ -163,3 +163,65 @@ def test_random_mla_chunk(it):
     if heads > 32 and bt % 32 == 0:
         wide = run_mla_chunk(case, q_kind=q_kind, wide_tiles=True).cpu().numpy()
         assert_attention_close(wide.reshape(want.shape), want, what + " (wide tiles)")
+
+
+@pytest.mark.parametrize("it", range(16))
+def test_random_q8_head_dim_192(it):
+    """Decode steps and prefill chunks at head_dim 192 (three Q8g64 groups a head): every scale rule, pages of 1 to 64 tokens,
+    windows, soft caps, the token-count hint on every other case."""
+    rng = np.random.default_rng([505, it])
+    hkv = pick(rng, [1, 2, 3, 4, 8])
+    group = pick(rng, [1, 2, 3, 4, 8, 16])
+    rule = pick(rng, [O.RULE_METAL_GQA, O.RULE_ROCM_MLA, O.RULE_CUDA_GQA])
+    page = pick(rng, PAGE_SIZES)
+    window = pick(rng, [0, 0, 1, 33, 1024])
+    softcap = pick(rng, [0.0, 0.0, 30.0])
+    if it % 2 == 0:
+        lens = [pick(rng, LENGTHS) for _ in range(int(rng.integers(1, 6)))]
+        if max(lens) == 0:
+            lens[0] = 5
+        what = f"decode d=192 {it}: {hkv * group}/{hkv} rule={rule} page={page} lens={lens} window={window} softcap={softcap}"
+        print(what, flush=True)
+        case = make_gqa_q8_case(5000 + it, lens, hkv * group, hkv, 192, block_tokens=page, rule=rule, outliers=bool(it % 4), poison=True)
+        visible = [min(l, window) if window else l for l in lens]
+        got = run_decode(case, 0.07, window=window, softcap=softcap, total_kv_tokens=sum(visible) if it % 4 == 0 else 0)
+        assert_attention_close(got, oracle_gqa_decode(case, 0.07, window=window, softcap=softcap), what)
+    else:
+        prefix, chunk = pick(rng, [0, 1, 100, 777, 2100]), pick(rng, [1, 2, 17, 64, 100])
+        what = f"prefill d=192 {it}: {hkv * group}/{hkv} rule={rule} page={page} prefix={prefix} chunk={chunk} window={window} softcap={softcap}"
+        print(what, flush=True)
+        out, want = run_case(5000 + it, prefix, chunk, hkv * group, hkv, window=window, softcap=softcap, block_tokens=page, rule=rule,
+                             q_bf16=bool(it % 3), d=192, outliers=True)
+        assert_attention_close(out.cpu().numpy(), want, what)
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_random_mla_other_widths_and_weight_forms(it):
+    """MLA decode steps and chunks at latent widths of one to sixteen Q8g64 groups, rope widths of 2 to 256, and kv_b as bf16,
+    f32, W8A16 or W4A16 (at 512 + 64 too, where only absorb and projection change kernels)."""
+    from tests.test_gpu_mla_decode import set_weight_form
+
+    rng = np.random.default_rng([606, it])
+    usual = it % 4 == 3
+    latent = 512 if usual else pick(rng, [64, 128, 192, 256, 320, 448, 576, 1024])
+    rope = 64 if usual else pick(rng, [2, 16, 32, 64, 96, 128, 256])
+    nope, value = pick(rng, [16, 32, 64, 128, 192]), pick(rng, [16, 64, 128, 160])
+    heads = pick(rng, [1, 2, 3, 8, 20, 33])
+    page = pick(rng, [1, 16, 32, 48, 64])
+    form = pick(rng, ["bf16", "f32", "w8", "w8", "w4"]) if not usual else pick(rng, ["f32", "w8", "w4"])
+    rows = pick(rng, [1, 1, 1, 3, 9])
+    lens = [max(rows, pick(rng, MLA_LENGTHS[:18])) for _ in range(int(rng.integers(1, 4)))]
+    what = f"mla other {it}: latent={latent} rope={rope} nope={nope} value={value} heads={heads} page={page} kv_b={form} rows={rows} lens={lens}"
+    print(what, flush=True)
+    kw = dict(nope=nope, rope=rope, value=value, latent=latent, block_tokens=page)
+    case = make_mla_case(6000 + it, lens, heads, poison=bool(it % 2), **kw) if rows == 1 else make_mla_chunk_case(6000 + it, lens, rows, heads, **kw)
+    if form != "bf16":
+        group = pick(rng, [g for g in (32, 64, 128, latent) if latent % g == 0])
+        set_weight_form(case, {"f32": 32, "w8": 8, "w4": 4}[form], group=group, scale_dtype=pick(rng, [O.SCALE_BF16, O.SCALE_F16, O.SCALE_F32]))
+    if rows == 1:
+        want, _ = oracle_mla(case)
+        got = run_mla(case, total_ctx_tokens=int(sum(lens)) if it % 3 == 0 else 0).cpu().numpy()
+        assert_attention_close(got.reshape(want.shape), want, what)
+    else:
+        want, _ = oracle_mla_chunk(case)
+        assert_attention_close(run_mla_chunk(case).cpu().numpy(), want, what)

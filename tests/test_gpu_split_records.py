@@ -126,3 +126,29 @@ def test_mla_one_long_sequence_among_short_ones(heads, wide_tiles, page):
     layout = capi.SplitRecordLayout()
     assert capi.load().zllm_attn_mla_decode_record_layout(C.byref(args), C.byref(layout)) == 0
     assert layout.dense == 1 and layout.record_rows * 2 < len(lens) * layout.max_chunks
+
+
+def test_a_hint_below_the_real_sum_drops_splits_but_stays_in_bounds():
+    """`total_kv_tokens` sizes the record rows of a ragged plan.  Given a sum below the real one, the splits past the rows it
+    sized find nothing to do and write nothing: the sequences whose splits all fit are still right, and the same buffers
+    serve a correct call afterwards."""
+    from zllm_amd import capi
+
+    lens = [3000, 2000, 4000, 100]
+    case = make_gqa_q8_case(17, lens, 16, 4, 128)
+    want = oracle_gqa_decode(case, 0.09)
+    args, out, ws, keep = decode_call(case, 0.09, 3000)
+    layout = capi.SplitRecordLayout()
+    assert capi.load().zllm_attn_gqa_decode_record_layout(C.byref(args), C.byref(layout)) == 0
+    splits = [-(-l // layout.chunk_tokens) for l in lens]
+    assert layout.dense == 1 and splits[0] <= layout.record_rows < sum(splits)  # the first sequence fits, the batch does not
+    guard = torch.full((1 << 20,), 0x5A, dtype=torch.uint8, device="cuda")  # whatever follows the workspace stays untouched
+    ws.zero_()
+    capi.check(capi.load().zllm_attn_gqa_decode(C.byref(args), None))
+    torch.cuda.synchronize()
+    assert_attention_close(out[:1].cpu().numpy(), want[:1], "the sequence whose splits fit")
+    assert bool((guard == 0x5A).all())
+    args, out, ws, keep = decode_call(case, 0.09, sum(lens))
+    capi.check(capi.load().zllm_attn_gqa_decode(C.byref(args), None))
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), want, "the same call with an honest hint")
