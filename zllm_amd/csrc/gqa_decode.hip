@@ -1527,6 +1527,94 @@ __global__ __launch_bounds__(256) void gqa_decode_merge_wide(GqaDecodeParams p)
     }
 }
 
+// The combine for plans of nine to thirty-two splits at head_dim 128 -- a batch of long sequences cut into one round of
+// workgroups, config 2's own plan: one wave per (head, sequence), a lane owns four output dimensions and every other
+// split, all sixteen record loads of the lane issued before the first is used, the two halves of the wave combined with
+// one lane exchange.  No LDS and no barrier: the kernel is one memory round trip, the exchange and the store.
+__global__ __launch_bounds__(256) void gqa_decode_merge_wave(GqaDecodeParams p)
+{
+    const unsigned int lane = threadIdx.x & 63u;
+    const unsigned int quad = lane & 31u;
+    const unsigned int sl = lane >> 5;
+    const unsigned int head = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const unsigned int b = blockIdx.y;
+    if (head >= p.num_heads) {
+        return;
+    }
+    size_t base;
+    unsigned int last;
+    merge_rows(p, b, base, last);
+    const float* stats = p.stats + (base * p.num_heads + head) * 2;
+    const size_t stat_stride = (size_t)p.num_heads * 2;
+    const float* partial = p.partial + (base * p.num_heads + head) * 128u + quad * 4u;
+    const size_t partial_stride = (size_t)p.num_heads * 128u;
+    // addresses are clamped to the planned splits, so that the loads do not wait for the length
+    float2 st[16];
+    f32x4 part[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const unsigned int c = min(sl + 2u * u, last);
+        st[u] = *(const float2*)(stats + c * stat_stride);
+        part[u] = *(const f32x4*)(partial + c * partial_stride);
+    }
+    unsigned int chunks = p.fixed_chunks;
+    if (chunks == 0u) {
+        unsigned int len = p.kv_lens[b];
+        if (p.query_rows > 1u) {
+            const unsigned int behind = p.query_rows - 1u - b % p.query_rows;
+            len = p.kv_lens[b / p.query_rows];
+            len = len > behind ? len - behind : 0u;
+        }
+        unsigned int first = p.first_visible != nullptr ? p.first_visible[b] : 0u;
+        first = min(first, len);
+        const unsigned int first_al = first & ~31u;
+        chunks = min(p.max_chunks, (len - first_al + p.chunk_tokens - 1u) / p.chunk_tokens);
+    }
+    float m = kNegInf, l = 0.0f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const float cl = sl + 2u * u < chunks ? st[u].y : 0.0f;
+        if (cl > 0.0f) {
+            const float nm = fmaxf(m, st[u].x);
+            const float a = __builtin_amdgcn_exp2f(m - nm); // m = -inf -> 0
+            const float w = __builtin_amdgcn_exp2f(st[u].x - nm);
+            acc = acc * a + part[u] * w;
+            l = l * a + cl * w;
+            m = nm;
+        }
+    }
+    // the other half of the wave holds the other splits of the same four dimensions
+    const float om = __shfl_xor(m, 32), ol = __shfl_xor(l, 32);
+    const f32x4 oacc = {__shfl_xor(acc[0], 32), __shfl_xor(acc[1], 32), __shfl_xor(acc[2], 32), __shfl_xor(acc[3], 32)};
+    if (sl != 0u) {
+        return;
+    }
+    const float gm = fmaxf(l > 0.0f ? m : kNegInf, ol > 0.0f ? om : kNegInf);
+    const float wa = l > 0.0f ? __builtin_amdgcn_exp2f(m - gm) : 0.0f;
+    const float wb = ol > 0.0f ? __builtin_amdgcn_exp2f(om - gm) : 0.0f;
+    const float denom = l * wa + ol * wb;
+    f32x4 result = {0.f, 0.f, 0.f, 0.f};
+    if (denom > 0.0f && denom < __builtin_inff()) {
+        result = (acc * wa + oacc * wb) * (1.0f / denom);
+    }
+    if (p.gate != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            result[e] = gated(result[e], p.gate, p.gate_cols, p.gate_dtype, b, head * 128u + quad * 4u + e);
+        }
+    }
+    const size_t at = ((size_t)b * p.num_heads + head) * 128u + quad * 4u;
+    if (p.out_dtype == 0) {
+        *(f32x4*)(p.out + at) = result;
+    } else if (p.out_dtype == 1) {
+        *(u32x2*)((unsigned short*)p.out + at) = u32x2{pack_bf16_rne(result[0], result[1]), pack_bf16_rne(result[2], result[3])};
+    } else {
+        *(u32x2*)((unsigned short*)p.out + at) = u32x2{(unsigned int)f32_to_f16_bits(result[0]) | ((unsigned int)f32_to_f16_bits(result[1]) << 16),
+                                                        (unsigned int)f32_to_f16_bits(result[2]) | ((unsigned int)f32_to_f16_bits(result[3]) << 16)};
+    }
+}
+
 // The same combine for plans of at most eight splits (large batches, short contexts): a thread owns four output
 // dimensions of one (head, sequence) and folds the few records itself, 256 / (head_dim / 4) heads a workgroup.  One
 // workgroup of 256 threads per (head, sequence) is mostly idle lanes there, and with hundreds of sequences the launch
@@ -1770,6 +1858,8 @@ hipError_t launch_split_merge(const GqaDecodeParams& p, hipStream_t stream)
                                           (p.max_chunks > 4u * (256u / quads) && p.num_heads * p.batch <= 256u))) {
         // more splits than one workgroup per (row, head) reads in a round trip, and few such pairs
         gqa_decode_merge_wide<<<dim3(p.num_heads, p.batch, p.head_dim / 32u), dim3(256), 0, stream>>>(p);
+    } else if (p.head_dim == 128u && p.max_chunks <= 32u) {
+        gqa_decode_merge_wave<<<dim3((p.num_heads + 3u) / 4u, p.batch), dim3(256), 0, stream>>>(p);
     } else {
         gqa_decode_merge<<<dim3(p.num_heads, p.batch), dim3(256), 0, stream>>>(p);
     }
