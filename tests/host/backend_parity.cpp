@@ -702,6 +702,20 @@ static void test_block_attention(const RocmContext& ctx)
                                                        ctx.tensor_from_f32(k_tail, kv_rows - cut, kv_cols).unwrap(),
                                                        ctx.tensor_from_f32(v_tail, kv_rows - cut, kv_cols).unwrap(), spec.unwrap());
         CHECK(split.is_ok(), "block_attention_prefix_suffix: %s", split.is_err() ? split.unwrap_err().to_string().c_str() : "");
+        {
+            // the same rows as three segments, the middle one a single row
+            auto kt = ctx.tensor_from_f32(k_head, cut, kv_cols, DType::BF16).unwrap(), vt = ctx.tensor_from_f32(v_head, cut, kv_cols, DType::BF16).unwrap();
+            std::vector<float> k_one(k_tail.begin(), k_tail.begin() + kv_cols), v_one(v_tail.begin(), v_tail.begin() + kv_cols);
+            std::vector<float> k_rest(k_tail.begin() + kv_cols, k_tail.end()), v_rest(v_tail.begin() + kv_cols, v_tail.end());
+            auto k1 = ctx.tensor_from_f32(k_one, 1, kv_cols).unwrap(), v1 = ctx.tensor_from_f32(v_one, 1, kv_cols).unwrap();
+            auto k2 = ctx.tensor_from_f32(k_rest, kv_rows - cut - 1, kv_cols).unwrap(), v2 = ctx.tensor_from_f32(v_rest, kv_rows - cut - 1, kv_cols).unwrap();
+            auto three = ctx.block_attention_segments(qt.unwrap(), {&kt, &k1, &k2}, {&vt, &v1, &v2}, spec.unwrap());
+            CHECK(three.is_ok(), "block_attention_segments: %s", three.is_err() ? three.unwrap_err().to_string().c_str() : "");
+            if (three.is_ok() && split.is_ok()) {
+                CHECK(ctx.tensor_to_f32(three.unwrap()).unwrap() == ctx.tensor_to_f32(split.unwrap()).unwrap(), "three segments must give the bits of two");
+            }
+            CHECK(ctx.block_attention_segments(qt.unwrap(), {&kt, &k1}, {&vt}, spec.unwrap()).is_err(), "unequal K / V segment counts must be refused");
+        }
         if (split.is_ok()) {
             // the prefix arrives as bf16 here (a cache kept in bf16): the oracle reads what the planes hold
             std::vector<float> k_seen = k, v_seen = v;

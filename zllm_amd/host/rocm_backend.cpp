@@ -1374,28 +1374,32 @@ Result<RocmTensor> RocmContext::gqa_prefill_attention_visible(const RocmTensor& 
                         (const uint32_t*)ends.unwrap().data());
 }
 
-Result<RocmTensor> RocmContext::block_attention_prefix_suffix(const RocmTensor& query, const RocmTensor& prefix_key, const RocmTensor& prefix_value,
-                                                              const RocmTensor& suffix_key, const RocmTensor& suffix_value,
-                                                              const BlockAttentionSpec& spec) const
+Result<RocmTensor> RocmContext::block_attention_segments(const RocmTensor& query, const std::vector<const RocmTensor*>& keys,
+                                                         const std::vector<const RocmTensor*>& values, const BlockAttentionSpec& spec) const
 {
-    const size_t kv_rows = prefix_key.rows + suffix_key.rows;
+    if (keys.size() != values.size() || keys.empty()) {
+        return compute_error("block attention segments K/V count=" + std::to_string(keys.size()) + "/" + std::to_string(values.size()));
+    }
+    const size_t query_cols = spec.geometry.num_heads * spec.geometry.head_dim, kv_cols = spec.geometry.num_kv_heads * spec.geometry.head_dim;
+    size_t kv_rows = 0;
+    for (size_t i = 0; i < keys.size(); ++i) {
+        if (keys[i] == nullptr || values[i] == nullptr || keys[i]->cols != kv_cols || values[i]->cols != kv_cols || keys[i]->rows != values[i]->rows) {
+            return compute_error("ROCm block attention shape mismatch in K/V segment " + std::to_string(i));
+        }
+        kv_rows += keys[i]->rows;
+    }
     if (auto bad = spec.validate(query.rows, kv_rows)) {
         return compute_error(*bad);
     }
-    const size_t query_cols = spec.geometry.num_heads * spec.geometry.head_dim, kv_cols = spec.geometry.num_kv_heads * spec.geometry.head_dim;
-    if (query.cols != query_cols || prefix_key.cols != kv_cols || prefix_value.rows != prefix_key.rows || prefix_value.cols != kv_cols ||
-        suffix_key.cols != kv_cols || suffix_value.rows != suffix_key.rows || suffix_value.cols != kv_cols) {
-        return compute_error("ROCm block attention shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "] K=[" +
-                             std::to_string(prefix_key.rows) + "+" + std::to_string(suffix_key.rows) + "," + std::to_string(prefix_key.cols) +
-                             "] V=[" + std::to_string(prefix_value.rows) + "+" + std::to_string(suffix_value.rows) + "," +
-                             std::to_string(prefix_value.cols) + "]");
+    if (query.cols != query_cols) {
+        return compute_error("ROCm block attention shape mismatch: Q=[" + std::to_string(query.rows) + "," + std::to_string(query.cols) + "]");
     }
     if (kv_rows > UINT32_MAX || query.rows > UINT32_MAX) {
         return compute_error("ROCm block attention visible range beyond u32");
     }
     // the entry point reads no cache row at or past position + rows: put the query rows at the end of whichever is longer
     const size_t cache_rows = std::max(kv_rows, query.rows);
-    auto planes = dense_f16_planes({&prefix_key, &suffix_key}, {&prefix_value, &suffix_value}, kv_cols, cache_rows);
+    auto planes = dense_f16_planes(keys, values, kv_cols, cache_rows);
     if (planes.is_err()) {
         return planes.unwrap_err();
     }
@@ -1412,13 +1416,17 @@ Result<RocmTensor> RocmContext::block_attention_prefix_suffix(const RocmTensor& 
     return attend_dense(query, planes.unwrap(), cache_rows - query.rows, spec.geometry, spec.score_scale, 0, starts, starts + query.rows);
 }
 
+Result<RocmTensor> RocmContext::block_attention_prefix_suffix(const RocmTensor& query, const RocmTensor& prefix_key, const RocmTensor& prefix_value,
+                                                              const RocmTensor& suffix_key, const RocmTensor& suffix_value,
+                                                              const BlockAttentionSpec& spec) const
+{
+    return block_attention_segments(query, {&prefix_key, &suffix_key}, {&prefix_value, &suffix_value}, spec);
+}
+
 Result<RocmTensor> RocmContext::block_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value,
                                                 const BlockAttentionSpec& spec) const
 {
-    RocmTensor none;
-    none.cols = key.cols;
-    none.dtype = key.dtype;
-    return block_attention_prefix_suffix(query, key, value, none, none, spec);
+    return block_attention_segments(query, {&key}, {&value}, spec);
 }
 
 Result<Unit> RocmContext::append_mla_impl(RocmKvCache& cache, size_t layer, const RocmTensor& latent, const RocmTensor& rope, size_t rotary_dim,

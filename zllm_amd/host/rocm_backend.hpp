@@ -265,6 +265,10 @@ class RocmContext {
     // BlockAttentionBackend::block_attention (src/backend/mod.rs:1582-1584; ROCm body src/backend/rocm/attention.rs:118-144):
     // query and KV lengths differ, every query row sees exactly its range.  Returns f32 [query.rows, num_heads * head_dim].
     Result<RocmTensor> block_attention(const RocmTensor& query, const RocmTensor& key, const RocmTensor& value, const BlockAttentionSpec& spec) const;
+    // block_attention_segments (src/backend/mod.rs:1586-1598): the KV rows arrive as several tensors in order; each is
+    // written behind the one before it into the scratch planes, no concatenated copy is made on the way.
+    Result<RocmTensor> block_attention_segments(const RocmTensor& query, const std::vector<const RocmTensor*>& keys,
+                                                const std::vector<const RocmTensor*>& values, const BlockAttentionSpec& spec) const;
     // block_attention_prefix_suffix (src/backend/mod.rs:1601-1616): the KV rows are a resident prefix followed by this
     // step's short suffix; the two are written one behind the other into the scratch planes, never concatenated on the host.
     Result<RocmTensor> block_attention_prefix_suffix(const RocmTensor& query, const RocmTensor& prefix_key, const RocmTensor& prefix_value,
