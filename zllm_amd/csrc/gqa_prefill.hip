@@ -722,11 +722,22 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
     constexpr int G = C::kG;
     constexpr bool Q8 = KV == 0;
     static_assert(C::kLoads >= 1, "a staging thread owns at least one chunk");
-    __shared__ __align__(16) unsigned char lds_k[2][C::kTile];
-    __shared__ __align__(16) unsigned char lds_v[2][C::kTile];
-    __shared__ __align__(16) float lds_ks[Q8 ? 2 : 1][Q8 ? G : 1][kStep]; // [buffer][group][token], Q8g64 only
-    __shared__ __align__(16) float lds_vs[Q8 ? 2 : 1][Q8 ? G : 1][kStep];
-    __shared__ __align__(16) float lds_top[2][8];                         // [buffer][staging wave]: largest scale it converted
+    // Four tile buffers, as in gqa_prefill_q8: a pass attends two tiles while the next two go into the other pair, one
+    // barrier per 64 tokens.  The small arrays come first so that as many buffer addresses as possible are a lane
+    // register plus an immediate inside the LDS offset field.
+    struct Lds {
+        float ks[Q8 ? 4 : 1][Q8 ? G : 1][kStep]; // [buffer][group][token], Q8g64 only
+        float vs[Q8 ? 4 : 1][Q8 ? G : 1][kStep];
+        float top[4][8];                         // [buffer][staging wave]: largest scale it converted
+        unsigned char k[4][C::kTile];
+        unsigned char v[4][C::kTile];
+    };
+    __shared__ __align__(16) Lds lds;
+    auto& lds_k = lds.k;
+    auto& lds_v = lds.v;
+    auto& lds_ks = lds.ks;
+    auto& lds_vs = lds.vs;
+    auto& lds_top = lds.top;
 
     const unsigned int tid = threadIdx.x;
     const unsigned int lane = tid & 63u;
@@ -1158,19 +1169,19 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
         }
     };
 
-    // ---- main loop: the rows of step n + 1 are loaded while step n computes, and stored before the barrier
-    // (requesting them a step earlier still was measured: no change, the loads are not what a step waits for) ----
+    // ---- main loop: two tiles are attended per pass while the next two travel, one at a time through the same registers,
+    // into the other pair of buffers, which nobody reads before the barrier ----
     StageRegs regs;
     load_step(regs, part.begin, entry_of(part.begin + st_token));
     unsigned int entry_next = entry_of(part.begin + kStep + st_token);
     store_step(regs, 0);
+    load_step(regs, part.begin + kStep, entry_next); // past the end of the range the last row repeats: loads stay inside the pages
+    entry_next = entry_of(part.begin + 2u * kStep + st_token);
+    store_step(regs, 1);
     __syncthreads();
     unsigned int wv = 2u; // Q8g64: (biased) exponent of the largest V scale up to the tile being attended
     float v_shift = Q8 ? kPBias + 125.0f : kPBias;
-    auto one_step = [&](unsigned int step, int buf) __attribute__((always_inline)) {
-        const unsigned int t0 = part.begin + step * kStep;
-        load_step(regs, t0 + kStep, entry_next); // past the end of the range the last row repeats: loads stay inside the pages
-        entry_next = entry_of(t0 + 2u * kStep + st_token);
+    auto attend_tile = [&](unsigned int t0, int buf) __attribute__((always_inline)) {
         bool window_moved = false;
         float acc_fix = 1.0f;
         if constexpr (Q8) {
@@ -1183,16 +1194,33 @@ __global__ __launch_bounds__(512) void gqa_prefill_tiles(GqaPrefillParams p)
             }
         }
         compute_step(buf, t0, v_shift, acc_fix, window_moved);
-        store_step(regs, buf ^ 1);
+    };
+    auto two_steps = [&](unsigned int step, int set) __attribute__((always_inline)) {
+        const unsigned int t0 = part.begin + step * kStep;
+        load_step(regs, t0 + 2u * kStep, entry_next);
+        entry_next = entry_of(t0 + 3u * kStep + st_token);
+        attend_tile(t0, 2 * set);
+        store_step(regs, 2 * (set ^ 1));
+        PREFILL_PHASE_FENCE(); // the two tiles are attended one after the other: interleaved, their operands do not fit the registers
+        load_step(regs, t0 + 3u * kStep, entry_next);
+        entry_next = entry_of(t0 + 4u * kStep + st_token);
+        attend_tile(t0 + kStep, 2 * set + 1);
+        store_step(regs, 2 * (set ^ 1) + 1);
         __syncthreads();
     };
     unsigned int step = 0;
-    for (; step + 1 < steps; step += 2) {
-        one_step(step, 0);
-        one_step(step + 1u, 1);
+    for (; step + 4 <= steps; step += 4) {
+        two_steps(step, 0);
+        two_steps(step + 2u, 1);
     }
-    if (step < steps) {
-        one_step(step, 0);
+    if (step + 2 <= steps) {
+        two_steps(step, 0);
+        step += 2;
+        if (step < steps) { // the odd tile at the end sits in the first buffer of the other pair
+            attend_tile(part.begin + step * kStep, 2);
+        }
+    } else if (step < steps) {
+        attend_tile(part.begin + step * kStep, 0);
     }
 
     // ---- normalise and store ------------------------------------------------------------------------
