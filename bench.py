@@ -477,8 +477,8 @@ def run_copy_calibration(args):
 
 def other_configs(args):
     """The other benchmark configurations in the same process, each replayed or launched at least 100 times and checked
-    against the oracle on a slice: the ragged draw of config 2, config 4 (MLA decode at 64K, the MFMA-bound one) and config 5
-    (the prefill chunk).  Keys per entry: ms_per_step, value + unit, roofline {kernel, achieved, peak, frac, kernel_ms},
+    against the oracle on a slice: the ragged draw of config 2, config 4 (MLA decode at 64K, the MFMA-bound one), config 5
+    (the prefill chunk) and config 3 (f16 cache at head_dim 256, a full and a sliding-window layer).  Keys per entry: ms_per_step, value + unit, roofline {kernel, achieved, peak, frac, kernel_ms},
     parity_vs_oracle_max_abs."""
     import copy
 
@@ -488,7 +488,7 @@ def other_configs(args):
 
     def brief(record):
         keep = ("ms_per_step", "value", "unit", "steps", "pct_of_hbm_peak", "pct_of_mfma_peak", "tokens_per_s", "stage_ms", "parity_vs_oracle_max_abs",
-                "parity_sample", "ms_per_step_regions")
+                "parity_sample", "ms_per_step_regions", "window_layer")
         out = {k: record[k] for k in keep if k in record}
         out["workload"] = record["config"]["workload"]
         out["roofline"] = {k: v for k, v in record["roofline"].items() if k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "kernel_ms",
@@ -513,6 +513,11 @@ def other_configs(args):
     sub.steps, sub.warmup = 100, 5
     sub.no_cpu_baseline, sub.workload = False, "gqa_prefill_chunk"
     results["gqa_prefill_chunk"] = brief(bench_extra.workload_record(sub))
+    torch.cuda.empty_cache()
+    sub = copy.copy(args)
+    sub.steps, sub.warmup = max(args.steps, 100), max(args.warmup, 10)
+    sub.no_cpu_baseline, sub.workload = False, "gqa_decode_f16_window"
+    results["gqa_decode_f16_window"] = brief(bench_extra.workload_record(sub))
     torch.cuda.empty_cache()
     return results
 
