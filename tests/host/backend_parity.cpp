@@ -473,6 +473,15 @@ static void test_gqa_shared_and_visible(const RocmContext& ctx)
     if (seen.is_ok()) {
         compare(ctx.tensor_to_f32(seen.unwrap()).unwrap(), want, "gqa_prefill_attention_cached_visible, 16-row blocks");
     }
+    // a layer that shares layer 1's K/V sees the same visual blocks: the rows are in the cache already, so the bits are the same
+    auto shared_seen = ctx.gqa_prefill_attention_cached_from_visible(cache, 1, prefix, qt.unwrap(), spec, ends);
+    CHECK(shared_seen.is_ok(), "cached_from_visible: %s", shared_seen.is_err() ? shared_seen.unwrap_err().to_string().c_str() : "");
+    if (shared_seen.is_ok() && seen.is_ok()) {
+        CHECK(ctx.tensor_to_f32(shared_seen.unwrap()).unwrap() == ctx.tensor_to_f32(seen.unwrap()).unwrap(),
+              "gqa_prefill_attention_cached_from_visible must give the bits of the appending call");
+    }
+    CHECK(ctx.gqa_prefill_attention_cached_from_visible(cache, 1, prefix, qt.unwrap(), spec, std::vector<uint32_t>(rows - 1, 1u)).is_err(),
+          "one visible end too few must be refused");
     // layer 0 shares layer 1's K/V: the same chunk, causal, nothing appended
     auto shared = ctx.gqa_prefill_attention_cached_from(cache, 1, prefix, qt.unwrap(), spec);
     CHECK(shared.is_ok(), "cached_from: %s", shared.is_err() ? shared.unwrap_err().to_string().c_str() : "");
