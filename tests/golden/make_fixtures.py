@@ -10,6 +10,10 @@ kernel shows up as a difference against committed bytes:
                         32-entry token selection per sequence
   gqa_prologue_small.npz 5 rows, 4q/2kv, d=128: per-head Gemma RMSNorm + split-half RoPE of Q and K, K/V quantized into pages
   gqa_prefill_small.npz prefix 200 + chunk 48, 8q/2kv, window 0 and 64 -> chunk outputs
+  block_attention_small.npz 40 query rows over 100 KV rows, 8q/2kv, d=128: varlen segments (offsets Q [0, 7, 8, 40], KV [0, 50,
+                        51, 100]) and free per-row ranges -> outputs of the block attention with explicit ranges
+  mla_other_widths_small.npz B=2, 3 heads, latent 128 + rope 32, nope 64 / value 64, kv_b as W8A16 codes (groups of 64, bf16
+                        scales) -> output before the final bf16 rounding
 """
 import os
 import sys
@@ -117,7 +121,47 @@ def gqa_prefill():
                         score_scale=np.float32(0.0884), **planes, **out)
 
 
+def block_attention():
+    rng = np.random.default_rng(507)
+    hq, hkv, d, bt, q_rows, kv_rows = 8, 2, 128, 16, 40, 100
+    cols = hkv * d
+    table = rng.permutation(12)[: (kv_rows + bt - 1) // bt].astype(np.uint32)
+    planes = {n: np.zeros((12 * bt, cols if "codes" in n else cols // 64), dtype=np.int8 if "codes" in n else np.uint16)
+              for n in ("k_codes", "k_scales", "v_codes", "v_scales")}
+    k = rng.standard_normal((kv_rows, cols)).astype(np.float32)
+    v = rng.standard_normal((kv_rows, cols)).astype(np.float32)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, k, planes["k_codes"], planes["k_scales"], table, 0, bt)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, planes["v_codes"], planes["v_scales"], table, 0, bt)
+    q_bits = O.f32_to_bf16(rng.standard_normal((q_rows, hq * d)).astype(np.float32))
+    kd = O.gather_dequant_rows(O.FMT_Q8, planes["k_codes"], planes["k_scales"], O.SCALE_F16, table, bt, 0, kv_rows, cols)
+    vd = O.gather_dequant_rows(O.FMT_Q8, planes["v_codes"], planes["v_scales"], O.SCALE_F16, table, bt, 0, kv_rows, cols)
+    varlen = np.array([(0, 50)] * 7 + [(50, 51)] + [(51, 100)] * 32, dtype=np.uint32)
+    starts = rng.integers(0, kv_rows, size=q_rows)
+    free = np.stack([starts, starts + 1 + (rng.integers(0, kv_rows, size=q_rows) % (kv_rows - starts))], axis=1).astype(np.uint32)
+    out = {}
+    for name, visible in (("varlen", varlen), ("free", free)):
+        rc, want = O.block_attention(O.bf16_to_f32(q_bits), kd, vd, hq, hkv, d, 0.0884, visible)
+        assert rc == 0
+        out[f"visible_{name}"] = visible
+        out[f"expected_{name}"] = want
+    np.savez_compressed(os.path.join(HERE, "block_attention_small.npz"), q_bits=q_bits, table=table, score_scale=np.float32(0.0884), **planes, **out)
+
+
+def mla_other_widths():
+    from tests.test_gpu_mla_decode import make_mla_case, oracle_mla, set_weight_form
+
+    case = make_mla_case(509, [70, 33], 3, nope=64, rope=32, value=64, latent=128)
+    set_weight_form(case, 8, group=64, scale_dtype=O.SCALE_BF16)
+    want, _ = oracle_mla(case)
+    form = case["kv_b_form"]
+    np.savez_compressed(os.path.join(HERE, "mla_other_widths_small.npz"), q_bits=case["q_bits"], kv_b_words=form["data"], kv_b_scales=form["scales"],
+                        kv_b_values=case["kv_b_f32"], codes=case["codes"], scales=case["scales"], rope=case["rope"], tables=case["tables"],
+                        lens=case["lens"], expected_f32=want)
+
+
 if __name__ == "__main__":
+    block_attention()
+    mla_other_widths()
     quantizer()
     gqa_decode()
     mla_decode()

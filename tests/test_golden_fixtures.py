@@ -128,3 +128,59 @@ def test_prefill_kernel_matches_the_prefill_fixture(window):
                                 window=window, scale_dtype=capi.SCALE_F16)
     torch.cuda.synchronize()
     assert_attention_close(out.cpu().numpy(), g[f"expected_window_{window}"], f"prefill fixture, window {window}")
+
+
+def test_oracle_reproduces_the_block_attention_fixture():
+    g = load("block_attention_small.npz")
+    kd = O.gather_dequant_rows(O.FMT_Q8, g["k_codes"], g["k_scales"], O.SCALE_F16, g["table"], 16, 0, 100, 256)
+    vd = O.gather_dequant_rows(O.FMT_Q8, g["v_codes"], g["v_scales"], O.SCALE_F16, g["table"], 16, 0, 100, 256)
+    for name in ("varlen", "free"):
+        rc, out = O.block_attention(O.bf16_to_f32(g["q_bits"]), kd, vd, 8, 2, 128, float(g["score_scale"]), g[f"visible_{name}"])
+        assert rc == 0
+        assert np.array_equal(out, g[f"expected_{name}"]), name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["varlen", "free"])
+def test_prefill_kernel_matches_the_block_attention_fixture(name):
+    torch = pytest.importorskip("torch")
+    from zllm_amd import ops
+
+    g = load("block_attention_small.npz")
+    visible = g[f"visible_{name}"]
+    out = ops.gqa_prefill_chunk(to_torch_bf16(g["q_bits"], "cuda"), upload(g["k_codes"]), upload(g["k_scales"]), upload(g["v_codes"]),
+                                upload(g["v_scales"]), upload(g["table"]), 100 - 40, 8, 2, 128, 16, float(g["score_scale"]),
+                                visible_starts=upload(visible[:, 0].copy()), visible_ends=upload(visible[:, 1].copy()))
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g[f"expected_{name}"], f"block attention fixture ({name})")
+
+
+def test_oracle_reproduces_the_other_widths_mla_fixture():
+    g = load("mla_other_widths_small.npz")
+    spec = O.MlaSpec(128, 32, 3 * 96, 3 * 128, 3)
+    for b, l in enumerate(g["lens"]):
+        l = int(l)
+        codes = O.gather_rows_bytes(g["codes"], g["tables"][b], 16, 0, l, 128)
+        scales = O.gather_rows_bytes(g["scales"], g["tables"][b], 16, 0, l, 4).view(np.uint16)
+        rope = O.gather_rows_bytes(g["rope"], g["tables"][b], 16, 0, l, 64).view(np.uint16)
+        rc, _, out, _ = O.mla_absorbed_q8_history(spec, g["q_bits"][b:b + 1], 1, l - 1, codes, scales, 64, rope, l, g["kv_b_values"])
+        assert rc == 0
+        assert np.array_equal(out.reshape(-1), g["expected_f32"][b].reshape(-1))
+    # the stored values are what the stored codes stand for: (code - 128) x bf16 scale of the row's 64-column group
+    words, scale_bits = g["kv_b_words"], g["kv_b_scales"]
+    codes = np.stack([(words >> np.uint32(8 * i)) & np.uint32(255) for i in range(4)], axis=2).reshape(words.shape[0], -1).astype(np.int32) - 128
+    values = codes.astype(np.float32) * np.repeat(O.bf16_to_f32(scale_bits), 64, axis=1)
+    assert np.array_equal(values, g["kv_b_values"])
+
+
+@pytest.mark.gpu
+def test_mla_kernels_match_the_other_widths_fixture():
+    torch = pytest.importorskip("torch")
+    from zllm_amd import capi, ops
+
+    g = load("mla_other_widths_small.npz")
+    out = ops.mla_decode(to_torch_bf16(g["q_bits"], "cuda"), upload(g["kv_b_words"]), upload(g["codes"]), upload(g["scales"]), upload(g["rope"]),
+                         upload(g["tables"]), upload(g["lens"]), 3, 96, 128, 128, 32, 16, int(g["lens"].max()), kv_b_bits=8,
+                         kv_b_scales=upload(g["kv_b_scales"]), kv_b_group=64, kv_b_scale_dtype=capi.SCALE_BF16)
+    torch.cuda.synchronize()
+    assert_attention_close(out.cpu().numpy(), g["expected_f32"].reshape(out.shape), "MLA fixture at latent 128 + rope 32 with W8 kv_b")
