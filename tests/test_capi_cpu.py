@@ -285,3 +285,44 @@ def test_prefill_and_mla_argument_checks_without_a_gpu(lib):
     one = capi.MlaDecodeArgs.from_buffer_copy(mla)
     one.query_rows = 0
     assert lib.zllm_attn_mla_decode_workspace_bytes(C.byref(mla)) > lib.zllm_attn_mla_decode_workspace_bytes(C.byref(one)) > 0
+
+
+def test_mla_widths_and_weight_forms_are_validated_on_the_host(lib):
+    """Latent widths are multiples of 64 up to 1,024, rope widths even up to 256, kv_b is bf16 / f32 or 8- / 4-bit codes with
+    scales and a group size that divides the latent width: everything else is refused before a workspace size is named."""
+    def args(**kw):
+        a = capi.MlaDecodeArgs()
+        a.batch, a.heads, a.q_head_dim, a.kv_head_dim, a.latent_dim, a.rope_dim = 2, 4, 96, 128, 128, 32
+        a.block_tokens, a.max_ctx_len, a.q_dtype, a.out_dtype = 16, 500, capi.DTYPE_BF16, capi.DTYPE_F32
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    size = lib.zllm_attn_mla_decode_workspace_bytes
+    assert size(C.byref(args())) > 0
+    assert size(C.byref(args(latent_dim=1024, rope_dim=256, q_head_dim=320))) > 0
+    assert size(C.byref(args(kv_b_bits=32))) > 0
+    scales = C.c_void_p(0x1000)  # never read on the host
+    assert size(C.byref(args(kv_b_bits=8, kv_b_scales=scales, kv_b_group=64, kv_b_scale_dtype=capi.SCALE_F16))) > 0
+    assert size(C.byref(args(kv_b_bits=4, kv_b_scales=scales, kv_b_group=128))) > 0
+    for bad, word in ((dict(latent_dim=96), "multiple of 64"), (dict(latent_dim=1088), "multiple of 64"), (dict(rope_dim=31), "even"),
+                      (dict(rope_dim=258, q_head_dim=322), "even"), (dict(kv_b_bits=5), "kv_b_bits"),
+                      (dict(kv_b_bits=8, kv_b_group=64), "scales"), (dict(kv_b_bits=8, kv_b_scales=scales, kv_b_group=48), "group size"),
+                      (dict(kv_b_bits=4, kv_b_scales=scales, kv_b_group=64, kv_b_scale_dtype=7), "scale dtype")):
+        assert size(C.byref(args(**bad))) == 0
+        assert word in capi.last_error(), (bad, capi.last_error())
+
+
+def test_head_dim_192_is_taken_over_q8g64_only(lib):
+    a = capi.GqaDecodeArgs()
+    a.batch, a.num_heads, a.num_kv_heads, a.head_dim, a.max_kv_len, a.block_tokens, a.score_scale = 2, 12, 3, 192, 4000, 16, 0.07
+    a.kv_format, a.scale_dtype, a.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(a)) > 0
+    a.kv_format = capi.KV_F16
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(a)) == 0 and "f16 KV supports head_dim 128 and 256" in capi.last_error()
+    a.kv_format, a.head_dim = capi.KV_Q8G64, 96
+    assert lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(a)) == 0
+    pre = capi.GqaPrefillArgs()
+    pre.rows, pre.position, pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens, pre.score_scale = 64, 500, 12, 3, 192, 16, 0.07
+    pre.kv_format, pre.scale_dtype, pre.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16
+    assert lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre)) > 0  # its rows run as decode items: ranges and split records
