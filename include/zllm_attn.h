@@ -299,7 +299,11 @@ ZLLM_API int zllm_attn_gqa_decode_split_plan(const zllm_gqa_decode_args* args, u
  * with query_rows > 1, a query row) is row g * max_chunks + c when dense == 0 -- a plan for equal lengths -- and row
  * first_rows[g] + c when dense == 1: a ragged plan numbers its records over the live splits only, in group order, so the
  * workspace grows with the tokens there are and not with batch x longest sequence; first_rows is u32 [groups] at
- * first_rows_offset, written by the partial stage (entries of groups without splits are not written). */
+ * first_rows_offset, written by the partial stage (entries of groups without splits are not written).  A group has
+ * min(max_chunks, ceil(n / chunk_tokens)) splits, n = its visible tokens (GQA: counted from first_visible rounded down to
+ * a multiple of 32).  A record is un-normalised: partial = sum of p x value with p = 2^(score - max), max the largest
+ * scaled score of the split in base-2 units (score x score_scale x log2 e), sum = sum of p; an empty split has
+ * (max, sum) = (-inf, 0).  Combined: out = sum_c partial_c 2^(max_c - M) / sum_c sum_c 2^(max_c - M), M = max_c max_c. */
 typedef struct zllm_split_record_layout {
     uint64_t record_rows;
     uint64_t partial_offset;
