@@ -39,7 +39,7 @@ def close_at_scale(got, want, what, extra=0.0):
     return assert_attention_close(np.asarray(got, dtype=np.float64) / top, want / top, what, atol=2e-3 + extra)
 
 
-@pytest.mark.parametrize("it", range(40))
+@pytest.mark.parametrize("it", [*range(40), 265, 273, 497])  # the last three: 128 query heads at head_dim 256 over outlier channels
 def test_random_q8_decode(it):
     rng = np.random.default_rng([101, it])
     hkv = pick(rng, [1, 2, 4, 8])
@@ -57,7 +57,7 @@ def test_random_q8_decode(it):
     assert_attention_close(got, oracle_gqa_decode(case, 0.09, window=window, softcap=softcap), what)
 
 
-@pytest.mark.parametrize("it", range(48))
+@pytest.mark.parametrize("it", [*range(48), 1298])  # 1298: f32 queries, score scale 0.3, outlier channels
 def test_random_q8_prefill_chunk(it):
     """All three head sizes, the three scale-storage rules, visible ends, gates, K and V gains over 2^-8..2^8."""
     rng = np.random.default_rng([202, it])
@@ -165,7 +165,7 @@ def test_random_mla_chunk(it):
         assert_attention_close(wide.reshape(want.shape), want, what + " (wide tiles)")
 
 
-@pytest.mark.parametrize("it", range(16))
+@pytest.mark.parametrize("it", [*range(16), 779])  # 779: 24 heads on 3, soft cap, a first chunk of 64 rows
 def test_random_q8_head_dim_192(it):
     """Decode steps and prefill chunks at head_dim 192 (three Q8g64 groups a head): every scale rule, pages of 1 to 64 tokens,
     windows, soft caps, the token-count hint on every other case."""

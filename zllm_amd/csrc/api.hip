@@ -1103,7 +1103,7 @@ void plan_prefill_splits(const zllm_gqa_prefill_args* a, uint32_t* chunk_tokens,
 {
     const uint32_t group = a->num_heads / a->num_kv_heads;
     const bool half_tiles = zllm::gqa_prefill_half_tiles(a->rows, a->position, a->window, a->num_heads, a->num_kv_heads, a->head_dim, a->kv_format,
-                                                         a->scale_dtype);
+                                                         a->scale_dtype, a->q_dtype);
     const uint32_t columns = a->head_dim == 256 || half_tiles ? 128u : 256u; // (row, head-in-group) pairs of a workgroup
     const uint32_t tile_rows = columns / group > 0 ? columns / group : 1u;
     const uint64_t tiles = ((uint64_t)a->rows + tile_rows - 1) / tile_rows;
@@ -1218,7 +1218,7 @@ static bool few_rows_as_decode_items(const zllm_gqa_prefill_args* a)
     // the chunk kernel's half-size row tiles (Q8g64 with 16-bit scales at head_dim 128, a chunk whose pairs fit one) walk
     // a key in 0.8 ns: eight rows over 32 K tokens 54 us, where they would cost 104 as decode items
     const bool half_tiles = zllm::gqa_prefill_half_tiles(a->rows, a->position, a->window, a->num_heads, a->num_kv_heads, a->head_dim, a->kv_format,
-                                                         a->scale_dtype);
+                                                         a->scale_dtype, a->q_dtype);
     return (uint64_t)a->rows * tokens * 34u < tokens * (half_tiles ? 80u : 150u) + 1300000u;
 }
 

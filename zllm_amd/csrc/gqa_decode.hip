@@ -10,7 +10,7 @@
 //
 // Per wave, per 32-token step (two 16-token tiles):
 //   S^T[token, head] = K[token, :] . Q[head, :]      int8 MFMA 16x16x64, A = K codes as stored,
-//                                                    B = Q in 15-bit fixed point, two 8-bit digits
+//                                                    B = Q in 16-bit fixed point, two 8-bit digits
 //     one MFMA pair per 64-column scale group, so the group scale is applied to the finished
 //     integer dot: s = sum_g scale_g * dot_g  (no per-element multiply, no K conversion)
 //   online softmax: row max / row sum over the four 16-lane groups by wave shuffles
@@ -228,9 +228,9 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
 }
 
 // Q fragments: B operand of the int8 MFMA, lane = (head column m, k-slice j).
-// The head's query row is quantized to 15-bit fixed point (step = max|q| / 16256) and split into two
-// signed-byte digits q = 128 * hi + lo, hi in [-127, 127], lo in [-64, 63]: K codes then feed the matrix
-// cores as raw bytes and the integer dot products are exact.
+// The head's query row is quantized to 16-bit fixed point (step = max|q| / 32512) and split into two
+// signed-byte digits q = 256 * hi + lo, hi in [-127, 127], lo in [-128, 127]: K codes then feed the matrix
+// cores as raw bytes and the integer dot products are exact (|256 * dot_hi + dot_lo| < 2^28 for 64 columns).
 // Fetching and quantizing are separate so that a kernel can start the fetch, issue other loads, and
 // quantize when the data is needed.
 template <int D> struct QueryRaw {
@@ -301,8 +301,8 @@ __device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const Q
     }
     q_absmax = wave_max_16x4(q_absmax);
     const bool q_ok = q_absmax > 0.0f && q_absmax < __builtin_inff();
-    q_step = q_ok ? q_absmax * (1.0f / 16256.0f) : 0.0f;
-    const float inv_step = q_ok ? 16256.0f / q_absmax : 0.0f;
+    q_step = q_ok ? q_absmax * (1.0f / 32512.0f) : 0.0f;
+    const float inv_step = q_ok ? 32512.0f / q_absmax : 0.0f;
 #pragma unroll
     for (int a = 0; a < G; ++a) {
 #pragma unroll
@@ -311,9 +311,9 @@ __device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const Q
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 int qi = (int)rintf(x[a][4 * w + e] * inv_step);
-                qi = max(-16256, min(16256, qi));
-                const int hi = (qi + 64) >> 7;
-                const int lo = qi - hi * 128;
+                qi = max(-32512, min(32512, qi));
+                const int hi = (qi + 128) >> 8;
+                const int lo = qi - hi * 256;
                 hi_word |= ((unsigned int)hi & 0xffu) << (8 * e);
                 lo_word |= ((unsigned int)lo & 0xffu) << (8 * e);
             }
@@ -356,7 +356,7 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Ro
             f32x4 d;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                d[r] = (float)(dh[r] * 128 + dl[r]);
+                d[r] = (float)(dh[r] * 256 + dl[r]);
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {

@@ -149,7 +149,7 @@ __device__ __forceinline__ void store_split_record(const GqaPrefillParams& p, un
 // fragment read from LDS feeds two MFMAs; one makes it 128 pairs, for chunks whose full-size row tiles would be one round
 // of very unequal workgroups (a first chunk: the last tile walks the whole chunk, the first 64 keys) -- twice as many
 // workgroups, handed out longest first, even that out.
-template <int SDT, bool SOFTCAP, bool POW2, int CT = 2>
+template <int SDT, bool SOFTCAP, bool POW2, int CT = 2, bool QLO = false>
 __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 {
     constexpr int kColTiles = CT; // inside the kernel the name means this instantiation's count
@@ -224,10 +224,14 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 
     // ---- this wave's columns and Q fragments -------------------------------------------------
     // The wave's queries are carried as f16 after a multiplication by one power of two that puts the largest
-    // magnitude of its 32 columns into [2^8, 2^9); the inverse goes into the score factor.
+    // magnitude of its 32 columns into [2^8, 2^9); the inverse goes into the score factor.  bf16 and f16 queries are
+    // exact in that form.  An f32 query keeps 11 of its 24 bits, which moves peaked rows by up to 2e-3 of the output
+    // (a score scale of 0.3 over outlier channels), so QLO carries what the rounding dropped as a second f16 fragment
+    // and multiplies every K fragment by both: products stay exact, the query is good to 22 bits.
     unsigned int col_row[kColTiles], col_head[kColTiles];
     bool col_valid[kColTiles];
     Frag qf[kColTiles][4];
+    Frag ql[QLO ? kColTiles : 1][QLO ? 4 : 1];
     float q_fac;
     {
         float qx[kColTiles][4][8];
@@ -261,7 +265,13 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
             for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    qf[ct][ks].u[e] = pack_f16_hw(qx[ct][ks][2 * e] * q_mul, qx[ct][ks][2 * e + 1] * q_mul);
+                    const float x0 = qx[ct][ks][2 * e] * q_mul, x1 = qx[ct][ks][2 * e + 1] * q_mul;
+                    const unsigned int word = pack_f16_hw(x0, x1);
+                    qf[ct][ks].u[e] = word;
+                    if constexpr (QLO) {
+                        const f16x2 hi = __builtin_bit_cast(f16x2, word);
+                        ql[ct][ks].u[e] = pack_f16_hw(x0 - (float)hi[0], x1 - (float)hi[1]);
+                    }
                 }
             }
         }
@@ -432,6 +442,10 @@ __global__ __launch_bounds__(kThreads) void gqa_prefill_q8(GqaPrefillParams p)
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ++ct) {
                     f32x4 d = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (QLO) {
+                        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0.h, ql[ct][2 * g].h, d, 0, 0, 0);
+                        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1.h, ql[ct][2 * g + 1].h, d, 0, 0, 0);
+                    }
                     d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0.h, qf[ct][2 * g].h, d, 0, 0, 0);
                     d = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1.h, qf[ct][2 * g + 1].h, d, 0, 0, 0);
 #pragma unroll
@@ -1290,7 +1304,7 @@ template <int D, int KV, int SDT> static hipError_t launch_prefill_tiles(const G
 } // namespace
 
 bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned int window, unsigned int num_heads, unsigned int num_kv_heads,
-                            unsigned int head_dim, int kv_format, int scale_dtype)
+                            unsigned int head_dim, int kv_format, int scale_dtype, int q_dtype)
 {
     if (kv_format != 0 || head_dim != (unsigned int)kD || scale_dtype == 2 || num_kv_heads == 0) {
         return false; // not gqa_prefill_q8's geometry
@@ -1298,6 +1312,9 @@ bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned i
     const unsigned int group = num_heads / num_kv_heads;
     if (group == 0 || group > 128u) {
         return false;
+    }
+    if (q_dtype == 0) {
+        return true; // f32 queries travel as two f16 fragments: a wave has the registers for one column tile of them
     }
     if ((unsigned long long)rows * group <= 128u) {
         return true; // the whole chunk fits a half tile: a full one would be half empty at least
@@ -1341,7 +1358,7 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
         return launch_prefill_tiles<128, 0, 2>(p, stream);
     }
     const unsigned int full_rows = p.group >= 256u ? 1u : 256u / p.group;
-    const bool halves = gqa_prefill_half_tiles(p.rows, p.position, p.window, p.num_heads, p.num_kv_heads, p.head_dim, kv_format, scale_dtype);
+    const bool halves = gqa_prefill_half_tiles(p.rows, p.position, p.window, p.num_heads, p.num_kv_heads, p.head_dim, kv_format, scale_dtype, p.q_dtype);
     const unsigned int rows_per_wg = halves ? (p.group >= 128u ? 1u : 128u / p.group) : full_rows;
     const dim3 grid((p.rows + rows_per_wg - 1) / rows_per_wg * p.num_kv_heads, 1, p.max_chunks > 1u ? p.max_chunks : 1u);
     const bool cap = p.softcap > 0.0f;
@@ -1350,7 +1367,9 @@ hipError_t launch_gqa_prefill(const GqaPrefillParams& p, int kv_format, int scal
     auto launch = [&](auto sdt, auto softcap, auto table_pow2) {
         constexpr int S = decltype(sdt)::value;
         constexpr bool C = decltype(softcap)::value, P = decltype(table_pow2)::value;
-        if (halves) {
+        if (halves && p.q_dtype == 0) {
+            gqa_prefill_q8<S, C, P, 1, true><<<grid, block, 0, stream>>>(p);
+        } else if (halves) {
             gqa_prefill_q8<S, C, P, 1><<<grid, block, 0, stream>>>(p);
         } else {
             gqa_prefill_q8<S, C, P, 2><<<grid, block, 0, stream>>>(p);

@@ -184,7 +184,7 @@ struct MlaDecodeParams {
 // nothing to the whole chunk) when the full-size tiles would be at most one workgroup per compute unit: twice as many
 // workgroups, handed out longest first, even the launch out.  The split planner and the launcher both ask.
 bool gqa_prefill_half_tiles(unsigned int rows, unsigned int position, unsigned int window, unsigned int num_heads, unsigned int num_kv_heads,
-                            unsigned int head_dim, int kv_format, int scale_dtype);
+                            unsigned int head_dim, int kv_format, int scale_dtype, int q_dtype);
 
 // KV heads (= waves) per GQA decode workgroup for a head dimension.
 unsigned int gqa_decode_max_waves(unsigned int head_dim);
