@@ -349,7 +349,7 @@ def run_gqa_decode(args, ragged, config1=False):
                                 + ", 16-token pages"),
                    "kv_lens": lens, "kv_bytes_per_call": kv_bytes, "bytes_per_token": bytes_per_token, "seed": args.seed,
                    "pool_bytes": pool["pool_bytes"], "pool_blocks": pool["pool_blocks"], "max_code_plane_offset": pool["max_code_offset"],
-                   "q_dtype": "bf16", "scale_dtype": "f16", "kv_arithmetic": "K.Q on int8 MFMA (K codes raw, Q as two 8-bit digits); P.V on bf16 MFMA (V codes exact in bf16); f32 accumulate"},
+                   "q_dtype": "bf16", "scale_dtype": "f16", "kv_arithmetic": "K.Q on int8 MFMA (K codes raw, Q as three 8-bit digits); P.V on bf16 MFMA (V codes exact in bf16); f32 accumulate"},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(batch / (ms_step * 1e-3), 1),
         "ms_per_step_events": round(ms_events, 5),

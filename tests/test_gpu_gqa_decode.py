@@ -375,7 +375,7 @@ def test_every_kv_head_count_fits_its_workgroup(d):
 
 @pytest.mark.parametrize("q_kind", ["f32", "bf16", "f16"])
 def test_query_dtypes_through_fixed_point_digits(q_kind):
-    """The kernel quantizes each query row to 16-bit fixed point for the int8 matrix cores; every input
+    """The kernel quantizes each query row to 24-bit fixed point (three signed-byte digits) for the int8 matrix cores; every input
     dtype must stay within the attention tolerance, including rows whose elements span a wide range."""
     from zllm_amd import capi, ops
 

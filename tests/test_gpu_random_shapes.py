@@ -57,6 +57,43 @@ def test_random_q8_decode(it):
     assert_attention_close(got, oracle_gqa_decode(case, 0.09, window=window, softcap=softcap), what)
 
 
+@pytest.mark.parametrize("it", [*range(32), 52, 190, 266, 814])  # the last four: score scale 0.2 over outlier channels
+def test_random_q8_decode_pages_rules_and_hints(it):
+    """The decode sweep over what the one above keeps fixed: the three scale rules, pages of 1 to 64 tokens in random,
+    identity or reversed pool order, pools that were never cleared, longer sequences, a gate, the score scale, and the
+    token-count hint (records over the live splits) on every other case."""
+    rng = np.random.default_rng([606, it])
+    hkv = pick(rng, [1, 2, 3, 4, 8])
+    group = pick(rng, [1, 2, 4, 5, 8, 16])
+    d = pick(rng, [64, 128, 128, 128, 256])
+    rule = pick(rng, [O.RULE_METAL_GQA, O.RULE_ROCM_MLA, O.RULE_CUDA_GQA])
+    page = pick(rng, PAGE_SIZES + [32, 128])
+    lens = [pick(rng, LENGTHS + [6000, 9000, 20000]) for _ in range(int(rng.integers(1, 9)))]
+    if max(lens) == 0:
+        lens[0] = 5
+    window = pick(rng, [0, 0, 0, 1, 33, 500, 4096])
+    softcap = pick(rng, [0.0, 0.0, 50.0])
+    scale = pick(rng, [0.09, 1.0 / np.sqrt(d), 0.2])
+    layout = pick(rng, ["random", "random", "identity", "reversed"])
+    gated = bool(rng.integers(0, 4) == 0)
+    hint = it % 2 == 0
+    what = (f"decode {it}: {hkv * group}/{hkv} d={d} rule={rule} page={page} layout={layout} lens={lens} window={window} "
+            f"softcap={softcap} scale={scale:.3f} gated={gated} hint={hint}")
+    print(what, flush=True)
+    case = make_gqa_q8_case(6000 + it, lens, hkv * group, hkv, d, block_tokens=page, rule=rule, outliers=bool(it % 3), layout=layout,
+                            q_bf16=bool(it % 4 == 1), poison=bool(it % 5 == 0))
+    gate = (rng.standard_normal((len(lens), hkv * group * d)) * 3).astype(np.float32) if gated else None
+    visible = [min(l, window) if window else l for l in lens]
+    from tests.cases import upload
+    got = run_decode(case, scale, window=window, softcap=softcap, gate=None if gate is None else upload(gate),
+                     total_kv_tokens=sum(visible) if hint else 0)
+    want = oracle_gqa_decode(case, scale, window=window, softcap=softcap)
+    if gated:
+        rc, want = O.sigmoid_gate(want, gate)
+        assert rc == 0
+    assert_attention_close(got, want, what)
+
+
 @pytest.mark.parametrize("it", [*range(48), 1298])  # 1298: f32 queries, score scale 0.3, outlier channels
 def test_random_q8_prefill_chunk(it):
     """All three head sizes, the three scale-storage rules, visible ends, gates, K and V gains over 2^-8..2^8."""

@@ -10,7 +10,7 @@
 //
 // Per wave, per 32-token step (two 16-token tiles):
 //   S^T[token, head] = K[token, :] . Q[head, :]      int8 MFMA 16x16x64, A = K codes as stored,
-//                                                    B = Q in 16-bit fixed point, two 8-bit digits
+//                                                    B = Q in 24-bit fixed point, three 8-bit digits
 //     one MFMA pair per 64-column scale group, so the group scale is applied to the finished
 //     integer dot: s = sum_g scale_g * dot_g  (no per-element multiply, no K conversion)
 //   online softmax: row max / row sum over the four 16-lane groups by wave shuffles
@@ -228,9 +228,11 @@ __device__ __forceinline__ bool locate_split(const GqaDecodeParams& p, unsigned 
 }
 
 // Q fragments: B operand of the int8 MFMA, lane = (head column m, k-slice j).
-// The head's query row is quantized to 16-bit fixed point (step = max|q| / 32512) and split into two
-// signed-byte digits q = 256 * hi + lo, hi in [-127, 127], lo in [-128, 127]: K codes then feed the matrix
-// cores as raw bytes and the integer dot products are exact (|256 * dot_hi + dot_lo| < 2^28 for 64 columns).
+// The head's query row is quantized to 24-bit fixed point and split into three signed-byte digits,
+// q = step * (256 * hi + lo + ex / 256) with step = max|q| / 32512, hi in [-127, 127], lo and ex in [-128, 127]:
+// K codes then feed the matrix cores as raw bytes and the integer dot products are exact
+// (|256 * dot_hi + dot_lo| < 2^28 for 64 columns).  Two digits were not enough: with a score scale of 0.2 over
+// x8 outlier channels a 2^-17 step of the row's largest element moves outputs of magnitude 20 by up to 3e-3.
 // Fetching and quantizing are separate so that a kernel can start the fetch, issue other loads, and
 // quantize when the data is needed.
 template <int D> struct QueryRaw {
@@ -272,9 +274,12 @@ __device__ __forceinline__ QueryRaw<D> fetch_query(const GqaDecodeParams& p, uns
     return raw;
 }
 
+template <int G> struct QueryDigits {
+    i32x4 hi[G], lo[G], ex[G];
+};
+
 template <int D>
-__device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const QueryRaw<D>& raw, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64],
-                                               float& q_step)
+__device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const QueryRaw<D>& raw, QueryDigits<D / 64>& qd, float& q_step)
 {
     constexpr int G = D / 64;
     float x[G][16];
@@ -302,33 +307,37 @@ __device__ __forceinline__ void quantize_query(const GqaDecodeParams& p, const Q
     q_absmax = wave_max_16x4(q_absmax);
     const bool q_ok = q_absmax > 0.0f && q_absmax < __builtin_inff();
     q_step = q_ok ? q_absmax * (1.0f / 32512.0f) : 0.0f;
-    const float inv_step = q_ok ? 32512.0f / q_absmax : 0.0f;
+    const float inv_step = q_ok ? (32512.0f * 256.0f) / q_absmax : 0.0f; // to units of the last digit
 #pragma unroll
     for (int a = 0; a < G; ++a) {
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            unsigned int hi_word = 0, lo_word = 0;
+            unsigned int hi_word = 0, lo_word = 0, ex_word = 0;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                int qi = (int)rintf(x[a][4 * w + e] * inv_step);
-                qi = max(-32512, min(32512, qi));
-                const int hi = (qi + 128) >> 8;
-                const int lo = qi - hi * 256;
+                int qi = (int)rintf(x[a][4 * w + e] * inv_step); // |x * inv_step| <= 2^23: an exact integer
+                qi = max(-32512 * 256, min(32512 * 256, qi));
+                const int top = (qi + 128) >> 8; // the upper two digits, |top| <= 32512
+                const int ex = qi - top * 256;
+                const int hi = (top + 128) >> 8;
+                const int lo = top - hi * 256;
                 hi_word |= ((unsigned int)hi & 0xffu) << (8 * e);
                 lo_word |= ((unsigned int)lo & 0xffu) << (8 * e);
+                ex_word |= ((unsigned int)ex & 0xffu) << (8 * e);
             }
-            qhi[a][w] = (int)hi_word;
-            qlo[a][w] = (int)lo_word;
+            qd.hi[a][w] = (int)hi_word;
+            qd.lo[a][w] = (int)lo_word;
+            qd.ex[a][w] = (int)ex_word;
         }
     }
 }
 
 template <int D>
 __device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsigned int b, unsigned int head, bool head_valid,
-                                                  unsigned int j, i32x4 (&qhi)[D / 64], i32x4 (&qlo)[D / 64], float& q_step)
+                                                  unsigned int j, QueryDigits<D / 64>& qd, float& q_step)
 {
     const QueryRaw<D> raw = fetch_query<D>(p, b, head, head_valid, j);
-    quantize_query<D>(p, raw, qhi, qlo, q_step);
+    quantize_query<D>(p, raw, qd, q_step);
 }
 
 // One 32-token step, first half: scores, masking and the online-softmax update.
@@ -336,8 +345,8 @@ __device__ __forceinline__ void load_query_digits(const GqaDecodeParams& p, unsi
 //   ksr[i*4+r] scale row of token slot (tile i, row 4j + r) -- the C layout of the score tile
 // Leaves the step's probabilities in pr[] (same slots) and rescales acc when the running max moved.
 template <int G, int SDT, bool SOFTCAP, class Row>
-__device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Row (&ksr)[8], const i32x4 (&qhi)[G],
-                                            const i32x4 (&qlo)[G], float scale_log2, float inv_cap, float cap_log2,
+__device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Row (&ksr)[8], const QueryDigits<G>& qd,
+                                            float scale_log2, float inv_cap, float cap_log2,
                                             unsigned int t0, unsigned int j, unsigned int first, unsigned int len,
                                             float& run_max, float& run_sum, f32x4 (&acc)[G * 4], float (&pr)[8])
 {
@@ -351,12 +360,13 @@ __device__ __forceinline__ void qk_softmax_step(const u32x4 (&k)[2][G], const Ro
         for (int a = 0; a < G; ++a) {
             const i32x4 kc = __builtin_bit_cast(i32x4, k[i][a]);
             const i32x4 zero = {0, 0, 0, 0};
-            const i32x4 dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qhi[a], zero, 0, 0, 0);
-            const i32x4 dl = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qlo[a], zero, 0, 0, 0);
+            const i32x4 dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qd.hi[a], zero, 0, 0, 0);
+            const i32x4 dl = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qd.lo[a], zero, 0, 0, 0);
+            const i32x4 de = __builtin_amdgcn_mfma_i32_16x16x64_i8(kc, qd.ex[a], zero, 0, 0, 0);
             f32x4 d;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                d[r] = (float)(dh[r] * 256 + dl[r]);
+                d[r] = fmaf((float)de[r], 1.0f / 256.0f, (float)(dh[r] * 256 + dl[r]));
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -498,9 +508,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
     const unsigned int c_end = (unsigned int)min((unsigned long long)len, c_start64 + span);
     const unsigned int steps = (c_end - c_start + 31u) / 32u;
 
-    i32x4 qhi[G], qlo[G];
-    float q_step; // value of one fixed-point unit of this lane's head
-    load_query_digits<D>(p, b, head, head_valid, j, qhi, qlo, q_step);
+    QueryDigits<G> qd;
+    float q_step; // value of one unit of the middle digit for this lane's head
+    load_query_digits<D>(p, b, head, head_valid, j, qd, q_step);
 
     const unsigned int* table = p.tables + (p.table_shared ? 0 : (size_t)b * p.table_stride);
     const unsigned int k_row = p.num_kv_heads * D;           // bytes per cache row (codes)
@@ -648,7 +658,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void gqa_decode_q8_partial(Gqa
             }
         }
         float pr[8];
-        qk_softmax_step<G, SDT, SOFTCAP>(s.k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
+        qk_softmax_step<G, SDT, SOFTCAP>(s.k, ksr, qd, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
         clear_hidden_scale_rows<G>(vsr, t0, j, first, len);
         pv_step<G, SDT>(s.v, vsr, pr, acc);
     };
@@ -869,9 +879,9 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
         issue_scales(1, t1);
         issue_codes(v_base, lds_v, 1, t1);
     }
-    i32x4 qhi[G], qlo[G];
+    QueryDigits<G> qd;
     float q_step;
-    quantize_query<D>(p, q_raw, qhi, qlo, q_step);
+    quantize_query<D>(p, q_raw, qd, q_step);
 
     const float scale_log2 = (SOFTCAP ? p.score_scale : p.score_scale * kLog2e) * q_step;
     const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
@@ -910,7 +920,7 @@ __global__ __launch_bounds__(512) void gqa_decode_q8_dma128(GqaDecodeParams p)
             issue_scales(slot, t_next);
         }
         float pr[8];
-        qk_softmax_step<G, SDT, SOFTCAP>(k, ksr, qhi, qlo, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
+        qk_softmax_step<G, SDT, SOFTCAP>(k, ksr, qd, scale_log2, inv_cap, cap_log2, t0, j, first, len, run_max, run_sum, acc, pr);
         wait_vmcnt<behind == 2 ? 14 : behind == 1 ? 9 : 0>();
         unsigned int v[8][G];
 #pragma unroll
