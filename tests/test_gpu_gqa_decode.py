@@ -269,9 +269,12 @@ def test_pages_spread_over_64_gib_give_the_compact_pool_bits():
 
 
 # ---------------------------------------------------------------------------- f16 KV (config 3)
-def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0, poison=False):
+def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_gain=1.0, v_gain=1.0, q_std=1.0, poison=False, outliers=False):
     rng = np.random.default_rng(seed)
     cols = hkv * d
+    channel_gain = np.ones(cols, dtype=np.float32)
+    if outliers:  # 1 % of the channels carry values eight times larger
+        channel_gain[rng.choice(cols, size=max(1, cols // 100), replace=False)] = 8.0
     cap_lens = [min(l, ring_capacity) if ring_capacity else l for l in lens]
     tables, pool_blocks = draw_tables(rng, cap_lens, block_tokens)
     rows = pool_blocks * block_tokens
@@ -282,8 +285,8 @@ def make_f16_case(seed, lens, hq, hkv, d, block_tokens=16, ring_capacity=0, k_ga
     for b, l in enumerate(lens):
         kg = np.reshape(np.asarray(k_gain, dtype=np.float32), (-1, 1))
         vg = np.reshape(np.asarray(v_gain, dtype=np.float32), (-1, 1))
-        k = rng.standard_normal((l, cols)).astype(np.float32) * (kg if kg.shape[0] == 1 else kg[:l])
-        v = rng.standard_normal((l, cols)).astype(np.float32) * (vg if vg.shape[0] == 1 else vg[:l])
+        k = rng.standard_normal((l, cols)).astype(np.float32) * channel_gain * (kg if kg.shape[0] == 1 else kg[:l])
+        v = rng.standard_normal((l, cols)).astype(np.float32) * channel_gain * (vg if vg.shape[0] == 1 else vg[:l])
         O.half_append_paged(1, k, planes["k"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
         O.half_append_paged(1, v, planes["v"], tables[b], 0, block_tokens, ring_capacity=ring_capacity)
     q = (rng.standard_normal((len(lens), hq * d)) * q_std).astype(np.float32)

@@ -8,7 +8,7 @@ import pytest
 
 import oracle as O
 from tests.cases import assert_attention_close, make_gqa_q8_case, oracle_gqa_decode
-from tests.test_gpu_gqa_decode import run_decode
+from tests.test_gpu_gqa_decode import make_f16_case, run_decode, run_f16
 from tests.test_gpu_gqa_prefill import run_case, run_f16_case
 from tests.test_gpu_mla_decode import (draw_selection, make_mla_case, make_mla_chunk_case, oracle_mla, oracle_mla_chunk, run_mla,
                                        run_mla_chunk)
@@ -92,6 +92,26 @@ def test_random_q8_decode_pages_rules_and_hints(it):
         rc, want = O.sigmoid_gate(want, gate)
         assert rc == 0
     assert_attention_close(got, want, what)
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_random_f16_decode(it):
+    """Decode over f16 rows (the cache of the f16 model family, src/kv_cache/mod.rs:179-331) at head_dim 128 and 256: pages
+    of 1 to 64 tokens, windows, soft caps, score scales up to 0.2 over outlier channels, never-cleared pools."""
+    rng = np.random.default_rng([707, it])
+    hkv = pick(rng, [1, 2, 4, 8])
+    group = pick(rng, [1, 2, 4, 8, 16])
+    d = pick(rng, [128, 256])
+    page = pick(rng, PAGE_SIZES)
+    lens = [max(1, pick(rng, LENGTHS + [6000])) for _ in range(int(rng.integers(1, 7)))]
+    window = pick(rng, [0, 0, 1, 33, 1024])
+    softcap = pick(rng, [0.0, 0.0, 50.0])
+    scale = pick(rng, [1.0 / np.sqrt(d), 0.09, 0.2])
+    what = f"f16 decode {it}: {hkv * group}/{hkv} d={d} page={page} lens={lens} window={window} softcap={softcap} scale={scale:.3f}"
+    print(what, flush=True)
+    case = make_f16_case(7000 + it, lens, hkv * group, hkv, d, block_tokens=page, poison=bool(it % 3 == 0), outliers=bool(it % 2))
+    got = run_f16(case, scale, window=window, softcap=softcap)
+    assert_attention_close(got, oracle_gqa_decode(case, scale, window=window, softcap=softcap, fmt=O.FMT_F16), what)
 
 
 @pytest.mark.parametrize("it", [*range(48), 1298])  # 1298: f32 queries, score scale 0.3, outlier channels
