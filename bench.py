@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 # HBM bytes one launch of the partial kernel moves on the default workload: rocprofv3 FETCH_SIZE and WRITE_SIZE
 # per dispatch, each scaled by what the same counter reads for a 1 GiB device copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the runs and their numbers are in profiles/gqa_decode_q8_dma128__gqa_decode_32k.md.
-GQA_32K_TRAFFIC_BYTES = 564313293
+GQA_32K_TRAFFIC_BYTES = 564179558
 METRIC = "decode attn effective KV GB/s (% of HBM peak) + tokens/s at 32K ctx, 1 GPU"
 
 
