@@ -282,3 +282,68 @@ def test_random_mla_other_widths_and_weight_forms(it):
     else:
         want, _ = oracle_mla_chunk(case)
         assert_attention_close(run_mla_chunk(case).cpu().numpy(), want, what)
+
+
+@pytest.mark.parametrize("it", range(40))
+def test_random_q8g64_append(it):
+    """The quantizing append, bit for bit: the three scale rules, f32 / bf16 / f16 sources, 64 to 4,096 columns, pages of 1
+    to 128 tokens, any start row, rings, and the values a quantizer can get wrong -- codes exactly between two integers,
+    all-zero and one-element groups, subnormal and huge magnitudes, negative zero."""
+    from zllm_amd import ops
+    from tests.cases import draw_tables, upload
+
+    rng = np.random.default_rng([808, it])
+    rule = pick(rng, [O.RULE_ROCM_MLA, O.RULE_METAL_GQA, O.RULE_CUDA_GQA])
+    cols = pick(rng, [64, 128, 192, 512, 576, 1024, 2048, 4096])
+    page = pick(rng, PAGE_SIZES + [128])
+    rows = int(rng.integers(1, 300))
+    start = int(rng.integers(0, 200))
+    src = pick(rng, ["f32", "f32", "bf16", "f16"])
+    ring = pick(rng, [0, 0, 0, 64, 100])
+    what = f"append {it}: rule={rule} cols={cols} page={page} rows={rows} start={start} src={src} ring={ring}"
+    print(what, flush=True)
+    x = rng.standard_normal((rows, cols)).astype(np.float32) * np.float32(2.0 ** rng.integers(-20, 20))
+    groups = x.reshape(rows, cols // 64, 64)
+    for _ in range(min(rows, 12)):  # special groups
+        r, g, kind = int(rng.integers(0, rows)), int(rng.integers(0, cols // 64)), int(rng.integers(0, 6))
+        if kind == 0:
+            groups[r, g] = 0.0
+        elif kind == 1:
+            groups[r, g] = -0.0
+            groups[r, g, 3] = 1e-41  # a subnormal alone
+        elif kind == 2:  # codes exactly halfway: the largest element is 127 units, the others k + 0.5 units
+            unit = np.float32(2.0 ** rng.integers(-10, 10))
+            groups[r, g] = (rng.integers(-126, 126, size=64) + 0.5).astype(np.float32) * unit
+            groups[r, g, 0] = 127.0 * unit
+        elif kind == 3:
+            groups[r, g] *= np.float32(1e30)
+        elif kind == 4:
+            groups[r, g] = 0.0
+            groups[r, g, 63] = -3.0
+        else:
+            groups[r, g] = np.float32(65504.0) if src == "f16" else np.float32(3e38)
+    if src == "bf16":
+        bits = O.f32_to_bf16(x)
+        x = O.bf16_to_f32(bits)
+        dev = upload(bits).view(torch.bfloat16)
+    elif src == "f16":
+        x = np.clip(x, -65504.0, 65504.0)
+        half = x.astype(np.float16)
+        x = half.astype(np.float32)
+        dev = upload(half)
+    else:
+        dev = upload(x)
+    stored = min(start + rows, ring) if ring else start + rows
+    tables, pool_blocks = draw_tables(rng, [max(stored, 1)], page)
+    pool_rows = pool_blocks * page
+    sdt = {O.RULE_ROCM_MLA: O.SCALE_BF16, O.RULE_METAL_GQA: O.SCALE_F16, O.RULE_CUDA_GQA: O.SCALE_F32}[rule]
+    ref_codes = np.full((pool_rows, cols), 77, dtype=np.int8)
+    ref_scales = np.full((pool_rows, cols // 64), 3, dtype=np.float32 if sdt == O.SCALE_F32 else np.uint16)
+    codes, scales = upload(ref_codes), upload(ref_scales)
+    if ring and rows > ring:  # a ring takes at most its capacity in one call
+        x, dev, rows = x[:ring], dev[:ring], ring
+    O.q8g64_append_paged(rule, x, ref_codes, ref_scales, tables[0], start, page, ring_capacity=ring)
+    ops.q8g64_append(dev, codes, scales, upload(tables[0]), start, page, rule, ring_capacity=ring)
+    torch.cuda.synchronize()
+    assert np.array_equal(scales.cpu().numpy().view(ref_scales.dtype).view(np.uint8), ref_scales.view(np.uint8)), what + ": scale bits differ"
+    assert np.array_equal(codes.cpu().numpy(), ref_codes), what + ": codes differ"
