@@ -347,3 +347,102 @@ def test_random_q8g64_append(it):
     torch.cuda.synchronize()
     assert np.array_equal(scales.cpu().numpy().view(ref_scales.dtype).view(np.uint8), ref_scales.view(np.uint8)), what + ": scale bits differ"
     assert np.array_equal(codes.cpu().numpy(), ref_codes), what + ": codes differ"
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_random_gqa_prologue(it):
+    """Per-head RMSNorm + RoPE of Q and K and the quantizing append of K and V in one launch, against the CPU chain
+    rmsnorm_heads -> rope_apply -> q8g64_append_paged: head sizes 64 to 256, rotary widths, both layouts, the Gemma weight
+    offset, pages of 1 to 128 tokens, any start row; Q, codes and scale bits compared bit for bit."""
+    from zllm_amd import ops
+    from tests.cases import draw_tables, upload
+    from tests.test_gpu_gqa_prologue import cpu_chain, rope_table
+
+    rng = np.random.default_rng([909, it])
+    d = pick(rng, [64, 128, 128, 256])
+    hkv = pick(rng, [1, 2, 4, 8])
+    hq = hkv * pick(rng, [1, 2, 4, 8])
+    rotary = pick(rng, [0, d // 2, d, d])
+    split_half = bool(rng.integers(0, 2))
+    offset = pick(rng, [0.0, 1.0])
+    rows = int(rng.integers(1, 90))
+    position = int(rng.integers(0, 300))
+    page = pick(rng, PAGE_SIZES + [128])
+    eps = pick(rng, [1e-6, 1e-5])
+    what = f"prologue {it}: d={d} {hq}/{hkv} rotary={rotary} split_half={split_half} offset={offset} rows={rows} position={position} page={page}"
+    print(what, flush=True)
+    q = rng.standard_normal((rows, hq * d)).astype(np.float32) * np.float32(2.0 ** rng.integers(-6, 7))
+    k = rng.standard_normal((rows, hkv * d)).astype(np.float32) * np.float32(2.0 ** rng.integers(-6, 7))
+    v = rng.standard_normal((rows, hkv * d)).astype(np.float32) * np.float32(2.0 ** rng.integers(-6, 7))
+    k[:, :64] *= 40.0
+    if rows > 2:
+        k[1] = 0.0  # an all-zero row: the norm divides by sqrt(eps)
+        v[2, 64:128] = 0.0 if hkv * d > 64 else v[2, 64:128]
+    qw = (rng.standard_normal(d) * 0.2).astype(np.float32)
+    kw = (rng.standard_normal(d) * 0.2).astype(np.float32)
+    cos, sin = rope_table(position + rows + 3, max(rotary // 2, 1))
+    tables, pool_blocks = draw_tables(rng, [position + rows], page)
+    pool_rows = pool_blocks * page
+    want_q = cpu_chain(q, hq, d, qw, eps, offset, rotary, position, cos, sin, split_half)
+    want_k = cpu_chain(k, hkv, d, kw, eps, offset, rotary, position, cos, sin, split_half)
+    ref = {n: np.zeros((pool_rows, hkv * d), dtype=np.int8) for n in ("k", "v")}
+    ref_s = {n: np.zeros((pool_rows, hkv * d // 64), dtype=np.uint16) for n in ("k", "v")}
+    O.q8g64_append_paged(O.RULE_METAL_GQA, want_k, ref["k"], ref_s["k"], tables[0], position, page)
+    O.q8g64_append_paged(O.RULE_METAL_GQA, v, ref["v"], ref_s["v"], tables[0], position, page)
+    dev = {n: torch.zeros((pool_rows, hkv * d), dtype=torch.int8, device="cuda") for n in ("k", "v")}
+    dev_s = {n: torch.zeros((pool_rows, hkv * d // 64), dtype=torch.int16, device="cuda") for n in ("k", "v")}
+    got_q = ops.gqa_prologue(upload(q), upload(k), upload(v), upload(qw), upload(kw), upload(cos) if rotary else None,
+                             upload(sin) if rotary else None, dev["k"], dev_s["k"], dev["v"], dev_s["v"], upload(tables[0]),
+                             position, hq, hkv, d, rotary, page, eps=eps, weight_offset=offset, split_half=split_half)
+    torch.cuda.synchronize()
+    assert np.array_equal(got_q.cpu().numpy().view(np.uint32), want_q.view(np.uint32)), what + ": Q bits differ"
+    for n in ("k", "v"):
+        assert np.array_equal(dev_s[n].cpu().numpy().view(np.uint16), ref_s[n]), what + f": {n} scale bits differ"
+        assert np.array_equal(dev[n].cpu().numpy(), ref[n]), what + f": {n} codes differ"
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_random_mla_append(it):
+    """The fused MLA append (latent rows quantized with the bf16-scale rule, rope rows rotated and stored as bf16) at latent
+    widths of 64 to 1,024 and rope widths of 2 to 256, both rotary layouts, any page size and start row, rope positions
+    apart from cache positions: every byte against q8g64_append_paged + rope_apply + half_append_paged."""
+    from zllm_amd import ops
+    from tests.cases import draw_tables, upload
+
+    rng = np.random.default_rng([1010, it])
+    latent_cols = pick(rng, [64, 128, 256, 512, 512, 512, 576, 1024])
+    rope_cols = pick(rng, [2, 32, 64, 64, 64, 128, 256])
+    rotary_dim = pick(rng, [0, rope_cols, rope_cols, max(2, rope_cols // 2)])
+    layout = int(rng.integers(0, 2))
+    rows = int(rng.integers(1, 120))
+    position = int(rng.integers(0, 300))
+    rope_position = position + int(rng.integers(0, 5))
+    page = pick(rng, PAGE_SIZES + [128])
+    what = f"mla append {it}: latent={latent_cols} rope={rope_cols} rotary={rotary_dim} layout={layout} rows={rows} position={position} page={page}"
+    print(what, flush=True)
+    tables, pool_blocks = draw_tables(rng, [position + rows], page)
+    latent = rng.standard_normal((rows, latent_cols)).astype(np.float32) * np.float32(2.0 ** rng.integers(-8, 9))
+    k_rope = rng.standard_normal((rows, rope_cols)).astype(np.float32) * np.float32(2.0 ** rng.integers(-4, 5))
+    half = max(rotary_dim // 2, 1)
+    angles = rng.uniform(0, 6.28, size=(rope_position + rows + 3, half)).astype(np.float32)
+    cos, sin = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    pool = pool_blocks * page
+    ref_codes = np.zeros((pool, latent_cols), dtype=np.int8)
+    ref_scales = np.zeros((pool, latent_cols // 64), dtype=np.uint16)
+    ref_rope = np.zeros((pool, rope_cols), dtype=np.uint16)
+    O.q8g64_append_paged(O.RULE_ROCM_MLA, latent, ref_codes, ref_scales, tables[0], position, page)
+    rotated = k_rope
+    if rotary_dim:
+        rc, rotated = O.rope_apply(k_rope, 1, rotary_dim, rope_position, cos, sin, layout=0 if layout == 1 else 1, placement=1)
+        assert rc == 0
+    O.half_append_paged(0, rotated, ref_rope, tables[0], position, page)
+    codes = torch.zeros((pool, latent_cols), dtype=torch.int8, device="cuda")
+    scales = torch.zeros((pool, latent_cols // 64), dtype=torch.int16, device="cuda")
+    rope_cache = torch.zeros((pool, rope_cols), dtype=torch.int16, device="cuda")
+    ops.mla_append(upload(latent), upload(k_rope), codes, scales, rope_cache, upload(tables[0]), position, page,
+                   cos=upload(cos) if rotary_dim else None, sin=upload(sin) if rotary_dim else None,
+                   rotary_dim=rotary_dim, rotary_layout=layout, rope_position=rope_position)
+    torch.cuda.synchronize()
+    assert np.array_equal(codes.cpu().numpy(), ref_codes), what + ": codes differ"
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), ref_scales), what + ": scale bits differ"
+    assert np.array_equal(rope_cache.cpu().numpy().view(np.uint16), ref_rope), what + ": rope bits differ"
