@@ -7,6 +7,7 @@
 
 #include <algorithm>
 #include <map>
+#include <mutex>
 #include <numeric>
 
 #include "../../include/zllm_attn.h"
@@ -396,7 +397,9 @@ struct RocmContext::Scratch {
     size_t next = 0;
     uint8_t* stage_host = nullptr; // pinned, kStageBytes
     size_t stage_next = 0;
-    // idle blocks by capacity; a block is reused for a request of at least half its size
+    // idle blocks by capacity; a block is reused for a request of at least half its size.  Tensors may be dropped on any
+    // thread, so the map has a lock of its own; everything else here belongs to the thread that drives the context.
+    std::mutex pool_lock;
     std::multimap<size_t, void*> idle;
     size_t idle_bytes = 0;
     DeviceBuffer identity;         // u32 [identity_pages]: 0, 1, 2, ...
@@ -432,12 +435,15 @@ struct RocmContext::Scratch {
     }
     void give_back(void* block, size_t capacity)
     {
-        if (idle_bytes + capacity > kPoolKeepBytes) {
-            (void)hipFree(block);
-            return;
+        {
+            std::lock_guard<std::mutex> hold(pool_lock);
+            if (idle_bytes + capacity <= kPoolKeepBytes) {
+                idle.emplace(capacity, block);
+                idle_bytes += capacity;
+                return;
+            }
         }
-        idle.emplace(capacity, block);
-        idle_bytes += capacity;
+        (void)hipFree(block);
     }
 };
 
@@ -497,13 +503,17 @@ Result<DeviceBuffer> RocmContext::pooled(size_t bytes) const
     Scratch& s = *scratch_;
     size_t real = Scratch::size_class(std::max<size_t>(bytes, 1));
     void* block = nullptr;
-    auto found = s.idle.lower_bound(real);
-    if (found != s.idle.end() && found->first <= real * 2) {
-        block = found->second;
-        real = found->first;
-        s.idle_bytes -= real;
-        s.idle.erase(found);
-    } else {
+    {
+        std::lock_guard<std::mutex> hold(s.pool_lock);
+        auto found = s.idle.lower_bound(real);
+        if (found != s.idle.end() && found->first <= real * 2) {
+            block = found->second;
+            real = found->first;
+            s.idle_bytes -= real;
+            s.idle.erase(found);
+        }
+    }
+    if (block == nullptr) {
         const hipError_t err = hipMalloc(&block, real);
         if (err != hipSuccess) {
             return hip_error("hipMalloc", err);

@@ -237,6 +237,10 @@ struct HostCounters {
     size_t staged_uploads = 0;      // small host arrays (visible ends, selections) sent through the pinned ring
 };
 
+// One context drives one HIP stream and keeps that stream's scratch.  A context and its copies (they share the scratch)
+// belong to one thread at a time; a thread that wants a stream of its own creates a context of its own, which is the
+// reference's model as well -- its active device and stream are thread-local (src/kernel/rocm/hip/mod.rs:15-50).
+// Tensors and buffers a context handed out may be dropped on any thread.
 class RocmContext {
   public:
     static Result<RocmContext> create(int device_id);
