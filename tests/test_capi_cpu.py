@@ -326,3 +326,68 @@ def test_head_dim_192_is_taken_over_q8g64_only(lib):
     pre.rows, pre.position, pre.num_heads, pre.num_kv_heads, pre.head_dim, pre.block_tokens, pre.score_scale = 64, 500, 12, 3, 192, 16, 0.07
     pre.kv_format, pre.scale_dtype, pre.q_dtype = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16
     assert lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(pre)) > 0  # its rows run as decode items: ranges and split records
+
+
+def test_planning_entry_points_survive_arbitrary_argument_blocks(lib):
+    """The entry points that run on the host alone (workspace sizes, split plans, record layouts) take argument blocks
+    whose numbers are zero, huge or inconsistent: each answers 0 / -1 with a message, or a size, and never divides by zero
+    or walks a null pointer.  Pointers stay null: nothing here reads device memory."""
+    rng = np.random.default_rng(4242)
+    edge = [0, 1, 2, 3, 15, 16, 31, 32, 33, 63, 64, 65, 127, 128, 192, 255, 256, 512, 576, 1024, 4096, 65535, 65536, 1 << 20, (1 << 31) - 1,
+            1 << 31, (1 << 32) - 1]
+
+    def fill(args, skip=()):
+        for name, ctype in args._fields_:
+            if name in skip or ctype is C.c_void_p:
+                continue
+            if ctype is C.c_float:
+                setattr(args, name, float(rng.choice([0.0, -1.0, 0.09, 1e30, float("inf"), float("nan")])))
+            elif ctype is C.c_uint64:
+                setattr(args, name, int(rng.choice(edge)) * int(rng.choice([1, 1 << 20])))
+            elif ctype is C.c_int:
+                setattr(args, name, int(rng.choice([-1, 0, 1, 2, 3, 7])))
+            else:
+                setattr(args, name, int(rng.choice(edge)))
+
+    for _ in range(3000):
+        g = capi.GqaDecodeArgs()
+        fill(g)
+        if rng.random() < 0.7:  # mostly near-valid blocks: the plans' arithmetic is what is under test
+            g.kv_format, g.scale_dtype, g.q_dtype, g.score_scale = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16, 0.1
+            g.num_kv_heads = int(rng.choice([1, 2, 3, 8]))
+            g.num_heads = g.num_kv_heads * int(rng.choice([1, 4, 16, 17, 64]))
+            g.head_dim = int(rng.choice([64, 128, 192, 256]))
+            g.block_tokens = int(rng.choice([1, 16, 48, 64, 1 << 20]))
+        need = lib.zllm_attn_gqa_decode_workspace_bytes(C.byref(g))
+        chunk, chunks, layout = C.c_uint32(), C.c_uint32(), capi.SplitRecordLayout()
+        rc = lib.zllm_attn_gqa_decode_split_plan(C.byref(g), C.byref(chunk), C.byref(chunks))
+        assert lib.zllm_attn_gqa_decode_record_layout(C.byref(g), C.byref(layout)) == rc
+        assert (need > 0) == (rc == 0)
+        if rc == 0:
+            assert chunk.value >= 32 and chunks.value >= 1 and layout.record_rows >= 1
+        p = capi.GqaPrefillArgs()
+        fill(p)
+        if rng.random() < 0.7:
+            p.kv_format, p.scale_dtype, p.q_dtype, p.out_dtype, p.score_scale = capi.KV_Q8G64, capi.SCALE_F16, capi.DTYPE_BF16, capi.DTYPE_F32, 0.1
+            p.num_kv_heads = int(rng.choice([1, 2, 8]))
+            p.num_heads = p.num_kv_heads * int(rng.choice([1, 4, 16, 200]))
+            p.head_dim = int(rng.choice([64, 128, 192, 256]))
+            p.block_tokens = int(rng.choice([1, 16, 48, 64]))
+            p.rows = int(rng.choice([1, 2, 16, 17, 300, 5000]))
+            p.position = int(rng.choice([0, 1, 1000, 50000, 1 << 22]))
+            p.gate_cols, p.softcap = 0, 0.0
+        lib.zllm_attn_gqa_prefill_workspace_bytes(C.byref(p))
+        m = capi.MlaDecodeArgs()
+        fill(m)
+        if rng.random() < 0.7:
+            m.q_dtype, m.out_dtype = capi.DTYPE_BF16, capi.DTYPE_F32
+            m.heads = int(rng.choice([1, 16, 33, 128]))
+            m.latent_dim, m.rope_dim = int(rng.choice([64, 512, 1024])), int(rng.choice([2, 64, 256]))
+            nope, value = int(rng.choice([16, 128])), int(rng.choice([16, 128, 192]))
+            m.q_head_dim, m.kv_head_dim = nope + m.rope_dim, nope + value
+            m.block_tokens = int(rng.choice([1, 16, 48, 64]))
+            m.kv_b_bits, m.stage_mask, m.top_k = 0, 0, 0
+            m.batch, m.query_rows = int(rng.choice([1, 4, 33, 3000])), int(rng.choice([0, 1, 5, 512]))
+        need = lib.zllm_attn_mla_decode_workspace_bytes(C.byref(m))
+        rc = lib.zllm_attn_mla_decode_record_layout(C.byref(m), C.byref(layout))
+        assert (need > 0) == (rc == 0)

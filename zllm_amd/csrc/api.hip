@@ -160,6 +160,9 @@ void plan_splits(uint32_t max_len, uint64_t units, uint32_t units_per_group, uin
     *max_chunks = (uint32_t)(chunks == 0 ? 1 : chunks);
 }
 
+// Token positions are 32-bit in the kernels, which also round them up to steps and splits: lengths stay below 2^31.
+constexpr uint32_t kMaxTokens = 0x7fffff00u;
+
 int validate_gqa_decode(const zllm_gqa_decode_args* a)
 {
     if (a == nullptr) {
@@ -175,8 +178,8 @@ int validate_gqa_decode(const zllm_gqa_decode_args* a)
     if (a->batch > 65535u) {
         return fail(-1, "GQA decode: batch=%u exceeds 65535 rows per call", a->batch);
     }
-    if (a->block_tokens == 0 || a->max_kv_len == 0) {
-        return fail(-1, "GQA decode: block_tokens=%u max_kv_len=%u must be non-zero", a->block_tokens, a->max_kv_len);
+    if (a->block_tokens == 0 || a->max_kv_len == 0 || a->max_kv_len > kMaxTokens) {
+        return fail(-1, "GQA decode: block_tokens=%u max_kv_len=%u must be non-zero, max_kv_len below 2^31", a->block_tokens, a->max_kv_len);
     }
     if (!isfinite(a->score_scale) || a->score_scale <= 0.0f || !(a->softcap >= 0.0f) || !isfinite(a->softcap)) {
         return fail(-1, "GQA decode: invalid score_scale=%g softcap=%g", (double)a->score_scale, (double)a->softcap);
@@ -326,8 +329,8 @@ int validate_mla_decode(const zllm_mla_decode_args* a)
         return fail(-1, "MLA decode: %u-bit kv_b needs scales, a group size that divides latent_dim=%u (got %u) and a scale dtype", a->kv_b_bits,
                     a->latent_dim, a->kv_b_group);
     }
-    if (a->block_tokens == 0 || a->max_ctx_len == 0) {
-        return fail(-1, "MLA decode: block_tokens=%u max_ctx_len=%u must be non-zero", a->block_tokens, a->max_ctx_len);
+    if (a->block_tokens == 0 || a->max_ctx_len == 0 || a->max_ctx_len > kMaxTokens) {
+        return fail(-1, "MLA decode: block_tokens=%u max_ctx_len=%u must be non-zero, max_ctx_len below 2^31", a->block_tokens, a->max_ctx_len);
     }
     if ((a->q_dtype != ZLLM_DTYPE_F32 && a->q_dtype != ZLLM_DTYPE_BF16) || (a->out_dtype != ZLLM_DTYPE_F32 && a->out_dtype != ZLLM_DTYPE_BF16)) {
         return fail(-1, "MLA decode: q_dtype / out_dtype must be f32 or bf16");
@@ -1077,8 +1080,8 @@ static int validate_gqa_prefill(const zllm_gqa_prefill_args* a)
         return fail(-1, "GQA prefill: table_stride=%u pages of %u tokens cannot cover position + rows = %llu", a->table_stride,
                     a->block_tokens, (unsigned long long)a->position + a->rows);
     }
-    if (a->block_tokens == 0 || (uint64_t)a->position + a->rows > 0xffffffffull) {
-        return fail(-1, "GQA prefill: block_tokens must be non-zero and position + rows fit u32");
+    if (a->block_tokens == 0 || (uint64_t)a->position + a->rows > kMaxTokens) {
+        return fail(-1, "GQA prefill: block_tokens must be non-zero and position + rows stay below 2^31");
     }
     if (!isfinite(a->score_scale) || a->score_scale <= 0.0f || !(a->softcap >= 0.0f) || !isfinite(a->softcap)) {
         return fail(-1, "GQA prefill: invalid score_scale=%g softcap=%g", (double)a->score_scale, (double)a->softcap);
