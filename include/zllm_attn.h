@@ -253,7 +253,7 @@ typedef struct zllm_gqa_decode_args {
     uint32_t batch;
     uint32_t num_heads, num_kv_heads, head_dim; /* head_dim in {64, 128, 192, 256}; f16 caches 128 / 256 */
     uint32_t table_stride;         /* entries per sequence in `tables` */
-    uint32_t max_kv_len;           /* host upper bound of kv_lens: sizes the grid and the split plan.  A call
+    uint32_t max_kv_len;           /* host upper bound of kv_lens, below 2^31: sizes the grid and the split plan.  A call
                                       recorded into a HIP graph stays valid only while every kv_lens[b] on the
                                       device is <= max_kv_len; tokens past the planned splits are not read */
     uint32_t total_kv_tokens;      /* host bound: sum of the visible lengths (0 = unknown, batch * max_kv_len is
@@ -364,7 +364,7 @@ typedef struct zllm_gqa_prefill_args {
     void* workspace;       /* [dev] */
     uint64_t workspace_bytes;
     uint32_t rows;         /* chunk length T */
-    uint32_t position;     /* tokens already cached before the chunk */
+    uint32_t position;     /* tokens already cached before the chunk; position + rows stays below 2^31 */
     uint32_t window;       /* 0 = full causal, else sliding window size */
     uint32_t num_heads, num_kv_heads, head_dim;
     uint32_t block_tokens;
@@ -471,7 +471,7 @@ typedef struct zllm_mla_decode_args {
     uint32_t latent_dim;          /* a multiple of 64 up to 1024; 512 runs the matrix-core kernels */
     uint32_t rope_dim;            /* even, up to 256; 64 runs the matrix-core kernels */
     uint32_t table_stride;
-    uint32_t max_ctx_len;         /* host upper bound of ctx_lens (split plan); a recorded graph stays valid
+    uint32_t max_ctx_len;         /* host upper bound of ctx_lens, below 2^31 (split plan); a recorded graph stays valid
                                      only while every ctx_lens[b] <= max_ctx_len */
     uint32_t block_tokens;
     int q_dtype;                  /* ZLLM_DTYPE_F32 or ZLLM_DTYPE_BF16 */
