@@ -316,7 +316,7 @@ def test_random_q8g64_append(it):
             groups[r, g] = (rng.integers(-126, 126, size=64) + 0.5).astype(np.float32) * unit
             groups[r, g, 0] = 127.0 * unit
         elif kind == 3:
-            groups[r, g] *= np.float32(1e30)
+            groups[r, g] = np.clip(groups[r, g].astype(np.float64) * 1e30, -3e38, 3e38).astype(np.float32)
         elif kind == 4:
             groups[r, g] = 0.0
             groups[r, g, 63] = -3.0
