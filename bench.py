@@ -29,6 +29,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 # per dispatch, each scaled by what the same counter reads for a 1 GiB device copy (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0); the runs and their numbers are in profiles/gqa_decode_q8_dma128__gqa_decode_32k.md.
 GQA_32K_TRAFFIC_BYTES = 564179558
+GQA_RAGGED_TRAFFIC_BYTES = 246880256  # seed 2's draw: profiles/gqa_decode_q8_dma128__gqa_decode_ragged.md
 METRIC = "decode attn effective KV GB/s (% of HBM peak) + tokens/s at 32K ctx, 1 GPU"
 
 
@@ -359,9 +360,10 @@ def run_gqa_decode(args, ragged, config1=False):
                   f"regions of exactly {args.steps} steps each, bracketed by synchronize: ms_per_step is the median region",
         "roofline": {"bound": "hbm", "kernel": "gqa_decode_q8_dma128", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None if ragged or config1 or args.seed != 2 else GQA_32K_TRAFFIC_BYTES,
-                     "traffic_source": None if ragged or config1 or args.seed != 2 else
-                     "profiles/gqa_decode_q8_dma128__gqa_decode_32k.md: rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload, scaled by a 1 GiB copy; not read in this run",
+                     "traffic": None if config1 or args.seed != 2 else GQA_RAGGED_TRAFFIC_BYTES if ragged else GQA_32K_TRAFFIC_BYTES,
+                     "traffic_source": None if config1 or args.seed != 2 else
+                     f"profiles/gqa_decode_q8_dma128__gqa_decode_{'ragged' if ragged else '32k'}.md: rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload, "
+                     "scaled by a 1 GiB copy; not read in this run",
                      "kernel_ms": round(ms_partial, 5), "kernel_ms_single_launch_median": round(ms_partial_median, 5),
                      "kernel_ms_single_launch_min": round(ms_partial_min, 5)},
     }
@@ -493,7 +495,7 @@ def other_configs(args):
         out["workload"] = record["config"]["workload"]
         out["roofline"] = {k: v for k, v in record["roofline"].items() if k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "kernel_ms",
                                                                                  "kernel_ms_single_launch_median", "kernel_ms_single_launch_min",
-                                                                                 "second_kernel_wide_tiles")}
+                                                                                 "second_kernel_wide_tiles", "traffic", "traffic_source")}
         if "cpu_baseline" in record:
             out["cpu_baseline"] = {k: record["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind", "sample")}
         return out

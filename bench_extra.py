@@ -10,6 +10,7 @@ import time
 import numpy as np
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+MLA_64K_TRAFFIC_BYTES = 210674278  # mla_partial_ws on seed 2's config 4: 177.0 MB read (cache rows: 172.0 MB) + 33.7 MB of split records written
 HBM_PEAK_GBPS = 8000.0
 
 
@@ -133,7 +134,10 @@ def run_mla_decode(args):
         "launch": f"hipGraph replay, {per_graph} decode calls (absorb + partial + merge/project each) per graph; 0.1 s of untimed replays before the timed ones",
         "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()},
         "roofline": {"bound": "mfma", "kernel": "mla_partial", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": MLA_64K_TRAFFIC_BYTES if args.seed == 2 else None,
+                     "traffic_source": "profiles/mla_partial_ws__mla_decode_64k.md: rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload, scaled by a 1 GiB copy; "
+                                       "not read in this run" if args.seed == 2 else None,
                      "kernel_ms": round(stage_ms["partial"], 5), "kernel_ms_single_launch_median": round(singles[len(singles) // 2], 5),
                      "kernel_ms_single_launch_min": round(singles[0], 5),
                      "second_kernel_wide_tiles": {"kernel_ms": round(stage_ms["partial_wide_tiles"], 5),
