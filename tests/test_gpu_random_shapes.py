@@ -446,3 +446,35 @@ def test_random_mla_append(it):
     assert np.array_equal(codes.cpu().numpy(), ref_codes), what + ": codes differ"
     assert np.array_equal(scales.cpu().numpy().view(np.uint16), ref_scales), what + ": scale bits differ"
     assert np.array_equal(rope_cache.cpu().numpy().view(np.uint16), ref_rope), what + ": rope bits differ"
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_random_block_attention(it):
+    """Explicit per-row key ranges (BlockAttentionSpec::visible and its varlen form, src/attention/block.rs:10-119) drawn at
+    random: free [start, end) per row, packed isolated segments, one-key rows, more rows than keys; Q8g64 and f16 rows, every
+    head size a chunk kernel takes, with and without the workspace."""
+    from tests.test_gpu_block_attention import run_block, varlen_ranges
+
+    rng = np.random.default_rng([1111, it])
+    kv = pick(rng, ["q8", "q8", "f16"])
+    d = pick(rng, [128, 256] if kv == "f16" else [64, 128, 128, 256])
+    hkv = pick(rng, [1, 2, 4, 8])
+    hq = hkv * pick(rng, [1, 2, 4, 8])
+    q_kind = "bf16" if d != 128 or kv == "f16" else pick(rng, ["bf16", "f32"])
+    page = pick(rng, [16, 16, 64, 48, 1])
+    workspace = bool(rng.integers(0, 3))
+    if rng.integers(0, 2):  # isolated segments packed into one call
+        segments = int(rng.integers(1, 7))
+        q_off = np.concatenate([[0], np.cumsum(rng.integers(1, 120, size=segments))])
+        kv_off = np.concatenate([[0], np.cumsum(rng.integers(1, 900, size=segments))])
+        visible = varlen_ranges([int(x) for x in q_off], [int(x) for x in kv_off])
+        q_rows, kv_rows = int(q_off[-1]), int(kv_off[-1])
+    else:
+        q_rows, kv_rows = int(rng.integers(1, 200)), int(rng.integers(2, 4000))
+        starts = rng.integers(0, kv_rows - 1, size=q_rows)
+        ends = np.minimum(starts + rng.integers(1, max(2, kv_rows), size=q_rows), kv_rows)
+        visible = np.stack([starts, ends], axis=1)
+    what = f"block {it}: {kv} d={d} {hq}/{hkv} q={q_kind} page={page} rows={q_rows} keys={kv_rows} workspace={workspace}"
+    print(what, flush=True)
+    out, want = run_block(11000 + it, q_rows, kv_rows, hq, hkv, d, visible, kv=kv, q_kind=q_kind, block_tokens=page, workspace=workspace)
+    assert_attention_close(out, want, what)
