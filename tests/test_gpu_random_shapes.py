@@ -478,3 +478,21 @@ def test_random_block_attention(it):
     print(what, flush=True)
     out, want = run_block(11000 + it, q_rows, kv_rows, hq, hkv, d, visible, kv=kv, q_kind=q_kind, block_tokens=page, workspace=workspace)
     assert_attention_close(out, want, what)
+
+
+def test_the_cases_that_found_the_query_step_stay_far_inside_the_bound(monkeypatch):
+    """Nine draws of the sweeps once exceeded 2e-3 through the query alone (a fixed-point step of 2^-15 of the row's largest
+    element in the decode kernels, f16's eleven bits for an f32 query in the chunk kernel).  With three query digits and
+    hi + lo fragments they measure 1.5e-5 to 1.4e-4 on outputs of magnitude 12 to 22: held to 4e-4 here, a fifth of the
+    bound, so that a query carried with fewer bits again shows."""
+    import sys
+
+    this = sys.modules[__name__]
+    usual = assert_attention_close
+    monkeypatch.setattr(this, "assert_attention_close", lambda got, want, what="", atol=4e-4, rtol=1e-2: usual(got, want, what, atol=4e-4, rtol=rtol))
+    for it in (52, 190, 266, 814):
+        test_random_q8_decode_pages_rules_and_hints(it)
+    for it in (265, 273, 497):
+        test_random_q8_decode(it)
+    test_random_q8_head_dim_192(779)
+    test_random_q8_prefill_chunk(1298)
